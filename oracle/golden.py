@@ -1,0 +1,217 @@
+"""ctypes/numpy front end of the CPU oracle (``oracle/golden.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke()`` and by
+the ``cpu_baseline`` leg of ``bench.py`` as the checker.  The shipped package never
+imports it.
+
+bfloat16 / float16 data cross this boundary as ``numpy.uint16`` bit patterns; the
+helpers at the bottom convert from and to torch tensors.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle_golden.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile ``golden.c`` with the committed Makefile and return the library path."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-C", _HERE, "liboracle_golden.so"], check=True,
+                   stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+        L.orc_set_threads.argtypes = [i32]
+        L.orc_get_threads.restype = i32
+        L.orc_dynamic_quant.argtypes = [vp, i32, vp, i64, i64, i64, vp, vp]
+        L.orc_int8_gemm.argtypes = [vp, i64, vp, i64, i64, i64, i64, i64, vp]
+        L.orc_quant_matmul_epilogue.argtypes = [vp, vp, vp, i64, vp, i64, i64, vp]
+        L.orc_unpack_int4.argtypes = [vp, i64, vp]
+        L.orc_pack_int4.argtypes = [vp, i64, vp]
+        L.orc_antiquant.argtypes = [vp, vp, vp, i64, i64, vp]
+        L.orc_weight_quant_matmul.argtypes = [vp, i64, vp, i32, i64, i64, vp, vp,
+                                              i64, i64, i64, i64, i32, vp, vp]
+        L.orc_swiglu.argtypes = [vp, i64, i64, vp]
+        L.orc_bf16_to_f32.argtypes = [vp, vp, i64]
+        L.orc_f32_to_bf16.argtypes = [vp, vp, i64]
+        _lib = L
+    return _lib
+
+
+def set_threads(n: int) -> None:
+    lib().orc_set_threads(int(n))
+
+
+def get_threads() -> int:
+    return int(lib().orc_get_threads())
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+# ------------------------------------------------------------------ operators
+
+def dynamic_quant(x_u16: np.ndarray, in_dtype: str = "bf16", smooth_u16: np.ndarray | None = None):
+    """x: uint16 bit patterns [..., cols] -> (y int8 same shape, scale float32 [...])."""
+    x = _c(x_u16, np.uint16)
+    cols = x.shape[-1]
+    rows = x.size // cols if cols else 0
+    y = np.empty(x.shape, dtype=np.int8)
+    scale = np.empty(x.shape[:-1], dtype=np.float32)
+    sm = None if smooth_u16 is None else _c(smooth_u16, np.uint16)
+    if rows and cols:
+        lib().orc_dynamic_quant(_p(x), 0 if in_dtype == "bf16" else 1, _p(sm), rows, cols, cols,
+                                _p(y), _p(scale))
+    elif rows:
+        scale[...] = 0.0
+    return y, scale
+
+
+def int8_gemm(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """a int8 [M,K] (row-major), b int8 [K,N] with arbitrary numpy strides -> int32 [M,N]."""
+    a = _c(a, np.int8)
+    assert b.dtype == np.int8 and a.shape[1] == b.shape[0]
+    M, K = a.shape
+    N = b.shape[1]
+    acc = np.empty((M, N), dtype=np.int32)
+    if M and N:
+        lib().orc_int8_gemm(_p(a), K, _p(b), b.strides[0], b.strides[1], M, N, K, _p(acc))
+    return acc
+
+
+def quant_matmul_epilogue(acc, scale, pertoken_scale=None, bias_u16=None) -> np.ndarray:
+    acc = _c(acc, np.int32)
+    M, N = acc.shape
+    scale = _c(scale, np.float32).reshape(-1)
+    assert scale.size in (1, N)
+    ps = None if pertoken_scale is None else _c(pertoken_scale, np.float32).reshape(-1)
+    if ps is not None:
+        assert ps.size == M
+    bias = None if bias_u16 is None else _c(bias_u16, np.uint16).reshape(-1)
+    out = np.empty((M, N), dtype=np.uint16)
+    if M and N:
+        lib().orc_quant_matmul_epilogue(_p(acc), _p(ps), _p(scale), scale.size, _p(bias), M, N, _p(out))
+    return out
+
+
+def quant_matmul(a, b, scale, pertoken_scale=None, bias_u16=None):
+    """Full W8A8 path -> (out bf16 bit patterns [M,N], acc int32 [M,N])."""
+    acc = int8_gemm(a, b)
+    return quant_matmul_epilogue(acc, scale, pertoken_scale, bias_u16), acc
+
+
+def unpack_int4(packed: np.ndarray) -> np.ndarray:
+    p = _c(packed, np.int32)
+    out = np.empty(p.shape[:-1] + (p.shape[-1] * 8,), dtype=np.int8)
+    lib().orc_unpack_int4(_p(p), p.size, _p(out))
+    return out
+
+
+def pack_int4(vals: np.ndarray) -> np.ndarray:
+    v = _c(vals, np.int8)
+    assert v.shape[-1] % 8 == 0
+    out = np.empty(v.shape[:-1] + (v.shape[-1] // 8,), dtype=np.int32)
+    lib().orc_pack_int4(_p(v), out.size, _p(out))
+    return out
+
+
+def antiquant(w_i8, scale_f32, offset_f32=None) -> np.ndarray:
+    w = _c(w_i8, np.int8)
+    rows, cols = w.shape
+    s = _c(scale_f32, np.float32)
+    o = None if offset_f32 is None else _c(offset_f32, np.float32)
+    out = np.empty((rows, cols), dtype=np.float32)
+    lib().orc_antiquant(_p(w), _p(s), _p(o), rows, cols, _p(out))
+    return out
+
+
+def weight_quant_matmul(x_u16, w, scale_u16, off_u16=None, group_size: int = 0, accum: str = "f32"):
+    """x bf16 bits [M,K]; w int8 [K,N] (any strides) or int32 [K,N/8] (packed int4);
+    scale/off bf16 bits [N] or [G,N].  Returns (out bf16 bits [M,N], unrounded float32 [M,N])."""
+    x = _c(x_u16, np.uint16)
+    M, K = x.shape
+    if w.dtype == np.int8:
+        bits, N = 8, w.shape[1]
+        ldk, ldn = w.strides
+        wbuf = w
+    else:
+        wbuf = _c(w, np.int32)
+        bits, N = 4, wbuf.shape[1] * 8
+        ldk, ldn = 0, 0
+    assert w.shape[0] == K
+    s = _c(scale_u16, np.uint16).reshape(-1, N)
+    o = None if off_u16 is None else _c(off_u16, np.uint16).reshape(-1, N)
+    G = 1 if group_size <= 0 else (K + group_size - 1) // group_size
+    assert s.shape[0] == G, (s.shape, G)
+    out = np.empty((M, N), dtype=np.uint16)
+    outf = np.empty((M, N), dtype=np.float32)
+    if M and N:
+        lib().orc_weight_quant_matmul(_p(x), K, _p(wbuf), bits, ldk, ldn, _p(s), _p(o),
+                                      M, N, K, group_size, 0 if accum == "f32" else 1,
+                                      _p(out), _p(outf))
+    return out, outf
+
+
+def swiglu(x_u16: np.ndarray) -> np.ndarray:
+    x = _c(x_u16, np.uint16)
+    rows, two_half = x.shape
+    assert two_half % 2 == 0
+    out = np.empty((rows, two_half // 2), dtype=np.uint16)
+    if out.size:
+        lib().orc_swiglu(_p(x), rows, two_half // 2, _p(out))
+    return out
+
+
+# ------------------------------------------------------ bit-pattern helpers
+
+def bf16_bits_to_f32(u16: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(u16, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16_bits(f32: np.ndarray) -> np.ndarray:
+    f = _c(f32, np.float32)
+    out = np.empty(f.shape, dtype=np.uint16)
+    lib().orc_f32_to_bf16(_p(f), _p(out), f.size)
+    return out
+
+
+def bits_of(t) -> np.ndarray:
+    """torch bf16/fp16 tensor (any device) -> numpy uint16 bit patterns."""
+    import torch
+    assert t.dtype in (torch.bfloat16, torch.float16)
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def bf16_tensor(u16: np.ndarray):
+    """numpy uint16 bit patterns -> torch bf16 CPU tensor."""
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(u16).view(np.int16).copy()).view(torch.bfloat16)
+
+
+def bf16_ulp_distance(a_u16: np.ndarray, b_u16: np.ndarray) -> np.ndarray:
+    """Distance in bf16 units-in-the-last-place between two bit-pattern arrays
+    (sign-magnitude patterns mapped onto a monotone integer line)."""
+    def key(u):
+        u = u.astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7fff), u & 0x7fff)
+    return np.abs(key(np.asarray(a_u16)) - key(np.asarray(b_u16)))

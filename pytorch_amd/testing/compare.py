@@ -1,0 +1,79 @@
+"""Comparison rules for operator outputs.
+
+``rtol_failures`` / ``assert_rtol_equal`` restate the element rule of
+``TestCase.assertRtolEqual`` (torch_npu/testing/testcase.py:158-227): an element fails
+only if it violates BOTH the absolute and the relative bound, and the comparison as a
+whole fails only if more than ``size * prec`` elements fail.
+
+``bf16_gate`` is the acceptance gate for bf16 outputs of this operator path:
+  * at least 99.9 % of the elements lie within one bf16 unit in the last place of the
+    float32 golden value, and
+  * no element fails the abs-OR-rel rule at 1e-2 (relative error measured against
+    max(|a|, |b|), so values that cancel to ~0 are judged by their absolute error).
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+
+def _np(a):
+    if isinstance(a, torch.Tensor):
+        a = a.detach().cpu()
+        if a.dtype in (torch.bfloat16, torch.float16):
+            a = a.float()
+        a = a.numpy()
+    return np.asarray(a)
+
+
+def rtol_failures(x, y, prec: float = 1e-4) -> int:
+    x = _np(x).astype(np.float64)
+    y = _np(y).astype(np.float64)
+    d = np.abs(x - y)
+    denom = np.maximum(np.abs(x), np.abs(y)) + np.finfo(np.float64).tiny
+    return int(np.count_nonzero((d > prec) & (d / denom > prec)))
+
+
+def assert_rtol_equal(x, y, prec: float = 1e-4, prec16: float = 1e-3) -> None:
+    xa, ya = _np(x), _np(y)
+    if xa.shape != ya.shape:
+        raise AssertionError(f"shape error: {xa.shape} vs {ya.shape}")
+    tx = x.dtype if hasattr(x, "dtype") else xa.dtype
+    ty = y.dtype if hasattr(y, "dtype") else ya.dtype
+    if tx != ty:
+        raise AssertionError(f"dtype error: {tx} vs {ty}")
+    p = prec16 if tx in (torch.float16, torch.bfloat16, np.float16) else prec
+    bad = rtol_failures(xa, ya, p)
+    if bad > xa.size * p:
+        raise AssertionError(f"result error: {bad} of {xa.size} elements outside tolerance {p}")
+
+
+def _bf16_line(t: torch.Tensor) -> np.ndarray:
+    u = t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16).astype(np.int32)
+    return np.where(u & 0x8000, -(u & 0x7fff), u & 0x7fff)
+
+
+def bf16_gate(out_bf16: torch.Tensor, golden_f32: torch.Tensor, *, min_within_1ulp: float = 0.999,
+              max_rel: float = 1e-2) -> dict:
+    """Return the gate statistics; raise AssertionError when the gate is not met.
+
+    ``golden_f32`` is the unrounded float32 golden.  "Within one ulp" is measured on the
+    bf16 number line between ``out`` and the golden rounded to bf16 (distance <= 1)."""
+    assert out_bf16.dtype == torch.bfloat16
+    g32 = golden_f32.detach().cpu().float()
+    o = out_bf16.detach().cpu()
+    dist = np.abs(_bf16_line(o) - _bf16_line(g32.to(torch.bfloat16)))
+    within = float(np.count_nonzero(dist <= 1)) / max(dist.size, 1)
+    exact = float(np.count_nonzero(dist == 0)) / max(dist.size, 1)
+    of = o.float().numpy().astype(np.float64)
+    gf = g32.numpy().astype(np.float64)
+    d = np.abs(of - gf)
+    denom = np.maximum(np.abs(of), np.abs(gf)) + np.finfo(np.float64).tiny
+    bad = int(np.count_nonzero((d > max_rel) & (d / denom > max_rel)))
+    stats = {"within_1ulp": within, "bit_identical": exact, "max_ulp": int(dist.max()) if dist.size else 0,
+             "abs_or_rel_failures": bad, "n": int(dist.size)}
+    if not np.all(np.isfinite(of) == np.isfinite(gf)):
+        raise AssertionError(f"non-finite mismatch: {stats}")
+    if within < min_within_1ulp or bad:
+        raise AssertionError(f"bf16 gate not met: {stats}")
+    return stats

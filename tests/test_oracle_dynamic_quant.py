@@ -1,0 +1,128 @@
+"""Pins oracle.dynamic_quant: library evaluation (torch), exact rational arithmetic,
+hand-typed round-half-even answers and invariants of symmetric per-token quantisation."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from pytorch_amd.testing import workloads
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def test_matches_torch_float32_evaluation(golden):
+    x = workloads.dynamic_quant_input(seed=0, rows=64, cols=4096)
+    y, s = golden.dynamic_quant(_bits(x))
+    xf = x.float()
+    scale = xf.abs().amax(-1) / 127.0
+    yt = torch.round(xf / scale[:, None]).clamp(-127, 127).to(torch.int8)
+    assert np.array_equal(s, scale.numpy())
+    assert np.array_equal(y, yt.numpy())
+    # the sample must actually contain exact .5 ties, or half-even is not exercised
+    q = (xf / scale[:, None])
+    assert int(((q - torch.floor(q)) == 0.5).sum()) > 0
+
+
+def test_fp16_input_matches_torch(golden):
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(16, 1024, generator=g) * 3).to(torch.float16)
+    y, s = golden.dynamic_quant(_bits(x), in_dtype="fp16")
+    xf = x.float()
+    scale = xf.abs().amax(-1) / 127.0
+    assert np.array_equal(s, scale.numpy())
+    assert np.array_equal(y, torch.round(xf / scale[:, None]).clamp(-127, 127).to(torch.int8).numpy())
+
+
+def _rne_f32(fr: Fraction) -> np.float32:
+    """Correctly rounded (nearest-even) binary32 of a positive rational in the normal range."""
+    assert fr > 0
+    e = 0
+    while fr >= 2:
+        fr /= 2
+        e += 1
+    while fr < 1:
+        fr *= 2
+        e -= 1
+    m = fr * (1 << 23)           # in [2^23, 2^24)
+    lo = m.numerator // m.denominator
+    rem = m - lo
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and (lo & 1)):
+        lo += 1
+    return np.float32(float(lo) * 2.0 ** (e - 23))
+
+
+def _rint_half_even(fr: Fraction) -> int:
+    lo = fr.numerator // fr.denominator
+    rem = fr - lo
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and (lo & 1)):
+        lo += 1
+    return lo
+
+
+def test_exact_rational_arithmetic(golden):
+    """scale = RN(amax/127), q = RN(x/scale), y = rint_half_even(q) with every step done in
+    exact rational arithmetic and rounded by hand."""
+    x = workloads.dynamic_quant_input(seed=5, rows=4, cols=512)
+    y, s = golden.dynamic_quant(_bits(x))
+    xf = x.float().numpy()
+    for r in range(xf.shape[0]):
+        amax = Fraction(float(np.abs(xf[r]).max()))
+        sc = _rne_f32(amax / 127)
+        assert sc == s[r]
+        for j in range(xf.shape[1]):
+            v = Fraction(float(xf[r, j]))
+            if v == 0:
+                assert y[r, j] == 0
+                continue
+            q = Fraction(float(_rne_f32(abs(v) / Fraction(float(sc)))))
+            k = _rint_half_even(q)
+            assert y[r, j] == (k if v > 0 else -k), (r, j)
+
+
+def test_known_answers_half_even(golden):
+    # amax = 127 -> scale exactly 1.0, so y = rint_half_even(x)
+    vals = [127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5, 126.5, -126.5, 0.0, 0.25, 0.75, -3.5, 100.5, 101.5]
+    want = [127, 0, 2, 2, 0, -2, -2, 4, 126, -126, 0, 0, 1, -4, 100, 102]
+    x = torch.tensor([vals], dtype=torch.bfloat16)
+    assert x.float().tolist()[0] == vals  # all representable in bf16
+    y, s = golden.dynamic_quant(_bits(x))
+    assert s[0] == np.float32(1.0)
+    assert y[0].tolist() == want
+
+
+def test_zero_row_and_shapes(golden):
+    x = torch.zeros(3, 5, 16, dtype=torch.bfloat16)
+    x[1, 2, 3] = 2.0
+    y, s = golden.dynamic_quant(_bits(x))
+    assert y.shape == (3, 5, 16) and s.shape == (3, 5) and y.dtype == np.int8 and s.dtype == np.float32
+    assert s[0, 0] == 0 and not y[0].any()
+    assert y[1, 2, 3] == 127 and s[1, 2] == np.float32(2.0) / np.float32(127.0)
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_invariants(golden, seed):
+    x = workloads.dynamic_quant_input(seed=seed, rows=128, cols=2048)
+    y, s = golden.dynamic_quant(_bits(x))
+    xf = x.float().numpy()
+    assert (np.abs(y.astype(np.int32)).max(-1) == 127).all()          # every row reaches +-127
+    err = np.abs(y.astype(np.float64) * s[:, None].astype(np.float64) - xf)
+    # half-step reconstruction bound; the quotient itself carries one rounding (|q| <= 127)
+    assert (err <= s[:, None] * (0.5 + 127 * 2.0 ** -23)).all()
+    y2, s2 = golden.dynamic_quant(_bits(-x))                             # odd symmetry
+    assert np.array_equal(s2, s) and np.array_equal(y2, -y)
+    y3, s3 = golden.dynamic_quant(_bits(x * 4))                          # power-of-two scaling is exact
+    assert np.array_equal(y3, y) and np.array_equal(s3, s * 4)
+
+
+def test_smooth_scales(golden):
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(8, 256, generator=g).to(torch.bfloat16)
+    sm = (torch.rand(256, generator=g) + 0.5).to(torch.bfloat16)
+    y, s = golden.dynamic_quant(_bits(x), smooth_u16=_bits(sm))
+    xf = x.float() * sm.float()
+    scale = xf.abs().amax(-1) / 127.0
+    assert np.array_equal(s, scale.numpy())
+    assert np.array_equal(y, torch.round(xf / scale[:, None]).clamp(-127, 127).to(torch.int8).numpy())
