@@ -1,0 +1,127 @@
+/*
+ * C ABI of the MI355X (gfx950) quantized-inference operator library, libmi355_quant.so.
+ *
+ * These entry points are what a torch_npu-style operator adapter binds instead of the
+ * aclnn* functions that the reference resolves from CANN's libopapi.so by dlsym and
+ * calls through typed function pointers returning an int status, 0 = success
+ * (torch_npu/csrc/core/npu/interface/OpInterface.cpp:8-17,28-56;
+ *  torch_npu/csrc/core/npu/register/FunctionLoader.h:86-96).
+ *
+ * Conventions (all entry points)
+ *   - plain pointers and sizes only; every pointer is DEVICE memory owned by the caller;
+ *   - the launcher never allocates, never synchronises and never throws: it validates its
+ *     arguments on the host, enqueues kernels on `stream` (a hipStream_t passed as void*,
+ *     NULL = the default stream) and returns;
+ *   - return value: MI355_OK (0) or a negative mi355_status; mi355_status_string() names it;
+ *   - re-entrant; no mutable global state.
+ *   - strides ("ld*", "*_stride") are in ELEMENTS of the respective array.
+ */
+#ifndef MI355_QUANT_H
+#define MI355_QUANT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum mi355_status {
+    MI355_OK = 0,
+    MI355_ERR_BAD_ARGUMENT = -1,   /* null pointer, negative size, bad enum value          */
+    MI355_ERR_UNSUPPORTED = -2,    /* valid request outside what the kernels implement     */
+    MI355_ERR_ALIGNMENT = -3,      /* pointer / stride alignment the kernels cannot handle */
+    MI355_ERR_WORKSPACE = -4,      /* workspace missing or smaller than *_workspace() says */
+    MI355_ERR_LAUNCH = -5          /* hipGetLastError() != hipSuccess after the launch     */
+} mi355_status;
+
+/* 16-bit floating-point element formats of activations. */
+#define MI355_DTYPE_BF16 0
+#define MI355_DTYPE_FP16 1
+
+/* Output formats of mi355_quant_matmul. */
+#define MI355_OUT_BF16 0
+#define MI355_OUT_INT32 1   /* raw int32 accumulators (+ int32 bias is not applied) */
+
+const char *mi355_status_string(int status);
+
+/* Library/ABI version: major * 1000 + minor. */
+int mi355_quant_abi_version(void);
+
+/*
+ * npu_dynamic_quant, per-token symmetric int8.
+ * Replaces the aclnn DynamicQuant call behind torch_npu.npu_dynamic_quant
+ * (signature and output shapes: test/test_fake_tensor.py:1670-1687,
+ *  torch_npu/onnx/wrapper_onnx_ops.py:740-759).
+ *
+ *   x      [rows, cols] in_dtype, row r starts at x + r * x_row_stride
+ *   smooth NULL, or [cols] in_dtype: x is multiplied by it (in float32) before quantisation
+ *   y      [rows, cols] int8, contiguous
+ *   scale  [rows] float32:  scale = max_j |x| / 127,  y = rint_half_even(x / scale) in [-127, 127]
+ * A row of zeros yields scale 0 and y 0.  rows == 0 or cols == 0 is a no-op.
+ */
+int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth,
+                        int8_t *y, float *scale,
+                        int64_t rows, int64_t cols, int64_t x_row_stride, void *stream);
+
+/*
+ * npu_quant_matmul, W8A8 with int32 accumulation and fused dequantisation.
+ * Replaces the aclnn QuantMatmul call behind torch_npu.npu_quant_matmul
+ * (callers: torch_npu/contrib/module/linear_quant.py:96-112, linear_a8w8_quant.py:87-120;
+ *  shapes/dtypes: test/test_fake_tensor.py:1883-1925).
+ *
+ *   a   int8 [M, K], element (m,k) at a[m*lda + k]
+ *   b   int8 logical [K, N], element (k,n) at b[k*ldb_k + n*ldb_n]; one of ldb_k, ldb_n must be 1
+ *       (ldb_n == 1: contiguous [K,N]; ldb_k == 1: the transposed view of an [N,K] weight)
+ *   pertoken_scale  float32 [M] or NULL;   scale float32 [scale_len], scale_len in {1, N}
+ *   bias            bf16 [N] or NULL (MI355_OUT_BF16 only)
+ *   out_dtype MI355_OUT_BF16:  out[m*ldc+n] = bf16(((float(acc) * pertoken_scale[m]) * scale[n]) + float(bias[n]))
+ *             MI355_OUT_INT32: out[m*ldc+n] = acc (scales and bias are ignored and may be NULL)
+ *   workspace: at least mi355_quant_matmul_workspace(...) bytes (may be NULL when that is 0)
+ */
+size_t mi355_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n);
+
+int mi355_quant_matmul(const int8_t *a, const int8_t *b,
+                       const float *pertoken_scale, const float *scale, int64_t scale_len,
+                       const void *bias_bf16, void *out, int out_dtype,
+                       int64_t M, int64_t N, int64_t K,
+                       int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * npu_weight_quant_batchmatmul, W8A16 per channel and W4A16 per group.
+ * Replaces the aclnn WeightQuantBatchMatmulV2 call behind torch_npu.npu_weight_quant_batchmatmul
+ * (caller: torch_npu/contrib/module/linear_weight_quant.py:98-109; CPU golden:
+ *  test/contrib/test_linear_weight_quant.py:20-28; int4 nibble order:
+ *  test/custom_ops/test_npu_anti_quant.py:12-24).
+ *
+ *   x       bf16 [M, K], element (m,k) at x[m*ldx + k]
+ *   w       w_bits == 8: int8 logical [K, N], element (k,n) at w[k*ldw_k + n*ldw_n], one stride == 1
+ *           w_bits == 4: int32 [K, N/8] contiguous along N (ldw_k = N/8 words, ldw_n ignored);
+ *                        word j of a row holds n = 8j..8j+7, element i in bits [4i, 4i+3], two's complement
+ *   scale   bf16 [G, N] row-major, G = 1 when group_size == 0 else K / group_size
+ *   offset  bf16 [G, N] or NULL
+ *   out[m*ldo+n] = bf16( sum_k float(x[m,k]) * ((float(w[k,n]) + float(offset[g,n])) * float(scale[g,n])) )
+ *   group_size: 0 (per channel) or a multiple of 32 that divides K
+ *   workspace: at least mi355_weight_quant_matmul_workspace(...) bytes
+ */
+size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size);
+
+int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int w_bits,
+                              const void *scale_bf16, const void *offset_bf16, void *out_bf16,
+                              int64_t M, int64_t N, int64_t K, int64_t group_size,
+                              int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo,
+                              void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * npu_swiglu on the last dimension: out = silu(x[:, :half]) * x[:, half:], bf16 arithmetic
+ * (silu rounded to bf16, then the product rounded to bf16).
+ * Formula: torch_npu/_inductor/decomposition.py:186-188.
+ *   x bf16 [rows, 2*half] with row stride ldx; out bf16 [rows, half] contiguous.
+ */
+int mi355_swiglu(const void *x_bf16, void *out_bf16, int64_t rows, int64_t half, int64_t ldx, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_QUANT_H */

@@ -1,0 +1,128 @@
+"""ctypes binding of the C ABI (``include/mi355_quant.h``) for torch tensors on the GPU.
+
+This is the thinnest possible host side: it validates nothing beyond what is needed to
+form the pointer/size arguments, so tests that call it exercise the C entry points
+themselves.  The torch operators (``torch.ops.npu.*``) reach the same entry points from C++.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
+
+EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant",
+           "mi355_quant_matmul_workspace", "mi355_quant_matmul",
+           "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu")
+
+_lib = None
+
+
+class Mi355Error(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is missing: run `python -m pytorch_amd.build` (hipcc, gfx950) first")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i64, i32, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
+        L.mi355_status_string.restype = ctypes.c_char_p
+        L.mi355_status_string.argtypes = [i32]
+        L.mi355_quant_abi_version.restype = i32
+        L.mi355_dynamic_quant.argtypes = [vp, i32, vp, vp, vp, i64, i64, i64, vp]
+        L.mi355_quant_matmul_workspace.restype = sz
+        L.mi355_quant_matmul_workspace.argtypes = [i64, i64, i64, i64, i64]
+        L.mi355_quant_matmul.argtypes = [vp, vp, vp, vp, i64, vp, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
+        L.mi355_weight_quant_matmul_workspace.restype = sz
+        L.mi355_weight_quant_matmul_workspace.argtypes = [i64, i64, i64, i32, i64]
+        L.mi355_weight_quant_matmul.argtypes = [vp, vp, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
+                                                vp, sz, vp]
+        L.mi355_swiglu.argtypes = [vp, vp, i64, i64, i64, vp]
+        _lib = L
+    return _lib
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        raise Mi355Error(f"{what}: {lib().mi355_status_string(status).decode()} (status {status})")
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need_gpu(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise Mi355Error("the C ABI takes device pointers: tensors must live on the GPU")
+
+
+def dynamic_quant(x: torch.Tensor, smooth: torch.Tensor | None = None):
+    _need_gpu(x, smooth)
+    assert x.dtype in (torch.bfloat16, torch.float16)
+    if x.numel() and x.stride(-1) != 1:
+        x = x.contiguous()
+    cols = x.shape[-1]
+    x2 = x.reshape(-1, cols) if x.dim() != 2 else x
+    if x2.dim() == 2 and x2.shape[0] > 1 and x2.stride(0) < cols:
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    scale = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    st = lib().mi355_dynamic_quant(_ptr(x2), 0 if x.dtype == torch.bfloat16 else 1, _ptr(smooth), _ptr(y), _ptr(scale),
+                                   rows, cols, x2.stride(0) if rows > 1 else max(cols, 1), _stream())
+    _check(st, "mi355_dynamic_quant")
+    return y, scale
+
+
+def quant_matmul(x1, x2, scale, pertoken_scale=None, bias=None, out_dtype=torch.bfloat16, workspace=None):
+    """x1 int8 [M,K]; x2 int8 [K,N] with strides (N,1) or (1,K)."""
+    _need_gpu(x1, x2, scale, pertoken_scale, bias)
+    M, K = x1.shape
+    N = x2.shape[1]
+    out = torch.empty((M, N), dtype=out_dtype, device=x1.device)
+    need = lib().mi355_quant_matmul_workspace(M, N, K, x2.stride(0), x2.stride(1))
+    if workspace is None and need:
+        workspace = torch.empty(need, dtype=torch.int8, device=x1.device)
+    st = lib().mi355_quant_matmul(_ptr(x1), _ptr(x2), _ptr(pertoken_scale), _ptr(scale),
+                                  0 if scale is None else scale.numel(), _ptr(bias), _ptr(out),
+                                  0 if out_dtype == torch.bfloat16 else 1, M, N, K, x1.stride(0),
+                                  x2.stride(0), x2.stride(1), out.stride(0), _ptr(workspace),
+                                  0 if workspace is None else workspace.numel(), _stream())
+    _check(st, "mi355_quant_matmul")
+    return out
+
+
+def weight_quant_matmul(x, weight, scale, offset=None, group_size: int = 0):
+    """x bf16 [M,K]; weight int8 [K,N] (strides (N,1) or (1,K)) or int32 [K,N/8]; scale/offset bf16 [N] or [G,N]."""
+    _need_gpu(x, weight, scale, offset)
+    M, K = x.shape
+    if weight.dtype == torch.int32:
+        bits, N = 4, weight.shape[1] * 8
+        ldk, ldn = weight.stride(0), 1
+    else:
+        bits, N = 8, weight.shape[1]
+        ldk, ldn = weight.stride(0), weight.stride(1)
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    st = lib().mi355_weight_quant_matmul(_ptr(x), _ptr(weight), bits, _ptr(scale), _ptr(offset), _ptr(out),
+                                         M, N, K, group_size, x.stride(0), ldk, ldn, out.stride(0), None, 0, _stream())
+    _check(st, "mi355_weight_quant_matmul")
+    return out
+
+
+def swiglu(x):
+    _need_gpu(x)
+    rows, two = x.shape
+    out = torch.empty((rows, two // 2), dtype=torch.bfloat16, device=x.device)
+    _check(lib().mi355_swiglu(_ptr(x), _ptr(out), rows, two // 2, x.stride(0), _stream()), "mi355_swiglu")
+    return out

@@ -1,0 +1,268 @@
+// npu_dynamic_quant for gfx950: per-token symmetric int8 quantisation.
+//
+// One pass over HBM: every row is read once (16-byte loads), kept in registers while the
+// row maximum is reduced, then quantised and written as packed int8 (8-byte stores).
+// Algorithmic traffic per row: cols * 2 bytes in, cols bytes + 4 bytes out.
+//
+// Bit-exactness.  The contract is y = rint_half_even(fl(x / fl(amax / 127))) with IEEE
+// binary32 divisions.  A division per element is ~11 VALU operations; instead the row's
+// reciprocal r = fl(1 / scale) is formed once (correctly rounded division) and each element
+// uses  q0 = x * r;  e = fma(-scale, q0, x);  q = fma(e, r, q0).
+// For x and amax taken from bf16 or fp16 (8 / 11 significant bits) this sequence returns
+// exactly the correctly rounded quotient: verified exhaustively over every pair of
+// significands and every exponent distance that can produce a non-zero result.  Rows whose
+// scale lies outside [2^-60, 2^60], and rows pre-multiplied by smooth scales (arbitrary
+// binary32 significands), take the plain IEEE division instead.
+//
+// Rounding to int8 uses the add-magic-constant trick: q + 1.5 * 2^23 is rounded by the adder
+// to the nearest integer (ties to even, unit = 1 in that binade) and the low byte of the sum's
+// bit pattern is the two's-complement result.  |q| <= 127 * (1 + 2^-23), so no clamp is needed
+// on the fast path.
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int kBlock = 256;
+
+template <bool FP16>
+__device__ __forceinline__ void unpack2(uint32_t u, float &lo, float &hi)
+{
+    if constexpr (FP16) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 v = __builtin_bit_cast(h2, u);
+        lo = (float)v[0];
+        hi = (float)v[1];
+    } else {
+        lo = bf16_lo(u);
+        hi = bf16_hi(u);
+    }
+}
+
+template <bool FP16>
+__device__ __forceinline__ float cvt1(uint16_t h)
+{
+    if constexpr (FP16) {
+        return (float)__builtin_bit_cast(_Float16, h);
+    } else {
+        return bf16_1(h);
+    }
+}
+
+// Maximum over a wavefront of 64 lanes (all lanes receive it).
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        uint32_t o = (uint32_t)__shfl_xor((int)v, off, 64);
+        v = v > o ? v : o;
+    }
+    return v;
+}
+
+__device__ __forceinline__ uint32_t quant_fast(float x, float scale, float r)
+{
+    float q0 = x * r;
+    float e = __builtin_fmaf(-scale, q0, x);
+    float q = __builtin_fmaf(e, r, q0);
+    return __float_as_uint(q + 12582912.0f);
+}
+
+__device__ __forceinline__ uint32_t quant_exact(float x, float scale)
+{
+    float q = x / scale;
+    q = __builtin_rintf(q);
+    q = q > 127.0f ? 127.0f : q;
+    q = q < -127.0f ? -127.0f : q; // NaN falls through both tests and converts to 0
+    return (uint32_t)(int)q;
+}
+
+__device__ __forceinline__ uint32_t pack4(uint32_t a, uint32_t b, uint32_t c, uint32_t d)
+{
+    // low bytes of a, b, c, d -> one dword (a lowest)
+    uint32_t ab = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);
+    uint32_t cd = __builtin_amdgcn_perm(d, c, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
+}
+
+// TPR threads cooperate on one row (64 = one wavefront, no barrier; 256 = whole block);
+// each thread holds ITERS vectors of 8 elements.
+template <int TPR, int ITERS, bool FP16>
+__global__ __launch_bounds__(kBlock) void dq_rows_kernel(const uint16_t *__restrict__ x, int8_t *__restrict__ y,
+                                                         float *__restrict__ scale_out, int64_t rows, int cols,
+                                                         int64_t row_stride)
+{
+    constexpr int RPB = kBlock / TPR;
+    const int t = threadIdx.x % TPR;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+    const bool live = row < rows;
+    const int nvec = cols >> 3;
+    const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + (live ? row : 0) * row_stride);
+
+    u32x4 v[ITERS];
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const int idx = t + i * TPR;
+        if (live && idx < nvec) {
+            v[i] = __builtin_nontemporal_load(xr + idx);
+        } else {
+            v[i] = u32x4{0, 0, 0, 0};
+        }
+        // |x| compared on the bit patterns: two 16-bit lanes per dword
+        typedef uint16_t us2 __attribute__((ext_vector_type(2)));
+        us2 mm = __builtin_bit_cast(us2, m);
+        mm = __builtin_elementwise_max(mm, __builtin_bit_cast(us2, v[i].x & 0x7fff7fffu));
+        mm = __builtin_elementwise_max(mm, __builtin_bit_cast(us2, v[i].y & 0x7fff7fffu));
+        mm = __builtin_elementwise_max(mm, __builtin_bit_cast(us2, v[i].z & 0x7fff7fffu));
+        mm = __builtin_elementwise_max(mm, __builtin_bit_cast(us2, v[i].w & 0x7fff7fffu));
+        m = __builtin_bit_cast(uint32_t, mm);
+    }
+    uint32_t m16 = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+    m16 = wave_max_u32(m16);
+    if constexpr (TPR > 64) {
+        __shared__ uint32_t part[kBlock / 64];
+        if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m16;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < kBlock / 64; w++) m16 = part[w] > m16 ? part[w] : m16;
+    }
+    if (!live) return;
+
+    const float amax = cvt1<FP16>((uint16_t)m16);
+    const float scale = amax / 127.0f;
+    if (t == 0) scale_out[row] = scale;
+    u32x2 *yr = reinterpret_cast<u32x2 *>(y + row * (int64_t)cols);
+
+    if (!(amax > 0.0f)) { // zero row (or NaN maximum): codes are all zero
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) {
+            const int idx = t + i * TPR;
+            if (idx < nvec) yr[idx] = u32x2{0, 0};
+        }
+        return;
+    }
+    const bool fast = scale >= 0x1p-60f && scale <= 0x1p60f;
+    if (fast) {
+        const float r = 1.0f / scale;
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) {
+            const int idx = t + i * TPR;
+            float f0, f1, f2, f3, f4, f5, f6, f7;
+            unpack2<FP16>(v[i].x, f0, f1);
+            unpack2<FP16>(v[i].y, f2, f3);
+            unpack2<FP16>(v[i].z, f4, f5);
+            unpack2<FP16>(v[i].w, f6, f7);
+            u32x2 o;
+            o.x = pack4(quant_fast(f0, scale, r), quant_fast(f1, scale, r), quant_fast(f2, scale, r),
+                        quant_fast(f3, scale, r));
+            o.y = pack4(quant_fast(f4, scale, r), quant_fast(f5, scale, r), quant_fast(f6, scale, r),
+                        quant_fast(f7, scale, r));
+            if (idx < nvec) __builtin_nontemporal_store(o, yr + idx);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) {
+            const int idx = t + i * TPR;
+            float f0, f1, f2, f3, f4, f5, f6, f7;
+            unpack2<FP16>(v[i].x, f0, f1);
+            unpack2<FP16>(v[i].y, f2, f3);
+            unpack2<FP16>(v[i].z, f4, f5);
+            unpack2<FP16>(v[i].w, f6, f7);
+            u32x2 o;
+            o.x = pack4(quant_exact(f0, scale), quant_exact(f1, scale), quant_exact(f2, scale),
+                        quant_exact(f3, scale));
+            o.y = pack4(quant_exact(f4, scale), quant_exact(f5, scale), quant_exact(f6, scale),
+                        quant_exact(f7, scale));
+            if (idx < nvec) yr[idx] = o;
+        }
+    }
+}
+
+// Any shape, stride and alignment; optional smooth scales.  One block per row, two passes
+// over the row (the second one hits in cache), IEEE division per element.
+template <bool FP16>
+__global__ __launch_bounds__(kBlock) void dq_generic_kernel(const uint16_t *__restrict__ x,
+                                                            const uint16_t *__restrict__ smooth,
+                                                            int8_t *__restrict__ y, float *__restrict__ scale_out,
+                                                            int64_t cols, int64_t row_stride)
+{
+    const int64_t row = blockIdx.x;
+    const uint16_t *xr = x + row * row_stride;
+    float amax = 0.0f;
+    for (int64_t j = threadIdx.x; j < cols; j += kBlock) {
+        float v = cvt1<FP16>(xr[j]);
+        if (smooth) v = v * cvt1<FP16>(smooth[j]);
+        amax = fmaxf(amax, fabsf(v));
+    }
+    uint32_t mb = wave_max_u32(__float_as_uint(amax)); // non-negative floats order like their bit patterns
+    __shared__ uint32_t part[kBlock / 64];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = mb;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; w++) mb = part[w] > mb ? part[w] : mb;
+    amax = __uint_as_float(mb);
+    const float scale = amax / 127.0f;
+    if (threadIdx.x == 0) scale_out[row] = scale;
+    int8_t *yr = y + row * cols;
+    const bool zero = !(amax > 0.0f);
+    for (int64_t j = threadIdx.x; j < cols; j += kBlock) {
+        float v = cvt1<FP16>(xr[j]);
+        if (smooth) v = v * cvt1<FP16>(smooth[j]);
+        yr[j] = zero ? (int8_t)0 : (int8_t)quant_exact(v, scale);
+    }
+}
+
+template <int TPR, int ITERS>
+void launch_rows(bool fp16, const uint16_t *x, int8_t *y, float *scale, int64_t rows, int cols, int64_t stride,
+                 hipStream_t s)
+{
+    constexpr int RPB = kBlock / TPR;
+    const unsigned grid = (unsigned)((rows + RPB - 1) / RPB);
+    if (fp16)
+        hipLaunchKernelGGL((dq_rows_kernel<TPR, ITERS, true>), dim3(grid), dim3(kBlock), 0, s, x, y, scale, rows, cols,
+                           stride);
+    else
+        hipLaunchKernelGGL((dq_rows_kernel<TPR, ITERS, false>), dim3(grid), dim3(kBlock), 0, s, x, y, scale, rows,
+                           cols, stride);
+}
+
+} // namespace
+} // namespace mi355
+
+extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth, int8_t *y, float *scale,
+                                   int64_t rows, int64_t cols, int64_t x_row_stride, void *stream)
+{
+    using namespace mi355;
+    if (rows < 0 || cols < 0) return MI355_ERR_BAD_ARGUMENT;
+    if (in_dtype != MI355_DTYPE_BF16 && in_dtype != MI355_DTYPE_FP16) return MI355_ERR_BAD_ARGUMENT;
+    if (rows == 0) return MI355_OK;
+    if (!scale) return MI355_ERR_BAD_ARGUMENT;
+    if (cols > 0 && (!x || !y || x_row_stride < cols)) return MI355_ERR_BAD_ARGUMENT;
+    if (rows > 0x7fffffff) return MI355_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool fp16 = in_dtype == MI355_DTYPE_FP16;
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+
+    const int64_t nvec = cols >> 3;
+    const bool vec_ok = !smooth && cols > 0 && (cols & 7) == 0 && (x_row_stride & 7) == 0 && aligned(x, 16) &&
+                        aligned(y, 8) && nvec <= kBlock * 8;
+    if (vec_ok) {
+        const int c = (int)cols;
+        if (nvec <= 64 * 1) launch_rows<64, 1>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+        else if (nvec <= 64 * 2) launch_rows<64, 2>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+        else if (nvec <= 64 * 4) launch_rows<64, 4>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+        else if (nvec <= 256 * 2) launch_rows<256, 2>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+        else if (nvec <= 256 * 4) launch_rows<256, 4>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+        else launch_rows<256, 8>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+    } else {
+        const uint16_t *sm = static_cast<const uint16_t *>(smooth);
+        if (fp16)
+            hipLaunchKernelGGL((dq_generic_kernel<true>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale,
+                               cols, x_row_stride);
+        else
+            hipLaunchKernelGGL((dq_generic_kernel<false>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale,
+                               cols, x_row_stride);
+    }
+    return check_launch();
+}

@@ -1,0 +1,370 @@
+// npu_quant_matmul for gfx950: int8 x int8 -> int32 on the MFMA units with the dequantising
+// epilogue fused (per-token scale, per-channel scale, bias, bf16 rounding).
+//
+// Data layout.  A is [M,K] row-major int8.  The B operand is consumed K-major ("[N,K]", the
+// storage of an nn.Linear-style weight whose transposed view the callers pass); a contiguous
+// [K,N] weight is first transposed into the caller's workspace.
+//
+// Kernel.  A workgroup of 8 wavefronts (two per SIMD, arranged WGM x WGN) owns a BM x BN tile of
+// the output.  K is walked in steps of BK = 128 bytes.  Global memory -> LDS goes through
+// the direct-to-LDS load (16 bytes per lane, no register staging); the 16-byte chunks of a row
+// are XOR-swizzled with the row number (applied on the global-address side, because the LDS
+// side of a direct load is fixed at lane * 16) so that the 16 rows x 16 bytes a wavefront
+// reads per MFMA operand spread over all banks.  Every wavefront keeps WTM x WTN
+// accumulator tiles of v_mfma_i32_16x16x64_i8 in registers.
+//
+// The MFMA is issued with the weight fragment as the first operand, so each lane ends up with
+// four consecutive output columns of one row: the epilogue then needs one per-token scale and
+// four consecutive per-channel scales per accumulator quad and stores 8 bytes per lane.
+//
+// Exactness.  Accumulation is integer and therefore independent of the tiling.  The epilogue
+// evaluates ((float(acc) * pertoken[m]) * scale[n]) + bias[n] with separately rounded binary32
+// operations (contraction is disabled for this library) and rounds once to bf16.
+#include "common.h"
+#include <stdio.h>
+#include <stdlib.h>
+
+namespace mi355 {
+namespace {
+
+constexpr int BK = 128;          // bytes (= int8 elements) of K per LDS stage
+constexpr int STAGES = 2;
+
+typedef int32_t i32x4v __attribute__((ext_vector_type(4)));
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+// Raw buffer descriptor (stride 0, 32-bit data format): loads beyond `bytes` return zero.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+
+struct QmmArgs {
+    const int8_t *a;
+    const int8_t *bt;          // [N, K] K-major
+    const float *pertoken;     // [M] or null
+    const float *scale;        // [scale_len]
+    const uint16_t *bias;      // bf16 [N] or null
+    void *out;
+    int64_t lda, ldbt, ldc;
+    int M, N, K;
+    int scale_len;
+    int out_i32;
+    int tiles_m, tiles_n, tiles_per_xcd;
+};
+
+// WGM x WGN wavefronts per workgroup, each owning (16*WTM) x (16*WTN) of the output tile.
+template <int WGM, int WGN, int WTM, int WTN>
+__global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
+{
+    constexpr int NW = WGM * WGN;
+    constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
+    constexpr int UNITS_A = BM / 8, UNITS_B = BN / 8;        // unit = 8 rows x 128 B = one wavefront-wide load
+    constexpr int STAGE_BYTES = (BM + BN) * BK;
+    static_assert(UNITS_A % NW == 0, "A units must divide evenly over the wavefronts");
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+    // XCD-aware rasterisation: workgroups are dealt round-robin to the 8 XCDs, each of which has
+    // a private L2; give every XCD a contiguous run of tiles, M fastest, so its workgroups
+    // share weight columns.
+    const int xcd = blockIdx.x & 7;
+    const int tile = xcd * p.tiles_per_xcd + (blockIdx.x >> 3);
+    if (tile >= p.tiles_m * p.tiles_n) return;
+    const int m0 = (tile % p.tiles_m) * BM;
+    const int n0 = (tile / p.tiles_m) * BN;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+
+    // Global -> LDS addressing.  Lane l of a unit fills LDS slot l (16 B): row l/8, chunk slot l%8,
+    // which must hold global chunk (l%8) ^ (l/8) of that row (XOR swizzle).
+    const int rows_a = min(BM, p.M - m0), rows_b = min(BN, p.N - n0);
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        make_rsrc(p.a + (int64_t)m0 * p.lda, (uint32_t)((int64_t)(rows_a - 1) * p.lda + p.K));
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        make_rsrc(p.bt + (int64_t)n0 * p.ldbt, (uint32_t)((int64_t)(rows_b - 1) * p.ldbt + p.K));
+    const int rr = lane >> 3;
+    const int gchunk = ((lane & 7) ^ rr) * 16;
+    const uint32_t voff_a = (uint32_t)(rr * (int)p.lda + gchunk);
+    const uint32_t voff_b = (uint32_t)(rr * (int)p.ldbt + gchunk);
+    const uint32_t unit_stride_a = 8u * (uint32_t)p.lda, unit_stride_b = 8u * (uint32_t)p.ldbt;
+
+    auto issue_stage = [&](int k0, char *stage) {
+#pragma unroll
+        for (int i = 0; i < UNITS_A / NW; i++) {
+            const int u = i * NW + wave;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void *)(stage + u * 1024), 16, voff_a,
+                                                     (uint32_t)u * unit_stride_a + k0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < (UNITS_B + NW - 1) / NW; i++) {
+            const int u = i * NW + wave;
+            if (UNITS_B % NW == 0 || u < UNITS_B) // wave-uniform
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void *)(stage + (UNITS_A + u) * 1024), 16, voff_b,
+                                                         (uint32_t)u * unit_stride_b + k0, 0, 0);
+        }
+    };
+
+    i32x4v acc[WTM][WTN];
+#pragma unroll
+    for (int i = 0; i < WTM; i++)
+#pragma unroll
+        for (int j = 0; j < WTN; j++) acc[i][j] = i32x4v{0, 0, 0, 0};
+
+    const int KT = p.K / BK;
+    issue_stage(0, lds);
+
+    // LDS read addressing: lane reads row (lane % 16) of a 16-row tile, 16-byte chunk (ks*4 + lane/16),
+    // stored at slot chunk ^ (row % 8).  For ks = 1 the slot is the ks = 0 slot with bit 2 flipped.
+    const int frow = lane & 15;
+    const int sw0 = ((lane >> 4) ^ (frow & 7)) * 16;
+    const int a_off = (wm * WTM * 16 + frow) * BK;
+    const int b_off = (BM + wn * WTN * 16 + frow) * BK;
+
+    for (int kt = 0; kt < KT; kt++) {
+        const char *cur = lds + (kt & 1) * STAGE_BYTES;
+        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the loads of this stage have landed
+        __syncthreads();
+        if (kt + 1 < KT) issue_stage((kt + 1) * BK, lds + ((kt + 1) & 1) * STAGE_BYTES);
+#pragma unroll
+        for (int ks = 0; ks < BK / 64; ks++) {
+            const int sw = sw0 ^ (ks * 64);
+            i32x4v af[WTM], bf[WTN];
+#pragma unroll
+            for (int i = 0; i < WTM; i++) af[i] = *reinterpret_cast<const i32x4v *>(cur + a_off + i * 16 * BK + sw);
+#pragma unroll
+            for (int j = 0; j < WTN; j++) bf[j] = *reinterpret_cast<const i32x4v *>(cur + b_off + j * 16 * BK + sw);
+#pragma unroll
+            for (int i = 0; i < WTM; i++)
+#pragma unroll
+                for (int j = 0; j < WTN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // Epilogue.  The weight fragment was the first MFMA operand, so
+    // acc[i][j][r] = C[m = tile row (lane % 16)][n = 4 * (lane / 16) + r].
+    const int mrow = lane & 15;
+    const int nquad = (lane >> 4) * 4;
+#pragma unroll
+    for (int i = 0; i < WTM; i++) {
+        const int m = m0 + (wm * WTM + i) * 16 + mrow;
+        if (m >= p.M) continue;
+        const float ps = p.pertoken ? p.pertoken[m] : 1.0f;
+#pragma unroll
+        for (int j = 0; j < WTN; j++) {
+            const int n = n0 + (wn * WTN + j) * 16 + nquad;
+            if (n >= p.N) continue;
+            const i32x4v c = acc[i][j];
+            if (p.out_i32) {
+                int32_t *o = static_cast<int32_t *>(p.out) + (int64_t)m * p.ldc + n;
+                if (n + 3 < p.N && (p.ldc & 3) == 0) {
+                    *reinterpret_cast<i32x4v *>(o) = c;
+                } else {
+                    for (int r = 0; r < 4; r++)
+                        if (n + r < p.N) o[r] = c[r];
+                }
+                continue;
+            }
+            float f[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int nn = n + r < p.N ? n + r : p.N - 1;
+                float v = (float)c[r];
+                if (p.pertoken) v = v * ps;
+                v = v * p.scale[p.scale_len == 1 ? 0 : nn];
+                if (p.bias) v = v + bf16_1(p.bias[nn]);
+                f[r] = v;
+            }
+            uint16_t *o = static_cast<uint16_t *>(p.out) + (int64_t)m * p.ldc + n;
+            if (n + 3 < p.N && (p.ldc & 3) == 0) {
+                u32x2 pk;
+                pk.x = pack_bf16x2(f[0], f[1]);
+                pk.y = pack_bf16x2(f[2], f[3]);
+                *reinterpret_cast<u32x2 *>(o) = pk;
+            } else {
+                for (int r = 0; r < 4; r++)
+                    if (n + r < p.N) o[r] = f32_to_bf16(f[r]);
+            }
+        }
+    }
+}
+
+// Correct for every shape, stride and alignment; used when the tiled kernel's preconditions
+// (K multiple of 128, 16-byte aligned rows) do not hold.  One thread per output element.
+__global__ __launch_bounds__(256) void qmm_generic_kernel(const int8_t *__restrict__ a, const int8_t *__restrict__ b,
+                                                          const float *__restrict__ pertoken,
+                                                          const float *__restrict__ scale, int scale_len,
+                                                          const uint16_t *__restrict__ bias, void *out, int out_i32,
+                                                          int M, int N, int K, int64_t lda, int64_t ldb_k,
+                                                          int64_t ldb_n, int64_t ldc)
+{
+    const int n = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int m = blockIdx.y * 16 + (threadIdx.x >> 4);
+    if (m >= M || n >= N) return;
+    int32_t s = 0;
+    for (int k = 0; k < K; k++) s += (int32_t)a[(int64_t)m * lda + k] * (int32_t)b[(int64_t)k * ldb_k + (int64_t)n * ldb_n];
+    if (out_i32) {
+        static_cast<int32_t *>(out)[(int64_t)m * ldc + n] = s;
+        return;
+    }
+    float v = (float)s;
+    if (pertoken) v = v * pertoken[m];
+    v = v * scale[scale_len == 1 ? 0 : n];
+    if (bias) v = v + bf16_1(bias[n]);
+    static_cast<uint16_t *>(out)[(int64_t)m * ldc + n] = f32_to_bf16(v);
+}
+
+// [K,N] contiguous -> [N,K] contiguous, 64x64 byte tiles through LDS.
+__global__ __launch_bounds__(256) void transpose_i8_kernel(const int8_t *__restrict__ src, int8_t *__restrict__ dst,
+                                                           int K, int N, int64_t ld_src)
+{
+    __shared__ int8_t tile[64][64 + 4];
+    const int k0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4) {
+        const int k = k0 + r, n = n0 + tx;
+        tile[r][tx] = (k < K && n < N) ? src[(int64_t)k * ld_src + n] : (int8_t)0;
+    }
+    __syncthreads();
+    for (int r = ty; r < 64; r += 4) {
+        const int n = n0 + r, k = k0 + tx;
+        if (n < N && k < K) dst[(int64_t)n * K + k] = tile[tx][r];
+    }
+}
+
+template <int WGM, int WGN, int WTM, int WTN>
+int launch_qmm(QmmArgs p, hipStream_t s)
+{
+    constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
+    constexpr size_t lds_bytes = (size_t)STAGES * (BM + BN) * BK;
+    static_assert(lds_bytes <= 160 * 1024, "LDS budget");
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const int tiles = p.tiles_m * p.tiles_n;
+    p.tiles_per_xcd = (tiles + 7) / 8;
+    auto kern = qmm_kernel<WGM, WGN, WTM, WTN>;
+    static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(8 * p.tiles_per_xcd), dim3(WGM * WGN * 64), lds_bytes, s, p);
+    return check_launch();
+}
+
+// Tile shapes (rows x columns of the workgroup tile) the library instantiates.
+struct TileChoice {
+    int bm, bn;
+};
+constexpr TileChoice kTiles[] = {{256, 256}, {256, 224}, {256, 192}, {128, 352}, {128, 320}, {128, 256},
+                                 {128, 192}, {128, 128}, {64, 256},  {64, 128}};
+
+// Pick the tile shape that minimises (waves of workgroups over the 256 CUs) x (time per tile).
+TileChoice choose_tile(int M, int N)
+{
+    if (const char *e = getenv("MI355_QMM_TILE")) { // debugging aid: "BMxBN"
+        int bm = 0, bn = 0;
+        if (sscanf(e, "%dx%d", &bm, &bn) == 2)
+            for (const TileChoice &c : kTiles)
+                if (c.bm == bm && c.bn == bn) return c;
+    }
+    TileChoice best = kTiles[0];
+    double best_cost = 1e300;
+    for (const TileChoice &c : kTiles) {
+        const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+        const long waves = (tiles + 255) / 256;
+        // per-tile time ~ MFMA work, inflated when the tile is small (LDS/L2 bytes per MFMA grow)
+        const double intensity = (double)c.bm * c.bn / (c.bm + c.bn);
+        const double eff = intensity / (intensity + 48.0);
+        const double cost = (double)waves * c.bm * c.bn / eff;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = c;
+        }
+    }
+    return best;
+}
+
+} // namespace
+} // namespace mi355
+
+extern "C" size_t mi355_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n)
+{
+    (void)M;
+    (void)ldb_k;
+    if (N <= 0 || K <= 0) return 0;
+    // a contiguous [K,N] weight is transposed into the workspace
+    return ldb_n == 1 && K > 1 ? (size_t)N * (size_t)K : 0;
+}
+
+extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale,
+                                  int64_t scale_len, const void *bias_bf16, void *out, int out_dtype, int64_t M,
+                                  int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                                  void *workspace, size_t workspace_bytes, void *stream)
+{
+    using namespace mi355;
+    if (M < 0 || N < 0 || K < 0) return MI355_ERR_BAD_ARGUMENT;
+    if (out_dtype != MI355_OUT_BF16 && out_dtype != MI355_OUT_INT32) return MI355_ERR_BAD_ARGUMENT;
+    if (M == 0 || N == 0) return MI355_OK;
+    if (!out || ldc < N) return MI355_ERR_BAD_ARGUMENT;
+    if (K > 0 && (!a || !b || lda < K)) return MI355_ERR_BAD_ARGUMENT;
+    if (ldb_k != 1 && ldb_n != 1) return MI355_ERR_UNSUPPORTED;
+    if (out_dtype == MI355_OUT_BF16 && (!scale || (scale_len != 1 && scale_len != N))) return MI355_ERR_BAD_ARGUMENT;
+    if (out_dtype == MI355_OUT_INT32 && bias_bf16) return MI355_ERR_UNSUPPORTED;
+    if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return MI355_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int out_i32 = out_dtype == MI355_OUT_INT32;
+
+    const int8_t *bt = b;
+    int64_t ldbt = ldb_n;
+    bool tiled = K >= BK && K % BK == 0 && (lda & 15) == 0 && aligned(a, 16);
+    if (tiled && ldb_k != 1) {
+        // contiguous [K,N]: transpose once into the workspace
+        const size_t need = (size_t)N * (size_t)K;
+        if (!workspace || workspace_bytes < need) return MI355_ERR_WORKSPACE;
+        if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+        hipLaunchKernelGGL(transpose_i8_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64)), dim3(256), 0,
+                           s, b, static_cast<int8_t *>(workspace), (int)K, (int)N, ldb_k);
+        bt = static_cast<const int8_t *>(workspace);
+        ldbt = K;
+    }
+    tiled = tiled && (ldbt & 15) == 0 && aligned(bt, 16);
+    if (!tiled) {
+        hipLaunchKernelGGL(qmm_generic_kernel, dim3((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16)), dim3(256), 0, s,
+                           a, b, pertoken_scale, scale, (int)scale_len, static_cast<const uint16_t *>(bias_bf16), out,
+                           out_i32, (int)M, (int)N, (int)K, lda, ldb_k, ldb_n, ldc);
+        return check_launch();
+    }
+
+    QmmArgs p;
+    p.a = a;
+    p.bt = bt;
+    p.pertoken = out_i32 ? nullptr : pertoken_scale;
+    p.scale = scale;
+    p.bias = static_cast<const uint16_t *>(bias_bf16);
+    p.out = out;
+    p.lda = lda;
+    p.ldbt = ldbt;
+    p.ldc = ldc;
+    p.M = (int)M;
+    p.N = (int)N;
+    p.K = (int)K;
+    p.scale_len = (int)scale_len;
+    p.out_i32 = out_i32;
+    const TileChoice c = choose_tile(p.M, p.N);
+#define MI355_QMM_CASE(bm_, bn_, wgm_, wgn_)  \
+    if (c.bm == bm_ && c.bn == bn_) return launch_qmm<wgm_, wgn_, bm_ / (16 * wgm_), bn_ / (16 * wgn_)>(p, s);
+    MI355_QMM_CASE(256, 256, 2, 4)
+    MI355_QMM_CASE(256, 224, 4, 2)
+    MI355_QMM_CASE(256, 192, 2, 4)
+    MI355_QMM_CASE(128, 352, 4, 2)
+    MI355_QMM_CASE(128, 320, 2, 4)
+    MI355_QMM_CASE(128, 256, 2, 4)
+    MI355_QMM_CASE(128, 192, 2, 4)
+    MI355_QMM_CASE(128, 128, 2, 4)
+    MI355_QMM_CASE(64, 256, 1, 8)
+    MI355_QMM_CASE(64, 128, 1, 8)
+#undef MI355_QMM_CASE
+    return MI355_ERR_UNSUPPORTED;
+}

@@ -1,0 +1,232 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI, against the CPU oracle on
+the same seeded inputs.  int8 codes, float32 row scales and int32 accumulators must be
+bit-exact; bf16 outputs must pass the bf16 gate (>= 99.9 % within one bf16 ulp of the
+float32 golden, no element outside 1e-2 abs-or-rel)."""
+import numpy as np
+import pytest
+import torch
+
+from pytorch_amd.testing import workloads, bf16_gate
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from pytorch_amd import _capi
+    _capi.lib()
+    return _capi
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+# ------------------------------------------------------------------ dynamic_quant
+
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (64, 14336), (7, 512), (33, 1024), (5, 8), (3, 40), (2, 16384),
+                                       (2, 20000), (9, 100), (1, 1)])
+def test_dynamic_quant_bit_exact(capi, golden, rows, cols):
+    x = workloads.dynamic_quant_input(seed=rows + cols, rows=rows, cols=cols)
+    y, s = capi.dynamic_quant(x.cuda())
+    yg, sg = golden.dynamic_quant(_bits(x))
+    assert np.array_equal(s.cpu().numpy(), sg)
+    assert np.array_equal(y.cpu().numpy(), yg)
+
+
+def test_dynamic_quant_fp16_and_strided(capi, golden):
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(40, 2048, generator=g) * 5).to(torch.float16)
+    y, s = capi.dynamic_quant(x.cuda())
+    yg, sg = golden.dynamic_quant(_bits(x), in_dtype="fp16")
+    assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(y.cpu().numpy(), yg)
+    xb = workloads.dynamic_quant_input(seed=1, rows=16, cols=4096)
+    view = xb.cuda()[:, :1024]                      # row stride 4096, 1024 columns
+    y, s = capi.dynamic_quant(view)
+    yg, sg = golden.dynamic_quant(_bits(xb[:, :1024]))
+    assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(y.cpu().numpy(), yg)
+
+
+def test_dynamic_quant_exhaustive_significands(capi, golden):
+    """Every bf16 significand of the row maximum x every bf16 value that can round to a non-zero
+    code, at several exponents including ones outside the fast-path range."""
+    rows = []
+    for e in (-100, -62, -30, -1, 0, 7, 40, 63, 100):
+        for ma in range(128):
+            amax = np.float32((1 + ma / 128.0) * 2.0 ** e)
+            vals = [amax]
+            for de in range(0, 10):
+                for mx in range(128):
+                    v = np.float32((1 + mx / 128.0) * 2.0 ** (e - de))
+                    if v <= amax:
+                        vals.append(v)
+            rows.append(np.array(vals, np.float32))
+    width = max(len(r) for r in rows)
+    width = (width + 7) // 8 * 8
+    mat = np.zeros((len(rows), width), np.float32)
+    for i, r in enumerate(rows):
+        mat[i, :len(r)] = r
+        mat[i, 1:len(r):2] *= -1
+    x = torch.from_numpy(mat).to(torch.bfloat16)
+    assert torch.equal(x.float(), torch.from_numpy(mat))
+    y, s = capi.dynamic_quant(x.cuda())
+    yg, sg = golden.dynamic_quant(_bits(x))
+    assert np.array_equal(s.cpu().numpy(), sg)
+    assert np.array_equal(y.cpu().numpy(), yg)
+
+
+def test_dynamic_quant_edge_cases(capi, golden):
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    x[1, 3] = -3.0
+    x[2] = torch.tensor([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5] * 8)
+    y, s = capi.dynamic_quant(x.cuda())
+    assert s.cpu().tolist()[0] == 0.0 and not y[0].any()
+    assert y[1, 3].item() == -127
+    assert y[2, :8].cpu().tolist() == [127, 0, 2, 2, 0, -2, -2, 4]
+    yg, sg = golden.dynamic_quant(_bits(x))
+    assert np.array_equal(y.cpu().numpy(), yg) and np.array_equal(s.cpu().numpy(), sg)
+    e = torch.empty(0, 128, dtype=torch.bfloat16, device="cuda")
+    y, s = capi.dynamic_quant(e)
+    assert y.shape == (0, 128) and s.shape == (0,)
+    x3 = workloads.dynamic_quant_input(seed=3, rows=24, cols=256).reshape(2, 12, 256)
+    y, s = capi.dynamic_quant(x3.cuda())
+    assert y.shape == (2, 12, 256) and s.shape == (2, 12)
+
+
+def test_dynamic_quant_smooth(capi, golden):
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(8, 512, generator=g).to(torch.bfloat16)
+    sm = (torch.rand(512, generator=g) + 0.5).to(torch.bfloat16)
+    y, s = capi.dynamic_quant(x.cuda(), sm.cuda())
+    yg, sg = golden.dynamic_quant(_bits(x), smooth_u16=_bits(sm))
+    assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(y.cpu().numpy(), yg)
+
+
+# ------------------------------------------------------------------ quant_matmul
+
+QMM_SHAPES = [(1024, 4096, 1024), (256, 512, 352), (64, 4096, 512), (100, 256, 200), (1, 128, 16), (300, 1024, 1000),
+              (17, 96, 33), (2048, 256, 4096)]
+
+
+@pytest.mark.parametrize("M,K,N", QMM_SHAPES)
+@pytest.mark.parametrize("weight_nk", [True, False])
+def test_quant_matmul_accumulators_bit_exact(capi, golden, M, K, N, weight_nk):
+    d = workloads.quant_matmul_inputs(seed=M + N, M=M, K=K, N=N, weight_nk=weight_nk)
+    acc = capi.quant_matmul(d["x1"].cuda(), d["x2"].cuda(), None, out_dtype=torch.int32)
+    want = golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy())
+    assert np.array_equal(acc.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("M,K,N", QMM_SHAPES[:6])
+@pytest.mark.parametrize("bias", [True, False])
+def test_quant_matmul_bf16(capi, golden, M, K, N, bias):
+    d = workloads.quant_matmul_inputs(seed=7 + M, M=M, K=K, N=N, weight_nk=True, bias=bias)
+    out = capi.quant_matmul(d["x1"].cuda(), d["x2"].cuda(), d["scale"].cuda(), d["pertoken_scale"].cuda(),
+                            None if not bias else d["bias"].cuda())
+    want, _ = golden.quant_matmul(d["x1"].numpy(), d["x2"].numpy(), d["scale"].numpy(), d["pertoken_scale"].numpy(),
+                                  None if not bias else _bits(d["bias"]))
+    assert np.array_equal(_bits(out), want)      # same operation order => bit-identical bf16
+
+
+def test_quant_matmul_extreme_accumulators(capi, golden):
+    M, K, N = 64, 4096, 64
+    a = torch.full((M, K), 127, dtype=torch.int8)
+    b = torch.full((N, K), -127, dtype=torch.int8).t()
+    acc = capi.quant_matmul(a.cuda(), b.cuda(), None, out_dtype=torch.int32)
+    assert (acc == -K * 16129).all()
+    one = torch.ones(N, device="cuda")
+    out = capi.quant_matmul(a.cuda(), b.cuda(), one, None, None)
+    assert (out.float() == torch.tensor(float(-K * 16129)).to(torch.bfloat16).float()).all()
+    half = capi.quant_matmul(a.cuda(), b.cuda(), torch.tensor([0.5], device="cuda"), None, None)
+    want, _ = golden.quant_matmul(a.numpy(), b.numpy(), np.array([0.5], np.float32))
+    assert np.array_equal(_bits(half), want)
+
+
+# ------------------------------------------------------------------ weight-quant matmul
+
+def _wq_golden(golden, d, group):
+    out, outf = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
+                                           None if d.get("antiquant_offset") is None else _bits(d["antiquant_offset"]),
+                                           group_size=group)
+    return torch.from_numpy(outf)
+
+
+@pytest.mark.parametrize("M,K,N", [(16, 8192, 512), (1, 1024, 256), (5, 512, 100), (40, 2048, 320), (16, 96, 64)])
+def test_w8a16(capi, golden, M, K, N):
+    d = workloads.w8a16_inputs(seed=M, M=M, K=K, N=N)
+    out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
+                                   d["antiquant_offset"].cuda())
+    stats = bf16_gate(out, _wq_golden(golden, d, 0))
+    print("w8a16", M, K, N, stats)
+
+
+def test_w8a16_kmajor_and_no_offset(capi, golden):
+    d = workloads.w8a16_inputs(seed=3, M=8, K=1024, N=192, weight_nk=True)
+    out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
+                                   d["antiquant_offset"].cuda())
+    bf16_gate(out, _wq_golden(golden, d, 0))
+    d2 = workloads.w8a16_inputs(seed=4, M=8, K=1024, N=192)
+    d2["antiquant_offset"] = None
+    out = capi.weight_quant_matmul(d2["x"].cuda(), d2["weight"].cuda(), d2["antiquant_scale"].cuda(), None)
+    bf16_gate(out, _wq_golden(golden, d2, 0))
+
+
+@pytest.mark.parametrize("M", [1, 8, 32, 128])
+def test_w4a16_grouped(capi, golden, M):
+    d = workloads.w4a16_inputs(seed=M, M=M, K=4096, N=1024, group_size=128)
+    out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
+                                   d["antiquant_offset"].cuda(), group_size=128)
+    stats = bf16_gate(out, _wq_golden(golden, d, 128))
+    print("w4a16", M, stats)
+
+
+def test_w4a16_other_groups_and_edges(capi, golden):
+    for (M, K, N, gs) in [(3, 512, 136, 64), (16, 256, 128, 256), (2, 1024, 8, 32), (20, 2048, 2056, 128)]:
+        d = workloads.w4a16_inputs(seed=K + N, M=M, K=K, N=N, group_size=gs)
+        out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
+                                       d["antiquant_offset"].cuda(), group_size=gs)
+        bf16_gate(out, _wq_golden(golden, d, gs))
+
+
+def test_weight_quant_exact_special_case(capi):
+    # small-integer activations, unit scale, zero offset: every partial sum is exact in float32
+    g = torch.Generator().manual_seed(0)
+    x = torch.randint(-8, 9, (16, 1024), generator=g).to(torch.bfloat16)
+    w = torch.randint(-127, 128, (1024, 256), generator=g, dtype=torch.int8)
+    one = torch.ones(256, dtype=torch.bfloat16)
+    out = capi.weight_quant_matmul(x.cuda(), w.cuda(), one.cuda(), None)
+    want = (x.double() @ w.double()).to(torch.bfloat16)
+    assert torch.equal(out.cpu(), want)
+    w4 = torch.randint(-8, 8, (1024, 256), generator=g, dtype=torch.int8)
+    out = capi.weight_quant_matmul(x.cuda(), workloads.pack_int4(w4).cuda(), torch.ones(8, 256, dtype=torch.bfloat16).cuda(),
+                                   None, group_size=128)
+    assert torch.equal(out.cpu(), (x.double() @ w4.double()).to(torch.bfloat16))
+
+
+# ------------------------------------------------------------------ swiglu
+
+def test_swiglu(capi, golden):
+    g = torch.Generator().manual_seed(0)
+    for rows, half in [(64, 14336), (3, 24), (5, 7)]:
+        x = (torch.randn(rows, 2 * half, generator=g) * 3).to(torch.bfloat16)
+        out = capi.swiglu(x.cuda())
+        want = golden.swiglu(_bits(x))
+        dist = golden.bf16_ulp_distance(_bits(out), want)
+        assert dist.max() <= 1 and (dist == 0).mean() > 0.995   # device expf vs libm expf
+
+
+# ------------------------------------------------------------------ error paths (host side, no kernel runs)
+
+def test_c_abi_rejects_bad_arguments(capi):
+    L = capi.lib()
+    assert L.mi355_dynamic_quant(None, 0, None, None, None, -1, 8, 8, None) == -1
+    assert L.mi355_dynamic_quant(None, 7, None, None, None, 1, 8, 8, None) == -1
+    assert L.mi355_quant_matmul(None, None, None, None, 0, None, None, 0, 4, 4, 4, 4, 4, 1, 4, None, 0, None) == -1
+    assert L.mi355_weight_quant_matmul(None, None, 5, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
+    assert b"workspace" in L.mi355_status_string(-4)
+    x1 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")
+    x2 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")
+    with pytest.raises(capi.Mi355Error, match="workspace"):
+        capi.quant_matmul(x1, x2, None, out_dtype=torch.int32, workspace=torch.empty(16, dtype=torch.int8, device="cuda"))
