@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-inference operator path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-others] [--skip-cpu]
+
+A "step" is one npu_quant_matmul call on the headline configuration (W8A8, x int8
+[1024, 4096], weight int8 logical [4096, 11008] stored [N, K] and passed as its transposed
+view the way torch_npu's LinearQuant passes it, per-token x per-channel dequantisation, bf16
+bias, bf16 output).  Inputs are resident in HBM before the timed region; the weight/activation
+sets are rotated over more than the 256 MB Infinity Cache so that repeated steps do not run
+out of cache.  One JSON line is printed; the remaining configurations (dynamic_quant, W8A16,
+W4A16, the MLP chain) are reported under "others" with their own roofline figures.
+
+The CPU oracle is used only to check the timed outputs and as the reported CPU baseline.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA
+BF16_PEAK_TFLOPS = 2500.0    # dense bf16 MFMA
+CACHE_BYTES = 256 << 20      # Infinity Cache
+
+
+def _parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--skip-others", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c3,c4,c5 for the 'others' section")
+    return ap.parse_args()
+
+
+def _bits(t):
+    import numpy as np
+    import torch
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _event_time_ms(torch, fn, iters):
+    """Average GPU time of fn() over `iters` back-to-back calls, HIP events on the launch stream."""
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def _graph_time_us(torch, calls, reps=20):
+    """Capture the list of launches in one HIP graph (removes host launch gaps for microsecond-scale
+    kernels), replay it `reps` times between two events and return the average time per launch in us."""
+    for c in calls:      # warm-up: lazy one-time initialisation must not happen during capture
+        c()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for c in calls:
+            c()
+    g.replay()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        g.replay()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) * 1e3 / (reps * len(calls))
+
+
+def _nsets(bytes_per_set):
+    return max(2, min(16, int(1.5 * CACHE_BYTES / max(bytes_per_set, 1)) + 1))
+
+
+def main():
+    args = _parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this operator path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    import pytorch_amd as pa          # fails loudly when the native libraries are missing
+    from pytorch_amd.testing import workloads
+
+    dev = torch.device("cuda:0")
+    props = torch.cuda.get_device_properties(0)
+    torch.cuda.set_device(0)
+
+    # ------------------------------------------------------------------ headline: C2 quant_matmul
+    M, K, N = 1024, 4096, 11008
+    d0 = workloads.quant_matmul_inputs(seed=0, M=M, K=K, N=N, weight_nk=True, bias=True)
+    set_bytes = M * K + K * N + M * N * 2
+    nsets = _nsets(set_bytes)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    sets = []
+    for i in range(nsets):
+        if i == 0:
+            x1, w_nk = d0["x1"].to(dev), d0["x2"].t().contiguous().to(dev)
+        else:
+            x1 = torch.randint(-127, 128, (M, K), generator=gen, dtype=torch.int8, device=dev)
+            w_nk = torch.randint(-127, 128, (N, K), generator=gen, dtype=torch.int8, device=dev)
+        sets.append((x1, w_nk.t()))
+    ps, sc, bias = d0["pertoken_scale"].to(dev), d0["scale"].to(dev), d0["bias"].to(dev)
+
+    state = {"i": 0, "out": None}
+
+    def step():
+        x1, w = sets[state["i"] % nsets]
+        state["i"] += 1
+        state["out"] = pa.npu_quant_matmul(x1, w, sc, pertoken_scale=ps, bias=bias, output_dtype=torch.bfloat16)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    wall_ms = (t1 - t0) * 1e3 / args.steps
+    kern_ms = ev0.elapsed_time(ev1) / args.steps
+    ops = 2.0 * M * N * K
+    value_tops = ops / (wall_ms * 1e-3) / 1e12
+    achieved_tops = ops / (kern_ms * 1e-3) / 1e12
+
+    # parity of the timed configuration (set 0), against the oracle on a row sample
+    state["i"] = 0
+    step()
+    out0 = state["out"].cpu()
+    parity = {}
+    cpu_baseline = None
+    if not args.skip_cpu:
+        from oracle import golden
+        threads = min(16, os.cpu_count() or 1)
+        golden.set_threads(threads)
+        rows = 48
+        a = d0["x1"][:rows].numpy()
+        b = d0["x2"].numpy()
+        golden.quant_matmul(a[:4], b, d0["scale"].numpy(), d0["pertoken_scale"][:4].numpy(), _bits(d0["bias"]))
+        c0 = time.perf_counter()
+        want, _ = golden.quant_matmul(a, b, d0["scale"].numpy(), d0["pertoken_scale"][:rows].numpy(), _bits(d0["bias"]))
+        c1 = time.perf_counter()
+        parity["c2_rows_bit_identical"] = bool(np.array_equal(_bits(out0[:rows]), want))
+        cpu_baseline = {"value": round(2.0 * rows * N * K / (c1 - c0) / 1e12, 5), "unit": "TOP/s", "cores": threads,
+                        "kind": "port",
+                        "sample": f"first {rows} of the {M} rows of the headline configuration against the full weight "
+                                  f"(int32 GEMM + dequant epilogue of oracle/golden.c, OpenMP), {c1 - c0:.2f} s"}
+
+    result = {
+        "metric": "npu_quant_matmul int8 TOPS (W8A8, int32 accumulate, fused dequant to bf16)",
+        "value": round(value_tops, 2),
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: npu_quant_matmul x int8[1024,4096] . weight int8[4096,11008] "
+                               "(stored [N,K], passed as transposed view), pertoken_scale f32[1024], scale f32[11008], "
+                               "bias bf16[11008], out bf16[1024,11008]",
+                   "rotating_sets": nsets, "device": props.name, "compute_units": props.multi_processor_count,
+                   "clock_mhz": getattr(props, "clock_rate", 0) // 1000},
+        "roofline": {"bound": "mfma", "achieved": round(achieved_tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": round(achieved_tops / INT8_PEAK_TOPS, 4), "traffic": None,
+                     "kernel": "qmm_kernel", "launch_us": round(kern_ms * 1e3, 3)},
+        "cpu_baseline": cpu_baseline,
+        "parity": parity,
+    }
+
+    # ------------------------------------------------------------------ the other configurations
+    others = []
+    only = set(filter(None, args.only.split(",")))
+
+    def want(tag):
+        return not args.skip_others and (not only or tag in only)
+
+    def hbm_entry(name, bytes_per_launch, us, **extra):
+        gbs = bytes_per_launch / (us * 1e-6) / 1e9
+        e = {"name": name, "launch_us": round(us, 3), "bytes": int(bytes_per_launch),
+             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
+        e.update(extra)
+        return e
+
+    if want("c2kn"):
+        # same problem with the weight contiguous as [K,N] (transposed into the workspace first)
+        w_kn = d0["x2"].contiguous().to(dev)
+        x1 = sets[0][0]
+        f = lambda: pa.npu_quant_matmul(x1, w_kn, sc, pertoken_scale=ps, bias=bias, output_dtype=torch.bfloat16)  # noqa: E731
+        for _ in range(3):
+            f()
+        ms = _event_time_ms(torch, f, 20)
+        others.append({"name": "c2 quant_matmul, weight contiguous [K,N]", "launch_us": round(ms * 1e3, 2),
+                       "roofline": {"bound": "mfma", "achieved": round(ops / (ms * 1e-3) / 1e12, 2), "peak": INT8_PEAK_TOPS,
+                                    "unit": "TOP/s", "frac": round(ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
+                                    "traffic": None}})
+        del w_kn
+
+    if want("c1"):
+        rows, cols = 2048, 4096
+        nb = rows * cols * 3 + rows * 4
+        ns = _nsets(nb)
+        xs = [workloads.dynamic_quant_input(seed=0, rows=rows, cols=cols).to(dev)]
+        for i in range(1, ns):
+            xs.append((torch.randn(rows, cols, generator=gen, device=dev)).to(torch.bfloat16))
+        keep = []
+        calls = [(lambda x=x: keep.append(pa.npu_dynamic_quant(x))) for x in xs] * 2
+        us = _graph_time_us(torch, calls)
+        e = hbm_entry("c1 dynamic_quant bf16[2048,4096] (rotating, > Infinity Cache)", nb, us)
+        keep.clear()
+        calls = [(lambda: keep.append(pa.npu_dynamic_quant(xs[0])))] * 8
+        e["cache_hot_us"] = round(_graph_time_us(torch, calls), 3)
+        if not args.skip_cpu:
+            from oracle import golden
+            y, s = pa.npu_dynamic_quant(xs[0])
+            c0 = time.perf_counter()
+            yg, sg = golden.dynamic_quant(_bits(xs[0]))
+            c1 = time.perf_counter()
+            e["parity_bit_exact"] = bool(np.array_equal(y.cpu().numpy(), yg) and np.array_equal(s.cpu().numpy(), sg))
+            e["cpu_baseline"] = {"value": round(nb / (c1 - c0) / 1e9, 3), "unit": "GB/s", "cores": golden.get_threads(),
+                                 "kind": "port", "sample": "the full configuration, one pass"}
+        others.append(e)
+        del xs, keep
+
+    if want("c3"):
+        Mx, Kx, Nx = 16, 8192, 28672
+        nb = Kx * Nx + Mx * Kx * 2 + 2 * Nx * 2 + Mx * Nx * 2
+        d3 = workloads.w8a16_inputs(seed=0, M=Mx, K=Kx, N=Nx)
+        ws = [d3["weight"].to(dev)] + [torch.randint(-127, 128, (Kx, Nx), generator=gen, dtype=torch.int8, device=dev)
+                                       for _ in range(1)]
+        x, s3, o3 = d3["x"].to(dev), d3["antiquant_scale"].to(dev), d3["antiquant_offset"].to(dev)
+        keep = []
+        calls = [(lambda w=w: keep.append(pa.npu_weight_quant_batchmatmul(x, w, s3, o3))) for w in ws] * 4
+        us = _graph_time_us(torch, calls, reps=10)
+        others.append(hbm_entry("c3 W8A16 x bf16[16,8192] . int8[8192,28672] (weight contiguous [K,N])", nb, us,
+                                tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2)))
+        del ws, keep
+
+    if want("c4"):
+        Kx, Nx = 4096, 14336
+        for Mx in (1, 8, 32, 128):
+            nb = Kx * Nx // 2 + 2 * (Kx // 128) * Nx * 2 + Mx * Kx * 2 + Mx * Nx * 2
+            d4 = workloads.w4a16_inputs(seed=0, M=Mx, K=Kx, N=Nx)
+            ns = _nsets(nb)
+            ws = [d4["weight"].to(dev)] + [torch.randint(-2 ** 31, 2 ** 31 - 1, (Kx, Nx // 8), generator=gen,
+                                                         dtype=torch.int32, device=dev) for _ in range(ns - 1)]
+            x, s4, o4 = d4["x"].to(dev), d4["antiquant_scale"].to(dev), d4["antiquant_offset"].to(dev)
+            keep = []
+            calls = [(lambda w=w: keep.append(pa.npu_weight_quant_batchmatmul(x, w, s4, o4, None, None, None, 128)))
+                     for w in ws] * 2
+            us = _graph_time_us(torch, calls)
+            e = hbm_entry(f"c4 W4A16 g128 x bf16[{Mx},4096] . int4[4096,14336]", nb, us,
+                          tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2))
+            if Mx == 128:
+                tf = 2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12
+                e["roofline_mfma"] = {"bound": "mfma", "achieved": round(tf, 1), "peak": BF16_PEAK_TFLOPS,
+                                      "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4), "traffic": None}
+            others.append(e)
+            del ws, keep
+
+    if want("c5"):
+        H, I = 4096, 14336
+        for Mx in (64, 2048):
+            d5 = workloads.mlp_inputs(seed=0, M=Mx, hidden=H, inter=I)
+            x = d5["x"].to(dev)
+            wgu, wd = d5["w_gate_up"].to(dev).t(), d5["w_down"].to(dev).t()
+            sgu, sd = d5["scale_gate_up"].to(dev), d5["scale_down"].to(dev)
+
+            def mlp():
+                xq, xsc = pa.npu_dynamic_quant(x)
+                gu = pa.npu_quant_matmul(xq, wgu, sgu, pertoken_scale=xsc, output_dtype=torch.bfloat16)
+                act = pa.npu_swiglu(gu)
+                aq, asc = pa.npu_dynamic_quant(act)
+                return pa.npu_quant_matmul(aq, wd, sd, pertoken_scale=asc, output_dtype=torch.bfloat16)
+
+            keep = []
+            us = _graph_time_us(torch, [lambda: keep.append(mlp())] * 4, reps=10)
+            mops = 2.0 * Mx * H * 2 * I + 2.0 * Mx * I * H
+            wbytes = H * 2 * I + I * H
+            others.append({"name": f"c5 Llama-3-8B-shaped W8A8 MLP, M={Mx} (5 kernels, cache-resident weights)",
+                           "chain_us": round(us, 2), "int8_tops": round(mops / (us * 1e-6) / 1e12, 2),
+                           "weight_gbs": round(wbytes / (us * 1e-6) / 1e9, 1),
+                           "frac_int8_peak": round(mops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4),
+                           "frac_hbm_peak_weights_only": round(wbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+            del keep
+
+    if others:
+        result["others"] = others
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,91 @@
+"""W8A8 linear layers on top of ``torch.ops.npu.npu_quant_matmul``.
+
+Counterparts of torch_npu/contrib/module/linear_quant.py:96-112 (``LinearQuant``) and
+linear_a8w8_quant.py:87-120 (``LinearA8W8Quant``, the deprecated twin that validates dtypes
+explicitly).  Parameter names, shapes and defaults are the reference's so a state dict moves
+over unchanged: ``weight`` is stored ``[out_features, in_features]`` and reaches the operator
+as its transposed view, i.e. logical ``[K, N]`` with strides ``(1, K)``.
+"""
+from __future__ import annotations
+
+import warnings
+
+import torch
+from torch import nn
+
+__all__ = ["LinearQuant", "LinearA8W8Quant"]
+
+
+class _QuantLinearBase(nn.Module):
+    _validate_dtypes = False
+
+    def __init__(self, in_features: int, out_features: int, *, bias: bool = True, offset: bool = False,
+                 pertoken_scale: bool = False, device=None, dtype=None, output_dtype=None) -> None:
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.output_dtype = output_dtype
+        frozen = lambda t: nn.Parameter(t, requires_grad=False)  # noqa: E731
+        self.weight = frozen(torch.empty((out_features, in_features)))
+        self.scale = frozen(torch.empty(out_features))
+        optional = {
+            "offset": (offset, torch.float32),
+            "pertoken_scale": (pertoken_scale, torch.float32),
+            "bias": (bias, torch.int32),
+        }
+        for name, (present, dt) in optional.items():
+            if present:
+                setattr(self, name, frozen(torch.empty(out_features, dtype=dt)))
+            else:
+                self.register_parameter(name, None)
+
+    def _check_dtypes(self, x: torch.Tensor) -> None:
+        pair = (x.dtype, self.weight.dtype)
+        if pair not in ((torch.int8, torch.int8), (torch.int32, torch.int32)):
+            raise ValueError("input and weight should be both torch.int32 or both torch.int8 datatype, "
+                             f"but now input is {x.dtype}, weight is {self.weight.dtype}.")
+        if not self._validate_dtypes:
+            return
+        rules = (
+            ("scale", self.scale, (torch.int64, torch.float32, torch.bfloat16),
+             "scale should be torch.int64, torch.float32 or torch.bfloat16 datatype, "),
+            ("offset", self.offset, (torch.float32,), "offset should be torch.float32 datatype, "),
+            ("bias", self.bias, (torch.int32, torch.bfloat16, torch.float16, torch.float32),
+             "bias should be torch.int32, torch.bfloat16, torch.float16 or torch.float32 datatype, "),
+            ("pertoken_scale", self.pertoken_scale, (torch.float32,), "pertoken_scale should be torch.float32 datatype, "),
+        )
+        for _, tensor, allowed, text in rules:
+            if tensor is not None and tensor.dtype not in allowed:
+                raise ValueError(text + f"but now it is {tensor.dtype}.")
+        if self.output_dtype is not None and self.output_dtype not in (torch.int8, torch.float16, torch.bfloat16):
+            raise ValueError("output_dtype should be torch.int8, torch.float16 or torch.bfloat16, "
+                             f"but now it is {self.output_dtype}.")
+
+    def forward(self, linear_quant_input: torch.Tensor) -> torch.Tensor:
+        self._check_dtypes(linear_quant_input)
+        scale = self.scale
+        needs_packed_scale = (self.pertoken_scale is None and scale.dtype == torch.float32
+                              and self.output_dtype not in (torch.bfloat16, torch.int32))
+        if needs_packed_scale:
+            # the reference converts the float32 scale with npu_trans_quant_param for the int8 / float16
+            # output paths; neither that packing nor those outputs exist in this build
+            raise NotImplementedError("float32 scale without pertoken_scale selects the int8/float16 output path "
+                                      "(npu_trans_quant_param), which is not implemented; use output_dtype="
+                                      "torch.bfloat16 or torch.int32")
+        return torch.ops.npu.npu_quant_matmul(linear_quant_input, self.weight.transpose(-2, -1), scale,
+                                              offset=self.offset, pertoken_scale=self.pertoken_scale, bias=self.bias,
+                                              output_dtype=self.output_dtype)
+
+
+class LinearQuant(_QuantLinearBase):
+    """``y = dequant(x_int8 @ weight_int8.T)``; see the module docstring."""
+
+
+class LinearA8W8Quant(_QuantLinearBase):
+    """Deprecated alias of :class:`LinearQuant` that validates parameter dtypes before the call."""
+    _validate_dtypes = True
+
+    def __init__(self, *args, **kwargs) -> None:
+        warnings.warn("LinearA8W8Quant is deprecated and will be removed in a future version. "
+                      "Use LinearQuant instead.", FutureWarning)
+        super().__init__(*args, **kwargs)

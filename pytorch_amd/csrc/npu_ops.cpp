@@ -1,0 +1,390 @@
+// torch.ops.npu.* operator library for the quantized-inference path on MI355X.
+//
+// Mirrors what torchnpugen generates for torch_npu (schema registration with
+// TORCH_LIBRARY(npu) and a backend wrapper per op that checks devices, guards the device and
+// calls the adapter: torchnpugen/templates/CustomRegisterSchema.cpp:49-70,
+// torchnpugen/custom_functions.py:94-255) and what the op-plugin adapter does (allocate the
+// outputs, infer shapes, call the aclnn entry point).  Here the adapter calls the C ABI of
+// include/mi355_quant.h on the current HIP stream.
+//
+// Dispatch keys: CUDA (PyTorch's name for the HIP device on ROCm builds) and Meta (shape
+// inference for FakeTensor).  There is deliberately no CPU kernel: calling these ops with CPU
+// tensors fails in the dispatcher.
+#include <ATen/ATen.h>
+#include <ATen/ExpandUtils.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/library.h>
+
+#include "mi355_quant.h"
+
+namespace {
+
+using at::Tensor;
+using c10::optional;
+
+void check_status(int status, const char *op)
+{
+    TORCH_CHECK(status == MI355_OK, op, ": ", mi355_status_string(status), " (status ", status, ")");
+}
+
+// Same text as the reference's generated wrapper check (asserted by
+// test/custom_ops/test_npu_anti_quant.py:86-88).
+void check_same_device(const char *op, std::initializer_list<const Tensor *> ts)
+{
+    const Tensor *first = nullptr;
+    for (const Tensor *t : ts) {
+        if (!t || !t->defined()) continue;
+        if (!first) {
+            first = t;
+            continue;
+        }
+        TORCH_CHECK(t->device() == first->device(),
+                    "Expected all tensors to be on the same device, but found at least two devices, ", first->device(),
+                    " and ", t->device(), "! (when checking arguments for ", op, ")");
+    }
+}
+
+const Tensor *opt(const optional<Tensor> &t) { return t.has_value() && t->defined() ? &*t : nullptr; }
+
+void *stream_of(const Tensor &t)
+{
+    // PyTorch-ROCm names its HIP device type "cuda"; these are its stream/guard classes for that device type
+    return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream();
+}
+
+// ---------------------------------------------------------------- npu_dynamic_quant
+
+void dynamic_quant_check(const Tensor &input, const optional<Tensor> &smooth_scales, const optional<Tensor> &group_index,
+                         optional<at::ScalarType> dst_type)
+{
+    TORCH_CHECK(input.scalar_type() == at::kBFloat16 || input.scalar_type() == at::kHalf,
+                "npu_dynamic_quant: input must be bfloat16 or float16, got ", input.scalar_type());
+    TORCH_CHECK(input.dim() >= 1, "npu_dynamic_quant: input must have at least one dimension");
+    TORCH_CHECK(!opt(group_index), "npu_dynamic_quant: group_index (per-expert smooth scales) is not supported");
+    TORCH_CHECK(!dst_type.has_value() || *dst_type == at::kChar,
+                "npu_dynamic_quant: only dst_type=torch.int8 is supported, got ", *dst_type);
+    if (const Tensor *s = opt(smooth_scales)) {
+        TORCH_CHECK(s->scalar_type() == input.scalar_type(), "npu_dynamic_quant: smooth_scales must have the dtype of input");
+        TORCH_CHECK(s->dim() == 1 && s->size(0) == input.size(-1),
+                    "npu_dynamic_quant: smooth_scales must have shape [", input.size(-1), "]");
+    }
+}
+
+std::tuple<Tensor, Tensor> dynamic_quant_alloc(const Tensor &input)
+{
+    auto scale_shape = input.sizes().vec();
+    scale_shape.pop_back();
+    return {at::empty(input.sizes(), input.options().dtype(at::kChar)),
+            at::empty(scale_shape, input.options().dtype(at::kFloat))};
+}
+
+std::tuple<Tensor, Tensor> dynamic_quant_meta(const Tensor &input, const optional<Tensor> &smooth_scales,
+                                              const optional<Tensor> &group_index, optional<at::ScalarType> dst_type)
+{
+    dynamic_quant_check(input, smooth_scales, group_index, dst_type);
+    return dynamic_quant_alloc(input);
+}
+
+std::tuple<Tensor, Tensor> dynamic_quant_hip(const Tensor &input, const optional<Tensor> &smooth_scales,
+                                             const optional<Tensor> &group_index, optional<at::ScalarType> dst_type)
+{
+    dynamic_quant_check(input, smooth_scales, group_index, dst_type);
+    check_same_device("npu_dynamic_quant", {&input, opt(smooth_scales)});
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+    auto [y, scale] = dynamic_quant_alloc(input);
+    const int64_t cols = input.size(-1);
+    const int64_t rows = cols ? input.numel() / cols : 0;
+    if (rows == 0 || cols == 0) {
+        scale.zero_();
+        return {y, scale};
+    }
+    // rows must be addressable with one stride: a 2-D view with unit inner stride, else a packed copy
+    Tensor x = input;
+    int64_t row_stride = cols;
+    if (x.dim() == 2 && x.stride(1) == 1 && x.stride(0) >= cols) {
+        row_stride = x.stride(0);
+    } else if (!x.is_contiguous()) {
+        x = x.contiguous();
+    }
+    Tensor smooth;
+    if (const Tensor *s = opt(smooth_scales)) smooth = s->contiguous();
+    check_status(mi355_dynamic_quant(x.data_ptr(), x.scalar_type() == at::kBFloat16 ? MI355_DTYPE_BF16 : MI355_DTYPE_FP16,
+                                     smooth.defined() ? smooth.data_ptr() : nullptr, y.data_ptr<int8_t>(),
+                                     scale.data_ptr<float>(), rows, cols, row_stride, stream_of(input)),
+                 "npu_dynamic_quant");
+    return {y, scale};
+}
+
+// ---------------------------------------------------------------- npu_quant_matmul
+
+struct QmmPlan {
+    std::vector<int64_t> out_shape;
+    std::vector<int64_t> batch;      // broadcast batch shape
+    int64_t M, N, K;
+    at::ScalarType out_dtype;
+};
+
+QmmPlan quant_matmul_plan(const Tensor &x1, const Tensor &x2, const Tensor &scale, const optional<Tensor> &offset,
+                          const optional<Tensor> &pertoken_scale, const optional<Tensor> &bias,
+                          optional<at::ScalarType> output_dtype)
+{
+    TORCH_CHECK(x1.scalar_type() == at::kChar && x2.scalar_type() == at::kChar,
+                "npu_quant_matmul: x1 and x2 must both be int8 (int4-packed int32 inputs are not supported), got ",
+                x1.scalar_type(), " and ", x2.scalar_type());
+    TORCH_CHECK(x1.dim() >= 2 && x2.dim() >= 2, "npu_quant_matmul: x1 and x2 must have at least 2 dimensions");
+    QmmPlan p;
+    p.M = x1.size(-2);
+    p.K = x1.size(-1);
+    p.N = x2.size(-1);
+    TORCH_CHECK(x2.size(-2) == p.K, "npu_quant_matmul: inner dimensions differ: x1 [..., ", p.M, ", ", p.K, "] x2 [..., ",
+                x2.size(-2), ", ", p.N, "]");
+    TORCH_CHECK(output_dtype.has_value(),
+                "npu_quant_matmul: output_dtype=None selects the int8 re-quantised output, which is not supported; "
+                "pass output_dtype=torch.bfloat16 or torch.int32");
+    p.out_dtype = *output_dtype;
+    TORCH_CHECK(p.out_dtype == at::kBFloat16 || p.out_dtype == at::kInt,
+                "npu_quant_matmul: output_dtype must be torch.bfloat16 or torch.int32, got ", p.out_dtype);
+    TORCH_CHECK(!opt(offset), "npu_quant_matmul: offset is only meaningful for int8 output, which is not supported");
+    if (p.out_dtype == at::kBFloat16) {
+        TORCH_CHECK(scale.scalar_type() == at::kFloat || scale.scalar_type() == at::kBFloat16,
+                    "npu_quant_matmul: scale must be float32 or bfloat16 for bfloat16 output, got ", scale.scalar_type());
+        TORCH_CHECK(scale.dim() == 1 && (scale.size(0) == 1 || scale.size(0) == p.N),
+                    "npu_quant_matmul: scale must have shape [1] or [", p.N, "]");
+        if (const Tensor *ps = opt(pertoken_scale)) {
+            TORCH_CHECK(ps->scalar_type() == at::kFloat, "npu_quant_matmul: pertoken_scale must be float32");
+            TORCH_CHECK(ps->dim() == 1 && ps->size(0) == p.M, "npu_quant_matmul: pertoken_scale must have shape [", p.M, "]");
+        }
+        if (const Tensor *b = opt(bias)) {
+            TORCH_CHECK(b->scalar_type() == at::kBFloat16,
+                        "npu_quant_matmul: bias must be bfloat16 for bfloat16 output, got ", b->scalar_type());
+            TORCH_CHECK(b->numel() == p.N && b->size(-1) == p.N, "npu_quant_matmul: bias must have shape [", p.N, "]");
+        }
+    } else {
+        TORCH_CHECK(!opt(bias), "npu_quant_matmul: bias with int32 output is not supported");
+        TORCH_CHECK(!opt(pertoken_scale), "npu_quant_matmul: pertoken_scale is not applicable to int32 output");
+    }
+    auto b1 = x1.sizes().slice(0, x1.dim() - 2), b2 = x2.sizes().slice(0, x2.dim() - 2);
+    p.batch = at::infer_size(b1, b2);
+    if (opt(pertoken_scale)) {
+        int64_t nb = 1;
+        for (auto d : p.batch) nb *= d;
+        TORCH_CHECK(nb == 1 || x1.dim() == 2, "npu_quant_matmul: pertoken_scale with batched x1 is not supported");
+    }
+    p.out_shape = p.batch;
+    p.out_shape.push_back(p.M);
+    p.out_shape.push_back(p.N);
+    return p;
+}
+
+Tensor quant_matmul_meta(const Tensor &x1, const Tensor &x2, const Tensor &scale, const optional<Tensor> &offset,
+                         const optional<Tensor> &pertoken_scale, const optional<Tensor> &bias,
+                         optional<at::ScalarType> output_dtype)
+{
+    QmmPlan p = quant_matmul_plan(x1, x2, scale, offset, pertoken_scale, bias, output_dtype);
+    return at::empty(p.out_shape, x1.options().dtype(p.out_dtype));
+}
+
+// A 2-D int8 matrix the kernel can address: one of its strides is 1 and the other covers a row.
+Tensor as_matrix(const Tensor &t)
+{
+    const bool row_major = t.stride(1) == 1 && t.stride(0) >= t.size(1);
+    const bool col_major = t.stride(0) == 1 && t.stride(1) >= t.size(0);
+    return (row_major || col_major) ? t : t.contiguous();
+}
+
+Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale, const optional<Tensor> &offset,
+                        const optional<Tensor> &pertoken_scale, const optional<Tensor> &bias,
+                        optional<at::ScalarType> output_dtype)
+{
+    QmmPlan p = quant_matmul_plan(x1, x2, scale, offset, pertoken_scale, bias, output_dtype);
+    check_same_device("npu_quant_matmul", {&x1, &x2, &scale, opt(pertoken_scale), opt(bias)});
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(x1.device());
+    Tensor out = at::empty(p.out_shape, x1.options().dtype(p.out_dtype));
+    if (out.numel() == 0) return out;
+    const bool bf16 = p.out_dtype == at::kBFloat16;
+    Tensor scale_f, ps, b;
+    if (bf16) {
+        scale_f = scale.to(at::kFloat).contiguous();
+        if (const Tensor *t = opt(pertoken_scale)) ps = t->contiguous();
+        if (const Tensor *t = opt(bias)) b = t->reshape({p.N}).contiguous();
+    }
+    int64_t nb = 1;
+    for (auto d : p.batch) nb *= d;
+    // x1 with batch dimensions against a single weight matrix is one tall matmul
+    bool x2_single = true;
+    for (int64_t d = 0; d < x2.dim() - 2; d++) x2_single = x2_single && x2.size(d) == 1;
+    std::vector<std::pair<Tensor, Tensor>> jobs; // (a [m,K], b [K,N]) pairs writing consecutive rows of out
+    Tensor out2d = out.view({-1, p.N});
+    if (x2_single) {
+        Tensor w2 = x2.dim() == 2 ? x2 : x2.as_strided({p.K, p.N}, {x2.stride(-2), x2.stride(-1)});
+        jobs.emplace_back(x1.reshape({-1, p.K}), w2);
+    } else {
+        auto x1s = p.batch, x2s = p.batch;
+        x1s.push_back(p.M), x1s.push_back(p.K), x2s.push_back(p.K), x2s.push_back(p.N);
+        Tensor x1e = x1.expand(x1s).reshape({nb, p.M, p.K});
+        Tensor x2e = x2.expand(x2s);
+        x2e = x2e.reshape({nb, p.K, p.N});
+        for (int64_t i = 0; i < nb; i++) jobs.emplace_back(x1e[i], x2e[i]);
+    }
+    int64_t row0 = 0;
+    for (auto &job : jobs) {
+        Tensor a = job.first.stride(1) == 1 && job.first.stride(0) >= p.K ? job.first : job.first.contiguous();
+        Tensor w = as_matrix(job.second);
+        const int64_t m = a.size(0);
+        Tensor ws;
+        const size_t ws_bytes = mi355_quant_matmul_workspace(m, p.N, p.K, w.stride(0), w.stride(1));
+        if (ws_bytes) ws = at::empty({(int64_t)ws_bytes}, x1.options().dtype(at::kChar));
+        Tensor o = out2d.narrow(0, row0, m);
+        check_status(mi355_quant_matmul(a.data_ptr<int8_t>(), w.data_ptr<int8_t>(), ps.defined() ? ps.data_ptr<float>() : nullptr,
+                                        bf16 ? scale_f.data_ptr<float>() : nullptr, bf16 ? scale_f.numel() : 0,
+                                        b.defined() ? b.data_ptr() : nullptr, o.data_ptr(),
+                                        bf16 ? MI355_OUT_BF16 : MI355_OUT_INT32, m, p.N, p.K, a.stride(0), w.stride(0),
+                                        w.stride(1), o.stride(0), ws.defined() ? ws.data_ptr() : nullptr, ws_bytes,
+                                        stream_of(x1)),
+                     "npu_quant_matmul");
+        row0 += m;
+    }
+    return out;
+}
+
+// ---------------------------------------------------------------- npu_weight_quant_batchmatmul
+
+struct WqPlan {
+    std::vector<int64_t> out_shape;
+    int64_t M, N, K, groups;
+    int bits;
+};
+
+WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &antiquant_scale,
+                         const optional<Tensor> &antiquant_offset, const optional<Tensor> &quant_scale,
+                         const optional<Tensor> &quant_offset, const optional<Tensor> &bias, int64_t group_size,
+                         int64_t inner_precise, optional<at::ScalarType> weight_dtype)
+{
+    const char *op = "npu_weight_quant_batchmatmul";
+    TORCH_CHECK(x.scalar_type() == at::kBFloat16, op, ": x must be bfloat16, got ", x.scalar_type());
+    TORCH_CHECK(weight.scalar_type() == at::kChar || weight.scalar_type() == at::kInt, op,
+                ": weight must be int8, or int32 holding 8 int4 values per word, got ", weight.scalar_type());
+    TORCH_CHECK(x.dim() >= 2 && weight.dim() == 2, op, ": x must be [..., K] with at least 2 dimensions and weight 2-D");
+    TORCH_CHECK(!opt(quant_scale) && !opt(quant_offset), op, ": quant_scale / quant_offset (int8 output) are not supported");
+    TORCH_CHECK(!opt(bias), op, ": bias is not supported");
+    TORCH_CHECK(inner_precise == 0, op, ": inner_precise must be 0");
+    TORCH_CHECK(!weight_dtype.has_value(), op, ": weight_dtype is not supported");
+    WqPlan p;
+    p.bits = weight.scalar_type() == at::kInt ? 4 : 8;
+    p.K = x.size(-1);
+    p.M = p.K ? x.numel() / p.K : 0;
+    p.N = weight.size(1) * (p.bits == 4 ? 8 : 1);
+    TORCH_CHECK(weight.size(0) == p.K, op, ": inner dimensions differ: x [..., ", p.K, "] weight [", weight.size(0), ", ...]");
+    TORCH_CHECK(group_size >= 0, op, ": antiquant_group_size must be >= 0");
+    if (group_size > 0)
+        TORCH_CHECK(p.K % group_size == 0 && group_size % 32 == 0, op,
+                    ": antiquant_group_size must be a multiple of 32 that divides K=", p.K);
+    p.groups = group_size > 0 ? p.K / group_size : 1;
+    auto check_param = [&](const Tensor &t, const char *name) {
+        TORCH_CHECK(t.scalar_type() == at::kBFloat16, op, ": ", name, " must be bfloat16 like x, got ", t.scalar_type());
+        const bool ok1 = t.dim() == 1 && t.size(0) == p.N && p.groups == 1;
+        const bool ok2 = t.dim() == 2 && t.size(0) == p.groups && t.size(1) == p.N;
+        TORCH_CHECK(ok1 || ok2, op, ": ", name, " must have shape [", p.N, "] (per channel) or [", p.groups, ", ", p.N,
+                    "] (per group), got ", t.sizes());
+    };
+    check_param(antiquant_scale, "antiquant_scale");
+    if (const Tensor *o = opt(antiquant_offset)) check_param(*o, "antiquant_offset");
+    p.out_shape = x.sizes().vec();
+    p.out_shape.back() = p.N;
+    return p;
+}
+
+Tensor weight_quant_meta(const Tensor &x, const Tensor &weight, const Tensor &antiquant_scale,
+                         const optional<Tensor> &antiquant_offset, const optional<Tensor> &quant_scale,
+                         const optional<Tensor> &quant_offset, const optional<Tensor> &bias, int64_t group_size,
+                         int64_t inner_precise, optional<at::ScalarType> weight_dtype)
+{
+    WqPlan p = weight_quant_plan(x, weight, antiquant_scale, antiquant_offset, quant_scale, quant_offset, bias, group_size,
+                                 inner_precise, weight_dtype);
+    return at::empty(p.out_shape, x.options());
+}
+
+Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &antiquant_scale,
+                        const optional<Tensor> &antiquant_offset, const optional<Tensor> &quant_scale,
+                        const optional<Tensor> &quant_offset, const optional<Tensor> &bias, int64_t group_size,
+                        int64_t inner_precise, optional<at::ScalarType> weight_dtype)
+{
+    WqPlan p = weight_quant_plan(x, weight, antiquant_scale, antiquant_offset, quant_scale, quant_offset, bias, group_size,
+                                 inner_precise, weight_dtype);
+    check_same_device("npu_weight_quant_batchmatmul", {&x, &weight, &antiquant_scale, opt(antiquant_offset)});
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+    Tensor out = at::empty(p.out_shape, x.options());
+    if (out.numel() == 0) return out;
+    Tensor x2 = x.reshape({p.M, p.K});
+    if (x2.stride(1) != 1 || x2.stride(0) < p.K) x2 = x2.contiguous();
+    Tensor w = p.bits == 4 ? (weight.stride(1) == 1 ? weight : weight.contiguous()) : as_matrix(weight);
+    // the contrib module hands 2-D parameters over as transposed views of [N, G] (linear_weight_quant.py:98-109)
+    Tensor s = antiquant_scale.contiguous(), o;
+    if (const Tensor *t = opt(antiquant_offset)) o = t->contiguous();
+    Tensor out2d = out.view({p.M, p.N});
+    check_status(mi355_weight_quant_matmul(x2.data_ptr(), w.data_ptr(), p.bits, s.data_ptr(), o.defined() ? o.data_ptr() : nullptr,
+                                           out2d.data_ptr(), p.M, p.N, p.K, group_size, x2.stride(0), w.stride(0),
+                                           p.bits == 4 ? 1 : w.stride(1), out2d.stride(0), nullptr, 0, stream_of(x)),
+                 "npu_weight_quant_batchmatmul");
+    return out;
+}
+
+// ---------------------------------------------------------------- npu_swiglu
+
+void swiglu_check(const Tensor &input, int64_t dim)
+{
+    TORCH_CHECK(input.scalar_type() == at::kBFloat16, "npu_swiglu: only bfloat16 is supported, got ", input.scalar_type());
+    TORCH_CHECK(input.dim() >= 1, "npu_swiglu: input must have at least one dimension");
+    TORCH_CHECK(dim == -1 || dim == input.dim() - 1, "npu_swiglu: only the last dimension is supported");
+    TORCH_CHECK(input.size(-1) % 2 == 0, "npu_swiglu: the split dimension must be even");
+}
+
+Tensor swiglu_meta(const Tensor &input, int64_t dim)
+{
+    swiglu_check(input, dim);
+    auto shape = input.sizes().vec();
+    shape.back() /= 2;
+    return at::empty(shape, input.options());
+}
+
+Tensor swiglu_hip(const Tensor &input, int64_t dim)
+{
+    Tensor out = swiglu_meta(input, dim);
+    if (out.numel() == 0) return out;
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+    Tensor x = input.contiguous();
+    const int64_t half = out.size(-1);
+    check_status(mi355_swiglu(x.data_ptr(), out.data_ptr(), out.numel() / half, half, 2 * half, stream_of(input)), "npu_swiglu");
+    return out;
+}
+
+} // namespace
+
+TORCH_LIBRARY_FRAGMENT(npu, m)
+{
+    m.def("npu_dynamic_quant(Tensor input, *, Tensor? smooth_scales=None, Tensor? group_index=None, "
+          "ScalarType? dst_type=None) -> (Tensor, Tensor)");
+    m.def("npu_quant_matmul(Tensor x1, Tensor x2, Tensor scale, *, Tensor? offset=None, Tensor? pertoken_scale=None, "
+          "Tensor? bias=None, ScalarType? output_dtype=None) -> Tensor");
+    m.def("npu_weight_quant_batchmatmul(Tensor x, Tensor weight, Tensor antiquant_scale, Tensor? antiquant_offset=None, "
+          "Tensor? quant_scale=None, Tensor? quant_offset=None, Tensor? bias=None, int antiquant_group_size=0, "
+          "int inner_precise=0, *, ScalarType? weight_dtype=None) -> Tensor");
+    m.def("npu_swiglu(Tensor input, int dim=-1) -> Tensor");
+}
+
+TORCH_LIBRARY_IMPL(npu, CUDA, m)
+{
+    m.impl("npu_dynamic_quant", TORCH_FN(dynamic_quant_hip));
+    m.impl("npu_quant_matmul", TORCH_FN(quant_matmul_hip));
+    m.impl("npu_weight_quant_batchmatmul", TORCH_FN(weight_quant_hip));
+    m.impl("npu_swiglu", TORCH_FN(swiglu_hip));
+}
+
+TORCH_LIBRARY_IMPL(npu, Meta, m)
+{
+    m.impl("npu_dynamic_quant", TORCH_FN(dynamic_quant_meta));
+    m.impl("npu_quant_matmul", TORCH_FN(quant_matmul_meta));
+    m.impl("npu_weight_quant_batchmatmul", TORCH_FN(weight_quant_meta));
+    m.impl("npu_swiglu", TORCH_FN(swiglu_meta));
+}

@@ -1,0 +1,184 @@
+"""GPU tests of the torch operators (torch.ops.npu.*) and the contrib modules at the benchmark
+shapes: full-size parity against the CPU oracle where the oracle finishes in seconds, row
+samples plus exact checksums where it does not, module-versus-operator equality as in the
+reference's test/contrib/test_linear_{quant,a8w8_quant,weight_quant}.py, and the
+Llama-3-8B-shaped W8A8 MLP chain checked stage by stage."""
+import numpy as np
+import pytest
+import torch
+
+from pytorch_amd.testing import workloads, bf16_gate, assert_rtol_equal
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pa():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import pytorch_amd
+    return pytorch_amd
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def test_c1_dynamic_quant_full_size(pa, golden):
+    for seed in (0, 1):
+        x = workloads.dynamic_quant_input(seed=seed)
+        y, s = pa.npu_dynamic_quant(x.cuda())
+        yg, sg = golden.dynamic_quant(_bits(x))
+        assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(y.cpu().numpy(), yg)
+        assert (y.abs().amax(-1) == 127).all()
+
+
+@pytest.mark.parametrize("weight_nk", [True, False])
+def test_c2_quant_matmul_full_size(pa, golden, weight_nk):
+    d = workloads.quant_matmul_inputs(seed=0, weight_nk=weight_nk)
+    x1, x2 = d["x1"].cuda(), d["x2"].cuda()
+    acc = pa.npu_quant_matmul(x1, x2, d["scale"].cuda(), output_dtype=torch.int32).cpu()
+    # exact checksum of every output row: sum_n acc[m,n] == x1[m,:] . (sum_n x2[:,n])
+    colsum = d["x2"].to(torch.int64).sum(1)
+    assert torch.equal(acc.to(torch.int64).sum(1), d["x1"].to(torch.int64) @ colsum)
+    # ... and of every output column
+    rowsum = d["x1"].to(torch.int64).sum(0)
+    assert torch.equal(acc.to(torch.int64).sum(0), rowsum @ d["x2"].to(torch.int64))
+    rows = torch.tensor([0, 1, 255, 256, 511, 640, 1000, 1023])
+    want = golden.int8_gemm(d["x1"][rows].numpy(), d["x2"].numpy())
+    assert np.array_equal(acc[rows].numpy(), want)
+    for bias in (d["bias"], None):
+        out = pa.npu_quant_matmul(x1, x2, d["scale"].cuda(), pertoken_scale=d["pertoken_scale"].cuda(),
+                                  bias=None if bias is None else bias.cuda(), output_dtype=torch.bfloat16)
+        want = golden.quant_matmul_epilogue(acc.numpy(), d["scale"].numpy(), d["pertoken_scale"].numpy(),
+                                            None if bias is None else _bits(bias))
+        assert np.array_equal(_bits(out), want)
+
+
+@pytest.mark.parametrize("weight_nk", [False, True])
+def test_c3_w8a16_full_size(pa, golden, weight_nk):
+    d = workloads.w8a16_inputs(seed=0, weight_nk=weight_nk)
+    out = pa.npu_weight_quant_batchmatmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
+                                          d["antiquant_offset"].cuda())
+    _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
+                                         _bits(d["antiquant_offset"]))
+    print("C3", weight_nk, bf16_gate(out, torch.from_numpy(gold)))
+
+
+@pytest.mark.parametrize("M", [1, 8, 32, 128])
+def test_c4_w4a16_full_size(pa, golden, M):
+    d = workloads.w4a16_inputs(seed=0, M=M)
+    out = pa.npu_weight_quant_batchmatmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
+                                          d["antiquant_offset"].cuda(), None, None, None, 128)
+    _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
+                                         _bits(d["antiquant_offset"]), group_size=128)
+    print("C4", M, bf16_gate(out, torch.from_numpy(gold)))
+
+
+def test_quant_matmul_batched_and_scale_variants(pa, golden):
+    g = torch.Generator().manual_seed(0)
+    x1 = torch.randint(-127, 128, (2, 3, 16, 256), generator=g, dtype=torch.int8)
+    x2 = torch.randint(-127, 128, (3, 256, 48), generator=g, dtype=torch.int8)
+    s = torch.rand(48, generator=g) * 1e-2
+    out = pa.npu_quant_matmul(x1.cuda(), x2.cuda(), s.cuda(), output_dtype=torch.bfloat16).cpu()
+    assert out.shape == (2, 3, 16, 48)
+    for b0 in range(2):
+        for b1 in range(3):
+            want, _ = golden.quant_matmul(x1[b0, b1].numpy(), x2[b1].numpy(), s.numpy())
+            assert np.array_equal(_bits(out[b0, b1]), want)
+    # leading batch of x1 against one weight (shapes of test/test_fake_tensor.py:1886-1894), per-tensor bf16 scale
+    x1 = torch.randint(-127, 128, (1, 1, 1024), generator=g, dtype=torch.int8)
+    x2 = torch.randint(-127, 128, (1, 1024, 100), generator=g, dtype=torch.int8)
+    sb = torch.tensor([0.0078125], dtype=torch.bfloat16)
+    bias = (torch.randn(1, 1, 100, generator=g)).to(torch.bfloat16)
+    out = pa.npu_quant_matmul(x1.cuda(), x2.cuda(), sb.cuda(), bias=bias.cuda(), output_dtype=torch.bfloat16).cpu()
+    want, _ = golden.quant_matmul(x1[0].numpy(), x2[0].numpy(), sb.float().numpy(), None, _bits(bias.reshape(-1)))
+    assert out.shape == (1, 1, 100) and np.array_equal(_bits(out[0]), want)
+
+
+def test_linear_quant_module_equals_operator(pa):
+    """Module output == direct operator output (test/contrib/test_linear_quant.py:24-63)."""
+    from pytorch_amd.contrib.module import LinearQuant, LinearA8W8Quant
+    d = workloads.quant_matmul_inputs(seed=3, M=96, K=512, N=384, weight_nk=True)
+    w_nk = d["x2"].t()                               # stored [N, K], contiguous
+    assert w_nk.is_contiguous()
+    for cls in (LinearQuant, LinearA8W8Quant):
+        import warnings
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            m = cls(512, 384, bias=True, pertoken_scale=True, output_dtype=torch.bfloat16).cuda()
+        m.weight.data = w_nk.cuda()
+        m.scale.data = d["scale"].cuda()
+        m.pertoken_scale.data = d["pertoken_scale"].cuda()
+        m.bias.data = d["bias"].cuda()
+        got = m(d["x1"].cuda())
+        want = pa.npu_quant_matmul(d["x1"].cuda(), d["x2"].cuda(), d["scale"].cuda(),
+                                   pertoken_scale=d["pertoken_scale"].cuda(), bias=d["bias"].cuda(),
+                                   output_dtype=torch.bfloat16)
+        assert_rtol_equal(got, want, 0.001)
+        assert torch.equal(got, want)
+
+
+def test_linear_weight_quant_module_equals_operator(pa, golden):
+    """test/contrib/test_linear_weight_quant.py:53-73 with bf16 parameters, plus the per-group int4 case."""
+    from pytorch_amd.contrib.module import LinearWeightQuant
+    d = workloads.w8a16_inputs(seed=5, M=32, K=1024, N=256, weight_nk=True)
+    m = LinearWeightQuant(1024, 256, bias=False, antiquant_offset=True).cuda()
+    m.weight.data = d["weight"].t().cuda()           # [N, K]
+    m.antiquant_scale.data = d["antiquant_scale"].cuda()
+    m.antiquant_offset.data = d["antiquant_offset"].cuda()
+    got = m(d["x"].cuda())
+    _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
+                                         _bits(d["antiquant_offset"]))
+    bf16_gate(got, torch.from_numpy(gold))
+    assert_rtol_equal(got.float().cpu().numpy(), gold, 0.01)
+    # per-group parameters stored [N, G] and passed transposed
+    d4 = workloads.w4a16_inputs(seed=6, M=4, K=512, N=128, group_size=128)
+    m4 = LinearWeightQuant(512, 128, bias=False, antiquant_offset=True, antiquant_group_size=128).cuda()
+    m4.antiquant_scale.data = d4["antiquant_scale"].t().contiguous().cuda()
+    m4.antiquant_offset.data = d4["antiquant_offset"].t().contiguous().cuda()
+    direct = pa.npu_weight_quant_batchmatmul(d4["x"].cuda(), d4["weight"].cuda(), d4["antiquant_scale"].cuda(),
+                                             d4["antiquant_offset"].cuda(), None, None, None, 128)
+    via = pa.npu_weight_quant_batchmatmul(d4["x"].cuda(), d4["weight"].cuda(), m4.antiquant_scale.t(),
+                                          m4.antiquant_offset.t(), None, None, None, 128)
+    assert torch.equal(direct, via)
+
+
+def _mlp_gpu(pa, d):
+    x = d["x"].cuda()
+    xq, xs = pa.npu_dynamic_quant(x)
+    gu = pa.npu_quant_matmul(xq, d["w_gate_up"].cuda().t(), d["scale_gate_up"].cuda(), pertoken_scale=xs,
+                             output_dtype=torch.bfloat16)
+    act = pa.npu_swiglu(gu)
+    aq, as_ = pa.npu_dynamic_quant(act)
+    out = pa.npu_quant_matmul(aq, d["w_down"].cuda().t(), d["scale_down"].cuda(), pertoken_scale=as_,
+                              output_dtype=torch.bfloat16)
+    return xq, xs, gu, act, aq, as_, out
+
+
+def test_c5_mlp_chain_stagewise(pa, golden):
+    """Each GPU stage against the oracle applied to that stage's actual GPU input."""
+    d = workloads.mlp_inputs(seed=0, M=64)
+    xq, xs, gu, act, aq, as_, out = _mlp_gpu(pa, d)
+    yg, sg = golden.dynamic_quant(_bits(d["x"]))
+    assert np.array_equal(xq.cpu().numpy(), yg) and np.array_equal(xs.cpu().numpy(), sg)
+    want, _ = golden.quant_matmul(xq.cpu().numpy(), d["w_gate_up"].t().numpy(), d["scale_gate_up"].numpy(), xs.cpu().numpy())
+    assert np.array_equal(_bits(gu), want)
+    dist = golden.bf16_ulp_distance(_bits(act), golden.swiglu(_bits(gu)))
+    assert dist.max() <= 1 and (dist == 0).mean() > 0.995
+    yg, sg = golden.dynamic_quant(_bits(act))
+    assert np.array_equal(aq.cpu().numpy(), yg) and np.array_equal(as_.cpu().numpy(), sg)
+    want, _ = golden.quant_matmul(aq.cpu().numpy(), d["w_down"].t().numpy(), d["scale_down"].numpy(), as_.cpu().numpy())
+    assert np.array_equal(_bits(out), want)
+    assert torch.isfinite(out.float()).all()
+
+
+def test_c5_mlp_prefill_properties(pa, golden):
+    """M = 2048: rows are independent, so any subset of rows run alone must reproduce the same bits."""
+    d = workloads.mlp_inputs(seed=1, M=2048)
+    full = _mlp_gpu(pa, d)[-1]
+    rows = torch.tensor([0, 5, 777, 2047])
+    sub = dict(d)
+    sub["x"] = d["x"][rows]
+    part = _mlp_gpu(pa, sub)[-1]
+    assert torch.equal(full[rows.cuda()], part)

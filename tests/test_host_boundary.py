@@ -1,0 +1,217 @@
+"""Host-side tests that need no GPU: the C ABI library loads and exports what the header
+declares, the torch operators are registered under torch_npu's names with its argument
+layout, Meta (FakeTensor) shape inference matches the expectations of the reference's
+test/test_fake_tensor.py:1670-1687,1883-1925, unsupported arguments raise instead of being
+ignored, and the contrib modules marshal their arguments as the reference's do."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_c_abi_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "mi355_quant.h")).read()
+    declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", header))
+    assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu"} <= declared
+    lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_amd", "csrc", "libmi355_quant.so"))
+    for name in declared:
+        assert hasattr(lib, name), name
+    lib.mi355_status_string.restype = ctypes.c_char_p
+    assert lib.mi355_status_string(0) == b"ok"
+    assert lib.mi355_quant_abi_version() >= 1000
+    from pytorch_amd import _capi
+    assert set(_capi.EXPORTS) == declared
+
+
+@pytest.fixture(scope="module")
+def pa():
+    import pytorch_amd
+    return pytorch_amd
+
+
+def test_operator_names_and_schemas(pa):
+    assert set(pa.__all__) >= {"npu_dynamic_quant", "npu_quant_matmul", "npu_weight_quant_batchmatmul", "npu_swiglu"}
+    assert pa.npu_quant_matmul is torch.ops.npu.npu_quant_matmul
+    s = str(torch.ops.npu.npu_dynamic_quant.default._schema)
+    assert s.startswith("npu::npu_dynamic_quant(Tensor input, *, Tensor? smooth_scales=None, Tensor? group_index=None")
+    s = str(torch.ops.npu.npu_quant_matmul.default._schema)
+    assert "Tensor x1, Tensor x2, Tensor scale, *, Tensor? offset=None, Tensor? pertoken_scale=None, Tensor? bias=None" in s
+    s = str(torch.ops.npu.npu_weight_quant_batchmatmul.default._schema)
+    assert ("Tensor x, Tensor weight, Tensor antiquant_scale, Tensor? antiquant_offset=None, Tensor? quant_scale=None, "
+            "Tensor? quant_offset=None, Tensor? bias=None, int antiquant_group_size=0, int inner_precise=0, *, "
+            "ScalarType? weight_dtype=None") in s
+
+
+def test_no_cpu_implementation(pa):
+    with pytest.raises(NotImplementedError, match="CPU"):
+        pa.npu_dynamic_quant(torch.zeros(4, 8, dtype=torch.bfloat16))
+    with pytest.raises(NotImplementedError, match="CPU"):
+        pa.npu_swiglu(torch.zeros(4, 8, dtype=torch.bfloat16))
+
+
+def _m(*shape, dtype):
+    return torch.empty(*shape, dtype=dtype, device="meta")
+
+
+def test_meta_dynamic_quant(pa):
+    # test/test_fake_tensor.py:1670-1687
+    x = _m(4, 2048, 1024, dtype=torch.float16)
+    sm = _m(1024, dtype=torch.float16)
+    y, s = pa.npu_dynamic_quant(x, smooth_scales=sm)
+    assert y.shape == (4, 2048, 1024) and y.dtype == torch.int8 and y.device == x.device
+    assert s.shape == (4, 2048) and s.dtype == torch.float32
+    y, s = pa.npu_dynamic_quant(_m(7, 64, dtype=torch.bfloat16), dst_type=torch.int8)
+    assert y.shape == (7, 64) and s.shape == (7,)
+    with pytest.raises(RuntimeError, match="group_index"):
+        pa.npu_dynamic_quant(x, group_index=_m(4, dtype=torch.int32))
+    with pytest.raises(RuntimeError, match="dst_type"):
+        pa.npu_dynamic_quant(x, dst_type=torch.quint4x2)
+    with pytest.raises(RuntimeError, match="bfloat16 or float16"):
+        pa.npu_dynamic_quant(_m(4, 8, dtype=torch.float32))
+    with pytest.raises(RuntimeError, match="smooth_scales"):
+        pa.npu_dynamic_quant(x, smooth_scales=_m(8, dtype=torch.float16))
+
+
+def test_meta_quant_matmul(pa):
+    # shapes of test/test_fake_tensor.py:1883-1915 for the output types this build supports
+    x1 = _m(1, 1, 1024, dtype=torch.int8)
+    x2 = _m(1, 1024, 100, dtype=torch.int8)
+    r = pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.bfloat16), offset=None, bias=_m(1, 1, 100, dtype=torch.bfloat16),
+                            output_dtype=torch.bfloat16)
+    assert r.shape == (1, 1, 100) and r.dtype == torch.bfloat16
+    r = pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), output_dtype=torch.int32)
+    assert r.shape == (1, 1, 100) and r.dtype == torch.int32
+    r = pa.npu_quant_matmul(_m(5, 3, 16, 64, dtype=torch.int8), _m(3, 64, 32, dtype=torch.int8), _m(32, dtype=torch.float32),
+                            output_dtype=torch.bfloat16)
+    assert r.shape == (5, 3, 16, 32)
+    r = pa.npu_quant_matmul(_m(16, 64, dtype=torch.int8), _m(32, 64, dtype=torch.int8).t(), _m(32, dtype=torch.float32),
+                            pertoken_scale=_m(16, dtype=torch.float32), output_dtype=torch.bfloat16)
+    assert r.shape == (16, 32)
+    # unsupported variants raise, never silently ignored
+    with pytest.raises(RuntimeError, match="output_dtype=None"):
+        pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), offset=_m(1, dtype=torch.float32))
+    with pytest.raises(RuntimeError, match="offset"):
+        pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), offset=_m(1, dtype=torch.float32), output_dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="output_dtype must be"):
+        pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), output_dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="int4-packed"):
+        pa.npu_quant_matmul(_m(16, 8, dtype=torch.int32), _m(64, 5, dtype=torch.int32), _m(1, dtype=torch.float32),
+                            output_dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="inner dimensions"):
+        pa.npu_quant_matmul(_m(4, 8, dtype=torch.int8), _m(16, 4, dtype=torch.int8), _m(4, dtype=torch.float32),
+                            output_dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="pertoken_scale must have shape"):
+        pa.npu_quant_matmul(_m(4, 8, dtype=torch.int8), _m(8, 4, dtype=torch.int8), _m(4, dtype=torch.float32),
+                            pertoken_scale=_m(3, dtype=torch.float32), output_dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="bias must be bfloat16"):
+        pa.npu_quant_matmul(_m(4, 8, dtype=torch.int8), _m(8, 4, dtype=torch.int8), _m(4, dtype=torch.float32),
+                            bias=_m(4, dtype=torch.int32), output_dtype=torch.bfloat16)
+
+
+def test_meta_weight_quant_batchmatmul(pa):
+    x = _m(16, 8192, dtype=torch.bfloat16)
+    w = _m(28672, 8192, dtype=torch.int8).t()
+    s, o = _m(28672, dtype=torch.bfloat16), _m(28672, dtype=torch.bfloat16)
+    assert pa.npu_weight_quant_batchmatmul(x, w, s, o).shape == (16, 28672)
+    # int4: last dimension x 8 (test/test_fake_tensor.py:1917-1923 states the same rule for packed int32)
+    w4 = _m(4096, 1792, dtype=torch.int32)
+    sg, og = _m(32, 14336, dtype=torch.bfloat16), _m(32, 14336, dtype=torch.bfloat16)
+    r = pa.npu_weight_quant_batchmatmul(_m(2, 4, 4096, dtype=torch.bfloat16), w4, sg, og, None, None, None, 128)
+    assert r.shape == (2, 4, 14336) and r.dtype == torch.bfloat16
+    xs = _m(1, 4096, dtype=torch.bfloat16)
+    for kwargs, pat in [(dict(quant_scale=_m(14336, dtype=torch.float32)), "quant_scale"),
+                        (dict(bias=_m(14336, dtype=torch.bfloat16)), "bias"),
+                        (dict(inner_precise=1), "inner_precise"),
+                        (dict(weight_dtype=torch.int8), "weight_dtype")]:
+        with pytest.raises(RuntimeError, match=pat):
+            pa.npu_weight_quant_batchmatmul(xs, w4, sg, og, antiquant_group_size=128, **kwargs)
+    with pytest.raises(RuntimeError, match="antiquant_scale must have shape"):
+        pa.npu_weight_quant_batchmatmul(xs, w4, _m(14336, dtype=torch.bfloat16), None, antiquant_group_size=128)
+    with pytest.raises(RuntimeError, match="multiple of 32"):
+        pa.npu_weight_quant_batchmatmul(xs, w4, sg, og, antiquant_group_size=100)
+    with pytest.raises(RuntimeError, match="x must be bfloat16"):
+        pa.npu_weight_quant_batchmatmul(_m(1, 4096, dtype=torch.float16), w4, sg, og, antiquant_group_size=128)
+
+
+def test_meta_swiglu(pa):
+    assert pa.npu_swiglu(_m(64, 28672, dtype=torch.bfloat16)).shape == (64, 14336)
+    assert pa.npu_swiglu(_m(2, 3, 8, dtype=torch.bfloat16), -1).shape == (2, 3, 4)
+    with pytest.raises(RuntimeError, match="last dimension"):
+        pa.npu_swiglu(_m(4, 8, dtype=torch.bfloat16), 0)
+
+
+def test_fake_tensor_mode(pa):
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode():
+        x = torch.empty(4, 2048, 1024, dtype=torch.float16, device="cuda")
+        y, s = pa.npu_dynamic_quant(x)
+        assert y.shape == x.shape and y.dtype == torch.int8 and y.device == x.device
+        assert s.shape == (4, 2048) and s.dtype == torch.float32 and s.device == x.device
+
+
+# ---------------------------------------------------------------- contrib modules (argument marshalling)
+
+class _Recorder:
+    def __init__(self, monkeypatch, name):
+        self.calls = []
+        real = getattr(torch.ops.npu, name)
+
+        def fake(*args, **kwargs):
+            self.calls.append((args, kwargs))
+            return real(*args, **kwargs)
+        monkeypatch.setattr(torch.ops.npu, name, fake, raising=False)
+
+
+def test_linear_quant_marshalling(pa, monkeypatch):
+    from pytorch_amd.contrib.module import LinearQuant, LinearA8W8Quant
+    rec = _Recorder(monkeypatch, "npu_quant_matmul")
+    m = LinearQuant(64, 32, bias=False, pertoken_scale=True, output_dtype=torch.bfloat16)
+    assert m.weight.shape == (32, 64) and m.scale.shape == (32,) and m.bias is None and m.offset is None
+    assert not m.weight.requires_grad
+    m = m.to("meta")
+    m.weight.data = _m(32, 64, dtype=torch.int8)
+    m.pertoken_scale.data = _m(16, dtype=torch.float32)
+    out = m(_m(16, 64, dtype=torch.int8))
+    assert out.shape == (16, 32) and out.dtype == torch.bfloat16
+    (args, kwargs), = rec.calls
+    assert args[1].shape == (64, 32) and args[1].stride() == (1, 64)          # transposed view, K-contiguous
+    assert set(kwargs) == {"offset", "pertoken_scale", "bias", "output_dtype"}
+    with pytest.raises(ValueError, match="both torch.int32 or both torch.int8"):
+        m(_m(16, 64, dtype=torch.float16))
+    # float32 scale without pertoken_scale and without bf16/int32 output would need npu_trans_quant_param
+    m2 = LinearQuant(64, 32, bias=False).to("meta")
+    m2.weight.data = _m(32, 64, dtype=torch.int8)
+    with pytest.raises(NotImplementedError, match="npu_trans_quant_param"):
+        m2(_m(16, 64, dtype=torch.int8))
+    with pytest.warns(FutureWarning):
+        a = LinearA8W8Quant(64, 32, bias=True, output_dtype=torch.bfloat16)
+    assert a.bias.dtype == torch.int32
+    a = a.to("meta")
+    a.weight.data = _m(32, 64, dtype=torch.int8)
+    a.scale.data = _m(32, dtype=torch.float16)
+    with pytest.raises(ValueError, match="scale should be torch.int64, torch.float32 or torch.bfloat16"):
+        a(_m(16, 64, dtype=torch.int8))
+    a.scale.data = _m(32, dtype=torch.float32)
+    a.output_dtype = torch.int32
+    with pytest.raises(ValueError, match="output_dtype should be"):
+        a(_m(16, 64, dtype=torch.int8))
+
+
+def test_linear_weight_quant_marshalling(pa, monkeypatch):
+    from pytorch_amd.contrib.module import LinearWeightQuant
+    rec = _Recorder(monkeypatch, "npu_weight_quant_batchmatmul")
+    m = LinearWeightQuant(256, 64, bias=False, antiquant_offset=True, antiquant_group_size=128).to("meta")
+    assert m.weight.shape == (64, 256) and m.quant_scale is None and m.bias is None
+    m.weight.data = _m(64, 256, dtype=torch.int8)
+    m.antiquant_scale.data = _m(64, 2, dtype=torch.bfloat16)      # stored [N, G]
+    m.antiquant_offset.data = _m(64, 2, dtype=torch.bfloat16)
+    out = m(_m(3, 256, dtype=torch.bfloat16))
+    assert out.shape == (3, 64)
+    (args, kwargs), = rec.calls
+    assert args[1].shape == (256, 64) and args[1].stride() == (1, 256)
+    assert args[2].shape == (2, 64) and args[3].shape == (2, 64)   # handed over as [G, N] views
+    assert args[7] == 128 and args[8] == 0 and kwargs == {"weight_dtype": None}
