@@ -22,7 +22,7 @@ OPS_LIBRARY = _os.path.join(_CSRC, "libmi355_npu_ops.so")
 
 for _p in (KERNEL_LIBRARY, OPS_LIBRARY):
     if not _os.path.exists(_p):
-        raise ImportError(f"{_p} is missing: build the native libraries first with `python -m pytorch_amd.build` "
+        raise ImportError(f"{_p} is missing: build the native libraries first with `python pytorch_amd/build.py` "
                           "(hipcc, --offload-arch=gfx950)")
 
 _torch.ops.load_library(OPS_LIBRARY)

@@ -29,7 +29,7 @@ def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
         if not os.path.exists(LIB_PATH):
-            raise ImportError(f"{LIB_PATH} is missing: run `python -m pytorch_amd.build` (hipcc, gfx950) first")
+            raise ImportError(f"{LIB_PATH} is missing: run `python pytorch_amd/build.py` (hipcc, gfx950) first")
         L = ctypes.CDLL(LIB_PATH)
         vp, i64, i32, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
         L.mi355_status_string.restype = ctypes.c_char_p
@@ -103,6 +103,20 @@ def quant_matmul(x1, x2, scale, pertoken_scale=None, bias=None, out_dtype=torch.
     return out
 
 
+_wq_workspaces = {}
+
+
+def _wq_workspace(device, nbytes: int):
+    """Zero-initialised workspace reused across calls on one stream: the kernel needs its counters
+    to start at zero and leaves them at zero."""
+    key = (device.index, torch.cuda.current_stream().cuda_stream)
+    ws = _wq_workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.int8, device=device)
+        _wq_workspaces[key] = ws
+    return ws
+
+
 def weight_quant_matmul(x, weight, scale, offset=None, group_size: int = 0):
     """x bf16 [M,K]; weight int8 [K,N] (strides (N,1) or (1,K)) or int32 [K,N/8]; scale/offset bf16 [N] or [G,N]."""
     _need_gpu(x, weight, scale, offset)
@@ -114,8 +128,11 @@ def weight_quant_matmul(x, weight, scale, offset=None, group_size: int = 0):
         bits, N = 8, weight.shape[1]
         ldk, ldn = weight.stride(0), weight.stride(1)
     out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    need = lib().mi355_weight_quant_matmul_workspace(M, N, K, bits, group_size)
+    ws = _wq_workspace(x.device, need) if need else None
     st = lib().mi355_weight_quant_matmul(_ptr(x), _ptr(weight), bits, _ptr(scale), _ptr(offset), _ptr(out),
-                                         M, N, K, group_size, x.stride(0), ldk, ldn, out.stride(0), None, 0, _stream())
+                                         M, N, K, group_size, x.stride(0), ldk, ldn, out.stride(0), _ptr(ws),
+                                         0 if ws is None else ws.numel(), _stream())
     _check(st, "mi355_weight_quant_matmul")
     return out
 

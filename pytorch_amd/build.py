@@ -3,7 +3,8 @@
 * ``csrc/libmi355_quant.so``  - the HIP kernels behind the C ABI of ``include/mi355_quant.h``
 * ``csrc/libmi355_npu_ops.so`` - the torch operator library registering ``torch.ops.npu.*``
 
-Usage: ``python -m pytorch_amd.build`` (compiles every time it is called).
+Usage: ``python pytorch_amd/build.py`` (compiles every time it is called; run it as a script, because
+importing the package requires the libraries this builds).
 """
 from __future__ import annotations
 
@@ -47,6 +48,10 @@ def build_kernels(verbose: bool = False) -> str:
     with ThreadPoolExecutor(max_workers=4) as ex:
         objs = list(ex.map(compile_one, KERNEL_SOURCES))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", KERNEL_LIB, *objs])
+    # a kernel whose host stub the compiler silently dropped would only fail at load time
+    undefined = [l for l in _run(["nm", "-u", KERNEL_LIB]).splitlines() if "mi355" in l]
+    if undefined:
+        raise RuntimeError("unresolved kernel symbols in %s:\n%s" % (KERNEL_LIB, "\n".join(undefined)))
     return KERNEL_LIB
 
 

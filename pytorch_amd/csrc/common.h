@@ -36,6 +36,8 @@ inline int check_launch()
     return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ERR_LAUNCH;
 }
 
+__device__ __forceinline__ bool aligned_dev(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 } // namespace mi355

@@ -16,6 +16,9 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/library.h>
 
+#include <map>
+#include <mutex>
+
 #include "mi355_quant.h"
 
 namespace {
@@ -305,6 +308,21 @@ Tensor weight_quant_meta(const Tensor &x, const Tensor &weight, const Tensor &an
     return at::empty(p.out_shape, x.options());
 }
 
+// The split-K reduction of the weight-quant kernel counts arrivals in its workspace: the counters
+// must be zero before a launch and the kernel leaves them zero.  One zero-initialised buffer per
+// (device, stream) is kept and reused; launches on one stream are ordered, so they never overlap.
+Tensor zeroed_workspace(const Tensor &like, size_t bytes)
+{
+    static std::mutex mu;
+    static std::map<std::pair<int, void *>, Tensor> cache;
+    std::lock_guard<std::mutex> lock(mu);
+    const auto key = std::make_pair((int)like.device().index(), stream_of(like));
+    Tensor &ws = cache[key];
+    if (!ws.defined() || (size_t)ws.numel() < bytes)
+        ws = at::zeros({(int64_t)std::max<size_t>(bytes, (size_t)1 << 20)}, like.options().dtype(at::kChar));
+    return ws;
+}
+
 Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &antiquant_scale,
                         const optional<Tensor> &antiquant_offset, const optional<Tensor> &quant_scale,
                         const optional<Tensor> &quant_offset, const optional<Tensor> &bias, int64_t group_size,
@@ -323,9 +341,14 @@ Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &ant
     Tensor s = antiquant_scale.contiguous(), o;
     if (const Tensor *t = opt(antiquant_offset)) o = t->contiguous();
     Tensor out2d = out.view({p.M, p.N});
+    const size_t ws_bytes = mi355_weight_quant_matmul_workspace(p.M, p.N, p.K, p.bits, group_size);
+    Tensor ws;
+    if (ws_bytes) ws = zeroed_workspace(x, ws_bytes);
     check_status(mi355_weight_quant_matmul(x2.data_ptr(), w.data_ptr(), p.bits, s.data_ptr(), o.defined() ? o.data_ptr() : nullptr,
                                            out2d.data_ptr(), p.M, p.N, p.K, group_size, x2.stride(0), w.stride(0),
-                                           p.bits == 4 ? 1 : w.stride(1), out2d.stride(0), nullptr, 0, stream_of(x)),
+                                           p.bits == 4 ? 1 : w.stride(1), out2d.stride(0),
+                                           ws.defined() ? ws.data_ptr() : nullptr, ws.defined() ? (size_t)ws.numel() : 0,
+                                           stream_of(x)),
                  "npu_weight_quant_batchmatmul");
     return out;
 }

@@ -230,3 +230,23 @@ def test_c_abi_rejects_bad_arguments(capi):
     x2 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")
     with pytest.raises(capi.Mi355Error, match="workspace"):
         capi.quant_matmul(x1, x2, None, out_dtype=torch.int32, workspace=torch.empty(16, dtype=torch.int8, device="cuda"))
+
+
+def test_w4a16_repeated_launches_reuse_workspace(capi, golden):
+    """The split-K exchange reuses one workspace and its arrival counters across launches: alternate two
+    problems many times and check every result (a stale partial sum or counter would show up here)."""
+    cases = []
+    for seed in (11, 12):
+        d = workloads.w4a16_inputs(seed=seed, M=8, K=4096, N=2048, group_size=128)
+        _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
+                                             _bits(d["antiquant_offset"]), group_size=128)
+        cases.append(([d[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset")], torch.from_numpy(gold)))
+    first = [None, None]
+    for it in range(40):
+        args, gold = cases[it % 2]
+        out = capi.weight_quant_matmul(*args, group_size=128)
+        if first[it % 2] is None:
+            bf16_gate(out, gold)
+            first[it % 2] = out.clone()
+        else:
+            assert torch.equal(out, first[it % 2]), f"launch {it} differs from the first launch of the same problem"
