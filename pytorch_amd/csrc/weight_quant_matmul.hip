@@ -81,17 +81,19 @@ __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcn
 // B fragments of the two MFMAs that share byte position jb of the dword (int4) / of MFMA #i (int8).
 // w holds this lane's dword from its 8 k rows; fragment VGPR v pairs rows (2v, 2v+1).
 template <int WBITS>
-__device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, u32x4 &b0, u32x4 &b1)
+__device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint32_t magic, u32x4 &b0, u32x4 &b1)
 {
     if constexpr (WBITS == 4) {
+        // `magic` (0x41004100) lives in a VGPR so that (x & mask) | magic is one v_and_or_b32 (mask from an SGPR)
         const uint32_t sel = 0x0c000c00u | ((4u + jb) << 16) | (uint32_t)jb;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const uint32_t t = __builtin_amdgcn_perm(w[2 * v + 1], w[2 * v], sel); // [byte jb of row 2v, 0, byte jb of row 2v+1, 0]
-            b0[v] = ((t << 3) & 0x00780078u) | 0x41004100u;                        // low nibble  -> element 2*jb
-            b1[v] = ((t >> 1) & 0x00780078u) | 0x41004100u;                        // high nibble -> element 2*jb+1
+            b0[v] = ((t << 3) & 0x00780078u) | magic;                              // low nibble  -> element 2*jb
+            b1[v] = ((t >> 1) & 0x00780078u) | magic;                              // high nibble -> element 2*jb+1
         }
     } else {
+        (void)magic;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             b0[v] = pack_bf16x2((float)((w[2 * v] >> (16 * jb)) & 0xffu), (float)((w[2 * v + 1] >> (16 * jb)) & 0xffu));
@@ -178,6 +180,8 @@ __global__ __launch_bounds__(NWV * 64) void wq_stream_kernel(const WqArgs p)
         }
     }
     const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x41004100" : "=v"(magic));   // opaque to the optimiser: stays in a VGPR
     const int dwcol = strip * 32 + 2 * c;                      // first of this lane's two dword columns
     const int ncols_dw = (int)(p.row_bytes >> 2);
     const bool dw_ok[2] = {dwcol < ncols_dw, dwcol + 1 < ncols_dw};
@@ -190,27 +194,38 @@ __global__ __launch_bounds__(NWV * 64) void wq_stream_kernel(const WqArgs p)
     for (int h = 0; h < 2; h++) sv[h] = PV{}, ov[h] = PV{};
     const bool has_offset = p.offset != nullptr;
 
-    // fold one finished group: tot += scale * (P_MUL * P' + (offset - X_BIAS) * X)
+    // fold one finished group: tot += (scale * P_MUL) * (P' + ((offset - X_BIAS) / P_MUL) * X); both rescalings are
+    // exact (powers of two).  Only accumulator rows that exist are touched: lane (c, g) holds rows 4g + q.
+    const bool one_row = MT == 1 && rows_valid == 1;
     auto fold = [&]() {
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             if (!dw_ok[h]) continue;
 #pragma unroll
             for (int i = 0; i < EPD; i++) {
-                const float sc = (i & 1) ? bf16_hi(sv[h][i / 2]) : bf16_lo(sv[h][i / 2]);
-                const float of = (has_offset ? ((i & 1) ? bf16_hi(ov[h][i / 2]) : bf16_lo(ov[h][i / 2])) : 0.0f) - X_BIAS;
+                const float sc = ((i & 1) ? bf16_hi(sv[h][i / 2]) : bf16_lo(sv[h][i / 2])) * P_MUL;
+                const float of = ((has_offset ? ((i & 1) ? bf16_hi(ov[h][i / 2]) : bf16_lo(ov[h][i / 2])) : 0.0f) - X_BIAS) *
+                                 (1.0f / P_MUL);
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++)
+                for (int mt = 0; mt < MT; mt++) {
+                    const float inner0 = __builtin_fmaf(of, X[mt][0], P[mt][h * EPD + i][0]);
+                    tot[mt][h * EPD + i][0] = __builtin_fmaf(sc, inner0, tot[mt][h * EPD + i][0]);
+                    if (!one_row) {
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        const float inner = __builtin_fmaf(of, X[mt][q], P_MUL * P[mt][h * EPD + i][q]);
-                        tot[mt][h * EPD + i][q] = __builtin_fmaf(sc, inner, tot[mt][h * EPD + i][q]);
-                        P[mt][h * EPD + i][q] = 0.0f;
+                        for (int q = 1; q < 4; q++) {
+                            const float inner = __builtin_fmaf(of, X[mt][q], P[mt][h * EPD + i][q]);
+                            tot[mt][h * EPD + i][q] = __builtin_fmaf(sc, inner, tot[mt][h * EPD + i][q]);
+                        }
                     }
+                }
             }
         }
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) X[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int mt = 0; mt < MT; mt++) {
+            X[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < NT; i++) P[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
     };
 
     const int pro = nsteps < D ? nsteps : D;
@@ -251,7 +266,7 @@ __global__ __launch_bounds__(NWV * 64) void wq_stream_kernel(const WqArgs p)
 #pragma unroll
             for (int jb = 0; jb < EPD / 2; jb++) {
                 u32x4 b0, b1;
-                expand_pair<WBITS>(h ? w1 : w0, jb, b0, b1);
+                expand_pair<WBITS>(h ? w1 : w0, jb, magic, b0, b1);
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) {
                     const bf16x8 a = __builtin_bit_cast(bf16x8, xa[mt]);
