@@ -34,6 +34,15 @@ typedef int32_t i32x4v __attribute__((ext_vector_type(4)));
 
 typedef __attribute__((address_space(3))) void lds_void;
 
+template <int VM>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(VM >= 0 && VM < 64, "vmcnt range");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(VM) : "memory");
+}
+
+__device__ __forceinline__ void wait_vmcnt_lgkmcnt0() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+
 // Raw buffer descriptor (stride 0, 32-bit data format): loads beyond `bytes` return zero.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes)
 {
@@ -61,7 +70,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     constexpr int NW = WGM * WGN;
     constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
     constexpr int UNITS_A = BM / 8, UNITS_B = BN / 8;        // unit = 8 rows x 128 B = one wavefront-wide load
-    constexpr int STAGE_BYTES = (BM + BN) * BK;
+    constexpr int UNITS_BP = (UNITS_B + NW - 1) / NW * NW;
+    constexpr int LOADS_PER_STAGE = (UNITS_A + UNITS_BP) / NW;
+    constexpr int STAGE_BYTES = (UNITS_A + UNITS_BP) * 1024;
     static_assert(UNITS_A % NW == 0, "A units must divide evenly over the wavefronts");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -98,12 +109,13 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void *)(stage + u * 1024), 16, voff_a,
                                                      (uint32_t)u * unit_stride_a + k0, 0, 0);
         }
+        // B units are padded to a multiple of the wavefront count (rows past the tile read as zero), so every
+        // wavefront issues the same number of loads per stage
 #pragma unroll
-        for (int i = 0; i < (UNITS_B + NW - 1) / NW; i++) {
+        for (int i = 0; i < UNITS_BP / NW; i++) {
             const int u = i * NW + wave;
-            if (UNITS_B % NW == 0 || u < UNITS_B) // wave-uniform
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void *)(stage + (UNITS_A + u) * 1024), 16, voff_b,
-                                                         (uint32_t)u * unit_stride_b + k0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void *)(stage + (UNITS_A + u) * 1024), 16, voff_b,
+                                                     (uint32_t)u * unit_stride_b + k0, 0, 0);
         }
     };
 
@@ -113,9 +125,6 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 #pragma unroll
         for (int j = 0; j < WTN; j++) acc[i][j] = i32x4v{0, 0, 0, 0};
 
-    const int KT = p.K / BK;
-    issue_stage(0, lds);
-
     // LDS read addressing: lane reads row (lane % 16) of a 16-row tile, 16-byte chunk (ks*4 + lane/16),
     // stored at slot chunk ^ (row % 8).  For ks = 1 the slot is the ks = 0 slot with bit 2 flipped.
     const int frow = lane & 15;
@@ -123,63 +132,176 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     const int a_off = (wm * WTM * 16 + frow) * BK;
     const int b_off = (BM + wn * WTN * 16 + frow) * BK;
 
+    // Fragments are double buffered in registers: the LDS reads of the next 64-wide K step are issued before
+    // the MFMAs of the current one, so LDS latency hides behind the matrix pipe instead of in front of it.
+    i32x4v af0[WTM], bf0[WTN], af1[WTM], bf1[WTN];
+#define MI355_READ_FRAGS(AF, BF, STAGE, KS)                                                                      \
+    {                                                                                                            \
+        const char *st_ = (STAGE);                                                                               \
+        const int sw_ = sw0 ^ ((KS) * 64);                                                                       \
+        _Pragma("unroll") for (int i = 0; i < WTM; i++)                                                          \
+            AF[i] = *reinterpret_cast<const i32x4v *>(st_ + a_off + i * 16 * BK + sw_);                          \
+        _Pragma("unroll") for (int j = 0; j < WTN; j++)                                                          \
+            BF[j] = *reinterpret_cast<const i32x4v *>(st_ + b_off + j * 16 * BK + sw_);                          \
+    }
+#define MI355_MFMA_BLOCK(AF, BF)                                                                                 \
+    {                                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < WTM; i++)                                                          \
+            _Pragma("unroll") for (int j = 0; j < WTN; j++)                                                      \
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(BF[j], AF[i], acc[i][j], 0, 0, 0);             \
+    }
+
+    const int KT = p.K / BK;
+    issue_stage(0, lds);
+    if (KT > 1) issue_stage(BK, lds + STAGE_BYTES);
+    if (KT > 1) wait_vmcnt<LOADS_PER_STAGE>(); else wait_vmcnt<0>();   // stage 0 has landed
+    __syncthreads();
+    MI355_READ_FRAGS(af0, bf0, lds, 0)
+
     for (int kt = 0; kt < KT; kt++) {
         const char *cur = lds + (kt & 1) * STAGE_BYTES;
-        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the loads of this stage have landed
+        char *nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+        MI355_READ_FRAGS(af1, bf1, cur, 1)
+        __builtin_amdgcn_sched_barrier(0);
+        MI355_MFMA_BLOCK(af0, bf0)
+        __builtin_amdgcn_sched_barrier(0);
+        // stage kt+1 (issued one tile ago) has landed, and this wavefront is done reading stage kt
+        wait_vmcnt_lgkmcnt0();
         __syncthreads();
-        if (kt + 1 < KT) issue_stage((kt + 1) * BK, lds + ((kt + 1) & 1) * STAGE_BYTES);
-#pragma unroll
-        for (int ks = 0; ks < BK / 64; ks++) {
-            const int sw = sw0 ^ (ks * 64);
-            i32x4v af[WTM], bf[WTN];
-#pragma unroll
-            for (int i = 0; i < WTM; i++) af[i] = *reinterpret_cast<const i32x4v *>(cur + a_off + i * 16 * BK + sw);
-#pragma unroll
-            for (int j = 0; j < WTN; j++) bf[j] = *reinterpret_cast<const i32x4v *>(cur + b_off + j * 16 * BK + sw);
-#pragma unroll
-            for (int i = 0; i < WTM; i++)
-#pragma unroll
-                for (int j = 0; j < WTN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
-        }
+        if (kt + 2 < KT) issue_stage((kt + 2) * BK, lds + (kt & 1) * STAGE_BYTES);
+        if (kt + 1 < KT) MI355_READ_FRAGS(af0, bf0, nxt, 0)
+        __builtin_amdgcn_sched_barrier(0);
+        MI355_MFMA_BLOCK(af1, bf1)
+        __builtin_amdgcn_sched_barrier(0);
     }
+#undef MI355_READ_FRAGS
+#undef MI355_MFMA_BLOCK
 
     // Epilogue.  The weight fragment was the first MFMA operand, so
     // acc[i][j][r] = C[m = tile row (lane % 16)][n = 4 * (lane / 16) + r].
     const int mrow = lane & 15;
     const int nquad = (lane >> 4) * 4;
+    if (p.out_i32) {
+        const bool vec = (p.ldc & 3) == 0 && aligned_dev(p.out, 16);
+#pragma unroll
+        for (int i = 0; i < WTM; i++) {
+            const int m = m0 + (wm * WTM + i) * 16 + mrow;
+#pragma unroll
+            for (int j = 0; j < WTN; j++) {
+                const int n = n0 + (wn * WTN + j) * 16 + nquad;
+                if (m >= p.M || n >= p.N) continue;
+                int32_t *o = static_cast<int32_t *>(p.out) + (int64_t)m * p.ldc + n;
+                if (vec && n + 3 < p.N) {
+                    *reinterpret_cast<i32x4v *>(o) = acc[i][j];
+                } else {
+                    for (int r = 0; r < 4; r++)
+                        if (n + r < p.N) o[r] = acc[i][j][r];
+                }
+            }
+        }
+        return;
+    }
+    // All dequantisation parameters of this wavefront are fetched in one batch (indices clamped so that every
+    // load is in bounds), then every accumulator quad is scaled and rounded.
+    float psv[WTM];
+#pragma unroll
+    for (int i = 0; i < WTM; i++) {
+        const int m = min(m0 + (wm * WTM + i) * 16 + mrow, p.M - 1);
+        psv[i] = p.pertoken ? p.pertoken[m] : 1.0f;
+    }
+    f32x4 scv[WTN], bsv[WTN];
+    const bool quads = (p.N & 3) == 0 && aligned_dev(p.scale, 16) && (!p.bias || aligned_dev(p.bias, 8));
+#pragma unroll
+    for (int j = 0; j < WTN; j++) {
+        const int n = n0 + (wn * WTN + j) * 16 + nquad;
+        if (p.scale_len == 1) {
+            const float s1 = p.scale[0];
+            scv[j] = f32x4{s1, s1, s1, s1};
+        } else if (quads) {
+            scv[j] = *reinterpret_cast<const f32x4 *>(p.scale + min(n, p.N - 4));
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; r++) scv[j][r] = p.scale[min(n + r, p.N - 1)];
+        }
+        bsv[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (p.bias) {
+            if (quads) {
+                const u32x2 b2 = *reinterpret_cast<const u32x2 *>(p.bias + min(n, p.N - 4));
+                bsv[j] = f32x4{bf16_lo(b2.x), bf16_hi(b2.x), bf16_lo(b2.y), bf16_hi(b2.y)};
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++) bsv[j][r] = bf16_1(p.bias[min(n + r, p.N - 1)]);
+            }
+        }
+    }
+    const bool has_ps = p.pertoken != nullptr, has_bias = p.bias != nullptr;
+
+    // The rounded bf16 tile of a wavefront goes through its own LDS region (the stage buffers are idle after the
+    // last barrier) so that global stores are 16 bytes per lane and cover whole rows of the wavefront tile.
+    constexpr int ROWB = WTN * 32 + 16;                       // padded row pitch: spreads rows over the banks
+    constexpr int CHUNKS = WTN * 2;                           // 16-byte chunks per row
+    static_assert(NW * WTM * 16 * ROWB <= 160 * 1024, "epilogue staging must fit in LDS");
+    char *stg = lds + wave * (WTM * 16 * ROWB);
+    const bool wide = (p.ldc & 7) == 0 && aligned_dev(p.out, 16);
+    if (wide) {
+#pragma unroll
+        for (int i = 0; i < WTM; i++)
+#pragma unroll
+            for (int j = 0; j < WTN; j++) {
+                float f[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float v = (float)acc[i][j][r];
+                    if (has_ps) v = v * psv[i];
+                    v = v * scv[j][r];
+                    if (has_bias) v = v + bsv[j][r];
+                    f[r] = v;
+                }
+                u32x2 pk;
+                pk.x = pack_bf16x2(f[0], f[1]);
+                pk.y = pack_bf16x2(f[2], f[3]);
+                *reinterpret_cast<u32x2 *>(stg + (i * 16 + mrow) * ROWB + (j * 16 + nquad) * 2) = pk;
+            }
+        const int mw = m0 + wm * WTM * 16, nw = n0 + wn * WTN * 16;
+#pragma unroll
+        for (int q0 = 0; q0 < WTM * 16 * CHUNKS; q0 += 64) {
+            const int q = q0 + lane;
+            const int row = q / CHUNKS, ch = q % CHUNKS;
+            if ((WTM * 16 * CHUNKS) % 64 != 0 && row >= WTM * 16) continue;
+            const int m = mw + row, n = nw + ch * 8;
+            if (m >= p.M || n >= p.N) continue;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(stg + row * ROWB + ch * 16);
+            uint16_t *o = static_cast<uint16_t *>(p.out) + (int64_t)m * p.ldc + n;
+            if (n + 7 < p.N) {
+                *reinterpret_cast<u32x4 *>(o) = v;
+            } else {
+                const uint16_t *e = reinterpret_cast<const uint16_t *>(&v);
+                for (int r = 0; r < 8; r++)
+                    if (n + r < p.N) o[r] = (uint16_t)(v[r >> 1] >> ((r & 1) * 16));
+                (void)e;
+            }
+        }
+        return;
+    }
+    const bool vec = (p.ldc & 3) == 0 && aligned_dev(p.out, 8);
 #pragma unroll
     for (int i = 0; i < WTM; i++) {
         const int m = m0 + (wm * WTM + i) * 16 + mrow;
-        if (m >= p.M) continue;
-        const float ps = p.pertoken ? p.pertoken[m] : 1.0f;
 #pragma unroll
         for (int j = 0; j < WTN; j++) {
             const int n = n0 + (wn * WTN + j) * 16 + nquad;
-            if (n >= p.N) continue;
-            const i32x4v c = acc[i][j];
-            if (p.out_i32) {
-                int32_t *o = static_cast<int32_t *>(p.out) + (int64_t)m * p.ldc + n;
-                if (n + 3 < p.N && (p.ldc & 3) == 0) {
-                    *reinterpret_cast<i32x4v *>(o) = c;
-                } else {
-                    for (int r = 0; r < 4; r++)
-                        if (n + r < p.N) o[r] = c[r];
-                }
-                continue;
-            }
             float f[4];
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const int nn = n + r < p.N ? n + r : p.N - 1;
-                float v = (float)c[r];
-                if (p.pertoken) v = v * ps;
-                v = v * p.scale[p.scale_len == 1 ? 0 : nn];
-                if (p.bias) v = v + bf16_1(p.bias[nn]);
+                float v = (float)acc[i][j][r];
+                if (has_ps) v = v * psv[i];
+                v = v * scv[j][r];
+                if (has_bias) v = v + bsv[j][r];
                 f[r] = v;
             }
+            if (m >= p.M || n >= p.N) continue;
             uint16_t *o = static_cast<uint16_t *>(p.out) + (int64_t)m * p.ldc + n;
-            if (n + 3 < p.N && (p.ldc & 3) == 0) {
+            if (vec && n + 3 < p.N) {
                 u32x2 pk;
                 pk.x = pack_bf16x2(f[0], f[1]);
                 pk.y = pack_bf16x2(f[2], f[3]);
@@ -239,7 +361,10 @@ template <int WGM, int WGN, int WTM, int WTN>
 int launch_qmm(QmmArgs p, hipStream_t s)
 {
     constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
-    constexpr size_t lds_bytes = (size_t)STAGES * (BM + BN) * BK;
+    constexpr int NWL = WGM * WGN;
+    constexpr size_t stage_bytes = (size_t)STAGES * (BM / 8 + (BN / 8 + NWL - 1) / NWL * NWL) * 1024;
+    constexpr size_t staging_bytes = (size_t)BM * WGN * ((BN / WGN) * 2 + 16);   // epilogue: padded bf16 tile rows
+    constexpr size_t lds_bytes = stage_bytes > staging_bytes ? stage_bytes : staging_bytes;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
