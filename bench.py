@@ -150,18 +150,18 @@ def main():
         from oracle import golden
         threads = min(16, os.cpu_count() or 1)
         golden.set_threads(threads)
-        rows = 48
+        rows = M          # the whole configuration: ~1.5 s on 16 host threads, and every output element is checked
         a = d0["x1"][:rows].numpy()
         b = d0["x2"].numpy()
         golden.quant_matmul(a[:4], b, d0["scale"].numpy(), d0["pertoken_scale"][:4].numpy(), _bits(d0["bias"]))
         c0 = time.perf_counter()
         want, _ = golden.quant_matmul(a, b, d0["scale"].numpy(), d0["pertoken_scale"][:rows].numpy(), _bits(d0["bias"]))
         c1 = time.perf_counter()
-        parity["c2_rows_bit_identical"] = bool(np.array_equal(_bits(out0[:rows]), want))
+        parity["c2_bit_identical_to_oracle"] = bool(np.array_equal(_bits(out0[:rows]), want))
         cpu_baseline = {"value": round(2.0 * rows * N * K / (c1 - c0) / 1e12, 5), "unit": "TOP/s", "cores": threads,
                         "kind": "port",
-                        "sample": f"first {rows} of the {M} rows of the headline configuration against the full weight "
-                                  f"(int32 GEMM + dequant epilogue of oracle/golden.c, OpenMP), {c1 - c0:.2f} s"}
+                        "sample": f"one pass over the full headline configuration ({rows} rows; int32 GEMM + dequant "
+                                  f"epilogue of oracle/golden.c, OpenMP), {c1 - c0:.2f} s"}
 
     result = {
         "metric": "npu_quant_matmul int8 TOPS (W8A8, int32 accumulate, fused dequant to bf16)",

@@ -378,14 +378,17 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     return check_launch();
 }
 
-// Tile shapes (rows x columns of the workgroup tile) the library instantiates.
+// Tile shapes (rows x columns of the workgroup tile) the library instantiates, with the measured cost of one
+// tile element per 4096 of K (ns, single resident tile per CU): larger tiles amortise LDS and L2 traffic better.
 struct TileChoice {
     int bm, bn;
+    double ns_per_elt;
 };
-constexpr TileChoice kTiles[] = {{256, 256}, {256, 224}, {256, 192}, {128, 352}, {128, 320}, {128, 256},
-                                 {128, 192}, {128, 128}, {64, 256},  {64, 128}};
+constexpr TileChoice kTiles[] = {{256, 256, 0.78}, {256, 224, 0.87}, {256, 192, 0.90}, {128, 352, 1.04},
+                                 {128, 320, 1.00}, {128, 256, 0.92}, {128, 192, 0.85}, {128, 128, 0.98},
+                                 {64, 256, 1.60},  {64, 128, 1.78}};
 
-// Pick the tile shape that minimises (waves of workgroups over the 256 CUs) x (time per tile).
+// Pick the tile shape that minimises (rounds of workgroups over the 256 CUs) x (time per tile).
 TileChoice choose_tile(int M, int N)
 {
     if (const char *e = getenv("MI355_QMM_TILE")) { // debugging aid: "BMxBN"
@@ -398,11 +401,8 @@ TileChoice choose_tile(int M, int N)
     double best_cost = 1e300;
     for (const TileChoice &c : kTiles) {
         const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
-        const long waves = (tiles + 255) / 256;
-        // per-tile time ~ MFMA work, inflated when the tile is small (LDS/L2 bytes per MFMA grow)
-        const double intensity = (double)c.bm * c.bn / (c.bm + c.bn);
-        const double eff = intensity / (intensity + 48.0);
-        const double cost = (double)waves * c.bm * c.bn / eff;
+        const long rounds = (tiles + 255) / 256;
+        const double cost = (double)rounds * ((double)c.bm * c.bn * c.ns_per_elt + 2000.0);
         if (cost < best_cost) {
             best_cost = cost;
             best = c;

@@ -1,0 +1,119 @@
+"""Golden fixtures of tests/golden: hand-typed known answers and frozen seeded problems.
+CPU part: the oracle reproduces them.  GPU part: the HIP kernels, through the C ABI, reproduce them."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+KAT = json.load(open(os.path.join(HERE, "known_answers.json")))
+
+
+def _npz(name):
+    return np.load(os.path.join(HERE, name), allow_pickle=False)
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _bf16(u16):
+    return torch.from_numpy(np.ascontiguousarray(u16).view(np.int16).copy()).view(torch.bfloat16)
+
+
+# ------------------------------------------------------------------ CPU: oracle vs fixtures
+
+def test_oracle_known_answers(golden):
+    for case in KAT["dynamic_quant"]:
+        x = torch.tensor([case["x"]], dtype=torch.bfloat16)
+        assert x.float().tolist()[0] == case["x"]
+        y, s = golden.dynamic_quant(_bits(x))
+        assert y[0].tolist() == case["y"] and float(s[0]) == case["scale"]
+    for case in KAT["unpack_int4"]:
+        assert golden.unpack_int4(np.array([[case["word"]]], np.int32))[0].tolist() == case["values"]
+    for case in KAT["quant_matmul"]:
+        bias = torch.tensor(case["bias"], dtype=torch.bfloat16)
+        out, acc = golden.quant_matmul(np.array(case["x1"], np.int8), np.array(case["x2"], np.int8),
+                                       np.array(case["scale"], np.float32), np.array(case["pertoken_scale"], np.float32),
+                                       _bits(bias))
+        assert acc.tolist() == case["acc"] and golden.bf16_bits_to_f32(out).tolist() == case["out"]
+    for case in KAT["weight_quant"]:
+        x = torch.tensor(case["x"], dtype=torch.bfloat16)
+        out, _ = golden.weight_quant_matmul(_bits(x), np.array(case["w"], np.int8),
+                                            _bits(torch.tensor(case["scale"], dtype=torch.bfloat16)),
+                                            _bits(torch.tensor(case["offset"], dtype=torch.bfloat16)))
+        assert golden.bf16_bits_to_f32(out).tolist() == case["out"]
+
+
+def test_oracle_reproduces_frozen_fixtures(golden):
+    f = _npz("dynamic_quant.npz")
+    y, s = golden.dynamic_quant(f["x"])
+    assert np.array_equal(y, f["y"]) and np.array_equal(s, f["scale"])
+    f = _npz("quant_matmul.npz")
+    out, acc = golden.quant_matmul(f["x1"], f["x2"], f["scale"], f["pertoken_scale"], f["bias"])
+    assert np.array_equal(acc, f["acc"]) and np.array_equal(out, f["out"])
+    f = _npz("w8a16.npz")
+    out, outf = golden.weight_quant_matmul(f["x"], f["weight"], f["scale"], f["offset"])
+    assert np.array_equal(out, f["out"]) and np.array_equal(outf, f["out_f32"])
+    f = _npz("w4a16.npz")
+    out, outf = golden.weight_quant_matmul(f["x"], f["weight"], f["scale"], f["offset"], group_size=128)
+    assert np.array_equal(out, f["out"]) and np.array_equal(outf, f["out_f32"])
+    f = _npz("swiglu.npz")
+    assert np.array_equal(golden.swiglu(f["x"]), f["out"])
+
+
+# ------------------------------------------------------------------ GPU: kernels vs fixtures
+
+@pytest.fixture(scope="module")
+def capi():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from pytorch_amd import _capi
+    return _capi
+
+
+@pytest.mark.gpu
+def test_gpu_known_answers(capi):
+    for case in KAT["dynamic_quant"]:
+        x = torch.tensor([case["x"]], dtype=torch.bfloat16).cuda()
+        y, s = capi.dynamic_quant(x)
+        assert y[0].cpu().tolist() == case["y"] and float(s[0]) == case["scale"]
+    for case in KAT["quant_matmul"]:
+        x1 = torch.tensor(case["x1"], dtype=torch.int8).cuda()
+        x2 = torch.tensor(case["x2"], dtype=torch.int8).cuda()
+        acc = capi.quant_matmul(x1, x2, None, out_dtype=torch.int32)
+        assert acc.cpu().tolist() == case["acc"]
+        out = capi.quant_matmul(x1, x2, torch.tensor(case["scale"]).cuda(), torch.tensor(case["pertoken_scale"]).cuda(),
+                                torch.tensor(case["bias"], dtype=torch.bfloat16).cuda())
+        assert out.float().cpu().tolist() == case["out"]
+    for case in KAT["weight_quant"]:
+        out = capi.weight_quant_matmul(torch.tensor(case["x"], dtype=torch.bfloat16).cuda(),
+                                       torch.tensor(case["w"], dtype=torch.int8).cuda(),
+                                       torch.tensor(case["scale"], dtype=torch.bfloat16).cuda(),
+                                       torch.tensor(case["offset"], dtype=torch.bfloat16).cuda())
+        assert out.float().cpu().tolist() == case["out"]
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_frozen_fixtures(capi):
+    from pytorch_amd.testing import bf16_gate
+    f = _npz("dynamic_quant.npz")
+    y, s = capi.dynamic_quant(_bf16(f["x"]).cuda())
+    assert np.array_equal(y.cpu().numpy(), f["y"]) and np.array_equal(s.cpu().numpy(), f["scale"])
+    f = _npz("quant_matmul.npz")
+    x1, x2 = torch.from_numpy(f["x1"]).cuda(), torch.from_numpy(f["x2"]).cuda()
+    assert np.array_equal(capi.quant_matmul(x1, x2, None, out_dtype=torch.int32).cpu().numpy(), f["acc"])
+    out = capi.quant_matmul(x1, x2, torch.from_numpy(f["scale"]).cuda(), torch.from_numpy(f["pertoken_scale"]).cuda(),
+                            _bf16(f["bias"]).cuda())
+    assert np.array_equal(_bits(out), f["out"])
+    for name, gs in (("w8a16.npz", 0), ("w4a16.npz", 128)):
+        f = _npz(name)
+        out = capi.weight_quant_matmul(_bf16(f["x"]).cuda(), torch.from_numpy(f["weight"]).cuda(), _bf16(f["scale"]).cuda(),
+                                       _bf16(f["offset"]).cuda(), gs)
+        bf16_gate(out, torch.from_numpy(f["out_f32"]))
+    f = _npz("swiglu.npz")
+    out = capi.swiglu(_bf16(f["x"]).cuda())
+    d = np.abs(_bits(out).astype(np.int32) - f["out"].astype(np.int32))
+    assert d.max() <= 1
