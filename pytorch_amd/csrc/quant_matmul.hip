@@ -28,7 +28,6 @@ namespace mi355 {
 namespace {
 
 constexpr int BK = 128;          // bytes (= int8 elements) of K per LDS stage
-constexpr int STAGES = 2;
 
 typedef int32_t i32x4v __attribute__((ext_vector_type(4)));
 
@@ -41,7 +40,12 @@ __device__ __forceinline__ void wait_vmcnt()
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(VM) : "memory");
 }
 
-__device__ __forceinline__ void wait_vmcnt_lgkmcnt0() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+template <int VM>
+__device__ __forceinline__ void wait_vmcnt_lgkm0()
+{
+    static_assert(VM >= 0 && VM < 64, "vmcnt range");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(VM) : "memory");
+}
 
 // Raw buffer descriptor (stride 0, 32-bit data format): loads beyond `bytes` return zero.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes)
@@ -64,7 +68,7 @@ struct QmmArgs {
 };
 
 // WGM x WGN wavefronts per workgroup, each owning (16*WTM) x (16*WTN) of the output tile.
-template <int WGM, int WGN, int WTM, int WTN>
+template <int WGM, int WGN, int WTM, int WTN, int NS>
 __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 {
     constexpr int NW = WGM * WGN;
@@ -151,24 +155,37 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(BF[j], AF[i], acc[i][j], 0, 0, 0);             \
     }
 
+    // NS LDS stages: while stage kt is consumed, stages kt+1 .. kt+NS-1 are landing or in flight, which hides
+    // HBM latency when the operands are not cache resident.  Every wavefront issues L loads per stage, so
+    // "at most c*L loads outstanding" means "everything but the newest c stages has landed".
+    constexpr int L = LOADS_PER_STAGE;
+    static_assert(NS >= 2 && NS <= 4, "stage count");
     const int KT = p.K / BK;
-    issue_stage(0, lds);
-    if (KT > 1) issue_stage(BK, lds + STAGE_BYTES);
-    if (KT > 1) wait_vmcnt<LOADS_PER_STAGE>(); else wait_vmcnt<0>();   // stage 0 has landed
+    {
+        const int pro = KT < NS ? KT : NS;
+        for (int s = 0; s < pro; s++) issue_stage(s * BK, lds + s * STAGE_BYTES);
+        if (pro >= 4) wait_vmcnt<3 * L>();
+        else if (pro == 3) wait_vmcnt<2 * L>();
+        else if (pro == 2) wait_vmcnt<1 * L>();
+        else wait_vmcnt<0>();                                          // stage 0 has landed
+    }
     __syncthreads();
     MI355_READ_FRAGS(af0, bf0, lds, 0)
 
     for (int kt = 0; kt < KT; kt++) {
-        const char *cur = lds + (kt & 1) * STAGE_BYTES;
-        char *nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+        const char *cur = lds + (kt % NS) * STAGE_BYTES;
+        const char *nxt = lds + ((kt + 1) % NS) * STAGE_BYTES;
         MI355_READ_FRAGS(af1, bf1, cur, 1)
         __builtin_amdgcn_sched_barrier(0);
         MI355_MFMA_BLOCK(af0, bf0)
         __builtin_amdgcn_sched_barrier(0);
-        // stage kt+1 (issued one tile ago) has landed, and this wavefront is done reading stage kt
-        wait_vmcnt_lgkmcnt0();
+        // stage kt+1 has landed (stages kt+2 .. may still be in flight) and this wavefront is done reading stage kt
+        const int newer = min(kt + NS - 1, KT - 1) - (kt + 1);
+        if (newer >= 2) wait_vmcnt_lgkm0<2 * L>();
+        else if (newer == 1) wait_vmcnt_lgkm0<1 * L>();
+        else wait_vmcnt_lgkm0<0>();
         __syncthreads();
-        if (kt + 2 < KT) issue_stage((kt + 2) * BK, lds + (kt & 1) * STAGE_BYTES);
+        if (kt + NS < KT) issue_stage((kt + NS) * BK, lds + (kt % NS) * STAGE_BYTES);
         if (kt + 1 < KT) MI355_READ_FRAGS(af0, bf0, nxt, 0)
         __builtin_amdgcn_sched_barrier(0);
         MI355_MFMA_BLOCK(af1, bf1)
@@ -362,7 +379,13 @@ int launch_qmm(QmmArgs p, hipStream_t s)
 {
     constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
     constexpr int NWL = WGM * WGN;
-    constexpr size_t stage_bytes = (size_t)STAGES * (BM / 8 + (BN / 8 + NWL - 1) / NWL * NWL) * 1024;
+    constexpr size_t one_stage = (size_t)(BM / 8 + (BN / 8 + NWL - 1) / NWL * NWL) * 1024;
+    // Two stages.  Deeper prefetch (3-4 stages) measured slower on every tile shape: for tiles of <= 40 KiB per
+    // stage two stages let two workgroups share a CU (sixteen resident wavefronts hide barriers and epilogues),
+    // and for larger tiles the extra stages did not pay either.
+    constexpr int NS = 2;
+    static_assert(NS >= 2, "LDS budget");
+    constexpr size_t stage_bytes = (size_t)NS * one_stage;
     constexpr size_t staging_bytes = (size_t)BM * WGN * ((BN / WGN) * 2 + 16);   // epilogue: padded bf16 tile rows
     constexpr size_t lds_bytes = stage_bytes > staging_bytes ? stage_bytes : staging_bytes;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
@@ -370,7 +393,7 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     p.tiles_n = (p.N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
-    auto kern = qmm_kernel<WGM, WGN, WTM, WTN>;
+    auto kern = qmm_kernel<WGM, WGN, WTM, WTN, NS>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
