@@ -24,15 +24,18 @@
 // bookkeeping of the epilogue.  The order of k inside a lane's operand is free as long as the
 // activation operand uses the same order.
 //
-// Streaming.  A workgroup owns a 128-byte-wide column strip of the weight (one cache line per
-// row) and one chunk of K; its wavefronts split that chunk.  Each wavefront streams its own rows
-// through a private LDS ring with direct-to-LDS buffer loads (16 bytes per lane, no register
-// staging, up to D steps of 32 rows in flight) and synchronises with nothing but its own
-// s_waitcnt counters, so the main loop has no barrier.  The activations of a step travel through
-// the same ring.  Partial sums are reduced over the wavefronts in LDS; when K is split over
-// several workgroups (to occupy all CUs when there are few strips) each workgroup writes its
-// float32 partial to the workspace and the workgroup that arrives last at a per-strip counter
-// adds them in chunk order, which keeps the result independent of scheduling.
+// Streaming.  A wavefront owns a 128-byte-wide column strip of the weight (one cache line per row)
+// and a contiguous range of K; it loads 32 rows per step straight into registers in the operand
+// layout (lane (c, g) takes 8 bytes at column 8c of rows 8g .. 8g+7, so one load instruction covers
+// four full cache lines) and keeps PF steps in flight.  The wavefronts of a workgroup cover W
+// adjacent strips (W * 128 contiguous bytes of every row: strips streamed side by side keep the
+// DRAM pages of a row busy together, which measures close to a linear read) times KS slices of
+// the workgroup's K chunk; there is no barrier in the main loop.  Activations and antiquant
+// parameters are small, stay in cache and are loaded by every wavefront that needs them.
+// Partial sums are reduced over the K slices in LDS; when K is split over several workgroups
+// (to occupy all CUs when there are few strips) each workgroup writes its float32 partial to the
+// workspace and the workgroup that arrives last at a per-tile counter adds them in chunk order,
+// which keeps the result independent of scheduling.
 #include "common.h"
 #include <stdlib.h>
 #include <type_traits>
@@ -52,15 +55,17 @@ struct WqArgs {
     const uint16_t *offset;         // bf16 [G, N] or null
     uint16_t *out;                  // bf16 [M, N]
     float *partial;                 // workspace [S][M][N] float32 (S > 1)
-    uint32_t *counter;              // workspace [mchunks][strips], zero on entry, left zero
+    uint32_t *counter;              // workspace [mchunks][sgroups], zero on entry, left zero
     int64_t ldx, ldo;
     uint32_t ldw_bytes;             // bytes between weight rows
     uint32_t row_bytes;             // valid bytes of a weight row
     int M, N, K;
-    int unit_steps;                 // 32-row steps per scale group (per channel: 1)
+    int unit_steps;                 // 32-row steps per unit of K: a scale group, or one loop body per channel
     int n_units;                    // K / (32 * unit_steps)
     int grouped;                    // 0: one scale row for all K
-    int strips, S;
+    int strips;                     // 128-byte strips of a weight row
+    int sgroups;                    // workgroup tiles along N: groups of W adjacent strips
+    int S;                          // workgroups that share the K range of a tile
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes)
@@ -103,71 +108,115 @@ __device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint
     }
 }
 
-template <int WBITS, int MT, int NWV, int D>
-__global__ __launch_bounds__(NWV * 64) void wq_stream_kernel(const WqArgs p)
+// One step of a wavefront: 32 weight rows of its strip (8 bytes per lane and row).
+// The loads are unconditional so that the main loop stays free of branches around memory instructions (the
+// compiler then tracks the outstanding loads exactly); a step past the end of the wavefront's range is given a
+// lane offset beyond every buffer size instead, which makes the loads return zero without touching memory.
+constexpr uint32_t kOutOfRange = 0x80000000u;
+constexpr int kNonTemporal = 2;           // cache-policy bit: weights are read once, keep them out of the way of the reused data
+
+__device__ __forceinline__ void load_step(u32x2 (&wq)[8], const __amdgpu_buffer_rsrc_t rsrc_w, const uint32_t voff_w,
+                                          const uint32_t ldw_bytes, const uint32_t krow, const bool valid)
 {
+    const uint32_t vw = valid ? voff_w : kOutOfRange;
+#pragma unroll
+    for (int t = 0; t < 8; t++) wq[t] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw, (krow + t) * ldw_bytes, kNonTemporal);
+}
+
+// Antiquant parameters of one group for this lane's NPV * 8 consecutive columns.
+template <int NPV>
+__device__ __forceinline__ void load_params(u32x4 (&sv)[NPV], u32x4 (&ov)[NPV], const __amdgpu_buffer_rsrc_t rsrc_s,
+                                            const __amdgpu_buffer_rsrc_t rsrc_o, const bool has_offset,
+                                            const uint32_t voff_p, const uint32_t row_off)
+{
+#pragma unroll
+    for (int v = 0; v < NPV; v++) {
+        sv[v] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, voff_p + 16u * v, row_off, 0);
+        // no offsets: rsrc_o aliases the scales and the loaded values are masked away (no branch around the load)
+        ov[v] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_o, voff_p + 16u * v, row_off, 0) & (has_offset ? ~0u : 0u);
+    }
+}
+
+// Fold one finished group into the running total: tot += (scale * P_MUL) * (P' + ((offset - X_BIAS) / P_MUL) * X);
+// both rescalings are exact (powers of two).  Lane (c, g) holds accumulator rows 4g + q; with a single activation
+// row only q = 0 of g = 0 is ever stored, so the other components are left alone.
+template <int WBITS, int MT, int NT, int NPV>
+__device__ __forceinline__ void fold_group(f32x4 (&tot)[MT][NT], f32x4 (&P)[MT][NT], f32x4 (&X)[MT], const u32x4 (&sv)[NPV],
+                                           const u32x4 (&ov)[NPV], const bool one_row)
+{
+    constexpr float P_MUL = WBITS == 4 ? 2.0f : 1.0f;
+    constexpr float X_BIAS = WBITS == 4 ? 24.0f : 128.0f;
+#pragma unroll
+    for (int i = 0; i < NT; i++) {
+        const uint32_t su = sv[i / 8][(i % 8) / 2], ou = ov[i / 8][(i % 8) / 2];
+        const float sc = ((i & 1) ? bf16_hi(su) : bf16_lo(su)) * P_MUL;
+        const float of = (((i & 1) ? bf16_hi(ou) : bf16_lo(ou)) - X_BIAS) * (1.0f / P_MUL);
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            const float inner0 = __builtin_fmaf(of, X[mt][0], P[mt][i][0]);
+            tot[mt][i][0] = __builtin_fmaf(sc, inner0, tot[mt][i][0]);
+            if (!one_row) {
+#pragma unroll
+                for (int q = 1; q < 4; q++) {
+                    const float inner = __builtin_fmaf(of, X[mt][q], P[mt][i][q]);
+                    tot[mt][i][q] = __builtin_fmaf(sc, inner, tot[mt][i][q]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        X[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < NT; i++) P[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+}
+
+// BS: steps per loop body (every wavefront's range and every scale group is a whole number of bodies);
+// PF: steps kept in flight (PF divides BS or equals it).
+template <int WBITS, int MT, int W, int KS, int BS, int PF>
+__global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
+{
+    static_assert(BS % PF == 0, "the register ring must divide the loop body");
     constexpr int EPD = 32 / WBITS;            // elements per dword
     constexpr int NB = 32 * EPD;               // columns per strip (128 bytes of a weight row)
     constexpr int NT = 2 * EPD;                // MFMA column sets per lane (it holds 2 dword columns)
-    constexpr int PB = NB * 4;                 // antiquant parameters of a group: NB scales + NB offsets, bf16
-    constexpr int SLOT = 4096 + MT * 1024 + PB; // ring slot: 32 weight rows x 128 B, MT activation fragments, parameters
-    constexpr int LOADS = 4 + MT;              // direct-to-LDS loads per step (one more on the first step of a group)
-    constexpr float P_MUL = WBITS == 4 ? 2.0f : 1.0f;
-    constexpr float X_BIAS = WBITS == 4 ? 24.0f : 128.0f;
-    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    constexpr int NPV = NT / 8;                // 16-byte vectors of bf16 parameters per lane
+    constexpr int NBW = W * NB;                // columns of the workgroup's tile
+    constexpr int THREADS = W * KS * 64;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, g = lane >> 4;
-    // workgroups are dealt round-robin to the 8 XCDs: keep the S chunks of a strip on one XCD
+    const int wstrip = wave % W, kslice = wave / W;
+    // workgroups are dealt round-robin to the 8 XCDs: keep the S chunks of a tile on one XCD
     const int xcd_slot = blockIdx.x >> 3;
-    const int strip = (blockIdx.x & 7) + 8 * (xcd_slot / p.S);
+    const int sgrp = (blockIdx.x & 7) + 8 * (xcd_slot / p.S);
     const int chunk = xcd_slot % p.S;
-    if (strip >= p.strips) return;
+    if (sgrp >= p.sgroups) return;
+    const int strip = sgrp * W + wstrip;
     const int m_base = blockIdx.y * (MT * 16);
     const int rows_valid = min(MT * 16, p.M - m_base);
 
-    // contiguous range of K units for this (chunk, wavefront)
-    const int R = p.S * NWV, r = chunk * NWV + wave;
+    // contiguous range of K units for this (chunk, slice); a wavefront whose strip lies past the row has none
+    const int R = p.S * KS, r = chunk * KS + kslice;
     const int u0 = (int)((int64_t)p.n_units * r / R), u1 = (int)((int64_t)p.n_units * (r + 1) / R);
     const int step0 = u0 * p.unit_steps;
-    const int nsteps = (u1 - u0) * p.unit_steps;
+    const int nsteps = strip < p.strips ? (u1 - u0) * p.unit_steps : 0;
+    const int ustep = p.grouped ? p.unit_steps : nsteps;   // steps between folds
 
-    const __amdgpu_buffer_rsrc_t rsrc_w =
-        make_rsrc(static_cast<const char *>(p.w) + (size_t)strip * 128,
-                  (uint32_t)((uint64_t)(p.K - 1) * p.ldw_bytes + p.row_bytes - (uint32_t)strip * 128u));
-    const __amdgpu_buffer_rsrc_t rsrc_x =
-        make_rsrc(p.x + (int64_t)m_base * p.ldx, (uint32_t)(((int64_t)(rows_valid - 1) * p.ldx + p.K) * 2));
-    const uint32_t voff_w = (uint32_t)(lane >> 3) * p.ldw_bytes + (uint32_t)(lane & 7) * 16u;
-    const uint32_t voff_x = (uint32_t)((c * (int)p.ldx + 8 * g) * 2);
-    const uint32_t mt_stride_x = 16u * (uint32_t)p.ldx * 2u;
-
-    // parameter load of a group: lanes [0, NB/8) fetch 16 bytes of the scale row each, the next NB/8 lanes the offset row
-    constexpr int PL = NB / 8;
-    const int pcol = strip * NB + (lane % PL) * 8;              // first of this lane's 8 parameter columns
-    const bool p_lane = lane < 2 * PL && pcol < p.N && (lane < PL || p.offset != nullptr);
-    const uint16_t *p_base = (lane < PL ? p.scale : p.offset) + pcol;
-
-    // per channel there is a single parameter row: it travels with step 0 only
-    auto group_first = [&](int s) { return p.grouped ? s % p.unit_steps == 0 : s == 0; };
-    char *ring = lds + wave * (D * SLOT);
-    auto issue = [&](int s) {
-        char *slot = ring + (s % D) * SLOT;
-        const uint32_t krow = (uint32_t)(step0 + s) * 32u;
-        if (group_first(s) && p_lane) {
-            const int grp = p.grouped ? u0 + s / p.unit_steps : 0;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p_base + (int64_t)grp * p.N),
-                                             (lds_void *)(slot + 4096 + MT * 1024), 16, 0, 0);
-        }
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_void *)(slot + 4096 + mt * 1024), 16, voff_x,
-                                                     krow * 2u + (uint32_t)mt * mt_stride_x, 0, 0);
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void *)(slot + u * 1024), 16, voff_w,
-                                                     (krow + 8u * u) * p.ldw_bytes, 0, 0);
-    };
+    // lanes past the end of the row read (and discard) the first bytes of the row instead
+    const bool lane_ok = (uint32_t)strip * 128u + (uint32_t)c * 8u < p.row_bytes;
+    const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(p.w, (uint32_t)((uint64_t)(p.K - 1) * p.ldw_bytes + p.row_bytes));
+    const uint32_t voff_w = (uint32_t)(8 * g) * p.ldw_bytes + (lane_ok ? (uint32_t)strip * 128u + (uint32_t)c * 8u : 0u);
+    // lane (c, g) owns columns strip * NB + (2c) * EPD .. + NT - 1
+    const bool has_offset = p.offset != nullptr;
+    const uint32_t param_bytes = (uint32_t)(p.grouped ? p.n_units : 1) * (uint32_t)p.N * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc_s = make_rsrc(p.scale, param_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_o = make_rsrc(has_offset ? p.offset : p.scale, param_bytes);
+    const uint32_t voff_p = lane_ok ? (uint32_t)(strip * NB + 2 * c * EPD) * 2u : 0u;
+    const uint32_t param_pitch = (uint32_t)p.N * 2u;
 
     f32x4 tot[MT][NT], P[MT][NT], X[MT];
 #pragma unroll
@@ -182,135 +231,128 @@ __global__ __launch_bounds__(NWV * 64) void wq_stream_kernel(const WqArgs p)
     const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
     uint32_t magic;
     asm volatile("v_mov_b32 %0, 0x41004100" : "=v"(magic));   // opaque to the optimiser: stays in a VGPR
-    const int dwcol = strip * 32 + 2 * c;                      // first of this lane's two dword columns
-    const int ncols_dw = (int)(p.row_bytes >> 2);
-    const bool dw_ok[2] = {dwcol < ncols_dw, dwcol + 1 < ncols_dw};
-
-    // Antiquant parameters of the current group: they arrive in the ring slot of the group's first step and are
-    // copied to registers when that step is consumed.  Lane (c, g) owns columns (2c)*EPD .. (2c+2)*EPD-1.
-    typedef typename std::conditional<EPD == 8, u32x4, u32x2>::type PV;
-    PV sv[2], ov[2];
-#pragma unroll
-    for (int h = 0; h < 2; h++) sv[h] = PV{}, ov[h] = PV{};
-    const bool has_offset = p.offset != nullptr;
-
-    // fold one finished group: tot += (scale * P_MUL) * (P' + ((offset - X_BIAS) / P_MUL) * X); both rescalings are
-    // exact (powers of two).  Only accumulator rows that exist are touched: lane (c, g) holds rows 4g + q.
     const bool one_row = MT == 1 && rows_valid == 1;
-    auto fold = [&]() {
+
+    // register ring: PF steps of weights and activations in flight, the next group's parameters behind them
+    u32x2 wq[PF][8];
+    u32x4 sv[NPV], ov[NPV], sv_next[NPV], ov_next[NPV];
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            if (!dw_ok[h]) continue;
+    for (int v = 0; v < NPV; v++) sv[v] = ov[v] = u32x4{0u, 0u, 0u, 0u};
+    // scale group of the loop body that follows the current one (parameters are requested a body ahead; per
+    // channel, and inside a group, that re-reads the same cached row, which keeps the loop free of branches)
+    const int grp_last = p.grouped ? u1 - 1 : 0;
+    const int gstep = p.grouped ? p.unit_steps : 0x7fffffff;
+    int grp_next = p.grouped ? u0 : 0, next_in_unit = 0;
+    load_params<NPV>(sv_next, ov_next, rsrc_s, rsrc_o, has_offset, voff_p, (uint32_t)grp_next * param_pitch);
 #pragma unroll
-            for (int i = 0; i < EPD; i++) {
-                const float sc = ((i & 1) ? bf16_hi(sv[h][i / 2]) : bf16_lo(sv[h][i / 2])) * P_MUL;
-                const float of = ((has_offset ? ((i & 1) ? bf16_hi(ov[h][i / 2]) : bf16_lo(ov[h][i / 2])) : 0.0f) - X_BIAS) *
-                                 (1.0f / P_MUL);
+    for (int j = 0; j < PF; j++)
+        load_step(wq[j], rsrc_w, voff_w, p.ldw_bytes, (uint32_t)(step0 + j) * 32u, j < nsteps);
+
+    // The activations of the workgroup's K chunk go to LDS once, already in MFMA operand order: the fragment of
+    // (step, m tile) is 1 KiB, lane (c, g) finds x[m tile * 16 + c][32 * step + 8g .. + 7] at lane * 16.  The global
+    // side reads whole rows (consecutive threads take consecutive 16-byte pieces of one row).  Rows past the last
+    // valid one stay unwritten: they only feed accumulator rows that are never stored.
+    const int cu0 = (int)((int64_t)p.n_units * (chunk * KS) / R), cu1 = (int)((int64_t)p.n_units * (chunk * KS + KS) / R);
+    const int cstep0 = cu0 * p.unit_steps;
+    const int pieces = (cu1 - cu0) * p.unit_steps * 4;      // 16-byte pieces per activation row
+    char *xs = lds + 16;
+    {
+        // rows are dealt to the wavefronts, the lanes walk along a row; the loads of a lane are independent of
+        // its LDS stores, so they all go out before the first one is needed
+        const uint16_t *xsrc = p.x + (int64_t)m_base * p.ldx + (int64_t)cstep0 * 32;
+        for (int r = wave; r < rows_valid; r += W * KS) {
+            const uint16_t *xrow = xsrc + (int64_t)r * p.ldx;
+            char *dst = xs + (((r >> 4) * 64 + (r & 15)) << 4);
+#pragma unroll 4
+            for (int q = lane; q < pieces; q += 64) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(xrow + q * 8);
+                *reinterpret_cast<u32x4 *>(dst + ((((q >> 2) * MT) * 64 + (q & 3) * 16) << 4)) = v;
+            }
+        }
+    }
+    __syncthreads();
+    const char *xw = xs + ((size_t)(step0 - cstep0) * MT * 64 + lane) * 16;   // this wavefront's first fragment
+
+    int in_unit = 0;
+#pragma unroll 1
+    for (int s = 0; s < nsteps; s += BS) {
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    const float inner0 = __builtin_fmaf(of, X[mt][0], P[mt][h * EPD + i][0]);
-                    tot[mt][h * EPD + i][0] = __builtin_fmaf(sc, inner0, tot[mt][h * EPD + i][0]);
-                    if (!one_row) {
+        for (int v = 0; v < NPV; v++) sv[v] = sv_next[v], ov[v] = ov_next[v];
+        next_in_unit += BS;
+        if (next_in_unit == gstep) next_in_unit = 0, grp_next = min(grp_next + 1, grp_last);
+        load_params<NPV>(sv_next, ov_next, rsrc_s, rsrc_o, has_offset, voff_p, (uint32_t)grp_next * param_pitch);
 #pragma unroll
-                        for (int q = 1; q < 4; q++) {
-                            const float inner = __builtin_fmaf(of, X[mt][q], P[mt][h * EPD + i][q]);
-                            tot[mt][h * EPD + i][q] = __builtin_fmaf(sc, inner, tot[mt][h * EPD + i][q]);
-                        }
+        for (int j = 0; j < BS; j++) {
+            const int slot = j % PF;
+            uint32_t w0[8], w1[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                w0[t] = wq[slot][t].x ^ (WBITS == 4 ? 0x88888888u : 0x80808080u);
+                w1[t] = wq[slot][t].y ^ (WBITS == 4 ? 0x88888888u : 0x80808080u);
+            }
+            u32x4 xa[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) xa[mt] = *reinterpret_cast<const u32x4 *>(xw + ((s + j) * MT + mt) * 1024);
+            // keep the order: wait for this slot, refill it, then compute
+            __builtin_amdgcn_sched_barrier(0);
+            load_step(wq[slot], rsrc_w, voff_w, p.ldw_bytes, (uint32_t)(step0 + s + j + PF) * 32u, s + j + PF < nsteps);
+            __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+#pragma unroll
+                for (int jb = 0; jb < EPD / 2; jb++) {
+                    u32x4 b0, b1;
+                    expand_pair<WBITS>(h ? w1 : w0, jb, magic, b0, b1);
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        const bf16x8 a = __builtin_bit_cast(bf16x8, xa[mt]);
+                        P[mt][h * EPD + 2 * jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, b0),
+                                                                                       P[mt][h * EPD + 2 * jb], 0, 0, 0);
+                        P[mt][h * EPD + 2 * jb + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            a, __builtin_bit_cast(bf16x8, b1), P[mt][h * EPD + 2 * jb + 1], 0, 0, 0);
                     }
                 }
             }
-        }
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            X[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int i = 0; i < NT; i++) P[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int mt = 0; mt < MT; mt++)
+                X[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[mt]),
+                                                                __builtin_bit_cast(bf16x8, ones), X[mt], 0, 0, 0);
         }
-    };
+        in_unit += BS;
+        if (in_unit == ustep) {
+            fold_group<WBITS, MT, NT, NPV>(tot, P, X, sv, ov, one_row);
+            in_unit = 0;
+        }
+    }
 
-    const int pro = nsteps < D ? nsteps : D;
-    for (int s = 0; s < pro; s++) issue(s);
-
-    for (int s = 0; s < nsteps; s++) {
-        // steps s+1 .. min(s+D-1, nsteps-1) may stay in flight; each has at least LOADS loads, so allowing
-        // ahead * LOADS outstanding loads guarantees that everything of step s has landed
-        const int ahead = min(D - 1, nsteps - 1 - s);
-        if (ahead >= 3) wait_vmcnt<3 * LOADS>();
-        else if (ahead == 2) wait_vmcnt<2 * LOADS>();
-        else if (ahead == 1) wait_vmcnt<1 * LOADS>();
-        else wait_vmcnt<0>();
-        const char *slot = ring + (s % D) * SLOT;
-        if (group_first(s)) {                 // first step of a group: take its parameters out of the slot
-            const char *pp = slot + 4096 + MT * 1024 + (2 * c) * EPD * 2;
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-                sv[h] = *reinterpret_cast<const PV *>(pp + h * EPD * 2);
-                ov[h] = *reinterpret_cast<const PV *>(pp + NB * 2 + h * EPD * 2);
-            }
-        }
-        uint32_t w0[8], w1[8];
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-            const u32x2 v = *reinterpret_cast<const u32x2 *>(slot + (8 * g + t) * 128 + c * 8);
-            w0[t] = v.x ^ (WBITS == 4 ? 0x88888888u : 0x80808080u);
-            w1[t] = v.y ^ (WBITS == 4 ? 0x88888888u : 0x80808080u);
-        }
-        u32x4 xa[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) xa[mt] = *reinterpret_cast<const u32x4 *>(slot + 4096 + mt * 1024 + lane * 16);
-        wait_lgkmcnt0();                      // the slot is in registers: it can be refilled
-        if (s + D < nsteps) issue(s + D);
-
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-#pragma unroll
-            for (int jb = 0; jb < EPD / 2; jb++) {
-                u32x4 b0, b1;
-                expand_pair<WBITS>(h ? w1 : w0, jb, magic, b0, b1);
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    const bf16x8 a = __builtin_bit_cast(bf16x8, xa[mt]);
-                    P[mt][h * EPD + 2 * jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, b0),
-                                                                                   P[mt][h * EPD + 2 * jb], 0, 0, 0);
-                    P[mt][h * EPD + 2 * jb + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        a, __builtin_bit_cast(bf16x8, b1), P[mt][h * EPD + 2 * jb + 1], 0, 0, 0);
-                }
-            }
-        }
+    // ---- reduce over the K slices: red[slice][row][column of the tile], rows_valid rows of NBW columns
+    int &is_last = *reinterpret_cast<int *>(lds);
+    float *red = reinterpret_cast<float *>(lds + 16);
+    __syncthreads();                          // the activation fragments are dead: their space is reused
+    if (lane_ok) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
-            X[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[mt]),
-                                                            __builtin_bit_cast(bf16x8, ones), X[mt], 0, 0, 0);
-        if (p.grouped && (s + 1) % p.unit_steps == 0) fold();
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int row = mt * 16 + 4 * g + q;
+                if (row >= rows_valid) continue;
+                float *dst = red + ((size_t)kslice * rows_valid + row) * NBW + wstrip * NB + (2 * c) * EPD;
+#pragma unroll
+                for (int i = 0; i < NT; i += 4)
+                    *reinterpret_cast<f32x4 *>(dst + i) = f32x4{tot[mt][i][q], tot[mt][i + 1][q], tot[mt][i + 2][q], tot[mt][i + 3][q]};
+            }
     }
-    if (!p.grouped && nsteps > 0) fold();
-
-    // ---- reduce over the wavefronts: red[wave][row][col], rows_valid rows of NB columns
-    __syncthreads();                          // every ring is drained: LDS can be reused
-    float *red = reinterpret_cast<float *>(lds);
-#pragma unroll
-    for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int row = mt * 16 + 4 * g + q;
-            if (row >= rows_valid) continue;
-            float *dst = red + ((size_t)wave * rows_valid + row) * NB + (2 * c) * EPD;
-#pragma unroll
-            for (int i = 0; i < NT; i++) dst[i] = tot[mt][i][q];
-        }
     __syncthreads();
-    // every thread owns quads of 4 consecutive columns of the [rows_valid x NB] tile
-    constexpr int QPR = NB / 4;
-    constexpr int THREADS = NWV * 64;
-    const int n0 = strip * NB;
+    // every thread owns quads of 4 consecutive columns of the [rows_valid x NBW] tile
+    constexpr int QPR = NBW / 4;
+    const int n0 = sgrp * NBW;
     const int nquads = rows_valid * QPR;
-    constexpr size_t RED_BYTES = (size_t)NWV * MT * 16 * NB * sizeof(float);
-    int &is_last = *reinterpret_cast<int *>(lds + RED_BYTES);   // just past the reduction buffer
-    auto sum_waves = [&](int qd) {
+    auto sum_slices = [&](int qd) {
         const int row = qd / QPR, nl = (qd % QPR) * 4;
-        f32x4 acc = *reinterpret_cast<const f32x4 *>(red + ((size_t)0 * rows_valid + row) * NB + nl);
+        f32x4 acc = *reinterpret_cast<const f32x4 *>(red + (size_t)row * NBW + nl);
 #pragma unroll
-        for (int wv = 1; wv < NWV; wv++) acc += *reinterpret_cast<const f32x4 *>(red + ((size_t)wv * rows_valid + row) * NB + nl);
+        for (int ks = 1; ks < KS; ks++) acc += *reinterpret_cast<const f32x4 *>(red + ((size_t)ks * rows_valid + row) * NBW + nl);
         return acc;
     };
     const bool out_vec = (p.ldo & 3) == 0 && aligned_dev(p.out, 8);
@@ -329,7 +371,7 @@ __global__ __launch_bounds__(NWV * 64) void wq_stream_kernel(const WqArgs p)
     };
     if (p.S == 1) {
         for (int qd = threadIdx.x; qd < nquads; qd += THREADS)
-            if (n0 + (qd % QPR) * 4 < p.N) store_out(qd, sum_waves(qd));
+            if (n0 + (qd % QPR) * 4 < p.N) store_out(qd, sum_slices(qd));
         return;
     }
     // K split over S workgroups: publish this chunk's partial, the last arrival adds them in chunk order.
@@ -346,12 +388,12 @@ __global__ __launch_bounds__(NWV * 64) void wq_stream_kernel(const WqArgs p)
     };
     for (int qd = threadIdx.x; qd < nquads; qd += THREADS) {
         if (n0 + (qd % QPR) * 4 >= p.N) continue;
-        const f32x4 v = sum_waves(qd);
+        const f32x4 v = sum_slices(qd);
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc_p, quad_off(qd), (uint32_t)chunk * chunk_bytes, SC1);
     }
     wait_vmcnt<0>();                          // this wavefront's partial sums have reached the coherence point
     __syncthreads();
-    uint32_t *cnt = p.counter + (size_t)blockIdx.y * p.strips + strip;
+    uint32_t *cnt = p.counter + (size_t)blockIdx.y * p.sgroups + sgrp;
     if (threadIdx.x == 0) {
         const uint32_t old = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = old == (uint32_t)(p.S - 1);
@@ -363,11 +405,12 @@ __global__ __launch_bounds__(NWV * 64) void wq_stream_kernel(const WqArgs p)
         const uint32_t off = quad_off(qd);
         f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int ch = 0; ch < p.S; ch += 4) {
-            // four loads in flight; chunks past S fall outside the buffer and read as zero
-            f32x4 v[4];
+            f32x4 v[4];                       // four loads in flight
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                v[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, off, (uint32_t)(ch + i) * chunk_bytes, SC1));
+                v[i] = ch + i < p.S ? __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                          rsrc_p, off, (uint32_t)(ch + i) * chunk_bytes, SC1))
+                                    : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < 4; i++) acc += v[i];
         }
@@ -408,13 +451,22 @@ __global__ __launch_bounds__(256) void wq_generic_kernel(const uint16_t *__restr
 struct WqPlan {
     bool fast;
     int mt, nwv;        // m tiles per workgroup, wavefronts per workgroup
-    int strips, mchunks, S;
+    int w;              // adjacent strips per workgroup
+    int strips, sgroups, mchunks, S;
     int unit_steps, n_units;
+    int bs;             // steps per loop body of the kernel
     size_t partial_bytes, counter_bytes;
+    size_t slab_bytes;  // activations of one K chunk in LDS
 };
 
+int env_int(const char *name)
+{
+    const char *e = getenv(name);
+    return e ? atoi(e) : 0;
+}
+
 WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size, bool n_major, int64_t ldw_k,
-                 int64_t ldx, const void *x, const void *w)
+                 int64_t ldx, const void *x, const void *w, const void *scale, const void *offset)
 {
     WqPlan pl{};
     const int64_t row_bytes = w_bits == 4 ? N / 2 : N;
@@ -422,49 +474,85 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
     const int64_t group = group_size > 0 ? group_size : K;
     pl.fast = K > 0 && K % 32 == 0 && group % 32 == 0 && n_major && row_bytes % 16 == 0 && ldw_bytes % 16 == 0 &&
               ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 16)) &&
-              (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 32) && (uint64_t)M * (uint64_t)ldx * 2 < (1ull << 32);
+              (scale == nullptr || aligned(scale, 16)) && (offset == nullptr || aligned(offset, 16)) &&
+              (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 32) && (uint64_t)M * (uint64_t)ldx * 2 < (1ull << 32) &&
+              (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 32);
     if (!pl.fast) return pl;
     pl.mt = M <= 16 ? 1 : 2;
     pl.nwv = pl.mt == 1 ? 8 : 4;
     pl.strips = (int)((row_bytes + 127) / 128);
     pl.mchunks = (int)((M + pl.mt * 16 - 1) / (pl.mt * 16));
     const bool grouped = group_size > 0 && group != K;
-    pl.unit_steps = grouped ? (int)(group / 32) : 1;
+    // loop body of 4, 2 or 1 steps: a scale group (per channel: the whole of K) must be a whole number of bodies
+    const int64_t span = (grouped ? group : K) / 32;
+    pl.bs = span % 4 == 0 ? 4 : span % 2 == 0 ? 2 : 1;
+    pl.unit_steps = grouped ? (int)(group / 32) : pl.bs;
     pl.n_units = (int)(K / (32 * pl.unit_steps));
+    // W adjacent strips per workgroup; the remaining wavefronts slice K.  Pairs of strips read DRAM markedly
+    // better, but halve the number of tiles: with few strips that means a deeper split of K and a longer exchange.
+    pl.w = pl.strips >= 112 ? 2 : 1;
+    if (const int f = env_int("MI355_WQ_W"))      // tuning aid
+        if (f == 1 || f == 2) pl.w = f;
+    pl.sgroups = (pl.strips + pl.w - 1) / pl.w;
+    const int ks = pl.nwv / pl.w;
     // split K over S workgroups until all CUs have work; every wavefront keeps at least one unit
-    int S = kNumCU / (pl.strips * pl.mchunks);
-    const int s_max = pl.n_units / pl.nwv;
+    int S = kNumCU / (pl.sgroups * pl.mchunks);
+    const int s_max = pl.n_units / ks;
     if (S > s_max) S = s_max;
     if (S > 16) S = 16;
     if (S < 1) S = 1;
-    if (const char *e = getenv("MI355_WQ_SPLIT")) { // debugging aid: force the number of K chunks
-        const int f = atoi(e);
+    // the activations of a workgroup's K chunk must fit in LDS (1 KiB per step and m tile)
+    constexpr int kMaxSlabSteps = (160 * 1024 - 16) / 1024;
+    auto slab_steps = [&](int chunks) { return (pl.n_units + chunks - 1) / chunks * pl.unit_steps * pl.mt; };
+    while (slab_steps(S) > kMaxSlabSteps && S < s_max) S++;
+    if (const int f = env_int("MI355_WQ_SPLIT"))  // tuning aid: force the number of K chunks
         if (f >= 1 && f <= s_max) S = f;
-    }
     if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1; // exchange offsets are 32-bit
+    if (slab_steps(S) > kMaxSlabSteps) {
+        pl.fast = false;
+        return pl;
+    }
     pl.S = S;
+    pl.slab_bytes = (size_t)slab_steps(S) * 1024;
     pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
-    pl.counter_bytes = S > 1 ? (((size_t)pl.strips * pl.mchunks * sizeof(uint32_t)) + 255) / 256 * 256 : 0;
+    pl.counter_bytes = S > 1 ? (((size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t)) + 255) / 256 * 256 : 0;
     return pl;
 }
 
-template <int WBITS, int MT, int NWV>
+template <int WBITS, int MT, int W, int KS, int BS>
 int launch_stream(const WqArgs &p, const WqPlan &pl, hipStream_t s)
 {
-    constexpr int EPD = 32 / WBITS, NB = 32 * EPD, SLOT = 4096 + MT * 1024 + NB * 4;
-    constexpr int D = (160 * 1024) / (NWV * SLOT) >= 4 ? 4 : (160 * 1024) / (NWV * SLOT);   // ring depth that fits LDS
-    static_assert(D >= 2, "ring depth");
-    constexpr size_t ring_bytes = (size_t)NWV * D * SLOT;
-    constexpr size_t red_bytes = (size_t)NWV * MT * 16 * NB * sizeof(float);
-    constexpr size_t lds_bytes = ring_bytes > red_bytes + 16 ? ring_bytes : red_bytes + 16;
-    static_assert(lds_bytes <= 160 * 1024, "LDS budget");
-    auto kern = wq_stream_kernel<WBITS, MT, NWV, D>;
+    constexpr int EPD = 32 / WBITS, NB = 32 * EPD;
+    constexpr int PF = BS >= 2 ? 2 : 1;
+    constexpr size_t max_lds = 16 + (size_t)KS * MT * 16 * W * NB * sizeof(float);
+    static_assert(max_lds <= 160 * 1024, "LDS budget");
+    const int rows = p.M < MT * 16 ? p.M : MT * 16;
+    const size_t red_bytes = (size_t)KS * rows * W * NB * sizeof(float);
+    const size_t lds_bytes = 16 + (red_bytes > pl.slab_bytes ? red_bytes : pl.slab_bytes);
+    auto kern = wq_stream_kernel<WBITS, MT, W, KS, BS, PF>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)((pl.strips + 7) / 8 * 8 * pl.S), (unsigned)pl.mchunks), dim3(NWV * 64), lds_bytes, s,
-                       p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((pl.sgroups + 7) / 8 * 8 * pl.S), (unsigned)pl.mchunks), dim3(W * KS * 64),
+                       lds_bytes, s, p);
     return check_launch();
+}
+
+template <int WBITS, int MT, int W, int KS>
+int launch_body(const WqArgs &p, const WqPlan &pl, hipStream_t s)
+{
+    switch (pl.bs) {
+    case 4: return launch_stream<WBITS, MT, W, KS, 4>(p, pl, s);
+    case 2: return launch_stream<WBITS, MT, W, KS, 2>(p, pl, s);
+    default: return launch_stream<WBITS, MT, W, KS, 1>(p, pl, s);
+    }
+}
+
+template <int WBITS>
+int launch_bits(const WqArgs &p, const WqPlan &pl, hipStream_t s)
+{
+    if (pl.mt == 1) return pl.w == 1 ? launch_body<WBITS, 1, 1, 8>(p, pl, s) : launch_body<WBITS, 1, 2, 4>(p, pl, s);
+    return pl.w == 1 ? launch_body<WBITS, 2, 1, 4>(p, pl, s) : launch_body<WBITS, 2, 2, 2>(p, pl, s);
 }
 
 } // namespace
@@ -475,7 +563,7 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
     using namespace mi355;
     if (M <= 0 || N <= 0 || K <= 0 || (w_bits != 4 && w_bits != 8) || group_size < 0) return 0;
     // the largest request over the layouts the streaming kernel accepts (row pitch = row length)
-    const WqPlan pl = make_plan(M, N, K, w_bits, group_size, true, w_bits == 4 ? N / 8 : N, K, nullptr, nullptr);
+    const WqPlan pl = make_plan(M, N, K, w_bits, group_size, true, w_bits == 4 ? N / 8 : N, K, nullptr, nullptr, nullptr, nullptr);
     return pl.fast ? pl.partial_bytes + pl.counter_bytes : 0;
 }
 
@@ -498,7 +586,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int 
     const int group = (int)(group_size > 0 ? group_size : (K > 0 ? K : 1));
 
     const bool n_major = w_bits == 4 || (ldw_n == 1 && ldw_k >= N);
-    const WqPlan pl = make_plan(M, N, K, w_bits, group_size, n_major, ldw_k, ldx, x_bf16, w);
+    const WqPlan pl = make_plan(M, N, K, w_bits, group_size, n_major, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
     if (!pl.fast) {
         hipLaunchKernelGGL(wq_generic_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((M + 3) / 4)), dim3(256), 0, s,
                            static_cast<const uint16_t *>(x_bf16), w, w_bits, static_cast<const uint16_t *>(scale_bf16),
@@ -531,7 +619,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int 
     p.n_units = pl.n_units;
     p.grouped = group_size > 0 && group != K;
     p.strips = pl.strips;
+    p.sgroups = pl.sgroups;
     p.S = pl.S;
-    if (w_bits == 4) return pl.mt == 1 ? launch_stream<4, 1, 8>(p, pl, s) : launch_stream<4, 2, 4>(p, pl, s);
-    return pl.mt == 1 ? launch_stream<8, 1, 8>(p, pl, s) : launch_stream<8, 2, 4>(p, pl, s);
+    return w_bits == 4 ? launch_bits<4>(p, pl, s) : launch_bits<8>(p, pl, s);
 }
