@@ -101,7 +101,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     const __amdgpu_buffer_rsrc_t rsrc_b =
         make_rsrc(p.bt + (int64_t)n0 * p.ldbt, (uint32_t)((int64_t)(rows_b - 1) * p.ldbt + p.K));
     const int rr = lane >> 3;
-    const int gchunk = ((lane & 7) ^ rr) * 16;
+    // row of the tile = 8 * unit + rr and unit = i * NW + wave with NW even: (row >> 1) & 7 = 4 * (wave & 1) + rr / 2
+    const int gchunk = ((lane & 7) ^ (((wave & 1) << 2) | (rr >> 1))) * 16;
     const uint32_t voff_a = (uint32_t)(rr * (int)p.lda + gchunk);
     const uint32_t voff_b = (uint32_t)(rr * (int)p.ldbt + gchunk);
     const uint32_t unit_stride_a = 8u * (uint32_t)p.lda, unit_stride_b = 8u * (uint32_t)p.ldbt;
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     // LDS read addressing: lane reads row (lane % 16) of a 16-row tile, 16-byte chunk (ks*4 + lane/16),
     // stored at slot chunk ^ (row % 8).  For ks = 1 the slot is the ks = 0 slot with bit 2 flipped.
     const int frow = lane & 15;
-    const int sw0 = ((lane >> 4) ^ (frow & 7)) * 16;
+    const int sw0 = ((lane >> 4) ^ ((frow >> 1) & 7)) * 16;
     const int a_off = (wm * WTM * 16 + frow) * BK;
     const int b_off = (BM + wn * WTN * 16 + frow) * BK;
 

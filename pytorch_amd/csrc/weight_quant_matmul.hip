@@ -113,14 +113,15 @@ __device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint
 // compiler then tracks the outstanding loads exactly); a step past the end of the wavefront's range is given a
 // lane offset beyond every buffer size instead, which makes the loads return zero without touching memory.
 constexpr uint32_t kOutOfRange = 0x80000000u;
-constexpr int kNonTemporal = 2;           // cache-policy bit: weights are read once, keep them out of the way of the reused data
+constexpr int kNonTemporal = 2;           // cache-policy bit for data that is read once
 
+template <int POLICY>
 __device__ __forceinline__ void load_step(u32x2 (&wq)[8], const __amdgpu_buffer_rsrc_t rsrc_w, const uint32_t voff_w,
                                           const uint32_t ldw_bytes, const uint32_t krow, const bool valid)
 {
     const uint32_t vw = valid ? voff_w : kOutOfRange;
 #pragma unroll
-    for (int t = 0; t < 8; t++) wq[t] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw, (krow + t) * ldw_bytes, kNonTemporal);
+    for (int t = 0; t < 8; t++) wq[t] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw, (krow + t) * ldw_bytes, POLICY);
 }
 
 // Antiquant parameters of one group for this lane's NPV * 8 consecutive columns.
@@ -173,11 +174,16 @@ __device__ __forceinline__ void fold_group(f32x4 (&tot)[MT][NT], f32x4 (&P)[MT][
 }
 
 // BS: steps per loop body (every wavefront's range and every scale group is a whole number of bodies);
-// PF: steps kept in flight (PF divides BS or equals it).
-template <int WBITS, int MT, int W, int KS, int BS, int PF>
+// PF: steps kept in flight (PF divides BS or equals it);
+// ACCUM: a wavefront may meet more than one scale group, so finished groups are folded into a running total
+// inside the loop.  Without it (per channel, or at most one group per wavefront) the single fold happens after
+// the loop and the loop carries half as many accumulators.
+template <int WBITS, int MT, int W, int KS, int BS, int PF, bool ACCUM>
 __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
 {
     static_assert(BS % PF == 0, "the register ring must divide the loop body");
+    // with one m tile the weights are read exactly once; with more, other workgroups read the same strip again
+    constexpr int POLICY = MT == 1 ? kNonTemporal : 0;
     constexpr int EPD = 32 / WBITS;            // elements per dword
     constexpr int NB = 32 * EPD;               // columns per strip (128 bytes of a weight row)
     constexpr int NT = 2 * EPD;                // MFMA column sets per lane (it holds 2 dword columns)
@@ -224,7 +230,7 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
         X[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < NT; i++) {
-            tot[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if constexpr (ACCUM) tot[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
             P[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
     }
@@ -246,7 +252,7 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
     load_params<NPV>(sv_next, ov_next, rsrc_s, rsrc_o, has_offset, voff_p, (uint32_t)grp_next * param_pitch);
 #pragma unroll
     for (int j = 0; j < PF; j++)
-        load_step(wq[j], rsrc_w, voff_w, p.ldw_bytes, (uint32_t)(step0 + j) * 32u, j < nsteps);
+        load_step<POLICY>(wq[j], rsrc_w, voff_w, p.ldw_bytes, (uint32_t)(step0 + j) * 32u, j < nsteps);
 
     // The activations of the workgroup's K chunk go to LDS once, already in MFMA operand order: the fragment of
     // (step, m tile) is 1 KiB, lane (c, g) finds x[m tile * 16 + c][32 * step + 8g .. + 7] at lane * 16.  The global
@@ -295,7 +301,7 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
             for (int mt = 0; mt < MT; mt++) xa[mt] = *reinterpret_cast<const u32x4 *>(xw + ((s + j) * MT + mt) * 1024);
             // keep the order: wait for this slot, refill it, then compute
             __builtin_amdgcn_sched_barrier(0);
-            load_step(wq[slot], rsrc_w, voff_w, p.ldw_bytes, (uint32_t)(step0 + s + j + PF) * 32u, s + j + PF < nsteps);
+            load_step<POLICY>(wq[slot], rsrc_w, voff_w, p.ldw_bytes, (uint32_t)(step0 + s + j + PF) * 32u, s + j + PF < nsteps);
             __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
@@ -319,45 +325,30 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
                 X[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[mt]),
                                                                 __builtin_bit_cast(bf16x8, ones), X[mt], 0, 0, 0);
         }
-        in_unit += BS;
-        if (in_unit == ustep) {
-            fold_group<WBITS, MT, NT, NPV>(tot, P, X, sv, ov, one_row);
-            in_unit = 0;
+        if constexpr (ACCUM) {
+            in_unit += BS;
+            if (in_unit == ustep) {
+                fold_group<WBITS, MT, NT, NPV>(tot, P, X, sv, ov, one_row);
+                in_unit = 0;
+            }
         }
     }
-
-    // ---- reduce over the K slices: red[slice][row][column of the tile], rows_valid rows of NBW columns
-    int &is_last = *reinterpret_cast<int *>(lds);
-    float *red = reinterpret_cast<float *>(lds + 16);
-    __syncthreads();                          // the activation fragments are dead: their space is reused
-    if (lane_ok) {
+    if constexpr (!ACCUM) {
+        // the wavefront met a single parameter row: one fold, and the running total only starts to exist here
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int row = mt * 16 + 4 * g + q;
-                if (row >= rows_valid) continue;
-                float *dst = red + ((size_t)kslice * rows_valid + row) * NBW + wstrip * NB + (2 * c) * EPD;
-#pragma unroll
-                for (int i = 0; i < NT; i += 4)
-                    *reinterpret_cast<f32x4 *>(dst + i) = f32x4{tot[mt][i][q], tot[mt][i + 1][q], tot[mt][i + 2][q], tot[mt][i + 3][q]};
-            }
+            for (int i = 0; i < NT; i++) tot[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        fold_group<WBITS, MT, NT, NPV>(tot, P, X, sv, ov, one_row);
     }
-    __syncthreads();
-    // every thread owns quads of 4 consecutive columns of the [rows_valid x NBW] tile
-    constexpr int QPR = NBW / 4;
+
+    // ---- reduce over the K slices, one m tile at a time: red[slice][row of the m tile][column of the tile]
+    int &is_last = *reinterpret_cast<int *>(lds);
+    float *red = reinterpret_cast<float *>(lds + 16);
+    constexpr int QPR = NBW / 4;              // every thread owns quads of 4 consecutive columns
     const int n0 = sgrp * NBW;
-    const int nquads = rows_valid * QPR;
-    auto sum_slices = [&](int qd) {
-        const int row = qd / QPR, nl = (qd % QPR) * 4;
-        f32x4 acc = *reinterpret_cast<const f32x4 *>(red + (size_t)row * NBW + nl);
-#pragma unroll
-        for (int ks = 1; ks < KS; ks++) acc += *reinterpret_cast<const f32x4 *>(red + ((size_t)ks * rows_valid + row) * NBW + nl);
-        return acc;
-    };
     const bool out_vec = (p.ldo & 3) == 0 && aligned_dev(p.out, 8);
-    auto store_out = [&](int qd, f32x4 v) {
-        const int row = qd / QPR, nl = (qd % QPR) * 4;
+    auto store_out = [&](int row, int nl, f32x4 v) {
         uint16_t *o = p.out + (int64_t)(m_base + row) * p.ldo + n0 + nl;
         if (out_vec) {
             u32x2 pk;
@@ -369,28 +360,45 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
             for (int i = 0; i < 4; i++) o[i] = f32_to_bf16(v[i]);
         }
     };
-    if (p.S == 1) {
-        for (int qd = threadIdx.x; qd < nquads; qd += THREADS)
-            if (n0 + (qd % QPR) * 4 < p.N) store_out(qd, sum_slices(qd));
-        return;
-    }
-    // K split over S workgroups: publish this chunk's partial, the last arrival adds them in chunk order.
+    // K split over S workgroups: every workgroup publishes its partial, the last arrival adds them in chunk order.
     // The exchange uses agent-scope (sc1) write-through stores and cache-bypassing loads, ordered by the
     // wavefronts' own store counters, the workgroup barrier and a relaxed agent-scope counter; a full
     // release/acquire fence would write back and invalidate the whole L2 of the XCD, which costs far
     // more than the kernel itself.
     constexpr int SC1 = 16;                   // cache-policy bit: agent scope
     const uint32_t chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
-    const __amdgpu_buffer_rsrc_t rsrc_p = make_rsrc(p.partial, chunk_bytes * (uint32_t)p.S);
-    auto quad_off = [&](int qd) {
-        const int row = qd / QPR, nl = (qd % QPR) * 4;
-        return (uint32_t)(((m_base + row) * p.N + n0 + nl) * 4);
-    };
-    for (int qd = threadIdx.x; qd < nquads; qd += THREADS) {
-        if (n0 + (qd % QPR) * 4 >= p.N) continue;
-        const f32x4 v = sum_slices(qd);
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc_p, quad_off(qd), (uint32_t)chunk * chunk_bytes, SC1);
+    const __amdgpu_buffer_rsrc_t rsrc_p = make_rsrc(p.partial, p.S > 1 ? chunk_bytes * (uint32_t)p.S : 0u);
+    auto partial_off = [&](int row, int nl) { return (uint32_t)(((m_base + row) * p.N + n0 + nl) * 4); };
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const int rows_mt = min(16, rows_valid - mt * 16);
+        __syncthreads();                      // the activation fragments / the previous m tile's sums are dead
+        if (lane_ok) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int row = 4 * g + q;
+                if (row >= rows_mt) continue;
+                float *dst = red + ((size_t)kslice * 16 + row) * NBW + wstrip * NB + (2 * c) * EPD;
+#pragma unroll
+                for (int i = 0; i < NT; i += 4)
+                    *reinterpret_cast<f32x4 *>(dst + i) = f32x4{tot[mt][i][q], tot[mt][i + 1][q], tot[mt][i + 2][q], tot[mt][i + 3][q]};
+            }
+        }
+        __syncthreads();
+        for (int qd = threadIdx.x; qd < rows_mt * QPR; qd += THREADS) {
+            const int row = qd / QPR, nl = (qd % QPR) * 4;
+            if (n0 + nl >= p.N) continue;
+            f32x4 acc = *reinterpret_cast<const f32x4 *>(red + (size_t)row * NBW + nl);
+#pragma unroll
+            for (int ks = 1; ks < KS; ks++) acc += *reinterpret_cast<const f32x4 *>(red + ((size_t)ks * 16 + row) * NBW + nl);
+            if (p.S == 1)
+                store_out(mt * 16 + row, nl, acc);
+            else
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), rsrc_p, partial_off(mt * 16 + row, nl),
+                                                       (uint32_t)chunk * chunk_bytes, SC1);
+        }
     }
+    if (p.S == 1) return;
     wait_vmcnt<0>();                          // this wavefront's partial sums have reached the coherence point
     __syncthreads();
     uint32_t *cnt = p.counter + (size_t)blockIdx.y * p.sgroups + sgrp;
@@ -400,21 +408,22 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
     }
     __syncthreads();
     if (!is_last) return;
-    for (int qd = threadIdx.x; qd < nquads; qd += THREADS) {
-        if (n0 + (qd % QPR) * 4 >= p.N) continue;
-        const uint32_t off = quad_off(qd);
+    for (int qd = threadIdx.x; qd < rows_valid * QPR; qd += THREADS) {
+        const int row = qd / QPR, nl = (qd % QPR) * 4;
+        if (n0 + nl >= p.N) continue;
+        const uint32_t off = partial_off(row, nl);
         f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-        for (int ch = 0; ch < p.S; ch += 4) {
-            f32x4 v[4];                       // four loads in flight
+        for (int ch = 0; ch < p.S; ch += 8) {
+            f32x4 v[8];                       // eight loads in flight
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int i = 0; i < 8; i++)
                 v[i] = ch + i < p.S ? __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
                                           rsrc_p, off, (uint32_t)(ch + i) * chunk_bytes, SC1))
                                     : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc += v[i];
+            for (int i = 0; i < 8; i++) acc += v[i];
         }
-        store_out(qd, acc);
+        store_out(row, nl, acc);
     }
     if (threadIdx.x == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
 }
@@ -450,8 +459,9 @@ __global__ __launch_bounds__(256) void wq_generic_kernel(const uint16_t *__restr
 
 struct WqPlan {
     bool fast;
-    int mt, nwv;        // m tiles per workgroup, wavefronts per workgroup
-    int w;              // adjacent strips per workgroup
+    int mt;             // m tiles (16 rows) per workgroup
+    int w, ks;          // adjacent strips per workgroup, K slices per workgroup: w * ks wavefronts
+    bool accum;         // a wavefront may meet more than one scale group
     int strips, sgroups, mchunks, S;
     int unit_steps, n_units;
     int bs;             // steps per loop body of the kernel
@@ -479,13 +489,12 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
               (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 32);
     if (!pl.fast) return pl;
     pl.mt = M <= 16 ? 1 : 2;
-    pl.nwv = pl.mt == 1 ? 8 : 4;
     pl.strips = (int)((row_bytes + 127) / 128);
     pl.mchunks = (int)((M + pl.mt * 16 - 1) / (pl.mt * 16));
     const bool grouped = group_size > 0 && group != K;
-    // loop body of 4, 2 or 1 steps: a scale group (per channel: the whole of K) must be a whole number of bodies
+    // loop body of 4 steps when a scale group (per channel: the whole of K) is a whole number of them, else 1 step
     const int64_t span = (grouped ? group : K) / 32;
-    pl.bs = span % 4 == 0 ? 4 : span % 2 == 0 ? 2 : 1;
+    pl.bs = span % 4 == 0 ? 4 : 1;
     pl.unit_steps = grouped ? (int)(group / 32) : pl.bs;
     pl.n_units = (int)(K / (32 * pl.unit_steps));
     // W adjacent strips per workgroup; the remaining wavefronts slice K.  Pairs of strips read DRAM markedly
@@ -494,42 +503,50 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
     if (const int f = env_int("MI355_WQ_W"))      // tuning aid
         if (f == 1 || f == 2) pl.w = f;
     pl.sgroups = (pl.strips + pl.w - 1) / pl.w;
-    const int ks = pl.nwv / pl.w;
-    // split K over S workgroups until all CUs have work; every wavefront keeps at least one unit
-    int S = kNumCU / (pl.sgroups * pl.mchunks);
-    const int s_max = pl.n_units / ks;
-    if (S > s_max) S = s_max;
-    if (S > 16) S = 16;
-    if (S < 1) S = 1;
-    // the activations of a workgroup's K chunk must fit in LDS (1 KiB per step and m tile)
     constexpr int kMaxSlabSteps = (160 * 1024 - 16) / 1024;
-    auto slab_steps = [&](int chunks) { return (pl.n_units + chunks - 1) / chunks * pl.unit_steps * pl.mt; };
-    while (slab_steps(S) > kMaxSlabSteps && S < s_max) S++;
-    if (const int f = env_int("MI355_WQ_SPLIT"))  // tuning aid: force the number of K chunks
-        if (f >= 1 && f <= s_max) S = f;
-    if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1; // exchange offsets are 32-bit
-    if (slab_steps(S) > kMaxSlabSteps) {
-        pl.fast = false;
-        return pl;
+    // Eight wavefronts per workgroup, except where the accumulators of two m tiles plus a running total need the
+    // whole register file of a SIMD (int4, several groups per wavefront): then four.
+    for (int nwv = 8; nwv >= 4; nwv -= 4) {
+        pl.ks = nwv / pl.w;
+        // split K over S workgroups until all CUs have work; every wavefront keeps at least one unit
+        int S = kNumCU / (pl.sgroups * pl.mchunks);
+        const int s_max = pl.n_units / pl.ks > 0 ? pl.n_units / pl.ks : 1;
+        if (S > s_max) S = s_max;
+        if (S > 16) S = 16;
+        if (S < 1) S = 1;
+        // the activations of a workgroup's K chunk must fit in LDS (1 KiB per step and m tile)
+        auto slab_steps = [&](int chunks) { return (pl.n_units + chunks - 1) / chunks * pl.unit_steps * pl.mt; };
+        while (slab_steps(S) > kMaxSlabSteps && S < s_max) S++;
+        if (const int f = env_int("MI355_WQ_SPLIT"))  // tuning aid: force the number of K chunks
+            if (f >= 1 && f <= s_max) S = f;
+        if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1; // exchange offsets are 32-bit
+        pl.S = S;
+        pl.slab_bytes = (size_t)slab_steps(S) * 1024;
+        pl.accum = grouped && (pl.n_units + S * pl.ks - 1) / (S * pl.ks) > 1;
+        if (pl.bs == 1) pl.accum = true;              // only instantiated with the running total
+        if (slab_steps(S) > kMaxSlabSteps) {
+            pl.fast = false;
+            return pl;
+        }
+        if (!(w_bits == 4 && pl.mt == 2 && pl.accum)) break;
     }
-    pl.S = S;
-    pl.slab_bytes = (size_t)slab_steps(S) * 1024;
-    pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
-    pl.counter_bytes = S > 1 ? (((size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t)) + 255) / 256 * 256 : 0;
+    pl.partial_bytes = pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0;
+    pl.counter_bytes = pl.S > 1 ? (((size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t)) + 255) / 256 * 256 : 0;
     return pl;
 }
 
-template <int WBITS, int MT, int W, int KS, int BS>
+template <int WBITS, int MT, int W, int KS, int BS, bool ACCUM>
 int launch_stream(const WqArgs &p, const WqPlan &pl, hipStream_t s)
 {
     constexpr int EPD = 32 / WBITS, NB = 32 * EPD;
-    constexpr int PF = BS >= 2 ? 2 : 1;
-    constexpr size_t max_lds = 16 + (size_t)KS * MT * 16 * W * NB * sizeof(float);
-    static_assert(max_lds <= 160 * 1024, "LDS budget");
-    const int rows = p.M < MT * 16 ? p.M : MT * 16;
-    const size_t red_bytes = (size_t)KS * rows * W * NB * sizeof(float);
+    // Steps in flight per wavefront.  Measured: deeper register rings only lengthen the queues in front of HBM
+    // (int4, K = 4096: 11.8 / 12.7 / 13.6 us with 1 / 2 / 4 steps; int8, K = 8192: 46.5 / 46.1 / 47.9 us).
+    // Four-wavefront workgroups (int4, two m tiles, running total) have half the loads in flight: two steps.
+    constexpr int PF = BS > 1 && (WBITS == 8 || W * KS == 4) ? 2 : 1;
+    constexpr size_t red_bytes = (size_t)KS * 16 * W * NB * sizeof(float);
+    static_assert(16 + red_bytes <= 160 * 1024, "LDS budget");
     const size_t lds_bytes = 16 + (red_bytes > pl.slab_bytes ? red_bytes : pl.slab_bytes);
-    auto kern = wq_stream_kernel<WBITS, MT, W, KS, BS, PF>;
+    auto kern = wq_stream_kernel<WBITS, MT, W, KS, BS, PF, ACCUM>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
@@ -538,21 +555,31 @@ int launch_stream(const WqArgs &p, const WqPlan &pl, hipStream_t s)
     return check_launch();
 }
 
-template <int WBITS, int MT, int W, int KS>
+// ACC_MODES: 0 = both accumulation modes are instantiated, 1 = only the running total, 2 = only the single fold
+template <int WBITS, int MT, int W, int KS, int ACC_MODES>
 int launch_body(const WqArgs &p, const WqPlan &pl, hipStream_t s)
 {
-    switch (pl.bs) {
-    case 4: return launch_stream<WBITS, MT, W, KS, 4>(p, pl, s);
-    case 2: return launch_stream<WBITS, MT, W, KS, 2>(p, pl, s);
-    default: return launch_stream<WBITS, MT, W, KS, 1>(p, pl, s);
+    if constexpr (ACC_MODES != 2) {
+        if (pl.bs == 1) return launch_stream<WBITS, MT, W, KS, 1, true>(p, pl, s);
+        if (pl.accum) return launch_stream<WBITS, MT, W, KS, 4, true>(p, pl, s);
     }
+    if constexpr (ACC_MODES != 1) {
+        if (pl.bs == 4 && !pl.accum) return launch_stream<WBITS, MT, W, KS, 4, false>(p, pl, s);
+    }
+    return MI355_ERR_UNSUPPORTED;
 }
 
 template <int WBITS>
 int launch_bits(const WqArgs &p, const WqPlan &pl, hipStream_t s)
 {
-    if (pl.mt == 1) return pl.w == 1 ? launch_body<WBITS, 1, 1, 8>(p, pl, s) : launch_body<WBITS, 1, 2, 4>(p, pl, s);
-    return pl.w == 1 ? launch_body<WBITS, 2, 1, 4>(p, pl, s) : launch_body<WBITS, 2, 2, 2>(p, pl, s);
+    if (pl.mt == 1) return pl.w == 1 ? launch_body<WBITS, 1, 1, 8, 0>(p, pl, s) : launch_body<WBITS, 1, 2, 4, 0>(p, pl, s);
+    if constexpr (WBITS == 8) {
+        return pl.w == 1 ? launch_body<8, 2, 1, 8, 0>(p, pl, s) : launch_body<8, 2, 2, 4, 0>(p, pl, s);
+    } else {
+        // two m tiles of int4: eight wavefronts only without the running total (see make_plan)
+        if (pl.w * pl.ks == 8) return pl.w == 1 ? launch_body<4, 2, 1, 8, 2>(p, pl, s) : launch_body<4, 2, 2, 4, 2>(p, pl, s);
+        return pl.w == 1 ? launch_body<4, 2, 1, 4, 1>(p, pl, s) : launch_body<4, 2, 2, 2, 1>(p, pl, s);
+    }
 }
 
 } // namespace
