@@ -77,7 +77,11 @@ int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth,
  *   bias            bf16 [N] or NULL (MI355_OUT_BF16 only)
  *   out_dtype MI355_OUT_BF16:  out[m*ldc+n] = bf16(((float(acc) * pertoken_scale[m]) * scale[n]) + float(bias[n]))
  *             MI355_OUT_INT32: out[m*ldc+n] = acc (scales and bias are ignored and may be NULL)
- *   workspace: at least mi355_quant_matmul_workspace(...) bytes (may be NULL when that is 0)
+ *   workspace: at least mi355_quant_matmul_workspace(...) bytes (may be NULL when that is 0), 16-byte aligned.
+ *              It holds a transposed copy of a contiguous [K,N] weight and, for narrow outputs with a long K,
+ *              the partial sums and arrival counters of a split over K.  The counters lie at its start and
+ *              must be zero before the first launch that uses the buffer; every launch leaves them zero, so
+ *              one zero-initialised buffer can serve all later launches on the same stream.
  */
 size_t mi355_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n);
 

@@ -93,7 +93,7 @@ def quant_matmul(x1, x2, scale, pertoken_scale=None, bias=None, out_dtype=torch.
     out = torch.empty((M, N), dtype=out_dtype, device=x1.device)
     need = lib().mi355_quant_matmul_workspace(M, N, K, x2.stride(0), x2.stride(1))
     if workspace is None and need:
-        workspace = torch.empty(need, dtype=torch.int8, device=x1.device)
+        workspace = _wq_workspace(x1.device, need)      # its leading counters must start at zero
     st = lib().mi355_quant_matmul(_ptr(x1), _ptr(x2), _ptr(pertoken_scale), _ptr(scale),
                                   0 if scale is None else scale.numel(), _ptr(bias), _ptr(out),
                                   0 if out_dtype == torch.bfloat16 else 1, M, N, K, x1.stride(0),

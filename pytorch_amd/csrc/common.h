@@ -31,6 +31,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
     return __builtin_bit_cast(uint32_t, v);
 }
 
+// Every workspace of this library starts with this many bytes of arrival counters (zero before the first launch,
+// left zero by every launch); whatever else a launch keeps in the workspace lies behind them, so one
+// zero-initialised buffer can be shared by all launches of a stream.
+constexpr size_t kWorkspaceCounterBytes = 16384;
+
 inline int check_launch()
 {
     return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ERR_LAUNCH;

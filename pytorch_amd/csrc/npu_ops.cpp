@@ -119,6 +119,21 @@ std::tuple<Tensor, Tensor> dynamic_quant_hip(const Tensor &input, const optional
     return {y, scale};
 }
 
+// The split-K reductions of the matmul kernels count arrivals in their workspace: the counters must
+// be zero before a launch and the kernels leave them zero.  One zero-initialised buffer per
+// (device, stream) is kept and reused; launches on one stream are ordered, so they never overlap.
+Tensor zeroed_workspace(const Tensor &like, size_t bytes)
+{
+    static std::mutex mu;
+    static std::map<std::pair<int, void *>, Tensor> cache;
+    std::lock_guard<std::mutex> lock(mu);
+    const auto key = std::make_pair((int)like.device().index(), stream_of(like));
+    Tensor &ws = cache[key];
+    if (!ws.defined() || (size_t)ws.numel() < bytes)
+        ws = at::zeros({(int64_t)std::max<size_t>(bytes, (size_t)1 << 20)}, like.options().dtype(at::kChar));
+    return ws;
+}
+
 // ---------------------------------------------------------------- npu_quant_matmul
 
 struct QmmPlan {
@@ -237,7 +252,7 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
         const int64_t m = a.size(0);
         Tensor ws;
         const size_t ws_bytes = mi355_quant_matmul_workspace(m, p.N, p.K, w.stride(0), w.stride(1));
-        if (ws_bytes) ws = at::empty({(int64_t)ws_bytes}, x1.options().dtype(at::kChar));
+        if (ws_bytes) ws = zeroed_workspace(x1, ws_bytes);
         Tensor o = out2d.narrow(0, row0, m);
         check_status(mi355_quant_matmul(a.data_ptr<int8_t>(), w.data_ptr<int8_t>(), ps.defined() ? ps.data_ptr<float>() : nullptr,
                                         bf16 ? scale_f.data_ptr<float>() : nullptr, bf16 ? scale_f.numel() : 0,
@@ -306,21 +321,6 @@ Tensor weight_quant_meta(const Tensor &x, const Tensor &weight, const Tensor &an
     WqPlan p = weight_quant_plan(x, weight, antiquant_scale, antiquant_offset, quant_scale, quant_offset, bias, group_size,
                                  inner_precise, weight_dtype);
     return at::empty(p.out_shape, x.options());
-}
-
-// The split-K reduction of the weight-quant kernel counts arrivals in its workspace: the counters
-// must be zero before a launch and the kernel leaves them zero.  One zero-initialised buffer per
-// (device, stream) is kept and reused; launches on one stream are ordered, so they never overlap.
-Tensor zeroed_workspace(const Tensor &like, size_t bytes)
-{
-    static std::mutex mu;
-    static std::map<std::pair<int, void *>, Tensor> cache;
-    std::lock_guard<std::mutex> lock(mu);
-    const auto key = std::make_pair((int)like.device().index(), stream_of(like));
-    Tensor &ws = cache[key];
-    if (!ws.defined() || (size_t)ws.numel() < bytes)
-        ws = at::zeros({(int64_t)std::max<size_t>(bytes, (size_t)1 << 20)}, like.options().dtype(at::kChar));
-    return ws;
 }
 
 Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &antiquant_scale,

@@ -65,6 +65,9 @@ struct QmmArgs {
     int scale_len;
     int out_i32;
     int tiles_m, tiles_n, tiles_per_xcd;
+    int S;                     // workgroups that share the K range of a tile
+    int32_t *partial;          // workspace [tile][chunk][wavefront][accumulator quad][lane] int32x4 (S > 1)
+    uint32_t *counter;         // workspace [tile], zero on entry, left zero (S > 1)
 };
 
 // WGM x WGN wavefronts per workgroup, each owning (16*WTM) x (16*WTN) of the output tile.
@@ -84,7 +87,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     // a private L2; give every XCD a contiguous run of tiles, M fastest, so its workgroups
     // share weight columns.
     const int xcd = blockIdx.x & 7;
-    const int tile = xcd * p.tiles_per_xcd + (blockIdx.x >> 3);
+    const int slot = blockIdx.x >> 3;
+    const int tile = xcd * p.tiles_per_xcd + slot % p.tiles_per_xcd;
+    const int chunk = slot / p.tiles_per_xcd;                // K chunk of this workgroup (split K)
     if (tile >= p.tiles_m * p.tiles_n) return;
     const int m0 = (tile % p.tiles_m) * BM;
     const int n0 = (tile / p.tiles_m) * BN;
@@ -161,10 +166,11 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     // "at most c*L loads outstanding" means "everything but the newest c stages has landed".
     constexpr int L = LOADS_PER_STAGE;
     static_assert(NS >= 2 && NS <= 4, "stage count");
-    const int KT = p.K / BK;
+    const int kt0 = (int)((int64_t)(p.K / BK) * chunk / p.S);
+    const int KT = (int)((int64_t)(p.K / BK) * (chunk + 1) / p.S) - kt0;
     {
         const int pro = KT < NS ? KT : NS;
-        for (int s = 0; s < pro; s++) issue_stage(s * BK, lds + s * STAGE_BYTES);
+        for (int s = 0; s < pro; s++) issue_stage((kt0 + s) * BK, lds + s * STAGE_BYTES);
         if (pro >= 4) wait_vmcnt<3 * L>();
         else if (pro == 3) wait_vmcnt<2 * L>();
         else if (pro == 2) wait_vmcnt<1 * L>();
@@ -186,7 +192,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         else if (newer == 1) wait_vmcnt_lgkm0<1 * L>();
         else wait_vmcnt_lgkm0<0>();
         __syncthreads();
-        if (kt + NS < KT) issue_stage((kt + NS) * BK, lds + (kt % NS) * STAGE_BYTES);
+        if (kt + NS < KT) issue_stage((kt0 + kt + NS) * BK, lds + (kt % NS) * STAGE_BYTES);
         if (kt + 1 < KT) MI355_READ_FRAGS(af0, bf0, nxt, 0)
         __builtin_amdgcn_sched_barrier(0);
         MI355_MFMA_BLOCK(af1, bf1)
@@ -194,6 +200,47 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     }
 #undef MI355_READ_FRAGS
 #undef MI355_MFMA_BLOCK
+
+    if (p.S > 1) {
+        // Split K: every workgroup of the tile publishes its int32 partial sums in register order (16 bytes per
+        // lane, fully coalesced); the one that arrives last at the tile's counter adds the others to its own and
+        // runs the epilogue.  Integer addition is exact, so the result does not depend on the order of arrival.
+        // Publication uses agent-scope (sc1) write-through stores and cache-bypassing loads, ordered by the
+        // wavefronts' own store counters, the workgroup barrier and a relaxed agent-scope counter (a full
+        // release/acquire fence would write back and invalidate the whole L2 of the XCD).
+        constexpr int SC1 = 16;
+        constexpr uint32_t WAVE_BYTES = WTM * WTN * 64 * 16;
+        constexpr uint32_t CHUNK_BYTES = NW * WAVE_BYTES;
+        const __amdgpu_buffer_rsrc_t rsrc_p = make_rsrc(p.partial + (size_t)tile * p.S * (CHUNK_BYTES / 4), (uint32_t)p.S * CHUNK_BYTES);
+        const uint32_t lane_off = (uint32_t)wave * WAVE_BYTES + (uint32_t)lane * 16u;
+#pragma unroll
+        for (int i = 0; i < WTM; i++)
+#pragma unroll
+            for (int j = 0; j < WTN; j++)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rsrc_p, lane_off + (i * WTN + j) * 1024,
+                                                       (uint32_t)chunk * CHUNK_BYTES, SC1);
+        wait_vmcnt<0>();                                          // this wavefront's partial sums have reached the coherence point
+        __syncthreads();                                          // (also: every wavefront is done with the LDS stages)
+        int &is_last = *reinterpret_cast<int *>(lds);
+        if (threadIdx.x == 0) {
+            const uint32_t old = __hip_atomic_fetch_add(p.counter + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = old == (uint32_t)(p.S - 1);
+        }
+        __syncthreads();
+        const bool last = is_last != 0;
+        __syncthreads();                                          // the flag's LDS word is reused by the epilogue
+        if (!last) return;
+        for (int ch = 0; ch < p.S; ch++) {
+            if (ch == chunk) continue;
+#pragma unroll
+            for (int i = 0; i < WTM; i++)
+#pragma unroll
+                for (int j = 0; j < WTN; j++)
+                    acc[i][j] += __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(
+                        rsrc_p, lane_off + (i * WTN + j) * 1024, (uint32_t)ch * CHUNK_BYTES, SC1));
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(p.counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 
     // Epilogue.  The weight fragment was the first MFMA operand, so
     // acc[i][j][r] = C[m = tile row (lane % 16)][n = 4 * (lane / 16) + r].
@@ -394,11 +441,12 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     p.tiles_n = (p.N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
+    if (p.S > 1 && (uint64_t)p.S * BM * BN * 4 >= (1ull << 32)) return MI355_ERR_UNSUPPORTED;
     auto kern = qmm_kernel<WGM, WGN, WTM, WTN, NS>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(8 * p.tiles_per_xcd), dim3(WGM * WGN * 64), lds_bytes, s, p);
+    hipLaunchKernelGGL(kern, dim3(8 * p.tiles_per_xcd * p.S), dim3(WGM * WGN * 64), lds_bytes, s, p);
     return check_launch();
 }
 
@@ -435,16 +483,50 @@ TileChoice choose_tile(int M, int N)
     return best;
 }
 
+// Workspace layout: [arrival counters | split-K partial sums | transposed weight].
+struct QmmPlan {
+    TileChoice tile;
+    int S;                       // K chunks per tile
+    size_t counter_bytes, partial_bytes, transpose_bytes;
+};
+
+QmmPlan make_qmm_plan(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n)
+{
+    QmmPlan pl{};
+    pl.tile = choose_tile((int)M, (int)N);
+    pl.S = 1;
+    const bool tiled_shape = K >= BK && K % BK == 0;
+    if (tiled_shape) {
+        // Few tiles and a long K (the narrow GEMMs of small batches): split K until the CUs are busy, keeping at
+        // least four K steps per workgroup.
+        const int64_t tiles = ((M + pl.tile.bm - 1) / pl.tile.bm) * ((N + pl.tile.bn - 1) / pl.tile.bn);
+        const int64_t kt = K / BK;
+        int64_t S = tiles <= 128 ? 256 / tiles : 1;
+        if (S > kt / 4) S = kt / 4;
+        if (S > 16) S = 16;
+        if (S < 1) S = 1;
+        if (const char *e = getenv("MI355_QMM_SPLIT")) { // debugging aid
+            const int f = atoi(e);
+            if (f >= 1 && f <= kt) S = f;
+        }
+        pl.S = (int)S;
+        if (pl.S > 1) pl.partial_bytes = (size_t)tiles * pl.S * pl.tile.bm * pl.tile.bn * 4;   // tiles <= 128 counters
+    }
+    // a contiguous [K,N] weight is transposed into the workspace
+    pl.transpose_bytes = tiled_shape && ldb_k != 1 && ldb_n == 1 ? (size_t)N * (size_t)K : 0;
+    pl.counter_bytes = pl.partial_bytes + pl.transpose_bytes > 0 ? kWorkspaceCounterBytes : 0;
+    return pl;
+}
+
 } // namespace
 } // namespace mi355
 
 extern "C" size_t mi355_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n)
 {
-    (void)M;
-    (void)ldb_k;
-    if (N <= 0 || K <= 0) return 0;
-    // a contiguous [K,N] weight is transposed into the workspace
-    return ldb_n == 1 && K > 1 ? (size_t)N * (size_t)K : 0;
+    using namespace mi355;
+    if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff) return 0;
+    const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n);
+    return pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes;
 }
 
 extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale,
@@ -468,14 +550,18 @@ extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float 
     const int8_t *bt = b;
     int64_t ldbt = ldb_n;
     bool tiled = K >= BK && K % BK == 0 && (lda & 15) == 0 && aligned(a, 16);
+    const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n);
+    char *ws = static_cast<char *>(workspace);
+    if (tiled && pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes > 0) {
+        if (!ws || workspace_bytes < pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes) return MI355_ERR_WORKSPACE;
+        if (!aligned(ws, 16)) return MI355_ERR_ALIGNMENT;
+    }
     if (tiled && ldb_k != 1) {
         // contiguous [K,N]: transpose once into the workspace
-        const size_t need = (size_t)N * (size_t)K;
-        if (!workspace || workspace_bytes < need) return MI355_ERR_WORKSPACE;
-        if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+        int8_t *dst = reinterpret_cast<int8_t *>(ws + pl.counter_bytes + pl.partial_bytes);
         hipLaunchKernelGGL(transpose_i8_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64)), dim3(256), 0,
-                           s, b, static_cast<int8_t *>(workspace), (int)K, (int)N, ldb_k);
-        bt = static_cast<const int8_t *>(workspace);
+                           s, b, dst, (int)K, (int)N, ldb_k);
+        bt = dst;
         ldbt = K;
     }
     tiled = tiled && (ldbt & 15) == 0 && aligned(bt, 16);
@@ -501,7 +587,10 @@ extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float 
     p.K = (int)K;
     p.scale_len = (int)scale_len;
     p.out_i32 = out_i32;
-    const TileChoice c = choose_tile(p.M, p.N);
+    const TileChoice c = pl.tile;
+    p.S = pl.S;
+    p.counter = pl.S > 1 ? reinterpret_cast<uint32_t *>(ws) : nullptr;
+    p.partial = pl.S > 1 ? reinterpret_cast<int32_t *>(ws + pl.counter_bytes) : nullptr;
 #define MI355_QMM_CASE(bm_, bn_, wgm_, wgn_)  \
     if (c.bm == bm_ && c.bn == bn_) return launch_qmm<wgm_, wgn_, bm_ / (16 * wgm_), bn_ / (16 * wgn_)>(p, s);
     MI355_QMM_CASE(256, 256, 2, 4)

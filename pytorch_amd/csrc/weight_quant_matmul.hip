@@ -531,7 +531,11 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
         if (!(w_bits == 4 && pl.mt == 2 && pl.accum)) break;
     }
     pl.partial_bytes = pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0;
-    pl.counter_bytes = pl.S > 1 ? (((size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t)) + 255) / 256 * 256 : 0;
+    if (pl.S > 1 && (size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) {
+        pl.fast = false;                              // more tiles than arrival counters
+        return pl;
+    }
+    pl.counter_bytes = pl.S > 1 ? kWorkspaceCounterBytes : 0;
     return pl;
 }
 

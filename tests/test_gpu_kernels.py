@@ -144,6 +144,22 @@ def test_quant_matmul_extreme_accumulators(capi, golden):
     assert np.array_equal(_bits(half), want)
 
 
+def test_quant_matmul_split_k_repeated_launches(capi, golden):
+    """A narrow output with a long K is split over K (workgroups meet at counters in the shared workspace): the
+    down-projection shape of the MLP configuration, launched repeatedly on the same zero-initialised workspace."""
+    M, K, N = 64, 14336, 4096
+    assert capi.lib().mi355_quant_matmul_workspace(M, N, K, 1, K) > 0        # this shape does split
+    for seed in (1, 2, 3):
+        d = workloads.quant_matmul_inputs(seed=seed, M=M, K=K, N=N, weight_nk=True, bias=True)
+        x1, x2 = d["x1"].cuda(), d["x2"].cuda()
+        acc = capi.quant_matmul(x1, x2, None, out_dtype=torch.int32)
+        assert np.array_equal(acc.cpu().numpy(), golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy()))
+        out = capi.quant_matmul(x1, x2, d["scale"].cuda(), d["pertoken_scale"].cuda(), d["bias"].cuda())
+        want, _ = golden.quant_matmul(d["x1"].numpy(), d["x2"].numpy(), d["scale"].numpy(), d["pertoken_scale"].numpy(),
+                                      _bits(d["bias"]))
+        assert np.array_equal(_bits(out), want)
+
+
 # ------------------------------------------------------------------ weight-quant matmul
 
 def _wq_golden(golden, d, group):
