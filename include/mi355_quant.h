@@ -125,6 +125,21 @@ int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int w_bits,
  */
 int mi355_swiglu(const void *x_bf16, void *out_bf16, int64_t rows, int64_t half, int64_t ldx, void *stream);
 
+/*
+ * Fused SwiGLU + per-token dynamic quantisation: y, scale = dynamic_quant(swiglu(x)) without the bf16
+ * intermediate in memory; bit-identical to mi355_swiglu followed by mi355_dynamic_quant.
+ * Stands for the aclnn SwiGluQuant call behind torch_npu.npu_swiglu_quant in its dynamic mode (the operator is
+ * only named in the reference tree, docs/zh/release_notes.md:303; its fused relative
+ * npu_grouped_matmul_swiglu_quant_v2 appears in torch_npu/profiler/_flops_formulas.py:161-183).
+ *
+ *   x  bf16 [rows, 2*half], row pitch x_row_stride elements
+ *   activate_left != 0: silu(x[:, :half]) * x[:, half:]  (the orientation of npu_swiglu,
+ *                       torch_npu/_inductor/decomposition.py:186-188);  0: silu(x[:, half:]) * x[:, :half]
+ *   y  int8 [rows, half] contiguous;  scale float32 [rows]
+ */
+int mi355_swiglu_quant(const void *x_bf16, int activate_left, int8_t *y, float *scale,
+                       int64_t rows, int64_t half, int64_t x_row_stride, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

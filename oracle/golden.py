@@ -182,6 +182,16 @@ def swiglu(x_u16: np.ndarray) -> np.ndarray:
     return out
 
 
+def swiglu_quant(x_u16: np.ndarray, activate_left: bool = True):
+    """dynamic_quant(swiglu(x)): the composition of the two restatements above (no arithmetic of its own).
+    activate_left=False activates the right half: silu(x[:, half:]) * x[:, :half]."""
+    x = _c(x_u16, np.uint16)
+    half = x.shape[1] // 2
+    if not activate_left:
+        x = np.concatenate([x[:, half:], x[:, :half]], axis=1)
+    return dynamic_quant(swiglu(x))
+
+
 # ------------------------------------------------------ bit-pattern helpers
 
 def bf16_bits_to_f32(u16: np.ndarray) -> np.ndarray:

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
 
 EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant",
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
-           "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu")
+           "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant")
 
 _lib = None
 
@@ -44,6 +44,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_weight_quant_matmul.argtypes = [vp, vp, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
                                                 vp, sz, vp]
         L.mi355_swiglu.argtypes = [vp, vp, i64, i64, i64, vp]
+        L.mi355_swiglu_quant.argtypes = [vp, i32, vp, vp, i64, i64, i64, vp]
         _lib = L
     return _lib
 
@@ -143,3 +144,14 @@ def swiglu(x):
     out = torch.empty((rows, two // 2), dtype=torch.bfloat16, device=x.device)
     _check(lib().mi355_swiglu(_ptr(x), _ptr(out), rows, two // 2, x.stride(0), _stream()), "mi355_swiglu")
     return out
+
+
+def swiglu_quant(x, activate_left: bool = True):
+    """x bf16 [rows, 2*half] -> (int8 [rows, half], float32 [rows]) = dynamic_quant(swiglu(x))."""
+    _need_gpu(x)
+    rows, two = x.shape
+    y = torch.empty((rows, two // 2), dtype=torch.int8, device=x.device)
+    scale = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    _check(lib().mi355_swiglu_quant(_ptr(x), 1 if activate_left else 0, _ptr(y), _ptr(scale), rows, two // 2, x.stride(0),
+                                    _stream()), "mi355_swiglu_quant")
+    return y, scale

@@ -31,6 +31,17 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
     return __builtin_bit_cast(uint32_t, v);
 }
 
+// SwiGLU on two packed bf16 pairs the way eager bf16 tensor ops evaluate it: s = bf16(a / (1 + exp(-a))) in
+// float32, result = bf16(float(s) * float(b)).
+__device__ __forceinline__ float silu_f32(float a) { return a / (1.0f + expf(-a)); }
+
+__device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2)
+{
+    const float s0 = bf16_1(f32_to_bf16(silu_f32(bf16_lo(a2))));
+    const float s1 = bf16_1(f32_to_bf16(silu_f32(bf16_hi(a2))));
+    return pack_bf16x2(s0 * bf16_lo(b2), s1 * bf16_hi(b2));
+}
+
 // Every workspace of this library starts with this many bytes of arrival counters (zero before the first launch,
 // left zero by every launch); whatever else a launch keeps in the workspace lies behind them, so one
 // zero-initialised buffer can be shared by all launches of a stream.

@@ -87,10 +87,13 @@ __device__ __forceinline__ uint32_t pack4(uint32_t a, uint32_t b, uint32_t c, ui
 
 // TPR threads cooperate on one row (64 = one wavefront, no barrier; 256 = whole block);
 // each thread holds ITERS vectors of 8 elements.
-template <int TPR, int ITERS, bool FP16>
+// SWIGLU: the input row holds two halves of `cols` elements each and the quantised row is
+// bf16(silu(act half)) * other half (rounded to bf16 like the stand-alone SwiGLU kernel): the fused
+// SwiGLU + dynamic_quant of an MLP, which saves writing and re-reading the bf16 activation.
+template <int TPR, int ITERS, bool FP16, bool SWIGLU = false>
 __global__ __launch_bounds__(kBlock) void dq_rows_kernel(const uint16_t *__restrict__ x, int8_t *__restrict__ y,
                                                          float *__restrict__ scale_out, int64_t rows, int cols,
-                                                         int64_t row_stride)
+                                                         int64_t row_stride, int act_offset = 0, int mul_offset = 0)
 {
     constexpr int RPB = kBlock / TPR;
     const int t = threadIdx.x % TPR;
@@ -105,7 +108,14 @@ __global__ __launch_bounds__(kBlock) void dq_rows_kernel(const uint16_t *__restr
     for (int i = 0; i < ITERS; i++) {
         const int idx = t + i * TPR;
         if (live && idx < nvec) {
-            v[i] = __builtin_nontemporal_load(xr + idx);
+            if constexpr (SWIGLU) {
+                // act_offset / mul_offset: position (in 16-byte vectors) of the activated and of the other half
+                const u32x4 a = __builtin_nontemporal_load(xr + act_offset + idx);
+                const u32x4 b = __builtin_nontemporal_load(xr + mul_offset + idx);
+                v[i] = u32x4{swiglu2(a.x, b.x), swiglu2(a.y, b.y), swiglu2(a.z, b.z), swiglu2(a.w, b.w)};
+            } else {
+                v[i] = __builtin_nontemporal_load(xr + idx);
+            }
         } else {
             v[i] = u32x4{0, 0, 0, 0};
         }
@@ -227,8 +237,74 @@ void launch_rows(bool fp16, const uint16_t *x, int8_t *y, float *scale, int64_t 
                            cols, stride);
 }
 
+template <int TPR, int ITERS>
+void launch_swiglu_rows(const uint16_t *x, int8_t *y, float *scale, int64_t rows, int cols, int64_t stride, int act_off,
+                        int mul_off, hipStream_t s)
+{
+    constexpr int RPB = kBlock / TPR;
+    const unsigned grid = (unsigned)((rows + RPB - 1) / RPB);
+    hipLaunchKernelGGL((dq_rows_kernel<TPR, ITERS, false, true>), dim3(grid), dim3(kBlock), 0, s, x, y, scale, rows, cols,
+                       stride, act_off, mul_off);
+}
+
+// Any shape and alignment: one block per row, SwiGLU recomputed in the second pass.
+__global__ __launch_bounds__(kBlock) void swiglu_dq_generic_kernel(const uint16_t *__restrict__ x, int8_t *__restrict__ y,
+                                                                  float *__restrict__ scale_out, int64_t half,
+                                                                  int64_t row_stride, int64_t act_off, int64_t mul_off)
+{
+    const int64_t row = blockIdx.x;
+    const uint16_t *xr = x + row * row_stride;
+    auto value = [&](int64_t j) {
+        const float sl = bf16_1(f32_to_bf16(silu_f32(bf16_1(xr[act_off + j]))));
+        return bf16_1(f32_to_bf16(sl * bf16_1(xr[mul_off + j])));
+    };
+    float amax = 0.0f;
+    for (int64_t j = threadIdx.x; j < half; j += kBlock) amax = fmaxf(amax, fabsf(value(j)));
+    uint32_t mb = wave_max_u32(__float_as_uint(amax));
+    __shared__ uint32_t part[kBlock / 64];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = mb;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; w++) mb = part[w] > mb ? part[w] : mb;
+    amax = __uint_as_float(mb);
+    const float scale = amax / 127.0f;
+    if (threadIdx.x == 0) scale_out[row] = scale;
+    const bool zero = !(amax > 0.0f);
+    for (int64_t j = threadIdx.x; j < half; j += kBlock) y[row * half + j] = zero ? (int8_t)0 : (int8_t)quant_exact(value(j), scale);
+}
+
 } // namespace
 } // namespace mi355
+
+extern "C" int mi355_swiglu_quant(const void *x_bf16, int activate_left, int8_t *y, float *scale, int64_t rows, int64_t half,
+                                  int64_t x_row_stride, void *stream)
+{
+    using namespace mi355;
+    if (rows < 0 || half < 0) return MI355_ERR_BAD_ARGUMENT;
+    if (rows == 0) return MI355_OK;
+    if (!scale) return MI355_ERR_BAD_ARGUMENT;
+    if (half > 0 && (!x_bf16 || !y || x_row_stride < 2 * half)) return MI355_ERR_BAD_ARGUMENT;
+    if (rows > 0x7fffffff) return MI355_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint16_t *xp = static_cast<const uint16_t *>(x_bf16);
+    const int64_t act = activate_left ? 0 : half, mul = activate_left ? half : 0;
+    const int64_t nvec = half >> 3;
+    const bool vec_ok = half > 0 && (half & 7) == 0 && (x_row_stride & 7) == 0 && aligned(xp, 16) && aligned(y, 8) &&
+                        nvec <= kBlock * 8;
+    if (vec_ok) {
+        const int c = (int)half, ao = (int)(act >> 3), mo = (int)(mul >> 3);
+        if (nvec <= 64 * 1) launch_swiglu_rows<64, 1>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
+        else if (nvec <= 64 * 2) launch_swiglu_rows<64, 2>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
+        else if (nvec <= 64 * 4) launch_swiglu_rows<64, 4>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
+        else if (nvec <= 256 * 2) launch_swiglu_rows<256, 2>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
+        else if (nvec <= 256 * 4) launch_swiglu_rows<256, 4>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
+        else launch_swiglu_rows<256, 8>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
+    } else {
+        hipLaunchKernelGGL(swiglu_dq_generic_kernel, dim3((unsigned)rows), dim3(kBlock), 0, s, xp, y, scale, half, x_row_stride,
+                           act, mul);
+    }
+    return check_launch();
+}
 
 extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth, int8_t *y, float *scale,
                                    int64_t rows, int64_t cols, int64_t x_row_stride, void *stream)

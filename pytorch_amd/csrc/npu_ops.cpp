@@ -382,6 +382,72 @@ Tensor swiglu_hip(const Tensor &input, int64_t dim)
     return out;
 }
 
+// ---------------------------------------------------------------- npu_swiglu_quant
+
+// The operator is only named in the reference tree (docs/zh/release_notes.md:303); the argument list follows the
+// vendor's published Python signature.  Implemented: dynamic per-token quantisation (quant_mode = 1) of the SwiGLU
+// of the last dimension, without smooth scales, offsets or expert groups.
+void swiglu_quant_check(const Tensor &x, const optional<Tensor> &smooth_scales, const optional<Tensor> &offsets,
+                        const optional<Tensor> &group_index, int64_t quant_mode, int64_t group_list_type,
+                        optional<at::ScalarType> dst_type)
+{
+    TORCH_CHECK(x.scalar_type() == at::kBFloat16, "npu_swiglu_quant: only bfloat16 input is supported, got ", x.scalar_type());
+    TORCH_CHECK(x.dim() >= 1 && x.size(-1) % 2 == 0, "npu_swiglu_quant: the last dimension must be even");
+    TORCH_CHECK(!opt(smooth_scales), "npu_swiglu_quant: smooth_scales is not supported");
+    TORCH_CHECK(!opt(offsets), "npu_swiglu_quant: offsets (static quantisation) is not supported");
+    TORCH_CHECK(!opt(group_index), "npu_swiglu_quant: group_index is not supported");
+    TORCH_CHECK(quant_mode == 1, "npu_swiglu_quant: only quant_mode=1 (dynamic per-token quantisation) is supported, got ",
+                quant_mode);
+    TORCH_CHECK(group_list_type == 0, "npu_swiglu_quant: group_list_type is not supported");
+    TORCH_CHECK(!dst_type.has_value() || *dst_type == at::kChar, "npu_swiglu_quant: only dst_type=torch.int8 is supported");
+}
+
+std::tuple<Tensor, Tensor> swiglu_quant_alloc(const Tensor &x)
+{
+    auto shape = x.sizes().vec();
+    shape.back() /= 2;
+    auto scale_shape = shape;
+    scale_shape.pop_back();
+    return {at::empty(shape, x.options().dtype(at::kChar)), at::empty(scale_shape, x.options().dtype(at::kFloat))};
+}
+
+std::tuple<Tensor, Tensor> swiglu_quant_meta(const Tensor &x, const optional<Tensor> &smooth_scales,
+                                             const optional<Tensor> &offsets, const optional<Tensor> &group_index,
+                                             bool activate_left, int64_t quant_mode, int64_t group_list_type,
+                                             optional<at::ScalarType> dst_type)
+{
+    (void)activate_left;
+    swiglu_quant_check(x, smooth_scales, offsets, group_index, quant_mode, group_list_type, dst_type);
+    return swiglu_quant_alloc(x);
+}
+
+std::tuple<Tensor, Tensor> swiglu_quant_hip(const Tensor &x, const optional<Tensor> &smooth_scales,
+                                            const optional<Tensor> &offsets, const optional<Tensor> &group_index,
+                                            bool activate_left, int64_t quant_mode, int64_t group_list_type,
+                                            optional<at::ScalarType> dst_type)
+{
+    swiglu_quant_check(x, smooth_scales, offsets, group_index, quant_mode, group_list_type, dst_type);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+    auto [y, scale] = swiglu_quant_alloc(x);
+    const int64_t half = x.size(-1) / 2;
+    const int64_t rows = half ? y.numel() / half : 0;
+    if (rows == 0 || half == 0) {
+        scale.zero_();
+        return {y, scale};
+    }
+    Tensor xin = x;
+    int64_t row_stride = 2 * half;
+    if (xin.dim() == 2 && xin.stride(1) == 1 && xin.stride(0) >= 2 * half) {
+        row_stride = xin.stride(0);
+    } else if (!xin.is_contiguous()) {
+        xin = xin.contiguous();
+    }
+    check_status(mi355_swiglu_quant(xin.data_ptr(), activate_left ? 1 : 0, y.data_ptr<int8_t>(), scale.data_ptr<float>(), rows,
+                                    half, row_stride, stream_of(x)),
+                 "npu_swiglu_quant");
+    return {y, scale};
+}
+
 } // namespace
 
 TORCH_LIBRARY_FRAGMENT(npu, m)
@@ -394,6 +460,8 @@ TORCH_LIBRARY_FRAGMENT(npu, m)
           "Tensor? quant_scale=None, Tensor? quant_offset=None, Tensor? bias=None, int antiquant_group_size=0, "
           "int inner_precise=0, *, ScalarType? weight_dtype=None) -> Tensor");
     m.def("npu_swiglu(Tensor input, int dim=-1) -> Tensor");
+    m.def("npu_swiglu_quant(Tensor x, *, Tensor? smooth_scales=None, Tensor? offsets=None, Tensor? group_index=None, "
+          "bool activate_left=False, int quant_mode=0, int group_list_type=0, ScalarType? dst_type=None) -> (Tensor, Tensor)");
 }
 
 TORCH_LIBRARY_IMPL(npu, CUDA, m)
@@ -402,6 +470,7 @@ TORCH_LIBRARY_IMPL(npu, CUDA, m)
     m.impl("npu_quant_matmul", TORCH_FN(quant_matmul_hip));
     m.impl("npu_weight_quant_batchmatmul", TORCH_FN(weight_quant_hip));
     m.impl("npu_swiglu", TORCH_FN(swiglu_hip));
+    m.impl("npu_swiglu_quant", TORCH_FN(swiglu_quant_hip));
 }
 
 TORCH_LIBRARY_IMPL(npu, Meta, m)
@@ -410,4 +479,5 @@ TORCH_LIBRARY_IMPL(npu, Meta, m)
     m.impl("npu_quant_matmul", TORCH_FN(quant_matmul_meta));
     m.impl("npu_weight_quant_batchmatmul", TORCH_FN(weight_quant_meta));
     m.impl("npu_swiglu", TORCH_FN(swiglu_meta));
+    m.impl("npu_swiglu_quant", TORCH_FN(swiglu_quant_meta));
 }

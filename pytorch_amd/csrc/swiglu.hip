@@ -6,15 +6,6 @@
 namespace mi355 {
 namespace {
 
-__device__ __forceinline__ float silu_f32(float a) { return a / (1.0f + expf(-a)); }
-
-__device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2)
-{
-    const float s0 = bf16_1(f32_to_bf16(silu_f32(bf16_lo(a2))));
-    const float s1 = bf16_1(f32_to_bf16(silu_f32(bf16_hi(a2))));
-    return pack_bf16x2(s0 * bf16_lo(b2), s1 * bf16_hi(b2));
-}
-
 // vectorised: half % 8 == 0, 16-byte aligned rows
 __global__ __launch_bounds__(256) void swiglu_vec_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ out,
                                                          int64_t rows, int half_vec, int64_t ldx)

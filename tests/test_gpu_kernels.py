@@ -235,6 +235,21 @@ def test_swiglu(capi, golden):
 
 # ------------------------------------------------------------------ error paths (host side, no kernel runs)
 
+@pytest.mark.parametrize("rows,half", [(64, 14336), (2048, 14336), (33, 512), (5, 100), (3, 16384 + 8), (7, 24)])
+@pytest.mark.parametrize("left", [True, False])
+def test_swiglu_quant_equals_composition(capi, golden, rows, half, left):
+    g = torch.Generator().manual_seed(rows + half)
+    x = (torch.randn(rows, 2 * half, generator=g) * 2).to(torch.bfloat16)
+    x[0, :] = 0                                                     # a zero row: scale 0, codes 0
+    y, s = capi.swiglu_quant(x.cuda(), activate_left=left)
+    want_y, want_s = golden.swiglu_quant(_bits(x), activate_left=left)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+    assert np.array_equal(y.cpu().numpy(), want_y)
+    if left:                                                        # and the two separate kernels give the same bits
+        y2, s2 = capi.dynamic_quant(capi.swiglu(x.cuda()))
+        assert torch.equal(y, y2) and torch.equal(s, s2)
+
+
 def test_c_abi_rejects_bad_arguments(capi):
     L = capi.lib()
     assert L.mi355_dynamic_quant(None, 0, None, None, None, -1, 8, 8, None) == -1

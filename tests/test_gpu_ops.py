@@ -173,6 +173,28 @@ def test_c5_mlp_chain_stagewise(pa, golden):
     assert torch.isfinite(out.float()).all()
 
 
+def test_swiglu_quant_operator(pa, golden):
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 40, 1024, generator=g).to(torch.bfloat16)
+    for left in (True, False):
+        y, s = pa.npu_swiglu_quant(x.cuda(), activate_left=left, quant_mode=1)
+        wy, ws = golden.swiglu_quant(_bits(x).reshape(120, 1024), activate_left=left)
+        assert y.shape == (3, 40, 512) and s.shape == (3, 40)
+        assert np.array_equal(y.cpu().numpy().reshape(120, 512), wy)
+        assert np.array_equal(s.cpu().numpy().reshape(120).view(np.uint32), ws.view(np.uint32))
+    # the default orientation of the vendor signature activates the right half
+    y0, _ = pa.npu_swiglu_quant(x.cuda(), quant_mode=1)
+    assert torch.equal(y0, pa.npu_swiglu_quant(x.cuda(), activate_left=False, quant_mode=1)[0])
+    with pytest.raises(RuntimeError, match="quant_mode"):
+        pa.npu_swiglu_quant(x.cuda())
+    # a strided 2-D view (the columns of a wider buffer) is read in place
+    wide = torch.randn(16, 3000, generator=g).to(torch.bfloat16).cuda()
+    view = wide[:, :2048]
+    y1, s1 = pa.npu_swiglu_quant(view, activate_left=True, quant_mode=1)
+    y2, s2 = pa.npu_dynamic_quant(pa.npu_swiglu(view.contiguous()))
+    assert torch.equal(y1, y2) and torch.equal(s1, s2)
+
+
 def test_c5_mlp_prefill_properties(pa, golden):
     """M = 2048: rows are independent, so any subset of rows run alone must reproduce the same bits."""
     d = workloads.mlp_inputs(seed=1, M=2048)

@@ -16,7 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def test_c_abi_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "mi355_quant.h")).read()
     declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", header))
-    assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu"} <= declared
+    assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant"} <= declared
     lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_amd", "csrc", "libmi355_quant.so"))
     for name in declared:
         assert hasattr(lib, name), name
@@ -34,7 +34,8 @@ def pa():
 
 
 def test_operator_names_and_schemas(pa):
-    assert set(pa.__all__) >= {"npu_dynamic_quant", "npu_quant_matmul", "npu_weight_quant_batchmatmul", "npu_swiglu"}
+    assert set(pa.__all__) >= {"npu_dynamic_quant", "npu_quant_matmul", "npu_weight_quant_batchmatmul", "npu_swiglu",
+                                "npu_swiglu_quant"}
     assert pa.npu_quant_matmul is torch.ops.npu.npu_quant_matmul
     s = str(torch.ops.npu.npu_dynamic_quant.default._schema)
     assert s.startswith("npu::npu_dynamic_quant(Tensor input, *, Tensor? smooth_scales=None, Tensor? group_index=None")
@@ -135,6 +136,17 @@ def test_meta_weight_quant_batchmatmul(pa):
         pa.npu_weight_quant_batchmatmul(xs, w4, sg, og, antiquant_group_size=100)
     with pytest.raises(RuntimeError, match="x must be bfloat16"):
         pa.npu_weight_quant_batchmatmul(_m(1, 4096, dtype=torch.float16), w4, sg, og, antiquant_group_size=128)
+
+
+def test_meta_swiglu_quant(pa):
+    y, s = pa.npu_swiglu_quant(_m(64, 28672, dtype=torch.bfloat16), quant_mode=1)
+    assert y.shape == (64, 14336) and y.dtype == torch.int8 and s.shape == (64,) and s.dtype == torch.float32
+    y, s = pa.npu_swiglu_quant(_m(2, 3, 8, dtype=torch.bfloat16), activate_left=True, quant_mode=1)
+    assert y.shape == (2, 3, 4) and s.shape == (2, 3)
+    with pytest.raises(RuntimeError, match="quant_mode"):
+        pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16))                      # static quantisation is not built
+    with pytest.raises(RuntimeError, match="smooth_scales"):
+        pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(4, dtype=torch.bfloat16), quant_mode=1)
 
 
 def test_meta_swiglu(pa):
