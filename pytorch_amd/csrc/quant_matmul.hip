@@ -78,8 +78,10 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
     constexpr int UNITS_A = BM / 8, UNITS_B = BN / 8;        // unit = 8 rows x 128 B = one wavefront-wide load
     constexpr int UNITS_BP = (UNITS_B + NW - 1) / NW * NW;
-    constexpr int LOADS_PER_STAGE = (UNITS_A + UNITS_BP) / NW;
-    constexpr int STAGE_BYTES = (UNITS_A + UNITS_BP) * 1024;
+    constexpr int LA = UNITS_A / NW, LB = UNITS_BP / NW;     // loads of a wavefront per activation / weight stage
+    constexpr int A_BYTES = UNITS_A * 1024, B_BYTES = UNITS_BP * 1024;
+    constexpr int NSA = 2;                                   // activation slots; NS weight slots follow them in LDS
+    constexpr uint32_t kOutOfRange = 0x80000000u;            // lane offset beyond every buffer: the load writes zeros
     static_assert(UNITS_A % NW == 0, "A units must divide evenly over the wavefronts");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -97,6 +99,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
+    const int kt0 = (int)((int64_t)(p.K / BK) * chunk / p.S);            // first K step of this workgroup
+    const int KT = (int)((int64_t)(p.K / BK) * (chunk + 1) / p.S) - kt0;  // its number of K steps
 
     // Global -> LDS addressing.  Lane l of a unit fills LDS slot l (16 B): row l/8, chunk slot l%8,
     // which must hold global chunk (l%8) ^ (l/8) of that row (XOR swizzle).
@@ -112,20 +116,28 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     const uint32_t voff_b = (uint32_t)(rr * (int)p.ldbt + gchunk);
     const uint32_t unit_stride_a = 8u * (uint32_t)p.lda, unit_stride_b = 8u * (uint32_t)p.ldbt;
 
-    auto issue_stage = [&](int k0, char *stage) {
+    // Loads are never skipped, so that the number of outstanding loads at every point of the loop is a
+    // compile-time constant; a K step past the end gets an out-of-range lane offset instead (no memory traffic).
+    auto issue_a = [&](int kt, int KT) {
+        char *slot = lds + (kt % NSA) * A_BYTES;
+        const uint32_t vo = kt < KT ? voff_a : kOutOfRange;
 #pragma unroll
-        for (int i = 0; i < UNITS_A / NW; i++) {
+        for (int i = 0; i < LA; i++) {
             const int u = i * NW + wave;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void *)(stage + u * 1024), 16, voff_a,
-                                                     (uint32_t)u * unit_stride_a + k0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void *)(slot + u * 1024), 16, vo,
+                                                     (uint32_t)u * unit_stride_a + (uint32_t)(kt0 + kt) * BK, 0, 0);
         }
-        // B units are padded to a multiple of the wavefront count (rows past the tile read as zero), so every
-        // wavefront issues the same number of loads per stage
+    };
+    // B units are padded to a multiple of the wavefront count (rows past the tile read as zero), so every
+    // wavefront issues the same number of loads per stage
+    auto issue_b = [&](int kt, int KT) {
+        char *slot = lds + NSA * A_BYTES + (kt % NS) * B_BYTES;
+        const uint32_t vo = kt < KT ? voff_b : kOutOfRange;
 #pragma unroll
-        for (int i = 0; i < UNITS_BP / NW; i++) {
+        for (int i = 0; i < LB; i++) {
             const int u = i * NW + wave;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void *)(stage + (UNITS_A + u) * 1024), 16, voff_b,
-                                                     (uint32_t)u * unit_stride_b + k0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void *)(slot + u * 1024), 16, vo,
+                                                     (uint32_t)u * unit_stride_b + (uint32_t)(kt0 + kt) * BK, 0, 0);
         }
     };
 
@@ -140,19 +152,19 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     const int frow = lane & 15;
     const int sw0 = ((lane >> 4) ^ ((frow >> 1) & 7)) * 16;
     const int a_off = (wm * WTM * 16 + frow) * BK;
-    const int b_off = (BM + wn * WTN * 16 + frow) * BK;
+    const int b_off = NSA * A_BYTES + (wn * WTN * 16 + frow) * BK;
 
     // Fragments are double buffered in registers: the LDS reads of the next 64-wide K step are issued before
     // the MFMAs of the current one, so LDS latency hides behind the matrix pipe instead of in front of it.
     i32x4v af0[WTM], bf0[WTN], af1[WTM], bf1[WTN];
-#define MI355_READ_FRAGS(AF, BF, STAGE, KS)                                                                      \
+#define MI355_READ_FRAGS(AF, BF, KT_, KS)                                                                        \
     {                                                                                                            \
-        const char *st_ = (STAGE);                                                                               \
+        const char *sa_ = lds + ((KT_) % NSA) * A_BYTES + a_off, *sb_ = lds + ((KT_) % NS) * B_BYTES + b_off;    \
         const int sw_ = sw0 ^ ((KS) * 64);                                                                       \
         _Pragma("unroll") for (int i = 0; i < WTM; i++)                                                          \
-            AF[i] = *reinterpret_cast<const i32x4v *>(st_ + a_off + i * 16 * BK + sw_);                          \
+            AF[i] = *reinterpret_cast<const i32x4v *>(sa_ + i * 16 * BK + sw_);                                  \
         _Pragma("unroll") for (int j = 0; j < WTN; j++)                                                          \
-            BF[j] = *reinterpret_cast<const i32x4v *>(st_ + b_off + j * 16 * BK + sw_);                          \
+            BF[j] = *reinterpret_cast<const i32x4v *>(sb_ + j * 16 * BK + sw_);                                  \
     }
 #define MI355_MFMA_BLOCK(AF, BF)                                                                                 \
     {                                                                                                            \
@@ -161,43 +173,39 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(BF[j], AF[i], acc[i][j], 0, 0, 0);             \
     }
 
-    // NS LDS stages: while stage kt is consumed, stages kt+1 .. kt+NS-1 are landing or in flight, which hides
-    // HBM latency when the operands are not cache resident.  Every wavefront issues L loads per stage, so
-    // "at most c*L loads outstanding" means "everything but the newest c stages has landed".
-    constexpr int L = LOADS_PER_STAGE;
-    static_assert(NS >= 2 && NS <= 4, "stage count");
-    const int kt0 = (int)((int64_t)(p.K / BK) * chunk / p.S);
-    const int KT = (int)((int64_t)(p.K / BK) * (chunk + 1) / p.S) - kt0;
-    {
-        const int pro = KT < NS ? KT : NS;
-        for (int s = 0; s < pro; s++) issue_stage((kt0 + s) * BK, lds + s * STAGE_BYTES);
-        if (pro >= 4) wait_vmcnt<3 * L>();
-        else if (pro == 3) wait_vmcnt<2 * L>();
-        else if (pro == 2) wait_vmcnt<1 * L>();
-        else wait_vmcnt<0>();                                          // stage 0 has landed
-    }
+    // Two activation slots and NS weight slots (NS = 3 described).  In the middle of K step kt, once every wavefront is done
+    // with stage kt, its slots are refilled with the activations of step kt+2 and the weights of step kt+3:
+    // activations come from cache and get one step to land, weights come from HBM and get two.  Loads retire in
+    // order and every refill issues the activation loads first, so "at most LB outstanding" means that
+    // everything up to the activations of step kt+1 has landed and only the newest weight refill may be in flight.
+    // (With NS = 2 the weights of step kt+2 are requested instead and nothing may stay in flight; small tiles
+    // use that to keep two workgroups resident per CU.)
+    static_assert(NS == 2 || NS == 3, "weight slots");
+    issue_a(0, KT);
+    issue_b(0, KT);
+    issue_a(1, KT);
+    issue_b(1, KT);
+    if constexpr (NS == 3) issue_b(2, KT);
+    wait_vmcnt<LA + (NS - 1) * LB>();                                  // stage 0 has landed
     __syncthreads();
-    MI355_READ_FRAGS(af0, bf0, lds, 0)
+    MI355_READ_FRAGS(af0, bf0, 0, 0)
 
     for (int kt = 0; kt < KT; kt++) {
-        const char *cur = lds + (kt % NS) * STAGE_BYTES;
-        const char *nxt = lds + ((kt + 1) % NS) * STAGE_BYTES;
-        MI355_READ_FRAGS(af1, bf1, cur, 1)
+        MI355_READ_FRAGS(af1, bf1, kt, 1)
         __builtin_amdgcn_sched_barrier(0);
         MI355_MFMA_BLOCK(af0, bf0)
         __builtin_amdgcn_sched_barrier(0);
-        // stage kt+1 has landed (stages kt+2 .. may still be in flight) and this wavefront is done reading stage kt
-        const int newer = min(kt + NS - 1, KT - 1) - (kt + 1);
-        if (newer >= 2) wait_vmcnt_lgkm0<2 * L>();
-        else if (newer == 1) wait_vmcnt_lgkm0<1 * L>();
-        else wait_vmcnt_lgkm0<0>();
+        wait_vmcnt_lgkm0<(NS - 2) * LB>(); // stage kt+1 has landed and this wavefront is done reading stage kt
         __syncthreads();
-        if (kt + NS < KT) issue_stage((kt0 + kt + NS) * BK, lds + (kt % NS) * STAGE_BYTES);
-        if (kt + 1 < KT) MI355_READ_FRAGS(af0, bf0, nxt, 0)
+        issue_a(kt + 2, KT);
+        issue_b(kt + NS, KT);
+        MI355_READ_FRAGS(af0, bf0, kt + 1, 0)
         __builtin_amdgcn_sched_barrier(0);
         MI355_MFMA_BLOCK(af1, bf1)
         __builtin_amdgcn_sched_barrier(0);
     }
+    wait_vmcnt<0>();                       // the refills past the end (zeros) must not land in the epilogue's LDS
+    __syncthreads();
 #undef MI355_READ_FRAGS
 #undef MI355_MFMA_BLOCK
 
@@ -427,14 +435,13 @@ int launch_qmm(QmmArgs p, hipStream_t s)
 {
     constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
     constexpr int NWL = WGM * WGN;
-    constexpr size_t one_stage = (size_t)(BM / 8 + (BN / 8 + NWL - 1) / NWL * NWL) * 1024;
-    // Two stages.  Deeper prefetch (3-4 stages) measured slower on every tile shape: for tiles of <= 40 KiB per
-    // stage two stages let two workgroups share a CU (sixteen resident wavefronts hide barriers and epilogues),
-    // and for larger tiles the extra stages did not pay either.
-    constexpr int NS = 2;
-    static_assert(NS >= 2, "LDS budget");
-    constexpr size_t stage_bytes = (size_t)NS * one_stage;
+    // Two activation slots and three weight slots (weights come from HBM and need the longer lead), unless two
+    // weight slots let two workgroups share a CU (80 KiB each): sixteen resident wavefronts hide barriers and
+    // epilogues better than the deeper ring does.
+    constexpr size_t a_bytes = (size_t)(BM / 8) * 1024, b_bytes = (size_t)((BN / 8 + NWL - 1) / NWL * NWL) * 1024;
     constexpr size_t staging_bytes = (size_t)BM * WGN * ((BN / WGN) * 2 + 16);   // epilogue: padded bf16 tile rows
+    constexpr int NS = 2 * a_bytes + 2 * b_bytes <= 80 * 1024 && staging_bytes <= 80 * 1024 ? 2 : 3;
+    constexpr size_t stage_bytes = 2 * a_bytes + NS * b_bytes;
     constexpr size_t lds_bytes = stage_bytes > staging_bytes ? stage_bytes : staging_bytes;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -450,17 +457,18 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     return check_launch();
 }
 
-// Tile shapes (rows x columns of the workgroup tile) the library instantiates, with the measured cost of one
-// tile element per 4096 of K (ns, single resident tile per CU): larger tiles amortise LDS and L2 traffic better.
+// Tile shapes (rows x columns of the workgroup tile) the library instantiates, with measured times at K = 4096
+// on operands that are not cache resident: `slots` workgroups are resident at once (256 CUs x 1 or 2), a launch
+// that fits in one round of them takes `single_us` in all, longer launches take `round_us` per round.
 struct TileChoice {
-    int bm, bn;
-    double ns_per_elt;
+    int bm, bn, slots;
+    double single_us, round_us;
 };
-constexpr TileChoice kTiles[] = {{256, 256, 0.78}, {256, 224, 0.87}, {256, 192, 0.90}, {128, 352, 1.04},
-                                 {128, 320, 1.00}, {128, 256, 0.92}, {128, 192, 0.85}, {128, 128, 0.98},
-                                 {64, 256, 1.60},  {64, 128, 1.78}};
+constexpr TileChoice kTiles[] = {{256, 256, 256, 62.2, 70.7}, {256, 224, 256, 60.4, 67.5}, {256, 192, 256, 53.0, 58.0},
+                                 {128, 320, 256, 45.0, 50.0}, {128, 256, 256, 40.0, 45.6}, {128, 192, 512, 55.8, 58.8},
+                                 {128, 128, 512, 40.0, 43.3}, {64, 256, 512, 40.0, 52.6},  {64, 128, 512, 24.0, 30.0}};
 
-// Pick the tile shape that minimises (rounds of workgroups over the 256 CUs) x (time per tile).
+// Pick the tile shape that minimises (rounds of resident workgroups) x (time per round).
 TileChoice choose_tile(int M, int N)
 {
     if (const char *e = getenv("MI355_QMM_TILE")) { // debugging aid: "BMxBN"
@@ -473,8 +481,8 @@ TileChoice choose_tile(int M, int N)
     double best_cost = 1e300;
     for (const TileChoice &c : kTiles) {
         const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
-        const long rounds = (tiles + 255) / 256;
-        const double cost = (double)rounds * ((double)c.bm * c.bn * c.ns_per_elt + 2000.0);
+        const long rounds = (tiles + c.slots - 1) / c.slots;
+        const double cost = rounds == 1 ? c.single_us : (double)rounds * c.round_us;
         if (cost < best_cost) {
             best_cost = cost;
             best = c;
@@ -596,7 +604,6 @@ extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float 
     MI355_QMM_CASE(256, 256, 2, 4)
     MI355_QMM_CASE(256, 224, 4, 2)
     MI355_QMM_CASE(256, 192, 2, 4)
-    MI355_QMM_CASE(128, 352, 4, 2)
     MI355_QMM_CASE(128, 320, 2, 4)
     MI355_QMM_CASE(128, 256, 2, 4)
     MI355_QMM_CASE(128, 192, 2, 4)
