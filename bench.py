@@ -27,7 +27,7 @@ BF16_PEAK_TFLOPS = 2500.0    # dense bf16 MFMA
 CACHE_BYTES = 256 << 20      # Infinity Cache
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter
 # reads for a plain 256 MiB copy (factors 2.00 and 1.00); see profiles/hbm_traffic_pmc_all_kernels.txt
-TRAFFIC_BYTES = {"c1": 25305300, "c2": 106306300, "c3": 238189200, "c4_m8": 35842700}
+TRAFFIC_BYTES = {"c1": 25294848, "c2": 106311680, "c3": 245647360, "c4_m8": 35886080}
 
 
 def _parse():
