@@ -294,6 +294,14 @@ def main():
                                 TRAFFIC_BYTES["c3"],
                                 tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2)))
         del ws, keep
+        # the layout torch_npu's LinearWeightQuant passes: weight stored [N, K], given as its transposed view
+        ws = [torch.randint(-127, 128, (Nx, Kx), generator=gen, dtype=torch.int8, device=dev).t() for _ in range(2)]
+        keep = []
+        calls = [(lambda w=w: keep.append(pa.npu_weight_quant_batchmatmul(x, w, s3, o3))) for w in ws] * 4
+        us = _graph_time_us(torch, calls, reps=10)
+        others.append(hbm_entry("c3 W8A16 x bf16[16,8192] . int8[8192,28672] (weight stored [N,K], transposed view)", nb, us,
+                                None, tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2)))
+        del ws, keep
 
     if want("c4"):
         Kx, Nx = 4096, 14336

@@ -108,6 +108,98 @@ __device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint
     }
 }
 
+// Output side of a workgroup tile of NBW columns whose partial sums lie in LDS as red[slice][16 rows][NBW].
+// Every thread owns quads of 4 consecutive columns.  Without a split over K the sums go straight to the output.
+// With K split over S workgroups every workgroup publishes its partial and the last arrival adds them in chunk
+// order: the exchange uses agent-scope (sc1) write-through stores and cache-bypassing loads, ordered by the
+// wavefronts' own store counters, the workgroup barrier and a relaxed agent-scope counter; a full release/acquire
+// fence would write back and invalidate the whole L2 of the XCD, which costs far more than the kernel itself.
+template <int NBW, int KS, int THREADS>
+struct TileOut {
+    static constexpr int QPR = NBW / 4;
+    static constexpr int SC1 = 16;            // cache-policy bit: agent scope
+    const WqArgs &p;
+    char *lds;
+    const int m_base, n0, chunk;
+    const bool out_vec;
+    const uint32_t chunk_bytes;
+    const __amdgpu_buffer_rsrc_t rsrc_p;
+
+    __device__ TileOut(const WqArgs &p_, char *lds_, int m_base_, int n0_, int chunk_)
+        : p(p_), lds(lds_), m_base(m_base_), n0(n0_), chunk(chunk_), out_vec((p_.ldo & 3) == 0 && aligned_dev(p_.out, 8)),
+          chunk_bytes((uint32_t)p_.M * (uint32_t)p_.N * 4u),
+          rsrc_p(make_rsrc(p_.partial, p_.S > 1 ? (uint32_t)p_.M * (uint32_t)p_.N * 4u * (uint32_t)p_.S : 0u))
+    {
+    }
+
+    __device__ __forceinline__ void store_out(int row, int nl, f32x4 v) const
+    {
+        uint16_t *o = p.out + (int64_t)(m_base + row) * p.ldo + n0 + nl;
+        if (out_vec) {
+            u32x2 pk;
+            pk.x = pack_bf16x2(v[0], v[1]);
+            pk.y = pack_bf16x2(v[2], v[3]);
+            *reinterpret_cast<u32x2 *>(o) = pk;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] = f32_to_bf16(v[i]);
+        }
+    }
+
+    __device__ __forceinline__ uint32_t partial_off(int row, int nl) const { return (uint32_t)(((m_base + row) * p.N + n0 + nl) * 4); }
+
+    // rows row0 .. row0+rows_mt-1 of the tile: add the slices, then store or publish
+    __device__ __forceinline__ void emit_mtile(const float *red, int row0, int rows_mt) const
+    {
+        for (int qd = threadIdx.x; qd < rows_mt * QPR; qd += THREADS) {
+            const int row = qd / QPR, nl = (qd % QPR) * 4;
+            if (n0 + nl >= p.N) continue;
+            f32x4 acc = *reinterpret_cast<const f32x4 *>(red + (size_t)row * NBW + nl);
+#pragma unroll
+            for (int ks = 1; ks < KS; ks++) acc += *reinterpret_cast<const f32x4 *>(red + ((size_t)ks * 16 + row) * NBW + nl);
+            if (p.S == 1)
+                store_out(row0 + row, nl, acc);
+            else
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), rsrc_p, partial_off(row0 + row, nl),
+                                                       (uint32_t)chunk * chunk_bytes, SC1);
+        }
+    }
+
+    // after every m tile has been emitted: meet the other K chunks of the tile
+    __device__ __forceinline__ void finish(int rows_valid, int tile) const
+    {
+        if (p.S == 1) return;
+        int &is_last = *reinterpret_cast<int *>(lds);
+        wait_vmcnt<0>();                      // this wavefront's partial sums have reached the coherence point
+        __syncthreads();
+        uint32_t *cnt = p.counter + (size_t)blockIdx.y * p.sgroups + tile;
+        if (threadIdx.x == 0) {
+            const uint32_t old = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = old == (uint32_t)(p.S - 1);
+        }
+        __syncthreads();
+        if (!is_last) return;
+        for (int qd = threadIdx.x; qd < rows_valid * QPR; qd += THREADS) {
+            const int row = qd / QPR, nl = (qd % QPR) * 4;
+            if (n0 + nl >= p.N) continue;
+            const uint32_t off = partial_off(row, nl);
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int ch = 0; ch < p.S; ch += 8) {
+                f32x4 v[8];                   // eight loads in flight
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+                    v[i] = ch + i < p.S ? __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                              rsrc_p, off, (uint32_t)(ch + i) * chunk_bytes, SC1))
+                                        : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc += v[i];
+            }
+            store_out(row, nl, acc);
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
+    }
+};
+
 // One step of a wavefront: 32 weight rows of its strip (8 bytes per lane and row).
 // The loads are unconditional so that the main loop stays free of branches around memory instructions (the
 // compiler then tracks the outstanding loads exactly); a step past the end of the wavefront's range is given a
@@ -343,32 +435,8 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
     }
 
     // ---- reduce over the K slices, one m tile at a time: red[slice][row of the m tile][column of the tile]
-    int &is_last = *reinterpret_cast<int *>(lds);
     float *red = reinterpret_cast<float *>(lds + 16);
-    constexpr int QPR = NBW / 4;              // every thread owns quads of 4 consecutive columns
-    const int n0 = sgrp * NBW;
-    const bool out_vec = (p.ldo & 3) == 0 && aligned_dev(p.out, 8);
-    auto store_out = [&](int row, int nl, f32x4 v) {
-        uint16_t *o = p.out + (int64_t)(m_base + row) * p.ldo + n0 + nl;
-        if (out_vec) {
-            u32x2 pk;
-            pk.x = pack_bf16x2(v[0], v[1]);
-            pk.y = pack_bf16x2(v[2], v[3]);
-            *reinterpret_cast<u32x2 *>(o) = pk;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; i++) o[i] = f32_to_bf16(v[i]);
-        }
-    };
-    // K split over S workgroups: every workgroup publishes its partial, the last arrival adds them in chunk order.
-    // The exchange uses agent-scope (sc1) write-through stores and cache-bypassing loads, ordered by the
-    // wavefronts' own store counters, the workgroup barrier and a relaxed agent-scope counter; a full
-    // release/acquire fence would write back and invalidate the whole L2 of the XCD, which costs far
-    // more than the kernel itself.
-    constexpr int SC1 = 16;                   // cache-policy bit: agent scope
-    const uint32_t chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
-    const __amdgpu_buffer_rsrc_t rsrc_p = make_rsrc(p.partial, p.S > 1 ? chunk_bytes * (uint32_t)p.S : 0u);
-    auto partial_off = [&](int row, int nl) { return (uint32_t)(((m_base + row) * p.N + n0 + nl) * 4); };
+    TileOut<NBW, KS, THREADS> outp(p, lds, m_base, sgrp * NBW, chunk);
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
         const int rows_mt = min(16, rows_valid - mt * 16);
@@ -385,47 +453,215 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
             }
         }
         __syncthreads();
-        for (int qd = threadIdx.x; qd < rows_mt * QPR; qd += THREADS) {
-            const int row = qd / QPR, nl = (qd % QPR) * 4;
-            if (n0 + nl >= p.N) continue;
-            f32x4 acc = *reinterpret_cast<const f32x4 *>(red + (size_t)row * NBW + nl);
+        outp.emit_mtile(red, mt * 16, rows_mt);
+    }
+    outp.finish(rows_valid, sgrp);
+}
+
+// int8 weights stored K-major ([N, K] row-major: the transposed view that torch_npu's LinearWeightQuant passes,
+// torch_npu/contrib/module/linear_weight_quant.py:106).  Here a weight row already holds consecutive k of one output
+// column, which is what an MFMA operand lane wants, so a wavefront simply owns 16 columns (16 weight rows) for the whole
+// K range of its workgroup and keeps one accumulator tile per m tile; the eight wavefronts of a workgroup cover 128
+// columns, i.e. one contiguous block of 128 weight rows in memory.  Nothing is reduced across wavefronts.
+// K advances in steps of 128: lane (c, g) loads bytes [16g, 16g+16) and [64+16g, 64+16g+16) of the step from row c
+// (two 16-byte loads) and feeds four MFMAs with the 8-byte halves; the activation fragments are laid out to match.
+// Activations are staged through LDS in chunks of 8 steps, already in fragment order, double buffered: the loads of
+// the next chunk are issued at the top of a chunk, written to LDS at its end, one barrier per chunk.
+// Per group:  out = sum_g scale_g * (P'_g + (offset_g - 128) * X_g)  with the int8 image w + 128 (see the top of the file).
+template <int MT, bool GROUPED>
+__global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
+{
+    constexpr int NBW = 128, THREADS = 512;
+    constexpr int CH = 8 / MT;                          // steps per chunk of activations (32 KiB of LDS per buffer)
+    constexpr int BODY = CH / 2;                        // steps per batch of weight loads: two batches per chunk, so
+                                                        // that the register slot of a step is known at compile time
+    constexpr int POLICY = MT == 1 ? kNonTemporal : 0;
+    constexpr int XBUF = CH * MT * 4096;       // bytes of one activation chunk in LDS
+    constexpr int TBUF = 2048;                 // one step of one wavefront's weights (16 rows x 128 bytes)
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int xcd_slot = blockIdx.x >> 3;
+    const int tile = (blockIdx.x & 7) + 8 * (xcd_slot / p.S);
+    const int chunk = xcd_slot % p.S;
+    if (tile >= p.sgroups) return;
+    const int m_base = blockIdx.y * (MT * 16);
+    const int rows_valid = min(MT * 16, p.M - m_base);
+    const int n0 = tile * NBW;
+
+    // K range of this workgroup in steps of 128 (whole units: scale groups, or single steps per channel)
+    const int u0 = (int)((int64_t)p.n_units * chunk / p.S), u1 = (int)((int64_t)p.n_units * (chunk + 1) / p.S);
+    const int step0 = u0 * p.unit_steps, nsteps = (u1 - u0) * p.unit_steps;
+    const int nchunks = (nsteps + CH - 1) / CH;
+
+    // Weights: this wavefront's 16 rows (rows past N repeat the last valid row; their columns are never stored).
+    // A load instruction fetches whole cache lines - lane l takes 16 bytes of row l/8 (+8 for the second load) - which
+    // reads HBM a quarter faster than fetching the MFMA operand layout directly (16 rows x 64 bytes per
+    // instruction); the wavefront then turns the step around through a private 2 KiB LDS tile.  The 16-byte chunk a
+    // lane fetches is XOR-swizzled with the row pair so that the operand reads (16 rows x 16 bytes) are free of bank
+    // conflicts; LDS slot s of row r holds chunk s ^ ((r >> 1) & 7).
+    const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(p.w, (uint32_t)((uint64_t)(p.N - 1) * p.ldw_bytes + (uint32_t)p.K));
+    uint32_t voff_w[2];
 #pragma unroll
-            for (int ks = 1; ks < KS; ks++) acc += *reinterpret_cast<const f32x4 *>(red + ((size_t)ks * 16 + row) * NBW + nl);
-            if (p.S == 1)
-                store_out(mt * 16 + row, nl, acc);
-            else
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), rsrc_p, partial_off(mt * 16 + row, nl),
-                                                       (uint32_t)chunk * chunk_bytes, SC1);
+    for (int h = 0; h < 2; h++) {
+        const int rl = 8 * h + (lane >> 3);
+        voff_w[h] = (uint32_t)min(n0 + wave * 16 + rl, p.N - 1) * p.ldw_bytes + (uint32_t)(((lane & 7) ^ ((rl >> 1) & 7)) * 16);
+    }
+    char *tbuf = lds + 16 + 2 * XBUF + wave * (2 * TBUF);
+    const int t_rd = c * 128 + ((g ^ ((c >> 1) & 7)) * 16);   // chunk g of row c; chunk g + 4 is at slot ^ 4, i.e. +-64 bytes
+    // activations: staging reads whole rows, rows are dealt to the wavefronts; what lies past the last row or the
+    // last step is given an out-of-range offset (zeros, no memory traffic, no branch around the load)
+    const __amdgpu_buffer_rsrc_t rsrc_x =
+        make_rsrc(p.x + (int64_t)m_base * p.ldx, (uint32_t)(((int64_t)(rows_valid - 1) * p.ldx + p.K) * 2));
+    // antiquant parameters of this lane's column (accumulator column = c)
+    const int pcol = min(n0 + wave * 16 + c, p.N - 1);
+    const bool has_offset = p.offset != nullptr;
+
+    // Weight loads are issued in batches of BODY steps (512 consecutive bytes of each of the 16 rows go out back to
+    // back, so the memory controller sees them together), two batches in registers: one being consumed, one in flight.
+    u32x4 wq[2][BODY][2];
+    auto load_body = [&](int slot, int st) {    // st: first step of the batch, relative to step0
+#pragma unroll
+        for (int j = 0; j < BODY; j++) {
+            const bool ok = st + j < nsteps;
+            const uint32_t kb = (uint32_t)(step0 + st + j) * 128u;
+            wq[slot][j][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ok ? voff_w[0] : kOutOfRange, kb, POLICY);
+            wq[slot][j][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ok ? voff_w[1] : kOutOfRange, kb, POLICY);
         }
-    }
-    if (p.S == 1) return;
-    wait_vmcnt<0>();                          // this wavefront's partial sums have reached the coherence point
-    __syncthreads();
-    uint32_t *cnt = p.counter + (size_t)blockIdx.y * p.sgroups + sgrp;
-    if (threadIdx.x == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = old == (uint32_t)(p.S - 1);
-    }
-    __syncthreads();
-    if (!is_last) return;
-    for (int qd = threadIdx.x; qd < rows_valid * QPR; qd += THREADS) {
-        const int row = qd / QPR, nl = (qd % QPR) * 4;
-        if (n0 + nl >= p.N) continue;
-        const uint32_t off = partial_off(row, nl);
-        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-        for (int ch = 0; ch < p.S; ch += 8) {
-            f32x4 v[8];                       // eight loads in flight
+    };
+    // staging: 16-byte piece q of a row's chunk (8 consecutive k) belongs to step q/16, sub-step t and lane group g with
+    // q % 16 = 8 * (t / 2) + 2 * g + (t % 2); it goes to fragment (step, m tile, t) at lane (g, row % 16)
+    constexpr int XR = (MT * 16 + 7) / 8;          // rows per wavefront
+    u32x4 xst[XR][2];
+    auto stage_load = [&](int ch) {
 #pragma unroll
-            for (int i = 0; i < 8; i++)
-                v[i] = ch + i < p.S ? __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                          rsrc_p, off, (uint32_t)(ch + i) * chunk_bytes, SC1))
-                                    : f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < XR; i++) {
+            const int r = wave + 8 * i;
 #pragma unroll
-            for (int i = 0; i < 8; i++) acc += v[i];
+            for (int h = 0; h < 2; h++) {
+                const int q = lane + 64 * h;
+                const int st = ch * CH + (q >> 4);
+                const bool ok = r < rows_valid && st < nsteps;
+                // lane-dependent part in the vector offset, the chunk's position in the scalar offset
+                xst[i][h] = __builtin_amdgcn_raw_buffer_load_b128(
+                    rsrc_x, ok ? (uint32_t)((r * (int)p.ldx + q * 8) * 2) : kOutOfRange, (uint32_t)(step0 + ch * CH) * 256u, 0);
+            }
         }
-        store_out(row, nl, acc);
+    };
+    auto stage_store = [&](int ch) {
+        char *buf = lds + 16 + (ch & 1) * XBUF;
+#pragma unroll
+        for (int i = 0; i < XR; i++) {
+            const int r = wave + 8 * i;
+            if (r >= MT * 16) continue;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int q = lane + 64 * h;
+                const int sl = q >> 4, rr = q & 15;
+                const int t = 2 * (rr >> 3) + (rr & 1), gg = (rr & 7) >> 1;
+                *reinterpret_cast<u32x4 *>(buf + (((sl * MT + (r >> 4)) * 4 + t) * 64 + gg * 16 + (r & 15)) * 16) = xst[i][h];
+            }
+        }
+    };
+
+    f32x4 P[MT], X[MT], tot[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) P[mt] = X[mt] = tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+    auto fold = [&](int grp) {
+        const float sc = bf16_1(p.scale[(int64_t)grp * p.N + pcol]);
+        const float of = (has_offset ? bf16_1(p.offset[(int64_t)grp * p.N + pcol]) : 0.0f) - 128.0f;
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) tot[mt][q] = __builtin_fmaf(sc, __builtin_fmaf(of, X[mt][q], P[mt][q]), tot[mt][q]);
+            P[mt] = X[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+
+    // prologue: first weight steps in flight, first activation chunk in LDS
+    stage_load(0);                              // before the weights: loads retire in order, and these come from cache
+    load_body(0, 0);
+    load_body(1, BODY);
+    stage_store(0);
+    __syncthreads();
+    // step 0 of the weights goes into the wavefront's turn-around tile
+    *reinterpret_cast<u32x4 *>(tbuf + lane * 16) = wq[0][0][0];
+    *reinterpret_cast<u32x4 *>(tbuf + 1024 + lane * 16) = wq[0][0][1];
+
+    int in_unit = 0, grp = GROUPED ? u0 : 0;
+    for (int ch = 0; ch < nchunks; ch++) {
+        stage_load(ch + 1);                     // past the end: zeros, no memory traffic
+        const char *xb = lds + 16 + (ch & 1) * XBUF + lane * 16;
+#pragma unroll
+        for (int j = 0; j < CH; j++) {
+            const int st = ch * CH + j;
+            const int slot = j / BODY, js = j % BODY;
+            u32x4 xa[4][MT];                    // this step's activation fragments, all requested up front
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) xa[t][mt] = *reinterpret_cast<const u32x4 *>(xb + ((j * MT + mt) * 4 + t) * 1024);
+            // this step's weights in operand order (written during the previous step), then the next step's
+            // registers take their place in the other half of the tile
+            const char *tr = tbuf + (j & 1) * TBUF + t_rd;
+            u32x4 w0 = *reinterpret_cast<const u32x4 *>(tr) ^ 0x80808080u;
+            u32x4 w1 = *reinterpret_cast<const u32x4 *>(tbuf + (j & 1) * TBUF + (t_rd ^ 64)) ^ 0x80808080u;
+            {
+                const int sn = ((j + 1) / BODY) & 1, jsn = (j + 1) % BODY;
+                char *tw = tbuf + ((j + 1) & 1) * TBUF + lane * 16;
+                *reinterpret_cast<u32x4 *>(tw) = wq[sn][jsn][0];
+                *reinterpret_cast<u32x4 *>(tw + 1024) = wq[sn][jsn][1];
+            }
+            if (js == BODY - 1) {               // the batch has left the registers: refill its slot two batches ahead
+                __builtin_amdgcn_sched_barrier(0);
+                load_body(slot, st + 1 + BODY);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const uint32_t lo = t < 2 ? w0[2 * (t & 1)] : w1[2 * (t & 1)], hi = t < 2 ? w0[2 * (t & 1) + 1] : w1[2 * (t & 1) + 1];
+                u32x4 b;
+                b[0] = pack_bf16x2((float)(lo & 0xffu), (float)((lo >> 8) & 0xffu));
+                b[1] = pack_bf16x2((float)((lo >> 16) & 0xffu), (float)(lo >> 24));
+                b[2] = pack_bf16x2((float)(hi & 0xffu), (float)((hi >> 8) & 0xffu));
+                b[3] = pack_bf16x2((float)((hi >> 16) & 0xffu), (float)(hi >> 24));
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    P[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[t][mt]), __builtin_bit_cast(bf16x8, b), P[mt], 0, 0, 0);
+                    X[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[t][mt]), __builtin_bit_cast(bf16x8, ones), X[mt], 0, 0, 0);
+                }
+            }
+            if constexpr (GROUPED) {
+                if (st < nsteps && ++in_unit == p.unit_steps) {
+                    fold(grp);
+                    in_unit = 0;
+                    grp++;
+                }
+            }
+        }
+        stage_store(ch + 1);
+        __syncthreads();
     }
-    if (threadIdx.x == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
+    if constexpr (!GROUPED) fold(0);
+
+    // ---- output: the wavefront's [rows x 16 columns] tile goes through LDS to the shared output / exchange code
+    float *red = reinterpret_cast<float *>(lds + 16);
+    TileOut<NBW, 1, THREADS> outp(p, lds, m_base, n0, chunk);
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const int rows_mt = min(16, rows_valid - mt * 16);
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int row = 4 * g + q;
+            if (row < rows_mt) red[row * NBW + wave * 16 + c] = tot[mt][q];
+        }
+        __syncthreads();
+        outp.emit_mtile(red, mt * 16, rows_mt);
+    }
+    outp.finish(rows_valid, tile);
 }
 
 // Any layout (including K-major int8 weights, i.e. the transposed view of an [N,K] tensor),
@@ -573,6 +809,55 @@ int launch_body(const WqArgs &p, const WqPlan &pl, hipStream_t s)
     return MI355_ERR_UNSUPPORTED;
 }
 
+// K-major int8 weights ([N, K] storage).
+struct WqKmPlan {
+    bool fast;
+    int mt, mchunks, tiles, S, unit_steps, n_units;
+    bool grouped;
+    size_t partial_bytes, counter_bytes, lds_bytes;
+};
+
+WqKmPlan make_kmajor_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, int64_t ldw_n, int64_t ldx, const void *x,
+                          const void *w)
+{
+    WqKmPlan pl{};
+    const int64_t group = group_size > 0 ? group_size : K;
+    pl.fast = K > 0 && K % 128 == 0 && group % 128 == 0 && ldw_n >= K && ldw_n % 16 == 0 && ldx % 8 == 0 &&
+              (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 16)) &&
+              (uint64_t)N * (uint64_t)ldw_n < (1ull << 32) && (uint64_t)M * (uint64_t)ldx * 2 < (1ull << 32);
+    if (!pl.fast) return pl;
+    pl.mt = M <= 16 ? 1 : 2;
+    pl.mchunks = (int)((M + pl.mt * 16 - 1) / (pl.mt * 16));
+    pl.tiles = (int)((N + 127) / 128);
+    pl.grouped = group_size > 0 && group != K;
+    pl.unit_steps = pl.grouped ? (int)(group / 128) : 1;
+    pl.n_units = (int)(K / (128 * pl.unit_steps));
+    int S = kNumCU / (pl.tiles * pl.mchunks);
+    if (S > pl.n_units) S = pl.n_units;
+    if (S > 16) S = 16;
+    if (S < 1) S = 1;
+    if (const int f = env_int("MI355_WQ_SPLIT"))
+        if (f >= 1 && f <= pl.n_units) S = f;
+    if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1;
+    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) S = 1;
+    pl.S = S;
+    pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
+    pl.counter_bytes = S > 1 ? kWorkspaceCounterBytes : 0;
+    pl.lds_bytes = 16 + (size_t)2 * 32768 + 8 * 2 * 2048;   // two activation chunks + the turn-around tiles
+    return pl;
+}
+
+template <int MT, bool GROUPED>
+int launch_kmajor(const WqArgs &p, const WqKmPlan &pl, hipStream_t s)
+{
+    auto kern = wq_kmajor_kernel<MT, GROUPED>;
+    static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)((pl.tiles + 7) / 8 * 8 * pl.S), (unsigned)pl.mchunks), dim3(512), pl.lds_bytes, s, p);
+    return check_launch();
+}
+
 template <int WBITS>
 int launch_bits(const WqArgs &p, const WqPlan &pl, hipStream_t s)
 {
@@ -595,7 +880,12 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
     if (M <= 0 || N <= 0 || K <= 0 || (w_bits != 4 && w_bits != 8) || group_size < 0) return 0;
     // the largest request over the layouts the streaming kernel accepts (row pitch = row length)
     const WqPlan pl = make_plan(M, N, K, w_bits, group_size, true, w_bits == 4 ? N / 8 : N, K, nullptr, nullptr, nullptr, nullptr);
-    return pl.fast ? pl.partial_bytes + pl.counter_bytes : 0;
+    size_t need = pl.fast ? pl.partial_bytes + pl.counter_bytes : 0;
+    if (w_bits == 8) {                      // the K-major layout may split differently
+        const WqKmPlan km = make_kmajor_plan(M, N, K, group_size, K, K, nullptr, nullptr);
+        if (km.fast && km.partial_bytes + km.counter_bytes > need) need = km.partial_bytes + km.counter_bytes;
+    }
+    return need;
 }
 
 extern "C" int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int w_bits, const void *scale_bf16,
@@ -616,6 +906,40 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int group = (int)(group_size > 0 ? group_size : (K > 0 ? K : 1));
 
+    if (w_bits == 8 && ldw_k == 1 && ldw_n != 1) {
+        // K-major: the transposed view of an [N, K] weight
+        const WqKmPlan km = make_kmajor_plan(M, N, K, group_size, ldw_n, ldx, x_bf16, w);
+        const bool params_ok = aligned(scale_bf16, 2) && (!offset_bf16 || aligned(offset_bf16, 2));
+        if (km.fast && params_ok) {
+            if (km.S > 1) {
+                if (!workspace || workspace_bytes < km.partial_bytes + km.counter_bytes) return MI355_ERR_WORKSPACE;
+                if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+            }
+            WqArgs p{};
+            p.x = static_cast<const uint16_t *>(x_bf16);
+            p.w = w;
+            p.scale = static_cast<const uint16_t *>(scale_bf16);
+            p.offset = static_cast<const uint16_t *>(offset_bf16);
+            p.out = static_cast<uint16_t *>(out_bf16);
+            p.counter = km.S > 1 ? static_cast<uint32_t *>(workspace) : nullptr;
+            p.partial = km.S > 1 ? reinterpret_cast<float *>(static_cast<char *>(workspace) + km.counter_bytes) : nullptr;
+            p.ldx = ldx;
+            p.ldo = ldo;
+            p.ldw_bytes = (uint32_t)ldw_n;
+            p.row_bytes = (uint32_t)K;
+            p.M = (int)M;
+            p.N = (int)N;
+            p.K = (int)K;
+            p.unit_steps = km.unit_steps;
+            p.n_units = km.n_units;
+            p.grouped = km.grouped;
+            p.strips = km.tiles;
+            p.sgroups = km.tiles;
+            p.S = km.S;
+            if (km.mt == 1) return km.grouped ? launch_kmajor<1, true>(p, km, s) : launch_kmajor<1, false>(p, km, s);
+            return km.grouped ? launch_kmajor<2, true>(p, km, s) : launch_kmajor<2, false>(p, km, s);
+        }
+    }
     const bool n_major = w_bits == 4 || (ldw_n == 1 && ldw_k >= N);
     const WqPlan pl = make_plan(M, N, K, w_bits, group_size, n_major, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
     if (!pl.fast) {
