@@ -755,6 +755,13 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
         while (slab_steps(S) > kMaxSlabSteps && S < s_max) S++;
         if (const int f = env_int("MI355_WQ_SPLIT"))  // tuning aid: force the number of K chunks
             if (f >= 1 && f <= s_max) S = f;
+        if (w_bits == 4 && pl.mt == 2 && grouped && nwv == 8 && pl.bs == 4) {
+            // two m tiles of int4 run much better without the running total (eight wavefronts, no spills): split K
+            // further, down to one scale group per wavefront, when that stays within 16 chunks (measured at
+            // M = 128, K = 4096: 73 us against 92 us)
+            const int s_one = (pl.n_units + pl.ks - 1) / pl.ks;
+            if (s_one > S && s_one <= 16 && s_one <= s_max && !env_int("MI355_WQ_SPLIT")) S = s_one;
+        }
         if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1; // exchange offsets are 32-bit
         pl.S = S;
         pl.slab_bytes = (size_t)slab_steps(S) * 1024;
