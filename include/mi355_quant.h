@@ -41,7 +41,14 @@ typedef enum mi355_status {
 
 /* Output formats of mi355_quant_matmul. */
 #define MI355_OUT_BF16 0
-#define MI355_OUT_INT32 1   /* raw int32 accumulators (+ int32 bias is not applied) */
+#define MI355_OUT_INT32 1   /* int32 accumulators (plus an int32 bias if given); scales are ignored */
+#define MI355_OUT_FP16 2
+
+/* bias element types of mi355_quant_matmul */
+#define MI355_BIAS_NONE 0
+#define MI355_BIAS_BF16 1   /* added after both scales */
+#define MI355_BIAS_INT32 2  /* added to the int32 accumulator before dequantisation (wraps like the accumulator) */
+#define MI355_BIAS_FP32 3   /* added after both scales */
 
 const char *mi355_status_string(int status);
 
@@ -74,9 +81,13 @@ int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth,
  *   b   int8 logical [K, N], element (k,n) at b[k*ldb_k + n*ldb_n]; one of ldb_k, ldb_n must be 1
  *       (ldb_n == 1: contiguous [K,N]; ldb_k == 1: the transposed view of an [N,K] weight)
  *   pertoken_scale  float32 [M] or NULL;   scale float32 [scale_len], scale_len in {1, N}
- *   bias            bf16 [N] or NULL (MI355_OUT_BF16 only)
- *   out_dtype MI355_OUT_BF16:  out[m*ldc+n] = bf16(((float(acc) * pertoken_scale[m]) * scale[n]) + float(bias[n]))
- *             MI355_OUT_INT32: out[m*ldc+n] = acc (scales and bias are ignored and may be NULL)
+ *   bias            [N] of bias_dtype (MI355_BIAS_*) or NULL with MI355_BIAS_NONE.  LinearQuant's default bias is
+ *                   int32 (linear_quant.py:92), the bf16-output configuration uses bf16.
+ *   out_dtype MI355_OUT_BF16 / MI355_OUT_FP16:
+ *                 out[m*ldc+n] = round(((float(acc + bias_i32[n]) * pertoken_scale[m]) * scale[n]) + float(bias[n]))
+ *                 (each bias term only for its type), rounded once to bf16 / fp16
+ *             MI355_OUT_INT32: out[m*ldc+n] = acc + bias_i32[n] (scales are ignored and may be NULL; other bias
+ *                 types are rejected)
  *   workspace: at least mi355_quant_matmul_workspace(...) bytes (may be NULL when that is 0), 16-byte aligned.
  *              It holds a transposed copy of a contiguous [K,N] weight and, for narrow outputs with a long K,
  *              the partial sums and arrival counters of a split over K.  The counters lie at its start and
@@ -87,7 +98,7 @@ size_t mi355_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int64_t ldb
 
 int mi355_quant_matmul(const int8_t *a, const int8_t *b,
                        const float *pertoken_scale, const float *scale, int64_t scale_len,
-                       const void *bias_bf16, void *out, int out_dtype,
+                       const void *bias, int bias_dtype, void *out, int out_dtype,
                        int64_t M, int64_t N, int64_t K,
                        int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                        void *workspace, size_t workspace_bytes, void *stream);

@@ -221,6 +221,58 @@ void orc_quant_matmul_epilogue(const int32_t *acc, const float *pertoken_scale, 
     }
 }
 
+/* binary32 -> binary16, round to nearest even (overflow to infinity, gradual underflow). */
+static inline uint16_t f32_to_f16(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);              /* NaN */
+    if (a >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);             /* >= 65536 (or inf): infinity; 65520..65535.99 round below */
+    if (a < 0x33000000u) return sign;                                    /* < 2^-25: rounds to zero */
+    int e = (int)(a >> 23) - 127;                                        /* unbiased exponent */
+    uint32_t mant = (a & 0x7fffffu) | 0x800000u;                         /* 24-bit significand */
+    int shift = e < -14 ? 13 + (-14 - e) : 13;                           /* bits dropped */
+    uint32_t kept = mant >> shift, rest = mant & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rest > half || (rest == half && (kept & 1u))) kept++;
+    /* normal: kept has bit 10 set (or 11 after a carry); subnormal: kept < 1024 */
+    uint32_t h = e < -14 ? kept : ((uint32_t)(e + 15) << 10) + (kept - 1024u);
+    return (uint16_t)(sign | (h > 0x7c00u ? 0x7c00u : h));
+}
+
+/*
+ * The wider signature surface of npu_quant_matmul (shapes and dtypes: test/test_fake_tensor.py:1886-1915;
+ * LinearQuant's default int32 bias: torch_npu/contrib/module/linear_quant.py:92):
+ *   bias_kind 0 none, 1 bf16 (added after both scales), 2 int32 (added to the int32 accumulator before
+ *   dequantisation, wrapping like the accumulator), 3 float32 (added after both scales);
+ *   out_kind 0 bf16, 1 fp16, 2 int32 (accumulator plus int32 bias, no scaling).
+ * Results on Ascend silicon: PARITY UNPINNED (no in-tree result test); the formula is the benchmark
+ * configuration's with the bias moved where its type puts it.
+ */
+void orc_quant_matmul_epilogue_ex(const int32_t *acc, const float *pertoken_scale, const float *scale,
+                                  int64_t scale_len, const void *bias, int bias_kind, int out_kind,
+                                  int64_t M, int64_t N, void *out)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; m++) {
+        for (int64_t n = 0; n < N; n++) {
+            int32_t a = acc[m * N + n];
+            if (bias_kind == 2) a = (int32_t)((uint32_t)a + (uint32_t)((const int32_t *)bias)[n]);
+            if (out_kind == 2) {
+                ((int32_t *)out)[m * N + n] = a;
+                continue;
+            }
+            float f = (float)a;
+            if (pertoken_scale) f = f * pertoken_scale[m];
+            f = f * scale[scale_len == 1 ? 0 : n];
+            if (bias_kind == 1) f = f + bf16_to_f32(((const uint16_t *)bias)[n]);
+            if (bias_kind == 3) f = f + ((const float *)bias)[n];
+            ((uint16_t *)out)[m * N + n] = out_kind == 1 ? f32_to_f16(f) : f32_to_bf16(f);
+        }
+    }
+}
+
 /* ------------------------------------------------ int4 packing / antiquant */
 /*
  * int32 word j of a row holds logical elements 8j..8j+7; element i sits in bits

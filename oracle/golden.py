@@ -41,6 +41,7 @@ def lib() -> ctypes.CDLL:
         L.orc_dynamic_quant.argtypes = [vp, i32, vp, i64, i64, i64, vp, vp]
         L.orc_int8_gemm.argtypes = [vp, i64, vp, i64, i64, i64, i64, i64, vp]
         L.orc_quant_matmul_epilogue.argtypes = [vp, vp, vp, i64, vp, i64, i64, vp]
+        L.orc_quant_matmul_epilogue_ex.argtypes = [vp, vp, vp, i64, vp, i32, i32, i64, i64, vp]
         L.orc_unpack_int4.argtypes = [vp, i64, vp]
         L.orc_pack_int4.argtypes = [vp, i64, vp]
         L.orc_antiquant.argtypes = [vp, vp, vp, i64, i64, vp]
@@ -112,6 +113,26 @@ def quant_matmul_epilogue(acc, scale, pertoken_scale=None, bias_u16=None) -> np.
     if M and N:
         lib().orc_quant_matmul_epilogue(_p(acc), _p(ps), _p(scale), scale.size, _p(bias), M, N, _p(out))
     return out
+
+
+def quant_matmul_epilogue_ex(acc, scale, pertoken_scale=None, bias=None, out: str = "bf16") -> np.ndarray:
+    """bias: None, uint16 (bf16 bit patterns), int32 or float32 array [N]; out: "bf16" / "fp16" (uint16 bit patterns)
+    or "int32"."""
+    acc = _c(acc, np.int32)
+    M, N = acc.shape
+    ps = None if pertoken_scale is None else _c(pertoken_scale, np.float32).reshape(-1)
+    sc = None if scale is None else _c(scale, np.float32).reshape(-1)
+    kind = 0
+    if bias is not None:
+        kind = {np.dtype(np.uint16): 1, np.dtype(np.int32): 2, np.dtype(np.float32): 3}[np.asarray(bias).dtype]
+        bias = np.ascontiguousarray(np.asarray(bias).reshape(-1))
+        assert bias.size == N
+    out_kind = {"bf16": 0, "fp16": 1, "int32": 2}[out]
+    res = np.empty((M, N), dtype=np.int32 if out_kind == 2 else np.uint16)
+    if M and N:
+        lib().orc_quant_matmul_epilogue_ex(_p(acc), _p(ps), _p(sc), 0 if sc is None else sc.size, _p(bias), kind,
+                                           out_kind, M, N, _p(res))
+    return res
 
 
 def quant_matmul(a, b, scale, pertoken_scale=None, bias_u16=None):

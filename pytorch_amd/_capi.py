@@ -38,7 +38,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_dynamic_quant.argtypes = [vp, i32, vp, vp, vp, i64, i64, i64, vp]
         L.mi355_quant_matmul_workspace.restype = sz
         L.mi355_quant_matmul_workspace.argtypes = [i64, i64, i64, i64, i64]
-        L.mi355_quant_matmul.argtypes = [vp, vp, vp, vp, i64, vp, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
+        L.mi355_quant_matmul.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
         L.mi355_weight_quant_matmul_workspace.restype = sz
         L.mi355_weight_quant_matmul_workspace.argtypes = [i64, i64, i64, i32, i64]
         L.mi355_weight_quant_matmul.argtypes = [vp, vp, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
@@ -95,10 +95,11 @@ def quant_matmul(x1, x2, scale, pertoken_scale=None, bias=None, out_dtype=torch.
     need = lib().mi355_quant_matmul_workspace(M, N, K, x2.stride(0), x2.stride(1))
     if workspace is None and need:
         workspace = _wq_workspace(x1.device, need)      # its leading counters must start at zero
+    bias_dtype = 0 if bias is None else {torch.bfloat16: 1, torch.int32: 2, torch.float32: 3}[bias.dtype]
+    out_code = {torch.bfloat16: 0, torch.int32: 1, torch.float16: 2}[out_dtype]
     st = lib().mi355_quant_matmul(_ptr(x1), _ptr(x2), _ptr(pertoken_scale), _ptr(scale),
-                                  0 if scale is None else scale.numel(), _ptr(bias), _ptr(out),
-                                  0 if out_dtype == torch.bfloat16 else 1, M, N, K, x1.stride(0),
-                                  x2.stride(0), x2.stride(1), out.stride(0), _ptr(workspace),
+                                  0 if scale is None else scale.numel(), _ptr(bias), bias_dtype, _ptr(out), out_code,
+                                  M, N, K, x1.stride(0), x2.stride(0), x2.stride(1), out.stride(0), _ptr(workspace),
                                   0 if workspace is None else workspace.numel(), _stream())
     _check(st, "mi355_quant_matmul")
     return out

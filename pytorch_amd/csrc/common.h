@@ -47,6 +47,15 @@ __device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2)
 // zero-initialised buffer can be shared by all launches of a stream.
 constexpr size_t kWorkspaceCounterBytes = 16384;
 
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 v;
+    v[0] = (_Float16)lo;        // round to nearest even
+    v[1] = (_Float16)hi;
+    return __builtin_bit_cast(uint32_t, v);
+}
+
 inline int check_launch()
 {
     return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ERR_LAUNCH;

@@ -159,14 +159,15 @@ QmmPlan quant_matmul_plan(const Tensor &x1, const Tensor &x2, const Tensor &scal
                 x2.size(-2), ", ", p.N, "]");
     TORCH_CHECK(output_dtype.has_value(),
                 "npu_quant_matmul: output_dtype=None selects the int8 re-quantised output, which is not supported; "
-                "pass output_dtype=torch.bfloat16 or torch.int32");
+                "pass output_dtype=torch.bfloat16, torch.float16 or torch.int32");
     p.out_dtype = *output_dtype;
-    TORCH_CHECK(p.out_dtype == at::kBFloat16 || p.out_dtype == at::kInt,
-                "npu_quant_matmul: output_dtype must be torch.bfloat16 or torch.int32, got ", p.out_dtype);
+    TORCH_CHECK(p.out_dtype == at::kBFloat16 || p.out_dtype == at::kHalf || p.out_dtype == at::kInt,
+                "npu_quant_matmul: output_dtype must be torch.bfloat16, torch.float16 or torch.int32, got ", p.out_dtype);
     TORCH_CHECK(!opt(offset), "npu_quant_matmul: offset is only meaningful for int8 output, which is not supported");
-    if (p.out_dtype == at::kBFloat16) {
+    if (p.out_dtype != at::kInt) {
+        // (an int64 scale is the packed output of npu_trans_quant_param, which is not built)
         TORCH_CHECK(scale.scalar_type() == at::kFloat || scale.scalar_type() == at::kBFloat16,
-                    "npu_quant_matmul: scale must be float32 or bfloat16 for bfloat16 output, got ", scale.scalar_type());
+                    "npu_quant_matmul: scale must be float32 or bfloat16 for a floating-point output, got ", scale.scalar_type());
         TORCH_CHECK(scale.dim() == 1 && (scale.size(0) == 1 || scale.size(0) == p.N),
                     "npu_quant_matmul: scale must have shape [1] or [", p.N, "]");
         if (const Tensor *ps = opt(pertoken_scale)) {
@@ -174,12 +175,18 @@ QmmPlan quant_matmul_plan(const Tensor &x1, const Tensor &x2, const Tensor &scal
             TORCH_CHECK(ps->dim() == 1 && ps->size(0) == p.M, "npu_quant_matmul: pertoken_scale must have shape [", p.M, "]");
         }
         if (const Tensor *b = opt(bias)) {
-            TORCH_CHECK(b->scalar_type() == at::kBFloat16,
-                        "npu_quant_matmul: bias must be bfloat16 for bfloat16 output, got ", b->scalar_type());
+            // int32: added to the accumulator (LinearQuant's default bias dtype, linear_quant.py:92); bf16 / float32:
+            // added after dequantisation
+            TORCH_CHECK(b->scalar_type() == at::kInt || b->scalar_type() == at::kFloat ||
+                            (b->scalar_type() == at::kBFloat16 && p.out_dtype == at::kBFloat16),
+                        "npu_quant_matmul: bias must be int32, float32 or (for bfloat16 output) bfloat16, got ", b->scalar_type());
             TORCH_CHECK(b->numel() == p.N && b->size(-1) == p.N, "npu_quant_matmul: bias must have shape [", p.N, "]");
         }
     } else {
-        TORCH_CHECK(!opt(bias), "npu_quant_matmul: bias with int32 output is not supported");
+        if (const Tensor *b = opt(bias)) {
+            TORCH_CHECK(b->scalar_type() == at::kInt, "npu_quant_matmul: bias must be int32 for int32 output, got ", b->scalar_type());
+            TORCH_CHECK(b->numel() == p.N && b->size(-1) == p.N, "npu_quant_matmul: bias must have shape [", p.N, "]");
+        }
         TORCH_CHECK(!opt(pertoken_scale), "npu_quant_matmul: pertoken_scale is not applicable to int32 output");
     }
     auto b1 = x1.sizes().slice(0, x1.dim() - 2), b2 = x2.sizes().slice(0, x2.dim() - 2);
@@ -220,13 +227,17 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
     c10::hip::HIPGuardMasqueradingAsCUDA guard(x1.device());
     Tensor out = at::empty(p.out_shape, x1.options().dtype(p.out_dtype));
     if (out.numel() == 0) return out;
-    const bool bf16 = p.out_dtype == at::kBFloat16;
+    const bool bf16 = p.out_dtype != at::kInt;            // a floating-point (dequantised) output
     Tensor scale_f, ps, b;
     if (bf16) {
         scale_f = scale.to(at::kFloat).contiguous();
         if (const Tensor *t = opt(pertoken_scale)) ps = t->contiguous();
-        if (const Tensor *t = opt(bias)) b = t->reshape({p.N}).contiguous();
     }
+    if (const Tensor *t = opt(bias)) b = t->reshape({p.N}).contiguous();
+    const int bias_dtype = !b.defined() ? MI355_BIAS_NONE
+                           : b.scalar_type() == at::kInt ? MI355_BIAS_INT32
+                           : b.scalar_type() == at::kFloat ? MI355_BIAS_FP32 : MI355_BIAS_BF16;
+    const int out_dtype = p.out_dtype == at::kInt ? MI355_OUT_INT32 : p.out_dtype == at::kHalf ? MI355_OUT_FP16 : MI355_OUT_BF16;
     int64_t nb = 1;
     for (auto d : p.batch) nb *= d;
     // x1 with batch dimensions against a single weight matrix is one tall matmul
@@ -256,8 +267,8 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
         Tensor o = out2d.narrow(0, row0, m);
         check_status(mi355_quant_matmul(a.data_ptr<int8_t>(), w.data_ptr<int8_t>(), ps.defined() ? ps.data_ptr<float>() : nullptr,
                                         bf16 ? scale_f.data_ptr<float>() : nullptr, bf16 ? scale_f.numel() : 0,
-                                        b.defined() ? b.data_ptr() : nullptr, o.data_ptr(),
-                                        bf16 ? MI355_OUT_BF16 : MI355_OUT_INT32, m, p.N, p.K, a.stride(0), w.stride(0),
+                                        b.defined() ? b.data_ptr() : nullptr, bias_dtype, o.data_ptr(), out_dtype, m, p.N, p.K,
+                                        a.stride(0), w.stride(0),
                                         w.stride(1), o.stride(0), ws.defined() ? ws.data_ptr() : nullptr, ws_bytes,
                                         stream_of(x1)),
                      "npu_quant_matmul");

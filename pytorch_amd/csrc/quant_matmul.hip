@@ -58,7 +58,9 @@ struct QmmArgs {
     const int8_t *bt;          // [N, K] K-major
     const float *pertoken;     // [M] or null
     const float *scale;        // [scale_len]
-    const uint16_t *bias;      // bf16 [N] or null
+    const void *bias;          // [N] of bias_kind, or null
+    int bias_kind;             // MI355_BIAS_*
+    int out_f16;               // round to fp16 instead of bf16
     void *out;
     int64_t lda, ldbt, ldc;
     int M, N, K;
@@ -255,6 +257,19 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     const int mrow = lane & 15;
     const int nquad = (lane >> 4) * 4;
     if (p.out_i32) {
+        if (p.bias_kind == MI355_BIAS_INT32) {
+            const int32_t *bb = static_cast<const int32_t *>(p.bias);
+#pragma unroll
+            for (int j = 0; j < WTN; j++) {
+                const int n = n0 + (wn * WTN + j) * 16 + nquad;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int32_t bi = bb[min(n + r, p.N - 1)];
+#pragma unroll
+                    for (int i = 0; i < WTM; i++) acc[i][j][r] = (int32_t)((uint32_t)acc[i][j][r] + (uint32_t)bi);
+                }
+            }
+        }
         const bool vec = (p.ldc & 3) == 0 && aligned_dev(p.out, 16);
 #pragma unroll
         for (int i = 0; i < WTM; i++) {
@@ -283,7 +298,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         psv[i] = p.pertoken ? p.pertoken[m] : 1.0f;
     }
     f32x4 scv[WTN], bsv[WTN];
-    const bool quads = (p.N & 3) == 0 && aligned_dev(p.scale, 16) && (!p.bias || aligned_dev(p.bias, 8));
+    i32x4v biv[WTN];                                          // int32 bias: added to the accumulator before dequantisation
+    const bool quads = (p.N & 3) == 0 && aligned_dev(p.scale, 16) && (!p.bias || aligned_dev(p.bias, 16));
 #pragma unroll
     for (int j = 0; j < WTN; j++) {
         const int n = n0 + (wn * WTN + j) * 16 + nquad;
@@ -297,17 +313,38 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             for (int r = 0; r < 4; r++) scv[j][r] = p.scale[min(n + r, p.N - 1)];
         }
         bsv[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (p.bias) {
+        biv[j] = i32x4v{0, 0, 0, 0};
+        if (p.bias_kind == MI355_BIAS_BF16) {
+            const uint16_t *bb = static_cast<const uint16_t *>(p.bias);
             if (quads) {
-                const u32x2 b2 = *reinterpret_cast<const u32x2 *>(p.bias + min(n, p.N - 4));
+                const u32x2 b2 = *reinterpret_cast<const u32x2 *>(bb + min(n, p.N - 4));
                 bsv[j] = f32x4{bf16_lo(b2.x), bf16_hi(b2.x), bf16_lo(b2.y), bf16_hi(b2.y)};
             } else {
 #pragma unroll
-                for (int r = 0; r < 4; r++) bsv[j][r] = bf16_1(p.bias[min(n + r, p.N - 1)]);
+                for (int r = 0; r < 4; r++) bsv[j][r] = bf16_1(bb[min(n + r, p.N - 1)]);
             }
+        } else if (p.bias_kind == MI355_BIAS_FP32) {
+            const float *bb = static_cast<const float *>(p.bias);
+#pragma unroll
+            for (int r = 0; r < 4; r++) bsv[j][r] = bb[min(n + r, p.N - 1)];
+        } else if (p.bias_kind == MI355_BIAS_INT32) {
+            const int32_t *bb = static_cast<const int32_t *>(p.bias);
+#pragma unroll
+            for (int r = 0; r < 4; r++) biv[j][r] = bb[min(n + r, p.N - 1)];
         }
     }
-    const bool has_ps = p.pertoken != nullptr, has_bias = p.bias != nullptr;
+    const bool has_ps = p.pertoken != nullptr;
+    const bool has_bias = p.bias_kind == MI355_BIAS_BF16 || p.bias_kind == MI355_BIAS_FP32;
+    const bool f16 = p.out_f16 != 0;
+    // (acc + int32 bias) wraps like the hardware accumulator; float bias is added after both scales
+    auto dequant = [&](int32_t a, int32_t bi, float ps, float sc, float bf) {
+        float v = (float)(int32_t)((uint32_t)a + (uint32_t)bi);
+        if (has_ps) v = v * ps;
+        v = v * sc;
+        if (has_bias) v = v + bf;
+        return v;
+    };
+    auto pack2 = [&](float lo, float hi) { return f16 ? pack_f16x2(lo, hi) : pack_bf16x2(lo, hi); };
 
     // The rounded bf16 tile of a wavefront goes through its own LDS region (the stage buffers are idle after the
     // last barrier) so that global stores are 16 bytes per lane and cover whole rows of the wavefront tile.
@@ -323,16 +360,10 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             for (int j = 0; j < WTN; j++) {
                 float f[4];
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    float v = (float)acc[i][j][r];
-                    if (has_ps) v = v * psv[i];
-                    v = v * scv[j][r];
-                    if (has_bias) v = v + bsv[j][r];
-                    f[r] = v;
-                }
+                for (int r = 0; r < 4; r++) f[r] = dequant(acc[i][j][r], biv[j][r], psv[i], scv[j][r], bsv[j][r]);
                 u32x2 pk;
-                pk.x = pack_bf16x2(f[0], f[1]);
-                pk.y = pack_bf16x2(f[2], f[3]);
+                pk.x = pack2(f[0], f[1]);
+                pk.y = pack2(f[2], f[3]);
                 *reinterpret_cast<u32x2 *>(stg + (i * 16 + mrow) * ROWB + (j * 16 + nquad) * 2) = pk;
             }
         const int mw = m0 + wm * WTM * 16, nw = n0 + wn * WTN * 16;
@@ -365,23 +396,17 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             const int n = n0 + (wn * WTN + j) * 16 + nquad;
             float f[4];
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                float v = (float)acc[i][j][r];
-                if (has_ps) v = v * psv[i];
-                v = v * scv[j][r];
-                if (has_bias) v = v + bsv[j][r];
-                f[r] = v;
-            }
+            for (int r = 0; r < 4; r++) f[r] = dequant(acc[i][j][r], biv[j][r], psv[i], scv[j][r], bsv[j][r]);
             if (m >= p.M || n >= p.N) continue;
             uint16_t *o = static_cast<uint16_t *>(p.out) + (int64_t)m * p.ldc + n;
             if (vec && n + 3 < p.N) {
                 u32x2 pk;
-                pk.x = pack_bf16x2(f[0], f[1]);
-                pk.y = pack_bf16x2(f[2], f[3]);
+                pk.x = pack2(f[0], f[1]);
+                pk.y = pack2(f[2], f[3]);
                 *reinterpret_cast<u32x2 *>(o) = pk;
             } else {
                 for (int r = 0; r < 4; r++)
-                    if (n + r < p.N) o[r] = f32_to_bf16(f[r]);
+                    if (n + r < p.N) o[r] = (uint16_t)pack2(f[r], 0.0f);
             }
         }
     }
@@ -392,7 +417,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 __global__ __launch_bounds__(256) void qmm_generic_kernel(const int8_t *__restrict__ a, const int8_t *__restrict__ b,
                                                           const float *__restrict__ pertoken,
                                                           const float *__restrict__ scale, int scale_len,
-                                                          const uint16_t *__restrict__ bias, void *out, int out_i32,
+                                                          const void *__restrict__ bias, int bias_kind, int out_f16, void *out,
+                                                          int out_i32,
                                                           int M, int N, int K, int64_t lda, int64_t ldb_k,
                                                           int64_t ldb_n, int64_t ldc)
 {
@@ -401,6 +427,7 @@ __global__ __launch_bounds__(256) void qmm_generic_kernel(const int8_t *__restri
     if (m >= M || n >= N) return;
     int32_t s = 0;
     for (int k = 0; k < K; k++) s += (int32_t)a[(int64_t)m * lda + k] * (int32_t)b[(int64_t)k * ldb_k + (int64_t)n * ldb_n];
+    if (bias_kind == MI355_BIAS_INT32) s = (int32_t)((uint32_t)s + (uint32_t)static_cast<const int32_t *>(bias)[n]);
     if (out_i32) {
         static_cast<int32_t *>(out)[(int64_t)m * ldc + n] = s;
         return;
@@ -408,8 +435,9 @@ __global__ __launch_bounds__(256) void qmm_generic_kernel(const int8_t *__restri
     float v = (float)s;
     if (pertoken) v = v * pertoken[m];
     v = v * scale[scale_len == 1 ? 0 : n];
-    if (bias) v = v + bf16_1(bias[n]);
-    static_cast<uint16_t *>(out)[(int64_t)m * ldc + n] = f32_to_bf16(v);
+    if (bias_kind == MI355_BIAS_BF16) v = v + bf16_1(static_cast<const uint16_t *>(bias)[n]);
+    if (bias_kind == MI355_BIAS_FP32) v = v + static_cast<const float *>(bias)[n];
+    static_cast<uint16_t *>(out)[(int64_t)m * ldc + n] = (uint16_t)(out_f16 ? pack_f16x2(v, 0.0f) : pack_bf16x2(v, 0.0f));
 }
 
 // [K,N] contiguous -> [N,K] contiguous, 64x64 byte tiles through LDS.
@@ -538,19 +566,22 @@ extern "C" size_t mi355_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, 
 }
 
 extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale,
-                                  int64_t scale_len, const void *bias_bf16, void *out, int out_dtype, int64_t M,
+                                  int64_t scale_len, const void *bias, int bias_dtype, void *out, int out_dtype, int64_t M,
                                   int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                                   void *workspace, size_t workspace_bytes, void *stream)
 {
     using namespace mi355;
     if (M < 0 || N < 0 || K < 0) return MI355_ERR_BAD_ARGUMENT;
-    if (out_dtype != MI355_OUT_BF16 && out_dtype != MI355_OUT_INT32) return MI355_ERR_BAD_ARGUMENT;
+    if (out_dtype != MI355_OUT_BF16 && out_dtype != MI355_OUT_INT32 && out_dtype != MI355_OUT_FP16) return MI355_ERR_BAD_ARGUMENT;
+    if (bias_dtype < MI355_BIAS_NONE || bias_dtype > MI355_BIAS_FP32) return MI355_ERR_BAD_ARGUMENT;
+    if ((bias != nullptr) != (bias_dtype != MI355_BIAS_NONE)) return MI355_ERR_BAD_ARGUMENT;
     if (M == 0 || N == 0) return MI355_OK;
     if (!out || ldc < N) return MI355_ERR_BAD_ARGUMENT;
     if (K > 0 && (!a || !b || lda < K)) return MI355_ERR_BAD_ARGUMENT;
     if (ldb_k != 1 && ldb_n != 1) return MI355_ERR_UNSUPPORTED;
-    if (out_dtype == MI355_OUT_BF16 && (!scale || (scale_len != 1 && scale_len != N))) return MI355_ERR_BAD_ARGUMENT;
-    if (out_dtype == MI355_OUT_INT32 && bias_bf16) return MI355_ERR_UNSUPPORTED;
+    if (out_dtype != MI355_OUT_INT32 && (!scale || (scale_len != 1 && scale_len != N))) return MI355_ERR_BAD_ARGUMENT;
+    if (out_dtype == MI355_OUT_INT32 && bias_dtype != MI355_BIAS_NONE && bias_dtype != MI355_BIAS_INT32) return MI355_ERR_UNSUPPORTED;
+    if (bias && !aligned(bias, bias_dtype == MI355_BIAS_BF16 ? 2 : 4)) return MI355_ERR_ALIGNMENT;
     if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return MI355_ERR_UNSUPPORTED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int out_i32 = out_dtype == MI355_OUT_INT32;
@@ -575,7 +606,7 @@ extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float 
     tiled = tiled && (ldbt & 15) == 0 && aligned(bt, 16);
     if (!tiled) {
         hipLaunchKernelGGL(qmm_generic_kernel, dim3((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16)), dim3(256), 0, s,
-                           a, b, pertoken_scale, scale, (int)scale_len, static_cast<const uint16_t *>(bias_bf16), out,
+                           a, b, pertoken_scale, scale, (int)scale_len, bias, bias_dtype, out_dtype == MI355_OUT_FP16 ? 1 : 0, out,
                            out_i32, (int)M, (int)N, (int)K, lda, ldb_k, ldb_n, ldc);
         return check_launch();
     }
@@ -585,7 +616,9 @@ extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float 
     p.bt = bt;
     p.pertoken = out_i32 ? nullptr : pertoken_scale;
     p.scale = scale;
-    p.bias = static_cast<const uint16_t *>(bias_bf16);
+    p.bias = bias;
+    p.bias_kind = bias_dtype;
+    p.out_f16 = out_dtype == MI355_OUT_FP16;
     p.out = out;
     p.lda = lda;
     p.ldbt = ldbt;

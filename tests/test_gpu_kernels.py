@@ -144,6 +144,27 @@ def test_quant_matmul_extreme_accumulators(capi, golden):
     assert np.array_equal(_bits(half), want)
 
 
+@pytest.mark.parametrize("M,K,N", [(256, 512, 352), (64, 4096, 512), (100, 256, 200), (17, 96, 33)])
+def test_quant_matmul_bias_kinds_and_fp16_output(capi, golden, M, K, N):
+    """int32 bias (LinearQuant's default, added to the accumulator), float32 bias, fp16 output, int32 output with bias:
+    bit-identical to the oracle's statement of the same formula."""
+    d = workloads.quant_matmul_inputs(seed=11 + M, M=M, K=K, N=N, weight_nk=True, bias=True)
+    g = torch.Generator().manual_seed(M)
+    bias_i32 = torch.randint(-(1 << 20), 1 << 20, (N,), generator=g, dtype=torch.int32)
+    bias_f32 = torch.randn(N, generator=g)
+    x1, x2, sc, ps = d["x1"].cuda(), d["x2"].cuda(), d["scale"].cuda(), d["pertoken_scale"].cuda()
+    acc = golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy())
+    cases = [(bias_i32, torch.bfloat16, "bf16"), (bias_f32, torch.bfloat16, "bf16"), (bias_i32, torch.float16, "fp16"),
+             (None, torch.float16, "fp16"), (bias_f32, torch.float16, "fp16")]
+    for bias, dt, name in cases:
+        out = capi.quant_matmul(x1, x2, sc, ps, None if bias is None else bias.cuda(), out_dtype=dt)
+        want = golden.quant_matmul_epilogue_ex(acc, d["scale"].numpy(), d["pertoken_scale"].numpy(),
+                                               None if bias is None else bias.numpy(), out=name)
+        assert np.array_equal(out.cpu().view(torch.int16).numpy().view(np.uint16), want), (name, None if bias is None else bias.dtype)
+    out = capi.quant_matmul(x1, x2, None, None, bias_i32.cuda(), out_dtype=torch.int32)
+    assert np.array_equal(out.cpu().numpy(), golden.quant_matmul_epilogue_ex(acc, None, None, bias_i32.numpy(), out="int32"))
+
+
 def test_quant_matmul_split_k_repeated_launches(capi, golden):
     """A narrow output with a long K is split over K (workgroups meet at counters in the shared workspace): the
     down-projection shape of the MLP configuration, launched repeatedly on the same zero-initialised workspace."""
@@ -254,7 +275,7 @@ def test_c_abi_rejects_bad_arguments(capi):
     L = capi.lib()
     assert L.mi355_dynamic_quant(None, 0, None, None, None, -1, 8, 8, None) == -1
     assert L.mi355_dynamic_quant(None, 7, None, None, None, 1, 8, 8, None) == -1
-    assert L.mi355_quant_matmul(None, None, None, None, 0, None, None, 0, 4, 4, 4, 4, 4, 1, 4, None, 0, None) == -1
+    assert L.mi355_quant_matmul(None, None, None, None, 0, None, 0, None, 0, 4, 4, 4, 4, 4, 1, 4, None, 0, None) == -1
     assert L.mi355_weight_quant_matmul(None, None, 5, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
     assert b"workspace" in L.mi355_status_string(-4)
     x1 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")

@@ -119,6 +119,29 @@ def test_linear_quant_module_equals_operator(pa):
         assert torch.equal(got, want)
 
 
+def test_linear_quant_module_default_int32_bias_and_fp16(pa, golden):
+    """LinearQuant as its constructor builds it (int32 bias, linear_quant.py:92) with float16 and bfloat16 outputs,
+    against the oracle's statement of the formula."""
+    from pytorch_amd.contrib.module import LinearQuant
+    d = workloads.quant_matmul_inputs(seed=5, M=48, K=256, N=192, weight_nk=True)
+    g = torch.Generator().manual_seed(9)
+    bias = torch.randint(-50000, 50000, (192,), generator=g, dtype=torch.int32)
+    acc = golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy())
+    for dt, name, pertoken in ((torch.float16, "fp16", False), (torch.bfloat16, "bf16", True), (torch.float16, "fp16", True)):
+        m = LinearQuant(256, 192, bias=True, pertoken_scale=pertoken, output_dtype=dt).cuda()
+        assert m.bias.dtype == torch.int32
+        m.weight.data = d["x2"].t().contiguous().cuda()
+        m.scale.data = d["scale"].cuda()
+        m.bias.data = bias.cuda()
+        if pertoken:
+            m.pertoken_scale.data = d["pertoken_scale"].cuda()
+        got = m(d["x1"].cuda())
+        want = golden.quant_matmul_epilogue_ex(acc, d["scale"].numpy(), d["pertoken_scale"].numpy() if pertoken else None,
+                                               bias.numpy(), out=name)
+        assert got.dtype == dt
+        assert np.array_equal(got.cpu().view(torch.int16).numpy().view(np.uint16), want)
+
+
 def test_linear_weight_quant_module_equals_operator(pa, golden):
     """test/contrib/test_linear_weight_quant.py:53-73 with bf16 parameters, plus the per-group int4 case."""
     from pytorch_amd.contrib.module import LinearWeightQuant

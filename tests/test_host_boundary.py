@@ -97,8 +97,10 @@ def test_meta_quant_matmul(pa):
         pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), offset=_m(1, dtype=torch.float32))
     with pytest.raises(RuntimeError, match="offset"):
         pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), offset=_m(1, dtype=torch.float32), output_dtype=torch.bfloat16)
+    r = pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), bias=_m(100, dtype=torch.int32), output_dtype=torch.float16)
+    assert r.shape == (1, 1, 100) and r.dtype == torch.float16          # test_fake_tensor.py:1903-1906
     with pytest.raises(RuntimeError, match="output_dtype must be"):
-        pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), output_dtype=torch.float16)
+        pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), output_dtype=torch.int8)
     with pytest.raises(RuntimeError, match="int4-packed"):
         pa.npu_quant_matmul(_m(16, 8, dtype=torch.int32), _m(64, 5, dtype=torch.int32), _m(1, dtype=torch.float32),
                             output_dtype=torch.bfloat16)
@@ -108,9 +110,15 @@ def test_meta_quant_matmul(pa):
     with pytest.raises(RuntimeError, match="pertoken_scale must have shape"):
         pa.npu_quant_matmul(_m(4, 8, dtype=torch.int8), _m(8, 4, dtype=torch.int8), _m(4, dtype=torch.float32),
                             pertoken_scale=_m(3, dtype=torch.float32), output_dtype=torch.bfloat16)
-    with pytest.raises(RuntimeError, match="bias must be bfloat16"):
+    r = pa.npu_quant_matmul(_m(4, 8, dtype=torch.int8), _m(8, 4, dtype=torch.int8), _m(4, dtype=torch.float32),
+                            bias=_m(4, dtype=torch.int32), output_dtype=torch.bfloat16)      # LinearQuant's bias dtype
+    assert r.shape == (4, 4)
+    with pytest.raises(RuntimeError, match="bias must be"):
         pa.npu_quant_matmul(_m(4, 8, dtype=torch.int8), _m(8, 4, dtype=torch.int8), _m(4, dtype=torch.float32),
-                            bias=_m(4, dtype=torch.int32), output_dtype=torch.bfloat16)
+                            bias=_m(4, dtype=torch.bfloat16), output_dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="bias must be int32"):
+        pa.npu_quant_matmul(_m(4, 8, dtype=torch.int8), _m(8, 4, dtype=torch.int8), _m(4, dtype=torch.float32),
+                            bias=_m(4, dtype=torch.float32), output_dtype=torch.int32)
 
 
 def test_meta_weight_quant_batchmatmul(pa):

@@ -82,3 +82,40 @@ def test_epilogue_operation_order_is_left_to_right(golden):
     assert (a != b).any()
     out = golden.quant_matmul_epilogue(acc.numpy(), s.numpy(), ps.numpy())
     assert np.array_equal(out, _bits(a.to(torch.bfloat16)))
+
+
+def test_epilogue_ex_fp16_rounding_and_bias_kinds(golden):
+    """The extended epilogue against numpy: float16 rounding is numpy's (IEEE round-to-nearest-even, including the
+    overflow tie at 65520, subnormals and the 2**-25 tie), int32 bias wraps with the accumulator, float biases are
+    added after both scales."""
+    rng = np.random.default_rng(3)
+    M, N = 37, 53
+    acc = rng.integers(-(1 << 22), 1 << 22, size=(M, N), dtype=np.int32)
+    ps = (rng.random(M, dtype=np.float32) * 1e-2 + 1e-4).astype(np.float32)
+    sc = (rng.random(N, dtype=np.float32) * 1e-2 + 1e-4).astype(np.float32)
+    bi = rng.integers(-(1 << 20), 1 << 20, size=N, dtype=np.int32)
+    bf = rng.standard_normal(N).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = ((acc + bi[None, :]).astype(np.float32) * ps[:, None]) * sc[None, :]
+        assert np.array_equal(golden.quant_matmul_epilogue_ex(acc, sc, ps, bi, out="fp16"), want.astype(np.float16).view(np.uint16))
+        want = (acc.astype(np.float32) * ps[:, None]) * sc[None, :] + bf[None, :]
+        assert np.array_equal(golden.quant_matmul_epilogue_ex(acc, sc, ps, bf, out="fp16"), want.astype(np.float16).view(np.uint16))
+        # float16 conversion alone (scale 1, no bias): every interesting magnitude
+        specials = np.array([0, 1, -1, 2047, 2048, 2049, 4097, 65503, 65504, 65519, 65520, 65535, 65536, 1 << 24, -(1 << 24),
+                             (1 << 31) - 1, -(1 << 31)], dtype=np.int64).astype(np.int32).reshape(1, -1)
+        one = np.ones(1, np.float32)
+        assert np.array_equal(golden.quant_matmul_epilogue_ex(specials, one, None, None, out="fp16"),
+                              specials.astype(np.float32).astype(np.float16).view(np.uint16))
+        tiny = np.array([[1, 2, 3, 5, 1023, 1025, 4099]], dtype=np.int32)
+        for s in (2.0 ** -25, 2.0 ** -24, 2.0 ** -26, 3 * 2.0 ** -27, 2.0 ** -14, 2.0 ** -20):
+            sv = np.array([s], np.float32)
+            assert np.array_equal(golden.quant_matmul_epilogue_ex(tiny, sv, None, None, out="fp16"),
+                                  (tiny.astype(np.float32) * sv).astype(np.float16).view(np.uint16)), s
+    # int32 bias wraps like the accumulator, and the int32 output carries it
+    big = np.array([[(1 << 31) - 1, -(1 << 31), 5]], dtype=np.int32)
+    b3 = np.array([1, -1, 7], dtype=np.int32)
+    assert np.array_equal(golden.quant_matmul_epilogue_ex(big, None, None, b3, out="int32"),
+                          np.array([[-(1 << 31), (1 << 31) - 1, 12]], dtype=np.int32))
+    # bf16 output with a bf16 bias is the original epilogue
+    bb = (rng.standard_normal(N).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    assert np.array_equal(golden.quant_matmul_epilogue_ex(acc, sc, ps, bb, out="bf16"), golden.quant_matmul_epilogue(acc, sc, ps, bb))
