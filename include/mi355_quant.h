@@ -110,20 +110,22 @@ int mi355_quant_matmul(const int8_t *a, const int8_t *b,
  *  test/contrib/test_linear_weight_quant.py:20-28; int4 nibble order:
  *  test/custom_ops/test_npu_anti_quant.py:12-24).
  *
- *   x       bf16 [M, K], element (m,k) at x[m*ldx + k]
+ *   x       [M, K] of act_dtype (MI355_DTYPE_BF16 or MI355_DTYPE_FP16, the dtype of the reference's own test,
+ *           test/contrib/test_linear_weight_quant.py:57-62), element (m,k) at x[m*ldx + k]; scale, offset and out
+ *           have the same element type
  *   w       w_bits == 8: int8 logical [K, N], element (k,n) at w[k*ldw_k + n*ldw_n], one stride == 1
  *           w_bits == 4: int32 [K, N/8] contiguous along N (ldw_k = N/8 words, ldw_n ignored);
  *                        word j of a row holds n = 8j..8j+7, element i in bits [4i, 4i+3], two's complement
- *   scale   bf16 [G, N] row-major, G = 1 when group_size == 0 else K / group_size
- *   offset  bf16 [G, N] or NULL
- *   out[m*ldo+n] = bf16( sum_k float(x[m,k]) * ((float(w[k,n]) + float(offset[g,n])) * float(scale[g,n])) )
+ *   scale   [G, N] row-major, G = 1 when group_size == 0 else K / group_size
+ *   offset  [G, N] or NULL
+ *   out[m*ldo+n] = round( sum_k float(x[m,k]) * ((float(w[k,n]) + float(offset[g,n])) * float(scale[g,n])) )
  *   group_size: 0 (per channel) or a multiple of 32 that divides K
  *   workspace: at least mi355_weight_quant_matmul_workspace(...) bytes
  */
 size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size);
 
-int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int w_bits,
-                              const void *scale_bf16, const void *offset_bf16, void *out_bf16,
+int mi355_weight_quant_matmul(const void *x, int act_dtype, const void *w, int w_bits,
+                              const void *scale, const void *offset, void *out,
                               int64_t M, int64_t N, int64_t K, int64_t group_size,
                               int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo,
                               void *workspace, size_t workspace_bytes, void *stream);

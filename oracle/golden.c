@@ -331,12 +331,15 @@ void orc_antiquant(const int8_t *w, const float *scale, const float *offset,
  * out_f32 (optional) receives the unrounded accumulator as float32 (accum 0) or the
  * double rounded to float32 (accum 1).
  */
-void orc_weight_quant_matmul(const uint16_t *x_bf16, int64_t ldx,
+static void weight_quant_matmul_impl(const uint16_t *x_bf16, int64_t ldx,
                              const void *w, int w_bits, int64_t ldw_k, int64_t ldw_n,
                              const uint16_t *scale_bf16, const uint16_t *off_bf16,
                              int64_t M, int64_t N, int64_t K, int64_t group_size, int accum,
-                             uint16_t *out_bf16, float *out_f32)
+                             uint16_t *out_bf16, float *out_f32, int f16)
 {
+    /* f16: activations, parameters and output are IEEE binary16 (the dtype of the reference's own test,
+     * test/contrib/test_linear_weight_quant.py:57-62) instead of bfloat16; nothing else changes */
+#define ACT_TO_F32(h) (f16 ? fp16_to_f32(h) : bf16_to_f32(h))
     int64_t gs = group_size > 0 ? group_size : K;
     float *wf = (float *)malloc(sizeof(float) * (size_t)K * (size_t)N); /* [N][K] */
     float *xf = (float *)malloc(sizeof(float) * (size_t)M * (size_t)K);
@@ -353,12 +356,12 @@ void orc_weight_quant_matmul(const uint16_t *x_bf16, int64_t ldx,
                 int v = (int)((word >> (4 * (n % 8))) & 0xfu);
                 wv = (float)((v ^ 8) - 8);
             }
-            if (off_bf16) wv = wv + bf16_to_f32(off_bf16[g * N + n]);
-            wf[n * K + k] = wv * bf16_to_f32(scale_bf16[g * N + n]);
+            if (off_bf16) wv = wv + ACT_TO_F32(off_bf16[g * N + n]);
+            wf[n * K + k] = wv * ACT_TO_F32(scale_bf16[g * N + n]);
         }
     }
     for (int64_t m = 0; m < M; m++)
-        for (int64_t k = 0; k < K; k++) xf[m * K + k] = bf16_to_f32(x_bf16[m * ldx + k]);
+        for (int64_t k = 0; k < K; k++) xf[m * K + k] = ACT_TO_F32(x_bf16[m * ldx + k]);
 #pragma omp parallel for schedule(static) collapse(2)
     for (int64_t m = 0; m < M; m++) {
         for (int64_t n = 0; n < N; n++) {
@@ -374,12 +377,33 @@ void orc_weight_quant_matmul(const uint16_t *x_bf16, int64_t ldx,
                 for (int64_t k = 0; k < K; k++) s += (double)xr[k] * (double)wr[k];
                 r = (float)s;
             }
-            if (out_bf16) out_bf16[m * N + n] = f32_to_bf16(r);
+            if (out_bf16) out_bf16[m * N + n] = f16 ? f32_to_f16(r) : f32_to_bf16(r);
             if (out_f32) out_f32[m * N + n] = r;
         }
     }
     free(wf);
     free(xf);
+}
+#undef ACT_TO_F32
+
+void orc_weight_quant_matmul(const uint16_t *x_bf16, int64_t ldx,
+                             const void *w, int w_bits, int64_t ldw_k, int64_t ldw_n,
+                             const uint16_t *scale_bf16, const uint16_t *off_bf16,
+                             int64_t M, int64_t N, int64_t K, int64_t group_size, int accum,
+                             uint16_t *out_bf16, float *out_f32)
+{
+    weight_quant_matmul_impl(x_bf16, ldx, w, w_bits, ldw_k, ldw_n, scale_bf16, off_bf16, M, N, K, group_size, accum,
+                             out_bf16, out_f32, 0);
+}
+
+void orc_weight_quant_matmul_f16(const uint16_t *x_f16, int64_t ldx,
+                                 const void *w, int w_bits, int64_t ldw_k, int64_t ldw_n,
+                                 const uint16_t *scale_f16, const uint16_t *off_f16,
+                                 int64_t M, int64_t N, int64_t K, int64_t group_size, int accum,
+                                 uint16_t *out_f16, float *out_f32)
+{
+    weight_quant_matmul_impl(x_f16, ldx, w, w_bits, ldw_k, ldw_n, scale_f16, off_f16, M, N, K, group_size, accum,
+                             out_f16, out_f32, 1);
 }
 
 /* ----------------------------------------------------------------- npu_swiglu */

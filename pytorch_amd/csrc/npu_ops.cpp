@@ -291,7 +291,8 @@ WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &an
                          int64_t inner_precise, optional<at::ScalarType> weight_dtype)
 {
     const char *op = "npu_weight_quant_batchmatmul";
-    TORCH_CHECK(x.scalar_type() == at::kBFloat16, op, ": x must be bfloat16, got ", x.scalar_type());
+    TORCH_CHECK(x.scalar_type() == at::kBFloat16 || x.scalar_type() == at::kHalf, op, ": x must be bfloat16 or float16, got ",
+                x.scalar_type());
     TORCH_CHECK(weight.scalar_type() == at::kChar || weight.scalar_type() == at::kInt, op,
                 ": weight must be int8, or int32 holding 8 int4 values per word, got ", weight.scalar_type());
     TORCH_CHECK(x.dim() >= 2 && weight.dim() == 2, op, ": x must be [..., K] with at least 2 dimensions and weight 2-D");
@@ -311,7 +312,8 @@ WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &an
                     ": antiquant_group_size must be a multiple of 32 that divides K=", p.K);
     p.groups = group_size > 0 ? p.K / group_size : 1;
     auto check_param = [&](const Tensor &t, const char *name) {
-        TORCH_CHECK(t.scalar_type() == at::kBFloat16, op, ": ", name, " must be bfloat16 like x, got ", t.scalar_type());
+        TORCH_CHECK(t.scalar_type() == x.scalar_type(), op, ": ", name, " must have the dtype of x (", x.scalar_type(), "), got ",
+                    t.scalar_type());
         const bool ok1 = t.dim() == 1 && t.size(0) == p.N && p.groups == 1;
         const bool ok2 = t.dim() == 2 && t.size(0) == p.groups && t.size(1) == p.N;
         TORCH_CHECK(ok1 || ok2, op, ": ", name, " must have shape [", p.N, "] (per channel) or [", p.groups, ", ", p.N,
@@ -355,7 +357,8 @@ Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &ant
     const size_t ws_bytes = mi355_weight_quant_matmul_workspace(p.M, p.N, p.K, p.bits, group_size);
     Tensor ws;
     if (ws_bytes) ws = zeroed_workspace(x, ws_bytes);
-    check_status(mi355_weight_quant_matmul(x2.data_ptr(), w.data_ptr(), p.bits, s.data_ptr(), o.defined() ? o.data_ptr() : nullptr,
+    check_status(mi355_weight_quant_matmul(x2.data_ptr(), x.scalar_type() == at::kHalf ? MI355_DTYPE_FP16 : MI355_DTYPE_BF16,
+                                           w.data_ptr(), p.bits, s.data_ptr(), o.defined() ? o.data_ptr() : nullptr,
                                            out2d.data_ptr(), p.M, p.N, p.K, group_size, x2.stride(0), w.stride(0),
                                            p.bits == 4 ? 1 : w.stride(1), out2d.stride(0),
                                            ws.defined() ? ws.data_ptr() : nullptr, ws.defined() ? (size_t)ws.numel() : 0,

@@ -85,24 +85,76 @@ __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcn
 
 // B fragments of the two MFMAs that share byte position jb of the dword (int4) / of MFMA #i (int8).
 // w holds this lane's dword from its 8 k rows; fragment VGPR v pairs rows (2v, 2v+1).
+// Activation / scale / output element type: ACT = 0 bfloat16, 1 float16.  Everything below is the same for both
+// except the 16-bit encodings: conversions, the MFMA variant and the bit positions of the int4 image.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+template <int ACT>
+__device__ __forceinline__ float act_lo(uint32_t u)
+{
+    if constexpr (ACT == 0) return bf16_lo(u);
+    else return (float)__builtin_bit_cast(_Float16, (uint16_t)(u & 0xffffu));
+}
+template <int ACT>
+__device__ __forceinline__ float act_hi(uint32_t u)
+{
+    if constexpr (ACT == 0) return bf16_hi(u);
+    else return (float)__builtin_bit_cast(_Float16, (uint16_t)(u >> 16));
+}
+template <int ACT>
+__device__ __forceinline__ float act_1(uint16_t h)
+{
+    if constexpr (ACT == 0) return bf16_1(h);
+    else return (float)__builtin_bit_cast(_Float16, h);
+}
+template <int ACT>
+__device__ __forceinline__ uint32_t pack_act2(float lo, float hi)
+{
+    if constexpr (ACT == 0) return pack_bf16x2(lo, hi);
+    else return pack_f16x2(lo, hi);
+}
+template <int ACT>
+__device__ __forceinline__ f32x4 mfma_act(u32x4 a, u32x4 b, f32x4 c)
+{
+    if constexpr (ACT == 0)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+template <int ACT>
+constexpr uint32_t kOnes2 = ACT == 0 ? 0x3f803f80u : 0x3c003c00u;      // two ones
+// int4 image: the nibble u = w + 8 goes into the top four mantissa bits of 8.0 (bf16: 8 + u/2 = (w + 24) / 2) or of
+// 16.0 (fp16: 16 + u = w + 24)
+template <int ACT>
+constexpr uint32_t kInt4Magic = ACT == 0 ? 0x41004100u : 0x4c004c00u;
+template <int WBITS, int ACT>
+constexpr float kImageMul = (WBITS == 4 && ACT == 0) ? 2.0f : 1.0f;    // weight = kImageMul * image - kImageBias
 template <int WBITS>
+constexpr float kImageBias = WBITS == 4 ? 24.0f : 128.0f;
+
+template <int WBITS, int ACT>
 __device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint32_t magic, u32x4 &b0, u32x4 &b1)
 {
     if constexpr (WBITS == 4) {
-        // `magic` (0x41004100) lives in a VGPR so that (x & mask) | magic is one v_and_or_b32 (mask from an SGPR)
+        // `magic` (kInt4Magic) lives in a VGPR so that (x & mask) | magic is one v_and_or_b32 (mask from an SGPR)
         const uint32_t sel = 0x0c000c00u | ((4u + jb) << 16) | (uint32_t)jb;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const uint32_t t = __builtin_amdgcn_perm(w[2 * v + 1], w[2 * v], sel); // [byte jb of row 2v, 0, byte jb of row 2v+1, 0]
-            b0[v] = ((t << 3) & 0x00780078u) | magic;                              // low nibble  -> element 2*jb
-            b1[v] = ((t >> 1) & 0x00780078u) | magic;                              // high nibble -> element 2*jb+1
+            if constexpr (ACT == 0) {
+                b0[v] = ((t << 3) & 0x00780078u) | magic;                          // low nibble  -> element 2*jb
+                b1[v] = ((t >> 1) & 0x00780078u) | magic;                          // high nibble -> element 2*jb+1
+            } else {
+                b0[v] = ((t << 6) & 0x03c003c0u) | magic;
+                b1[v] = ((t << 2) & 0x03c003c0u) | magic;
+            }
         }
     } else {
         (void)magic;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            b0[v] = pack_bf16x2((float)((w[2 * v] >> (16 * jb)) & 0xffu), (float)((w[2 * v + 1] >> (16 * jb)) & 0xffu));
-            b1[v] = pack_bf16x2((float)((w[2 * v] >> (16 * jb + 8)) & 0xffu),
+            b0[v] = pack_act2<ACT>((float)((w[2 * v] >> (16 * jb)) & 0xffu), (float)((w[2 * v + 1] >> (16 * jb)) & 0xffu));
+            b1[v] = pack_act2<ACT>((float)((w[2 * v] >> (16 * jb + 8)) & 0xffu),
                                 (float)((w[2 * v + 1] >> (16 * jb + 8)) & 0xffu));
         }
     }
@@ -114,7 +166,7 @@ __device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint
 // order: the exchange uses agent-scope (sc1) write-through stores and cache-bypassing loads, ordered by the
 // wavefronts' own store counters, the workgroup barrier and a relaxed agent-scope counter; a full release/acquire
 // fence would write back and invalidate the whole L2 of the XCD, which costs far more than the kernel itself.
-template <int NBW, int KS, int THREADS>
+template <int NBW, int KS, int THREADS, int ACT>
 struct TileOut {
     static constexpr int QPR = NBW / 4;
     static constexpr int SC1 = 16;            // cache-policy bit: agent scope
@@ -137,12 +189,12 @@ struct TileOut {
         uint16_t *o = p.out + (int64_t)(m_base + row) * p.ldo + n0 + nl;
         if (out_vec) {
             u32x2 pk;
-            pk.x = pack_bf16x2(v[0], v[1]);
-            pk.y = pack_bf16x2(v[2], v[3]);
+            pk.x = pack_act2<ACT>(v[0], v[1]);
+            pk.y = pack_act2<ACT>(v[2], v[3]);
             *reinterpret_cast<u32x2 *>(o) = pk;
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) o[i] = f32_to_bf16(v[i]);
+            for (int i = 0; i < 4; i++) o[i] = (uint16_t)pack_act2<ACT>(v[i], 0.0f);
         }
     }
 
@@ -233,17 +285,17 @@ __device__ __forceinline__ void load_params(u32x4 (&sv)[NPV], u32x4 (&ov)[NPV], 
 // Fold one finished group into the running total: tot += (scale * P_MUL) * (P' + ((offset - X_BIAS) / P_MUL) * X);
 // both rescalings are exact (powers of two).  Lane (c, g) holds accumulator rows 4g + q; with a single activation
 // row only q = 0 of g = 0 is ever stored, so the other components are left alone.
-template <int WBITS, int MT, int NT, int NPV>
+template <int WBITS, int ACT, int MT, int NT, int NPV>
 __device__ __forceinline__ void fold_group(f32x4 (&tot)[MT][NT], f32x4 (&P)[MT][NT], f32x4 (&X)[MT], const u32x4 (&sv)[NPV],
                                            const u32x4 (&ov)[NPV], const bool one_row)
 {
-    constexpr float P_MUL = WBITS == 4 ? 2.0f : 1.0f;
-    constexpr float X_BIAS = WBITS == 4 ? 24.0f : 128.0f;
+    constexpr float P_MUL = kImageMul<WBITS, ACT>;
+    constexpr float X_BIAS = kImageBias<WBITS>;
 #pragma unroll
     for (int i = 0; i < NT; i++) {
         const uint32_t su = sv[i / 8][(i % 8) / 2], ou = ov[i / 8][(i % 8) / 2];
-        const float sc = ((i & 1) ? bf16_hi(su) : bf16_lo(su)) * P_MUL;
-        const float of = (((i & 1) ? bf16_hi(ou) : bf16_lo(ou)) - X_BIAS) * (1.0f / P_MUL);
+        const float sc = ((i & 1) ? act_hi<ACT>(su) : act_lo<ACT>(su)) * P_MUL;
+        const float of = (((i & 1) ? act_hi<ACT>(ou) : act_lo<ACT>(ou)) - X_BIAS) * (1.0f / P_MUL);
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
             const float inner0 = __builtin_fmaf(of, X[mt][0], P[mt][i][0]);
@@ -270,7 +322,7 @@ __device__ __forceinline__ void fold_group(f32x4 (&tot)[MT][NT], f32x4 (&P)[MT][
 // ACCUM: a wavefront may meet more than one scale group, so finished groups are folded into a running total
 // inside the loop.  Without it (per channel, or at most one group per wavefront) the single fold happens after
 // the loop and the loop carries half as many accumulators.
-template <int WBITS, int MT, int W, int KS, int BS, int PF, bool ACCUM>
+template <int WBITS, int ACT, int MT, int W, int KS, int BS, int PF, bool ACCUM>
 __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
 {
     static_assert(BS % PF == 0, "the register ring must divide the loop body");
@@ -326,9 +378,9 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
             P[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
     }
-    const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+    const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
     uint32_t magic;
-    asm volatile("v_mov_b32 %0, 0x41004100" : "=v"(magic));   // opaque to the optimiser: stays in a VGPR
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "n"(kInt4Magic<ACT>));   // opaque to the optimiser: stays in a VGPR
     const bool one_row = MT == 1 && rows_valid == 1;
 
     // register ring: PF steps of weights and activations in flight, the next group's parameters behind them
@@ -401,26 +453,21 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
 #pragma unroll
                 for (int jb = 0; jb < EPD / 2; jb++) {
                     u32x4 b0, b1;
-                    expand_pair<WBITS>(h ? w1 : w0, jb, magic, b0, b1);
+                    expand_pair<WBITS, ACT>(h ? w1 : w0, jb, magic, b0, b1);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
-                        const bf16x8 a = __builtin_bit_cast(bf16x8, xa[mt]);
-                        P[mt][h * EPD + 2 * jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, b0),
-                                                                                       P[mt][h * EPD + 2 * jb], 0, 0, 0);
-                        P[mt][h * EPD + 2 * jb + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            a, __builtin_bit_cast(bf16x8, b1), P[mt][h * EPD + 2 * jb + 1], 0, 0, 0);
+                        P[mt][h * EPD + 2 * jb] = mfma_act<ACT>(xa[mt], b0, P[mt][h * EPD + 2 * jb]);
+                        P[mt][h * EPD + 2 * jb + 1] = mfma_act<ACT>(xa[mt], b1, P[mt][h * EPD + 2 * jb + 1]);
                     }
                 }
             }
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-                X[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[mt]),
-                                                                __builtin_bit_cast(bf16x8, ones), X[mt], 0, 0, 0);
+            for (int mt = 0; mt < MT; mt++) X[mt] = mfma_act<ACT>(xa[mt], ones, X[mt]);
         }
         if constexpr (ACCUM) {
             in_unit += BS;
             if (in_unit == ustep) {
-                fold_group<WBITS, MT, NT, NPV>(tot, P, X, sv, ov, one_row);
+                fold_group<WBITS, ACT, MT, NT, NPV>(tot, P, X, sv, ov, one_row);
                 in_unit = 0;
             }
         }
@@ -431,12 +478,12 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
             for (int i = 0; i < NT; i++) tot[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-        fold_group<WBITS, MT, NT, NPV>(tot, P, X, sv, ov, one_row);
+        fold_group<WBITS, ACT, MT, NT, NPV>(tot, P, X, sv, ov, one_row);
     }
 
     // ---- reduce over the K slices, one m tile at a time: red[slice][row of the m tile][column of the tile]
     float *red = reinterpret_cast<float *>(lds + 16);
-    TileOut<NBW, KS, THREADS> outp(p, lds, m_base, sgrp * NBW, chunk);
+    TileOut<NBW, KS, THREADS, ACT> outp(p, lds, m_base, sgrp * NBW, chunk);
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
         const int rows_mt = min(16, rows_valid - mt * 16);
@@ -468,7 +515,7 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
 // Activations are staged through LDS in chunks of 8 steps, already in fragment order, double buffered: the loads of
 // the next chunk are issued at the top of a chunk, written to LDS at its end, one barrier per chunk.
 // Per group:  out = sum_g scale_g * (P'_g + (offset_g - 128) * X_g)  with the int8 image w + 128 (see the top of the file).
-template <int MT, bool GROUPED>
+template <int MT, bool GROUPED, int ACT>
 __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
 {
     constexpr int NBW = 128, THREADS = 512;
@@ -568,10 +615,10 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
     f32x4 P[MT], X[MT], tot[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) P[mt] = X[mt] = tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+    const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
     auto fold = [&](int grp) {
-        const float sc = bf16_1(p.scale[(int64_t)grp * p.N + pcol]);
-        const float of = (has_offset ? bf16_1(p.offset[(int64_t)grp * p.N + pcol]) : 0.0f) - 128.0f;
+        const float sc = act_1<ACT>(p.scale[(int64_t)grp * p.N + pcol]);
+        const float of = (has_offset ? act_1<ACT>(p.offset[(int64_t)grp * p.N + pcol]) : 0.0f) - 128.0f;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
@@ -623,14 +670,14 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
             for (int t = 0; t < 4; t++) {
                 const uint32_t lo = t < 2 ? w0[2 * (t & 1)] : w1[2 * (t & 1)], hi = t < 2 ? w0[2 * (t & 1) + 1] : w1[2 * (t & 1) + 1];
                 u32x4 b;
-                b[0] = pack_bf16x2((float)(lo & 0xffu), (float)((lo >> 8) & 0xffu));
-                b[1] = pack_bf16x2((float)((lo >> 16) & 0xffu), (float)(lo >> 24));
-                b[2] = pack_bf16x2((float)(hi & 0xffu), (float)((hi >> 8) & 0xffu));
-                b[3] = pack_bf16x2((float)((hi >> 16) & 0xffu), (float)(hi >> 24));
+                b[0] = pack_act2<ACT>((float)(lo & 0xffu), (float)((lo >> 8) & 0xffu));
+                b[1] = pack_act2<ACT>((float)((lo >> 16) & 0xffu), (float)(lo >> 24));
+                b[2] = pack_act2<ACT>((float)(hi & 0xffu), (float)((hi >> 8) & 0xffu));
+                b[3] = pack_act2<ACT>((float)((hi >> 16) & 0xffu), (float)(hi >> 24));
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) {
-                    P[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[t][mt]), __builtin_bit_cast(bf16x8, b), P[mt], 0, 0, 0);
-                    X[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[t][mt]), __builtin_bit_cast(bf16x8, ones), X[mt], 0, 0, 0);
+                    P[mt] = mfma_act<ACT>(xa[t][mt], b, P[mt]);
+                    X[mt] = mfma_act<ACT>(xa[t][mt], ones, X[mt]);
                 }
             }
             if constexpr (GROUPED) {
@@ -648,7 +695,7 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
 
     // ---- output: the wavefront's [rows x 16 columns] tile goes through LDS to the shared output / exchange code
     float *red = reinterpret_cast<float *>(lds + 16);
-    TileOut<NBW, 1, THREADS> outp(p, lds, m_base, n0, chunk);
+    TileOut<NBW, 1, THREADS, ACT> outp(p, lds, m_base, n0, chunk);
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
         const int rows_mt = min(16, rows_valid - mt * 16);
@@ -670,7 +717,7 @@ __global__ __launch_bounds__(256) void wq_generic_kernel(const uint16_t *__restr
                                                          int w_bits, const uint16_t *__restrict__ scale,
                                                          const uint16_t *__restrict__ offset,
                                                          uint16_t *__restrict__ out, int M, int N, int K, int group,
-                                                         int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo)
+                                                         int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo, int act)
 {
     const int n = blockIdx.x * 64 + (threadIdx.x & 63);
     const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -686,11 +733,12 @@ __global__ __launch_bounds__(256) void wq_generic_kernel(const uint16_t *__restr
             const int v = (int)((word >> (4 * (n & 7))) & 0xfu);
             wv = (float)((v ^ 8) - 8);
         }
-        if (offset) wv = wv + bf16_1(offset[(int64_t)gidx * N + n]);
-        wv = wv * bf16_1(scale[(int64_t)gidx * N + n]);
-        acc = acc + bf16_1(x[(int64_t)m * ldx + k]) * wv;
+        auto cvt = [&](uint16_t h) { return act ? act_1<1>(h) : act_1<0>(h); };
+        if (offset) wv = wv + cvt(offset[(int64_t)gidx * N + n]);
+        wv = wv * cvt(scale[(int64_t)gidx * N + n]);
+        acc = acc + cvt(x[(int64_t)m * ldx + k]) * wv;
     }
-    out[(int64_t)m * ldo + n] = f32_to_bf16(acc);
+    out[(int64_t)m * ldo + n] = (uint16_t)(act ? pack_act2<1>(acc, 0.0f) : pack_act2<0>(acc, 0.0f));
 }
 
 struct WqPlan {
@@ -782,7 +830,7 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
     return pl;
 }
 
-template <int WBITS, int MT, int W, int KS, int BS, bool ACCUM>
+template <int WBITS, int ACT, int MT, int W, int KS, int BS, bool ACCUM>
 int launch_stream(const WqArgs &p, const WqPlan &pl, hipStream_t s)
 {
     constexpr int EPD = 32 / WBITS, NB = 32 * EPD;
@@ -793,7 +841,7 @@ int launch_stream(const WqArgs &p, const WqPlan &pl, hipStream_t s)
     constexpr size_t red_bytes = (size_t)KS * 16 * W * NB * sizeof(float);
     static_assert(16 + red_bytes <= 160 * 1024, "LDS budget");
     const size_t lds_bytes = 16 + (red_bytes > pl.slab_bytes ? red_bytes : pl.slab_bytes);
-    auto kern = wq_stream_kernel<WBITS, MT, W, KS, BS, PF, ACCUM>;
+    auto kern = wq_stream_kernel<WBITS, ACT, MT, W, KS, BS, PF, ACCUM>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
@@ -803,15 +851,15 @@ int launch_stream(const WqArgs &p, const WqPlan &pl, hipStream_t s)
 }
 
 // ACC_MODES: 0 = both accumulation modes are instantiated, 1 = only the running total, 2 = only the single fold
-template <int WBITS, int MT, int W, int KS, int ACC_MODES>
+template <int WBITS, int ACT, int MT, int W, int KS, int ACC_MODES>
 int launch_body(const WqArgs &p, const WqPlan &pl, hipStream_t s)
 {
     if constexpr (ACC_MODES != 2) {
-        if (pl.bs == 1) return launch_stream<WBITS, MT, W, KS, 1, true>(p, pl, s);
-        if (pl.accum) return launch_stream<WBITS, MT, W, KS, 4, true>(p, pl, s);
+        if (pl.bs == 1) return launch_stream<WBITS, ACT, MT, W, KS, 1, true>(p, pl, s);
+        if (pl.accum) return launch_stream<WBITS, ACT, MT, W, KS, 4, true>(p, pl, s);
     }
     if constexpr (ACC_MODES != 1) {
-        if (pl.bs == 4 && !pl.accum) return launch_stream<WBITS, MT, W, KS, 4, false>(p, pl, s);
+        if (pl.bs == 4 && !pl.accum) return launch_stream<WBITS, ACT, MT, W, KS, 4, false>(p, pl, s);
     }
     return MI355_ERR_UNSUPPORTED;
 }
@@ -854,10 +902,10 @@ WqKmPlan make_kmajor_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, i
     return pl;
 }
 
-template <int MT, bool GROUPED>
+template <int MT, bool GROUPED, int ACT>
 int launch_kmajor(const WqArgs &p, const WqKmPlan &pl, hipStream_t s)
 {
-    auto kern = wq_kmajor_kernel<MT, GROUPED>;
+    auto kern = wq_kmajor_kernel<MT, GROUPED, ACT>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
@@ -865,17 +913,26 @@ int launch_kmajor(const WqArgs &p, const WqKmPlan &pl, hipStream_t s)
     return check_launch();
 }
 
-template <int WBITS>
+template <int WBITS, int ACT>
 int launch_bits(const WqArgs &p, const WqPlan &pl, hipStream_t s)
 {
-    if (pl.mt == 1) return pl.w == 1 ? launch_body<WBITS, 1, 1, 8, 0>(p, pl, s) : launch_body<WBITS, 1, 2, 4, 0>(p, pl, s);
+    if (pl.mt == 1)
+        return pl.w == 1 ? launch_body<WBITS, ACT, 1, 1, 8, 0>(p, pl, s) : launch_body<WBITS, ACT, 1, 2, 4, 0>(p, pl, s);
     if constexpr (WBITS == 8) {
-        return pl.w == 1 ? launch_body<8, 2, 1, 8, 0>(p, pl, s) : launch_body<8, 2, 2, 4, 0>(p, pl, s);
+        return pl.w == 1 ? launch_body<8, ACT, 2, 1, 8, 0>(p, pl, s) : launch_body<8, ACT, 2, 2, 4, 0>(p, pl, s);
     } else {
         // two m tiles of int4: eight wavefronts only without the running total (see make_plan)
-        if (pl.w * pl.ks == 8) return pl.w == 1 ? launch_body<4, 2, 1, 8, 2>(p, pl, s) : launch_body<4, 2, 2, 4, 2>(p, pl, s);
-        return pl.w == 1 ? launch_body<4, 2, 1, 4, 1>(p, pl, s) : launch_body<4, 2, 2, 2, 1>(p, pl, s);
+        if (pl.w * pl.ks == 8)
+            return pl.w == 1 ? launch_body<4, ACT, 2, 1, 8, 2>(p, pl, s) : launch_body<4, ACT, 2, 2, 4, 2>(p, pl, s);
+        return pl.w == 1 ? launch_body<4, ACT, 2, 1, 4, 1>(p, pl, s) : launch_body<4, ACT, 2, 2, 2, 1>(p, pl, s);
     }
+}
+
+template <int ACT>
+int launch_kmajor_any(const WqArgs &p, const WqKmPlan &km, hipStream_t s)
+{
+    if (km.mt == 1) return km.grouped ? launch_kmajor<1, true, ACT>(p, km, s) : launch_kmajor<1, false, ACT>(p, km, s);
+    return km.grouped ? launch_kmajor<2, true, ACT>(p, km, s) : launch_kmajor<2, false, ACT>(p, km, s);
 }
 
 } // namespace
@@ -895,7 +952,7 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
     return need;
 }
 
-extern "C" int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int w_bits, const void *scale_bf16,
+extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, const void *w, int w_bits, const void *scale_bf16,
                                          const void *offset_bf16, void *out_bf16, int64_t M, int64_t N, int64_t K,
                                          int64_t group_size, int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo,
                                          void *workspace, size_t workspace_bytes, void *stream)
@@ -903,6 +960,8 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int 
     using namespace mi355;
     if (M < 0 || N < 0 || K < 0 || group_size < 0) return MI355_ERR_BAD_ARGUMENT;
     if (w_bits != 8 && w_bits != 4) return MI355_ERR_BAD_ARGUMENT;
+    if (act_dtype != MI355_DTYPE_BF16 && act_dtype != MI355_DTYPE_FP16) return MI355_ERR_BAD_ARGUMENT;
+    const bool f16 = act_dtype == MI355_DTYPE_FP16;
     if (M == 0 || N == 0) return MI355_OK;
     if (!out_bf16 || ldo < N) return MI355_ERR_BAD_ARGUMENT;
     if (K > 0 && (!x_bf16 || !w || !scale_bf16 || ldx < K)) return MI355_ERR_BAD_ARGUMENT;
@@ -943,8 +1002,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int 
             p.strips = km.tiles;
             p.sgroups = km.tiles;
             p.S = km.S;
-            if (km.mt == 1) return km.grouped ? launch_kmajor<1, true>(p, km, s) : launch_kmajor<1, false>(p, km, s);
-            return km.grouped ? launch_kmajor<2, true>(p, km, s) : launch_kmajor<2, false>(p, km, s);
+            return f16 ? launch_kmajor_any<1>(p, km, s) : launch_kmajor_any<0>(p, km, s);
         }
     }
     const bool n_major = w_bits == 4 || (ldw_n == 1 && ldw_k >= N);
@@ -953,7 +1011,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int 
         hipLaunchKernelGGL(wq_generic_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((M + 3) / 4)), dim3(256), 0, s,
                            static_cast<const uint16_t *>(x_bf16), w, w_bits, static_cast<const uint16_t *>(scale_bf16),
                            static_cast<const uint16_t *>(offset_bf16), static_cast<uint16_t *>(out_bf16), (int)M, (int)N,
-                           (int)K, group, ldx, ldw_k, ldw_n, ldo);
+                           (int)K, group, ldx, ldw_k, ldw_n, ldo, f16 ? 1 : 0);
         return check_launch();
     }
     if (pl.S > 1) {
@@ -983,5 +1041,6 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, const void *w, int 
     p.strips = pl.strips;
     p.sgroups = pl.sgroups;
     p.S = pl.S;
-    return w_bits == 4 ? launch_bits<4>(p, pl, s) : launch_bits<8>(p, pl, s);
+    if (f16) return w_bits == 4 ? launch_bits<4, 1>(p, pl, s) : launch_bits<8, 1>(p, pl, s);
+    return w_bits == 4 ? launch_bits<4, 0>(p, pl, s) : launch_bits<8, 0>(p, pl, s);
 }

@@ -5,7 +5,7 @@
 only if it violates BOTH the absolute and the relative bound, and the comparison as a
 whole fails only if more than ``size * prec`` elements fail.
 
-``bf16_gate`` is the acceptance gate for bf16 outputs of this operator path:
+``bf16_gate`` is the acceptance gate for bf16 (and float16) outputs of this operator path:
   * at least 99.9 % of the elements lie within one bf16 unit in the last place of the
     float32 golden value, and
   * no element fails the abs-OR-rel rule at 1e-2 (relative error measured against
@@ -59,10 +59,10 @@ def bf16_gate(out_bf16: torch.Tensor, golden_f32: torch.Tensor, *, min_within_1u
 
     ``golden_f32`` is the unrounded float32 golden.  "Within one ulp" is measured on the
     bf16 number line between ``out`` and the golden rounded to bf16 (distance <= 1)."""
-    assert out_bf16.dtype == torch.bfloat16
+    assert out_bf16.dtype in (torch.bfloat16, torch.float16)     # the same gate serves float16 outputs (fp16 ulps)
     g32 = golden_f32.detach().cpu().float()
     o = out_bf16.detach().cpu()
-    dist = np.abs(_bf16_line(o) - _bf16_line(g32.to(torch.bfloat16)))
+    dist = np.abs(_bf16_line(o) - _bf16_line(g32.to(out_bf16.dtype)))
     within = float(np.count_nonzero(dist <= 1)) / max(dist.size, 1)
     exact = float(np.count_nonzero(dist == 0)) / max(dist.size, 1)
     of = o.float().numpy().astype(np.float64)

@@ -227,6 +227,38 @@ def test_w4a16_other_groups_and_edges(capi, golden):
         bf16_gate(out, _wq_golden(golden, d, gs))
 
 
+def _to_f16(d):
+    """The same seeded problem with float16 activations and parameters (values re-rounded to float16)."""
+    return {k: (v.to(torch.float16) if torch.is_tensor(v) and v.dtype == torch.bfloat16 else v) for k, v in d.items()}
+
+
+def _f16_bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("M,K,N,nk", [(16, 2048, 512, False), (16, 2048, 512, True), (1, 1024, 256, True), (40, 2048, 320, False),
+                                      (33, 1024, 384, True)])
+def test_w8a16_float16(capi, golden, M, K, N, nk):
+    """float16 activations (the dtype of the reference's own test, test/contrib/test_linear_weight_quant.py:57-62), both
+    weight layouts."""
+    d = _to_f16(workloads.w8a16_inputs(seed=M + N, M=M, K=K, N=N, weight_nk=nk))
+    out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(), d["antiquant_offset"].cuda())
+    assert out.dtype == torch.float16
+    _, gold = golden.weight_quant_matmul(_f16_bits(d["x"]), d["weight"].numpy(), _f16_bits(d["antiquant_scale"]),
+                                         _f16_bits(d["antiquant_offset"]), dtype="fp16")
+    print("w8a16 fp16", M, K, N, nk, bf16_gate(out, torch.from_numpy(gold)))
+
+
+@pytest.mark.parametrize("M", [1, 8, 32, 100])
+def test_w4a16_float16(capi, golden, M):
+    d = _to_f16(workloads.w4a16_inputs(seed=M, M=M, K=2048, N=1024, group_size=128))
+    out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(), d["antiquant_offset"].cuda(),
+                                   group_size=128)
+    _, gold = golden.weight_quant_matmul(_f16_bits(d["x"]), d["weight"].numpy(), _f16_bits(d["antiquant_scale"]),
+                                         _f16_bits(d["antiquant_offset"]), group_size=128, dtype="fp16")
+    print("w4a16 fp16", M, bf16_gate(out, torch.from_numpy(gold)))
+
+
 def test_weight_quant_exact_special_case(capi):
     # small-integer activations, unit scale, zero offset: every partial sum is exact in float32
     g = torch.Generator().manual_seed(0)
@@ -276,7 +308,8 @@ def test_c_abi_rejects_bad_arguments(capi):
     assert L.mi355_dynamic_quant(None, 0, None, None, None, -1, 8, 8, None) == -1
     assert L.mi355_dynamic_quant(None, 7, None, None, None, 1, 8, 8, None) == -1
     assert L.mi355_quant_matmul(None, None, None, None, 0, None, 0, None, 0, 4, 4, 4, 4, 4, 1, 4, None, 0, None) == -1
-    assert L.mi355_weight_quant_matmul(None, None, 5, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
+    assert L.mi355_weight_quant_matmul(None, 0, None, 5, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
+    assert L.mi355_weight_quant_matmul(None, 9, None, 8, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
     assert b"workspace" in L.mi355_status_string(-4)
     x1 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")
     x2 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")

@@ -142,8 +142,13 @@ def test_meta_weight_quant_batchmatmul(pa):
         pa.npu_weight_quant_batchmatmul(xs, w4, _m(14336, dtype=torch.bfloat16), None, antiquant_group_size=128)
     with pytest.raises(RuntimeError, match="multiple of 32"):
         pa.npu_weight_quant_batchmatmul(xs, w4, sg, og, antiquant_group_size=100)
-    with pytest.raises(RuntimeError, match="x must be bfloat16"):
+    with pytest.raises(RuntimeError, match="must have the dtype of x"):
         pa.npu_weight_quant_batchmatmul(_m(1, 4096, dtype=torch.float16), w4, sg, og, antiquant_group_size=128)
+    r = pa.npu_weight_quant_batchmatmul(_m(1, 4096, dtype=torch.float16), w4, sg.to(torch.float16), og.to(torch.float16),
+                                        antiquant_group_size=128)
+    assert r.dtype == torch.float16 and r.shape == (1, 14336)          # float16 as in test_linear_weight_quant.py:57-62
+    with pytest.raises(RuntimeError, match="x must be bfloat16 or float16"):
+        pa.npu_weight_quant_batchmatmul(_m(1, 4096, dtype=torch.float32), w4, sg, og, antiquant_group_size=128)
 
 
 def test_meta_swiglu_quant(pa):

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from pytorch_amd.testing import workloads
+from pytorch_amd.testing import workloads, rtol_failures
 
 
 def _bits(t):
@@ -131,3 +131,25 @@ def test_swiglu_vs_torch_cpu_bf16(golden):
     z = torch.tensor([[0.0, 1.0, -1.0, 2.0, 1.0, 1.0]], dtype=torch.bfloat16)
     out = golden.bf16_bits_to_f32(golden.swiglu(_bits(z)))[0]
     assert out[0] == 0.0 and abs(out[1] - 0.7311) < 4e-3 and abs(out[2] + 0.2689) < 2e-3
+
+
+def test_float16_variant_follows_the_reference_test_recipe(golden):
+    """The float16 statement of the golden against the recipe of test/contrib/test_linear_weight_quant.py:20-28 typed
+    independently in torch: that recipe rounds (w + offset) and (. * scale) to float16 before the float32 matmul, the
+    oracle keeps them in float32, and the reference accepts 1e-2 between the two."""
+    g = torch.Generator().manual_seed(4)
+    M, K, N = 24, 512, 96
+    x = torch.randn(M, K, generator=g).to(torch.float16)
+    w = torch.randn(N, K, generator=g).mul(40).to(torch.int8)                  # stored [N, K] like the module's weight
+    scale = (torch.rand(N, generator=g) * 9e-3 + 1e-3).to(torch.float16)
+    off = (torch.rand(N, generator=g) * 8 - 4).to(torch.float16)
+    wt = w.to(torch.float16).t()                                               # [K, N] view, as the test passes it
+    want = torch.matmul(x.float(), ((wt + off) * scale).float())               # the in-tree recipe, float16 intermediates
+    bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    out, outf = golden.weight_quant_matmul(bits(x), w.t().numpy(), bits(scale), bits(off), dtype="fp16")
+    got = torch.from_numpy(out.view(np.float16).astype(np.float32))
+    assert rtol_failures(got, want.to(torch.float16).float(), 1e-2) == 0
+    # and exactly the float32-intermediate evaluation, computed in float64
+    ref = x.double() @ ((wt.double() + off.double()).float() * scale.float()).double()
+    assert np.allclose(outf, ref.numpy(), rtol=2e-5, atol=1e-5)
+    assert np.array_equal(out, torch.from_numpy(outf).to(torch.float16).view(torch.int16).numpy().view(np.uint16))
