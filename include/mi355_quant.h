@@ -117,15 +117,15 @@ int mi355_quant_matmul(const int8_t *a, const int8_t *b,
  *           w_bits == 4: int32 [K, N/8] contiguous along N (ldw_k = N/8 words, ldw_n ignored);
  *                        word j of a row holds n = 8j..8j+7, element i in bits [4i, 4i+3], two's complement
  *   scale   [G, N] row-major, G = 1 when group_size == 0 else K / group_size
- *   offset  [G, N] or NULL
- *   out[m*ldo+n] = round( sum_k float(x[m,k]) * ((float(w[k,n]) + float(offset[g,n])) * float(scale[g,n])) )
+ *   offset  [G, N] or NULL;  bias [N] or NULL (the module's optional bias, linear_weight_quant.py:89-92)
+ *   out[m*ldo+n] = round( sum_k float(x[m,k]) * ((float(w[k,n]) + float(offset[g,n])) * float(scale[g,n])) + float(bias[n]) )
  *   group_size: 0 (per channel) or a multiple of 32 that divides K
  *   workspace: at least mi355_weight_quant_matmul_workspace(...) bytes
  */
 size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size);
 
 int mi355_weight_quant_matmul(const void *x, int act_dtype, const void *w, int w_bits,
-                              const void *scale, const void *offset, void *out,
+                              const void *scale, const void *offset, const void *bias, void *out,
                               int64_t M, int64_t N, int64_t K, int64_t group_size,
                               int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo,
                               void *workspace, size_t workspace_bytes, void *stream);

@@ -335,7 +335,7 @@ static void weight_quant_matmul_impl(const uint16_t *x_bf16, int64_t ldx,
                              const void *w, int w_bits, int64_t ldw_k, int64_t ldw_n,
                              const uint16_t *scale_bf16, const uint16_t *off_bf16,
                              int64_t M, int64_t N, int64_t K, int64_t group_size, int accum,
-                             uint16_t *out_bf16, float *out_f32, int f16)
+                             uint16_t *out_bf16, float *out_f32, int f16, const uint16_t *bias)
 {
     /* f16: activations, parameters and output are IEEE binary16 (the dtype of the reference's own test,
      * test/contrib/test_linear_weight_quant.py:57-62) instead of bfloat16; nothing else changes */
@@ -377,6 +377,7 @@ static void weight_quant_matmul_impl(const uint16_t *x_bf16, int64_t ldx,
                 for (int64_t k = 0; k < K; k++) s += (double)xr[k] * (double)wr[k];
                 r = (float)s;
             }
+            if (bias) r = r + ACT_TO_F32(bias[n]);   /* the module's optional bias: added to the float32 sum (results on Ascend: parity unpinned) */
             if (out_bf16) out_bf16[m * N + n] = f16 ? f32_to_f16(r) : f32_to_bf16(r);
             if (out_f32) out_f32[m * N + n] = r;
         }
@@ -393,7 +394,16 @@ void orc_weight_quant_matmul(const uint16_t *x_bf16, int64_t ldx,
                              uint16_t *out_bf16, float *out_f32)
 {
     weight_quant_matmul_impl(x_bf16, ldx, w, w_bits, ldw_k, ldw_n, scale_bf16, off_bf16, M, N, K, group_size, accum,
-                             out_bf16, out_f32, 0);
+                             out_bf16, out_f32, 0, NULL);
+}
+
+/* dtype: 0 bfloat16, 1 float16; bias: [N] of that type or NULL */
+void orc_weight_quant_matmul_bias(const uint16_t *x, int64_t ldx, const void *w, int w_bits, int64_t ldw_k, int64_t ldw_n,
+                                  const uint16_t *scale, const uint16_t *off, const uint16_t *bias, int dtype,
+                                  int64_t M, int64_t N, int64_t K, int64_t group_size, int accum,
+                                  uint16_t *out, float *out_f32)
+{
+    weight_quant_matmul_impl(x, ldx, w, w_bits, ldw_k, ldw_n, scale, off, M, N, K, group_size, accum, out, out_f32, dtype, bias);
 }
 
 void orc_weight_quant_matmul_f16(const uint16_t *x_f16, int64_t ldx,
@@ -403,7 +413,7 @@ void orc_weight_quant_matmul_f16(const uint16_t *x_f16, int64_t ldx,
                                  uint16_t *out_f16, float *out_f32)
 {
     weight_quant_matmul_impl(x_f16, ldx, w, w_bits, ldw_k, ldw_n, scale_f16, off_f16, M, N, K, group_size, accum,
-                             out_f16, out_f32, 1);
+                             out_f16, out_f32, 1, NULL);
 }
 
 /* ----------------------------------------------------------------- npu_swiglu */

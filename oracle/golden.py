@@ -48,6 +48,7 @@ def lib() -> ctypes.CDLL:
         L.orc_weight_quant_matmul.argtypes = [vp, i64, vp, i32, i64, i64, vp, vp,
                                               i64, i64, i64, i64, i32, vp, vp]
         L.orc_weight_quant_matmul_f16.argtypes = L.orc_weight_quant_matmul.argtypes
+        L.orc_weight_quant_matmul_bias.argtypes = [vp, i64, vp, i32, i64, i64, vp, vp, vp, i32, i64, i64, i64, i64, i32, vp, vp]
         L.orc_swiglu.argtypes = [vp, i64, i64, vp]
         L.orc_bf16_to_f32.argtypes = [vp, vp, i64]
         L.orc_f32_to_bf16.argtypes = [vp, vp, i64]
@@ -167,7 +168,8 @@ def antiquant(w_i8, scale_f32, offset_f32=None) -> np.ndarray:
     return out
 
 
-def weight_quant_matmul(x_u16, w, scale_u16, off_u16=None, group_size: int = 0, accum: str = "f32", dtype: str = "bf16"):
+def weight_quant_matmul(x_u16, w, scale_u16, off_u16=None, group_size: int = 0, accum: str = "f32", dtype: str = "bf16",
+                        bias_u16=None):
     """x bf16 (or, with dtype="fp16", float16) bits [M,K]; w int8 [K,N] (any strides) or int32 [K,N/8] (packed int4);
     scale/off bits of the same type [N] or [G,N].  Returns (out bits [M,N], unrounded float32 [M,N])."""
     x = _c(x_u16, np.uint16)
@@ -188,9 +190,15 @@ def weight_quant_matmul(x_u16, w, scale_u16, off_u16=None, group_size: int = 0, 
     out = np.empty((M, N), dtype=np.uint16)
     outf = np.empty((M, N), dtype=np.float32)
     if M and N:
-        fn = lib().orc_weight_quant_matmul if dtype == "bf16" else lib().orc_weight_quant_matmul_f16
-        fn(_p(x), K, _p(wbuf), bits, ldk, ldn, _p(s), _p(o), M, N, K, group_size, 0 if accum == "f32" else 1,
-           _p(out), _p(outf))
+        if bias_u16 is not None:
+            b = _c(bias_u16, np.uint16).reshape(-1)
+            assert b.size == N
+            lib().orc_weight_quant_matmul_bias(_p(x), K, _p(wbuf), bits, ldk, ldn, _p(s), _p(o), _p(b), 0 if dtype == "bf16" else 1,
+                                               M, N, K, group_size, 0 if accum == "f32" else 1, _p(out), _p(outf))
+        else:
+            fn = lib().orc_weight_quant_matmul if dtype == "bf16" else lib().orc_weight_quant_matmul_f16
+            fn(_p(x), K, _p(wbuf), bits, ldk, ldn, _p(s), _p(o), M, N, K, group_size, 0 if accum == "f32" else 1,
+               _p(out), _p(outf))
     return out, outf
 
 

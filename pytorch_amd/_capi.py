@@ -41,7 +41,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_quant_matmul.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
         L.mi355_weight_quant_matmul_workspace.restype = sz
         L.mi355_weight_quant_matmul_workspace.argtypes = [i64, i64, i64, i32, i64]
-        L.mi355_weight_quant_matmul.argtypes = [vp, i32, vp, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
+        L.mi355_weight_quant_matmul.argtypes = [vp, i32, vp, i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
                                                 vp, sz, vp]
         L.mi355_swiglu.argtypes = [vp, vp, i64, i64, i64, vp]
         L.mi355_swiglu_quant.argtypes = [vp, i32, vp, vp, i64, i64, i64, vp]
@@ -119,7 +119,7 @@ def _wq_workspace(device, nbytes: int):
     return ws
 
 
-def weight_quant_matmul(x, weight, scale, offset=None, group_size: int = 0):
+def weight_quant_matmul(x, weight, scale, offset=None, group_size: int = 0, bias=None):
     """x bf16/fp16 [M,K]; weight int8 [K,N] (strides (N,1) or (1,K)) or int32 [K,N/8]; scale/offset of x's dtype, [N] or [G,N]."""
     _need_gpu(x, weight, scale, offset)
     M, K = x.shape
@@ -133,7 +133,7 @@ def weight_quant_matmul(x, weight, scale, offset=None, group_size: int = 0):
     need = lib().mi355_weight_quant_matmul_workspace(M, N, K, bits, group_size)
     ws = _wq_workspace(x.device, need) if need else None
     st = lib().mi355_weight_quant_matmul(_ptr(x), 1 if x.dtype == torch.float16 else 0, _ptr(weight), bits, _ptr(scale),
-                                         _ptr(offset), _ptr(out),
+                                         _ptr(offset), _ptr(bias), _ptr(out),
                                          M, N, K, group_size, x.stride(0), ldk, ldn, out.stride(0), _ptr(ws),
                                          0 if ws is None else ws.numel(), _stream())
     _check(st, "mi355_weight_quant_matmul")

@@ -297,7 +297,6 @@ WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &an
                 ": weight must be int8, or int32 holding 8 int4 values per word, got ", weight.scalar_type());
     TORCH_CHECK(x.dim() >= 2 && weight.dim() == 2, op, ": x must be [..., K] with at least 2 dimensions and weight 2-D");
     TORCH_CHECK(!opt(quant_scale) && !opt(quant_offset), op, ": quant_scale / quant_offset (int8 output) are not supported");
-    TORCH_CHECK(!opt(bias), op, ": bias is not supported");
     TORCH_CHECK(inner_precise == 0, op, ": inner_precise must be 0");
     TORCH_CHECK(!weight_dtype.has_value(), op, ": weight_dtype is not supported");
     WqPlan p;
@@ -321,6 +320,11 @@ WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &an
     };
     check_param(antiquant_scale, "antiquant_scale");
     if (const Tensor *o = opt(antiquant_offset)) check_param(*o, "antiquant_offset");
+    if (const Tensor *b = opt(bias)) {
+        TORCH_CHECK(b->scalar_type() == x.scalar_type(), op, ": bias must have the dtype of x (", x.scalar_type(), "), got ",
+                    b->scalar_type());
+        TORCH_CHECK(b->numel() == p.N && b->size(-1) == p.N, op, ": bias must have shape [", p.N, "]");
+    }
     p.out_shape = x.sizes().vec();
     p.out_shape.back() = p.N;
     return p;
@@ -343,7 +347,7 @@ Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &ant
 {
     WqPlan p = weight_quant_plan(x, weight, antiquant_scale, antiquant_offset, quant_scale, quant_offset, bias, group_size,
                                  inner_precise, weight_dtype);
-    check_same_device("npu_weight_quant_batchmatmul", {&x, &weight, &antiquant_scale, opt(antiquant_offset)});
+    check_same_device("npu_weight_quant_batchmatmul", {&x, &weight, &antiquant_scale, opt(antiquant_offset), opt(bias)});
     c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
     Tensor out = at::empty(p.out_shape, x.options());
     if (out.numel() == 0) return out;
@@ -353,12 +357,15 @@ Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &ant
     // the contrib module hands 2-D parameters over as transposed views of [N, G] (linear_weight_quant.py:98-109)
     Tensor s = antiquant_scale.contiguous(), o;
     if (const Tensor *t = opt(antiquant_offset)) o = t->contiguous();
+    Tensor bias_c;
+    if (const Tensor *t = opt(bias)) bias_c = t->reshape({p.N}).contiguous();
     Tensor out2d = out.view({p.M, p.N});
     const size_t ws_bytes = mi355_weight_quant_matmul_workspace(p.M, p.N, p.K, p.bits, group_size);
     Tensor ws;
     if (ws_bytes) ws = zeroed_workspace(x, ws_bytes);
     check_status(mi355_weight_quant_matmul(x2.data_ptr(), x.scalar_type() == at::kHalf ? MI355_DTYPE_FP16 : MI355_DTYPE_BF16,
                                            w.data_ptr(), p.bits, s.data_ptr(), o.defined() ? o.data_ptr() : nullptr,
+                                           bias_c.defined() ? bias_c.data_ptr() : nullptr,
                                            out2d.data_ptr(), p.M, p.N, p.K, group_size, x2.stride(0), w.stride(0),
                                            p.bits == 4 ? 1 : w.stride(1), out2d.stride(0),
                                            ws.defined() ? ws.data_ptr() : nullptr, ws.defined() ? (size_t)ws.numel() : 0,

@@ -53,6 +53,7 @@ struct WqArgs {
     const void *w;                  // weight rows, contiguous along N
     const uint16_t *scale;          // bf16 [G, N]
     const uint16_t *offset;         // bf16 [G, N] or null
+    const uint16_t *bias;           // [N] or null: added to the float32 sum before the final rounding
     uint16_t *out;                  // bf16 [M, N]
     float *partial;                 // workspace [S][M][N] float32 (S > 1)
     uint32_t *counter;              // workspace [mchunks][sgroups], zero on entry, left zero
@@ -186,6 +187,10 @@ struct TileOut {
 
     __device__ __forceinline__ void store_out(int row, int nl, f32x4 v) const
     {
+        if (p.bias) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = v[i] + act_1<ACT>(p.bias[min(n0 + nl + i, p.N - 1)]);
+        }
         uint16_t *o = p.out + (int64_t)(m_base + row) * p.ldo + n0 + nl;
         if (out_vec) {
             u32x2 pk;
@@ -716,6 +721,7 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
 __global__ __launch_bounds__(256) void wq_generic_kernel(const uint16_t *__restrict__ x, const void *__restrict__ w,
                                                          int w_bits, const uint16_t *__restrict__ scale,
                                                          const uint16_t *__restrict__ offset,
+                                                         const uint16_t *__restrict__ bias,
                                                          uint16_t *__restrict__ out, int M, int N, int K, int group,
                                                          int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo, int act)
 {
@@ -738,6 +744,7 @@ __global__ __launch_bounds__(256) void wq_generic_kernel(const uint16_t *__restr
         wv = wv * cvt(scale[(int64_t)gidx * N + n]);
         acc = acc + cvt(x[(int64_t)m * ldx + k]) * wv;
     }
+    if (bias) acc = acc + (act ? act_1<1>(bias[n]) : act_1<0>(bias[n]));
     out[(int64_t)m * ldo + n] = (uint16_t)(act ? pack_act2<1>(acc, 0.0f) : pack_act2<0>(acc, 0.0f));
 }
 
@@ -953,7 +960,7 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
 }
 
 extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, const void *w, int w_bits, const void *scale_bf16,
-                                         const void *offset_bf16, void *out_bf16, int64_t M, int64_t N, int64_t K,
+                                         const void *offset_bf16, const void *bias, void *out_bf16, int64_t M, int64_t N, int64_t K,
                                          int64_t group_size, int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo,
                                          void *workspace, size_t workspace_bytes, void *stream)
 {
@@ -986,6 +993,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
             p.w = w;
             p.scale = static_cast<const uint16_t *>(scale_bf16);
             p.offset = static_cast<const uint16_t *>(offset_bf16);
+            p.bias = static_cast<const uint16_t *>(bias);
             p.out = static_cast<uint16_t *>(out_bf16);
             p.counter = km.S > 1 ? static_cast<uint32_t *>(workspace) : nullptr;
             p.partial = km.S > 1 ? reinterpret_cast<float *>(static_cast<char *>(workspace) + km.counter_bytes) : nullptr;
@@ -1010,7 +1018,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
     if (!pl.fast) {
         hipLaunchKernelGGL(wq_generic_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((M + 3) / 4)), dim3(256), 0, s,
                            static_cast<const uint16_t *>(x_bf16), w, w_bits, static_cast<const uint16_t *>(scale_bf16),
-                           static_cast<const uint16_t *>(offset_bf16), static_cast<uint16_t *>(out_bf16), (int)M, (int)N,
+                           static_cast<const uint16_t *>(offset_bf16), static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out_bf16), (int)M, (int)N,
                            (int)K, group, ldx, ldw_k, ldw_n, ldo, f16 ? 1 : 0);
         return check_launch();
     }
@@ -1024,6 +1032,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
     p.w = w;
     p.scale = static_cast<const uint16_t *>(scale_bf16);
     p.offset = static_cast<const uint16_t *>(offset_bf16);
+    p.bias = static_cast<const uint16_t *>(bias);
     p.out = static_cast<uint16_t *>(out_bf16);
     // counters first (they must start at zero and are left at zero), partial sums after them
     p.counter = pl.S > 1 ? static_cast<uint32_t *>(workspace) : nullptr;

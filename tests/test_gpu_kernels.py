@@ -259,6 +259,28 @@ def test_w4a16_float16(capi, golden, M):
     print("w4a16 fp16", M, bf16_gate(out, torch.from_numpy(gold)))
 
 
+@pytest.mark.parametrize("bits,nk,M", [(8, False, 16), (8, True, 5), (4, False, 1), (4, False, 40)])
+def test_weight_quant_bias(capi, golden, bits, nk, M):
+    """The module's optional bias (linear_weight_quant.py:89-92): added to the float32 sum before the final rounding, on
+    every kernel (N-major, K-major, int4, with and without a split over K)."""
+    if bits == 8:
+        d = workloads.w8a16_inputs(seed=M, M=M, K=2048, N=640, weight_nk=nk)
+        gs = 0
+    else:
+        d = workloads.w4a16_inputs(seed=M, M=M, K=2048, N=1024, group_size=128)
+        gs = 128
+    N = d["antiquant_scale"].shape[-1]
+    bias = torch.randn(N, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(), d["antiquant_offset"].cuda(),
+                                   group_size=gs, bias=bias.cuda())
+    _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
+                                         _bits(d["antiquant_offset"]), group_size=gs, bias_u16=_bits(bias))
+    bf16_gate(out, torch.from_numpy(gold))
+    nobias = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
+                                      d["antiquant_offset"].cuda(), group_size=gs)
+    assert not torch.equal(out, nobias)
+
+
 def test_weight_quant_exact_special_case(capi):
     # small-integer activations, unit scale, zero offset: every partial sum is exact in float32
     g = torch.Generator().manual_seed(0)
@@ -308,8 +330,8 @@ def test_c_abi_rejects_bad_arguments(capi):
     assert L.mi355_dynamic_quant(None, 0, None, None, None, -1, 8, 8, None) == -1
     assert L.mi355_dynamic_quant(None, 7, None, None, None, 1, 8, 8, None) == -1
     assert L.mi355_quant_matmul(None, None, None, None, 0, None, 0, None, 0, 4, 4, 4, 4, 4, 1, 4, None, 0, None) == -1
-    assert L.mi355_weight_quant_matmul(None, 0, None, 5, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
-    assert L.mi355_weight_quant_matmul(None, 9, None, 8, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
+    assert L.mi355_weight_quant_matmul(None, 0, None, 5, None, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
+    assert L.mi355_weight_quant_matmul(None, 9, None, 8, None, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
     assert b"workspace" in L.mi355_status_string(-4)
     x1 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")
     x2 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")

@@ -133,7 +133,7 @@ def test_meta_weight_quant_batchmatmul(pa):
     assert r.shape == (2, 4, 14336) and r.dtype == torch.bfloat16
     xs = _m(1, 4096, dtype=torch.bfloat16)
     for kwargs, pat in [(dict(quant_scale=_m(14336, dtype=torch.float32)), "quant_scale"),
-                        (dict(bias=_m(14336, dtype=torch.bfloat16)), "bias"),
+                        (dict(bias=_m(14336, dtype=torch.float16)), "bias must have the dtype of x"),
                         (dict(inner_precise=1), "inner_precise"),
                         (dict(weight_dtype=torch.int8), "weight_dtype")]:
         with pytest.raises(RuntimeError, match=pat):
