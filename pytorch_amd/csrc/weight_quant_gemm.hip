@@ -1,0 +1,436 @@
+// npu_weight_quant_batchmatmul for more than 32 activation rows: a tiled GEMM that decodes every weight once
+// per workgroup tile instead of streaming the weight once per 32 rows.
+//
+// A workgroup of eight wavefronts owns BM activation rows x one 128-byte strip of the weight rows (128 int8 or
+// 256 int4 columns) and walks its K range in stages of 64 rows:
+//   * weights: wavefront w copies rows 8w .. 8w+7 of the stage global -> LDS with one 1 KiB load instruction, three
+//     stages ahead (vector-memory instructions cost the CU ~16 clocks each however few bytes they move, so the raw
+//     bytes travel 16 per lane); it then reads its two bytes of each of the eight rows back, expands them to the
+//     exact 16-bit images of the integers (the same images as the streaming kernel) and writes them to LDS as
+//     [column][8 k] 16-byte chunks;
+//   * activations: copied global -> LDS without passing registers, one stage ahead;
+//   * both LDS tiles have a 128-byte row pitch (64 k x 2 bytes) with the 16-byte chunks XOR-swizzled by the row
+//     pair, so the fragment reads of the 16x16x32 MFMA are conflict free; two slots, one barrier per stage.
+// The antiquant parameters are applied to the float32 sums per scale group exactly as in the streaming kernel:
+//     out[m,n] = sum_g scale[g,n] * ( P_g[m,n] + offset[g,n] * X_g[m] ),   X_g from an MFMA against ones.
+// The weight fragment is the first MFMA operand, so a lane owns four consecutive output columns of one row.
+// K may be split over S workgroups per tile: each publishes its float32 sums in register order and the last
+// arrival adds all of them in chunk order (the result does not depend on the order of arrival).
+#include "weight_quant_common.h"
+#include "weight_quant_gemm.h"
+
+namespace mi355 {
+namespace {
+
+struct WqGemmArgs {
+    const uint16_t *x;
+    const void *w;
+    const uint16_t *scale, *offset, *bias;
+    uint16_t *out;
+    float *partial;                 // workspace [tile][chunk][wavefront][accumulator quad][lane] float32x4 (S > 1)
+    uint32_t *counter;              // workspace [tile], zero on entry, left zero (S > 1)
+    int64_t ldx, ldo;
+    uint32_t ldw_bytes, row_bytes;
+    int M, N, K;
+    int unit_stages, n_units, grouped;
+    int tiles_m, tiles_n, tiles_per_xcd, S;
+};
+
+template <int WBITS, int ACT, int BM, bool ACCUM>
+__global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
+{
+    constexpr int NW = 8;
+    constexpr int BN = WBITS == 4 ? 256 : 128;
+    constexpr int WGM = BM / 64, WGN = NW / WGM;
+    constexpr int WTM = 4, WTN = BN / (16 * WGN);
+    constexpr int PITCH = 128;                                 // bytes per LDS tile row: 64 k of 16 bits
+    constexpr int A_BYTES = BM * PITCH, B_BYTES = BN * PITCH;
+    constexpr int A_RING = 3 * A_BYTES;                        // LDS: three activation slots, two image slots, raw weight ring
+    constexpr int LA = BM / 8 / NW;                            // activation loads of a wavefront per stage
+    constexpr int CPL = WBITS == 4 ? 4 : 2;                    // weight columns per lane of the loader
+    constexpr float P_MUL = kImageMul<WBITS, ACT>;
+    constexpr float X_BIAS = kImageBias<WBITS>;
+    static_assert(BM == 64 || BM == 128, "tile rows");
+    static_assert(WTN >= 1, "tile columns");
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+    // workgroup -> (tile, K chunk): every XCD gets a contiguous run of tiles, rows fastest, so the row tiles
+    // of one weight strip share an L2
+    const int xcd = blockIdx.x & 7;
+    const int slot_id = blockIdx.x >> 3;
+    const int tile = xcd * p.tiles_per_xcd + slot_id % p.tiles_per_xcd;
+    const int chunk = slot_id / p.tiles_per_xcd;
+    if (tile >= p.tiles_m * p.tiles_n) return;
+    const int m0 = (tile % p.tiles_m) * BM;
+    const int tn = tile / p.tiles_m;
+    const int n0 = tn * BN;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int u0 = (int)((int64_t)p.n_units * chunk / p.S), u1 = (int)((int64_t)p.n_units * (chunk + 1) / p.S);
+    const int s0 = u0 * p.unit_stages;                         // first stage of this workgroup
+    const int NSTG = (u1 - u0) * p.unit_stages;                // its number of stages (even)
+
+    // ---- activations: global -> LDS.  Lane l of a unit (8 rows x 128 B) fills LDS slot l: row l/8, chunk slot
+    // l%8, which must hold global chunk (l%8) ^ ((row >> 1) & 7).  unit = i * 8 + wave, so (row >> 1) & 7 =
+    // 4 * (wave & 1) + (l/8) / 2.
+    const int rows_a = min(BM, p.M - m0);
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        make_rsrc(p.x + (int64_t)m0 * p.ldx, (uint32_t)(((int64_t)(rows_a - 1) * p.ldx + p.K) * 2));
+    const int rr = lane >> 3;
+    const uint32_t voff_a = (uint32_t)(rr * (int)p.ldx * 2 + (((lane & 7) ^ (((wave & 1) << 2) | (rr >> 1))) * 16));
+    const uint32_t unit_stride_a = 16u * (uint32_t)p.ldx;
+    auto issue_a = [&](int s) {
+        char *slot = lds + (s % 3) * A_BYTES;
+        const uint32_t vo = s < NSTG ? voff_a : kOutOfRange;
+#pragma unroll
+        for (int i = 0; i < LA; i++) {
+            const int u = i * NW + wave;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void *)(slot + u * 1024), 16, vo,
+                                                     (uint32_t)u * unit_stride_a + (uint32_t)(s0 + s) * PITCH, 0, 0);
+        }
+    };
+
+    // ---- weights: global -> LDS raw ring (three slots of 64 rows x 128 B), one octet of rows per wavefront and load
+    constexpr int RAW_BYTES = 64 * 128;
+    char *const raw = lds + A_RING + 2 * B_BYTES;
+    const uint32_t strip_valid = min(128u, p.row_bytes - (uint32_t)tn * 128u);
+    const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(static_cast<const char *>(p.w) + (size_t)tn * 128,
+                                                    (uint32_t)(p.K - 1) * p.ldw_bytes + strip_valid);
+    const uint32_t voff_w = (uint32_t)(lane & 7) * 16u < strip_valid
+                                ? (uint32_t)(lane >> 3) * p.ldw_bytes + (uint32_t)(lane & 7) * 16u
+                                : kOutOfRange;
+    auto issue_w = [&](int s) {
+        const uint32_t vo = s < NSTG ? voff_w : kOutOfRange;
+        const uint32_t row = (uint32_t)(s0 + s) * 64u + (uint32_t)wave * 8u;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void *)(raw + (s % 3) * RAW_BYTES + wave * 1024), 16, vo,
+                                                 row * p.ldw_bytes, 0, 0);
+    };
+    // this lane's two bytes (2 int8 / 4 int4 columns) of the wavefront's eight rows
+    auto read_raw = [&](uint32_t (&wr)[8], int s) {
+        const char *src = raw + (s % 3) * RAW_BYTES + wave * 1024 + lane * 2;
+#pragma unroll
+        for (int t = 0; t < 8; t++) wr[t] = *reinterpret_cast<const uint16_t *>(src + t * 128);
+    };
+    // registers -> LDS: column n of the tile, k rows 8 * wave .. 8 * wave + 7 of the stage -> chunk slot wave ^ ((n >> 1) & 7)
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "n"(kInt4Magic<ACT>));   // opaque to the optimiser: stays in a VGPR
+    // two's complement -> offset binary (w + 128 / nibble + 8), then the 16-bit images -> LDS
+    auto flip_w = [&](uint32_t (&wx)[8], const uint32_t (&wr)[8]) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) wx[t] = wr[t] ^ (WBITS == 4 ? 0x8888u : 0x8080u);
+    };
+    auto expand_w = [&](const uint32_t (&wx)[8], int s) {
+        char *bs = lds + A_RING + (s & 1) * B_BYTES;
+#pragma unroll
+        for (int jb = 0; jb < CPL / 2; jb++) {
+            u32x4 b0, b1;
+            expand_pair<WBITS, ACT>(wx, jb, magic, b0, b1);
+            const int n = lane * CPL + 2 * jb;                 // even: n and n + 1 share the swizzle
+            const int sw = (wave ^ ((n >> 1) & 7)) * 16;
+            *reinterpret_cast<u32x4 *>(bs + n * PITCH + sw) = b0;
+            *reinterpret_cast<u32x4 *>(bs + (n + 1) * PITCH + sw) = b1;
+        }
+    };
+
+    // ---- antiquant parameters of this lane's columns: tile j covers n0 + (wn * WTN + j) * 16 + 4 * (lane / 16) + r
+    const int ncol0 = n0 + wn * WTN * 16 + (lane >> 4) * 4;
+    const uint32_t param_bytes = (uint32_t)(p.grouped ? p.K / (64 * p.unit_stages) : 1) * (uint32_t)p.N * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc_s = make_rsrc(p.scale, param_bytes);
+    const bool has_offset = p.offset != nullptr;
+    const __amdgpu_buffer_rsrc_t rsrc_o = make_rsrc(has_offset ? p.offset : p.scale, param_bytes);
+    const uint32_t omask = has_offset ? ~0u : 0u;
+    const uint32_t voff_p = (uint32_t)ncol0 * 2u;
+    u32x2 sv[WTN], ov[WTN];
+    auto load_params = [&](int group_row, bool wanted) {
+        const uint32_t vo = wanted ? voff_p : kOutOfRange;
+        const uint32_t ro = (uint32_t)group_row * (uint32_t)p.N * 2u;
+#pragma unroll
+        for (int j = 0; j < WTN; j++) {
+            sv[j] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, vo + 32u * j, ro, 0);
+            ov[j] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_o, vo + 32u * j, ro, 0);   // masked where it is used
+        }
+    };
+
+    f32x4 P[WTM][WTN], tot[WTM][WTN], X[WTM];
+#pragma unroll
+    for (int i = 0; i < WTM; i++) {
+        X[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < WTN; j++) {
+            P[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+            tot[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    // tot += (scale * P_MUL) * (P' + ((offset - X_BIAS) / P_MUL) * X); both rescalings are exact (powers of two)
+    auto fold = [&]() {
+#pragma unroll
+        for (int j = 0; j < WTN; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t su = sv[j][r >> 1], ou = ov[j][r >> 1] & omask;
+                const float sc = ((r & 1) ? act_hi<ACT>(su) : act_lo<ACT>(su)) * P_MUL;
+                const float of = (((r & 1) ? act_hi<ACT>(ou) : act_lo<ACT>(ou)) - X_BIAS) * (1.0f / P_MUL);
+#pragma unroll
+                for (int i = 0; i < WTM; i++) {
+                    const float inner = __builtin_fmaf(of, X[i][0], P[i][j][r]);
+                    tot[i][j][r] = __builtin_fmaf(sc, inner, tot[i][j][r]);
+                }
+            }
+#pragma unroll
+        for (int i = 0; i < WTM; i++) {
+            X[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < WTN; j++) P[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+
+    // ---- fragment reads: lane reads row (lane % 16) of a 16-row tile, chunk (ks * 4 + lane / 16), stored at slot
+    // chunk ^ ((row >> 1) & 7); for ks = 1 the slot is the ks = 0 slot with bit 2 flipped
+    const int frow = lane & 15;
+    const int sw0 = ((lane >> 4) ^ ((frow >> 1) & 7)) * 16;
+    const int a_off = (wm * 64 + frow) * PITCH;
+    const int b_off = A_RING + (wn * WTN * 16 + frow) * PITCH;
+    const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
+    // Small wavefront tiles issue all fragment reads of the stage up front (the reads of the second half overlap the
+    // MFMAs of the first); the 64 x 64 tile has no registers to spare for that.
+    constexpr int AHEAD = WTM * WTN <= 8 ? 2 : 1;
+    auto compute = [&](int s) {
+        const char *sa = lds + (s % 3) * A_BYTES + a_off, *sb = lds + (s & 1) * B_BYTES + b_off;
+#pragma unroll
+        for (int k0 = 0; k0 < 2; k0 += AHEAD) {
+            u32x4 AF[AHEAD][WTM], BF[AHEAD][WTN];
+#pragma unroll
+            for (int ks = 0; ks < AHEAD; ks++) {
+                const int sw = sw0 ^ ((k0 + ks) * 64);
+#pragma unroll
+                for (int i = 0; i < WTM; i++) AF[ks][i] = *reinterpret_cast<const u32x4 *>(sa + i * 16 * PITCH + sw);
+#pragma unroll
+                for (int j = 0; j < WTN; j++) BF[ks][j] = *reinterpret_cast<const u32x4 *>(sb + j * 16 * PITCH + sw);
+            }
+#pragma unroll
+            for (int ks = 0; ks < AHEAD; ks++) {
+#pragma unroll
+                for (int j = 0; j < WTN; j++)
+#pragma unroll
+                    for (int i = 0; i < WTM; i++) P[i][j] = mfma_act<ACT>(BF[ks][j], AF[ks][i], P[i][j]);
+#pragma unroll
+                for (int i = 0; i < WTM; i++) X[i] = mfma_act<ACT>(ones, AF[ks][i], X[i]);
+            }
+        }
+    };
+
+    // ---- main loop.  Stage s is computed from activation slot s % 3 and image slot s & 1.  Meanwhile image slot
+    // (s + 1) & 1 receives the images of stage s + 1, expanded from the raw ring, and memory is asked for the
+    // activations of stage s + 2 and the raw weights of stage s + 3.  Loads are never skipped (a stage past the end
+    // gets an out-of-range lane offset and moves no bytes), so the number of loads in flight is the same in every
+    // iteration: at the top, "at most LA + 1 outstanding" means everything but the newest refills has landed.
+    uint32_t wr[8], wx[8];
+    issue_w(0);
+    issue_a(0);
+    issue_w(1);
+    issue_a(1);
+    issue_w(2);
+    wait_vmcnt<2 * LA + 2>();
+    __syncthreads();
+    read_raw(wr, 0);
+    flip_w(wx, wr);
+    expand_w(wx, 0);
+    auto body = [&](int s) {
+        wait_vmcnt<LA + 1>();
+        wait_lgkmcnt0();
+        __syncthreads();                                       // stage s is complete in LDS; everyone is done with stage s - 1
+        const bool fold_stage = ACCUM && (s0 + s + 1) % p.unit_stages == 0;   // the last stage of a scale group
+        if (fold_stage) load_params((s0 + s) / p.unit_stages, true);            // first: the fold must not wait for the refills
+        issue_a(s + 2);
+        issue_w(s + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        // the two wavefronts of a SIMD (w and w + 4) expand and compute in opposite order, so that the VALU work
+        // of one overlaps the MFMA work of the other
+        if (wave < 4) {
+            read_raw(wr, s + 1);
+            flip_w(wx, wr);
+            expand_w(wx, s + 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        compute(s);
+        __builtin_amdgcn_sched_barrier(0);
+        if (wave >= 4) {
+            read_raw(wr, s + 1);
+            flip_w(wx, wr);
+            expand_w(wx, s + 1);
+        }
+        if (fold_stage) fold();
+    };
+    for (int s = 0; s < NSTG; s++) body(s);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the refills past the end (zeros) have landed
+    __syncthreads();
+    if constexpr (!ACCUM) {
+        load_params(p.grouped ? u0 : 0, true);
+        fold();
+    }
+
+    // ---- split K: publish, count, last arrival sums in chunk order
+    if (p.S > 1) {
+        constexpr int SC1 = 16;                                // cache-policy bit: agent scope
+        constexpr uint32_t WAVE_BYTES = WTM * WTN * 64 * 16;
+        constexpr uint32_t CHUNK_BYTES = NW * WAVE_BYTES;
+        const __amdgpu_buffer_rsrc_t rsrc_p =
+            make_rsrc(p.partial + (size_t)tile * p.S * (CHUNK_BYTES / 4), (uint32_t)p.S * CHUNK_BYTES);
+        const uint32_t lane_off = (uint32_t)wave * WAVE_BYTES + (uint32_t)lane * 16u;
+#pragma unroll
+        for (int i = 0; i < WTM; i++)
+#pragma unroll
+            for (int j = 0; j < WTN; j++)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, tot[i][j]), rsrc_p,
+                                                       lane_off + (i * WTN + j) * 1024, (uint32_t)chunk * CHUNK_BYTES, SC1);
+        wait_vmcnt<0>();                                       // this wavefront's sums have reached the coherence point
+        __syncthreads();
+        int &is_last = *reinterpret_cast<int *>(lds);
+        if (threadIdx.x == 0) {
+            const uint32_t old = __hip_atomic_fetch_add(p.counter + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = old == (uint32_t)(p.S - 1);
+        }
+        __syncthreads();
+        if (!is_last) return;
+#pragma unroll
+        for (int i = 0; i < WTM; i++)
+#pragma unroll
+            for (int j = 0; j < WTN; j++) tot[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int ch = 0; ch < p.S; ch++) {
+#pragma unroll
+            for (int i = 0; i < WTM; i++)
+#pragma unroll
+                for (int j = 0; j < WTN; j++)
+                    tot[i][j] += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                        rsrc_p, lane_off + (i * WTN + j) * 1024, (uint32_t)ch * CHUNK_BYTES, SC1));
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(p.counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // ---- output: lane holds row m = ... + lane % 16, columns ncol0 + 16 j + r
+    const bool out_vec = (p.ldo & 3) == 0 && aligned_dev(p.out, 8);
+#pragma unroll
+    for (int j = 0; j < WTN; j++) {
+        const int n = ncol0 + j * 16;
+        if (n >= p.N) continue;                                // N is a multiple of 8: a quad is valid as a whole
+        f32x4 bv = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (p.bias) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) bv[r] = act_1<ACT>(p.bias[n + r]);
+        }
+#pragma unroll
+        for (int i = 0; i < WTM; i++) {
+            const int m = m0 + wm * 64 + i * 16 + frow;
+            if (m >= p.M) continue;
+            const f32x4 v = tot[i][j] + bv;
+            uint16_t *o = p.out + (int64_t)m * p.ldo + n;
+            if (out_vec) {
+                u32x2 pk;
+                pk.x = pack_act2<ACT>(v[0], v[1]);
+                pk.y = pack_act2<ACT>(v[2], v[3]);
+                *reinterpret_cast<u32x2 *>(o) = pk;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[r] = (uint16_t)pack_act2<ACT>(v[r], 0.0f);
+            }
+        }
+    }
+}
+
+template <int WBITS, int ACT, int BM, bool ACCUM>
+int launch_tile(WqGemmArgs &p, hipStream_t s)
+{
+    constexpr int BN = WBITS == 4 ? 256 : 128;
+    constexpr size_t lds_bytes = (size_t)(3 * BM + 2 * BN) * 128 + 3 * 64 * 128;   // activation ring, image slots, raw ring
+    static_assert(lds_bytes <= 160 * 1024, "LDS budget");
+    auto kern = wq_gemm_kernel<WBITS, ACT, BM, ACCUM>;
+    static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(8 * p.tiles_per_xcd * p.S)), dim3(512), lds_bytes, s, p);
+    return check_launch();
+}
+
+template <int WBITS, int ACT>
+int launch_any(WqGemmArgs &p, const WqGemmPlan &pl, hipStream_t s)
+{
+    if (pl.bm == 64)
+        return pl.accum ? launch_tile<WBITS, ACT, 64, true>(p, s) : launch_tile<WBITS, ACT, 64, false>(p, s);
+    return pl.accum ? launch_tile<WBITS, ACT, 128, true>(p, s) : launch_tile<WBITS, ACT, 128, false>(p, s);
+}
+
+} // namespace
+
+WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size, bool n_major, int64_t ldw_k,
+                             int64_t ldx, const void *x, const void *w, const void *scale, const void *offset)
+{
+    WqGemmPlan pl{};
+    const int64_t row_bytes = w_bits == 4 ? N / 2 : N;
+    const int64_t ldw_bytes = w_bits == 4 ? ldw_k * 4 : ldw_k;
+    const int64_t group = group_size > 0 ? group_size : K;
+    pl.grouped = group_size > 0 && group != K;
+    const char *off_env = getenv("MI355_WQ_GEMM");             // tuning aid: "0" keeps every shape on the streaming kernels
+    pl.ok = M > 32 && n_major && K >= 128 && K % 128 == 0 && group % 128 == 0 && N % 8 == 0 && ldw_bytes % 4 == 0 &&
+            ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 4)) &&
+            (scale == nullptr || aligned(scale, 4)) && (offset == nullptr || aligned(offset, 4)) &&
+            (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 32) && (uint64_t)128 * (uint64_t)ldx * 2 < (1ull << 31) &&
+            (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && !(off_env && off_env[0] == '0');
+    if (!pl.ok) return pl;
+    const int bn = w_bits == 4 ? 256 : 128;
+    pl.bm = M <= 64 ? 64 : 128;
+    if (const int f = env_int("MI355_WQG_BM"))                 // tuning aid
+        if (f == 64 || f == 128) pl.bm = f;
+    pl.tiles_m = (int)((M + pl.bm - 1) / pl.bm);
+    pl.tiles_n = (int)((row_bytes + 127) / 128);
+    pl.unit_stages = pl.grouped ? (int)(group / 64) : 2;
+    pl.n_units = (int)(K / (64 * pl.unit_stages));
+    const int64_t tiles = (int64_t)pl.tiles_m * pl.tiles_n;
+    int64_t S = tiles < kNumCU ? kNumCU / tiles : 1;
+    if (S > pl.n_units) S = pl.n_units;
+    if (S > 8) S = 8;
+    if (const int f = env_int("MI355_WQG_SPLIT"))              // tuning aid
+        if (f >= 1 && f <= pl.n_units) S = f;
+    if (S > 1 && ((uint64_t)S * pl.bm * bn * 4 >= (1ull << 32) || (size_t)tiles * 4 > kWorkspaceCounterBytes)) S = 1;
+    pl.S = (int)S;
+    pl.accum = pl.grouped && (pl.n_units + pl.S - 1) / pl.S > 1;
+    pl.partial_bytes = pl.S > 1 ? (size_t)tiles * pl.S * pl.bm * bn * 4 : 0;
+    pl.counter_bytes = pl.S > 1 ? kWorkspaceCounterBytes : 0;
+    (void)bn;
+    return pl;
+}
+
+int launch_wq_gemm(const WqGemmPlan &pl, const void *x, int act_f16, const void *w, int w_bits, const void *scale,
+                   const void *offset, const void *bias, void *out, int64_t M, int64_t N, int64_t K, int64_t ldx,
+                   int64_t ldw_k, int64_t ldo, void *workspace, void *stream)
+{
+    WqGemmArgs p{};
+    p.x = static_cast<const uint16_t *>(x);
+    p.w = w;
+    p.scale = static_cast<const uint16_t *>(scale);
+    p.offset = static_cast<const uint16_t *>(offset);
+    p.bias = static_cast<const uint16_t *>(bias);
+    p.out = static_cast<uint16_t *>(out);
+    p.counter = pl.S > 1 ? static_cast<uint32_t *>(workspace) : nullptr;
+    p.partial = pl.S > 1 ? reinterpret_cast<float *>(static_cast<char *>(workspace) + pl.counter_bytes) : nullptr;
+    p.ldx = ldx;
+    p.ldo = ldo;
+    p.ldw_bytes = (uint32_t)(w_bits == 4 ? ldw_k * 4 : ldw_k);
+    p.row_bytes = (uint32_t)(w_bits == 4 ? N / 2 : N);
+    p.M = (int)M;
+    p.N = (int)N;
+    p.K = (int)K;
+    p.unit_stages = pl.unit_stages;
+    p.n_units = pl.n_units;
+    p.grouped = pl.grouped;
+    p.tiles_m = pl.tiles_m;
+    p.tiles_n = pl.tiles_n;
+    p.tiles_per_xcd = (pl.tiles_m * pl.tiles_n + 7) / 8;
+    p.S = pl.S;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (act_f16) return w_bits == 4 ? launch_any<4, 1>(p, pl, s) : launch_any<8, 1>(p, pl, s);
+    return w_bits == 4 ? launch_any<4, 0>(p, pl, s) : launch_any<8, 0>(p, pl, s);
+}
+
+} // namespace mi355

@@ -281,6 +281,60 @@ def test_weight_quant_bias(capi, golden, bits, nk, M):
     assert not torch.equal(out, nobias)
 
 
+TILED_CASES = [  # bits, M, K, N, group, float16, bias
+    (8, 33, 1024, 384, 0, False, False),      # 64-row tile, ragged rows
+    (8, 128, 2048, 1000, 0, False, True),     # 128-row tile, last strip partly valid
+    (8, 200, 1024, 256, 0, False, False),     # two row tiles, the second ragged
+    (8, 64, 8192, 256, 0, True, False),       # few tiles: K split eight ways, per channel
+    (8, 96, 1024, 512, 256, False, False),    # int8 with scale groups
+    (4, 128, 4096, 1024, 128, False, False),  # several groups per workgroup and a K split
+    (4, 40, 2048, 264, 128, False, True),     # second strip holds 8 columns
+    (4, 100, 1024, 512, 256, True, False),
+    (4, 130, 512, 2048, 512, False, False),   # one group = per channel
+    (4, 320, 1024, 768, 128, False, False),   # three row tiles
+]
+
+
+@pytest.mark.parametrize("bits,M,K,N,gs,f16,with_bias", TILED_CASES)
+def test_weight_quant_tiled_kernel(capi, golden, bits, M, K, N, gs, f16, with_bias):
+    """More than 32 activation rows take the tiled kernel (weights decoded once per 64/128 rows): every tile shape,
+    ragged rows and strips, grouped and per-channel parameters, both activation dtypes, with and without a K split."""
+    if bits == 8:
+        d = workloads.w8a16_inputs(seed=M + N, M=M, K=K, N=N)
+        if gs:
+            g = torch.Generator().manual_seed(5)
+            d["antiquant_scale"] = (torch.rand(K // gs, N, generator=g) * 9e-3 + 1e-3).to(torch.bfloat16)
+            d["antiquant_offset"] = (torch.rand(K // gs, N, generator=g) * 8 - 4).to(torch.bfloat16)
+    else:
+        d = workloads.w4a16_inputs(seed=M + N, M=M, K=K, N=N, group_size=gs)
+    bits_of = _bits
+    if f16:
+        d = _to_f16(d)
+        bits_of = _f16_bits
+    bias = None
+    if with_bias:
+        bias = torch.randn(N, generator=torch.Generator().manual_seed(1)).to(d["x"].dtype)
+    group = gs
+    args = [d[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset")]
+    out = capi.weight_quant_matmul(*args, group_size=group, bias=None if bias is None else bias.cuda())
+    _, gold = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(d["antiquant_scale"]),
+                                         bits_of(d["antiquant_offset"]), group_size=group, dtype="fp16" if f16 else "bf16",
+                                         bias_u16=None if bias is None else bits_of(bias))
+    print("tiled", bits, M, K, N, gs, bf16_gate(out, torch.from_numpy(gold)))
+    # the split over K must not change a bit of the result, whatever the number of chunks, and repeated launches
+    # (which reuse the workspace and its arrival counters) must repeat the result
+    import os
+    for split in ("1", "2"):
+        os.environ["MI355_WQG_SPLIT"] = split
+        try:
+            again = capi.weight_quant_matmul(*args, group_size=group, bias=None if bias is None else bias.cuda())
+        finally:
+            del os.environ["MI355_WQG_SPLIT"]
+        bf16_gate(again, torch.from_numpy(gold))
+    for _ in range(5):
+        assert torch.equal(capi.weight_quant_matmul(*args, group_size=group, bias=None if bias is None else bias.cuda()), out)
+
+
 def test_weight_quant_exact_special_case(capi):
     # small-integer activations, unit scale, zero offset: every partial sum is exact in float32
     g = torch.Generator().manual_seed(0)
