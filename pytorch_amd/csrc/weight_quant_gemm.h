@@ -13,7 +13,7 @@ struct WqGemmPlan {
     int unit_stages;         // 64-row stages per unit of K: a scale group, or two stages per channel
     int n_units;
     bool grouped, accum;     // accum: a workgroup meets more than one scale group
-    size_t partial_bytes, counter_bytes;
+    size_t counter_bytes, partial_bytes, rowsum_bytes;   // workspace: [arrival counters | partial sums | row sums]
 };
 
 __attribute__((visibility("hidden"))) WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits,
@@ -21,7 +21,7 @@ __attribute__((visibility("hidden"))) WqGemmPlan make_wq_gemm_plan(int64_t M, in
                                                                    int64_t ldx, const void *x, const void *w,
                                                                    const void *scale, const void *offset);
 
-// Launches the tiled kernel; `workspace` holds [arrival counters | partial sums] when plan.S > 1.
+// Launches the row-sum kernel and the tiled kernel; `workspace` holds counter_bytes + partial_bytes + rowsum_bytes.
 __attribute__((visibility("hidden"))) int launch_wq_gemm(const WqGemmPlan &plan, const void *x, int act_f16, const void *w,
                                                          int w_bits, const void *scale, const void *offset, const void *bias,
                                                          void *out, int64_t M, int64_t N, int64_t K, int64_t ldx,

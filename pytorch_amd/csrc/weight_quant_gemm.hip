@@ -8,11 +8,15 @@
 //     bytes travel 16 per lane); it then reads its two bytes of each of the eight rows back, expands them to the
 //     exact 16-bit images of the integers (the same images as the streaming kernel) and writes them to LDS as
 //     [column][8 k] 16-byte chunks;
-//   * activations: copied global -> LDS without passing registers, one stage ahead;
+//   * activations: copied global -> LDS without passing registers, two stages ahead (three slots);
 //   * both LDS tiles have a 128-byte row pitch (64 k x 2 bytes) with the 16-byte chunks XOR-swizzled by the row
-//     pair, so the fragment reads of the 16x16x32 MFMA are conflict free; two slots, one barrier per stage.
+//     pair, so the fragment reads of the 16x16x32 MFMA are conflict free; two image slots, one barrier per stage;
+//   * the VALU work (folding a finished scale group into the running total, expanding the next stage's weights)
+//     is placed between the MFMAs of a stage, so that it runs in their shadow.
 // The antiquant parameters are applied to the float32 sums per scale group exactly as in the streaming kernel:
-//     out[m,n] = sum_g scale[g,n] * ( P_g[m,n] + offset[g,n] * X_g[m] ),   X_g from an MFMA against ones.
+//     out[m,n] = sum_g scale[g,n] * ( P_g[m,n] + offset[g,n] * X_g[m] ),
+// where the row sums X_g[m] of the activations come from a small kernel that runs first (they are shared by all
+// columns; computing them per tile would cost a fifth to a third more MFMAs and sixteen accumulator registers).
 // The weight fragment is the first MFMA operand, so a lane owns four consecutive output columns of one row.
 // K may be split over S workgroups per tile: each publishes its float32 sums in register order and the last
 // arrival adds all of them in chunk order (the result does not depend on the order of arrival).
@@ -27,6 +31,7 @@ struct WqGemmArgs {
     const void *w;
     const uint16_t *scale, *offset, *bias;
     uint16_t *out;
+    float *rowsum;                  // workspace [unit][M] float32: sums of the activations over a unit of K
     float *partial;                 // workspace [tile][chunk][wavefront][accumulator quad][lane] float32x4 (S > 1)
     uint32_t *counter;              // workspace [tile], zero on entry, left zero (S > 1)
     int64_t ldx, ldo;
@@ -35,6 +40,24 @@ struct WqGemmArgs {
     int unit_stages, n_units, grouped;
     int tiles_m, tiles_n, tiles_per_xcd, S;
 };
+
+// rowsum[u][m] = sum of x[m, u * unit_k .. (u + 1) * unit_k): one thread per sum, 16-byte loads.
+template <int ACT>
+__global__ __launch_bounds__(256) void wq_rowsum_kernel(const uint16_t *__restrict__ x, float *__restrict__ rowsum, int M,
+                                                        int n_units, int unit_k, int64_t ldx)
+{
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= M * n_units) return;
+    const int m = idx / n_units, u = idx % n_units;         // neighbouring threads read neighbouring units of one row
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + (int64_t)m * ldx + (int64_t)u * unit_k);
+    float acc = 0.0f;
+    for (int c = 0; c < unit_k / 8; c++) {
+        const u32x4 v = src[c];
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc += act_lo<ACT>(v[e]) + act_hi<ACT>(v[e]);
+    }
+    rowsum[(int64_t)u * M + m] = acc;
+}
 
 template <int WBITS, int ACT, int BM, bool ACCUM>
 __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
@@ -142,47 +165,65 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
     const __amdgpu_buffer_rsrc_t rsrc_o = make_rsrc(has_offset ? p.offset : p.scale, param_bytes);
     const uint32_t omask = has_offset ? ~0u : 0u;
     const uint32_t voff_p = (uint32_t)ncol0 * 2u;
+    // Inside the loop the parameters of a finished group travel through LDS: wavefront 0 copies the tile's BN scales and
+    // offsets global -> LDS (a few load instructions for the whole workgroup instead of 2 * WTN per wavefront, and no
+    // registers held across the stage); two slots, by group parity.  After the loop they are loaded into registers.
+    constexpr int PRM_SLOT = 2048;                             // [BN scales | +512: BN offsets], 16-bit each, [+1024: BM row sums] float32
+    char *const prm = lds + A_RING + 2 * B_BYTES + 3 * RAW_BYTES;
+    const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(p.rowsum, (uint32_t)p.n_units * (uint32_t)p.M * 4u);
+    auto issue_params = [&](int group_row) {
+        const uint32_t ro = (uint32_t)group_row * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
+        char *dst = prm + (group_row & 1) * PRM_SLOT;
+#pragma unroll
+        for (int h = 0; h < BM / 64; h++)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_void *)(dst + 1024 + h * 256), 4, (uint32_t)lane * 4u,
+                                                     ((uint32_t)group_row * (uint32_t)p.M + (uint32_t)m0) * 4u + h * 256u, 0, 0);
+#pragma unroll
+        for (int h = 0; h < BN / 128; h++) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_s, (lds_void *)(dst + h * 256), 4, (uint32_t)lane * 4u, ro + h * 256u, 0, 0);
+            if (has_offset)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_o, (lds_void *)(dst + 512 + h * 256), 4, (uint32_t)lane * 4u,
+                                                         ro + h * 256u, 0, 0);
+        }
+    };
+    const int prm_col = (wn * WTN * 16 + (lane >> 4) * 4) * 2;  // byte offset of this lane's first column in a slot
     u32x2 sv[WTN], ov[WTN];
-    auto load_params = [&](int group_row, bool wanted) {
-        const uint32_t vo = wanted ? voff_p : kOutOfRange;
+    auto load_params = [&](int group_row) {
         const uint32_t ro = (uint32_t)group_row * (uint32_t)p.N * 2u;
 #pragma unroll
         for (int j = 0; j < WTN; j++) {
-            sv[j] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, vo + 32u * j, ro, 0);
-            ov[j] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_o, vo + 32u * j, ro, 0);   // masked where it is used
+            sv[j] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, voff_p + 32u * j, ro, 0);
+            ov[j] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_o, voff_p + 32u * j, ro, 0);   // masked where it is used
         }
     };
 
-    f32x4 P[WTM][WTN], tot[WTM][WTN], X[WTM];
+    f32x4 P[WTM][WTN], tot[WTM][WTN];
+    float X[WTM];                                              // row sums of the group being folded
 #pragma unroll
     for (int i = 0; i < WTM; i++) {
-        X[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        X[i] = 0.0f;
 #pragma unroll
         for (int j = 0; j < WTN; j++) {
             P[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
             tot[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
     }
-    // tot += (scale * P_MUL) * (P' + ((offset - X_BIAS) / P_MUL) * X); both rescalings are exact (powers of two)
-    auto fold = [&]() {
+    // Folding a finished group: tot += scale * (P' + ((offset - X_BIAS) / P_MUL) * X), with the common factor P_MUL
+    // applied once at the output (both rescalings are powers of two, hence exact).
+    float sc[4], of[4];
+    auto fold_params = [&](const u32x2 s2, const u32x2 o2) {
 #pragma unroll
-        for (int j = 0; j < WTN; j++)
+        for (int r = 0; r < 4; r++) {
+            const uint32_t su = s2[r >> 1], ou = o2[r >> 1] & omask;
+            sc[r] = (r & 1) ? act_hi<ACT>(su) : act_lo<ACT>(su);
+            of[r] = __builtin_fmaf((r & 1) ? act_hi<ACT>(ou) : act_lo<ACT>(ou), 1.0f / P_MUL, -X_BIAS / P_MUL);
+        }
+    };
+    auto fold_tile = [&](int i, int j) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const uint32_t su = sv[j][r >> 1], ou = ov[j][r >> 1] & omask;
-                const float sc = ((r & 1) ? act_hi<ACT>(su) : act_lo<ACT>(su)) * P_MUL;
-                const float of = (((r & 1) ? act_hi<ACT>(ou) : act_lo<ACT>(ou)) - X_BIAS) * (1.0f / P_MUL);
-#pragma unroll
-                for (int i = 0; i < WTM; i++) {
-                    const float inner = __builtin_fmaf(of, X[i][0], P[i][j][r]);
-                    tot[i][j][r] = __builtin_fmaf(sc, inner, tot[i][j][r]);
-                }
-            }
-#pragma unroll
-        for (int i = 0; i < WTM; i++) {
-            X[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int j = 0; j < WTN; j++) P[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int r = 0; r < 4; r++) {
+            const float inner = __builtin_fmaf(of[r], X[i], P[i][j][r]);
+            tot[i][j][r] = __builtin_fmaf(sc[r], inner, tot[i][j][r]);
         }
     };
 
@@ -192,41 +233,32 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
     const int sw0 = ((lane >> 4) ^ ((frow >> 1) & 7)) * 16;
     const int a_off = (wm * 64 + frow) * PITCH;
     const int b_off = A_RING + (wn * WTN * 16 + frow) * PITCH;
-    const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
-    // Small wavefront tiles issue all fragment reads of the stage up front (the reads of the second half overlap the
-    // MFMAs of the first); the 64 x 64 tile has no registers to spare for that.
-    constexpr int AHEAD = WTM * WTN <= 8 ? 2 : 1;
-    auto compute = [&](int s) {
-        const char *sa = lds + (s % 3) * A_BYTES + a_off, *sb = lds + (s & 1) * B_BYTES + b_off;
+    const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+    // activation fragments of a half stage are read together; weight fragments are streamed one tile column ahead
+    // (two live instead of WTN: the 64 x 64 tile with a running total has no registers to spare)
+    u32x4 AF[WTM], BF[2];
+    const char *sb_cur = nullptr;
+    auto read_frags = [&](int s, int ks) {
+        const char *sa = lds + (s % 3) * A_BYTES + a_off;
+        const int sw = sw0 ^ (ks * 64);
+        sb_cur = lds + (s & 1) * B_BYTES + b_off + sw;
 #pragma unroll
-        for (int k0 = 0; k0 < 2; k0 += AHEAD) {
-            u32x4 AF[AHEAD][WTM], BF[AHEAD][WTN];
-#pragma unroll
-            for (int ks = 0; ks < AHEAD; ks++) {
-                const int sw = sw0 ^ ((k0 + ks) * 64);
-#pragma unroll
-                for (int i = 0; i < WTM; i++) AF[ks][i] = *reinterpret_cast<const u32x4 *>(sa + i * 16 * PITCH + sw);
-#pragma unroll
-                for (int j = 0; j < WTN; j++) BF[ks][j] = *reinterpret_cast<const u32x4 *>(sb + j * 16 * PITCH + sw);
-            }
-#pragma unroll
-            for (int ks = 0; ks < AHEAD; ks++) {
-#pragma unroll
-                for (int j = 0; j < WTN; j++)
-#pragma unroll
-                    for (int i = 0; i < WTM; i++) P[i][j] = mfma_act<ACT>(BF[ks][j], AF[ks][i], P[i][j]);
-#pragma unroll
-                for (int i = 0; i < WTM; i++) X[i] = mfma_act<ACT>(ones, AF[ks][i], X[i]);
-            }
-        }
+        for (int i = 0; i < WTM; i++) AF[i] = *reinterpret_cast<const u32x4 *>(sa + i * 16 * PITCH + sw);
+        BF[0] = *reinterpret_cast<const u32x4 *>(sb_cur);
     };
+    auto read_b = [&](int j) { BF[j & 1] = *reinterpret_cast<const u32x4 *>(sb_cur + j * 16 * PITCH); };
 
     // ---- main loop.  Stage s is computed from activation slot s % 3 and image slot s & 1.  Meanwhile image slot
     // (s + 1) & 1 receives the images of stage s + 1, expanded from the raw ring, and memory is asked for the
     // activations of stage s + 2 and the raw weights of stage s + 3.  Loads are never skipped (a stage past the end
     // gets an out-of-range lane offset and moves no bytes), so the number of loads in flight is the same in every
     // iteration: at the top, "at most LA + 1 outstanding" means everything but the newest refills has landed.
-    uint32_t wr[8], wx[8];
+    //
+    // The VALU work rides in the shadow of the MFMAs of the same wavefront: a finished scale group is folded tile by
+    // tile in the first half of the next stage (fold tile t, then restart its accumulator with an MFMA whose C
+    // operand is zero, while the VALU goes on to tile t + 1), and the images of stage s + 1 are expanded between the
+    // MFMAs of the second half.  sched_barrier pins that order.
+    uint32_t wx[8];
     issue_w(0);
     issue_a(0);
     issue_w(1);
@@ -234,41 +266,100 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
     issue_w(2);
     wait_vmcnt<2 * LA + 2>();
     __syncthreads();
-    read_raw(wr, 0);
-    flip_w(wx, wr);
+    read_raw(wx, 0);
+    flip_w(wx, wx);
     expand_w(wx, 0);
-    auto body = [&](int s) {
+    bool pending = false;                                      // a finished group awaits its fold
+    int pending_row = 0;
+    for (int s = 0; s < NSTG; s++) {
         wait_vmcnt<LA + 1>();
         wait_lgkmcnt0();
         __syncthreads();                                       // stage s is complete in LDS; everyone is done with stage s - 1
-        const bool fold_stage = ACCUM && (s0 + s + 1) % p.unit_stages == 0;   // the last stage of a scale group
-        if (fold_stage) load_params((s0 + s) / p.unit_stages, true);            // first: the fold must not wait for the refills
+        read_frags(s, 0);
+        // the parameters of a group are fetched in its last stage, ahead of the refills (the wait at the next top
+        // then covers them)
+        const bool last_of_group = ACCUM && (s0 + s + 1) % p.unit_stages == 0;
+        const int group_row = (s0 + s) / p.unit_stages;
+        if (last_of_group && wave == 0) issue_params(group_row);
         issue_a(s + 2);
         issue_w(s + 3);
         __builtin_amdgcn_sched_barrier(0);
-        // the two wavefronts of a SIMD (w and w + 4) expand and compute in opposite order, so that the VALU work
-        // of one overlaps the MFMA work of the other
-        if (wave < 4) {
-            read_raw(wr, s + 1);
-            flip_w(wx, wr);
-            expand_w(wx, s + 1);
+        if (ACCUM && pending) {
+            const char *pb = prm + (pending_row & 1) * PRM_SLOT + prm_col;
+            const char *px = prm + (pending_row & 1) * PRM_SLOT + 1024 + (wm * 64 + frow) * 4;
+#pragma unroll
+            for (int i = 0; i < WTM; i++) X[i] = *reinterpret_cast<const float *>(px + i * 64);
+#pragma unroll
+            for (int j = 0; j < WTN; j++) {
+                if (j + 1 < WTN) read_b(j + 1);
+                fold_params(*reinterpret_cast<const u32x2 *>(pb + j * 32), *reinterpret_cast<const u32x2 *>(pb + 512 + j * 32));
+#pragma unroll
+                for (int i = 0; i < WTM; i++) {
+                    fold_tile(i, j);
+                    P[i][j] = mfma_act<ACT>(BF[j & 1], AF[i], zero4);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < WTN; j++) {
+                if (j + 1 < WTN) read_b(j + 1);
+#pragma unroll
+                for (int i = 0; i < WTM; i++) P[i][j] = mfma_act<ACT>(BF[j & 1], AF[i], P[i][j]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
-        compute(s);
+        pending = last_of_group;
+        pending_row = group_row;
+        read_raw(wx, s + 1);
+        read_frags(s, 1);
+        flip_w(wx, wx);
         __builtin_amdgcn_sched_barrier(0);
-        if (wave >= 4) {
-            read_raw(wr, s + 1);
-            flip_w(wx, wr);
-            expand_w(wx, s + 1);
+        // second half: MFMAs with the expansion of stage s + 1 in between
+        {
+            char *bs = lds + A_RING + ((s + 1) & 1) * B_BYTES;
+#pragma unroll
+            for (int j = 0; j < WTN; j++) {
+                if (j + 1 < WTN) read_b(j + 1);
+#pragma unroll
+                for (int i = 0; i < WTM; i++) P[i][j] = mfma_act<ACT>(BF[j & 1], AF[i], P[i][j]);
+                if (j < CPL / 2) {
+                    u32x4 b0, b1;
+                    expand_pair<WBITS, ACT>(wx, j, magic, b0, b1);
+                    const int n = lane * CPL + 2 * j;          // even: n and n + 1 share the swizzle
+                    const int sw = (wave ^ ((n >> 1) & 7)) * 16;
+                    *reinterpret_cast<u32x4 *>(bs + n * PITCH + sw) = b0;
+                    *reinterpret_cast<u32x4 *>(bs + (n + 1) * PITCH + sw) = b1;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        if (fold_stage) fold();
-    };
-    for (int s = 0; s < NSTG; s++) body(s);
+    }
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the refills past the end (zeros) have landed
     __syncthreads();
-    if constexpr (!ACCUM) {
-        load_params(p.grouped ? u0 : 0, true);
-        fold();
+    // the last group (without the running total: the only one)
+    load_params(p.grouped ? u1 - 1 : 0);
+    {
+        const int ufirst = ACCUM ? u1 - 1 : u0;                // without the running total: every unit of this workgroup
+#pragma unroll
+        for (int i = 0; i < WTM; i++) X[i] = 0.0f;
+        for (int u = ufirst; u < u1; u++) {
+#pragma unroll
+            for (int i = 0; i < WTM; i++) {
+                const int m = min(m0 + wm * 64 + i * 16 + frow, p.M - 1);
+                X[i] += p.rowsum[(int64_t)u * p.M + m];
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < WTN; j++) {
+        fold_params(sv[j], ov[j]);
+#pragma unroll
+        for (int i = 0; i < WTM; i++) {
+            fold_tile(i, j);
+            tot[i][j] = tot[i][j] * P_MUL;
+        }
     }
 
     // ---- split K: publish, count, last arrival sums in chunk order
@@ -343,7 +434,7 @@ template <int WBITS, int ACT, int BM, bool ACCUM>
 int launch_tile(WqGemmArgs &p, hipStream_t s)
 {
     constexpr int BN = WBITS == 4 ? 256 : 128;
-    constexpr size_t lds_bytes = (size_t)(3 * BM + 2 * BN) * 128 + 3 * 64 * 128;   // activation ring, image slots, raw ring
+    constexpr size_t lds_bytes = (size_t)(3 * BM + 2 * BN) * 128 + 3 * 64 * 128 + 2 * 2048;   // activation ring, image slots, raw ring, parameters
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
     auto kern = wq_gemm_kernel<WBITS, ACT, BM, ACCUM>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -376,7 +467,7 @@ WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_
             ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 4)) &&
             (scale == nullptr || aligned(scale, 4)) && (offset == nullptr || aligned(offset, 4)) &&
             (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 32) && (uint64_t)128 * (uint64_t)ldx * 2 < (1ull << 31) &&
-            (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && !(off_env && off_env[0] == '0');
+            (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && (uint64_t)(K / 128) * (uint64_t)M * 4 < (1ull << 31) && !(off_env && off_env[0] == '0');
     if (!pl.ok) return pl;
     const int bn = w_bits == 4 ? 256 : 128;
     pl.bm = M <= 64 ? 64 : 128;
@@ -396,7 +487,8 @@ WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_
     pl.S = (int)S;
     pl.accum = pl.grouped && (pl.n_units + pl.S - 1) / pl.S > 1;
     pl.partial_bytes = pl.S > 1 ? (size_t)tiles * pl.S * pl.bm * bn * 4 : 0;
-    pl.counter_bytes = pl.S > 1 ? kWorkspaceCounterBytes : 0;
+    pl.counter_bytes = kWorkspaceCounterBytes;                 // the workspace always starts with the counters
+    pl.rowsum_bytes = (size_t)pl.n_units * (size_t)M * sizeof(float);
     (void)bn;
     return pl;
 }
@@ -414,6 +506,7 @@ int launch_wq_gemm(const WqGemmPlan &pl, const void *x, int act_f16, const void 
     p.out = static_cast<uint16_t *>(out);
     p.counter = pl.S > 1 ? static_cast<uint32_t *>(workspace) : nullptr;
     p.partial = pl.S > 1 ? reinterpret_cast<float *>(static_cast<char *>(workspace) + pl.counter_bytes) : nullptr;
+    p.rowsum = reinterpret_cast<float *>(static_cast<char *>(workspace) + pl.counter_bytes + pl.partial_bytes);
     p.ldx = ldx;
     p.ldo = ldo;
     p.ldw_bytes = (uint32_t)(w_bits == 4 ? ldw_k * 4 : ldw_k);
@@ -429,6 +522,15 @@ int launch_wq_gemm(const WqGemmPlan &pl, const void *x, int act_f16, const void 
     p.tiles_per_xcd = (pl.tiles_m * pl.tiles_n + 7) / 8;
     p.S = pl.S;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    {
+        const int unit_k = 64 * pl.unit_stages;
+        const unsigned blocks = (unsigned)(((int64_t)M * pl.n_units + 255) / 256);
+        if (act_f16)
+            hipLaunchKernelGGL(wq_rowsum_kernel<1>, dim3(blocks), dim3(256), 0, s, p.x, p.rowsum, p.M, pl.n_units, unit_k, ldx);
+        else
+            hipLaunchKernelGGL(wq_rowsum_kernel<0>, dim3(blocks), dim3(256), 0, s, p.x, p.rowsum, p.M, pl.n_units, unit_k, ldx);
+        if (check_launch() != MI355_OK) return MI355_ERR_LAUNCH;
+    }
     if (act_f16) return w_bits == 4 ? launch_any<4, 1>(p, pl, s) : launch_any<8, 1>(p, pl, s);
     return w_bits == 4 ? launch_any<4, 0>(p, pl, s) : launch_any<8, 0>(p, pl, s);
 }

@@ -848,7 +848,7 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
     size_t need = pl.fast ? pl.partial_bytes + pl.counter_bytes : 0;
     const WqGemmPlan gp = make_wq_gemm_plan(M, N, K, w_bits, group_size, true, w_bits == 4 ? N / 8 : N, K, nullptr, nullptr,
                                             nullptr, nullptr);
-    if (gp.ok && gp.partial_bytes + gp.counter_bytes > need) need = gp.partial_bytes + gp.counter_bytes;
+    if (gp.ok && gp.counter_bytes + gp.partial_bytes + gp.rowsum_bytes > need) need = gp.counter_bytes + gp.partial_bytes + gp.rowsum_bytes;
     if (w_bits == 8) {                      // the K-major layout may split differently
         const WqKmPlan km = make_kmajor_plan(M, N, K, group_size, K, K, nullptr, nullptr);
         if (km.fast && km.partial_bytes + km.counter_bytes > need) need = km.partial_bytes + km.counter_bytes;
@@ -914,10 +914,8 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
     // more than 32 rows: the tiled kernel decodes every weight once per 64 or 128 rows
     const WqGemmPlan gp = make_wq_gemm_plan(M, N, K, w_bits, group_size, n_major, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
     if (gp.ok && aligned(out_bf16, 2) && (!bias || aligned(bias, 2))) {
-        if (gp.S > 1) {
-            if (!workspace || workspace_bytes < gp.partial_bytes + gp.counter_bytes) return MI355_ERR_WORKSPACE;
-            if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
-        }
+        if (!workspace || workspace_bytes < gp.counter_bytes + gp.partial_bytes + gp.rowsum_bytes) return MI355_ERR_WORKSPACE;
+        if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
         return launch_wq_gemm(gp, x_bf16, f16 ? 1 : 0, w, w_bits, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, ldx, ldw_k,
                               ldo, workspace, stream);
     }
