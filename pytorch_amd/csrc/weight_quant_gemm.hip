@@ -41,22 +41,26 @@ struct WqGemmArgs {
     int tiles_m, tiles_n, tiles_per_xcd, S;
 };
 
-// rowsum[u][m] = sum of x[m, u * unit_k .. (u + 1) * unit_k): one thread per sum, 16-byte loads.
+// rowsum[u][m] = sum of x[m, u * unit_k .. (u + 1) * unit_k).  Sixteen lanes share one sum: each takes 16 bytes of
+// every 256-byte piece of the unit (coalesced), then the sixteen partial sums are added with four butterfly steps.
 template <int ACT>
 __global__ __launch_bounds__(256) void wq_rowsum_kernel(const uint16_t *__restrict__ x, float *__restrict__ rowsum, int M,
                                                         int n_units, int unit_k, int64_t ldx)
 {
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= M * n_units) return;
-    const int m = idx / n_units, u = idx % n_units;         // neighbouring threads read neighbouring units of one row
-    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + (int64_t)m * ldx + (int64_t)u * unit_k);
+    const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;   // which sum
+    const int sub = threadIdx.x & 15;
+    const bool valid = idx < (int64_t)M * n_units;
+    const int m = valid ? (int)(idx / n_units) : 0, u = valid ? (int)(idx % n_units) : 0;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + (int64_t)m * ldx + (int64_t)u * unit_k) + sub;
     float acc = 0.0f;
-    for (int c = 0; c < unit_k / 8; c++) {
-        const u32x4 v = src[c];
+    for (int c = 0; c < unit_k / 128; c++) {
+        const u32x4 v = src[c * 16];
 #pragma unroll
         for (int e = 0; e < 4; e++) acc += act_lo<ACT>(v[e]) + act_hi<ACT>(v[e]);
     }
-    rowsum[(int64_t)u * M + m] = acc;
+#pragma unroll
+    for (int d = 8; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, 16);
+    if (valid && sub == 0) rowsum[(int64_t)u * M + m] = acc;
 }
 
 template <int WBITS, int ACT, int BM, bool ACCUM>
@@ -389,13 +393,23 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
         for (int i = 0; i < WTM; i++)
 #pragma unroll
             for (int j = 0; j < WTN; j++) tot[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        for (int ch = 0; ch < p.S; ch++) {
+        // two chunks per round: all their loads are in flight together; the sums stay in chunk order
+        for (int ch = 0; ch < p.S; ch += 2) {
+            f32x4 v0[WTM][WTN], v1[WTM][WTN];
+            const uint32_t second = ch + 1 < p.S ? 0u : kOutOfRange;   // an odd tail reads zeros
 #pragma unroll
             for (int i = 0; i < WTM; i++)
 #pragma unroll
-                for (int j = 0; j < WTN; j++)
-                    tot[i][j] += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                for (int j = 0; j < WTN; j++) {
+                    v0[i][j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
                         rsrc_p, lane_off + (i * WTN + j) * 1024, (uint32_t)ch * CHUNK_BYTES, SC1));
+                    v1[i][j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                        rsrc_p, (lane_off + (i * WTN + j) * 1024) | second, (uint32_t)(ch + 1) * CHUNK_BYTES, SC1));
+                }
+#pragma unroll
+            for (int i = 0; i < WTM; i++)
+#pragma unroll
+                for (int j = 0; j < WTN; j++) tot[i][j] = (tot[i][j] + v0[i][j]) + v1[i][j];
         }
         if (threadIdx.x == 0) __hip_atomic_store(p.counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -524,7 +538,7 @@ int launch_wq_gemm(const WqGemmPlan &pl, const void *x, int act_f16, const void 
     hipStream_t s = static_cast<hipStream_t>(stream);
     {
         const int unit_k = 64 * pl.unit_stages;
-        const unsigned blocks = (unsigned)(((int64_t)M * pl.n_units + 255) / 256);
+        const unsigned blocks = (unsigned)(((int64_t)M * pl.n_units * 16 + 255) / 256);
         if (act_f16)
             hipLaunchKernelGGL(wq_rowsum_kernel<1>, dim3(blocks), dim3(256), 0, s, p.x, p.rowsum, p.M, pl.n_units, unit_k, ldx);
         else
