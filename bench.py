@@ -363,6 +363,25 @@ def main():
                 others.append(e)
                 del keep
 
+    if want("aq"):
+        # standalone antiquantisation of a decoder-MLP-sized weight: int8 / packed int4 [4096, 14336] -> bf16
+        R, C = 4096, 14336
+        sc_f = (torch.rand(C, generator=gen, device=dev) * 9e-3 + 1e-3)
+        of_f = (torch.rand(C, generator=gen, device=dev) * 8 - 4)
+        for bits in (8, 4):
+            nb = R * C * bits // 8 + R * C * 2 + 2 * C * 4
+            ns = _nsets(nb)
+            if bits == 8:
+                xs = [torch.randint(-128, 128, (R, C), generator=gen, dtype=torch.int8, device=dev) for _ in range(ns)]
+            else:
+                xs = [torch.randint(-2 ** 31, 2 ** 31 - 1, (R, C // 8), generator=gen, dtype=torch.int32, device=dev)
+                      for _ in range(ns)]
+            keep = []
+            calls = [(lambda x=x: keep.append(pa.npu_anti_quant(x, sc_f, offset=of_f, dst_dtype=torch.bfloat16))) for x in xs] * 2
+            us = _graph_time_us(torch, calls)
+            others.append(hbm_entry(f"npu_anti_quant int{bits}[4096,14336] -> bf16 (per-column float32 scale and offset)", nb, us))
+            del xs, keep
+
     if others:
         result["others"] = others
     print(json.dumps(result))

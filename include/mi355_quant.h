@@ -158,6 +158,23 @@ int mi355_swiglu(const void *x_bf16, void *out_bf16, int64_t rows, int64_t half,
 int mi355_swiglu_quant(const void *x_bf16, int activate_left, int8_t *y, float *scale,
                        int64_t rows, int64_t half, int64_t x_row_stride, void *stream);
 
+/*
+ * npu_anti_quant: the standalone antiquantisation out = cast((float(x) + offset) * scale).
+ * Replaces the aclnn AscendAntiQuant call behind torch_npu.npu_anti_quant (signature test/torch_npu_schema.json:2117-2119,
+ * wrapper torch_npu/onnx/wrapper_onnx_ops.py:824-828; CPU golden test/custom_ops/test_npu_anti_quant.py:29-42, int4
+ * unpacking :12-24).
+ *
+ *   x       x_bits == 8: int8 [rows, cols], row pitch ldx bytes
+ *           x_bits == 4: int32 [rows, cols/8], row pitch ldx words; word j of a row holds columns 8j..8j+7,
+ *                        element i in bits [4i, 4i+3], two's complement (cols must be a multiple of 8)
+ *   scale   float32 [scale_len], scale_len == cols or 1;  offset float32 [offset_len] likewise, or NULL (zero)
+ *   out     [rows, cols] of out_dtype (MI355_DTYPE_BF16 or MI355_DTYPE_FP16), row pitch ldo elements:
+ *           out[r,c] = round((float(x[r,c]) + offset[c]) * scale[c]), the sum and the product each rounded to float32
+ */
+int mi355_anti_quant(const void *x, int x_bits, const float *scale, int64_t scale_len, const float *offset,
+                     int64_t offset_len, void *out, int out_dtype, int64_t rows, int64_t cols, int64_t ldx, int64_t ldo,
+                     void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -168,6 +168,23 @@ def antiquant(w_i8, scale_f32, offset_f32=None) -> np.ndarray:
     return out
 
 
+def anti_quant(x, scale_f32, offset_f32=None, dst: str = "fp16") -> np.ndarray:
+    """npu_anti_quant: x int8 [rows, cols] or int32 [rows, cols/8] (packed int4); scale / offset float32 with cols
+    elements or one.  Returns the bit patterns of the float16 / bfloat16 result.  A composition of the restatements
+    above (unpack, (x + offset) * scale in float32) and one IEEE rounding to the output type."""
+    xa = np.asarray(x)
+    vals = unpack_int4(xa) if xa.dtype == np.int32 else _c(xa, np.int8)
+    vals = vals.reshape(-1, vals.shape[-1])
+    cols = vals.shape[1]
+    s = np.broadcast_to(_c(scale_f32, np.float32).reshape(-1), (cols,))
+    o = None if offset_f32 is None else np.broadcast_to(_c(offset_f32, np.float32).reshape(-1), (cols,))
+    f = antiquant(vals, s, o)
+    if dst == "bf16":
+        return f32_to_bf16_bits(f)
+    assert dst == "fp16"
+    return f.astype(np.float16).view(np.uint16)          # IEEE round to nearest even
+
+
 def weight_quant_matmul(x_u16, w, scale_u16, off_u16=None, group_size: int = 0, accum: str = "f32", dtype: str = "bf16",
                         bias_u16=None):
     """x bf16 (or, with dtype="fp16", float16) bits [M,K]; w int8 [K,N] (any strides) or int32 [K,N/8] (packed int4);

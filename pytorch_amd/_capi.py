@@ -16,7 +16,8 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
 
 EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant",
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
-           "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant")
+           "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
+           "mi355_anti_quant")
 
 _lib = None
 
@@ -45,6 +46,7 @@ def lib() -> ctypes.CDLL:
                                                 vp, sz, vp]
         L.mi355_swiglu.argtypes = [vp, vp, i64, i64, i64, vp]
         L.mi355_swiglu_quant.argtypes = [vp, i32, vp, vp, i64, i64, i64, vp]
+        L.mi355_anti_quant.argtypes = [vp, i32, vp, i64, vp, i64, vp, i32, i64, i64, i64, i64, vp]
         _lib = L
     return _lib
 
@@ -157,3 +159,16 @@ def swiglu_quant(x, activate_left: bool = True):
     _check(lib().mi355_swiglu_quant(_ptr(x), 1 if activate_left else 0, _ptr(y), _ptr(scale), rows, two // 2, x.stride(0),
                                     _stream()), "mi355_swiglu_quant")
     return y, scale
+
+
+def anti_quant(x, scale, offset=None, dst_dtype=torch.float16):
+    """x int8 [rows, cols] or int32 [rows, cols/8] (packed int4), scale / offset float32 [cols] or [1] ->
+    dst_dtype [rows, cols] = (float(x) + offset) * scale."""
+    assert x.dim() == 2 and x.stride(1) == 1
+    bits = 4 if x.dtype == torch.int32 else 8
+    rows, cols = x.shape[0], x.shape[1] * (8 if bits == 4 else 1)
+    out = torch.empty((rows, cols), dtype=dst_dtype, device=x.device)
+    _check(lib().mi355_anti_quant(_ptr(x), bits, _ptr(scale), scale.numel(), _ptr(offset), 0 if offset is None else offset.numel(),
+                                  _ptr(out), 1 if dst_dtype == torch.float16 else 0, rows, cols, x.stride(0), cols, _stream()),
+           "mi355_anti_quant")
+    return out

@@ -469,6 +469,59 @@ std::tuple<Tensor, Tensor> swiglu_quant_hip(const Tensor &x, const optional<Tens
     return {y, scale};
 }
 
+// ---------------------------------------------------------------- npu_anti_quant
+// torch_npu.npu_anti_quant(x, scale, *, offset=None, dst_dtype=None, src_dtype=None)
+// (test/torch_npu_schema.json:2117-2119; golden test/custom_ops/test_npu_anti_quant.py:29-42)
+
+at::ScalarType anti_quant_check(const Tensor &x, const Tensor &scale, const optional<Tensor> &offset,
+                                optional<at::ScalarType> dst_dtype, optional<at::ScalarType> src_dtype)
+{
+    TORCH_CHECK(x.scalar_type() == at::kChar || x.scalar_type() == at::kInt,
+                "npu_anti_quant: x must be int8 or int32 (packed int4), got ", x.scalar_type());
+    TORCH_CHECK(x.dim() >= 1, "npu_anti_quant: x must have at least one dimension");
+    TORCH_CHECK(!src_dtype.has_value() || *src_dtype == at::kChar, "npu_anti_quant: src_dtype must be torch.int8");
+    const at::ScalarType dst = dst_dtype.value_or(at::kHalf);
+    TORCH_CHECK(dst == at::kHalf || dst == at::kBFloat16, "npu_anti_quant: dst_dtype must be torch.float16 or torch.bfloat16");
+    const int64_t cols = x.size(-1) * (x.scalar_type() == at::kInt ? 8 : 1);
+    TORCH_CHECK(scale.scalar_type() == at::kFloat, "npu_anti_quant: scale must be float32, got ", scale.scalar_type());
+    TORCH_CHECK(scale.dim() <= 1 && (scale.numel() == cols || scale.numel() == 1),
+                "npu_anti_quant: scale must have one element or one per element of the last dimension (", cols, ")");
+    if (const Tensor *o = opt(offset)) {
+        TORCH_CHECK(o->scalar_type() == at::kFloat, "npu_anti_quant: offset must be float32, got ", o->scalar_type());
+        TORCH_CHECK(o->dim() <= 1 && (o->numel() == cols || o->numel() == 1),
+                    "npu_anti_quant: offset must have one element or one per element of the last dimension (", cols, ")");
+    }
+    return dst;
+}
+
+Tensor anti_quant_meta(const Tensor &x, const Tensor &scale, const optional<Tensor> &offset,
+                       optional<at::ScalarType> dst_dtype, optional<at::ScalarType> src_dtype)
+{
+    const at::ScalarType dst = anti_quant_check(x, scale, offset, dst_dtype, src_dtype);
+    auto shape = x.sizes().vec();
+    if (x.scalar_type() == at::kInt) shape.back() *= 8;
+    return at::empty(shape, x.options().dtype(dst));
+}
+
+Tensor anti_quant_hip(const Tensor &x, const Tensor &scale, const optional<Tensor> &offset,
+                      optional<at::ScalarType> dst_dtype, optional<at::ScalarType> src_dtype)
+{
+    check_same_device("npu_anti_quant", {&x, &scale, opt(offset)});
+    Tensor out = anti_quant_meta(x, scale, offset, dst_dtype, src_dtype);
+    if (out.numel() == 0) return out;
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+    Tensor xin = x.contiguous(), sc = scale.contiguous();
+    Tensor of = opt(offset) ? opt(offset)->contiguous() : Tensor();
+    const int64_t cols = out.size(-1), rows = out.numel() / cols;
+    const bool int4 = x.scalar_type() == at::kInt;
+    check_status(mi355_anti_quant(xin.data_ptr(), int4 ? 4 : 8, sc.data_ptr<float>(), sc.numel(),
+                                  of.defined() ? of.data_ptr<float>() : nullptr, of.defined() ? of.numel() : 0, out.data_ptr(),
+                                  out.scalar_type() == at::kHalf ? MI355_DTYPE_FP16 : MI355_DTYPE_BF16, rows, cols,
+                                  int4 ? cols / 8 : cols, cols, stream_of(x)),
+                 "npu_anti_quant");
+    return out;
+}
+
 } // namespace
 
 TORCH_LIBRARY_FRAGMENT(npu, m)
@@ -483,6 +536,8 @@ TORCH_LIBRARY_FRAGMENT(npu, m)
     m.def("npu_swiglu(Tensor input, int dim=-1) -> Tensor");
     m.def("npu_swiglu_quant(Tensor x, *, Tensor? smooth_scales=None, Tensor? offsets=None, Tensor? group_index=None, "
           "bool activate_left=False, int quant_mode=0, int group_list_type=0, ScalarType? dst_type=None) -> (Tensor, Tensor)");
+    m.def("npu_anti_quant(Tensor x, Tensor scale, *, Tensor? offset=None, ScalarType? dst_dtype=None, "
+          "ScalarType? src_dtype=None) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(npu, CUDA, m)
@@ -492,6 +547,7 @@ TORCH_LIBRARY_IMPL(npu, CUDA, m)
     m.impl("npu_weight_quant_batchmatmul", TORCH_FN(weight_quant_hip));
     m.impl("npu_swiglu", TORCH_FN(swiglu_hip));
     m.impl("npu_swiglu_quant", TORCH_FN(swiglu_quant_hip));
+    m.impl("npu_anti_quant", TORCH_FN(anti_quant_hip));
 }
 
 TORCH_LIBRARY_IMPL(npu, Meta, m)
@@ -501,4 +557,5 @@ TORCH_LIBRARY_IMPL(npu, Meta, m)
     m.impl("npu_weight_quant_batchmatmul", TORCH_FN(weight_quant_meta));
     m.impl("npu_swiglu", TORCH_FN(swiglu_meta));
     m.impl("npu_swiglu_quant", TORCH_FN(swiglu_quant_meta));
+    m.impl("npu_anti_quant", TORCH_FN(anti_quant_meta));
 }

@@ -362,6 +362,29 @@ def test_swiglu(capi, golden):
         assert dist.max() <= 1 and (dist == 0).mean() > 0.995   # device expf vs libm expf
 
 
+# ------------------------------------------------------------------ anti_quant
+
+@pytest.mark.parametrize("rows,cols,packed", [(10, 100, False), (10, 200, True), (4096, 14336, False), (512, 4096, True),
+                                              (7, 24, False), (3, 8, True), (33, 1000, False)])
+@pytest.mark.parametrize("dst", [torch.float16, torch.bfloat16])
+def test_anti_quant(capi, golden, rows, cols, packed, dst):
+    """Bit-exact against the oracle: int8 and packed-int4 inputs (the shapes of test/custom_ops/test_npu_anti_quant.py:49-58
+    and large ones), per-column, single and absent parameters, both output types."""
+    g = torch.Generator().manual_seed(rows + cols)
+    if packed:
+        x = torch.randint(-2 ** 31, 2 ** 31 - 1, (rows, cols // 8), generator=g, dtype=torch.int64).to(torch.int32)
+    else:
+        x = torch.randint(-128, 128, (rows, cols), generator=g, dtype=torch.int8)
+    scale = torch.rand(cols, generator=g) * 200 - 100
+    offset = torch.rand(cols, generator=g) * 200 - 100
+    name = "fp16" if dst == torch.float16 else "bf16"
+    for sc, of in [(scale, offset), (scale, None), (scale[:1].clone(), offset[:1].clone())]:
+        out = capi.anti_quant(x.cuda(), sc.cuda(), None if of is None else of.cuda(), dst_dtype=dst)
+        want = golden.anti_quant(x.numpy(), sc.numpy(), None if of is None else of.numpy(), dst=name)
+        got = out.cpu().view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(got, want)
+
+
 # ------------------------------------------------------------------ error paths (host side, no kernel runs)
 
 @pytest.mark.parametrize("rows,half", [(64, 14336), (2048, 14336), (33, 512), (5, 100), (3, 16384 + 8), (7, 24)])
@@ -386,6 +409,8 @@ def test_c_abi_rejects_bad_arguments(capi):
     assert L.mi355_quant_matmul(None, None, None, None, 0, None, 0, None, 0, 4, 4, 4, 4, 4, 1, 4, None, 0, None) == -1
     assert L.mi355_weight_quant_matmul(None, 0, None, 5, None, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
     assert L.mi355_weight_quant_matmul(None, 9, None, 8, None, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
+    assert L.mi355_anti_quant(None, 5, None, 1, None, 0, None, 0, 1, 8, 8, 8, None) == -1
+    assert L.mi355_anti_quant(None, 4, None, 1, None, 0, None, 7, 1, 8, 1, 8, None) == -1
     assert b"workspace" in L.mi355_status_string(-4)
     x1 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")
     x2 = torch.zeros(128, 128, dtype=torch.int8, device="cuda")

@@ -218,6 +218,31 @@ def test_swiglu_quant_operator(pa, golden):
     assert torch.equal(y1, y2) and torch.equal(s1, s2)
 
 
+def test_anti_quant_operator(pa, golden):
+    """torch_npu.npu_anti_quant(x, scale, offset=..., dst_dtype=..., src_dtype=...) as test/custom_ops/test_npu_anti_quant.py
+    calls it: default float16 output, leading batch dimensions, packed int4 widening the last dimension by 8, and the
+    same-device error message of :86-88."""
+    g = torch.Generator().manual_seed(2)
+    x = torch.randint(-127, 128, (2, 10, 100), generator=g, dtype=torch.int8)
+    scale, offset = torch.rand(100, generator=g) * 200 - 100, torch.rand(100, generator=g) * 200 - 100
+    out = pa.npu_anti_quant(x.cuda(), scale.cuda(), offset=offset.cuda())
+    assert out.dtype == torch.float16 and out.shape == (2, 10, 100)
+    want = golden.anti_quant(x.numpy().reshape(20, 100), scale.numpy(), offset.numpy(), dst="fp16")
+    assert np.array_equal(out.cpu().view(torch.int16).numpy().view(np.uint16).reshape(20, 100), want)
+    out = pa.npu_anti_quant(x.cuda(), scale.cuda(), dst_dtype=torch.bfloat16, src_dtype=torch.int8)
+    want = golden.anti_quant(x.numpy().reshape(20, 100), scale.numpy(), None, dst="bf16")
+    assert np.array_equal(_bits(out).reshape(20, 100), want)
+    x4 = torch.randint(-2 ** 31, 2 ** 31 - 1, (10, 25), generator=g, dtype=torch.int64).to(torch.int32)
+    s4, o4 = torch.rand(200, generator=g) * 2 - 1, torch.rand(200, generator=g) * 16 - 8
+    out = pa.npu_anti_quant(x4.cuda(), s4.cuda(), offset=o4.cuda(), dst_dtype=torch.bfloat16)
+    assert out.shape == (10, 200)
+    assert np.array_equal(_bits(out), golden.anti_quant(x4.numpy(), s4.numpy(), o4.numpy(), dst="bf16"))
+    with pytest.raises(RuntimeError, match="Expected all tensors to be on the same device"):
+        pa.npu_anti_quant(x.cuda(), scale.cuda(), offset=offset)
+    with pytest.raises(RuntimeError, match="dst_dtype"):
+        pa.npu_anti_quant(x.cuda(), scale.cuda(), dst_dtype=torch.float32)
+
+
 def test_c5_mlp_prefill_properties(pa, golden):
     """M = 2048: rows are independent, so any subset of rows run alone must reproduce the same bits."""
     d = workloads.mlp_inputs(seed=1, M=2048)

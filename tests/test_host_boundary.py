@@ -16,7 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def test_c_abi_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "mi355_quant.h")).read()
     declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", header))
-    assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant"} <= declared
+    assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant", "mi355_anti_quant"} <= declared
     lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_amd", "csrc", "libmi355_quant.so"))
     for name in declared:
         assert hasattr(lib, name), name
@@ -160,6 +160,20 @@ def test_meta_swiglu_quant(pa):
         pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16))                      # static quantisation is not built
     with pytest.raises(RuntimeError, match="smooth_scales"):
         pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(4, dtype=torch.bfloat16), quant_mode=1)
+
+
+def test_meta_anti_quant(pa):
+    """Shapes and dtypes of test/test_fake_tensor.py:1949-1959 (same shape, float16) plus the int4 widening."""
+    res = pa.npu_anti_quant(_m(20, 100, dtype=torch.int8), _m(100, dtype=torch.float32), offset=_m(100, dtype=torch.float32),
+                            dst_dtype=torch.float16)
+    assert res.shape == (20, 100) and res.dtype == torch.float16
+    res = pa.npu_anti_quant(_m(10, 25, dtype=torch.int32), _m(200, dtype=torch.float32), dst_dtype=torch.bfloat16)
+    assert res.shape == (10, 200) and res.dtype == torch.bfloat16
+    assert pa.npu_anti_quant(_m(4, 8, dtype=torch.int8), _m(1, dtype=torch.float32)).dtype == torch.float16
+    with pytest.raises(RuntimeError, match="scale must have"):
+        pa.npu_anti_quant(_m(4, 8, dtype=torch.int8), _m(7, dtype=torch.float32))
+    with pytest.raises(RuntimeError, match="int8 or int32"):
+        pa.npu_anti_quant(_m(4, 8, dtype=torch.int16), _m(8, dtype=torch.float32))
 
 
 def test_meta_swiglu(pa):

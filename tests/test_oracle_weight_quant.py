@@ -153,3 +153,34 @@ def test_float16_variant_follows_the_reference_test_recipe(golden):
     ref = x.double() @ ((wt.double() + off.double()).float() * scale.float()).double()
     assert np.allclose(outf, ref.numpy(), rtol=2e-5, atol=1e-5)
     assert np.array_equal(out, torch.from_numpy(outf).to(torch.float16).view(torch.int16).numpy().view(np.uint16))
+
+
+@pytest.mark.parametrize("dst", ["fp16", "bf16"])
+def test_anti_quant_matches_the_in_tree_golden(golden, dst):
+    """npu_anti_quant as the reference's own CPU golden evaluates it (test/custom_ops/test_npu_anti_quant.py:29-42,
+    inputs of :49-66): x.to(float32) + offset, times scale, then .to(dst_dtype), with torch on the CPU; int32 inputs are
+    unpacked with the numpy recipe of :12-24 first."""
+    tdst = torch.float16 if dst == "fp16" else torch.bfloat16
+    g = torch.Generator().manual_seed(0)
+    for packed in (False, True):
+        if packed:
+            words = torch.randint(-2 ** 31, 2 ** 31 - 1, (10, 25), generator=g, dtype=torch.int64).to(torch.int32)
+            by = np.frombuffer(words.numpy().tobytes(), dtype=np.uint8)
+            nib = (by.reshape(-1, 1) >> np.array([0, 4], dtype=np.uint8)) & 0xF
+            vals = torch.from_numpy(((nib.astype(np.int16) ^ 8) - 8).astype(np.int8).reshape(10, 200))
+            x = words
+        else:
+            vals = torch.randint(-127, 128, (10, 100), generator=g, dtype=torch.int8)
+            x = vals
+        n = vals.shape[1]
+        scale = (torch.rand(n, generator=g) * 200 - 100)
+        offset = (torch.rand(n, generator=g) * 200 - 100)
+        for off in (offset, None):
+            want = ((vals.to(torch.float32) + (off if off is not None else 0.0)) * scale).to(tdst)
+            got = golden.anti_quant(x.numpy(), scale.numpy(), None if off is None else off.numpy(), dst=dst)
+            assert np.array_equal(got, want.view(torch.int16).numpy().view(np.uint16))
+    # a single scale / offset broadcasts
+    vals = torch.randint(-127, 128, (3, 16), generator=g, dtype=torch.int8)
+    want = ((vals.float() + 1.5) * 0.25).to(tdst)
+    got = golden.anti_quant(vals.numpy(), np.array([0.25], np.float32), np.array([1.5], np.float32), dst=dst)
+    assert np.array_equal(got, want.view(torch.int16).numpy().view(np.uint16))
