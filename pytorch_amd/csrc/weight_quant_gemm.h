@@ -13,11 +13,14 @@ struct WqGemmPlan {
     int unit_stages;         // 64-row stages per unit of K: a scale group, or two stages per channel
     int n_units;
     bool grouped, accum;     // accum: a workgroup meets more than one scale group
+    bool k_major;            // int8 weights stored [N, K]
     size_t counter_bytes, partial_bytes, rowsum_bytes;   // workspace: [arrival counters | partial sums | row sums]
 };
 
+// layout 1: weight rows contiguous along N, `ldw` elements (int8 bytes / int32 words) between k rows;
+// layout 2: int8 stored [N, K], `ldw` bytes between columns; anything else: not eligible.
 __attribute__((visibility("hidden"))) WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits,
-                                                                   int64_t group_size, bool n_major, int64_t ldw_k,
+                                                                   int64_t group_size, int layout, int64_t ldw,
                                                                    int64_t ldx, const void *x, const void *w,
                                                                    const void *scale, const void *offset);
 
@@ -25,6 +28,6 @@ __attribute__((visibility("hidden"))) WqGemmPlan make_wq_gemm_plan(int64_t M, in
 __attribute__((visibility("hidden"))) int launch_wq_gemm(const WqGemmPlan &plan, const void *x, int act_f16, const void *w,
                                                          int w_bits, const void *scale, const void *offset, const void *bias,
                                                          void *out, int64_t M, int64_t N, int64_t K, int64_t ldx,
-                                                         int64_t ldw_k, int64_t ldo, void *workspace, void *stream);
+                                                         int64_t ldw, int64_t ldo, void *workspace, void *stream);
 
 } // namespace mi355

@@ -63,9 +63,12 @@ __global__ __launch_bounds__(256) void wq_rowsum_kernel(const uint16_t *__restri
     if (valid && sub == 0) rowsum[(int64_t)u * M + m] = acc;
 }
 
-template <int WBITS, int ACT, int BM, bool ACCUM>
+// KM: int8 weights stored [N, K] (K-major, the transposed view the LinearWeightQuant module passes); otherwise the
+// weight rows are contiguous along N.
+template <int WBITS, int ACT, int BM, bool ACCUM, bool KM>
 __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
 {
+    static_assert(!KM || WBITS == 8, "K-major weights are int8");
     constexpr int NW = 8;
     constexpr int BN = WBITS == 4 ? 256 : 128;
     constexpr int WGM = BM / 64, WGN = NW / WGM;
@@ -75,6 +78,8 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
     constexpr int A_RING = 3 * A_BYTES;                        // LDS: three activation slots, two image slots, raw weight ring
     constexpr int LA = BM / 8 / NW;                            // activation loads of a wavefront per stage
     constexpr int CPL = WBITS == 4 ? 4 : 2;                    // weight columns per lane of the loader
+    constexpr int NPIECE = KM ? 2 : CPL / 2;                   // expansion steps of a lane per stage (two 16-byte chunks each... one for int8 rows)
+    constexpr int PPJ = (NPIECE + WTN - 1) / WTN;              // of which this many follow each tile column of the second half
     constexpr float P_MUL = kImageMul<WBITS, ACT>;
     constexpr float X_BIAS = kImageBias<WBITS>;
     static_assert(BM == 64 || BM == 128, "tile rows");
@@ -119,46 +124,75 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
         }
     };
 
-    // ---- weights: global -> LDS raw ring (three slots of 64 rows x 128 B), one octet of rows per wavefront and load
+    // ---- weights: global -> LDS raw ring (three slots of 8 KiB = one stage of the strip), 1 KiB per wavefront and load.
+    // Row-major along N: wavefront w copies k rows 8w .. 8w+7 (128 B each).  K-major: it copies columns 16w .. 16w+15
+    // (64 B = the stage's 64 k each).
     constexpr int RAW_BYTES = 64 * 128;
     char *const raw = lds + A_RING + 2 * B_BYTES;
-    const uint32_t strip_valid = min(128u, p.row_bytes - (uint32_t)tn * 128u);
-    const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(static_cast<const char *>(p.w) + (size_t)tn * 128,
-                                                    (uint32_t)(p.K - 1) * p.ldw_bytes + strip_valid);
-    const uint32_t voff_w = (uint32_t)(lane & 7) * 16u < strip_valid
-                                ? (uint32_t)(lane >> 3) * p.ldw_bytes + (uint32_t)(lane & 7) * 16u
-                                : kOutOfRange;
+    const uint32_t strip_valid = KM ? 0u : min(128u, p.row_bytes - (uint32_t)tn * 128u);
+    const int cols_valid = min(BN, p.N - n0);
+    const __amdgpu_buffer_rsrc_t rsrc_w =
+        KM ? make_rsrc(static_cast<const char *>(p.w) + (size_t)n0 * p.ldw_bytes, (uint32_t)(cols_valid - 1) * p.ldw_bytes + (uint32_t)p.K)
+           : make_rsrc(static_cast<const char *>(p.w) + (size_t)tn * 128, (uint32_t)(p.K - 1) * p.ldw_bytes + strip_valid);
+    const uint32_t voff_w = KM ? (uint32_t)(lane >> 2) * p.ldw_bytes + (uint32_t)(lane & 3) * 16u
+                               : ((uint32_t)(lane & 7) * 16u < strip_valid
+                                      ? (uint32_t)(lane >> 3) * p.ldw_bytes + (uint32_t)(lane & 7) * 16u
+                                      : kOutOfRange);
     auto issue_w = [&](int s) {
         const uint32_t vo = s < NSTG ? voff_w : kOutOfRange;
-        const uint32_t row = (uint32_t)(s0 + s) * 64u + (uint32_t)wave * 8u;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void *)(raw + (s % 3) * RAW_BYTES + wave * 1024), 16, vo,
-                                                 row * p.ldw_bytes, 0, 0);
+        const uint32_t so = KM ? (uint32_t)wave * 16u * p.ldw_bytes + (uint32_t)(s0 + s) * 64u
+                               : ((uint32_t)(s0 + s) * 64u + (uint32_t)wave * 8u) * p.ldw_bytes;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void *)(raw + (s % 3) * RAW_BYTES + wave * 1024), 16, vo, so, 0, 0);
     };
-    // this lane's two bytes (2 int8 / 4 int4 columns) of the wavefront's eight rows
+    // Row-major: this lane's two bytes (2 int8 / 4 int4 columns) of the wavefront's eight rows.  K-major: two runs of
+    // eight consecutive k of one column each (chunk c = t * 512 + wave * 64 + lane: column c / 8, k octet c % 8).
     auto read_raw = [&](uint32_t (&wr)[8], int s) {
-        const char *src = raw + (s % 3) * RAW_BYTES + wave * 1024 + lane * 2;
+        if constexpr (KM) {
+            const char *src = raw + (s % 3) * RAW_BYTES + (wave * 64 + lane) * 8;
 #pragma unroll
-        for (int t = 0; t < 8; t++) wr[t] = *reinterpret_cast<const uint16_t *>(src + t * 128);
+            for (int t = 0; t < 2; t++) {
+                const u32x2 v = *reinterpret_cast<const u32x2 *>(src + t * 4096);
+                wr[2 * t] = v.x;
+                wr[2 * t + 1] = v.y;
+            }
+        } else {
+            const char *src = raw + (s % 3) * RAW_BYTES + wave * 1024 + lane * 2;
+#pragma unroll
+            for (int t = 0; t < 8; t++) wr[t] = *reinterpret_cast<const uint16_t *>(src + t * 128);
+        }
     };
-    // registers -> LDS: column n of the tile, k rows 8 * wave .. 8 * wave + 7 of the stage -> chunk slot wave ^ ((n >> 1) & 7)
     uint32_t magic;
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "n"(kInt4Magic<ACT>));   // opaque to the optimiser: stays in a VGPR
     // two's complement -> offset binary (w + 128 / nibble + 8), then the 16-bit images -> LDS
     auto flip_w = [&](uint32_t (&wx)[8], const uint32_t (&wr)[8]) {
 #pragma unroll
-        for (int t = 0; t < 8; t++) wx[t] = wr[t] ^ (WBITS == 4 ? 0x8888u : 0x8080u);
+        for (int t = 0; t < (KM ? 4 : 8); t++) wx[t] = wr[t] ^ (KM ? 0x80808080u : WBITS == 4 ? 0x8888u : 0x8080u);
     };
-    auto expand_w = [&](const uint32_t (&wx)[8], int s) {
+    // registers -> LDS, one piece: column n, k octet o -> chunk slot o ^ ((n >> 1) & 7) of row n
+    auto expand_piece = [&](const uint32_t (&wx)[8], int piece, int s) {
         char *bs = lds + A_RING + (s & 1) * B_BYTES;
-#pragma unroll
-        for (int jb = 0; jb < CPL / 2; jb++) {
+        if constexpr (KM) {
+            const int c = piece * 512 + wave * 64 + lane;
+            const int n = c >> 3, o = c & 7;
+            const uint32_t lo = wx[2 * piece], hi = wx[2 * piece + 1];
+            u32x4 b;
+            b[0] = pack_act2<ACT>((float)(lo & 0xffu), (float)((lo >> 8) & 0xffu));
+            b[1] = pack_act2<ACT>((float)((lo >> 16) & 0xffu), (float)(lo >> 24));
+            b[2] = pack_act2<ACT>((float)(hi & 0xffu), (float)((hi >> 8) & 0xffu));
+            b[3] = pack_act2<ACT>((float)((hi >> 16) & 0xffu), (float)(hi >> 24));
+            *reinterpret_cast<u32x4 *>(bs + n * PITCH + ((o ^ ((n >> 1) & 7)) * 16)) = b;
+        } else {
             u32x4 b0, b1;
-            expand_pair<WBITS, ACT>(wx, jb, magic, b0, b1);
-            const int n = lane * CPL + 2 * jb;                 // even: n and n + 1 share the swizzle
+            expand_pair<WBITS, ACT>(wx, piece, magic, b0, b1);
+            const int n = lane * CPL + 2 * piece;              // even: n and n + 1 share the swizzle
             const int sw = (wave ^ ((n >> 1) & 7)) * 16;
             *reinterpret_cast<u32x4 *>(bs + n * PITCH + sw) = b0;
             *reinterpret_cast<u32x4 *>(bs + (n + 1) * PITCH + sw) = b1;
         }
+    };
+    auto expand_w = [&](const uint32_t (&wx)[8], int s) {
+#pragma unroll
+        for (int piece = 0; piece < NPIECE; piece++) expand_piece(wx, piece, s);
     };
 
     // ---- antiquant parameters of this lane's columns: tile j covers n0 + (wn * WTN + j) * 16 + 4 * (lane / 16) + r
@@ -322,20 +356,13 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
         __builtin_amdgcn_sched_barrier(0);
         // second half: MFMAs with the expansion of stage s + 1 in between
         {
-            char *bs = lds + A_RING + ((s + 1) & 1) * B_BYTES;
 #pragma unroll
             for (int j = 0; j < WTN; j++) {
                 if (j + 1 < WTN) read_b(j + 1);
 #pragma unroll
                 for (int i = 0; i < WTM; i++) P[i][j] = mfma_act<ACT>(BF[j & 1], AF[i], P[i][j]);
-                if (j < CPL / 2) {
-                    u32x4 b0, b1;
-                    expand_pair<WBITS, ACT>(wx, j, magic, b0, b1);
-                    const int n = lane * CPL + 2 * j;          // even: n and n + 1 share the swizzle
-                    const int sw = (wave ^ ((n >> 1) & 7)) * 16;
-                    *reinterpret_cast<u32x4 *>(bs + n * PITCH + sw) = b0;
-                    *reinterpret_cast<u32x4 *>(bs + (n + 1) * PITCH + sw) = b1;
-                }
+#pragma unroll
+                for (int piece = j * PPJ; piece < (j + 1) * PPJ && piece < NPIECE; piece++) expand_piece(wx, piece, s + 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -444,13 +471,13 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
     }
 }
 
-template <int WBITS, int ACT, int BM, bool ACCUM>
+template <int WBITS, int ACT, int BM, bool ACCUM, bool KM>
 int launch_tile(WqGemmArgs &p, hipStream_t s)
 {
     constexpr int BN = WBITS == 4 ? 256 : 128;
     constexpr size_t lds_bytes = (size_t)(3 * BM + 2 * BN) * 128 + 3 * 64 * 128 + 2 * 2048;   // activation ring, image slots, raw ring, parameters
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
-    auto kern = wq_gemm_kernel<WBITS, ACT, BM, ACCUM>;
+    auto kern = wq_gemm_kernel<WBITS, ACT, BM, ACCUM, KM>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
@@ -458,29 +485,32 @@ int launch_tile(WqGemmArgs &p, hipStream_t s)
     return check_launch();
 }
 
-template <int WBITS, int ACT>
+template <int WBITS, int ACT, bool KM>
 int launch_any(WqGemmArgs &p, const WqGemmPlan &pl, hipStream_t s)
 {
     if (pl.bm == 64)
-        return pl.accum ? launch_tile<WBITS, ACT, 64, true>(p, s) : launch_tile<WBITS, ACT, 64, false>(p, s);
-    return pl.accum ? launch_tile<WBITS, ACT, 128, true>(p, s) : launch_tile<WBITS, ACT, 128, false>(p, s);
+        return pl.accum ? launch_tile<WBITS, ACT, 64, true, KM>(p, s) : launch_tile<WBITS, ACT, 64, false, KM>(p, s);
+    return pl.accum ? launch_tile<WBITS, ACT, 128, true, KM>(p, s) : launch_tile<WBITS, ACT, 128, false, KM>(p, s);
 }
 
 } // namespace
 
-WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size, bool n_major, int64_t ldw_k,
+WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size, int layout, int64_t ldw,
                              int64_t ldx, const void *x, const void *w, const void *scale, const void *offset)
 {
     WqGemmPlan pl{};
+    pl.k_major = layout == 2;
     const int64_t row_bytes = w_bits == 4 ? N / 2 : N;
-    const int64_t ldw_bytes = w_bits == 4 ? ldw_k * 4 : ldw_k;
+    const int64_t ldw_bytes = w_bits == 4 ? ldw * 4 : ldw;     // bytes between k rows, or (K-major) between columns
     const int64_t group = group_size > 0 ? group_size : K;
     pl.grouped = group_size > 0 && group != K;
     const char *off_env = getenv("MI355_WQ_GEMM");             // tuning aid: "0" keeps every shape on the streaming kernels
-    pl.ok = M > 32 && n_major && K >= 128 && K % 128 == 0 && group % 128 == 0 && N % 8 == 0 && ldw_bytes % 4 == 0 &&
+    const bool layout_ok = layout == 1 ? ldw_bytes >= row_bytes && (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 32)
+                                       : layout == 2 && w_bits == 8 && ldw >= K && (uint64_t)N * (uint64_t)ldw < (1ull << 32);
+    pl.ok = M > 32 && layout_ok && K >= 128 && K % 128 == 0 && group % 128 == 0 && N % 8 == 0 && ldw_bytes % 4 == 0 &&
             ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 4)) &&
             (scale == nullptr || aligned(scale, 4)) && (offset == nullptr || aligned(offset, 4)) &&
-            (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 32) && (uint64_t)128 * (uint64_t)ldx * 2 < (1ull << 31) &&
+            (uint64_t)128 * (uint64_t)ldx * 2 < (1ull << 31) &&
             (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && (uint64_t)(K / 128) * (uint64_t)M * 4 < (1ull << 31) && !(off_env && off_env[0] == '0');
     if (!pl.ok) return pl;
     const int bn = w_bits == 4 ? 256 : 128;
@@ -488,7 +518,7 @@ WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_
     if (const int f = env_int("MI355_WQG_BM"))                 // tuning aid
         if (f == 64 || f == 128) pl.bm = f;
     pl.tiles_m = (int)((M + pl.bm - 1) / pl.bm);
-    pl.tiles_n = (int)((row_bytes + 127) / 128);
+    pl.tiles_n = pl.k_major ? (int)((N + 127) / 128) : (int)((row_bytes + 127) / 128);
     pl.unit_stages = pl.grouped ? (int)(group / 64) : 2;
     pl.n_units = (int)(K / (64 * pl.unit_stages));
     const int64_t tiles = (int64_t)pl.tiles_m * pl.tiles_n;
@@ -509,7 +539,7 @@ WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_
 
 int launch_wq_gemm(const WqGemmPlan &pl, const void *x, int act_f16, const void *w, int w_bits, const void *scale,
                    const void *offset, const void *bias, void *out, int64_t M, int64_t N, int64_t K, int64_t ldx,
-                   int64_t ldw_k, int64_t ldo, void *workspace, void *stream)
+                   int64_t ldw, int64_t ldo, void *workspace, void *stream)
 {
     WqGemmArgs p{};
     p.x = static_cast<const uint16_t *>(x);
@@ -523,7 +553,7 @@ int launch_wq_gemm(const WqGemmPlan &pl, const void *x, int act_f16, const void 
     p.rowsum = reinterpret_cast<float *>(static_cast<char *>(workspace) + pl.counter_bytes + pl.partial_bytes);
     p.ldx = ldx;
     p.ldo = ldo;
-    p.ldw_bytes = (uint32_t)(w_bits == 4 ? ldw_k * 4 : ldw_k);
+    p.ldw_bytes = (uint32_t)(w_bits == 4 ? ldw * 4 : ldw);
     p.row_bytes = (uint32_t)(w_bits == 4 ? N / 2 : N);
     p.M = (int)M;
     p.N = (int)N;
@@ -545,8 +575,9 @@ int launch_wq_gemm(const WqGemmPlan &pl, const void *x, int act_f16, const void 
             hipLaunchKernelGGL(wq_rowsum_kernel<0>, dim3(blocks), dim3(256), 0, s, p.x, p.rowsum, p.M, pl.n_units, unit_k, ldx);
         if (check_launch() != MI355_OK) return MI355_ERR_LAUNCH;
     }
-    if (act_f16) return w_bits == 4 ? launch_any<4, 1>(p, pl, s) : launch_any<8, 1>(p, pl, s);
-    return w_bits == 4 ? launch_any<4, 0>(p, pl, s) : launch_any<8, 0>(p, pl, s);
+    if (pl.k_major) return act_f16 ? launch_any<8, 1, true>(p, pl, s) : launch_any<8, 0, true>(p, pl, s);
+    if (act_f16) return w_bits == 4 ? launch_any<4, 1, false>(p, pl, s) : launch_any<8, 1, false>(p, pl, s);
+    return w_bits == 4 ? launch_any<4, 0, false>(p, pl, s) : launch_any<8, 0, false>(p, pl, s);
 }
 
 } // namespace mi355

@@ -292,15 +292,26 @@ TILED_CASES = [  # bits, M, K, N, group, float16, bias
     (4, 100, 1024, 512, 256, True, False),
     (4, 130, 512, 2048, 512, False, False),   # one group = per channel
     (4, 320, 1024, 768, 128, False, False),   # three row tiles
+    # int8 weights stored [N, K] (the transposed view that LinearWeightQuant passes, linear_weight_quant.py:106)
+    (8, 40, 1024, 384, 0, False, False, True),
+    (8, 128, 2048, 1000, 0, False, True, True),
+    (8, 200, 1024, 256, 256, False, False, True),
+    (8, 64, 8192, 256, 0, True, False, True),
 ]
 
 
-@pytest.mark.parametrize("bits,M,K,N,gs,f16,with_bias", TILED_CASES)
-def test_weight_quant_tiled_kernel(capi, golden, bits, M, K, N, gs, f16, with_bias):
+@pytest.mark.parametrize("case", TILED_CASES, ids=lambda c: "-".join(str(v) for v in c))
+def test_weight_quant_tiled_kernel(capi, golden, case):
+    bits, M, K, N, gs, f16, with_bias = case[:7]
+    nk = len(case) > 7 and case[7]
+    _tiled_case(capi, golden, bits, M, K, N, gs, f16, with_bias, nk)
+
+
+def _tiled_case(capi, golden, bits, M, K, N, gs, f16, with_bias, nk):
     """More than 32 activation rows take the tiled kernel (weights decoded once per 64/128 rows): every tile shape,
     ragged rows and strips, grouped and per-channel parameters, both activation dtypes, with and without a K split."""
     if bits == 8:
-        d = workloads.w8a16_inputs(seed=M + N, M=M, K=K, N=N)
+        d = workloads.w8a16_inputs(seed=M + N, M=M, K=K, N=N, weight_nk=nk)
         if gs:
             g = torch.Generator().manual_seed(5)
             d["antiquant_scale"] = (torch.rand(K // gs, N, generator=g) * 9e-3 + 1e-3).to(torch.bfloat16)
