@@ -27,7 +27,8 @@ BF16_PEAK_TFLOPS = 2500.0    # dense bf16 MFMA
 CACHE_BYTES = 256 << 20      # Infinity Cache
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter
 # reads for a plain 256 MiB copy (factors 2.00 and 1.00); see profiles/hbm_traffic_pmc_all_kernels.txt
-TRAFFIC_BYTES = {"c1": 25294848, "c2": 106311680, "c3": 245647360, "c4_m8": 35886080}
+TRAFFIC_BYTES = {"c1": 25296896, "c2": 106350592, "c3": 245574656, "c4_m8": 35894272, "c4_m128": 103514112,
+                 "aq_int8": 176668672}
 
 
 def _parse():
@@ -37,7 +38,7 @@ def _parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-others", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c3,c4,c5 for the 'others' section")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c3,c4,c5,aq for the 'others' section")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="launch a 256 MiB device copy and then each main kernel once on fresh buffers (for "
                          "`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: the copy calibrates the counters)")
@@ -112,6 +113,16 @@ def _pmc_pass(torch, pa, workloads, dev):
     pa.npu_weight_quant_batchmatmul(g3["x"], g3["weight"], g3["antiquant_scale"], g3["antiquant_offset"])
     pa.npu_weight_quant_batchmatmul(g4["x"], g4["weight"], g4["antiquant_scale"], g4["antiquant_offset"], None, None,
                                     None, 128)
+    # the tiled weight-only kernel (configuration 4 at M = 128) and the standalone antiquantisation, on fresh operands
+    d5 = workloads.w4a16_inputs(seed=1, M=128)
+    g5 = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d5.items()}
+    xa = torch.randint(-128, 128, (4096, 14336), dtype=torch.int8, device=dev)
+    sa = torch.rand(14336, device=dev) + 0.5
+    flush.fill_(1)
+    torch.cuda.synchronize()
+    pa.npu_weight_quant_batchmatmul(g5["x"], g5["weight"], g5["antiquant_scale"], g5["antiquant_offset"], None, None,
+                                    None, 128)
+    pa.npu_anti_quant(xa, sa, offset=sa, dst_dtype=torch.bfloat16)
     torch.cuda.synchronize()
     print(json.dumps({"pmc_pass": "done"}))
 
@@ -317,7 +328,7 @@ def main():
                      for w in ws] * 2
             us = _graph_time_us(torch, calls)
             e = hbm_entry(f"c4 W4A16 g128 x bf16[{Mx},4096] . int4[4096,14336]", nb, us,
-                          TRAFFIC_BYTES["c4_m8"] if Mx == 8 else None,
+                          TRAFFIC_BYTES["c4_m8"] if Mx == 8 else TRAFFIC_BYTES["c4_m128"] if Mx == 128 else None,
                           tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2))
             if Mx == 128:
                 tf = 2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12
@@ -379,7 +390,8 @@ def main():
             keep = []
             calls = [(lambda x=x: keep.append(pa.npu_anti_quant(x, sc_f, offset=of_f, dst_dtype=torch.bfloat16))) for x in xs] * 2
             us = _graph_time_us(torch, calls)
-            others.append(hbm_entry(f"npu_anti_quant int{bits}[4096,14336] -> bf16 (per-column float32 scale and offset)", nb, us))
+            others.append(hbm_entry(f"npu_anti_quant int{bits}[4096,14336] -> bf16 (per-column float32 scale and offset)", nb, us,
+                                    TRAFFIC_BYTES["aq_int8"] if bits == 8 else None))
             del xs, keep
 
     if others:

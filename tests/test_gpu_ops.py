@@ -165,6 +165,19 @@ def test_linear_weight_quant_module_equals_operator(pa, golden):
     via = pa.npu_weight_quant_batchmatmul(d4["x"].cuda(), d4["weight"].cuda(), m4.antiquant_scale.t(),
                                           m4.antiquant_offset.t(), None, None, None, 128)
     assert torch.equal(direct, via)
+    # a prefill-sized batch (3-D input, bias) through the module: the [N, K] weight takes the tiled kernel's K-major loader
+    d = workloads.w8a16_inputs(seed=7, M=96, K=1024, N=384, weight_nk=True)
+    mb = LinearWeightQuant(1024, 384, bias=True, antiquant_offset=True).cuda()
+    mb.weight.data = d["weight"].t().cuda()
+    mb.antiquant_scale.data = d["antiquant_scale"].cuda()
+    mb.antiquant_offset.data = d["antiquant_offset"].cuda()
+    bias = torch.randn(384, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    mb.bias.data = bias.cuda()
+    got = mb(d["x"].cuda().view(2, 48, 1024))
+    assert got.shape == (2, 48, 384)
+    _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
+                                         _bits(d["antiquant_offset"]), bias_u16=_bits(bias))
+    bf16_gate(got.view(96, 384), torch.from_numpy(gold))
 
 
 def _mlp_gpu(pa, d):
