@@ -78,7 +78,7 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
     constexpr int A_RING = 3 * A_BYTES;                        // LDS: three activation slots, two image slots, raw weight ring
     constexpr int LA = BM / 8 / NW;                            // activation loads of a wavefront per stage
     constexpr int CPL = WBITS == 4 ? 4 : 2;                    // weight columns per lane of the loader
-    constexpr int NPIECE = KM ? 2 : CPL / 2;                   // expansion steps of a lane per stage (two 16-byte chunks each... one for int8 rows)
+    constexpr int NPIECE = KM ? 2 : CPL / 2;                   // expansion steps of a lane per stage (row-major: two columns each; K-major: one 16-byte chunk each)
     constexpr int PPJ = (NPIECE + WTN - 1) / WTN;              // of which this many follow each tile column of the second half
     constexpr float P_MUL = kImageMul<WBITS, ACT>;
     constexpr float X_BIAS = kImageBias<WBITS>;
