@@ -256,6 +256,52 @@ def test_anti_quant_operator(pa, golden):
         pa.npu_anti_quant(x.cuda(), scale.cuda(), dst_dtype=torch.float32)
 
 
+def test_graph_replays_match_eager(pa):
+    """The operators launched from a captured HIP graph: every replay (with eager launches of the same operators in
+    between, which share the per-stream workspaces and their arrival counters) must reproduce the eager bits.  Covers
+    the K-split exchanges of both matmuls, the tiled weight-only kernel with its row-sum pre-kernel and the fused
+    SwiGLU quantisation."""
+    g = torch.Generator().manual_seed(11)
+    d = workloads.mlp_inputs(seed=3, M=64, hidden=1024, inter=4096)
+    x = d["x"].cuda()
+    wd, sd = d["w_down"].cuda().t(), d["scale_down"].cuda()
+    d4 = workloads.w4a16_inputs(seed=4, M=8, K=4096, N=1024, group_size=128)
+    d4b = workloads.w4a16_inputs(seed=5, M=96, K=2048, N=1024, group_size=128)
+    a4 = [d4[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset")]
+    a4b = [d4b[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset")]
+    act = torch.randn(64, 8192, generator=g).to(torch.bfloat16).cuda()
+
+    def run():
+        q, s = pa.npu_swiglu_quant(act, activate_left=True, quant_mode=1)          # [64, 4096] int8
+        o1 = pa.npu_quant_matmul(q, wd, sd, pertoken_scale=s, output_dtype=torch.bfloat16)   # narrow output: K split
+        o2 = pa.npu_weight_quant_batchmatmul(*a4, None, None, None, 128)            # streaming kernel, K split
+        o3 = pa.npu_weight_quant_batchmatmul(*a4b, None, None, None, 128)           # row sums + tiled kernel, K split
+        q1, s1 = pa.npu_dynamic_quant(x)
+        return q, s, o1, o2, o3, q1, s1
+
+    want = [t.clone() for t in run()]
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        run()                                                                      # warm-up on the capture stream
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            outs = run()
+    torch.cuda.current_stream().wait_stream(stream)
+    for it in range(4):
+        for t in outs:
+            t.zero_() if t.dtype != torch.int8 else t.fill_(7)
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, exp in zip(outs, want):
+            assert torch.equal(got, exp), f"replay {it} differs from the eager result"
+        eager = run()                                                              # eager work between the replays
+        torch.cuda.synchronize()
+        for got, exp in zip(eager, want):
+            assert torch.equal(got, exp)
+
+
 def test_c5_mlp_prefill_properties(pa, golden):
     """M = 2048: rows are independent, so any subset of rows run alone must reproduce the same bits."""
     d = workloads.mlp_inputs(seed=1, M=2048)
