@@ -121,11 +121,10 @@ int mi355_quant_matmul(const int8_t *a, const int8_t *b,
  *   out[m*ldo+n] = round( sum_k float(x[m,k]) * ((float(w[k,n]) + float(offset[g,n])) * float(scale[g,n])) + float(bias[n]) )
  *   group_size: 0 (per channel) or a multiple of 32 that divides K
  *   workspace: at least mi355_weight_quant_matmul_workspace(...) bytes (may be NULL when that is 0), 16-byte aligned.
- *              It holds the arrival counters and partial sums of a split over K and, for more than 32 rows, the
- *              per-group row sums of x that a small kernel computes ahead of the tiled kernel.  The counters lie at
- *              its start and must be zero before the first launch that uses the buffer; every launch leaves them
- *              zero, so one zero-initialised buffer can serve all later launches on the same stream.
- *   Launches: one kernel for M <= 32; two (row sums, tiled GEMM) above that.
+ *              It holds the arrival counters and partial sums of a split over K.  The counters lie at its start
+ *              and must be zero before the first launch that uses the buffer; every launch leaves them zero, so one
+ *              zero-initialised buffer can serve all later launches on the same stream.
+ *   One kernel launch per call: a weight-streaming kernel for M <= 32, a tiled GEMM above that.
  */
 size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size);
 

@@ -14,7 +14,7 @@ struct WqGemmPlan {
     int n_units;
     bool grouped, accum;     // accum: a workgroup meets more than one scale group
     bool k_major;            // int8 weights stored [N, K]
-    size_t counter_bytes, partial_bytes, rowsum_bytes;   // workspace: [arrival counters | partial sums | row sums]
+    size_t counter_bytes, partial_bytes;   // workspace when S > 1: [arrival counters | partial sums]
 };
 
 // layout 1: weight rows contiguous along N, `ldw` elements (int8 bytes / int32 words) between k rows;
@@ -24,7 +24,7 @@ __attribute__((visibility("hidden"))) WqGemmPlan make_wq_gemm_plan(int64_t M, in
                                                                    int64_t ldx, const void *x, const void *w,
                                                                    const void *scale, const void *offset);
 
-// Launches the row-sum kernel and the tiled kernel; `workspace` holds counter_bytes + partial_bytes + rowsum_bytes.
+// Launches the tiled kernel; `workspace` holds counter_bytes + partial_bytes when plan.S > 1.
 __attribute__((visibility("hidden"))) int launch_wq_gemm(const WqGemmPlan &plan, const void *x, int act_f16, const void *w,
                                                          int w_bits, const void *scale, const void *offset, const void *bias,
                                                          void *out, int64_t M, int64_t N, int64_t K, int64_t ldx,

@@ -15,8 +15,10 @@
 //     is placed between the MFMAs of a stage, so that it runs in their shadow.
 // The antiquant parameters are applied to the float32 sums per scale group exactly as in the streaming kernel:
 //     out[m,n] = sum_g scale[g,n] * ( P_g[m,n] + offset[g,n] * X_g[m] ),
-// where the row sums X_g[m] of the activations come from a small kernel that runs first (they are shared by all
-// columns; computing them per tile would cost a fifth to a third more MFMAs and sixteen accumulator registers).
+// where the row sums X_g[m] of the activations come from MFMAs against a vector of ones.  Every column tile needs the
+// same sums, so the wavefronts of a workgroup share the work: each accumulates the sums of ONE 16-row tile (one or two
+// extra MFMAs per stage and four registers instead of eight MFMAs and sixteen registers) and publishes them through
+// LDS when a group ends.
 // The weight fragment is the first MFMA operand, so a lane owns four consecutive output columns of one row.
 // K may be split over S workgroups per tile: each publishes its float32 sums in register order and the last
 // arrival adds all of them in chunk order (the result does not depend on the order of arrival).
@@ -31,7 +33,6 @@ struct WqGemmArgs {
     const void *w;
     const uint16_t *scale, *offset, *bias;
     uint16_t *out;
-    float *rowsum;                  // workspace [unit][M] float32: sums of the activations over a unit of K
     float *partial;                 // workspace [tile][chunk][wavefront][accumulator quad][lane] float32x4 (S > 1)
     uint32_t *counter;              // workspace [tile], zero on entry, left zero (S > 1)
     int64_t ldx, ldo;
@@ -40,28 +41,6 @@ struct WqGemmArgs {
     int unit_stages, n_units, grouped;
     int tiles_m, tiles_n, tiles_per_xcd, S;
 };
-
-// rowsum[u][m] = sum of x[m, u * unit_k .. (u + 1) * unit_k).  Sixteen lanes share one sum: each takes 16 bytes of
-// every 256-byte piece of the unit (coalesced), then the sixteen partial sums are added with four butterfly steps.
-template <int ACT>
-__global__ __launch_bounds__(256) void wq_rowsum_kernel(const uint16_t *__restrict__ x, float *__restrict__ rowsum, int M,
-                                                        int n_units, int unit_k, int64_t ldx)
-{
-    const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;   // which sum
-    const int sub = threadIdx.x & 15;
-    const bool valid = idx < (int64_t)M * n_units;
-    const int m = valid ? (int)(idx / n_units) : 0, u = valid ? (int)(idx % n_units) : 0;
-    const u32x4 *src = reinterpret_cast<const u32x4 *>(x + (int64_t)m * ldx + (int64_t)u * unit_k) + sub;
-    float acc = 0.0f;
-    for (int c = 0; c < unit_k / 128; c++) {
-        const u32x4 v = src[c * 16];
-#pragma unroll
-        for (int e = 0; e < 4; e++) acc += act_lo<ACT>(v[e]) + act_hi<ACT>(v[e]);
-    }
-#pragma unroll
-    for (int d = 8; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, 16);
-    if (valid && sub == 0) rowsum[(int64_t)u * M + m] = acc;
-}
 
 // KM: int8 weights stored [N, K] (K-major, the transposed view the LinearWeightQuant module passes); otherwise the
 // weight rows are contiguous along N.
@@ -206,16 +185,11 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
     // Inside the loop the parameters of a finished group travel through LDS: wavefront 0 copies the tile's BN scales and
     // offsets global -> LDS (a few load instructions for the whole workgroup instead of 2 * WTN per wavefront, and no
     // registers held across the stage); two slots, by group parity.  After the loop they are loaded into registers.
-    constexpr int PRM_SLOT = 2048;                             // [BN scales | +512: BN offsets], 16-bit each, [+1024: BM row sums] float32
+    constexpr int PRM_SLOT = 2048;                             // [BN scales | +512: BN offsets] 16-bit each, [+1024 | +1536: BM row sums] float32
     char *const prm = lds + A_RING + 2 * B_BYTES + 3 * RAW_BYTES;
-    const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(p.rowsum, (uint32_t)p.n_units * (uint32_t)p.M * 4u);
     auto issue_params = [&](int group_row) {
         const uint32_t ro = (uint32_t)group_row * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
         char *dst = prm + (group_row & 1) * PRM_SLOT;
-#pragma unroll
-        for (int h = 0; h < BM / 64; h++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_void *)(dst + 1024 + h * 256), 4, (uint32_t)lane * 4u,
-                                                     ((uint32_t)group_row * (uint32_t)p.M + (uint32_t)m0) * 4u + h * 256u, 0, 0);
 #pragma unroll
         for (int h = 0; h < BN / 128; h++) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_s, (lds_void *)(dst + h * 256), 4, (uint32_t)lane * 4u, ro + h * 256u, 0, 0);
@@ -265,6 +239,27 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
         }
     };
 
+    // ---- row sums: wavefront (wm, wn) owns 16-row tile wn % 4 of its 64 rows; with eight wavefronts across (64-row
+    // workgroup tiles) two wavefronts share a tile and take one half stage each.  acc[r] of the ones-MFMA is the sum
+    // of row lane % 16 for every r, so lanes 0..15 publish component 0.
+    constexpr int XSPLIT = WGN / 4;
+    const int xi = wn & 3, xk = wn >> 2;
+    f32x4 Xown = f32x4{0.f, 0.f, 0.f, 0.f};
+    const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
+    auto publish_x = [&](int slot) {
+        float *dst = reinterpret_cast<float *>(prm + slot * PRM_SLOT + 1024 + xk * 512) + wm * 64 + xi * 16 + (lane & 15);
+        if (lane < 16) *dst = Xown[0];
+        Xown = f32x4{0.f, 0.f, 0.f, 0.f};
+    };
+    auto read_x = [&](int slot) {
+        const float *src = reinterpret_cast<const float *>(prm + slot * PRM_SLOT + 1024) + wm * 64 + (lane & 15);
+#pragma unroll
+        for (int i = 0; i < WTM; i++) {
+            X[i] = src[i * 16];
+            if constexpr (XSPLIT == 2) X[i] = X[i] + src[128 + i * 16];
+        }
+    };
+
     // ---- fragment reads: lane reads row (lane % 16) of a 16-row tile, chunk (ks * 4 + lane / 16), stored at slot
     // chunk ^ ((row >> 1) & 7); for ks = 1 the slot is the ks = 0 slot with bit 2 flipped
     const int frow = lane & 15;
@@ -285,6 +280,14 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
         BF[0] = *reinterpret_cast<const u32x4 *>(sb_cur);
     };
     auto read_b = [&](int j) { BF[j & 1] = *reinterpret_cast<const u32x4 *>(sb_cur + j * 16 * PITCH); };
+    // this wavefront's share of the row sums for half stage ks (uniform branches: one MFMA is executed)
+    auto rowsum_mfma = [&](int ks) {
+        if (XSPLIT == 2 && xk != ks) return;
+        if (xi == 0) Xown = mfma_act<ACT>(ones, AF[0], Xown);
+        else if (xi == 1) Xown = mfma_act<ACT>(ones, AF[1], Xown);
+        else if (xi == 2) Xown = mfma_act<ACT>(ones, AF[2], Xown);
+        else Xown = mfma_act<ACT>(ones, AF[3], Xown);
+    };
 
     // ---- main loop.  Stage s is computed from activation slot s % 3 and image slot s & 1.  Meanwhile image slot
     // (s + 1) & 1 receives the images of stage s + 1, expanded from the raw ring, and memory is asked for the
@@ -324,9 +327,7 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
         __builtin_amdgcn_sched_barrier(0);
         if (ACCUM && pending) {
             const char *pb = prm + (pending_row & 1) * PRM_SLOT + prm_col;
-            const char *px = prm + (pending_row & 1) * PRM_SLOT + 1024 + (wm * 64 + frow) * 4;
-#pragma unroll
-            for (int i = 0; i < WTM; i++) X[i] = *reinterpret_cast<const float *>(px + i * 64);
+            read_x(pending_row & 1);
 #pragma unroll
             for (int j = 0; j < WTN; j++) {
                 if (j + 1 < WTN) read_b(j + 1);
@@ -347,6 +348,7 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        rowsum_mfma(0);
         __builtin_amdgcn_sched_barrier(0);
         pending = last_of_group;
         pending_row = group_row;
@@ -366,23 +368,15 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        rowsum_mfma(1);
+        if (last_of_group) publish_x(group_row & 1);           // read by everyone after the next barrier
     }
+    if constexpr (!ACCUM) publish_x(0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the refills past the end (zeros) have landed
     __syncthreads();
     // the last group (without the running total: the only one)
     load_params(p.grouped ? u1 - 1 : 0);
-    {
-        const int ufirst = ACCUM ? u1 - 1 : u0;                // without the running total: every unit of this workgroup
-#pragma unroll
-        for (int i = 0; i < WTM; i++) X[i] = 0.0f;
-        for (int u = ufirst; u < u1; u++) {
-#pragma unroll
-            for (int i = 0; i < WTM; i++) {
-                const int m = min(m0 + wm * 64 + i * 16 + frow, p.M - 1);
-                X[i] += p.rowsum[(int64_t)u * p.M + m];
-            }
-        }
-    }
+    read_x(ACCUM ? (u1 - 1) & 1 : 0);
 #pragma unroll
     for (int j = 0; j < WTN; j++) {
         fold_params(sv[j], ov[j]);
@@ -511,7 +505,7 @@ WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_
             ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 4)) &&
             (scale == nullptr || aligned(scale, 4)) && (offset == nullptr || aligned(offset, 4)) &&
             (uint64_t)128 * (uint64_t)ldx * 2 < (1ull << 31) &&
-            (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && (uint64_t)(K / 128) * (uint64_t)M * 4 < (1ull << 31) && !(off_env && off_env[0] == '0');
+            (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && !(off_env && off_env[0] == '0');
     if (!pl.ok) return pl;
     const int bn = w_bits == 4 ? 256 : 128;
     pl.bm = M <= 64 ? 64 : 128;
@@ -531,8 +525,7 @@ WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_
     pl.S = (int)S;
     pl.accum = pl.grouped && (pl.n_units + pl.S - 1) / pl.S > 1;
     pl.partial_bytes = pl.S > 1 ? (size_t)tiles * pl.S * pl.bm * bn * 4 : 0;
-    pl.counter_bytes = kWorkspaceCounterBytes;                 // the workspace always starts with the counters
-    pl.rowsum_bytes = (size_t)pl.n_units * (size_t)M * sizeof(float);
+    pl.counter_bytes = pl.S > 1 ? kWorkspaceCounterBytes : 0;
     (void)bn;
     return pl;
 }
@@ -550,7 +543,6 @@ int launch_wq_gemm(const WqGemmPlan &pl, const void *x, int act_f16, const void 
     p.out = static_cast<uint16_t *>(out);
     p.counter = pl.S > 1 ? static_cast<uint32_t *>(workspace) : nullptr;
     p.partial = pl.S > 1 ? reinterpret_cast<float *>(static_cast<char *>(workspace) + pl.counter_bytes) : nullptr;
-    p.rowsum = reinterpret_cast<float *>(static_cast<char *>(workspace) + pl.counter_bytes + pl.partial_bytes);
     p.ldx = ldx;
     p.ldo = ldo;
     p.ldw_bytes = (uint32_t)(w_bits == 4 ? ldw * 4 : ldw);
@@ -566,15 +558,6 @@ int launch_wq_gemm(const WqGemmPlan &pl, const void *x, int act_f16, const void 
     p.tiles_per_xcd = (pl.tiles_m * pl.tiles_n + 7) / 8;
     p.S = pl.S;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    {
-        const int unit_k = 64 * pl.unit_stages;
-        const unsigned blocks = (unsigned)(((int64_t)M * pl.n_units * 16 + 255) / 256);
-        if (act_f16)
-            hipLaunchKernelGGL(wq_rowsum_kernel<1>, dim3(blocks), dim3(256), 0, s, p.x, p.rowsum, p.M, pl.n_units, unit_k, ldx);
-        else
-            hipLaunchKernelGGL(wq_rowsum_kernel<0>, dim3(blocks), dim3(256), 0, s, p.x, p.rowsum, p.M, pl.n_units, unit_k, ldx);
-        if (check_launch() != MI355_OK) return MI355_ERR_LAUNCH;
-    }
     if (pl.k_major) return act_f16 ? launch_any<8, 1, true>(p, pl, s) : launch_any<8, 0, true>(p, pl, s);
     if (act_f16) return w_bits == 4 ? launch_any<4, 1, false>(p, pl, s) : launch_any<8, 1, false>(p, pl, s);
     return w_bits == 4 ? launch_any<4, 0, false>(p, pl, s) : launch_any<8, 0, false>(p, pl, s);

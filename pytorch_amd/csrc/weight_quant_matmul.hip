@@ -849,7 +849,7 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
     for (int layout = 1; layout <= (w_bits == 8 ? 2 : 1); layout++) {
         const WqGemmPlan gp = make_wq_gemm_plan(M, N, K, w_bits, group_size, layout, layout == 2 ? K : (w_bits == 4 ? N / 8 : N), K,
                                                 nullptr, nullptr, nullptr, nullptr);
-        const size_t gneed = gp.counter_bytes + gp.partial_bytes + gp.rowsum_bytes;
+        const size_t gneed = gp.counter_bytes + gp.partial_bytes;
         if (gp.ok && gneed > need) need = gneed;
     }
     if (w_bits == 8) {                      // the K-major layout may split differently
@@ -883,8 +883,10 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
         // K-major: the transposed view of an [N, K] weight
         const WqGemmPlan gk = make_wq_gemm_plan(M, N, K, 8, group_size, 2, ldw_n, ldx, x_bf16, w, scale_bf16, offset_bf16);
         if (gk.ok && aligned(out_bf16, 2) && (!bias || aligned(bias, 2))) {
-            if (!workspace || workspace_bytes < gk.counter_bytes + gk.partial_bytes + gk.rowsum_bytes) return MI355_ERR_WORKSPACE;
-            if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+            if (gk.S > 1) {
+                if (!workspace || workspace_bytes < gk.counter_bytes + gk.partial_bytes) return MI355_ERR_WORKSPACE;
+                if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+            }
             return launch_wq_gemm(gk, x_bf16, f16 ? 1 : 0, w, 8, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, ldx, ldw_n, ldo,
                                   workspace, stream);
         }
@@ -924,8 +926,10 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
     // more than 32 rows: the tiled kernel decodes every weight once per 64 or 128 rows
     const WqGemmPlan gp = make_wq_gemm_plan(M, N, K, w_bits, group_size, n_major ? 1 : 0, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
     if (gp.ok && aligned(out_bf16, 2) && (!bias || aligned(bias, 2))) {
-        if (!workspace || workspace_bytes < gp.counter_bytes + gp.partial_bytes + gp.rowsum_bytes) return MI355_ERR_WORKSPACE;
-        if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+        if (gp.S > 1) {
+            if (!workspace || workspace_bytes < gp.counter_bytes + gp.partial_bytes) return MI355_ERR_WORKSPACE;
+            if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+        }
         return launch_wq_gemm(gp, x_bf16, f16 ? 1 : 0, w, w_bits, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, ldx, ldw_k,
                               ldo, workspace, stream);
     }
