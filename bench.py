@@ -27,7 +27,7 @@ BF16_PEAK_TFLOPS = 2500.0    # dense bf16 MFMA
 CACHE_BYTES = 256 << 20      # Infinity Cache
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter
 # reads for a plain 256 MiB copy (factors 2.00 and 1.00); see profiles/hbm_traffic_pmc_all_kernels.txt
-TRAFFIC_BYTES = {"c1": 25296896, "c2": 106350592, "c3": 245574656, "c4_m8": 35894272, "c4_m128": 103514112,
+TRAFFIC_BYTES = {"c1": 25296896, "c2": 106350592, "c3": 245574656, "c4_m8": 35894272, "c4_m128": 102222080,
                  "aq_int8": 176668672}
 
 
