@@ -344,6 +344,11 @@ def _tiled_case(capi, golden, bits, M, K, N, gs, f16, with_bias, nk):
         bf16_gate(again, torch.from_numpy(gold))
     for _ in range(5):
         assert torch.equal(capi.weight_quant_matmul(*args, group_size=group, bias=None if bias is None else bias.cuda()), out)
+    # no offsets: the image bias alone is removed through the row sums
+    out0 = capi.weight_quant_matmul(args[0], args[1], args[2], None, group_size=group)
+    _, gold0 = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(d["antiquant_scale"]), None,
+                                          group_size=group, dtype="fp16" if f16 else "bf16")
+    bf16_gate(out0, torch.from_numpy(gold0))
 
 
 def test_weight_quant_exact_special_case(capi):
