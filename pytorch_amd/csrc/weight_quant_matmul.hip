@@ -722,6 +722,9 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
         }
         if (!(w_bits == 4 && pl.mt == 2 && pl.accum)) break;
     }
+    // the four-wavefront int4 kernel for two m tiles exists only with the running total (which also serves a
+    // wavefront that meets a single group)
+    if (w_bits == 4 && pl.mt == 2 && pl.w * pl.ks == 4) pl.accum = true;
     pl.partial_bytes = pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0;
     if (pl.S > 1 && (size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) {
         pl.fast = false;                              // more tiles than arrival counters

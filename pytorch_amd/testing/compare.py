@@ -6,8 +6,10 @@ only if it violates BOTH the absolute and the relative bound, and the comparison
 whole fails only if more than ``size * prec`` elements fail.
 
 ``bf16_gate`` is the acceptance gate for bf16 (and float16) outputs of this operator path:
-  * at least 99.9 % of the elements lie within one bf16 unit in the last place of the
-    float32 golden value, and
+  * at least 99.9 % of the elements lie within one unit in the last place (of the output type) of the
+    float32 golden value; for elements that cancel to almost nothing (|golden| below 1/256 of the
+    root mean square of the golden values) the unit is that of the floor magnitude, because there
+    the float32 golden itself is only accurate to a few float32 units of its much larger terms, and
   * no element fails the abs-OR-rel rule at 1e-2 (relative error measured against
     max(|a|, |b|), so values that cancel to ~0 are judged by their absolute error).
 """
@@ -63,10 +65,18 @@ def bf16_gate(out_bf16: torch.Tensor, golden_f32: torch.Tensor, *, min_within_1u
     g32 = golden_f32.detach().cpu().float()
     o = out_bf16.detach().cpu()
     dist = np.abs(_bf16_line(o) - _bf16_line(g32.to(out_bf16.dtype)))
-    within = float(np.count_nonzero(dist <= 1)) / max(dist.size, 1)
     exact = float(np.count_nonzero(dist == 0)) / max(dist.size, 1)
     of = o.float().numpy().astype(np.float64)
     gf = g32.numpy().astype(np.float64)
+    # one unit in the last place at the magnitude of the (rounded) golden value, not below the cancellation floor
+    gr = g32.to(out_bf16.dtype).float().numpy().astype(np.float64)
+    finite = np.isfinite(gr)
+    rms = float(np.sqrt(np.mean(np.square(gr[finite])))) if finite.any() else 0.0
+    mant_bits = 7 if out_bf16.dtype == torch.bfloat16 else 10
+    mag = np.maximum(np.abs(np.where(finite, gr, 0.0)), max(rms / 256.0, np.finfo(np.float64).tiny))
+    ulp = np.exp2(np.floor(np.log2(mag)) - mant_bits)
+    near = (dist <= 1) | (np.abs(of - gr) <= ulp * (1 + 1e-9))
+    within = float(np.count_nonzero(near)) / max(dist.size, 1)
     d = np.abs(of - gf)
     denom = np.maximum(np.abs(of), np.abs(gf)) + np.finfo(np.float64).tiny
     bad = int(np.count_nonzero((d > max_rel) & (d / denom > max_rel)))

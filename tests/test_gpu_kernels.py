@@ -130,6 +130,46 @@ def test_quant_matmul_bf16(capi, golden, M, K, N, bias):
     assert np.array_equal(_bits(out), want)      # same operation order => bit-identical bf16
 
 
+def test_quant_matmul_random_shapes(capi, golden):
+    """Seeded sweep over shapes (tiled, split over K, generic), weight layouts, bias kinds and output types: int32
+    accumulators and rounded outputs bit-identical to the oracle."""
+    import os
+    rng = np.random.default_rng(7)
+    for case in range(int(os.environ.get("MI355_SWEEP_CASES", "64"))):
+        M = int(rng.choice([1, 7, 16, 33, 64, 100, 128, 200, 256, 300, 513]))
+        K = int(rng.choice([16, 100, 128, 256, 384, 1024, 2048, 4096]))
+        N = int(rng.choice([8, 33, 64, 128, 200, 256, 352, 512, 1000, 1536]))
+        nk = bool(rng.random() < 0.6)
+        kind = str(rng.choice(["none", "bf16", "i32", "f32"]))
+        out_name = str(rng.choice(["bf16", "fp16", "int32"]))
+        if out_name == "int32" and kind in ("bf16", "f32"):
+            kind = "none"
+        if out_name == "fp16" and kind == "bf16":
+            kind = "f32"
+        d = workloads.quant_matmul_inputs(seed=case, M=M, K=K, N=N, weight_nk=nk, bias=True)
+        g = torch.Generator().manual_seed(case)
+        bias = {"none": None, "bf16": d["bias"], "i32": torch.randint(-(1 << 20), 1 << 20, (N,), generator=g, dtype=torch.int32),
+                "f32": torch.randn(N, generator=g)}[kind]
+        dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "int32": torch.int32}[out_name]
+        tag = f"case {case}: M={M} K={K} N={N} nk={nk} bias={kind} out={out_name}"
+        acc = golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy())
+        try:
+            if out_name == "int32":
+                out = capi.quant_matmul(d["x1"].cuda(), d["x2"].cuda(), None, None, None if bias is None else bias.cuda(),
+                                        out_dtype=dt)
+                want = acc if bias is None else (acc.astype(np.int64) + bias.numpy().astype(np.int64)).astype(np.int32)
+                assert np.array_equal(out.cpu().numpy(), want), tag
+            else:
+                out = capi.quant_matmul(d["x1"].cuda(), d["x2"].cuda(), d["scale"].cuda(), d["pertoken_scale"].cuda(),
+                                        None if bias is None else bias.cuda(), out_dtype=dt)
+                b = None if bias is None else (_bits(bias) if kind == "bf16" else bias.numpy())
+                want = golden.quant_matmul_epilogue_ex(acc, d["scale"].numpy(), d["pertoken_scale"].numpy(), b, out=out_name)
+                got = out.cpu().view(torch.int16).numpy().view(np.uint16)
+                assert np.array_equal(got, want), tag
+        except capi.Mi355Error as e:
+            raise AssertionError(f"{tag}: {e}")
+
+
 def test_quant_matmul_extreme_accumulators(capi, golden):
     M, K, N = 64, 4096, 64
     a = torch.full((M, K), 127, dtype=torch.int8)
@@ -220,7 +260,9 @@ def test_w4a16_grouped(capi, golden, M):
 
 
 def test_w4a16_other_groups_and_edges(capi, golden):
-    for (M, K, N, gs) in [(3, 512, 136, 64), (16, 256, 128, 256), (2, 1024, 8, 32), (20, 2048, 2056, 128)]:
+    # (31, 1536, 512, 128): twelve groups over four wavefronts in three K chunks - one group per wavefront, on the kernel
+    # that only exists with the running total
+    for (M, K, N, gs) in [(3, 512, 136, 64), (16, 256, 128, 256), (2, 1024, 8, 32), (20, 2048, 2056, 128), (31, 1536, 512, 128)]:
         d = workloads.w4a16_inputs(seed=K + N, M=M, K=K, N=N, group_size=gs)
         out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
                                        d["antiquant_offset"].cuda(), group_size=gs)
@@ -349,6 +391,47 @@ def _tiled_case(capi, golden, bits, M, K, N, gs, f16, with_bias, nk):
     _, gold0 = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(d["antiquant_scale"]), None,
                                           group_size=group, dtype="fp16" if f16 else "bf16")
     bf16_gate(out0, torch.from_numpy(gold0))
+
+
+def test_weight_quant_random_shapes(capi, golden):
+    """Seeded sweep over shapes, layouts, group sizes and dtypes: whichever kernel the library picks (streaming, K-major,
+    tiled, generic) must pass the gate against the oracle."""
+    import os
+    rng = np.random.default_rng(2024)
+    for case in range(int(os.environ.get("MI355_SWEEP_CASES", "96"))):
+        bits = int(rng.choice([8, 4]))
+        M = int(rng.choice([1, 3, 16, 17, 31, 32, 33, 48, 64, 65, 100, 129, 160, 257]))
+        K = int(rng.choice([32, 96, 128, 256, 384, 512, 1024, 1536]))
+        N = int(rng.choice([8, 24, 64, 128, 136, 256, 264, 512, 520, 1000, 1024]))
+        gs = 0
+        if rng.random() < 0.6 or bits == 4:
+            cands = [g for g in (32, 64, 128, 256, 512) if K % g == 0]
+            gs = int(rng.choice(cands))
+        nk = bool(bits == 8 and rng.random() < 0.4)
+        f16 = bool(rng.random() < 0.3)
+        with_off = bool(rng.random() < 0.8)
+        if bits == 8:
+            d = workloads.w8a16_inputs(seed=case, M=M, K=K, N=N, weight_nk=nk)
+            if gs:
+                g = torch.Generator().manual_seed(case)
+                d["antiquant_scale"] = (torch.rand(K // gs, N, generator=g) * 9e-3 + 1e-3).to(torch.bfloat16)
+                d["antiquant_offset"] = (torch.rand(K // gs, N, generator=g) * 8 - 4).to(torch.bfloat16)
+        else:
+            d = workloads.w4a16_inputs(seed=case, M=M, K=K, N=N, group_size=gs)
+        bits_of = _bits
+        if f16:
+            d = _to_f16(d)
+            bits_of = _f16_bits
+        off = d["antiquant_offset"] if with_off else None
+        _, gold = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(d["antiquant_scale"]),
+                                             None if off is None else bits_of(off), group_size=gs,
+                                             dtype="fp16" if f16 else "bf16")
+        try:
+            out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
+                                           None if off is None else off.cuda(), group_size=gs)
+            bf16_gate(out, torch.from_numpy(gold))
+        except (AssertionError, capi.Mi355Error) as e:
+            raise AssertionError(f"case {case}: bits={bits} M={M} K={K} N={N} gs={gs} nk={nk} f16={f16} offset={with_off}: {e}")
 
 
 def test_weight_quant_exact_special_case(capi):
