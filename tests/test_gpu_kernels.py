@@ -484,6 +484,37 @@ def test_anti_quant(capi, golden, rows, cols, packed, dst):
         assert np.array_equal(got, want)
 
 
+def test_rowwise_kernels_random_shapes(capi, golden):
+    """Seeded sweep over row counts and widths (every kernel variant: one wavefront per row, one block per row, the
+    two-pass kernel, odd widths, strided rows) for dynamic_quant with and without smooth scales, both input types, and
+    for the fused SwiGLU quantisation: codes and scales bit-identical to the oracle."""
+    import os
+    rng = np.random.default_rng(99)
+    for case in range(int(os.environ.get("MI355_SWEEP_CASES", "60"))):
+        rows = int(rng.choice([1, 2, 7, 33, 64, 129, 500]))
+        cols = int(rng.choice([1, 8, 24, 100, 512, 1000, 2048, 4096, 4104, 8192, 14336, 16384, 16392, 20000]))
+        f16 = bool(rng.random() < 0.3)
+        smooth = bool(rng.random() < 0.3)
+        strided = bool(rng.random() < 0.3)
+        g = torch.Generator().manual_seed(case)
+        dt = torch.float16 if f16 else torch.bfloat16
+        wide = (torch.randn(rows, cols + (16 if strided else 0), generator=g) * float(rng.choice([1e-3, 1.0, 30.0]))).to(dt)
+        x = wide[:, :cols]
+        sm = (torch.rand(cols, generator=g) + 0.5).to(dt) if smooth else None
+        bits = _f16_bits if f16 else _bits
+        tag = f"case {case}: rows={rows} cols={cols} f16={f16} smooth={smooth} strided={strided}"
+        y, sc = capi.dynamic_quant(x.cuda(), None if sm is None else sm.cuda())
+        wy, ws = golden.dynamic_quant(bits(x), "fp16" if f16 else "bf16", None if sm is None else bits(sm))
+        assert np.array_equal(y.cpu().numpy(), wy), tag
+        assert np.array_equal(sc.cpu().numpy().view(np.uint32), ws.view(np.uint32)), tag
+        if not f16 and not smooth and cols % 2 == 0:
+            left = bool(rng.random() < 0.5)
+            y, sc = capi.swiglu_quant(x.cuda(), activate_left=left)
+            wy, ws = golden.swiglu_quant(_bits(x), activate_left=left)
+            assert np.array_equal(sc.cpu().numpy().view(np.uint32), ws.view(np.uint32)), tag + " (swiglu_quant)"
+            assert np.array_equal(y.cpu().numpy(), wy), tag + " (swiglu_quant)"
+
+
 # ------------------------------------------------------------------ error paths (host side, no kernel runs)
 
 @pytest.mark.parametrize("rows,half", [(64, 14336), (2048, 14336), (33, 512), (5, 100), (3, 16384 + 8), (7, 24)])
