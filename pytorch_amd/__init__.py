@@ -42,3 +42,4 @@ def _export_npu_ops() -> None:
 _export_npu_ops()
 
 from . import contrib  # noqa: E402,F401
+from . import flops  # noqa: E402,F401  (registers the FLOP formulas of the matmul operators)

@@ -254,3 +254,22 @@ def test_linear_weight_quant_marshalling(pa, monkeypatch):
     assert args[1].shape == (256, 64) and args[1].stride() == (1, 256)
     assert args[2].shape == (2, 64) and args[3].shape == (2, 64)   # handed over as [G, N] views
     assert args[7] == 128 and args[8] == 0 and kwargs == {"weight_dtype": None}
+
+
+def test_flop_counter_formulas(pa):
+    """2*M*K*N for the quantised matmuls, as torch_npu/profiler/_flops_formulas.py:319-329 counts a matmul; counted on
+    meta tensors, so no kernel runs."""
+    from torch.utils.flop_counter import FlopCounterMode
+    with FlopCounterMode(display=False) as fc:
+        pa.npu_quant_matmul(_m(1024, 4096, dtype=torch.int8), _m(4096, 11008, dtype=torch.int8), _m(11008, dtype=torch.float32),
+                            pertoken_scale=_m(1024, dtype=torch.float32), output_dtype=torch.bfloat16)
+    assert fc.get_total_flops() == 2 * 1024 * 4096 * 11008
+    with FlopCounterMode(display=False) as fc:
+        pa.npu_weight_quant_batchmatmul(_m(2, 64, 4096, dtype=torch.bfloat16), _m(4096, 1792, dtype=torch.int32),
+                                        _m(32, 14336, dtype=torch.bfloat16), _m(32, 14336, dtype=torch.bfloat16), None, None,
+                                        None, 128)
+    assert fc.get_total_flops() == 2 * 128 * 4096 * 14336
+    with FlopCounterMode(display=False) as fc:
+        pa.npu_quant_matmul(_m(3, 16, 256, dtype=torch.int8), _m(256, 64, dtype=torch.int8), _m(64, dtype=torch.float32),
+                            output_dtype=torch.bfloat16)
+    assert fc.get_total_flops() == 2 * 3 * 16 * 256 * 64
