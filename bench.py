@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-inference operator path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-others] [--skip-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-others] [--skip-cpu] [--eager]
 
 A "step" is one npu_quant_matmul call on the headline configuration (W8A8, x int8
 [1024, 4096], weight int8 logical [4096, 11008] stored [N, K] and passed as its transposed
@@ -27,7 +27,7 @@ BF16_PEAK_TFLOPS = 2500.0    # dense bf16 MFMA
 CACHE_BYTES = 256 << 20      # Infinity Cache
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter
 # reads for a plain 256 MiB copy (factors 2.00 and 1.00); see profiles/hbm_traffic_pmc_all_kernels.txt
-TRAFFIC_BYTES = {"c1": 25296896, "c2": 106350592, "c3": 245574656, "c4_m8": 35894272, "c4_m128": 102222080,
+TRAFFIC_BYTES = {"c1": 25296896, "c2": 106379264, "c3": 245574656, "c4_m8": 35894272, "c4_m128": 102222080,
                  "aq_int8": 176668672}
 
 
@@ -38,6 +38,9 @@ def _parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-others", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch the timed headline steps one by one instead of from a captured graph (kernel traces:\n"
+                         "launches of a graph overlap, which blurs per-kernel durations)")
     ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c3,c4,c5,aq for the 'others' section")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="launch a 256 MiB device copy and then each main kernel once on fresh buffers (for "
@@ -173,12 +176,26 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # The K timed steps are launched from one captured HIP graph (the way a serving loop would issue them): the
+    # timed region is exactly one replay of those K launches, bracketed by synchronisation.
+    state["i"] = 0
+    graph = None
+    if not args.eager:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(args.steps):
+                step()
+        graph.replay()                               # untimed: first replay of a new graph
+        torch.cuda.synchronize()
     ev0 = torch.cuda.Event(enable_timing=True)
     ev1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
-    for _ in range(args.steps):
-        step()
+    if graph is not None:
+        graph.replay()
+    else:
+        for _ in range(args.steps):
+            step()
     ev1.record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
@@ -227,7 +244,7 @@ def main():
         "config": {"workload": "configs[1]: npu_quant_matmul x int8[1024,4096] . weight int8[4096,11008] "
                                "(stored [N,K], passed as transposed view), pertoken_scale f32[1024], scale f32[11008], "
                                "bias bf16[11008], out bf16[1024,11008]",
-                   "rotating_sets": nsets, "device": props.name, "compute_units": props.multi_processor_count,
+                   "rotating_sets": nsets, "launch": "eager" if args.eager else "one captured graph of the timed steps", "device": props.name, "compute_units": props.multi_processor_count,
                    "clock_mhz": getattr(props, "clock_rate", 0) // 1000},
         "roofline": {"bound": "mfma", "achieved": round(achieved_tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": round(achieved_tops / INT8_PEAK_TOPS, 4), "traffic": TRAFFIC_BYTES["c2"],

@@ -636,7 +636,7 @@ extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float 
     if (c.bm == bm_ && c.bn == bn_) return launch_qmm<wgm_, wgn_, bm_ / (16 * wgm_), bn_ / (16 * wgn_)>(p, s);
     MI355_QMM_CASE(256, 256, 2, 4)
     MI355_QMM_CASE(256, 224, 4, 2)
-    MI355_QMM_CASE(256, 192, 2, 4)
+    MI355_QMM_CASE(256, 192, 4, 2)
     MI355_QMM_CASE(128, 320, 2, 4)
     MI355_QMM_CASE(128, 256, 2, 4)
     MI355_QMM_CASE(128, 192, 2, 4)
