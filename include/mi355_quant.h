@@ -174,6 +174,18 @@ int mi355_anti_quant(const void *x, int x_bits, const float *scale, int64_t scal
                      int64_t offset_len, void *out, int out_dtype, int64_t rows, int64_t cols, int64_t ldx, int64_t ldo,
                      void *stream);
 
+/*
+ * Packed int4 -> int8: widens the A4W4 operands of npu_quant_matmul (both inputs int32, eight int4 values per word:
+ * test/test_fake_tensor.py:1917-1923, torch_npu/contrib/module/linear_quant.py:40-50 and :98-102) so that
+ * mi355_quant_matmul can multiply them; the int32 accumulators of the widened operands are those of the int4
+ * product.  Nibble order as in mi355_anti_quant (test/custom_ops/test_npu_anti_quant.py:12-24).
+ *
+ *   x    int32 [rows, cols/8], row pitch ldx words; word j of a row holds columns 8j..8j+7, element i in bits
+ *        [4i, 4i+3], two's complement (cols must be a multiple of 8)
+ *   out  int8 [rows, cols], row pitch ldo bytes, values in [-8, 7]
+ */
+int mi355_unpack_int4(const void *x, int8_t *out, int64_t rows, int64_t cols, int64_t ldx, int64_t ldo, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

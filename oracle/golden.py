@@ -158,6 +158,23 @@ def pack_int4(vals: np.ndarray) -> np.ndarray:
     return out
 
 
+def quant_matmul_a4w4(x1_words, x2_words, scale, pertoken_scale=None, bias=None, out: str = "bf16"):
+    """npu_quant_matmul with both operands packed int4 (test/test_fake_tensor.py:1917-1923,
+    torch_npu/contrib/module/linear_quant.py:40-50): x1 int32 [M, K/8]; x2 int32 [K, N/8] (words along N) or
+    [K/8, N] (words along K, the transposed view of a weight stored [N, K/8]), told apart by the row count.
+    The nibbles are widened (order pinned by test/custom_ops/test_npu_anti_quant.py:12-24) and the int8 path
+    runs on them -> (out [M, N], acc int32 [M, N])."""
+    a = unpack_int4(x1_words)
+    x2w = np.asarray(x2_words)
+    if x2w.shape[0] == a.shape[1]:
+        b = unpack_int4(x2w)
+    else:
+        assert x2w.shape[0] * 8 == a.shape[1], (x2w.shape, a.shape)
+        b = np.ascontiguousarray(unpack_int4(np.ascontiguousarray(x2w.T)).T)
+    acc = int8_gemm(a, b)
+    return quant_matmul_epilogue_ex(acc, scale, pertoken_scale, bias, out), acc
+
+
 def antiquant(w_i8, scale_f32, offset_f32=None) -> np.ndarray:
     w = _c(w_i8, np.int8)
     rows, cols = w.shape

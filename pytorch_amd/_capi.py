@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
 EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant",
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
-           "mi355_anti_quant")
+           "mi355_anti_quant", "mi355_unpack_int4")
 
 _lib = None
 
@@ -47,6 +47,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_swiglu.argtypes = [vp, vp, i64, i64, i64, vp]
         L.mi355_swiglu_quant.argtypes = [vp, i32, vp, vp, i64, i64, i64, vp]
         L.mi355_anti_quant.argtypes = [vp, i32, vp, i64, vp, i64, vp, i32, i64, i64, i64, i64, vp]
+        L.mi355_unpack_int4.argtypes = [vp, vp, i64, i64, i64, i64, vp]
         _lib = L
     return _lib
 
@@ -170,5 +171,17 @@ def anti_quant(x, scale, offset=None, dst_dtype=torch.float16):
     out = torch.empty((rows, cols), dtype=dst_dtype, device=x.device)
     _check(lib().mi355_anti_quant(_ptr(x), bits, _ptr(scale), scale.numel(), _ptr(offset), 0 if offset is None else offset.numel(),
                                   _ptr(out), 1 if dst_dtype == torch.float16 else 0, rows, cols, x.stride(0), cols, _stream()),
-           "mi355_anti_quant")
+           "mi355_anti_quant", "mi355_unpack_int4")
+    return out
+
+
+def unpack_int4(x, out=None):
+    """x int32 [rows, cols/8] (row pitch x.stride(0) words) -> int8 [rows, cols]; `out` may be a wider int8
+    matrix whose rows receive the result."""
+    _need_gpu(x, out)
+    rows, words = x.shape
+    if out is None:
+        out = torch.empty((rows, words * 8), dtype=torch.int8, device=x.device)
+    _check(lib().mi355_unpack_int4(_ptr(x), _ptr(out), rows, words * 8, x.stride(0), out.stride(0), _stream()),
+           "mi355_unpack_int4")
     return out

@@ -141,22 +141,38 @@ struct QmmPlan {
     std::vector<int64_t> batch;      // broadcast batch shape
     int64_t M, N, K;
     at::ScalarType out_dtype;
+    bool a4w4;                       // both inputs int32 words of eight int4 values
+    bool x2_packed_k;                // a4w4: x2 is [K/8, N] (words along K) instead of [K, N/8]
 };
 
 QmmPlan quant_matmul_plan(const Tensor &x1, const Tensor &x2, const Tensor &scale, const optional<Tensor> &offset,
                           const optional<Tensor> &pertoken_scale, const optional<Tensor> &bias,
                           optional<at::ScalarType> output_dtype)
 {
-    TORCH_CHECK(x1.scalar_type() == at::kChar && x2.scalar_type() == at::kChar,
-                "npu_quant_matmul: x1 and x2 must both be int8 (int4-packed int32 inputs are not supported), got ",
+    const bool a4w4 = x1.scalar_type() == at::kInt && x2.scalar_type() == at::kInt;
+    TORCH_CHECK(a4w4 || (x1.scalar_type() == at::kChar && x2.scalar_type() == at::kChar),
+                "npu_quant_matmul: x1 and x2 must both be int8, or both int32 holding eight int4 values per word, got ",
                 x1.scalar_type(), " and ", x2.scalar_type());
     TORCH_CHECK(x1.dim() >= 2 && x2.dim() >= 2, "npu_quant_matmul: x1 and x2 must have at least 2 dimensions");
     QmmPlan p;
+    p.a4w4 = a4w4;
+    p.x2_packed_k = false;
     p.M = x1.size(-2);
-    p.K = x1.size(-1);
+    p.K = x1.size(-1) * (a4w4 ? 8 : 1);
     p.N = x2.size(-1);
-    TORCH_CHECK(x2.size(-2) == p.K, "npu_quant_matmul: inner dimensions differ: x1 [..., ", p.M, ", ", p.K, "] x2 [..., ",
-                x2.size(-2), ", ", p.N, "]");
+    if (a4w4 && x2.size(-2) == p.K) {
+        // x2 [K, N/8]: words run along N (test/test_fake_tensor.py:1917-1923)
+        p.N = x2.size(-1) * 8;
+    } else if (a4w4) {
+        // x2 [K/8, N]: the transposed view of a weight stored [N, K/8] (linear_quant.py:40-50, :110)
+        TORCH_CHECK(x2.size(-2) * 8 == p.K, "npu_quant_matmul: int4 inner dimensions differ: x1 [..., ", p.M, ", ", x1.size(-1),
+                    "] words (K = ", p.K, ") against x2 [..., ", x2.size(-2), ", ", x2.size(-1),
+                    "] words; x2 must be [K, N/8] or [K/8, N]");
+        p.x2_packed_k = true;
+    } else {
+        TORCH_CHECK(x2.size(-2) == p.K, "npu_quant_matmul: inner dimensions differ: x1 [..., ", p.M, ", ", p.K,
+                    "] x2 [..., ", x2.size(-2), ", ", p.N, "]");
+    }
     TORCH_CHECK(output_dtype.has_value(),
                 "npu_quant_matmul: output_dtype=None selects the int8 re-quantised output, which is not supported; "
                 "pass output_dtype=torch.bfloat16, torch.float16 or torch.int32");
@@ -218,6 +234,21 @@ Tensor as_matrix(const Tensor &t)
     return (row_major || col_major) ? t : t.contiguous();
 }
 
+// int32 words of eight int4 values along the last dimension -> int8 of eight times that last dimension
+// (contiguous result; the input is made contiguous first if its rows are not)
+Tensor unpack_int4_rows(const Tensor &t)
+{
+    Tensor src = t.contiguous();
+    auto shape = src.sizes().vec();
+    const int64_t words = shape.back();
+    shape.back() = words * 8;
+    Tensor dst = at::empty(shape, src.options().dtype(at::kChar));
+    const int64_t rows = words ? src.numel() / words : 0;
+    check_status(mi355_unpack_int4(src.data_ptr(), dst.data_ptr<int8_t>(), rows, words * 8, words, words * 8, stream_of(t)),
+                 "npu_quant_matmul (int4 operands)");
+    return dst;
+}
+
 Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale, const optional<Tensor> &offset,
                         const optional<Tensor> &pertoken_scale, const optional<Tensor> &bias,
                         optional<at::ScalarType> output_dtype)
@@ -227,6 +258,12 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
     c10::hip::HIPGuardMasqueradingAsCUDA guard(x1.device());
     Tensor out = at::empty(p.out_shape, x1.options().dtype(p.out_dtype));
     if (out.numel() == 0) return out;
+    Tensor xa = x1, xb = x2;
+    if (p.a4w4) {
+        xa = unpack_int4_rows(x1);                                              // [..., M, K] int8
+        xb = p.x2_packed_k ? unpack_int4_rows(x2.transpose(-2, -1)).transpose(-2, -1)   // stored [..., N, K]
+                           : unpack_int4_rows(x2);                              // [..., K, N]
+    }
     const bool bf16 = p.out_dtype != at::kInt;            // a floating-point (dequantised) output
     Tensor scale_f, ps, b;
     if (bf16) {
@@ -242,17 +279,17 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
     for (auto d : p.batch) nb *= d;
     // x1 with batch dimensions against a single weight matrix is one tall matmul
     bool x2_single = true;
-    for (int64_t d = 0; d < x2.dim() - 2; d++) x2_single = x2_single && x2.size(d) == 1;
+    for (int64_t d = 0; d < xb.dim() - 2; d++) x2_single = x2_single && xb.size(d) == 1;
     std::vector<std::pair<Tensor, Tensor>> jobs; // (a [m,K], b [K,N]) pairs writing consecutive rows of out
     Tensor out2d = out.view({-1, p.N});
     if (x2_single) {
-        Tensor w2 = x2.dim() == 2 ? x2 : x2.as_strided({p.K, p.N}, {x2.stride(-2), x2.stride(-1)});
-        jobs.emplace_back(x1.reshape({-1, p.K}), w2);
+        Tensor w2 = xb.dim() == 2 ? xb : xb.as_strided({p.K, p.N}, {xb.stride(-2), xb.stride(-1)});
+        jobs.emplace_back(xa.reshape({-1, p.K}), w2);
     } else {
         auto x1s = p.batch, x2s = p.batch;
         x1s.push_back(p.M), x1s.push_back(p.K), x2s.push_back(p.K), x2s.push_back(p.N);
-        Tensor x1e = x1.expand(x1s).reshape({nb, p.M, p.K});
-        Tensor x2e = x2.expand(x2s);
+        Tensor x1e = xa.expand(x1s).reshape({nb, p.M, p.K});
+        Tensor x2e = xb.expand(x2s);
         x2e = x2e.reshape({nb, p.K, p.N});
         for (int64_t i = 0; i < nb; i++) jobs.emplace_back(x1e[i], x2e[i]);
     }
@@ -263,14 +300,14 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
         const int64_t m = a.size(0);
         Tensor ws;
         const size_t ws_bytes = mi355_quant_matmul_workspace(m, p.N, p.K, w.stride(0), w.stride(1));
-        if (ws_bytes) ws = zeroed_workspace(x1, ws_bytes);
+        if (ws_bytes) ws = zeroed_workspace(xa, ws_bytes);
         Tensor o = out2d.narrow(0, row0, m);
         check_status(mi355_quant_matmul(a.data_ptr<int8_t>(), w.data_ptr<int8_t>(), ps.defined() ? ps.data_ptr<float>() : nullptr,
                                         bf16 ? scale_f.data_ptr<float>() : nullptr, bf16 ? scale_f.numel() : 0,
                                         b.defined() ? b.data_ptr() : nullptr, bias_dtype, o.data_ptr(), out_dtype, m, p.N, p.K,
                                         a.stride(0), w.stride(0),
                                         w.stride(1), o.stride(0), ws.defined() ? ws.data_ptr() : nullptr, ws_bytes,
-                                        stream_of(x1)),
+                                        stream_of(xa)),
                      "npu_quant_matmul");
         row0 += m;
     }

@@ -484,6 +484,27 @@ def test_anti_quant(capi, golden, rows, cols, packed, dst):
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("rows,words,in_pad,out_pad,out_shift", [
+    (16, 8, 0, 0, 0), (64, 5, 0, 0, 0), (1024, 512, 0, 0, 0), (4096, 1376, 0, 0, 0),   # 16-byte stores / one odd word count
+    (33, 6, 1, 0, 0), (7, 3, 0, 8, 0), (9, 4, 2, 3, 0), (5, 2, 0, 0, 1), (1, 1, 0, 0, 0)])  # pitched and unaligned rows
+def test_unpack_int4(capi, golden, rows, words, in_pad, out_pad, out_shift):
+    """Packed int4 -> int8 bit-exact against the oracle's unpacking (nibble order of
+    test/custom_ops/test_npu_anti_quant.py:12-24) on random words, with pitched inputs and outputs and an output
+    that starts on an odd byte (every store width of the kernel); bytes between the rows stay untouched."""
+    g = torch.Generator().manual_seed(rows * 131 + words)
+    wide = torch.randint(-2 ** 31, 2 ** 31 - 1, (rows, words + in_pad), generator=g, dtype=torch.int64).to(torch.int32)
+    x = wide.cuda()[:, :words]
+    cols = words * 8
+    buf = torch.full((rows * (cols + out_pad) + out_shift + 16,), 99, dtype=torch.int8, device="cuda")
+    out = buf[out_shift:out_shift + rows * (cols + out_pad)].view(rows, cols + out_pad)
+    capi.unpack_int4(x, out)
+    want = golden.unpack_int4(wide[:, :words].contiguous().numpy())
+    assert want.min() >= -8 and want.max() <= 7
+    got = out.cpu().numpy()
+    assert np.array_equal(got[:, :cols], want)
+    assert (got[:, cols:] == 99).all() and (buf[:out_shift].cpu() == 99).all() and (buf[-16:].cpu() == 99).all()
+
+
 def test_rowwise_kernels_random_shapes(capi, golden):
     """Seeded sweep over row counts and widths (every kernel variant: one wavefront per row, one block per row, the
     two-pass kernel, odd widths, strided rows) for dynamic_quant with and without smooth scales, both input types, and

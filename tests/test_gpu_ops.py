@@ -256,6 +256,55 @@ def test_anti_quant_operator(pa, golden):
         pa.npu_anti_quant(x.cuda(), scale.cuda(), dst_dtype=torch.float32)
 
 
+def _rand_words(g, *shape):
+    return torch.randint(-2 ** 31, 2 ** 31 - 1, shape, generator=g, dtype=torch.int64).to(torch.int32)
+
+
+def test_quant_matmul_a4w4_operator(pa, golden):
+    """Both operands int32 words of eight int4 values: the reference's own shapes (16,8) x (64,5) -> (16,40) float16
+    with a single scale and an int32 bias (test/test_fake_tensor.py:1917-1923) and the transposed [N, K/8] weight of
+    the module example (linear_quant.py:40-50), then a larger case with every output type, a pertoken scale and a
+    batch of activations.  Accumulators bit-exact, floating outputs bit-identical to the oracle (same float32
+    operation order)."""
+    g = torch.Generator().manual_seed(5)
+    x1, x2 = _rand_words(g, 16, 8), _rand_words(g, 64, 5)
+    scale, bias = torch.rand(1, generator=g) * 0.01, torch.randint(-1000, 1000, (40,), generator=g, dtype=torch.int32)
+    out = pa.npu_quant_matmul(x1.cuda(), x2.cuda(), scale.cuda(), offset=None, bias=bias.cuda(), output_dtype=torch.float16)
+    assert out.shape == (16, 40) and out.dtype == torch.float16
+    want, acc = golden.quant_matmul_a4w4(x1.numpy(), x2.numpy(), scale.numpy(), None, bias.numpy(), out="fp16")
+    assert np.array_equal(out.cpu().view(torch.int16).numpy().view(np.uint16), want)
+    got_acc = pa.npu_quant_matmul(x1.cuda(), x2.cuda(), scale.cuda(), output_dtype=torch.int32)
+    assert np.array_equal(got_acc.cpu().numpy(), acc)
+
+    w = _rand_words(g, 128, 2)                                   # weight [N, K/8]; the module passes weight.T
+    xa = _rand_words(g, 1, 2)
+    out = pa.npu_quant_matmul(xa.cuda(), w.cuda().t(), scale.cuda(), output_dtype=torch.bfloat16)
+    assert out.shape == (1, 128)
+    want, _ = golden.quant_matmul_a4w4(xa.numpy(), w.numpy().T, scale.numpy(), out="bf16")
+    assert np.array_equal(_bits(out), want)
+
+    M, K, N = 200, 1024, 1536
+    x1, wn, wk = _rand_words(g, 3, M, K // 8), _rand_words(g, K, N // 8), _rand_words(g, N, K // 8)
+    sc, ps = torch.rand(N, generator=g) * 0.02 + 1e-3, torch.rand(M, generator=g) * 0.1 + 1e-3
+    for x2, x2_np in ((wn.cuda(), wn.numpy()), (wk.cuda().t(), wk.numpy().T)):
+        want, acc = golden.quant_matmul_a4w4(x1[1].numpy(), x2_np, sc.numpy(), ps.numpy(), None, out="bf16")
+        out = pa.npu_quant_matmul(x1[1].cuda(), x2, sc.cuda(), pertoken_scale=ps.cuda(), output_dtype=torch.bfloat16)
+        assert np.array_equal(_bits(out), want)
+        accs = pa.npu_quant_matmul(x1.cuda(), x2, sc.cuda(), output_dtype=torch.int32)      # batched activations
+        assert accs.shape == (3, M, N) and np.array_equal(accs[1].cpu().numpy(), acc)
+        assert np.array_equal(accs[2].cpu().numpy(), golden.quant_matmul_a4w4(x1[2].numpy(), x2_np, None, out="int32")[1])
+    # the module with an int32 weight [N, K/8] (linear_quant.py:40-50): same bits as the operator and the oracle
+    from pytorch_amd.contrib.module import LinearQuant
+    m = LinearQuant(K, N, bias=False, pertoken_scale=True, output_dtype=torch.bfloat16).cuda()
+    m.weight.data, m.scale.data, m.pertoken_scale.data = wk.cuda(), sc.cuda(), ps.cuda()
+    got = m(x1[1].cuda())
+    assert np.array_equal(_bits(got), golden.quant_matmul_a4w4(x1[1].numpy(), wk.numpy().T, sc.numpy(), ps.numpy(), out="bf16")[0])
+    with pytest.raises(RuntimeError, match="both be int8, or both int32"):
+        pa.npu_quant_matmul(x1[0].cuda(), torch.zeros(K, N, dtype=torch.int8, device="cuda"), sc.cuda(), output_dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="int4 inner dimensions differ"):
+        pa.npu_quant_matmul(x1[0].cuda(), wn.cuda()[:K - 8], sc.cuda(), output_dtype=torch.bfloat16)
+
+
 def test_graph_replays_match_eager(pa):
     """The operators launched from a captured HIP graph: every replay (with eager launches of the same operators in
     between, which share the per-stream workspaces and their arrival counters) must reproduce the eager bits.  Covers

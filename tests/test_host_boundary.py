@@ -16,7 +16,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def test_c_abi_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "mi355_quant.h")).read()
     declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", header))
-    assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant", "mi355_anti_quant"} <= declared
+    assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant", "mi355_anti_quant",
+            "mi355_unpack_int4"} <= declared
     lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_amd", "csrc", "libmi355_quant.so"))
     for name in declared:
         assert hasattr(lib, name), name
@@ -101,8 +102,19 @@ def test_meta_quant_matmul(pa):
     assert r.shape == (1, 1, 100) and r.dtype == torch.float16          # test_fake_tensor.py:1903-1906
     with pytest.raises(RuntimeError, match="output_dtype must be"):
         pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), output_dtype=torch.int8)
-    with pytest.raises(RuntimeError, match="int4-packed"):
-        pa.npu_quant_matmul(_m(16, 8, dtype=torch.int32), _m(64, 5, dtype=torch.int32), _m(1, dtype=torch.float32),
+    # both operands packed int4: last dimension of x2 times 8 (test_fake_tensor.py:1917-1923), or the transposed
+    # [N, K/8] weight of the module example (linear_quant.py:40-50)
+    r = pa.npu_quant_matmul(_m(16, 8, dtype=torch.int32), _m(64, 5, dtype=torch.int32), _m(1, dtype=torch.float32),
+                            offset=None, bias=_m(40, dtype=torch.int32), output_dtype=torch.float16)
+    assert r.shape == (16, 40) and r.dtype == torch.float16
+    r = pa.npu_quant_matmul(_m(1, 2, dtype=torch.int32), _m(128, 2, dtype=torch.int32).t(), _m(1, dtype=torch.float32),
+                            output_dtype=torch.bfloat16)
+    assert r.shape == (1, 128)
+    with pytest.raises(RuntimeError, match="both be int8, or both int32"):
+        pa.npu_quant_matmul(_m(16, 8, dtype=torch.int32), _m(64, 40, dtype=torch.int8), _m(1, dtype=torch.float32),
+                            output_dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="int4 inner dimensions differ"):
+        pa.npu_quant_matmul(_m(16, 8, dtype=torch.int32), _m(60, 5, dtype=torch.int32), _m(1, dtype=torch.float32),
                             output_dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="inner dimensions"):
         pa.npu_quant_matmul(_m(4, 8, dtype=torch.int8), _m(16, 4, dtype=torch.int8), _m(4, dtype=torch.float32),

@@ -119,3 +119,36 @@ def test_epilogue_ex_fp16_rounding_and_bias_kinds(golden):
     # bf16 output with a bf16 bias is the original epilogue
     bb = (rng.standard_normal(N).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
     assert np.array_equal(golden.quant_matmul_epilogue_ex(acc, sc, ps, bb, out="bf16"), golden.quant_matmul_epilogue(acc, sc, ps, bb))
+
+
+def _pack_nibbles(vals):
+    """int values in [-8, 7], last dimension a multiple of 8 -> int32 words, element i of a word in bits
+    [4i, 4i+3] (the order test/custom_ops/test_npu_anti_quant.py:12-24 unpacks), written with plain shifts."""
+    v = np.asarray(vals, dtype=np.int64) & 0xF
+    v = v.reshape(v.shape[:-1] + (v.shape[-1] // 8, 8))
+    w = np.zeros(v.shape[:-1], dtype=np.int64)
+    for i in range(8):
+        w |= v[..., i] << (4 * i)
+    return (w & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
+
+
+@pytest.mark.parametrize("words_along_k", [False, True])
+def test_a4w4_accumulator_is_the_integer_product(golden, words_along_k):
+    """Both operands packed int4: the accumulator equals numpy's int64 product of the values that were packed, for
+    x2 given as [K, N/8] and as [K/8, N]; includes the reference's own shape (16,8) x (64,5) -> (16,40), float16
+    output with a single scale and an int32 bias (test/test_fake_tensor.py:1917-1923)."""
+    rng = np.random.default_rng(11)
+    for (M, K, N) in [(16, 64, 40), (5, 128, 8), (33, 256, 72)]:
+        a = rng.integers(-8, 8, size=(M, K))
+        b = rng.integers(-8, 8, size=(K, N))
+        a[0, :8] = [-8, 7, -1, 0, 1, -7, 3, -4]                    # every sign case in one word
+        x1 = _pack_nibbles(a)
+        x2 = _pack_nibbles(b.T).T if words_along_k else _pack_nibbles(b)
+        assert x1.shape == (M, K // 8) and x2.shape == ((K // 8, N) if words_along_k else (K, N // 8))
+        scale = np.array([0.0123], np.float32)
+        bias = rng.integers(-500, 500, size=N, dtype=np.int32)
+        out, acc = golden.quant_matmul_a4w4(x1, x2, scale, None, bias, out="fp16")
+        want = a @ b
+        assert np.array_equal(acc.astype(np.int64), want)
+        ref = ((want + bias[None, :]).astype(np.float32) * scale[0]).astype(np.float16).view(np.uint16)
+        assert np.array_equal(out, ref)
