@@ -114,23 +114,31 @@ int mi355_quant_matmul(const int8_t *a, const int8_t *b,
  *           test/contrib/test_linear_weight_quant.py:57-62), element (m,k) at x[m*ldx + k]; scale, offset and out
  *           have the same element type
  *   w       w_bits == 8: int8 logical [K, N], element (k,n) at w[k*ldw_k + n*ldw_n], one stride == 1
- *           w_bits == 4: int32 [K, N/8] contiguous along N (ldw_k = N/8 words, ldw_n ignored);
- *                        word j of a row holds n = 8j..8j+7, element i in bits [4i, 4i+3], two's complement
- *   scale   [G, N] row-major, G = 1 when group_size == 0 else K / group_size
- *   offset  [G, N] or NULL;  bias [N] or NULL (the module's optional bias, linear_weight_quant.py:89-92)
+ *           w_bits == 4: int32 words of eight two's-complement int4 values, element i in bits [4i, 4i+3], either
+ *             ldw_n == 1: [K, N/8], rows ldw_k words apart; word j of row k holds n = 8j..8j+7, or
+ *             ldw_k == 1 (and ldw_n != 1): [N, K/8], columns ldw_n words apart; word j of column n holds
+ *                        k = 8j..8j+7 - the transposed view the contrib module passes (linear_weight_quant.py:71,106)
+ *   scale   element (g, n) at scale[g*ld_param_g + n*ld_param_n], G = 1 when group_size == 0 else K / group_size;
+ *           row-major [G, N] is (N, 1); the module's transposed view of [N, G] is (1, G)
+ *           (linear_weight_quant.py:98-105).  Only the kernel for words along K reads strided parameters at full
+ *           speed; every other layout falls back to a slow one-thread-per-output kernel unless they are row-major.
+ *   offset  same strides as scale, or NULL;  bias [N] or NULL (the module's optional bias, linear_weight_quant.py:89-92)
  *   out[m*ldo+n] = round( sum_k float(x[m,k]) * ((float(w[k,n]) + float(offset[g,n])) * float(scale[g,n])) + float(bias[n]) )
  *   group_size: 0 (per channel) or a multiple of 32 that divides K
  *   workspace: at least mi355_weight_quant_matmul_workspace(...) bytes (may be NULL when that is 0), 16-byte aligned.
  *              It holds the arrival counters and partial sums of a split over K.  The counters lie at its start
  *              and must be zero before the first launch that uses the buffer; every launch leaves them zero, so one
  *              zero-initialised buffer can serve all later launches on the same stream.
- *   One kernel launch per call: a weight-streaming kernel for M <= 32, a tiled GEMM above that.
+ *   One kernel launch per call: a weight-streaming kernel for M <= 32 and a tiled GEMM above that; int4 words along
+ *   K take a kernel of their own in which a wavefront owns 16 output columns for all of K (no split of K at
+ *   decode shapes).
  */
 size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size);
 
 int mi355_weight_quant_matmul(const void *x, int act_dtype, const void *w, int w_bits,
                               const void *scale, const void *offset, const void *bias, void *out,
                               int64_t M, int64_t N, int64_t K, int64_t group_size,
+                              int64_t ld_param_g, int64_t ld_param_n,
                               int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo,
                               void *workspace, size_t workspace_bytes, void *stream);
 

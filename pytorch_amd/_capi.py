@@ -43,7 +43,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_weight_quant_matmul_workspace.restype = sz
         L.mi355_weight_quant_matmul_workspace.argtypes = [i64, i64, i64, i32, i64]
         L.mi355_weight_quant_matmul.argtypes = [vp, i32, vp, i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
-                                                vp, sz, vp]
+                                                i64, i64, vp, sz, vp]
         L.mi355_swiglu.argtypes = [vp, vp, i64, i64, i64, vp]
         L.mi355_swiglu_quant.argtypes = [vp, i32, vp, vp, i64, i64, i64, vp]
         L.mi355_anti_quant.argtypes = [vp, i32, vp, i64, vp, i64, vp, i32, i64, i64, i64, i64, vp]
@@ -123,21 +123,30 @@ def _wq_workspace(device, nbytes: int):
 
 
 def weight_quant_matmul(x, weight, scale, offset=None, group_size: int = 0, bias=None):
-    """x bf16/fp16 [M,K]; weight int8 [K,N] (strides (N,1) or (1,K)) or int32 [K,N/8]; scale/offset of x's dtype, [N] or [G,N]."""
+    """x bf16/fp16 [M,K]; weight int8 [K,N] (strides (N,1) or (1,K)), int32 [K,N/8] (words along N) or int32 [K/8,N] with
+    strides (1, K/8) (words along K: the transposed view of an [N,K/8] tensor); scale/offset of x's dtype, [N] or [G,N]
+    with any strides (only the words-along-K kernel reads non-contiguous ones at full speed)."""
     _need_gpu(x, weight, scale, offset)
     M, K = x.shape
-    if weight.dtype == torch.int32:
+    if weight.dtype == torch.int32 and weight.shape[0] == K:
         bits, N = 4, weight.shape[1] * 8
         ldk, ldn = weight.stride(0), 1
+    elif weight.dtype == torch.int32:
+        assert weight.shape[0] * 8 == K and weight.stride(0) == 1, "words along K: pass the transposed view of [N, K/8]"
+        bits, N = 4, weight.shape[1]
+        ldk, ldn = 1, weight.stride(1)
     else:
         bits, N = 8, weight.shape[1]
         ldk, ldn = weight.stride(0), weight.stride(1)
+    if offset is not None:
+        assert offset.stride() == scale.stride()
+    ldg, ldp = (0, scale.stride(0)) if scale.dim() == 1 else (scale.stride(0), scale.stride(1))
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
     need = lib().mi355_weight_quant_matmul_workspace(M, N, K, bits, group_size)
     ws = _wq_workspace(x.device, need) if need else None
     st = lib().mi355_weight_quant_matmul(_ptr(x), 1 if x.dtype == torch.float16 else 0, _ptr(weight), bits, _ptr(scale),
                                          _ptr(offset), _ptr(bias), _ptr(out),
-                                         M, N, K, group_size, x.stride(0), ldk, ldn, out.stride(0), _ptr(ws),
+                                         M, N, K, group_size, ldg, ldp, x.stride(0), ldk, ldn, out.stride(0), _ptr(ws),
                                          0 if ws is None else ws.numel(), _stream())
     _check(st, "mi355_weight_quant_matmul")
     return out
@@ -171,7 +180,7 @@ def anti_quant(x, scale, offset=None, dst_dtype=torch.float16):
     out = torch.empty((rows, cols), dtype=dst_dtype, device=x.device)
     _check(lib().mi355_anti_quant(_ptr(x), bits, _ptr(scale), scale.numel(), _ptr(offset), 0 if offset is None else offset.numel(),
                                   _ptr(out), 1 if dst_dtype == torch.float16 else 0, rows, cols, x.stride(0), cols, _stream()),
-           "mi355_anti_quant", "mi355_unpack_int4")
+           "mi355_anti_quant")
     return out
 
 

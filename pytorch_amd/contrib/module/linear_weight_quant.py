@@ -3,6 +3,11 @@
 Counterpart of torch_npu/contrib/module/linear_weight_quant.py:98-109: ``weight`` is stored
 ``[out_features, in_features]`` and handed over as its transposed view; two-dimensional
 antiquant parameters (per-group, stored ``[N, G]``) are handed over transposed as well.
+
+An int4 weight is stored ``[out_features, in_features / 8]`` int32, so its transposed view holds the words along
+K; the operator has a kernel for that layout.  The layout the streaming and tiled kernels read fastest at decode
+sizes is the other one (words along N, row-major ``[G, N]`` parameters): ``prepare_()`` builds that copy once, the
+counterpart of casting a weight to the device's private format before deployment.
 """
 from __future__ import annotations
 
@@ -30,11 +35,36 @@ class LinearWeightQuant(nn.Module):
         self.inner_precise = inner_precise
         self.weight_dtype = weight_dtype
 
+    @torch.no_grad()
+    def prepare_(self) -> "LinearWeightQuant":
+        """One-time repack for inference (optional): an int4 weight is rewritten with its words along N and per-group
+        parameters are made row-major ``[G, N]``, the layout the decode kernels stream fastest.  The parameters the
+        module exposes (and its state_dict) stay as they are; the prepared copies are plain attributes, so they cost
+        the weight's size again and must be rebuilt by calling this again after the parameters change."""
+        self._prepared = None
+        if self.weight.dtype != torch.int32:
+            return self
+        w = self.weight                                             # [N, K/8], word j of a row holds k = 8j..8j+7
+        shifts = torch.arange(8, device=w.device, dtype=torch.int64) * 4
+        nib = (w.to(torch.int64).unsqueeze(-1) >> shifts) & 0xF     # [N, K/8, 8] raw nibbles
+        kn = nib.reshape(w.shape[0], -1).t().contiguous()           # [K, N]
+        words = (kn.reshape(kn.shape[0], -1, 8) << shifts).sum(-1)  # [K, N/8]: word j of a row holds n = 8j..8j+7
+        prepared_w = words.to(torch.int32)                          # wraps modulo 2**32: bit 31 becomes the sign
+        group_major = lambda t: None if t is None else self._as_group_major(t).contiguous()  # noqa: E731
+        self._prepared = (prepared_w, group_major(self.antiquant_scale), group_major(self.antiquant_offset))
+        return self
+
     @staticmethod
     def _as_group_major(param):
         return param.transpose(-1, -2) if param is not None and param.dim() == 2 else param
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        prepared = getattr(self, "_prepared", None)
+        if prepared is not None:
+            weight, scale, offset = prepared
+            return torch.ops.npu.npu_weight_quant_batchmatmul(x, weight, scale, offset, self.quant_scale, self.quant_offset,
+                                                              self.bias, self.antiquant_group_size, self.inner_precise,
+                                                              weight_dtype=self.weight_dtype)
         return torch.ops.npu.npu_weight_quant_batchmatmul(
             x, self.weight.transpose(-1, -2), self._as_group_major(self.antiquant_scale),
             self._as_group_major(self.antiquant_offset), self.quant_scale, self.quant_offset, self.bias,

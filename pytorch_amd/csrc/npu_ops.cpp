@@ -320,6 +320,7 @@ struct WqPlan {
     std::vector<int64_t> out_shape;
     int64_t M, N, K, groups;
     int bits;
+    bool packed_k;       // int4 words along K: weight [K/8, N], the transposed view of [N, K/8]
 };
 
 WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &antiquant_scale,
@@ -340,8 +341,12 @@ WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &an
     p.bits = weight.scalar_type() == at::kInt ? 4 : 8;
     p.K = x.size(-1);
     p.M = p.K ? x.numel() / p.K : 0;
-    p.N = weight.size(1) * (p.bits == 4 ? 8 : 1);
-    TORCH_CHECK(weight.size(0) == p.K, op, ": inner dimensions differ: x [..., ", p.K, "] weight [", weight.size(0), ", ...]");
+    // int4: [K, N/8] holds the words along N; [K/8, N] - what the contrib module passes, the transposed view of its
+    // [out_features, in_features/8] parameter (linear_weight_quant.py:71,106) - holds them along K
+    p.packed_k = p.bits == 4 && weight.size(0) != p.K && weight.size(0) * 8 == p.K;
+    p.N = weight.size(1) * (p.bits == 4 && !p.packed_k ? 8 : 1);
+    TORCH_CHECK(weight.size(0) == p.K || p.packed_k, op, ": inner dimensions differ: x [..., ", p.K, "] weight [", weight.size(0),
+                ", ...]", p.bits == 4 ? " (int4 weights are [K, N/8] or [K/8, N])" : "");
     TORCH_CHECK(group_size >= 0, op, ": antiquant_group_size must be >= 0");
     if (group_size > 0)
         TORCH_CHECK(p.K % group_size == 0 && group_size % 32 == 0, op,
@@ -390,10 +395,29 @@ Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &ant
     if (out.numel() == 0) return out;
     Tensor x2 = x.reshape({p.M, p.K});
     if (x2.stride(1) != 1 || x2.stride(0) < p.K) x2 = x2.contiguous();
-    Tensor w = p.bits == 4 ? (weight.stride(1) == 1 ? weight : weight.contiguous()) : as_matrix(weight);
-    // the contrib module hands 2-D parameters over as transposed views of [N, G] (linear_weight_quant.py:98-109)
-    Tensor s = antiquant_scale.contiguous(), o;
-    if (const Tensor *t = opt(antiquant_offset)) o = t->contiguous();
+    Tensor w;
+    int64_t ldw_k, ldw_n;
+    if (p.packed_k) {
+        // columns of K/8 consecutive words; a K of 8 would make both strides 1, which the C ABI reads as words along N
+        TORCH_CHECK(p.K >= 16, "npu_weight_quant_batchmatmul: int4 weights packed along K need K >= 16");
+        w = weight.stride(0) == 1 && weight.stride(1) >= weight.size(0) ? weight : weight.t().contiguous().t();
+        ldw_k = 1, ldw_n = w.stride(1);
+    } else if (p.bits == 4) {
+        w = weight.stride(1) == 1 && weight.stride(0) >= weight.size(1) ? weight : weight.contiguous();
+        ldw_k = w.stride(0), ldw_n = 1;
+    } else {
+        w = as_matrix(weight);
+        ldw_k = w.stride(0), ldw_n = w.stride(1);
+    }
+    // The contrib module hands 2-D parameters over as transposed views of [N, G] (linear_weight_quant.py:98-109).  The
+    // kernel for words along K reads them with their strides; the others want row-major [G, N].
+    Tensor s = antiquant_scale, o;
+    if (const Tensor *t = opt(antiquant_offset)) o = *t;
+    if (!p.packed_k || (o.defined() && o.strides() != s.strides())) {
+        s = s.contiguous();
+        if (o.defined()) o = o.contiguous();
+    }
+    const int64_t ld_param_g = s.dim() == 2 ? s.stride(0) : 0, ld_param_n = s.dim() == 2 ? s.stride(1) : s.stride(0);
     Tensor bias_c;
     if (const Tensor *t = opt(bias)) bias_c = t->reshape({p.N}).contiguous();
     Tensor out2d = out.view({p.M, p.N});
@@ -403,8 +427,8 @@ Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &ant
     check_status(mi355_weight_quant_matmul(x2.data_ptr(), x.scalar_type() == at::kHalf ? MI355_DTYPE_FP16 : MI355_DTYPE_BF16,
                                            w.data_ptr(), p.bits, s.data_ptr(), o.defined() ? o.data_ptr() : nullptr,
                                            bias_c.defined() ? bias_c.data_ptr() : nullptr,
-                                           out2d.data_ptr(), p.M, p.N, p.K, group_size, x2.stride(0), w.stride(0),
-                                           p.bits == 4 ? 1 : w.stride(1), out2d.stride(0),
+                                           out2d.data_ptr(), p.M, p.N, p.K, group_size, ld_param_g, ld_param_n, x2.stride(0),
+                                           ldw_k, ldw_n, out2d.stride(0),
                                            ws.defined() ? ws.data_ptr() : nullptr, ws.defined() ? (size_t)ws.numel() : 0,
                                            stream_of(x)),
                  "npu_weight_quant_batchmatmul");

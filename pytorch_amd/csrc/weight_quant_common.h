@@ -113,5 +113,125 @@ inline int env_int(const char *name)
     return e ? atoi(e) : 0;
 }
 
+struct WqArgs {
+    const uint16_t *x;              // bf16 [M, K]
+    const void *w;                  // weight rows, contiguous along N
+    const uint16_t *scale;          // bf16 [G, N]
+    const uint16_t *offset;         // bf16 [G, N] or null
+    const uint16_t *bias;           // [N] or null: added to the float32 sum before the final rounding
+    uint16_t *out;                  // bf16 [M, N]
+    float *partial;                 // workspace [S][M][N] float32 (S > 1)
+    uint32_t *counter;              // workspace [mchunks][sgroups], zero on entry, left zero
+    int64_t ldx, ldo;
+    uint32_t ldw_bytes;             // bytes between weight rows
+    uint32_t row_bytes;             // valid bytes of a weight row
+    int M, N, K;
+    int unit_steps;                 // 32-row steps per unit of K: a scale group, or one loop body per channel
+    int n_units;                    // K / (32 * unit_steps)
+    int grouped;                    // 0: one scale row for all K
+    int strips;                     // 128-byte strips of a weight row
+    int sgroups;                    // workgroup tiles along N: groups of W adjacent strips
+    int S;                          // workgroups that share the K range of a tile
+    // K-packed int4 kernel only
+    int unit_sub;                   // sub-steps of 128 k per scale group
+    int64_t ld_param_g, ld_param_n; // element strides of scale / offset: element (group, column)
+};
+
+// Output side of a workgroup tile of NBW columns whose partial sums lie in LDS as red[slice][16 rows][NBW].
+// Every thread owns quads of 4 consecutive columns.  Without a split over K the sums go straight to the output.
+// With K split over S workgroups every workgroup publishes its partial and the last arrival adds them in chunk
+// order: the exchange uses agent-scope (sc1) write-through stores and cache-bypassing loads, ordered by the
+// wavefronts' own store counters, the workgroup barrier and a relaxed agent-scope counter; a full release/acquire
+// fence would write back and invalidate the whole L2 of the XCD, which costs far more than the kernel itself.
+template <int NBW, int KS, int THREADS, int ACT>
+struct TileOut {
+    static constexpr int QPR = NBW / 4;
+    static constexpr int SC1 = 16;            // cache-policy bit: agent scope
+    const WqArgs &p;
+    char *lds;
+    const int m_base, n0, chunk;
+    const bool out_vec;
+    const uint32_t chunk_bytes;
+    const __amdgpu_buffer_rsrc_t rsrc_p;
+
+    __device__ TileOut(const WqArgs &p_, char *lds_, int m_base_, int n0_, int chunk_)
+        : p(p_), lds(lds_), m_base(m_base_), n0(n0_), chunk(chunk_), out_vec((p_.ldo & 3) == 0 && aligned_dev(p_.out, 8)),
+          chunk_bytes((uint32_t)p_.M * (uint32_t)p_.N * 4u),
+          rsrc_p(make_rsrc(p_.partial, p_.S > 1 ? (uint32_t)p_.M * (uint32_t)p_.N * 4u * (uint32_t)p_.S : 0u))
+    {
+    }
+
+    __device__ __forceinline__ void store_out(int row, int nl, f32x4 v) const
+    {
+        if (p.bias) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = v[i] + act_1<ACT>(p.bias[min(n0 + nl + i, p.N - 1)]);
+        }
+        uint16_t *o = p.out + (int64_t)(m_base + row) * p.ldo + n0 + nl;
+        if (out_vec) {
+            u32x2 pk;
+            pk.x = pack_act2<ACT>(v[0], v[1]);
+            pk.y = pack_act2<ACT>(v[2], v[3]);
+            *reinterpret_cast<u32x2 *>(o) = pk;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] = (uint16_t)pack_act2<ACT>(v[i], 0.0f);
+        }
+    }
+
+    __device__ __forceinline__ uint32_t partial_off(int row, int nl) const { return (uint32_t)(((m_base + row) * p.N + n0 + nl) * 4); }
+
+    // rows row0 .. row0+rows_mt-1 of the tile: add the slices, then store or publish
+    __device__ __forceinline__ void emit_mtile(const float *red, int row0, int rows_mt) const
+    {
+        for (int qd = threadIdx.x; qd < rows_mt * QPR; qd += THREADS) {
+            const int row = qd / QPR, nl = (qd % QPR) * 4;
+            if (n0 + nl >= p.N) continue;
+            f32x4 acc = *reinterpret_cast<const f32x4 *>(red + (size_t)row * NBW + nl);
+#pragma unroll
+            for (int ks = 1; ks < KS; ks++) acc += *reinterpret_cast<const f32x4 *>(red + ((size_t)ks * 16 + row) * NBW + nl);
+            if (p.S == 1)
+                store_out(row0 + row, nl, acc);
+            else
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), rsrc_p, partial_off(row0 + row, nl),
+                                                       (uint32_t)chunk * chunk_bytes, SC1);
+        }
+    }
+
+    // after every m tile has been emitted: meet the other K chunks of the tile
+    __device__ __forceinline__ void finish(int rows_valid, int tile) const
+    {
+        if (p.S == 1) return;
+        int &is_last = *reinterpret_cast<int *>(lds);
+        wait_vmcnt<0>();                      // this wavefront's partial sums have reached the coherence point
+        __syncthreads();
+        uint32_t *cnt = p.counter + (size_t)blockIdx.y * p.sgroups + tile;
+        if (threadIdx.x == 0) {
+            const uint32_t old = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = old == (uint32_t)(p.S - 1);
+        }
+        __syncthreads();
+        if (!is_last) return;
+        for (int qd = threadIdx.x; qd < rows_valid * QPR; qd += THREADS) {
+            const int row = qd / QPR, nl = (qd % QPR) * 4;
+            if (n0 + nl >= p.N) continue;
+            const uint32_t off = partial_off(row, nl);
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int ch = 0; ch < p.S; ch += 8) {
+                f32x4 v[8];                   // eight loads in flight
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+                    v[i] = ch + i < p.S ? __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                              rsrc_p, off, (uint32_t)(ch + i) * chunk_bytes, SC1))
+                                        : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc += v[i];
+            }
+            store_out(row, nl, acc);
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
+    }
+};
+
 } // namespace
 } // namespace mi355

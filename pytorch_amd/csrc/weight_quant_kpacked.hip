@@ -1,0 +1,416 @@
+// npu_weight_quant_batchmatmul with int4 weights packed along K: the int32 words of a column hold consecutive k
+// (storage [N, K/8]), which is what the contrib module passes - it keeps the weight [out_features, in_features/8] and
+// hands over the transposed view (torch_npu/contrib/module/linear_weight_quant.py:71,106).
+//
+// In this layout a weight row already holds consecutive k of ONE output column, the order an MFMA operand lane
+// wants: a wavefront owns 16 columns (16 weight rows) for the whole K range of its workgroup, loads them straight
+// into registers and keeps one accumulator tile per m tile.  Nothing is reduced across wavefronts, and with 16
+// columns per wavefront there are enough tiles to fill the chip without splitting K (the N-packed layout needs a
+// 32-way split of K at the same shape, and an exchange of partial sums after it).
+//
+// K advances in steps of 128 bytes per row = 256 k = two sub-steps of 128 k.  Lane (c, g) gets bytes [16g, 16g+16) of
+// both 64-byte halves of row c: 32 nibbles each, four MFMAs per half, one per dword.  The eight nibbles of a dword
+// are expanded to the exact integer image of weight_quant_common.h with two mask operations and four byte permutes,
+// which leaves them in the order 0,2,4,6,1,3,5,7; the activation fragments are staged in the same order.
+// Per scale group (a whole number of sub-steps):  out += scale_g * (P_g + offset_g * X_g), see weight_quant_matmul.hip.
+#include "weight_quant_common.h"
+#include "weight_quant_kpacked.h"
+
+namespace mi355 {
+namespace {
+
+// eight nibbles (already XORed with 8: u = w + 8) -> eight 16-bit images in the order 0,2,4,6,1,3,5,7
+template <int ACT>
+__device__ __forceinline__ u32x4 expand_word(uint32_t v)
+{
+    u32x4 b;
+    if constexpr (ACT == 0) {
+        // bf16 image 0x4100 | u << 3: the shifted nibble fills the low byte, 0x41 is the high byte
+        const uint32_t e = (v << 3) & 0x78787878u, o = (v >> 1) & 0x78787878u;
+        b[0] = __builtin_amdgcn_perm(0x41414141u, e, 0x04010400u);
+        b[1] = __builtin_amdgcn_perm(0x41414141u, e, 0x04030402u);
+        b[2] = __builtin_amdgcn_perm(0x41414141u, o, 0x04010400u);
+        b[3] = __builtin_amdgcn_perm(0x41414141u, o, 0x04030402u);
+    } else {
+        // fp16 image 0x4c00 | u << 6
+        const uint32_t e = v & 0x0f0f0f0fu, o = (v >> 4) & 0x0f0f0f0fu;
+        b[0] = (__builtin_amdgcn_perm(0u, e, 0x0c010c00u) << 6) | 0x4c004c00u;
+        b[1] = (__builtin_amdgcn_perm(0u, e, 0x0c030c02u) << 6) | 0x4c004c00u;
+        b[2] = (__builtin_amdgcn_perm(0u, o, 0x0c010c00u) << 6) | 0x4c004c00u;
+        b[3] = (__builtin_amdgcn_perm(0u, o, 0x0c030c02u) << 6) | 0x4c004c00u;
+    }
+    return b;
+}
+
+// 16-bit elements 0..7 of a 16-byte piece -> order 0,2,4,6,1,3,5,7
+__device__ __forceinline__ u32x4 even_odd(u32x4 v)
+{
+    u32x4 r;
+    r[0] = __builtin_amdgcn_perm(v[1], v[0], 0x05040100u);
+    r[1] = __builtin_amdgcn_perm(v[3], v[2], 0x05040100u);
+    r[2] = __builtin_amdgcn_perm(v[1], v[0], 0x07060302u);
+    r[3] = __builtin_amdgcn_perm(v[3], v[2], 0x07060302u);
+    return r;
+}
+
+// MT: m tiles (16 rows) per workgroup; NW: wavefronts = 16-column tiles per workgroup
+template <int MT, int NW, int ACT>
+__global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
+{
+    constexpr int NBW = NW * 16, THREADS = NW * 64;
+    constexpr int CH = 4 / MT;                          // steps per chunk of activations (32 KiB of LDS per buffer)
+    constexpr int RS = MT == 4 ? 4 : 8;                 // steps per round of the main loop: two batches of weight loads in
+    constexpr int BODY = RS / 2;                        // registers (one consumed, one in flight; 2 KiB per step and
+                                                        // wavefront), the slot of a step known at compile time
+    constexpr int POLICY = MT == 1 ? kNonTemporal : 0;
+    constexpr int XBUF = 32768;                         // bytes of one activation chunk in LDS
+    constexpr int TBUF = 2048;                          // one step of one wavefront's weights (16 rows x 128 bytes)
+    constexpr int PPR = CH * 32;                        // 16-byte pieces of an activation row per chunk
+    constexpr int PPT = 2048 / THREADS;                 // pieces per thread and chunk
+    constexpr float P_MUL = kImageMul<4, ACT>, X_BIAS = kImageBias<4>;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int xcd_slot = blockIdx.x >> 3;
+    const int tile = (blockIdx.x & 7) + 8 * (xcd_slot / p.S);
+    const int chunk = xcd_slot % p.S;
+    if (tile >= p.sgroups) return;
+    const int m_base = blockIdx.y * (MT * 16);
+    const int rows_valid = min(MT * 16, p.M - m_base);
+    const int n0 = tile * NBW;
+
+    // K range of this workgroup in steps of 256 (whole units: a unit is a whole number of steps and of scale groups)
+    const int u0 = (int)((int64_t)p.n_units * chunk / p.S), u1 = (int)((int64_t)p.n_units * (chunk + 1) / p.S);
+    const int step0 = u0 * p.unit_steps, nsteps = (u1 - u0) * p.unit_steps;
+    const int nrounds = (nsteps + RS - 1) / RS;
+    // scale groups of the range, in sub-steps of 128 k (per channel: one group that ends with the range)
+    const int gsub = p.grouped ? p.unit_sub : 2 * nsteps;
+    const int grp0 = p.grouped ? (2 * step0) / p.unit_sub : 0;
+    const int ngroups = (2 * nsteps + gsub - 1) / gsub;
+
+    // Weights: a load instruction fetches whole cache lines - lane l takes 16 bytes of row l/8 (+8 for the second
+    // load) - and the wavefront turns the step around through a private 2 KiB LDS tile into operand order.  The
+    // 16-byte chunk a lane fetches is XOR-swizzled with the row pair so that the operand reads (16 rows x 16 bytes)
+    // are free of bank conflicts; LDS slot s of row r holds chunk s ^ ((r >> 1) & 7).
+    const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(p.w, (uint32_t)((uint64_t)(p.N - 1) * p.ldw_bytes + p.row_bytes));
+    uint32_t voff_w[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int rl = 8 * h + (lane >> 3);
+        voff_w[h] = (uint32_t)min(n0 + wave * 16 + rl, p.N - 1) * p.ldw_bytes + (uint32_t)(((lane & 7) ^ ((rl >> 1) & 7)) * 16);
+    }
+    char *tbuf = lds + 16 + 2 * XBUF + wave * (2 * TBUF);
+    uint32_t *prm = reinterpret_cast<uint32_t *>(lds + 16 + 2 * XBUF + NW * 2 * TBUF);   // [group][column]: scale | offset << 16
+    const int t_rd = c * 128 + ((g ^ ((c >> 1) & 7)) * 16);   // chunk g of row c; chunk g + 4 is at slot ^ 4, i.e. +-64 bytes
+    const __amdgpu_buffer_rsrc_t rsrc_x =
+        make_rsrc(p.x + (int64_t)m_base * p.ldx, (uint32_t)(((int64_t)(rows_valid - 1) * p.ldx + p.K) * 2));
+
+    u32x4 wq[2][BODY][2];
+    auto load_body = [&](int slot, int st) {    // st: first step of the batch, relative to step0
+#pragma unroll
+        for (int j = 0; j < BODY; j++) {
+            const bool ok = st + j < nsteps;
+            const uint32_t kb = (uint32_t)(step0 + st + j) * 128u;
+            wq[slot][j][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ok ? voff_w[0] : kOutOfRange, kb, POLICY);
+            wq[slot][j][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ok ? voff_w[1] : kOutOfRange, kb, POLICY);
+        }
+    };
+    // Activation staging: piece q of a row's chunk (8 consecutive k) belongs to step q / 32, half (q % 32) / 16, lane
+    // group (q % 16) / 4 and dword q % 4 of that lane's 16 bytes; it goes to fragment (step, m tile, 4 * half + dword)
+    // at lane (group, row % 16).  Consecutive threads read consecutive pieces of a row.
+    u32x4 xst[PPT];
+    auto stage_load = [&](int ch) {
+#pragma unroll
+        for (int i = 0; i < PPT; i++) {
+            const int pid = i * THREADS + threadIdx.x;
+            const int r = pid / PPR, q = pid % PPR;
+            const bool ok = r < rows_valid && ch * CH + (q >> 5) < nsteps;
+            xst[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, ok ? (uint32_t)((r * (int)p.ldx + q * 8) * 2) : kOutOfRange,
+                                                           (uint32_t)(step0 + ch * CH) * 512u, 0);
+        }
+    };
+    auto stage_store = [&](int ch) {
+        char *buf = lds + 16 + (ch & 1) * XBUF;
+#pragma unroll
+        for (int i = 0; i < PPT; i++) {
+            const int pid = i * THREADS + threadIdx.x;
+            const int r = pid / PPR, q = pid % PPR;
+            const int sl = q >> 5, f = 4 * ((q >> 4) & 1) + (q & 3), gg = (q >> 2) & 3;
+            *reinterpret_cast<u32x4 *>(buf + ((((sl * MT + (r >> 4)) * 8 + f) * 64) + gg * 16 + (r & 15)) * 16) = even_odd(xst[i]);
+        }
+    };
+
+    f32x4 P[MT], X[MT], tot[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) P[mt] = X[mt] = tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
+    auto fold = [&](int gl) {
+        const uint32_t pr = prm[gl * NBW + wave * 16 + c];
+        const float sc = act_lo<ACT>(pr) * P_MUL;
+        const float of = (act_hi<ACT>(pr) - X_BIAS) * (1.0f / P_MUL);
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) tot[mt][q] = __builtin_fmaf(sc, __builtin_fmaf(of, X[mt][q], P[mt][q]), tot[mt][q]);
+            P[mt] = X[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+
+    // prologue: everything is requested up front - activations of chunk 0 and the antiquant parameters first (they
+    // come from cache, loads retire in order, and what the first barrier waits for must not queue behind 16 KiB of
+    // weights per wavefront), then the first two batches of weights
+    stage_load(0);
+    {
+        // parameters of the workgroup's columns and groups, any strides: walk along whichever dimension is
+        // contiguous in memory; eight loads in flight per thread, no branches (indices past the end repeat the
+        // last entry; without offsets the scale is loaded twice and masked)
+        const bool n_inner = p.ld_param_n == 1;
+        const int inner = n_inner ? NBW : ngroups, total = ngroups * NBW;
+        const uint16_t *offp = p.offset ? p.offset : p.scale;
+        const uint32_t omask = p.offset ? 0xffffu : 0u;
+        auto batch = [&](int base, bool with_weights) {
+            uint32_t sv[8], ov[8];
+            int at_lds[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int idx = min(base + i * THREADS + (int)threadIdx.x, total - 1);
+                const int a = idx % inner, b = idx / inner;
+                const int col = n_inner ? a : b, gl = n_inner ? b : a;
+                const int64_t at = (int64_t)(grp0 + gl) * p.ld_param_g + (int64_t)min(n0 + col, p.N - 1) * p.ld_param_n;
+                sv[i] = p.scale[at];
+                ov[i] = offp[at];
+                at_lds[i] = gl * NBW + col;
+            }
+            if (with_weights) {
+                __builtin_amdgcn_sched_barrier(0);
+                load_body(0, 0);
+                load_body(1, BODY);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) prm[at_lds[i]] = sv[i] | ((ov[i] & omask) << 16);
+        };
+        for (int base = 8 * THREADS; base < total; base += 8 * THREADS) batch(base, false);
+        batch(0, true);
+    }
+    stage_store(0);
+    __syncthreads();
+    // step 0 of the weights goes through the wavefront's turn-around tile into operand order
+    *reinterpret_cast<u32x4 *>(tbuf + lane * 16) = wq[0][0][0];
+    *reinterpret_cast<u32x4 *>(tbuf + 1024 + lane * 16) = wq[0][0][1];
+    u32x4 w[2];
+    w[0] = *reinterpret_cast<const u32x4 *>(tbuf + t_rd);
+    w[1] = *reinterpret_cast<const u32x4 *>(tbuf + (t_rd ^ 64));
+
+    // activation fragments of one half step (four MFMA k blocks per m tile); with one or two m tiles the next half
+    // of the same chunk is requested while the current one is multiplied
+    constexpr int XA = MT <= 2 ? 2 : 1;
+    u32x4 xa[XA][4][MT];
+    auto read_xa = [&](int buf, const char *xb, int jc, int h) {
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+                xa[buf][d][mt] = *reinterpret_cast<const u32x4 *>(xb + ((jc * MT + mt) * 8 + 4 * h + d) * 1024);
+    };
+
+    int in_group = 0, gl = 0, ch = 0;
+    for (int rd = 0; rd < nrounds; rd++) {
+#pragma unroll
+        for (int j = 0; j < RS; j++) {
+            const int st = rd * RS + j;
+            const int jc = j % CH;                          // step inside the activation chunk
+            const int slot = j / BODY, js = j % BODY;
+            if (jc == 0) stage_load(ch + 1);                // past the end: zeros, no memory traffic
+            const char *xb = lds + 16 + (ch & 1) * XBUF + lane * 16;
+            // this step's weights are in w (operand order); the next step's registers go through the other half of
+            // the turn-around tile and are read back at once, so that their latency hides behind this step
+            u32x4 wc[2];
+            wc[0] = w[0] ^ 0x88888888u;
+            wc[1] = w[1] ^ 0x88888888u;
+            {
+                const int sn = ((j + 1) / BODY) & 1, jsn = (j + 1) % BODY;
+                char *tn = tbuf + ((j + 1) & 1) * TBUF;
+                *reinterpret_cast<u32x4 *>(tn + lane * 16) = wq[sn][jsn][0];
+                *reinterpret_cast<u32x4 *>(tn + 1024 + lane * 16) = wq[sn][jsn][1];
+                w[0] = *reinterpret_cast<const u32x4 *>(tn + t_rd);
+                w[1] = *reinterpret_cast<const u32x4 *>(tn + (t_rd ^ 64));
+            }
+            if (js == BODY - 1) {               // the batch has left the registers: refill its slot two batches ahead
+                __builtin_amdgcn_sched_barrier(0);
+                load_body(slot, st + 1 + BODY);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int cur = XA == 2 ? (2 * j + h) & 1 : 0;
+                if (XA == 1 || (jc == 0 && h == 0)) read_xa(cur, xb, jc, h);
+                if (XA == 2 && !(jc == CH - 1 && h == 1)) read_xa(cur ^ 1, xb, h ? jc + 1 : jc, h ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    const u32x4 b = expand_word<ACT>(wc[h][d]);
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        P[mt] = mfma_act<ACT>(xa[cur][d][mt], b, P[mt]);
+                        X[mt] = mfma_act<ACT>(xa[cur][d][mt], ones, X[mt]);
+                    }
+                }
+                if (st < nsteps && ++in_group == gsub) {
+                    fold(gl);
+                    in_group = 0;
+                    gl++;
+                }
+            }
+            if (jc == CH - 1) {
+                stage_store(ch + 1);
+                __syncthreads();
+                ch++;
+            }
+        }
+    }
+
+    // ---- output: the wavefront's [rows x 16 columns] tile goes through LDS to the shared output / exchange code
+    float *red = reinterpret_cast<float *>(lds + 16);
+    TileOut<NBW, 1, THREADS, ACT> outp(p, lds, m_base, n0, chunk);
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const int rows_mt = min(16, rows_valid - mt * 16);
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int row = 4 * g + q;
+            if (row < rows_mt) red[row * NBW + wave * 16 + c] = tot[mt][q];
+        }
+        __syncthreads();
+        outp.emit_mtile(red, mt * 16, rows_mt);
+    }
+    outp.finish(rows_valid, tile);
+}
+
+template <int MT, int NW, int ACT>
+int launch_one(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
+{
+    auto kern = wq_kpacked_kernel<MT, NW, ACT>;
+    static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)((pl.tiles + 7) / 8 * 8 * pl.S), (unsigned)pl.mchunks), dim3(NW * 64), pl.lds_bytes, s, p);
+    return check_launch();
+}
+
+template <int ACT>
+int launch_act(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
+{
+    if (pl.nw == 4) {
+        if (pl.mt == 1) return launch_one<1, 4, ACT>(p, pl, s);
+        if (pl.mt == 2) return launch_one<2, 4, ACT>(p, pl, s);
+        return launch_one<4, 4, ACT>(p, pl, s);
+    }
+    if (pl.mt == 1) return launch_one<1, 8, ACT>(p, pl, s);
+    if (pl.mt == 2) return launch_one<2, 8, ACT>(p, pl, s);
+    return launch_one<4, 8, ACT>(p, pl, s);
+}
+
+int64_t gcd64(int64_t a, int64_t b)
+{
+    while (b) {
+        const int64_t t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
+}
+
+} // namespace
+
+WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, int64_t ldw_n, int64_t ldx, const void *x,
+                                   const void *w)
+{
+    WqKpackedPlan pl{};
+    const int64_t group = group_size > 0 ? group_size : K;
+    pl.ok = M > 0 && K > 0 && K % 256 == 0 && group % 128 == 0 && N % 8 == 0 && ldw_n >= K / 8 && ldw_n % 4 == 0 && ldx % 8 == 0 &&
+            (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 16)) &&
+            (uint64_t)N * (uint64_t)ldw_n * 4 < (1ull << 32) && (uint64_t)M * (uint64_t)ldx * 2 < (1ull << 32);
+    if (!pl.ok) return pl;
+    pl.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    if (const int f = env_int("MI355_WQK_MT"))      // tuning aid
+        if (f == 1 || f == 2 || f == 4) pl.mt = f;
+    pl.mchunks = (int)((M + pl.mt * 16 - 1) / (pl.mt * 16));
+    pl.grouped = group_size > 0 && group != K;
+    pl.unit_sub = pl.grouped ? (int)(group / 128) : 0;
+    // K may be split between workgroups at multiples of a step (256) that are also multiples of a scale group
+    const int64_t unit = pl.grouped ? group / gcd64(group, 256) * 256 : 256;
+    pl.unit_steps = (int)(unit / 256);
+    pl.n_units = (int)(K / unit);
+    if (K % unit != 0) {                  // one unit: no split
+        pl.unit_steps = (int)(K / 256);
+        pl.n_units = 1;
+    }
+    // eight wavefronts (128 columns) per workgroup when that still gives every CU a workgroup, else four
+    const int tiles8 = (int)((N + 127) / 128);
+    pl.nw = (int64_t)tiles8 * pl.mchunks >= 200 ? 8 : 4;
+    if (const int f = env_int("MI355_WQK_NW"))      // tuning aid
+        if (f == 4 || f == 8) pl.nw = f;
+    pl.tiles = (int)((N + pl.nw * 16 - 1) / (pl.nw * 16));
+    int S = kNumCU / (pl.tiles * pl.mchunks);
+    if (S > pl.n_units) S = pl.n_units;
+    if (S > 16) S = 16;
+    if (S < 1) S = 1;
+    if (const int f = env_int("MI355_WQ_SPLIT"))
+        if (f >= 1 && f <= pl.n_units) S = f;
+    if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1;
+    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) S = 1;
+    // the parameter table of a workgroup's K range must fit in LDS beside the activation chunks and turn-around tiles
+    auto lds_need = [&](int s) {
+        const int64_t units = (pl.n_units + s - 1) / s;
+        const int64_t groups = pl.grouped ? units * pl.unit_steps * 2 / pl.unit_sub : 1;
+        return (size_t)16 + 2 * 32768 + (size_t)pl.nw * 4096 + (size_t)groups * pl.nw * 16 * 4;
+    };
+    while (lds_need(S) > 160 * 1024 && S < pl.n_units && S < 16) S++;
+    if (lds_need(S) > 160 * 1024) {
+        pl.ok = false;
+        return pl;
+    }
+    pl.S = S;
+    pl.lds_bytes = lds_need(S);
+    pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
+    pl.counter_bytes = S > 1 ? kWorkspaceCounterBytes : 0;
+    return pl;
+}
+
+int launch_wq_kpacked(const WqKpackedPlan &pl, const void *x, int act_f16, const void *w, const void *scale, const void *offset,
+                      const void *bias, void *out, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw_n, int64_t ldo,
+                      int64_t ld_param_g, int64_t ld_param_n, void *workspace, void *stream)
+{
+    WqArgs p{};
+    p.x = static_cast<const uint16_t *>(x);
+    p.w = w;
+    p.scale = static_cast<const uint16_t *>(scale);
+    p.offset = static_cast<const uint16_t *>(offset);
+    p.bias = static_cast<const uint16_t *>(bias);
+    p.out = static_cast<uint16_t *>(out);
+    p.counter = pl.S > 1 ? static_cast<uint32_t *>(workspace) : nullptr;
+    p.partial = pl.S > 1 ? reinterpret_cast<float *>(static_cast<char *>(workspace) + pl.counter_bytes) : nullptr;
+    p.ldx = ldx;
+    p.ldo = ldo;
+    p.ldw_bytes = (uint32_t)(ldw_n * 4);
+    p.row_bytes = (uint32_t)(K / 2);
+    p.M = (int)M;
+    p.N = (int)N;
+    p.K = (int)K;
+    p.unit_steps = pl.unit_steps;
+    p.n_units = pl.n_units;
+    p.grouped = pl.grouped;
+    p.unit_sub = pl.unit_sub;
+    p.ld_param_g = ld_param_g;
+    p.ld_param_n = ld_param_n;
+    p.strips = pl.tiles;
+    p.sgroups = pl.tiles;
+    p.S = pl.S;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return act_f16 ? launch_act<1>(p, pl, s) : launch_act<0>(p, pl, s);
+}
+
+} // namespace mi355

@@ -38,127 +38,11 @@
 // which keeps the result independent of scheduling.
 #include "weight_quant_common.h"
 #include "weight_quant_gemm.h"
+#include "weight_quant_kpacked.h"
 #include <type_traits>
 
 namespace mi355 {
 namespace {
-
-struct WqArgs {
-    const uint16_t *x;              // bf16 [M, K]
-    const void *w;                  // weight rows, contiguous along N
-    const uint16_t *scale;          // bf16 [G, N]
-    const uint16_t *offset;         // bf16 [G, N] or null
-    const uint16_t *bias;           // [N] or null: added to the float32 sum before the final rounding
-    uint16_t *out;                  // bf16 [M, N]
-    float *partial;                 // workspace [S][M][N] float32 (S > 1)
-    uint32_t *counter;              // workspace [mchunks][sgroups], zero on entry, left zero
-    int64_t ldx, ldo;
-    uint32_t ldw_bytes;             // bytes between weight rows
-    uint32_t row_bytes;             // valid bytes of a weight row
-    int M, N, K;
-    int unit_steps;                 // 32-row steps per unit of K: a scale group, or one loop body per channel
-    int n_units;                    // K / (32 * unit_steps)
-    int grouped;                    // 0: one scale row for all K
-    int strips;                     // 128-byte strips of a weight row
-    int sgroups;                    // workgroup tiles along N: groups of W adjacent strips
-    int S;                          // workgroups that share the K range of a tile
-};
-
-// Output side of a workgroup tile of NBW columns whose partial sums lie in LDS as red[slice][16 rows][NBW].
-// Every thread owns quads of 4 consecutive columns.  Without a split over K the sums go straight to the output.
-// With K split over S workgroups every workgroup publishes its partial and the last arrival adds them in chunk
-// order: the exchange uses agent-scope (sc1) write-through stores and cache-bypassing loads, ordered by the
-// wavefronts' own store counters, the workgroup barrier and a relaxed agent-scope counter; a full release/acquire
-// fence would write back and invalidate the whole L2 of the XCD, which costs far more than the kernel itself.
-template <int NBW, int KS, int THREADS, int ACT>
-struct TileOut {
-    static constexpr int QPR = NBW / 4;
-    static constexpr int SC1 = 16;            // cache-policy bit: agent scope
-    const WqArgs &p;
-    char *lds;
-    const int m_base, n0, chunk;
-    const bool out_vec;
-    const uint32_t chunk_bytes;
-    const __amdgpu_buffer_rsrc_t rsrc_p;
-
-    __device__ TileOut(const WqArgs &p_, char *lds_, int m_base_, int n0_, int chunk_)
-        : p(p_), lds(lds_), m_base(m_base_), n0(n0_), chunk(chunk_), out_vec((p_.ldo & 3) == 0 && aligned_dev(p_.out, 8)),
-          chunk_bytes((uint32_t)p_.M * (uint32_t)p_.N * 4u),
-          rsrc_p(make_rsrc(p_.partial, p_.S > 1 ? (uint32_t)p_.M * (uint32_t)p_.N * 4u * (uint32_t)p_.S : 0u))
-    {
-    }
-
-    __device__ __forceinline__ void store_out(int row, int nl, f32x4 v) const
-    {
-        if (p.bias) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) v[i] = v[i] + act_1<ACT>(p.bias[min(n0 + nl + i, p.N - 1)]);
-        }
-        uint16_t *o = p.out + (int64_t)(m_base + row) * p.ldo + n0 + nl;
-        if (out_vec) {
-            u32x2 pk;
-            pk.x = pack_act2<ACT>(v[0], v[1]);
-            pk.y = pack_act2<ACT>(v[2], v[3]);
-            *reinterpret_cast<u32x2 *>(o) = pk;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; i++) o[i] = (uint16_t)pack_act2<ACT>(v[i], 0.0f);
-        }
-    }
-
-    __device__ __forceinline__ uint32_t partial_off(int row, int nl) const { return (uint32_t)(((m_base + row) * p.N + n0 + nl) * 4); }
-
-    // rows row0 .. row0+rows_mt-1 of the tile: add the slices, then store or publish
-    __device__ __forceinline__ void emit_mtile(const float *red, int row0, int rows_mt) const
-    {
-        for (int qd = threadIdx.x; qd < rows_mt * QPR; qd += THREADS) {
-            const int row = qd / QPR, nl = (qd % QPR) * 4;
-            if (n0 + nl >= p.N) continue;
-            f32x4 acc = *reinterpret_cast<const f32x4 *>(red + (size_t)row * NBW + nl);
-#pragma unroll
-            for (int ks = 1; ks < KS; ks++) acc += *reinterpret_cast<const f32x4 *>(red + ((size_t)ks * 16 + row) * NBW + nl);
-            if (p.S == 1)
-                store_out(row0 + row, nl, acc);
-            else
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), rsrc_p, partial_off(row0 + row, nl),
-                                                       (uint32_t)chunk * chunk_bytes, SC1);
-        }
-    }
-
-    // after every m tile has been emitted: meet the other K chunks of the tile
-    __device__ __forceinline__ void finish(int rows_valid, int tile) const
-    {
-        if (p.S == 1) return;
-        int &is_last = *reinterpret_cast<int *>(lds);
-        wait_vmcnt<0>();                      // this wavefront's partial sums have reached the coherence point
-        __syncthreads();
-        uint32_t *cnt = p.counter + (size_t)blockIdx.y * p.sgroups + tile;
-        if (threadIdx.x == 0) {
-            const uint32_t old = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            is_last = old == (uint32_t)(p.S - 1);
-        }
-        __syncthreads();
-        if (!is_last) return;
-        for (int qd = threadIdx.x; qd < rows_valid * QPR; qd += THREADS) {
-            const int row = qd / QPR, nl = (qd % QPR) * 4;
-            if (n0 + nl >= p.N) continue;
-            const uint32_t off = partial_off(row, nl);
-            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-            for (int ch = 0; ch < p.S; ch += 8) {
-                f32x4 v[8];                   // eight loads in flight
-#pragma unroll
-                for (int i = 0; i < 8; i++)
-                    v[i] = ch + i < p.S ? __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                              rsrc_p, off, (uint32_t)(ch + i) * chunk_bytes, SC1))
-                                        : f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int i = 0; i < 8; i++) acc += v[i];
-            }
-            store_out(row, nl, acc);
-        }
-        if (threadIdx.x == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
-    }
-};
 
 // One step of a wavefront: 32 weight rows of its strip (8 bytes per lane and row).
 // The loads are unconditional so that the main loop stays free of branches around memory instructions (the
@@ -616,14 +500,15 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
     outp.finish(rows_valid, tile);
 }
 
-// Any layout (including K-major int8 weights, i.e. the transposed view of an [N,K] tensor),
-// any alignment: one thread per output element, golden operation order.
+// Any layout (including K-major int8 weights, i.e. the transposed view of an [N,K] tensor, int4 words along either
+// dimension and strided parameters), any alignment: one thread per output element, golden operation order.
 __global__ __launch_bounds__(256) void wq_generic_kernel(const uint16_t *__restrict__ x, const void *__restrict__ w,
                                                          int w_bits, const uint16_t *__restrict__ scale,
                                                          const uint16_t *__restrict__ offset,
                                                          const uint16_t *__restrict__ bias,
                                                          uint16_t *__restrict__ out, int M, int N, int K, int group,
-                                                         int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo, int act)
+                                                         int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo,
+                                                         int64_t ld_param_g, int64_t ld_param_n, int kpacked, int act)
 {
     const int n = blockIdx.x * 64 + (threadIdx.x & 63);
     const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -635,13 +520,15 @@ __global__ __launch_bounds__(256) void wq_generic_kernel(const uint16_t *__restr
         if (w_bits == 8) {
             wv = (float)static_cast<const int8_t *>(w)[(int64_t)k * ldw_k + (int64_t)n * ldw_n];
         } else {
-            const uint32_t word = static_cast<const uint32_t *>(w)[(int64_t)k * ldw_k + (n >> 3)];
-            const int v = (int)((word >> (4 * (n & 7))) & 0xfu);
+            // words along N (element n & 7 of word n / 8 of row k) or along K (element k & 7 of word k / 8 of column n)
+            const uint32_t word = kpacked ? static_cast<const uint32_t *>(w)[(int64_t)n * ldw_n + (k >> 3)]
+                                          : static_cast<const uint32_t *>(w)[(int64_t)k * ldw_k + (n >> 3)];
+            const int v = (int)((word >> (4 * ((kpacked ? k : n) & 7))) & 0xfu);
             wv = (float)((v ^ 8) - 8);
         }
         auto cvt = [&](uint16_t h) { return act ? act_1<1>(h) : act_1<0>(h); };
-        if (offset) wv = wv + cvt(offset[(int64_t)gidx * N + n]);
-        wv = wv * cvt(scale[(int64_t)gidx * N + n]);
+        if (offset) wv = wv + cvt(offset[(int64_t)gidx * ld_param_g + (int64_t)n * ld_param_n]);
+        wv = wv * cvt(scale[(int64_t)gidx * ld_param_g + (int64_t)n * ld_param_n]);
         acc = acc + cvt(x[(int64_t)m * ldx + k]) * wv;
     }
     if (bias) acc = acc + (act ? act_1<1>(bias[n]) : act_1<0>(bias[n]));
@@ -855,6 +742,10 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
         const size_t gneed = gp.counter_bytes + gp.partial_bytes;
         if (gp.ok && gneed > need) need = gneed;
     }
+    if (w_bits == 4) {                      // words along K
+        const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, K / 8, K, nullptr, nullptr);
+        if (kp.ok && kp.partial_bytes + kp.counter_bytes > need) need = kp.partial_bytes + kp.counter_bytes;
+    }
     if (w_bits == 8) {                      // the K-major layout may split differently
         const WqKmPlan km = make_kmajor_plan(M, N, K, group_size, K, K, nullptr, nullptr);
         if (km.fast && km.partial_bytes + km.counter_bytes > need) need = km.partial_bytes + km.counter_bytes;
@@ -864,8 +755,9 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
 
 extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, const void *w, int w_bits, const void *scale_bf16,
                                          const void *offset_bf16, const void *bias, void *out_bf16, int64_t M, int64_t N, int64_t K,
-                                         int64_t group_size, int64_t ldx, int64_t ldw_k, int64_t ldw_n, int64_t ldo,
-                                         void *workspace, size_t workspace_bytes, void *stream)
+                                         int64_t group_size, int64_t ld_param_g, int64_t ld_param_n, int64_t ldx,
+                                         int64_t ldw_k, int64_t ldw_n, int64_t ldo, void *workspace, size_t workspace_bytes,
+                                         void *stream)
 {
     using namespace mi355;
     if (M < 0 || N < 0 || K < 0 || group_size < 0) return MI355_ERR_BAD_ARGUMENT;
@@ -875,13 +767,42 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
     if (M == 0 || N == 0) return MI355_OK;
     if (!out_bf16 || ldo < N) return MI355_ERR_BAD_ARGUMENT;
     if (K > 0 && (!x_bf16 || !w || !scale_bf16 || ldx < K)) return MI355_ERR_BAD_ARGUMENT;
-    if (w_bits == 4 && (N % 8 != 0 || ldw_k < N / 8)) return MI355_ERR_BAD_ARGUMENT;
+    // int4 words run along N (ldw_n == 1: rows of N/8 words, ldw_k words apart) or along K (ldw_k == 1: columns of K/8
+    // words, ldw_n words apart)
+    const bool kpacked = w_bits == 4 && ldw_n != 1 && ldw_k == 1;
+    if (w_bits == 4 && !kpacked && (ldw_n != 1 || N % 8 != 0 || ldw_k < N / 8)) return MI355_ERR_BAD_ARGUMENT;
+    if (kpacked && (K % 8 != 0 || ldw_n < K / 8)) return MI355_ERR_BAD_ARGUMENT;
     if (w_bits == 8 && ldw_k != 1 && ldw_n != 1) return MI355_ERR_UNSUPPORTED;
     if (group_size > 0 && (K % group_size != 0)) return MI355_ERR_BAD_ARGUMENT;
+    const int64_t n_groups = group_size > 0 && K > 0 ? K / group_size : 1;
+    if (ld_param_g < 0 || ld_param_n < 1) return MI355_ERR_BAD_ARGUMENT;
+    // every kernel but the one for K-packed int4 (and the generic one) reads [G, N] row-major parameters
+    const bool params_rowmajor = ld_param_n == 1 && (n_groups == 1 || ld_param_g == N);
     if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return MI355_ERR_UNSUPPORTED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int group = (int)(group_size > 0 ? group_size : (K > 0 ? K : 1));
 
+    const auto generic = [&]() {
+        hipLaunchKernelGGL(wq_generic_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((M + 3) / 4)), dim3(256), 0, s,
+                           static_cast<const uint16_t *>(x_bf16), w, w_bits, static_cast<const uint16_t *>(scale_bf16),
+                           static_cast<const uint16_t *>(offset_bf16), static_cast<const uint16_t *>(bias),
+                           static_cast<uint16_t *>(out_bf16), (int)M, (int)N, (int)K, group, ldx, ldw_k, ldw_n, ldo, ld_param_g,
+                           ld_param_n, kpacked ? 1 : 0, f16 ? 1 : 0);
+        return check_launch();
+    };
+    if (kpacked) {
+        const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, ldw_n, ldx, x_bf16, w);
+        const bool ptrs_ok = aligned(scale_bf16, 2) && (!offset_bf16 || aligned(offset_bf16, 2)) && aligned(out_bf16, 2) &&
+                             (!bias || aligned(bias, 2));
+        if (!kp.ok || !ptrs_ok) return generic();
+        if (kp.S > 1) {
+            if (!workspace || workspace_bytes < kp.counter_bytes + kp.partial_bytes) return MI355_ERR_WORKSPACE;
+            if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+        }
+        return launch_wq_kpacked(kp, x_bf16, f16 ? 1 : 0, w, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, ldx, ldw_n, ldo,
+                                 ld_param_g, ld_param_n, workspace, stream);
+    }
+    if (!params_rowmajor) return generic();
     if (w_bits == 8 && ldw_k == 1 && ldw_n != 1) {
         // K-major: the transposed view of an [N, K] weight
         const WqGemmPlan gk = make_wq_gemm_plan(M, N, K, 8, group_size, 2, ldw_n, ldx, x_bf16, w, scale_bf16, offset_bf16);
@@ -937,13 +858,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
                               ldo, workspace, stream);
     }
     const WqPlan pl = make_plan(M, N, K, w_bits, group_size, n_major, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
-    if (!pl.fast) {
-        hipLaunchKernelGGL(wq_generic_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((M + 3) / 4)), dim3(256), 0, s,
-                           static_cast<const uint16_t *>(x_bf16), w, w_bits, static_cast<const uint16_t *>(scale_bf16),
-                           static_cast<const uint16_t *>(offset_bf16), static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out_bf16), (int)M, (int)N,
-                           (int)K, group, ldx, ldw_k, ldw_n, ldo, f16 ? 1 : 0);
-        return check_launch();
-    }
+    if (!pl.fast) return generic();
     if (pl.S > 1) {
         if (!workspace || workspace_bytes < pl.partial_bytes + pl.counter_bytes) return MI355_ERR_WORKSPACE;
         if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;

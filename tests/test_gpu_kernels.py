@@ -393,6 +393,79 @@ def _tiled_case(capi, golden, bits, M, K, N, gs, f16, with_bias, nk):
     bf16_gate(out0, torch.from_numpy(gold0))
 
 
+KPACKED_CASES = [
+    # M, K, N, group_size, float16, parameters stored [N, G] (passed as the transposed view), bias
+    (1, 4096, 14336, 128, False, True, False),      # decode shape of the W4A16 configuration, module layout
+    (8, 4096, 14336, 128, False, False, False),
+    (32, 4096, 14336, 128, True, True, True),
+    (128, 4096, 14336, 128, False, True, False),    # four m tiles, two chunks of rows
+    (5, 512, 72, 128, False, True, True),           # ragged columns (N % 16 != 0, one partial workgroup)
+    (17, 1024, 200, 256, True, False, False),       # group of two sub-steps
+    (40, 768, 64, 384, False, True, False),         # group of three sub-steps: folds in the middle of a step
+    (3, 2048, 4096, 0, False, False, True),         # per channel, 1-D parameters
+    (70, 14336, 4096, 128, False, True, False),     # long K: K is split between workgroups, 112 groups
+    (16, 256, 16, 128, True, True, False),          # a single step, a single wavefront's worth of columns
+]
+
+
+@pytest.mark.parametrize("M,K,N,gs,f16,params_ng,with_bias", KPACKED_CASES)
+def test_weight_quant_int4_words_along_k(capi, golden, M, K, N, gs, f16, params_ng, with_bias):
+    """int4 weights stored [N, K/8] (words along K) and passed as the transposed view, the way the contrib module
+    passes its weight (linear_weight_quant.py:71,106): same values, same golden result as the [K, N/8] layout.
+    Parameters row-major [G, N] or the module's transposed [N, G]; both activation types; repeated launches and a
+    forced split of K must not change a bit."""
+    d = workloads.w4a16_inputs(seed=M + N + K, M=M, K=K, N=N, group_size=gs if gs else K)
+    if not gs:
+        d["antiquant_scale"], d["antiquant_offset"] = d["antiquant_scale"][0].clone(), d["antiquant_offset"][0].clone()
+    bits_of = _bits
+    if f16:
+        d = _to_f16(d)
+        bits_of = _f16_bits
+    w_nk = torch.from_numpy(golden.pack_int4(np.ascontiguousarray(d["weight_int4_values"].numpy().T)))   # [N, K/8]
+    assert w_nk.shape == (N, K // 8)
+    bias = torch.randn(N, generator=torch.Generator().manual_seed(1)).to(d["x"].dtype) if with_bias else None
+    sc, of = d["antiquant_scale"], d["antiquant_offset"]
+    if params_ng and gs:
+        sc_dev, of_dev = sc.t().contiguous().cuda().t(), of.t().contiguous().cuda().t()
+        assert sc_dev.stride() == (1, K // gs)
+    else:
+        sc_dev, of_dev = sc.cuda(), of.cuda()
+    x, w = d["x"].cuda(), w_nk.cuda().t()
+    call = lambda off=of_dev: capi.weight_quant_matmul(x, w, sc_dev, off, group_size=gs, bias=None if bias is None else bias.cuda())
+    out = call()
+    kw = dict(group_size=gs, dtype="fp16" if f16 else "bf16")
+    _, gold = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(sc), bits_of(of),
+                                         bias_u16=None if bias is None else bits_of(bias), **kw)
+    print("kpacked", M, K, N, gs, bf16_gate(out, torch.from_numpy(gold)))
+    for _ in range(3):
+        assert torch.equal(call(), out)
+    import os
+    for split in ("1", "2", "3"):
+        os.environ["MI355_WQ_SPLIT"] = split
+        try:
+            bf16_gate(call(), torch.from_numpy(gold))
+        finally:
+            del os.environ["MI355_WQ_SPLIT"]
+    assert torch.equal(call(), out)
+    out0 = call(None)
+    _, gold0 = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(sc), None,
+                                          bias_u16=None if bias is None else bits_of(bias), **kw)
+    bf16_gate(out0, torch.from_numpy(gold0))
+
+
+def test_weight_quant_int4_words_along_k_generic_fallback(capi, golden):
+    """Shapes the fast kernel does not take (K not a multiple of 256, a group of 32) go to the one-thread-per-output
+    kernel, which reads the same layout and strided parameters."""
+    for (M, K, N, gs) in [(3, 128, 24, 32), (2, 384, 40, 128)]:
+        d = workloads.w4a16_inputs(seed=K, M=M, K=K, N=N, group_size=gs)
+        w_nk = torch.from_numpy(golden.pack_int4(np.ascontiguousarray(d["weight_int4_values"].numpy().T)))
+        sc, of = d["antiquant_scale"], d["antiquant_offset"]
+        out = capi.weight_quant_matmul(d["x"].cuda(), w_nk.cuda().t(), sc.t().contiguous().cuda().t(),
+                                       of.t().contiguous().cuda().t(), group_size=gs)
+        _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(sc), _bits(of), group_size=gs)
+        bf16_gate(out, torch.from_numpy(gold))
+
+
 def test_weight_quant_random_shapes(capi, golden):
     """Seeded sweep over shapes, layouts, group sizes and dtypes: whichever kernel the library picks (streaming, K-major,
     tiled, generic) must pass the gate against the oracle."""
@@ -558,8 +631,8 @@ def test_c_abi_rejects_bad_arguments(capi):
     assert L.mi355_dynamic_quant(None, 0, None, None, None, -1, 8, 8, None) == -1
     assert L.mi355_dynamic_quant(None, 7, None, None, None, 1, 8, 8, None) == -1
     assert L.mi355_quant_matmul(None, None, None, None, 0, None, 0, None, 0, 4, 4, 4, 4, 4, 1, 4, None, 0, None) == -1
-    assert L.mi355_weight_quant_matmul(None, 0, None, 5, None, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
-    assert L.mi355_weight_quant_matmul(None, 9, None, 8, None, None, None, None, 1, 8, 32, 0, 32, 8, 1, 8, None, 0, None) == -1
+    assert L.mi355_weight_quant_matmul(None, 0, None, 5, None, None, None, None, 1, 8, 32, 0, 8, 1, 32, 8, 1, 8, None, 0, None) == -1
+    assert L.mi355_weight_quant_matmul(None, 9, None, 8, None, None, None, None, 1, 8, 32, 0, 8, 1, 32, 8, 1, 8, None, 0, None) == -1
     assert L.mi355_anti_quant(None, 5, None, 1, None, 0, None, 0, 1, 8, 8, 8, None) == -1
     assert L.mi355_anti_quant(None, 4, None, 1, None, 0, None, 7, 1, 8, 1, 8, None) == -1
     assert b"workspace" in L.mi355_status_string(-4)

@@ -180,6 +180,36 @@ def test_linear_weight_quant_module_equals_operator(pa, golden):
     bf16_gate(got.view(96, 384), torch.from_numpy(gold))
 
 
+def test_linear_weight_quant_module_int4(pa, golden):
+    """The module with an int4 weight stored [out_features, in_features / 8] int32 and per-group parameters stored
+    [N, G] (linear_weight_quant.py:71,98-109): its transposed views reach the kernel for words along K without a copy;
+    after prepare_() the same module runs on the repacked copy (words along N).  Both against the oracle."""
+    from pytorch_amd.contrib.module import LinearWeightQuant
+    for (M, K, N, f16) in [(4, 512, 128, False), (48, 1024, 384, True), (8, 4096, 2048, False)]:
+        d = workloads.w4a16_inputs(seed=M + N, M=M, K=K, N=N, group_size=128)
+        dt = torch.float16 if f16 else torch.bfloat16
+        m = LinearWeightQuant(K, N, bias=True, antiquant_offset=True, antiquant_group_size=128).cuda()
+        w_nk = torch.from_numpy(golden.pack_int4(np.ascontiguousarray(d["weight_int4_values"].numpy().T)))
+        sc, of = d["antiquant_scale"].to(dt), d["antiquant_offset"].to(dt)
+        bias = torch.randn(N, generator=torch.Generator().manual_seed(2)).to(dt)
+        m.weight.data = w_nk.cuda()
+        m.antiquant_scale.data, m.antiquant_offset.data = sc.t().contiguous().cuda(), of.t().contiguous().cuda()
+        m.bias.data = bias.cuda()
+        x = d["x"].to(dt)
+        bits = (lambda t: t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16))
+        _, gold = golden.weight_quant_matmul(bits(x), d["weight"].numpy(), bits(sc), bits(of), group_size=128,
+                                             dtype="fp16" if f16 else "bf16", bias_u16=bits(bias))
+        got = m(x.cuda())
+        assert got.shape == (M, N) and got.dtype == dt
+        bf16_gate(got, torch.from_numpy(gold))
+        m.prepare_()
+        assert m._prepared[0].shape == (K, N // 8) and torch.equal(m._prepared[0].cpu(), d["weight"])
+        assert m.weight.shape == (N, K // 8)                       # the parameter itself is untouched
+        bf16_gate(m(x.cuda()), torch.from_numpy(gold))
+    with pytest.raises(RuntimeError, match="inner dimensions differ"):
+        pa.npu_weight_quant_batchmatmul(x.cuda(), w_nk.cuda()[:, :-1].t(), sc.cuda(), of.cuda(), None, None, None, 128)
+
+
 def _mlp_gpu(pa, d):
     x = d["x"].cuda()
     xq, xs = pa.npu_dynamic_quant(x)

@@ -23,7 +23,7 @@ def test_c_abi_exports_every_declared_symbol():
         assert hasattr(lib, name), name
     lib.mi355_status_string.restype = ctypes.c_char_p
     assert lib.mi355_status_string(0) == b"ok"
-    assert lib.mi355_quant_abi_version() >= 1000
+    assert lib.mi355_quant_abi_version() >= 2000
     from pytorch_amd import _capi
     assert set(_capi.EXPORTS) == declared
 
@@ -143,6 +143,14 @@ def test_meta_weight_quant_batchmatmul(pa):
     sg, og = _m(32, 14336, dtype=torch.bfloat16), _m(32, 14336, dtype=torch.bfloat16)
     r = pa.npu_weight_quant_batchmatmul(_m(2, 4, 4096, dtype=torch.bfloat16), w4, sg, og, None, None, None, 128)
     assert r.shape == (2, 4, 14336) and r.dtype == torch.bfloat16
+    # the module's int4 weight [N, K/8] arrives as the transposed view [K/8, N]: words along K (linear_weight_quant.py:71,106)
+    w4k = _m(14336, 512, dtype=torch.int32).t()
+    r = pa.npu_weight_quant_batchmatmul(_m(3, 4096, dtype=torch.bfloat16), w4k, _m(14336, 32, dtype=torch.bfloat16).t(),
+                                        _m(14336, 32, dtype=torch.bfloat16).t(), None, None, None, 128)
+    assert r.shape == (3, 14336)
+    with pytest.raises(RuntimeError, match="inner dimensions differ"):
+        pa.npu_weight_quant_batchmatmul(_m(3, 4096, dtype=torch.bfloat16), _m(500, 14336, dtype=torch.int32), sg, og, None, None,
+                                        None, 128)
     xs = _m(1, 4096, dtype=torch.bfloat16)
     for kwargs, pat in [(dict(quant_scale=_m(14336, dtype=torch.float32)), "quant_scale"),
                         (dict(bias=_m(14336, dtype=torch.float16)), "bias must have the dtype of x"),
