@@ -41,7 +41,7 @@ def _parse():
     ap.add_argument("--eager", action="store_true",
                     help="launch the timed headline steps one by one instead of from a captured graph (kernel traces:\n"
                          "launches of a graph overlap, which blurs per-kernel durations)")
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c3,c4,c5,aq for the 'others' section")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c3,c4,a4w4,c5,aq for the 'others' section")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="launch a 256 MiB device copy and then each main kernel once on fresh buffers (for "
                          "`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: the copy calibrates the counters)")
@@ -353,6 +353,36 @@ def main():
                                       "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4), "traffic": None}
             others.append(e)
             del ws, keep
+            # the layout torch_npu's LinearWeightQuant passes: weight stored [N, K/8] (words along K), per-group
+            # parameters stored [N, G], all three given as transposed views
+            wks = [torch.randint(-2 ** 31, 2 ** 31 - 1, (Nx, Kx // 8), generator=gen, dtype=torch.int32, device=dev).t()
+                   for _ in range(ns)]
+            s4t, o4t = s4.t().contiguous().t(), o4.t().contiguous().t()
+            keep = []
+            calls = [(lambda w=w: keep.append(pa.npu_weight_quant_batchmatmul(x, w, s4t, o4t, None, None, None, 128)))
+                     for w in wks] * 2
+            us = _graph_time_us(torch, calls)
+            others.append(hbm_entry(f"c4 W4A16 g128 x bf16[{Mx},4096] . int4 stored [14336,4096/8] (words along K, parameters "
+                                    "[N,G]: the module's transposed views)", nb, us, None,
+                                    tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2)))
+            del wks, keep
+
+    if want("a4w4"):
+        # both operands packed int4 (A4W4) at the headline shape: the operator widens them to int8 and runs the int8 GEMM
+        Mx, Kx, Nx = 1024, 4096, 11008
+        rnd = lambda *sh: torch.randint(-2 ** 31, 2 ** 31 - 1, sh, generator=gen, dtype=torch.int32, device=dev)  # noqa: E731
+        nb = Mx * Kx // 2 + Kx * Nx // 2 + Mx * Nx * 2
+        xs, wsk = [rnd(Mx, Kx // 8) for _ in range(4)], [rnd(Nx, Kx // 8).t() for _ in range(4)]
+        sc = torch.rand(Nx, generator=gen, device=dev) * 1e-2
+        ps = torch.rand(Mx, generator=gen, device=dev) * 1e-2
+        keep = []
+        calls = [(lambda a=a, w=w: keep.append(pa.npu_quant_matmul(a, w, sc, pertoken_scale=ps, output_dtype=torch.bfloat16)))
+                 for a, w in zip(xs, wsk)] * 4
+        us = _graph_time_us(torch, calls, reps=10)
+        others.append({"name": "a4w4 quant_matmul int4[1024,4096] . int4 stored [11008,4096/8] -> bf16 (unpack kernels + int8 GEMM)",
+                       "us": round(us, 2), "tops": round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 1),
+                       "frac_int8_peak": round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4)})
+        del xs, wsk, keep
 
     if want("c5"):
         H, I = 4096, 14336

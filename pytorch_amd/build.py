@@ -27,6 +27,12 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-con
                 "-Wno-pass-failed"]
 
 
+# Per-file additions.  The kernels that fold their MFMA sums into float32 totals once per scale group keep the
+# accumulators in ordinary vector registers: the compiler's default (accumulation registers) costs a register move
+# per accumulator element and fold in each direction.
+EXTRA_FLAGS = {"weight_quant_kpacked.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def _run(cmd):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
@@ -40,7 +46,7 @@ def build_kernels(verbose: bool = False) -> str:
 
     def compile_one(src):
         obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
-        out = _run([HIPCC, *DEVICE_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        out = _run([HIPCC, *DEVICE_FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj])
         if verbose and out.strip():
             print(out)
         return obj

@@ -53,8 +53,10 @@ __device__ __forceinline__ u32x4 even_odd(u32x4 v)
     return r;
 }
 
-// MT: m tiles (16 rows) per workgroup; NW: wavefronts = 16-column tiles per workgroup
-template <int MT, int NW, int ACT>
+// MT: m tiles (16 rows) per workgroup; NW: wavefronts = 16-column tiles per workgroup; G128: a scale group is one
+// sub-step (group_size 128), so every half step starts its sums from zero and ends with a fold - no counters, and
+// the first MFMA of a half takes a zero accumulator instead of a cleared register
+template <int MT, int NW, int ACT, bool G128>
 __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
 {
     constexpr int NBW = NW * 16, THREADS = NW * 64;
@@ -63,7 +65,10 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
     constexpr int BODY = RS / 2;                        // registers (one consumed, one in flight; 2 KiB per step and
                                                         // wavefront), the slot of a step known at compile time
     constexpr int POLICY = MT == 1 ? kNonTemporal : 0;
-    constexpr int XBUF = 32768;                         // bytes of one activation chunk in LDS
+    constexpr int FP = 1024 + 16;                       // pitch of a 1 KiB activation fragment in LDS: the staging writes
+                                                        // of a wavefront go to sixteen fragments at the same lane
+                                                        // position, which an unpadded pitch puts into the same banks
+    constexpr int XBUF = 32 * FP;                       // bytes of one activation chunk in LDS
     constexpr int TBUF = 2048;                          // one step of one wavefront's weights (16 rows x 128 bytes)
     constexpr int PPR = CH * 32;                        // 16-byte pieces of an activation row per chunk
     constexpr int PPT = 2048 / THREADS;                 // pieces per thread and chunk
@@ -130,20 +135,24 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
                                                            (uint32_t)(step0 + ch * CH) * 512u, 0);
         }
     };
+    // rows past the last valid one are never written: they only feed accumulator rows that are never stored
+    const int valid_pieces = rows_valid * PPR;
     auto stage_store = [&](int ch) {
         char *buf = lds + 16 + (ch & 1) * XBUF;
 #pragma unroll
         for (int i = 0; i < PPT; i++) {
+            if (i * THREADS >= valid_pieces) break;         // uniform over the workgroup
             const int pid = i * THREADS + threadIdx.x;
             const int r = pid / PPR, q = pid % PPR;
             const int sl = q >> 5, f = 4 * ((q >> 4) & 1) + (q & 3), gg = (q >> 2) & 3;
-            *reinterpret_cast<u32x4 *>(buf + ((((sl * MT + (r >> 4)) * 8 + f) * 64) + gg * 16 + (r & 15)) * 16) = even_odd(xst[i]);
+            *reinterpret_cast<u32x4 *>(buf + ((sl * MT + (r >> 4)) * 8 + f) * FP + (gg * 16 + (r & 15)) * 16) = even_odd(xst[i]);
         }
     };
 
-    f32x4 P[MT], X[MT], tot[MT];
+    // two accumulators per sum, used alternately: a chain of dependent MFMAs is two long instead of four
+    f32x4 P[MT][2], X[MT][2], tot[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) P[mt] = X[mt] = tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; mt++) P[mt][0] = P[mt][1] = X[mt][0] = X[mt][1] = tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
     auto fold = [&](int gl) {
         const uint32_t pr = prm[gl * NBW + wave * 16 + c];
@@ -151,9 +160,10 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
         const float of = (act_hi<ACT>(pr) - X_BIAS) * (1.0f / P_MUL);
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
+            const f32x4 ps = P[mt][0] + P[mt][1], xs = X[mt][0] + X[mt][1];
 #pragma unroll
-            for (int q = 0; q < 4; q++) tot[mt][q] = __builtin_fmaf(sc, __builtin_fmaf(of, X[mt][q], P[mt][q]), tot[mt][q]);
-            P[mt] = X[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int q = 0; q < 4; q++) tot[mt][q] = __builtin_fmaf(sc, __builtin_fmaf(of, xs[q], ps[q]), tot[mt][q]);
+            if constexpr (!G128) P[mt][0] = P[mt][1] = X[mt][0] = X[mt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
     };
 
@@ -212,7 +222,7 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
         for (int d = 0; d < 4; d++)
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
-                xa[buf][d][mt] = *reinterpret_cast<const u32x4 *>(xb + ((jc * MT + mt) * 8 + 4 * h + d) * 1024);
+                xa[buf][d][mt] = *reinterpret_cast<const u32x4 *>(xb + ((jc * MT + mt) * 8 + 4 * h + d) * FP);
     };
 
     int in_group = 0, gl = 0, ch = 0;
@@ -253,11 +263,14 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
                     const u32x4 b = expand_word<ACT>(wc[h][d]);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
-                        P[mt] = mfma_act<ACT>(xa[cur][d][mt], b, P[mt]);
-                        X[mt] = mfma_act<ACT>(xa[cur][d][mt], ones, X[mt]);
+                        const f32x4 zero = f32x4{0.f, 0.f, 0.f, 0.f};
+                        P[mt][d & 1] = mfma_act<ACT>(xa[cur][d][mt], b, G128 && d < 2 ? zero : P[mt][d & 1]);
+                        X[mt][d & 1] = mfma_act<ACT>(xa[cur][d][mt], ones, G128 && d < 2 ? zero : X[mt][d & 1]);
                     }
                 }
-                if (st < nsteps && ++in_group == gsub) {
+                if constexpr (G128) {
+                    if (st < nsteps) fold(gl++);
+                } else if (st < nsteps && ++in_group == gsub) {
                     fold(gl);
                     in_group = 0;
                     gl++;
@@ -289,10 +302,10 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
     outp.finish(rows_valid, tile);
 }
 
-template <int MT, int NW, int ACT>
+template <int MT, int NW, int ACT, bool G128>
 int launch_one(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
 {
-    auto kern = wq_kpacked_kernel<MT, NW, ACT>;
+    auto kern = wq_kpacked_kernel<MT, NW, ACT, G128>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
@@ -300,17 +313,20 @@ int launch_one(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
     return check_launch();
 }
 
+template <int NW, int ACT, bool G128>
+int launch_mt(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
+{
+    if (pl.mt == 1) return launch_one<1, NW, ACT, G128>(p, pl, s);
+    if (pl.mt == 2) return launch_one<2, NW, ACT, G128>(p, pl, s);
+    return launch_one<4, NW, ACT, G128>(p, pl, s);
+}
+
 template <int ACT>
 int launch_act(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
 {
-    if (pl.nw == 4) {
-        if (pl.mt == 1) return launch_one<1, 4, ACT>(p, pl, s);
-        if (pl.mt == 2) return launch_one<2, 4, ACT>(p, pl, s);
-        return launch_one<4, 4, ACT>(p, pl, s);
-    }
-    if (pl.mt == 1) return launch_one<1, 8, ACT>(p, pl, s);
-    if (pl.mt == 2) return launch_one<2, 8, ACT>(p, pl, s);
-    return launch_one<4, 8, ACT>(p, pl, s);
+    const bool g128 = pl.grouped && pl.unit_sub == 1;
+    if (pl.nw == 4) return g128 ? launch_mt<4, ACT, true>(p, pl, s) : launch_mt<4, ACT, false>(p, pl, s);
+    return g128 ? launch_mt<8, ACT, true>(p, pl, s) : launch_mt<8, ACT, false>(p, pl, s);
 }
 
 int64_t gcd64(int64_t a, int64_t b)
@@ -366,7 +382,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     auto lds_need = [&](int s) {
         const int64_t units = (pl.n_units + s - 1) / s;
         const int64_t groups = pl.grouped ? units * pl.unit_steps * 2 / pl.unit_sub : 1;
-        return (size_t)16 + 2 * 32768 + (size_t)pl.nw * 4096 + (size_t)groups * pl.nw * 16 * 4;
+        return (size_t)16 + 2 * 32 * (1024 + 16) + (size_t)pl.nw * 4096 + (size_t)groups * pl.nw * 16 * 4;
     };
     while (lds_need(S) > 160 * 1024 && S < pl.n_units && S < 16) S++;
     if (lds_need(S) > 160 * 1024) {
