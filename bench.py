@@ -126,6 +126,16 @@ def _pmc_pass(torch, pa, workloads, dev):
     pa.npu_weight_quant_batchmatmul(g5["x"], g5["weight"], g5["antiquant_scale"], g5["antiquant_offset"], None, None,
                                     None, 128)
     pa.npu_anti_quant(xa, sa, offset=sa, dst_dtype=torch.bfloat16)
+    # int4 weights with their words along K (the module's layout) at M = 8, and the int4 -> int8 widening of an A4W4
+    # weight, on fresh operands
+    wk = torch.randint(-2 ** 31, 2 ** 31 - 1, (14336, 512), dtype=torch.int32, device=dev)
+    wa = torch.randint(-2 ** 31, 2 ** 31 - 1, (11008, 512), dtype=torch.int32, device=dev)
+    xa4 = torch.randint(-2 ** 31, 2 ** 31 - 1, (1024, 512), dtype=torch.int32, device=dev)
+    s4t, o4t = g4["antiquant_scale"].t().contiguous().t(), g4["antiquant_offset"].t().contiguous().t()
+    flush.fill_(2)
+    torch.cuda.synchronize()
+    pa.npu_weight_quant_batchmatmul(g4["x"], wk.t(), s4t, o4t, None, None, None, 128)
+    pa.npu_quant_matmul(xa4, wa.t(), g["scale"], pertoken_scale=g["pertoken_scale"], output_dtype=torch.bfloat16)
     torch.cuda.synchronize()
     print(json.dumps({"pmc_pass": "done"}))
 
