@@ -8,7 +8,8 @@ namespace mi355 {
 struct WqKpackedPlan {
     bool ok;                 // the kernel accepts this problem
     int mt;                  // m tiles (16 rows) per workgroup: 1, 2 or 4
-    int nw;                  // wavefronts (16-column tiles) per workgroup: 4 or 8
+    int nw;                  // 16-column tiles per workgroup: 4 or 8
+    int ks;                  // slices of the workgroup's K range (nw * ks wavefronts): 1 or 2
     int mchunks, tiles;      // workgroups along M and N
     int S;                   // workgroups that share the K range of a tile
     int unit_steps, n_units; // K is split between workgroups in units of unit_steps * 256

@@ -53,14 +53,17 @@ __device__ __forceinline__ u32x4 even_odd(u32x4 v)
     return r;
 }
 
-// MT: m tiles (16 rows) per workgroup; NW: wavefronts = 16-column tiles per workgroup; G128: a scale group is one
+// MT: m tiles (16 rows) per workgroup; NW: 16-column tiles per workgroup; KS: slices of the workgroup's K range -
+// NW * KS wavefronts, the slices are added in LDS at the end (two wavefronts per SIMD where the column tiles alone
+// would leave one: a single wavefront cannot hide its own MFMA and LDS latencies); G128: a scale group is one
 // sub-step (group_size 128), so every half step starts its sums from zero and ends with a fold - no counters, and
 // the first MFMA of a half takes a zero accumulator instead of a cleared register
-template <int MT, int NW, int ACT, bool G128>
-__global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
+template <int MT, int NW, int KS, int ACT, bool G128>
+__global__ __launch_bounds__(NW * KS * 64) void wq_kpacked_kernel(const WqArgs p)
 {
-    constexpr int NBW = NW * 16, THREADS = NW * 64;
-    constexpr int CH = 4 / MT;                          // steps per chunk of activations (32 KiB of LDS per buffer)
+    static_assert(MT * KS <= 4, "a chunk holds at least one step of every slice");
+    constexpr int WAVES = NW * KS, NBW = NW * 16, THREADS = WAVES * 64;
+    constexpr int CH = 4 / (MT * KS);                   // steps per slice and chunk of activations (32 KiB of LDS per buffer)
     constexpr int RS = MT == 4 ? 4 : 8;                 // steps per round of the main loop: two batches of weight loads in
     constexpr int BODY = RS / 2;                        // registers (one consumed, one in flight; 2 KiB per step and
                                                         // wavefront), the slot of a step known at compile time
@@ -70,13 +73,14 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
                                                         // position, which an unpadded pitch puts into the same banks
     constexpr int XBUF = 32 * FP;                       // bytes of one activation chunk in LDS
     constexpr int TBUF = 2048;                          // one step of one wavefront's weights (16 rows x 128 bytes)
-    constexpr int PPR = CH * 32;                        // 16-byte pieces of an activation row per chunk
+    constexpr int PPR = CH * 32;                        // 16-byte pieces of an activation row per slice and chunk
     constexpr int PPT = 2048 / THREADS;                 // pieces per thread and chunk
     constexpr float P_MUL = kImageMul<4, ACT>, X_BIAS = kImageBias<4>;
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, g = lane >> 4;
+    const int ct = wave % NW, ks = wave / NW;           // column tile and K slice of this wavefront
     const int xcd_slot = blockIdx.x >> 3;
     const int tile = (blockIdx.x & 7) + 8 * (xcd_slot / p.S);
     const int chunk = xcd_slot % p.S;
@@ -87,12 +91,16 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
 
     // K range of this workgroup in steps of 256 (whole units: a unit is a whole number of steps and of scale groups)
     const int u0 = (int)((int64_t)p.n_units * chunk / p.S), u1 = (int)((int64_t)p.n_units * (chunk + 1) / p.S);
-    const int step0 = u0 * p.unit_steps, nsteps = (u1 - u0) * p.unit_steps;
-    const int nrounds = (nsteps + RS - 1) / RS;
-    // scale groups of the range, in sub-steps of 128 k (per channel: one group that ends with the range)
+    const int wg_step0 = u0 * p.unit_steps, wg_nsteps = (u1 - u0) * p.unit_steps;
+    // ... and of slice s of the workgroup (whole units again); every wavefront runs the rounds of the longest slice
+    auto slice_u0 = [&](int s) { return (int)((int64_t)(u1 - u0) * s / KS); };
+    const int step0 = wg_step0 + slice_u0(ks) * p.unit_steps, nsteps = (slice_u0(ks + 1) - slice_u0(ks)) * p.unit_steps;
+    const int nrounds = ((u1 - u0 + KS - 1) / KS * p.unit_steps + RS - 1) / RS;
+    // scale groups in sub-steps of 128 k (per channel: one group that ends with the wavefront's range)
     const int gsub = p.grouped ? p.unit_sub : 2 * nsteps;
-    const int grp0 = p.grouped ? (2 * step0) / p.unit_sub : 0;
-    const int ngroups = (2 * nsteps + gsub - 1) / gsub;
+    const int grp0 = p.grouped ? (2 * wg_step0) / p.unit_sub : 0;                       // first group of the workgroup
+    const int ngroups = p.grouped ? (2 * wg_nsteps) / p.unit_sub : 1;                   // groups of the workgroup
+    const int gl0 = p.grouped ? (2 * (step0 - wg_step0)) / p.unit_sub : 0;              // first group of this wavefront
 
     // Weights: a load instruction fetches whole cache lines - lane l takes 16 bytes of row l/8 (+8 for the second
     // load) - and the wavefront turns the step around through a private 2 KiB LDS tile into operand order.  The
@@ -103,10 +111,10 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
 #pragma unroll
     for (int h = 0; h < 2; h++) {
         const int rl = 8 * h + (lane >> 3);
-        voff_w[h] = (uint32_t)min(n0 + wave * 16 + rl, p.N - 1) * p.ldw_bytes + (uint32_t)(((lane & 7) ^ ((rl >> 1) & 7)) * 16);
+        voff_w[h] = (uint32_t)min(n0 + ct * 16 + rl, p.N - 1) * p.ldw_bytes + (uint32_t)(((lane & 7) ^ ((rl >> 1) & 7)) * 16);
     }
     char *tbuf = lds + 16 + 2 * XBUF + wave * (2 * TBUF);
-    uint32_t *prm = reinterpret_cast<uint32_t *>(lds + 16 + 2 * XBUF + NW * 2 * TBUF);   // [group][column]: scale | offset << 16
+    uint32_t *prm = reinterpret_cast<uint32_t *>(lds + 16 + 2 * XBUF + WAVES * 2 * TBUF);   // [group][column]: scale | offset << 16
     const int t_rd = c * 128 + ((g ^ ((c >> 1) & 7)) * 16);   // chunk g of row c; chunk g + 4 is at slot ^ 4, i.e. +-64 bytes
     const __amdgpu_buffer_rsrc_t rsrc_x =
         make_rsrc(p.x + (int64_t)m_base * p.ldx, (uint32_t)(((int64_t)(rows_valid - 1) * p.ldx + p.K) * 2));
@@ -121,31 +129,34 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
             wq[slot][j][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ok ? voff_w[1] : kOutOfRange, kb, POLICY);
         }
     };
-    // Activation staging: piece q of a row's chunk (8 consecutive k) belongs to step q / 32, half (q % 32) / 16, lane
-    // group (q % 16) / 4 and dword q % 4 of that lane's 16 bytes; it goes to fragment (step, m tile, 4 * half + dword)
-    // at lane (group, row % 16).  Consecutive threads read consecutive pieces of a row.
+    // Activation staging: piece q of a row's chunk of one slice (8 consecutive k) belongs to step q / 32, half
+    // (q % 32) / 16, lane group (q % 16) / 4 and dword q % 4 of that lane's 16 bytes; it goes to fragment
+    // (slice, step, m tile, 4 * half + dword) at lane (group, row % 16).  Consecutive threads read consecutive pieces
+    // of a row.
     u32x4 xst[PPT];
     auto stage_load = [&](int ch) {
 #pragma unroll
         for (int i = 0; i < PPT; i++) {
             const int pid = i * THREADS + threadIdx.x;
-            const int r = pid / PPR, q = pid % PPR;
-            const bool ok = r < rows_valid && ch * CH + (q >> 5) < nsteps;
-            xst[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, ok ? (uint32_t)((r * (int)p.ldx + q * 8) * 2) : kOutOfRange,
-                                                           (uint32_t)(step0 + ch * CH) * 512u, 0);
+            const int r = pid / (KS * PPR), sl = (pid / PPR) % KS, q = pid % PPR;
+            const int s0 = slice_u0(sl) * p.unit_steps, sn = (slice_u0(sl + 1) - slice_u0(sl)) * p.unit_steps;
+            const bool ok = r < rows_valid && ch * CH + (q >> 5) < sn;
+            xst[i] = __builtin_amdgcn_raw_buffer_load_b128(
+                rsrc_x, ok ? (uint32_t)((r * (int)p.ldx + (wg_step0 + s0 + ch * CH) * 256 + q * 8) * 2) : kOutOfRange, 0u, 0);
         }
     };
     // rows past the last valid one are never written: they only feed accumulator rows that are never stored
-    const int valid_pieces = rows_valid * PPR;
+    const int valid_pieces = rows_valid * KS * PPR;
     auto stage_store = [&](int ch) {
         char *buf = lds + 16 + (ch & 1) * XBUF;
 #pragma unroll
         for (int i = 0; i < PPT; i++) {
             if (i * THREADS >= valid_pieces) break;         // uniform over the workgroup
             const int pid = i * THREADS + threadIdx.x;
-            const int r = pid / PPR, q = pid % PPR;
-            const int sl = q >> 5, f = 4 * ((q >> 4) & 1) + (q & 3), gg = (q >> 2) & 3;
-            *reinterpret_cast<u32x4 *>(buf + ((sl * MT + (r >> 4)) * 8 + f) * FP + (gg * 16 + (r & 15)) * 16) = even_odd(xst[i]);
+            const int r = pid / (KS * PPR), sl = (pid / PPR) % KS, q = pid % PPR;
+            const int st = q >> 5, f = 4 * ((q >> 4) & 1) + (q & 3), gg = (q >> 2) & 3;
+            *reinterpret_cast<u32x4 *>(buf + (((sl * CH + st) * MT + (r >> 4)) * 8 + f) * FP + (gg * 16 + (r & 15)) * 16) =
+                even_odd(xst[i]);
         }
     };
 
@@ -155,7 +166,7 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
     for (int mt = 0; mt < MT; mt++) P[mt][0] = P[mt][1] = X[mt][0] = X[mt][1] = tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
     auto fold = [&](int gl) {
-        const uint32_t pr = prm[gl * NBW + wave * 16 + c];
+        const uint32_t pr = prm[gl * NBW + ct * 16 + c];
         const float sc = act_lo<ACT>(pr) * P_MUL;
         const float of = (act_hi<ACT>(pr) - X_BIAS) * (1.0f / P_MUL);
 #pragma unroll
@@ -167,35 +178,37 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
         }
     };
 
-    // prologue: everything is requested up front - activations of chunk 0 and the antiquant parameters first (they
-    // come from cache, loads retire in order, and what the first barrier waits for must not queue behind 16 KiB of
-    // weights per wavefront), then the first two batches of weights
-    stage_load(0);
+    // prologue: the antiquant parameters are requested first (they come from HBM, and the first barrier waits for
+    // them), then the activations of chunk 0 (from cache) and the first batch of weights
     {
         // parameters of the workgroup's columns and groups, any strides: walk along whichever dimension is
-        // contiguous in memory; eight loads in flight per thread, no branches (indices past the end repeat the
-        // last entry; without offsets the scale is loaded twice and masked)
+        // contiguous in memory; eight loads in flight per thread, no branches around them (indices past the end
+        // repeat the last entry; without offsets the scale is loaded twice and masked).  `inner` is a power of two in
+        // all usual cases, which spares the integer divisions.
         const bool n_inner = p.ld_param_n == 1;
         const int inner = n_inner ? NBW : ngroups, total = ngroups * NBW;
+        const int shift = (inner & (inner - 1)) == 0 ? 31 - __builtin_clz(inner) : -1;
         const uint16_t *offp = p.offset ? p.offset : p.scale;
         const uint32_t omask = p.offset ? 0xffffu : 0u;
-        auto batch = [&](int base, bool with_weights) {
+        auto batch = [&](int base, bool first) {
             uint32_t sv[8], ov[8];
             int at_lds[8];
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 const int idx = min(base + i * THREADS + (int)threadIdx.x, total - 1);
-                const int a = idx % inner, b = idx / inner;
+                int a, b;
+                if (shift >= 0) a = idx & (inner - 1), b = idx >> shift;
+                else a = idx % inner, b = idx / inner;
                 const int col = n_inner ? a : b, gl = n_inner ? b : a;
                 const int64_t at = (int64_t)(grp0 + gl) * p.ld_param_g + (int64_t)min(n0 + col, p.N - 1) * p.ld_param_n;
                 sv[i] = p.scale[at];
                 ov[i] = offp[at];
                 at_lds[i] = gl * NBW + col;
             }
-            if (with_weights) {
+            if (first) {
                 __builtin_amdgcn_sched_barrier(0);
+                stage_load(0);
                 load_body(0, 0);
-                load_body(1, BODY);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
@@ -206,6 +219,10 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
     }
     stage_store(0);
     __syncthreads();
+    // the second batch of weights goes out behind the barrier: ahead of it, it would sit in the memory queues in
+    // front of the activation and parameter loads of the wavefronts that arrive later
+    load_body(1, BODY);
+    __builtin_amdgcn_sched_barrier(0);
     // step 0 of the weights goes through the wavefront's turn-around tile into operand order
     *reinterpret_cast<u32x4 *>(tbuf + lane * 16) = wq[0][0][0];
     *reinterpret_cast<u32x4 *>(tbuf + 1024 + lane * 16) = wq[0][0][1];
@@ -222,10 +239,10 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
         for (int d = 0; d < 4; d++)
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
-                xa[buf][d][mt] = *reinterpret_cast<const u32x4 *>(xb + ((jc * MT + mt) * 8 + 4 * h + d) * FP);
+                xa[buf][d][mt] = *reinterpret_cast<const u32x4 *>(xb + (((ks * CH + jc) * MT + mt) * 8 + 4 * h + d) * FP);
     };
 
-    int in_group = 0, gl = 0, ch = 0;
+    int in_group = 0, gl = gl0, ch = 0;
     for (int rd = 0; rd < nrounds; rd++) {
 #pragma unroll
         for (int j = 0; j < RS; j++) {
@@ -286,7 +303,7 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
 
     // ---- output: the wavefront's [rows x 16 columns] tile goes through LDS to the shared output / exchange code
     float *red = reinterpret_cast<float *>(lds + 16);
-    TileOut<NBW, 1, THREADS, ACT> outp(p, lds, m_base, n0, chunk);
+    TileOut<NBW, KS, THREADS, ACT> outp(p, lds, m_base, n0, chunk);
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
         const int rows_mt = min(16, rows_valid - mt * 16);
@@ -294,7 +311,7 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             const int row = 4 * g + q;
-            if (row < rows_mt) red[row * NBW + wave * 16 + c] = tot[mt][q];
+            if (row < rows_mt) red[(ks * 16 + row) * NBW + ct * 16 + c] = tot[mt][q];
         }
         __syncthreads();
         outp.emit_mtile(red, mt * 16, rows_mt);
@@ -302,31 +319,40 @@ __global__ __launch_bounds__(NW * 64) void wq_kpacked_kernel(const WqArgs p)
     outp.finish(rows_valid, tile);
 }
 
-template <int MT, int NW, int ACT, bool G128>
+template <int MT, int NW, int KS, int ACT, bool G128>
 int launch_one(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
 {
-    auto kern = wq_kpacked_kernel<MT, NW, ACT, G128>;
+    auto kern = wq_kpacked_kernel<MT, NW, KS, ACT, G128>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)((pl.tiles + 7) / 8 * 8 * pl.S), (unsigned)pl.mchunks), dim3(NW * 64), pl.lds_bytes, s, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((pl.tiles + 7) / 8 * 8 * pl.S), (unsigned)pl.mchunks), dim3(NW * KS * 64),
+                       pl.lds_bytes, s, p);
     return check_launch();
 }
 
-template <int NW, int ACT, bool G128>
-int launch_mt(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
+template <int ACT, bool G128>
+int launch_shape(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
 {
-    if (pl.mt == 1) return launch_one<1, NW, ACT, G128>(p, pl, s);
-    if (pl.mt == 2) return launch_one<2, NW, ACT, G128>(p, pl, s);
-    return launch_one<4, NW, ACT, G128>(p, pl, s);
+    if (pl.nw == 4 && pl.ks == 2) {
+        if (pl.mt == 1) return launch_one<1, 4, 2, ACT, G128>(p, pl, s);
+        return launch_one<2, 4, 2, ACT, G128>(p, pl, s);
+    }
+    if (pl.nw == 4) {
+        if (pl.mt == 1) return launch_one<1, 4, 1, ACT, G128>(p, pl, s);
+        if (pl.mt == 2) return launch_one<2, 4, 1, ACT, G128>(p, pl, s);
+        return launch_one<4, 4, 1, ACT, G128>(p, pl, s);
+    }
+    if (pl.mt == 1) return launch_one<1, 8, 1, ACT, G128>(p, pl, s);
+    if (pl.mt == 2) return launch_one<2, 8, 1, ACT, G128>(p, pl, s);
+    return launch_one<4, 8, 1, ACT, G128>(p, pl, s);
 }
 
 template <int ACT>
 int launch_act(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
 {
     const bool g128 = pl.grouped && pl.unit_sub == 1;
-    if (pl.nw == 4) return g128 ? launch_mt<4, ACT, true>(p, pl, s) : launch_mt<4, ACT, false>(p, pl, s);
-    return g128 ? launch_mt<8, ACT, true>(p, pl, s) : launch_mt<8, ACT, false>(p, pl, s);
+    return g128 ? launch_shape<ACT, true>(p, pl, s) : launch_shape<ACT, false>(p, pl, s);
 }
 
 int64_t gcd64(int64_t a, int64_t b)
@@ -370,6 +396,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     if (const int f = env_int("MI355_WQK_NW"))      // tuning aid
         if (f == 4 || f == 8) pl.nw = f;
     pl.tiles = (int)((N + pl.nw * 16 - 1) / (pl.nw * 16));
+    pl.ks = 1;
     int S = kNumCU / (pl.tiles * pl.mchunks);
     if (S > pl.n_units) S = pl.n_units;
     if (S > 16) S = 16;
@@ -382,7 +409,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     auto lds_need = [&](int s) {
         const int64_t units = (pl.n_units + s - 1) / s;
         const int64_t groups = pl.grouped ? units * pl.unit_steps * 2 / pl.unit_sub : 1;
-        return (size_t)16 + 2 * 32 * (1024 + 16) + (size_t)pl.nw * 4096 + (size_t)groups * pl.nw * 16 * 4;
+        return (size_t)16 + 2 * 32 * (1024 + 16) + (size_t)pl.nw * 2 * 4096 + (size_t)groups * pl.nw * 16 * 4;
     };
     while (lds_need(S) > 160 * 1024 && S < pl.n_units && S < 16) S++;
     if (lds_need(S) > 160 * 1024) {
@@ -390,6 +417,9 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
         return pl;
     }
     pl.S = S;
+    // with four column tiles and at most two m tiles the workgroup's K range is cut into two slices (eight wavefronts,
+    // two per SIMD) when it holds at least two units
+    if (pl.nw == 4 && pl.mt <= 2 && (pl.n_units + S - 1) / S >= 2 && env_int("MI355_WQK_KS") != 1) pl.ks = 2;
     pl.lds_bytes = lds_need(S);
     pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
     pl.counter_bytes = S > 1 ? kWorkspaceCounterBytes : 0;
