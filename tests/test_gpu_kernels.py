@@ -507,6 +507,39 @@ def test_weight_quant_random_shapes(capi, golden):
             raise AssertionError(f"case {case}: bits={bits} M={M} K={K} N={N} gs={gs} nk={nk} f16={f16} offset={with_off}: {e}")
 
 
+def test_weight_quant_int4_words_along_k_random_shapes(capi, golden):
+    """Seeded sweep for int4 weights stored [N, K/8]: shapes that take the fast kernel (K a multiple of 256, groups of
+    whole sub-steps; every m-tile count, ragged columns, one or two K slices, K split between workgroups) and shapes
+    that fall back to the generic kernel, parameters in either layout, both activation types."""
+    import os
+    rng = np.random.default_rng(4242)
+    for case in range(int(os.environ.get("MI355_SWEEP_CASES", "64"))):
+        M = int(rng.choice([1, 2, 15, 16, 17, 32, 33, 63, 64, 65, 100, 130]))
+        K = int(rng.choice([128, 256, 512, 768, 1024, 1280, 2048, 3072]))
+        N = int(rng.choice([8, 16, 24, 64, 72, 128, 136, 200, 256, 1000, 2048]))
+        gs = int(rng.choice([g for g in (0, 32, 64, 128, 256, 384, 512, 1024) if g == 0 or K % g == 0]))
+        f16 = bool(rng.random() < 0.3)
+        with_off = bool(rng.random() < 0.8)
+        params_ng = bool(rng.random() < 0.5)
+        d = workloads.w4a16_inputs(seed=case, M=M, K=K, N=N, group_size=gs if gs else K)
+        if not gs:
+            d["antiquant_scale"], d["antiquant_offset"] = d["antiquant_scale"][0].clone(), d["antiquant_offset"][0].clone()
+        bits_of = _bits
+        if f16:
+            d = _to_f16(d)
+            bits_of = _f16_bits
+        sc, of = d["antiquant_scale"], (d["antiquant_offset"] if with_off else None)
+        _, gold = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(sc), None if of is None else bits_of(of),
+                                             group_size=gs, dtype="fp16" if f16 else "bf16")
+        w_nk = torch.from_numpy(golden.pack_int4(np.ascontiguousarray(d["weight_int4_values"].numpy().T)))
+        dev = lambda t: None if t is None else (t.t().contiguous().cuda().t() if params_ng and t.dim() == 2 else t.cuda())  # noqa: E731
+        try:
+            out = capi.weight_quant_matmul(d["x"].cuda(), w_nk.cuda().t(), dev(sc), dev(of), group_size=gs)
+            bf16_gate(out, torch.from_numpy(gold))
+        except (AssertionError, capi.Mi355Error) as e:
+            raise AssertionError(f"case {case}: M={M} K={K} N={N} gs={gs} f16={f16} offset={with_off} params_ng={params_ng}: {e}")
+
+
 def test_weight_quant_exact_special_case(capi):
     # small-integer activations, unit scale, zero offset: every partial sum is exact in float32
     g = torch.Generator().manual_seed(0)
