@@ -316,6 +316,11 @@ def main():
             e["cpu_baseline"] = {"value": round(nb / (c1 - c0) / 1e9, 3), "unit": "GB/s", "cores": golden.get_threads(),
                                  "kind": "port", "sample": "the full configuration, one pass"}
         others.append(e)
+        # the asymmetric variant on the same inputs (three outputs: codes, scale, offset)
+        keep.clear()
+        calls = [(lambda x=x: keep.append(pa.npu_dynamic_quant_asymmetric(x))) for x in xs] * 2
+        us = _graph_time_us(torch, calls)
+        others.append(hbm_entry("dynamic_quant_asymmetric bf16[2048,4096] (rotating, > Infinity Cache)", nb + rows * 4, us, None))
         del xs, keep
 
     if want("c3"):

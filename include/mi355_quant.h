@@ -72,6 +72,21 @@ int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth,
                         int64_t rows, int64_t cols, int64_t x_row_stride, void *stream);
 
 /*
+ * npu_dynamic_quant_asymmetric, per-token asymmetric int8.
+ * Replaces the aclnn DynamicQuantV2 call behind torch_npu.npu_dynamic_quant_asymmetric (signature and output
+ * shapes: test/test_fake_tensor.py:1689-1709, test/torch_npu_schema.json:2147-2149).  The arithmetic is not in the
+ * reference tree; it follows the operator's published description:
+ *   scale  = (row_max - row_min) / 255          offset = 127 - row_max / scale
+ *   y      = rint_half_even(x / scale + offset) in [-128, 127]   (row_max -> 127, row_min -> -128)
+ * every operation rounded to float32 on its own.  x, smooth, y, rows, cols, x_row_stride as in mi355_dynamic_quant;
+ * scale and offset are float32 [rows].  A row whose elements are all equal yields scale 0, offset 0 and y 0
+ * (this library's choice).  cols == 0 leaves scale and offset unwritten.
+ */
+int mi355_dynamic_quant_asymmetric(const void *x, int in_dtype, const void *smooth,
+                                   int8_t *y, float *scale, float *offset,
+                                   int64_t rows, int64_t cols, int64_t x_row_stride, void *stream);
+
+/*
  * npu_quant_matmul, W8A8 with int32 accumulation and fused dequantisation.
  * Replaces the aclnn QuantMatmul call behind torch_npu.npu_quant_matmul
  * (callers: torch_npu/contrib/module/linear_quant.py:96-112, linear_a8w8_quant.py:87-120;

@@ -28,6 +28,9 @@
  *   orc_dynamic_quant       formula of the benchmark configuration, checked against torch fp32 /
  *                           numpy evaluation, hand-typed round-half-even cases and invariants;
  *                           behaviour of the Ascend kernel itself: PARITY UNPINNED.
+ *   orc_dynamic_quant_asymmetric  the operator's published description (scale = (max - min) / 255,
+ *                           offset = 127 - max / scale), checked against numpy float32 evaluation and
+ *                           hand-computed rows; behaviour of the Ascend kernel itself: PARITY UNPINNED.
  *   orc_swiglu              torch_npu/_inductor/decomposition.py:186-188 (silu(a)*b), checked against
  *                           torch CPU bf16 evaluation.
  *
@@ -161,6 +164,51 @@ void orc_dynamic_quant(const uint16_t *x, int in_dtype, const uint16_t *smooth,
             float rq = rintf(q); /* default rounding mode: to nearest, ties to even */
             if (rq > 127.0f) rq = 127.0f;
             if (rq < -127.0f) rq = -127.0f;
+            yr[j] = (int8_t)rq;
+        }
+    }
+}
+
+/*
+ * npu_dynamic_quant_asymmetric (signature and shapes: test/test_fake_tensor.py:1689-1709).  The arithmetic is not
+ * in the reference tree: this restates the operator's published description,
+ *   scale = (row_max - row_min) / 255,  offset = 127 - row_max / scale,  y = rint(x / scale + offset) in [-128, 127],
+ * one binary32 operation at a time.  A row of equal elements: scale 0, offset 0, y 0.  PARITY UNPINNED against the
+ * Ascend kernel; the function itself is checked against a numpy float32 evaluation and hand-computed rows.
+ */
+void orc_dynamic_quant_asymmetric(const uint16_t *x, int in_dtype, const uint16_t *smooth,
+                                  int64_t rows, int64_t cols, int64_t row_stride,
+                                  int8_t *y, float *scale, float *offset)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; r++) {
+        const uint16_t *xr = x + r * row_stride;
+        int8_t *yr = y + r * cols;
+        float mx = -INFINITY, mn = INFINITY;
+        for (int64_t j = 0; j < cols; j++) {
+            float v = in_dtype ? fp16_to_f32(xr[j]) : bf16_to_f32(xr[j]);
+            if (smooth) v = v * (in_dtype ? fp16_to_f32(smooth[j]) : bf16_to_f32(smooth[j]));
+            if (v > mx) mx = v;
+            if (v < mn) mn = v;
+        }
+        if (!(mx > mn)) {
+            scale[r] = 0.0f;
+            offset[r] = 0.0f;
+            for (int64_t j = 0; j < cols; j++) yr[j] = 0;
+            continue;
+        }
+        float s = (mx - mn) / 255.0f;
+        float o = 127.0f - mx / s;
+        scale[r] = s;
+        offset[r] = o;
+        for (int64_t j = 0; j < cols; j++) {
+            float v = in_dtype ? fp16_to_f32(xr[j]) : bf16_to_f32(xr[j]);
+            if (smooth) v = v * (in_dtype ? fp16_to_f32(smooth[j]) : bf16_to_f32(smooth[j]));
+            float q = v / s;
+            q = q + o;
+            float rq = rintf(q);
+            if (rq > 127.0f) rq = 127.0f;
+            if (rq < -128.0f) rq = -128.0f;
             yr[j] = (int8_t)rq;
         }
     }

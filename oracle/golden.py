@@ -39,6 +39,7 @@ def lib() -> ctypes.CDLL:
         L.orc_set_threads.argtypes = [i32]
         L.orc_get_threads.restype = i32
         L.orc_dynamic_quant.argtypes = [vp, i32, vp, i64, i64, i64, vp, vp]
+        L.orc_dynamic_quant_asymmetric.argtypes = [vp, i32, vp, i64, i64, i64, vp, vp, vp]
         L.orc_int8_gemm.argtypes = [vp, i64, vp, i64, i64, i64, i64, i64, vp]
         L.orc_quant_matmul_epilogue.argtypes = [vp, vp, vp, i64, vp, i64, i64, vp]
         L.orc_quant_matmul_epilogue_ex.argtypes = [vp, vp, vp, i64, vp, i32, i32, i64, i64, vp]
@@ -88,6 +89,21 @@ def dynamic_quant(x_u16: np.ndarray, in_dtype: str = "bf16", smooth_u16: np.ndar
     elif rows:
         scale[...] = 0.0
     return y, scale
+
+
+def dynamic_quant_asymmetric(x_u16: np.ndarray, in_dtype: str = "bf16", smooth_u16: np.ndarray | None = None):
+    """x: uint16 bit patterns [..., cols] -> (y int8 same shape, scale float32 [...], offset float32 [...])."""
+    x = _c(x_u16, np.uint16)
+    cols = x.shape[-1]
+    rows = x.size // cols if cols else 0
+    y = np.empty(x.shape, dtype=np.int8)
+    scale = np.zeros(x.shape[:-1], dtype=np.float32)
+    offset = np.zeros(x.shape[:-1], dtype=np.float32)
+    sm = None if smooth_u16 is None else _c(smooth_u16, np.uint16)
+    if rows and cols:
+        lib().orc_dynamic_quant_asymmetric(_p(x), 0 if in_dtype == "bf16" else 1, _p(sm), rows, cols, cols,
+                                           _p(y), _p(scale), _p(offset))
+    return y, scale, offset
 
 
 def int8_gemm(a: np.ndarray, b: np.ndarray) -> np.ndarray:

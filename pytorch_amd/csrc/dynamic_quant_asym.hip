@@ -1,0 +1,135 @@
+// npu_dynamic_quant_asymmetric for gfx950: per-token asymmetric int8 quantisation,
+//     scale = (row_max - row_min) / 255,   offset = 127 - row_max / scale,   y = rint_half_even(x / scale + offset)
+// with every operation a separately rounded IEEE binary32 operation (the compile flags keep multiply-adds apart).
+// A row whose elements are all equal has scale 0, offset 0 and y 0.
+//
+// One 256-thread block per row, two passes over the row: the first reduces the minimum and the maximum, the second
+// re-reads the row (it is in cache by then: HBM sees it once), divides, adds the offset and stores packed int8.
+// The division is IEEE-correct (about a dozen instructions per element), which at [2048, 4096] costs about as much
+// as the memory traffic.
+#include "common.h"
+#include <math.h>
+
+namespace mi355 {
+namespace {
+
+template <bool FP16>
+__device__ __forceinline__ float to_f32(uint16_t h)
+{
+    if constexpr (FP16) return (float)__builtin_bit_cast(_Float16, h);
+    else return bf16_1(h);
+}
+
+__device__ __forceinline__ uint32_t quant1(float x, float scale, float offset)
+{
+    float q = x / scale;
+    q = q + offset;
+    q = __builtin_rintf(q);
+    q = q > 127.0f ? 127.0f : q;
+    q = q < -128.0f ? -128.0f : q;
+    return (uint32_t)(int)q & 0xffu;
+}
+
+// VEC: cols % 8 == 0, rows (and smooth) 16-byte aligned, y rows 8-byte aligned
+template <bool FP16, bool VEC>
+__global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ smooth,
+                                                      int8_t *__restrict__ y, float *__restrict__ scale_out,
+                                                      float *__restrict__ offset_out, int64_t rows, int cols, int64_t row_stride)
+{
+    __shared__ float red[2][4];
+    const int t = threadIdx.x;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const uint16_t *xr = x + row * row_stride;
+        int8_t *yr = y + row * (int64_t)cols;
+        float mx = -INFINITY, mn = INFINITY;
+        if constexpr (VEC) {
+            for (int v = t; v < cols / 8; v += 256) {
+                const u32x4 a = reinterpret_cast<const u32x4 *>(xr)[v];
+                u32x4 s = u32x4{0, 0, 0, 0};
+                if (smooth) s = reinterpret_cast<const u32x4 *>(smooth)[v];
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float f = to_f32<FP16>((uint16_t)(a[i / 2] >> (16 * (i & 1))));
+                    if (smooth) f = f * to_f32<FP16>((uint16_t)(s[i / 2] >> (16 * (i & 1))));
+                    mx = fmaxf(mx, f);
+                    mn = fminf(mn, f);
+                }
+            }
+        } else {
+            for (int j = t; j < cols; j += 256) {
+                float f = to_f32<FP16>(xr[j]);
+                if (smooth) f = f * to_f32<FP16>(smooth[j]);
+                mx = fmaxf(mx, f);
+                mn = fminf(mn, f);
+            }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+            mn = fminf(mn, __shfl_xor(mn, off, 64));
+        }
+        __syncthreads();                                  // the previous row's readers are done with `red`
+        if ((t & 63) == 0) red[0][t >> 6] = mx, red[1][t >> 6] = mn;
+        __syncthreads();
+        mx = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+        mn = fminf(fminf(red[1][0], red[1][1]), fminf(red[1][2], red[1][3]));
+        float scale = (mx - mn) / 255.0f;
+        float offset = 127.0f - mx / scale;
+        const bool flat = !(mx > mn);                     // all elements equal (or no finite ordering): zeros
+        if (flat) scale = 0.0f, offset = 0.0f;
+        if (t == 0) scale_out[row] = scale, offset_out[row] = offset;
+        if constexpr (VEC) {
+            for (int v = t; v < cols / 8; v += 256) {
+                const u32x4 a = reinterpret_cast<const u32x4 *>(xr)[v];
+                u32x4 s = u32x4{0, 0, 0, 0};
+                if (smooth) s = reinterpret_cast<const u32x4 *>(smooth)[v];
+                uint32_t q[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float f = to_f32<FP16>((uint16_t)(a[i / 2] >> (16 * (i & 1))));
+                    if (smooth) f = f * to_f32<FP16>((uint16_t)(s[i / 2] >> (16 * (i & 1))));
+                    q[i] = flat ? 0u : quant1(f, scale, offset);
+                }
+                u32x2 o;
+                o.x = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
+                o.y = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
+                reinterpret_cast<u32x2 *>(yr)[v] = o;
+            }
+        } else {
+            for (int j = t; j < cols; j += 256) {
+                float f = to_f32<FP16>(xr[j]);
+                if (smooth) f = f * to_f32<FP16>(smooth[j]);
+                yr[j] = (int8_t)(flat ? 0u : quant1(f, scale, offset));
+            }
+        }
+    }
+}
+
+} // namespace
+} // namespace mi355
+
+extern "C" int mi355_dynamic_quant_asymmetric(const void *x, int in_dtype, const void *smooth, int8_t *y, float *scale,
+                                              float *offset, int64_t rows, int64_t cols, int64_t x_row_stride, void *stream)
+{
+    using namespace mi355;
+    if (rows < 0 || cols < 0) return MI355_ERR_BAD_ARGUMENT;
+    if (in_dtype != MI355_DTYPE_BF16 && in_dtype != MI355_DTYPE_FP16) return MI355_ERR_BAD_ARGUMENT;
+    if (rows == 0) return MI355_OK;
+    if (!scale || !offset) return MI355_ERR_BAD_ARGUMENT;
+    if (cols > 0 && (!x || !y || x_row_stride < cols)) return MI355_ERR_BAD_ARGUMENT;
+    if (cols > 0x7fffffff) return MI355_ERR_UNSUPPORTED;
+    if (!aligned(x, 2) || (smooth && !aligned(smooth, 2)) || !aligned(scale, 4) || !aligned(offset, 4)) return MI355_ERR_ALIGNMENT;
+    const bool vec = cols % 8 == 0 && x_row_stride % 8 == 0 && aligned(x, 16) && (!smooth || aligned(smooth, 16)) && aligned(y, 8);
+    const uint16_t *xp = static_cast<const uint16_t *>(x), *sp = static_cast<const uint16_t *>(smooth);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned blocks = (unsigned)(rows < 256 * 64 ? rows : 256 * 64);
+    const bool f16 = in_dtype == MI355_DTYPE_FP16;
+#define MI355_DQA_LAUNCH(F, V) \
+    hipLaunchKernelGGL((dq_asym_kernel<F, V>), dim3(blocks), dim3(256), 0, s, xp, sp, y, scale, offset, rows, (int)cols, x_row_stride)
+    if (f16 && vec) MI355_DQA_LAUNCH(true, true);
+    else if (f16) MI355_DQA_LAUNCH(true, false);
+    else if (vec) MI355_DQA_LAUNCH(false, true);
+    else MI355_DQA_LAUNCH(false, false);
+#undef MI355_DQA_LAUNCH
+    return check_launch();
+}

@@ -119,6 +119,57 @@ std::tuple<Tensor, Tensor> dynamic_quant_hip(const Tensor &input, const optional
     return {y, scale};
 }
 
+// ---------------------------------------------------------------- npu_dynamic_quant_asymmetric
+// torch_npu.npu_dynamic_quant_asymmetric(input, *, smooth_scales=None, group_index=None, dst_type=None)
+// -> (y int8, scale float32, offset float32)   (test/test_fake_tensor.py:1689-1709, test/torch_npu_schema.json:2147-2149)
+
+std::tuple<Tensor, Tensor, Tensor> dynamic_quant_asym_alloc(const Tensor &input)
+{
+    auto [y, scale] = dynamic_quant_alloc(input);
+    return {y, scale, at::empty_like(scale)};
+}
+
+std::tuple<Tensor, Tensor, Tensor> dynamic_quant_asym_meta(const Tensor &input, const optional<Tensor> &smooth_scales,
+                                                           const optional<Tensor> &group_index,
+                                                           optional<at::ScalarType> dst_type)
+{
+    dynamic_quant_check(input, smooth_scales, group_index, dst_type);
+    return dynamic_quant_asym_alloc(input);
+}
+
+std::tuple<Tensor, Tensor, Tensor> dynamic_quant_asym_hip(const Tensor &input, const optional<Tensor> &smooth_scales,
+                                                          const optional<Tensor> &group_index,
+                                                          optional<at::ScalarType> dst_type)
+{
+    dynamic_quant_check(input, smooth_scales, group_index, dst_type);
+    check_same_device("npu_dynamic_quant_asymmetric", {&input, opt(smooth_scales)});
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+    auto [y, scale, offset] = dynamic_quant_asym_alloc(input);
+    const int64_t cols = input.size(-1);
+    const int64_t rows = cols ? input.numel() / cols : 0;
+    if (rows == 0 || cols == 0) {
+        scale.zero_();
+        offset.zero_();
+        return {y, scale, offset};
+    }
+    Tensor x = input;
+    int64_t row_stride = cols;
+    if (x.dim() == 2 && x.stride(1) == 1 && x.stride(0) >= cols) {
+        row_stride = x.stride(0);
+    } else if (!x.is_contiguous()) {
+        x = x.contiguous();
+    }
+    Tensor smooth;
+    if (const Tensor *s = opt(smooth_scales)) smooth = s->contiguous();
+    check_status(mi355_dynamic_quant_asymmetric(x.data_ptr(),
+                                                x.scalar_type() == at::kBFloat16 ? MI355_DTYPE_BF16 : MI355_DTYPE_FP16,
+                                                smooth.defined() ? smooth.data_ptr() : nullptr, y.data_ptr<int8_t>(),
+                                                scale.data_ptr<float>(), offset.data_ptr<float>(), rows, cols, row_stride,
+                                                stream_of(input)),
+                 "npu_dynamic_quant_asymmetric");
+    return {y, scale, offset};
+}
+
 // The split-K reductions of the matmul kernels count arrivals in their workspace: the counters must
 // be zero before a launch and the kernels leave them zero.  One zero-initialised buffer per
 // (device, stream) is kept and reused; launches on one stream are ordered, so they never overlap.
@@ -589,6 +640,8 @@ TORCH_LIBRARY_FRAGMENT(npu, m)
 {
     m.def("npu_dynamic_quant(Tensor input, *, Tensor? smooth_scales=None, Tensor? group_index=None, "
           "ScalarType? dst_type=None) -> (Tensor, Tensor)");
+    m.def("npu_dynamic_quant_asymmetric(Tensor input, *, Tensor? smooth_scales=None, Tensor? group_index=None, "
+          "ScalarType? dst_type=None) -> (Tensor, Tensor, Tensor)");
     m.def("npu_quant_matmul(Tensor x1, Tensor x2, Tensor scale, *, Tensor? offset=None, Tensor? pertoken_scale=None, "
           "Tensor? bias=None, ScalarType? output_dtype=None) -> Tensor");
     m.def("npu_weight_quant_batchmatmul(Tensor x, Tensor weight, Tensor antiquant_scale, Tensor? antiquant_offset=None, "
@@ -604,6 +657,7 @@ TORCH_LIBRARY_FRAGMENT(npu, m)
 TORCH_LIBRARY_IMPL(npu, CUDA, m)
 {
     m.impl("npu_dynamic_quant", TORCH_FN(dynamic_quant_hip));
+    m.impl("npu_dynamic_quant_asymmetric", TORCH_FN(dynamic_quant_asym_hip));
     m.impl("npu_quant_matmul", TORCH_FN(quant_matmul_hip));
     m.impl("npu_weight_quant_batchmatmul", TORCH_FN(weight_quant_hip));
     m.impl("npu_swiglu", TORCH_FN(swiglu_hip));
@@ -614,6 +668,7 @@ TORCH_LIBRARY_IMPL(npu, CUDA, m)
 TORCH_LIBRARY_IMPL(npu, Meta, m)
 {
     m.impl("npu_dynamic_quant", TORCH_FN(dynamic_quant_meta));
+    m.impl("npu_dynamic_quant_asymmetric", TORCH_FN(dynamic_quant_asym_meta));
     m.impl("npu_quant_matmul", TORCH_FN(quant_matmul_meta));
     m.impl("npu_weight_quant_batchmatmul", TORCH_FN(weight_quant_meta));
     m.impl("npu_swiglu", TORCH_FN(swiglu_meta));

@@ -642,6 +642,26 @@ def test_rowwise_kernels_random_shapes(capi, golden):
             assert np.array_equal(y.cpu().numpy(), wy), tag + " (swiglu_quant)"
 
 
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (33, 1000), (7, 24), (5, 1), (3, 20000), (64, 14336), (1, 8)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_dynamic_quant_asymmetric(capi, golden, rows, cols, f16):
+    """Codes, scales and offsets bit-identical to the oracle (every operation a separate float32 operation): aligned
+    and odd widths, pitched rows, smooth scales, a constant row."""
+    g = torch.Generator().manual_seed(rows + cols)
+    dt = torch.float16 if f16 else torch.bfloat16
+    bits = _f16_bits if f16 else _bits
+    wide = (torch.randn(rows, cols + 8, generator=g) * 3 + 1).to(dt)
+    wide[0, :] = 2.5                                                # a constant row: scale 0, offset 0, codes 0
+    for x in (wide[:, :cols].contiguous(), wide[:, :cols]):
+        for sm in (None, (torch.rand(cols, generator=g) + 0.5).to(dt)):
+            y, s, o = capi.dynamic_quant_asymmetric(x.cuda(), None if sm is None else sm.cuda())
+            wy, ws, wo = golden.dynamic_quant_asymmetric(bits(x), "fp16" if f16 else "bf16", None if sm is None else bits(sm))
+            assert np.array_equal(s.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+            assert np.array_equal(o.cpu().numpy().view(np.uint32), wo.view(np.uint32))
+            assert np.array_equal(y.cpu().numpy(), wy)
+    assert not y[0].any() or sm is not None
+
+
 # ------------------------------------------------------------------ error paths (host side, no kernel runs)
 
 @pytest.mark.parametrize("rows,half", [(64, 14336), (2048, 14336), (33, 512), (5, 100), (3, 16384 + 8), (7, 24)])

@@ -261,6 +261,25 @@ def test_swiglu_quant_operator(pa, golden):
     assert torch.equal(y1, y2) and torch.equal(s1, s2)
 
 
+def test_dynamic_quant_asymmetric_operator(pa, golden):
+    """torch_npu.npu_dynamic_quant_asymmetric(input, smooth_scales=...) as test/test_fake_tensor.py:1689-1709 calls it:
+    three outputs, scale and offset shaped like the input without its last dimension."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(4, 64, 1024, generator=g).to(torch.float16)
+    sm = (torch.rand(1024, generator=g) + 0.5).to(torch.float16)
+    y, s, o = pa.npu_dynamic_quant_asymmetric(x.cuda(), smooth_scales=sm.cuda())
+    assert y.shape == (4, 64, 1024) and y.dtype == torch.int8
+    assert s.shape == (4, 64) and s.dtype == torch.float32 and o.shape == (4, 64) and o.dtype == torch.float32
+    bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)  # noqa: E731
+    wy, ws, wo = golden.dynamic_quant_asymmetric(bits(x), "fp16", bits(sm))
+    assert np.array_equal(y.cpu().numpy(), wy) and np.array_equal(s.cpu().numpy(), ws) and np.array_equal(o.cpu().numpy(), wo)
+    # what the quantisation means: (y - offset) * scale reproduces x * smooth to half a step
+    back = (y.float().cpu() - o.cpu().unsqueeze(-1)) * s.cpu().unsqueeze(-1)
+    assert ((back - x.float() * sm.float()).abs() <= 0.5001 * s.cpu().unsqueeze(-1) + 1e-6).all()
+    with pytest.raises(RuntimeError, match="group_index"):
+        pa.npu_dynamic_quant_asymmetric(x.cuda(), group_index=torch.zeros(1, dtype=torch.int32, device="cuda"))
+
+
 def test_anti_quant_operator(pa, golden):
     """torch_npu.npu_anti_quant(x, scale, offset=..., dst_dtype=..., src_dtype=...) as test/custom_ops/test_npu_anti_quant.py
     calls it: default float16 output, leading batch dimensions, packed int4 widening the last dimension by 8, and the

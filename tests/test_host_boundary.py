@@ -17,7 +17,7 @@ def test_c_abi_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "mi355_quant.h")).read()
     declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", header))
     assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant", "mi355_anti_quant",
-            "mi355_unpack_int4"} <= declared
+            "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric"} <= declared
     lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_amd", "csrc", "libmi355_quant.so"))
     for name in declared:
         assert hasattr(lib, name), name
@@ -76,6 +76,13 @@ def test_meta_dynamic_quant(pa):
         pa.npu_dynamic_quant(_m(4, 8, dtype=torch.float32))
     with pytest.raises(RuntimeError, match="smooth_scales"):
         pa.npu_dynamic_quant(x, smooth_scales=_m(8, dtype=torch.float16))
+
+
+def test_meta_dynamic_quant_asymmetric(pa):
+    # test/test_fake_tensor.py:1689-1709
+    y, s, o = pa.npu_dynamic_quant_asymmetric(_m(4, 2048, 1024, dtype=torch.float16), smooth_scales=_m(1024, dtype=torch.float16))
+    assert y.shape == (4, 2048, 1024) and y.dtype == torch.int8
+    assert s.shape == (4, 2048) and s.dtype == torch.float32 and o.shape == (4, 2048) and o.dtype == torch.float32
 
 
 def test_meta_quant_matmul(pa):

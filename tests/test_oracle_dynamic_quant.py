@@ -126,3 +126,63 @@ def test_smooth_scales(golden):
     scale = xf.abs().amax(-1) / 127.0
     assert np.array_equal(s, scale.numpy())
     assert np.array_equal(y, torch.round(xf / scale[:, None]).clamp(-127, 127).to(torch.int8).numpy())
+
+
+# ------------------------------------------------------------------ asymmetric variant
+
+def _asym_numpy(xf):
+    """scale = (max - min) / 255, offset = 127 - max / scale, y = rint(x / scale + offset) in numpy float32, one
+    operation at a time (numpy rounds every float32 operation separately; rint is half-even)."""
+    xf = xf.astype(np.float32)
+    mx, mn = xf.max(axis=-1, keepdims=True), xf.min(axis=-1, keepdims=True)
+    scale = ((mx - mn) / np.float32(255.0)).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        offset = (np.float32(127.0) - (mx / scale).astype(np.float32)).astype(np.float32)
+        q = np.rint(((xf / scale).astype(np.float32) + offset).astype(np.float32))
+    y = np.clip(q, -128, 127)
+    flat = ~(mx > mn)
+    y = np.where(flat, 0, y).astype(np.int8)
+    scale, offset = np.where(flat, 0, scale), np.where(flat, 0, offset)
+    return y, scale[..., 0].astype(np.float32), offset[..., 0].astype(np.float32)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_asymmetric_vs_numpy_float32(golden, dtype):
+    g = torch.Generator().manual_seed(7)
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float16
+    for rows, cols, mul, shift in [(33, 1000, 1.0, 0.0), (8, 4096, 30.0, 5.0), (5, 24, 0.25, -2.0), (3, 1, 1.0, 0.0)]:
+        x = (torch.randn(rows, cols, generator=g) * mul + shift).to(tdt)
+        bits = x.view(torch.int16).numpy().view(np.uint16)
+        y, s, o = golden.dynamic_quant_asymmetric(bits, dtype)
+        wy, ws, wo = _asym_numpy(x.float().numpy())
+        assert np.array_equal(s.view(np.uint32), ws.view(np.uint32)) and np.array_equal(o.view(np.uint32), wo.view(np.uint32))
+        assert np.array_equal(y, wy)
+        if cols > 1:                                     # the extremes of a row land on the ends of the int8 range
+            xf = x.float().numpy()
+            assert (y[np.arange(rows), xf.argmax(axis=1)] == 127).all() and (y[np.arange(rows), xf.argmin(axis=1)] == -128).all()
+    sm = (torch.rand(1000, generator=g) + 0.5).to(tdt)
+    x = torch.randn(7, 1000, generator=g).to(tdt)
+    y, s, o = golden.dynamic_quant_asymmetric(x.view(torch.int16).numpy().view(np.uint16), dtype, sm.view(torch.int16).numpy().view(np.uint16))
+    wy, ws, wo = _asym_numpy((x.float() * sm.float()).numpy())
+    assert np.array_equal(y, wy) and np.array_equal(s, ws) and np.array_equal(o, wo)
+
+
+def test_asymmetric_hand_computed_rows(golden):
+    """Rows whose answers can be written down: [0 .. 255] has scale 1 and offset -128 (y = x - 128); [-1, 0, 1] has
+    scale 2/255; [-255, 0, 255, ...] has scale 2 and offset -0.5 exactly, so 0, 1 and -2 land on ties and round to
+    even; a constant row gives zeros."""
+    x = torch.arange(256, dtype=torch.float32).to(torch.bfloat16).reshape(1, 256)
+    assert torch.equal(x.float(), torch.arange(256, dtype=torch.float32).reshape(1, 256))     # exact in bf16
+    y, s, o = golden.dynamic_quant_asymmetric(x.view(torch.int16).numpy().view(np.uint16))
+    assert s[0] == 1.0 and o[0] == -128.0 and np.array_equal(y[0].astype(np.int32), np.arange(256) - 128)
+    x = torch.tensor([[-1.0, 0.0, 1.0, 0.5]], dtype=torch.float16)
+    y, s, o = golden.dynamic_quant_asymmetric(x.view(torch.int16).numpy().view(np.uint16), "fp16")
+    assert s[0] == np.float32(2.0) / np.float32(255.0) and abs(o[0] + 0.5) < 1e-4     # 1 / fl(2/255) is not exactly 127.5
+    assert y[0].tolist() == [-128, 0, 127, 63]           # 0 -> -0.49999 -> 0;  0.5 / scale + offset = 63.25
+    x = torch.tensor([[-255.0, 0.0, 255.0, 1.0, 3.0, -2.0]], dtype=torch.bfloat16)   # scale 2, offset -0.5 exactly
+    y, s, o = golden.dynamic_quant_asymmetric(x.view(torch.int16).numpy().view(np.uint16))
+    assert s[0] == 2.0 and o[0] == -0.5
+    assert y[0].tolist() == [-128, 0, 127, 0, 1, -2]     # ties -0.5 -> -0, 0.0 -> 0, 1.0, -1.5 -> -2: half to even
+    x = torch.full((2, 16), 3.5, dtype=torch.bfloat16)
+    y, s, o = golden.dynamic_quant_asymmetric(x.view(torch.int16).numpy().view(np.uint16))
+    assert not y.any() and not s.any() and not o.any()
