@@ -9,6 +9,7 @@ struct WqKpackedPlan {
     bool ok;                 // the kernel accepts this problem
     int mt;                  // m tiles (16 rows) per workgroup: 1, 2 or 4
     int nw;                  // 16-column tiles per workgroup: 4 or 8
+    int ntw;                 // column tiles per wavefront: 2 with four m tiles, else 1
     int ks;                  // slices of the workgroup's K range (nw * ks wavefronts): 1 or 2
     int mchunks, tiles;      // workgroups along M and N
     int S;                   // workgroups that share the K range of a tile

@@ -53,18 +53,21 @@ __device__ __forceinline__ u32x4 even_odd(u32x4 v)
     return r;
 }
 
-// MT: m tiles (16 rows) per workgroup; NW: 16-column tiles per workgroup; KS: slices of the workgroup's K range -
+// MT: m tiles (16 rows) per workgroup; NW x NTW: 16-column tiles per workgroup, NTW of them per wavefront (with four
+// m tiles a wavefront takes two: an activation fragment read from LDS then feeds two weight tiles, and the row sums
+// are formed once per wavefront instead of once per column tile); KS: slices of the workgroup's K range -
 // NW * KS wavefronts, the slices are added in LDS at the end (two wavefronts per SIMD where the column tiles alone
 // would leave one: a single wavefront cannot hide its own MFMA and LDS latencies); G128: a scale group is one
 // sub-step (group_size 128), so every half step starts its sums from zero and ends with a fold - no counters, and
 // the first MFMA of a half takes a zero accumulator instead of a cleared register
-template <int MT, int NW, int KS, int ACT, bool G128>
+template <int MT, int NW, int KS, int NTW, int ACT, bool G128>
 __global__ __launch_bounds__(NW * KS * 64) void wq_kpacked_kernel(const WqArgs p)
 {
     static_assert(MT * KS <= 4, "a chunk holds at least one step of every slice");
-    constexpr int WAVES = NW * KS, NBW = NW * 16, THREADS = WAVES * 64;
+    constexpr int WAVES = NW * KS, NBW = NW * NTW * 16, THREADS = WAVES * 64;
+    constexpr int DA = MT * NTW >= 8 ? 1 : 2;           // accumulators per sum, used alternately (short dependent chains)
     constexpr int CH = 4 / (MT * KS);                   // steps per slice and chunk of activations (32 KiB of LDS per buffer)
-    constexpr int RS = MT == 4 ? 4 : 8;                 // steps per round of the main loop: two batches of weight loads in
+    constexpr int RS = MT == 4 ? (NW == 8 ? 2 : 4) : 8;                 // steps per round of the main loop: two batches of weight loads in
     constexpr int BODY = RS / 2;                        // registers (one consumed, one in flight; 2 KiB per step and
                                                         // wavefront), the slot of a step known at compile time
     constexpr int POLICY = MT == 1 ? kNonTemporal : 0;
@@ -107,26 +110,32 @@ __global__ __launch_bounds__(NW * KS * 64) void wq_kpacked_kernel(const WqArgs p
     // 16-byte chunk a lane fetches is XOR-swizzled with the row pair so that the operand reads (16 rows x 16 bytes)
     // are free of bank conflicts; LDS slot s of row r holds chunk s ^ ((r >> 1) & 7).
     const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(p.w, (uint32_t)((uint64_t)(p.N - 1) * p.ldw_bytes + p.row_bytes));
-    uint32_t voff_w[2];
+    uint32_t voff_w[NTW][2];
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
-        const int rl = 8 * h + (lane >> 3);
-        voff_w[h] = (uint32_t)min(n0 + ct * 16 + rl, p.N - 1) * p.ldw_bytes + (uint32_t)(((lane & 7) ^ ((rl >> 1) & 7)) * 16);
-    }
-    char *tbuf = lds + 16 + 2 * XBUF + wave * (2 * TBUF);
-    uint32_t *prm = reinterpret_cast<uint32_t *>(lds + 16 + 2 * XBUF + WAVES * 2 * TBUF);   // [group][column]: scale | offset << 16
+    for (int tt = 0; tt < NTW; tt++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int rl = 8 * h + (lane >> 3);
+            voff_w[tt][h] = (uint32_t)min(n0 + (ct * NTW + tt) * 16 + rl, p.N - 1) * p.ldw_bytes +
+                            (uint32_t)(((lane & 7) ^ ((rl >> 1) & 7)) * 16);
+        }
+    char *tbuf = lds + 16 + 2 * XBUF + wave * (NTW * 2 * TBUF);                               // [step parity][tile][2 KiB]
+    uint32_t *prm = reinterpret_cast<uint32_t *>(lds + 16 + 2 * XBUF + WAVES * NTW * 2 * TBUF);   // [group][column]: scale | offset << 16
     const int t_rd = c * 128 + ((g ^ ((c >> 1) & 7)) * 16);   // chunk g of row c; chunk g + 4 is at slot ^ 4, i.e. +-64 bytes
     const __amdgpu_buffer_rsrc_t rsrc_x =
         make_rsrc(p.x + (int64_t)m_base * p.ldx, (uint32_t)(((int64_t)(rows_valid - 1) * p.ldx + p.K) * 2));
 
-    u32x4 wq[2][BODY][2];
+    u32x4 wq[2][BODY][NTW][2];
     auto load_body = [&](int slot, int st) {    // st: first step of the batch, relative to step0
 #pragma unroll
         for (int j = 0; j < BODY; j++) {
             const bool ok = st + j < nsteps;
             const uint32_t kb = (uint32_t)(step0 + st + j) * 128u;
-            wq[slot][j][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ok ? voff_w[0] : kOutOfRange, kb, POLICY);
-            wq[slot][j][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ok ? voff_w[1] : kOutOfRange, kb, POLICY);
+#pragma unroll
+            for (int tt = 0; tt < NTW; tt++) {
+                wq[slot][j][tt][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ok ? voff_w[tt][0] : kOutOfRange, kb, POLICY);
+                wq[slot][j][tt][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ok ? voff_w[tt][1] : kOutOfRange, kb, POLICY);
+            }
         }
     };
     // Activation staging: piece q of a row's chunk of one slice (8 consecutive k) belongs to step q / 32, half
@@ -160,21 +169,42 @@ __global__ __launch_bounds__(NW * KS * 64) void wq_kpacked_kernel(const WqArgs p
         }
     };
 
-    // two accumulators per sum, used alternately: a chain of dependent MFMAs is two long instead of four
-    f32x4 P[MT][2], X[MT][2], tot[MT];
+    f32x4 P[MT][NTW][DA], X[MT][DA], tot[MT][NTW];
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) P[mt][0] = P[mt][1] = X[mt][0] = X[mt][1] = tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int a = 0; a < DA; a++) {
+            X[mt][a] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int tt = 0; tt < NTW; tt++) P[mt][tt][a] = tot[mt][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
     const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
     auto fold = [&](int gl) {
-        const uint32_t pr = prm[gl * NBW + ct * 16 + c];
-        const float sc = act_lo<ACT>(pr) * P_MUL;
-        const float of = (act_hi<ACT>(pr) - X_BIAS) * (1.0f / P_MUL);
+        f32x4 xs[MT];
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            const f32x4 ps = P[mt][0] + P[mt][1], xs = X[mt][0] + X[mt][1];
+        for (int mt = 0; mt < MT; mt++) xs[mt] = DA == 2 ? X[mt][0] + X[mt][DA - 1] : X[mt][0];
 #pragma unroll
-            for (int q = 0; q < 4; q++) tot[mt][q] = __builtin_fmaf(sc, __builtin_fmaf(of, xs[q], ps[q]), tot[mt][q]);
-            if constexpr (!G128) P[mt][0] = P[mt][1] = X[mt][0] = X[mt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int tt = 0; tt < NTW; tt++) {
+            const uint32_t pr = prm[gl * NBW + (ct * NTW + tt) * 16 + c];
+            const float sc = act_lo<ACT>(pr) * P_MUL;
+            const float of = (act_hi<ACT>(pr) - X_BIAS) * (1.0f / P_MUL);
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+                const f32x4 ps = DA == 2 ? P[mt][tt][0] + P[mt][tt][DA - 1] : P[mt][tt][0];
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    tot[mt][tt][q] = __builtin_fmaf(sc, __builtin_fmaf(of, xs[mt][q], ps[q]), tot[mt][tt][q]);
+            }
+        }
+        if constexpr (!G128) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int a = 0; a < DA; a++) {
+                    X[mt][a] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int tt = 0; tt < NTW; tt++) P[mt][tt][a] = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
         }
     };
 
@@ -224,22 +254,27 @@ __global__ __launch_bounds__(NW * KS * 64) void wq_kpacked_kernel(const WqArgs p
     load_body(1, BODY);
     __builtin_amdgcn_sched_barrier(0);
     // step 0 of the weights goes through the wavefront's turn-around tile into operand order
-    *reinterpret_cast<u32x4 *>(tbuf + lane * 16) = wq[0][0][0];
-    *reinterpret_cast<u32x4 *>(tbuf + 1024 + lane * 16) = wq[0][0][1];
-    u32x4 w[2];
-    w[0] = *reinterpret_cast<const u32x4 *>(tbuf + t_rd);
-    w[1] = *reinterpret_cast<const u32x4 *>(tbuf + (t_rd ^ 64));
+    u32x4 w[NTW][2];
+#pragma unroll
+    for (int tt = 0; tt < NTW; tt++) {
+        *reinterpret_cast<u32x4 *>(tbuf + tt * TBUF + lane * 16) = wq[0][0][tt][0];
+        *reinterpret_cast<u32x4 *>(tbuf + tt * TBUF + 1024 + lane * 16) = wq[0][0][tt][1];
+        w[tt][0] = *reinterpret_cast<const u32x4 *>(tbuf + tt * TBUF + t_rd);
+        w[tt][1] = *reinterpret_cast<const u32x4 *>(tbuf + tt * TBUF + (t_rd ^ 64));
+    }
 
     // activation fragments of one half step (four MFMA k blocks per m tile); with one or two m tiles the next half
     // of the same chunk is requested while the current one is multiplied
+    // (with four m tiles: one buffer, filled two k blocks at a time)
     constexpr int XA = MT <= 2 ? 2 : 1;
-    u32x4 xa[XA][4][MT];
-    auto read_xa = [&](int buf, const char *xb, int jc, int h) {
+    constexpr int DG = MT <= 2 ? 4 : 2;                 // k blocks per request
+    u32x4 xa[XA][DG][MT];
+    auto read_xa = [&](int buf, const char *xb, int jc, int h, int d0) {
 #pragma unroll
-        for (int d = 0; d < 4; d++)
+        for (int d = 0; d < DG; d++)
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
-                xa[buf][d][mt] = *reinterpret_cast<const u32x4 *>(xb + (((ks * CH + jc) * MT + mt) * 8 + 4 * h + d) * FP);
+                xa[buf][d][mt] = *reinterpret_cast<const u32x4 *>(xb + (((ks * CH + jc) * MT + mt) * 8 + 4 * h + d0 + d) * FP);
     };
 
     int in_group = 0, gl = gl0, ch = 0;
@@ -253,16 +288,17 @@ __global__ __launch_bounds__(NW * KS * 64) void wq_kpacked_kernel(const WqArgs p
             const char *xb = lds + 16 + (ch & 1) * XBUF + lane * 16;
             // this step's weights are in w (operand order); the next step's registers go through the other half of
             // the turn-around tile and are read back at once, so that their latency hides behind this step
-            u32x4 wc[2];
-            wc[0] = w[0] ^ 0x88888888u;
-            wc[1] = w[1] ^ 0x88888888u;
-            {
+            u32x4 wc[NTW][2];
+#pragma unroll
+            for (int tt = 0; tt < NTW; tt++) {
+                wc[tt][0] = w[tt][0] ^ 0x88888888u;
+                wc[tt][1] = w[tt][1] ^ 0x88888888u;
                 const int sn = ((j + 1) / BODY) & 1, jsn = (j + 1) % BODY;
-                char *tn = tbuf + ((j + 1) & 1) * TBUF;
-                *reinterpret_cast<u32x4 *>(tn + lane * 16) = wq[sn][jsn][0];
-                *reinterpret_cast<u32x4 *>(tn + 1024 + lane * 16) = wq[sn][jsn][1];
-                w[0] = *reinterpret_cast<const u32x4 *>(tn + t_rd);
-                w[1] = *reinterpret_cast<const u32x4 *>(tn + (t_rd ^ 64));
+                char *tn = tbuf + (((j + 1) & 1) * NTW + tt) * TBUF;
+                *reinterpret_cast<u32x4 *>(tn + lane * 16) = wq[sn][jsn][tt][0];
+                *reinterpret_cast<u32x4 *>(tn + 1024 + lane * 16) = wq[sn][jsn][tt][1];
+                w[tt][0] = *reinterpret_cast<const u32x4 *>(tn + t_rd);
+                w[tt][1] = *reinterpret_cast<const u32x4 *>(tn + (t_rd ^ 64));
             }
             if (js == BODY - 1) {               // the batch has left the registers: refill its slot two batches ahead
                 __builtin_amdgcn_sched_barrier(0);
@@ -272,17 +308,27 @@ __global__ __launch_bounds__(NW * KS * 64) void wq_kpacked_kernel(const WqArgs p
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 const int cur = XA == 2 ? (2 * j + h) & 1 : 0;
-                if (XA == 1 || (jc == 0 && h == 0)) read_xa(cur, xb, jc, h);
-                if (XA == 2 && !(jc == CH - 1 && h == 1)) read_xa(cur ^ 1, xb, h ? jc + 1 : jc, h ^ 1);
-                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (XA == 2) {
+                    if (jc == 0 && h == 0) read_xa(cur, xb, jc, h, 0);
+                    if (!(jc == CH - 1 && h == 1)) read_xa(cur ^ 1, xb, h ? jc + 1 : jc, h ^ 1, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
-                    const u32x4 b = expand_word<ACT>(wc[h][d]);
+                    if constexpr (XA == 1) {
+                        if (d % DG == 0) read_xa(0, xb, jc, h, d);
+                    }
+                    u32x4 b[NTW];
+#pragma unroll
+                    for (int tt = 0; tt < NTW; tt++) b[tt] = expand_word<ACT>(wc[tt][h][d]);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         const f32x4 zero = f32x4{0.f, 0.f, 0.f, 0.f};
-                        P[mt][d & 1] = mfma_act<ACT>(xa[cur][d][mt], b, G128 && d < 2 ? zero : P[mt][d & 1]);
-                        X[mt][d & 1] = mfma_act<ACT>(xa[cur][d][mt], ones, G128 && d < 2 ? zero : X[mt][d & 1]);
+                        const bool first = G128 && d < DA;          // a group starts with this half step
+#pragma unroll
+                        for (int tt = 0; tt < NTW; tt++)
+                            P[mt][tt][d % DA] = mfma_act<ACT>(xa[cur][d % DG][mt], b[tt], first ? zero : P[mt][tt][d % DA]);
+                        X[mt][d % DA] = mfma_act<ACT>(xa[cur][d % DG][mt], ones, first ? zero : X[mt][d % DA]);
                     }
                 }
                 if constexpr (G128) {
@@ -311,7 +357,9 @@ __global__ __launch_bounds__(NW * KS * 64) void wq_kpacked_kernel(const WqArgs p
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             const int row = 4 * g + q;
-            if (row < rows_mt) red[(ks * 16 + row) * NBW + ct * 16 + c] = tot[mt][q];
+#pragma unroll
+            for (int tt = 0; tt < NTW; tt++)
+                if (row < rows_mt) red[(ks * 16 + row) * NBW + (ct * NTW + tt) * 16 + c] = tot[mt][tt][q];
         }
         __syncthreads();
         outp.emit_mtile(red, mt * 16, rows_mt);
@@ -319,10 +367,10 @@ __global__ __launch_bounds__(NW * KS * 64) void wq_kpacked_kernel(const WqArgs p
     outp.finish(rows_valid, tile);
 }
 
-template <int MT, int NW, int KS, int ACT, bool G128>
+template <int MT, int NW, int KS, int NTW, int ACT, bool G128>
 int launch_one(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
 {
-    auto kern = wq_kpacked_kernel<MT, NW, KS, ACT, G128>;
+    auto kern = wq_kpacked_kernel<MT, NW, KS, NTW, ACT, G128>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
@@ -334,18 +382,12 @@ int launch_one(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
 template <int ACT, bool G128>
 int launch_shape(const WqArgs &p, const WqKpackedPlan &pl, hipStream_t s)
 {
-    if (pl.nw == 4 && pl.ks == 2) {
-        if (pl.mt == 1) return launch_one<1, 4, 2, ACT, G128>(p, pl, s);
-        return launch_one<2, 4, 2, ACT, G128>(p, pl, s);
-    }
-    if (pl.nw == 4) {
-        if (pl.mt == 1) return launch_one<1, 4, 1, ACT, G128>(p, pl, s);
-        if (pl.mt == 2) return launch_one<2, 4, 1, ACT, G128>(p, pl, s);
-        return launch_one<4, 4, 1, ACT, G128>(p, pl, s);
-    }
-    if (pl.mt == 1) return launch_one<1, 8, 1, ACT, G128>(p, pl, s);
-    if (pl.mt == 2) return launch_one<2, 8, 1, ACT, G128>(p, pl, s);
-    return launch_one<4, 8, 1, ACT, G128>(p, pl, s);
+    if (pl.mt == 4)     // two column tiles per wavefront
+        return pl.nw == 4 ? launch_one<4, 4, 1, 2, ACT, G128>(p, pl, s) : launch_one<4, 8, 1, 2, ACT, G128>(p, pl, s);
+    if (pl.nw == 4 && pl.ks == 2)
+        return pl.mt == 1 ? launch_one<1, 4, 2, 1, ACT, G128>(p, pl, s) : launch_one<2, 4, 2, 1, ACT, G128>(p, pl, s);
+    if (pl.nw == 4) return pl.mt == 1 ? launch_one<1, 4, 1, 1, ACT, G128>(p, pl, s) : launch_one<2, 4, 1, 1, ACT, G128>(p, pl, s);
+    return pl.mt == 1 ? launch_one<1, 8, 1, 1, ACT, G128>(p, pl, s) : launch_one<2, 8, 1, 1, ACT, G128>(p, pl, s);
 }
 
 template <int ACT>
@@ -390,12 +432,15 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
         pl.unit_steps = (int)(K / 256);
         pl.n_units = 1;
     }
-    // eight wavefronts (128 columns) per workgroup when that still gives every CU a workgroup, else four
-    const int tiles8 = (int)((N + 127) / 128);
+    // eight wavefronts per workgroup when that still gives every CU a workgroup, else four; with four m tiles a
+    // wavefront owns two column tiles
+    pl.ntw = pl.mt == 4 ? 2 : 1;
+    const int tiles8 = (int)((N + 8 * pl.ntw * 16 - 1) / (8 * pl.ntw * 16));
     pl.nw = (int64_t)tiles8 * pl.mchunks >= 200 ? 8 : 4;
     if (const int f = env_int("MI355_WQK_NW"))      // tuning aid
         if (f == 4 || f == 8) pl.nw = f;
-    pl.tiles = (int)((N + pl.nw * 16 - 1) / (pl.nw * 16));
+    const int wg_cols = pl.nw * pl.ntw * 16;
+    pl.tiles = (int)((N + wg_cols - 1) / wg_cols);
     pl.ks = 1;
     int S = kNumCU / (pl.tiles * pl.mchunks);
     if (S > pl.n_units) S = pl.n_units;
@@ -409,7 +454,8 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     auto lds_need = [&](int s) {
         const int64_t units = (pl.n_units + s - 1) / s;
         const int64_t groups = pl.grouped ? units * pl.unit_steps * 2 / pl.unit_sub : 1;
-        return (size_t)16 + 2 * 32 * (1024 + 16) + (size_t)pl.nw * 2 * 4096 + (size_t)groups * pl.nw * 16 * 4;
+        const int waves = pl.nw * (pl.nw == 4 && pl.mt <= 2 ? 2 : 1);                    // two K slices at most
+        return (size_t)16 + 2 * 32 * (1024 + 16) + (size_t)waves * pl.ntw * 4096 + (size_t)groups * wg_cols * 4;
     };
     while (lds_need(S) > 160 * 1024 && S < pl.n_units && S < 16) S++;
     if (lds_need(S) > 160 * 1024) {
