@@ -51,8 +51,36 @@ def main():
     g = torch.Generator().manual_seed(25)
     xs = (torch.randn(6, 64, generator=g) * 3).to(torch.bfloat16)
     np.savez_compressed(os.path.join(HERE, "swiglu.npz"), x=bits(xs), out=golden.swiglu(bits(xs)))
+    write_later_fixtures()
     print("fixtures written to", HERE)
 
 
+def write_later_fixtures():
+    """Fixtures of the operators added after the first set (kept in files of their own so that the first set's
+    bytes never change): standalone antiquantisation, A4W4 quant_matmul, asymmetric dynamic quantisation."""
+    g = torch.Generator().manual_seed(26)
+    rnd = lambda *sh: torch.randint(-2 ** 31, 2 ** 31 - 1, sh, generator=g, dtype=torch.int64).to(torch.int32).numpy()  # noqa: E731
+    xq = rnd(6, 5)                                                   # packed int4 [6, 40]
+    sc, of = (torch.rand(40, generator=g) * 4 - 2).numpy(), (torch.rand(40, generator=g) * 16 - 8).numpy()
+    np.savez_compressed(os.path.join(HERE, "anti_quant.npz"), x=xq, scale=sc, offset=of,
+                        out_fp16=golden.anti_quant(xq, sc, of, dst="fp16"), out_bf16=golden.anti_quant(xq, sc, of, dst="bf16"))
+
+    x1, x2n, x2k = rnd(16, 8), rnd(64, 5), rnd(40, 8)                # [16,64] x [64,40], words along N / along K
+    scale = (torch.rand(1, generator=g) * 0.02).numpy()
+    bias = torch.randint(-1000, 1000, (40,), generator=g, dtype=torch.int32).numpy()
+    out_n, acc_n = golden.quant_matmul_a4w4(x1, x2n, scale, None, bias, out="fp16")
+    out_k, acc_k = golden.quant_matmul_a4w4(x1, x2k.T, scale, None, bias, out="fp16")
+    np.savez_compressed(os.path.join(HERE, "a4w4.npz"), x1=x1, x2_n=x2n, x2_k=x2k, scale=scale, bias=bias,
+                        out_n=out_n, acc_n=acc_n, out_k=out_k, acc_k=acc_k)
+
+    x = (torch.randn(12, 264, generator=g) * 2 + 0.5).to(torch.bfloat16)
+    sm = (torch.rand(264, generator=g) + 0.5).to(torch.bfloat16)
+    y, s, o = golden.dynamic_quant_asymmetric(bits(x), "bf16", bits(sm))
+    np.savez_compressed(os.path.join(HERE, "dynamic_quant_asymmetric.npz"), x=bits(x), smooth=bits(sm), y=y, scale=s, offset=o)
+
+
 if __name__ == "__main__":
-    main()
+    if "--later-only" in sys.argv:
+        write_later_fixtures()
+    else:
+        main()

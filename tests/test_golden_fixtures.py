@@ -117,3 +117,37 @@ def test_gpu_reproduces_frozen_fixtures(capi):
     out = capi.swiglu(_bf16(f["x"]).cuda())
     d = np.abs(_bits(out).astype(np.int32) - f["out"].astype(np.int32))
     assert d.max() <= 1
+
+
+def test_oracle_reproduces_later_fixtures(golden):
+    f = _npz("anti_quant.npz")
+    assert np.array_equal(golden.anti_quant(f["x"], f["scale"], f["offset"], dst="fp16"), f["out_fp16"])
+    assert np.array_equal(golden.anti_quant(f["x"], f["scale"], f["offset"], dst="bf16"), f["out_bf16"])
+    f = _npz("a4w4.npz")
+    out, acc = golden.quant_matmul_a4w4(f["x1"], f["x2_n"], f["scale"], None, f["bias"], out="fp16")
+    assert np.array_equal(out, f["out_n"]) and np.array_equal(acc, f["acc_n"])
+    out, acc = golden.quant_matmul_a4w4(f["x1"], f["x2_k"].T, f["scale"], None, f["bias"], out="fp16")
+    assert np.array_equal(out, f["out_k"]) and np.array_equal(acc, f["acc_k"])
+    f = _npz("dynamic_quant_asymmetric.npz")
+    y, s, o = golden.dynamic_quant_asymmetric(f["x"], "bf16", f["smooth"])
+    assert np.array_equal(y, f["y"]) and np.array_equal(s, f["scale"]) and np.array_equal(o, f["offset"])
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_later_fixtures(capi):
+    import pytorch_amd as pa
+    f = _npz("anti_quant.npz")
+    x, sc, of = (torch.from_numpy(f[k]).cuda() for k in ("x", "scale", "offset"))
+    assert np.array_equal(capi.anti_quant(x, sc, of, dst_dtype=torch.float16).cpu().view(torch.int16).numpy().view(np.uint16), f["out_fp16"])
+    assert np.array_equal(_bits(capi.anti_quant(x, sc, of, dst_dtype=torch.bfloat16)), f["out_bf16"])
+    f = _npz("a4w4.npz")
+    x1, scale, bias = (torch.from_numpy(f[k]).cuda() for k in ("x1", "scale", "bias"))
+    for x2, tag in ((torch.from_numpy(f["x2_n"]).cuda(), "n"), (torch.from_numpy(f["x2_k"]).cuda().t(), "k")):
+        out = pa.npu_quant_matmul(x1, x2, scale, bias=bias, output_dtype=torch.float16)
+        assert np.array_equal(out.cpu().view(torch.int16).numpy().view(np.uint16), f["out_" + tag])
+        assert np.array_equal(pa.npu_quant_matmul(x1, x2, scale, output_dtype=torch.int32).cpu().numpy(),
+                              f["acc_" + tag])
+    f = _npz("dynamic_quant_asymmetric.npz")
+    y, s, o = capi.dynamic_quant_asymmetric(_bf16(f["x"]).cuda(), _bf16(f["smooth"]).cuda())
+    assert np.array_equal(y.cpu().numpy(), f["y"]) and np.array_equal(s.cpu().numpy(), f["scale"])
+    assert np.array_equal(o.cpu().numpy(), f["offset"])
