@@ -175,6 +175,23 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(BF[j], AF[i], acc[i][j], 0, 0, 0);             \
     }
 
+    // Instruction order of half a K step: the fragment reads of the next half, each followed by PER MFMAs, then the
+    // refills, each followed by two MFMAs, then the remaining MFMAs.  A wavefront that issues its memory
+    // instructions in a burst waits while their queues drain and issues no MFMA meanwhile.  (The refills follow
+    // the reads in program order because the compiler orders a direct-to-LDS load against later LDS reads.)
+#define MI355_INTERLEAVE(NDMA, PER)                                                                              \
+    {                                                                                                            \
+        _Pragma("unroll") for (int q = 0; q < WTM + WTN; q++) {                                                  \
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                   \
+            __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);                                                 \
+        }                                                                                                        \
+        _Pragma("unroll") for (int q = 0; q < (NDMA); q++) {                                                     \
+            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);                                                   \
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                                                   \
+        }                                                                                                        \
+        __builtin_amdgcn_sched_group_barrier(0x008, WTM * WTN, 0);                                               \
+    }
+
     // Two activation slots and NS weight slots (NS = 3 described).  In the middle of K step kt, once every wavefront is done
     // with stage kt, its slots are refilled with the activations of step kt+2 and the weights of step kt+3:
     // activations come from cache and get one step to land, weights come from HBM and get two.  Loads retire in
@@ -193,23 +210,40 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     MI355_READ_FRAGS(af0, bf0, 0, 0)
 
     for (int kt = 0; kt < KT; kt++) {
-        MI355_READ_FRAGS(af1, bf1, kt, 1)
-        __builtin_amdgcn_sched_barrier(0);
-        MI355_MFMA_BLOCK(af0, bf0)
-        __builtin_amdgcn_sched_barrier(0);
-        wait_vmcnt_lgkm0<(NS - 2) * LB>(); // stage kt+1 has landed and this wavefront is done reading stage kt
-        __syncthreads();
-        issue_a(kt + 2, KT);
-        issue_b(kt + NS, KT);
-        MI355_READ_FRAGS(af0, bf0, kt + 1, 0)
-        __builtin_amdgcn_sched_barrier(0);
-        MI355_MFMA_BLOCK(af1, bf1)
-        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (NS == 3) {
+            MI355_READ_FRAGS(af1, bf1, kt, 1)
+            MI355_MFMA_BLOCK(af0, bf0)
+            MI355_INTERLEAVE(0, 2)
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vmcnt_lgkm0<LB>();            // stage kt+1 has landed and this wavefront is done reading stage kt
+            __syncthreads();
+            MI355_READ_FRAGS(af0, bf0, kt + 1, 0)
+            issue_a(kt + 2, KT);
+            issue_b(kt + NS, KT);
+            MI355_MFMA_BLOCK(af1, bf1)
+            MI355_INTERLEAVE(LA + LB, 1)
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            // two resident workgroups per CU overlap each other's bursts; spreading the instructions gains nothing
+            MI355_READ_FRAGS(af1, bf1, kt, 1)
+            __builtin_amdgcn_sched_barrier(0);
+            MI355_MFMA_BLOCK(af0, bf0)
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vmcnt_lgkm0<0>();
+            __syncthreads();
+            issue_a(kt + 2, KT);
+            issue_b(kt + NS, KT);
+            MI355_READ_FRAGS(af0, bf0, kt + 1, 0)
+            __builtin_amdgcn_sched_barrier(0);
+            MI355_MFMA_BLOCK(af1, bf1)
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
     wait_vmcnt<0>();                       // the refills past the end (zeros) must not land in the epilogue's LDS
     __syncthreads();
 #undef MI355_READ_FRAGS
 #undef MI355_MFMA_BLOCK
+#undef MI355_INTERLEAVE
 
     if (p.S > 1) {
         // Split K: every workgroup of the tile publishes its int32 partial sums in register order (16 bytes per
@@ -492,8 +526,8 @@ struct TileChoice {
     int bm, bn, slots;
     double single_us, round_us;
 };
-constexpr TileChoice kTiles[] = {{256, 256, 256, 62.2, 70.7}, {256, 224, 256, 60.4, 67.5}, {256, 192, 256, 53.0, 58.0},
-                                 {128, 320, 256, 45.0, 50.0}, {128, 256, 256, 40.0, 45.6}, {128, 192, 512, 55.8, 58.8},
+constexpr TileChoice kTiles[] = {{256, 256, 256, 60.0, 57.0}, {256, 224, 256, 55.5, 55.5}, {256, 192, 256, 51.5, 52.5},
+                                 {128, 320, 256, 48.0, 43.0}, {128, 256, 256, 40.0, 45.6}, {128, 192, 512, 55.8, 58.8},
                                  {128, 128, 512, 40.0, 43.3}, {64, 256, 512, 40.0, 52.6},  {64, 128, 512, 24.0, 30.0}};
 
 // Pick the tile shape that minimises (rounds of resident workgroups) x (time per round).
