@@ -22,6 +22,7 @@
 // operations (contraction is disabled for this library) and rounds once to bf16.
 #include "common.h"
 #include <stdio.h>
+#include <type_traits>
 #include <stdlib.h>
 
 namespace mi355 {
@@ -210,7 +211,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     MI355_READ_FRAGS(af0, bf0, 0, 0)
 
     for (int kt = 0; kt < KT; kt++) {
-        if constexpr (NS == 3) {
+        if constexpr (NS == 3 && WTM * WTN > 16) {
             MI355_READ_FRAGS(af1, bf1, kt, 1)
             MI355_MFMA_BLOCK(af0, bf0)
             MI355_INTERLEAVE(0, 2)
@@ -224,12 +225,13 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             MI355_INTERLEAVE(LA + LB, 1)
             __builtin_amdgcn_sched_barrier(0);
         } else {
-            // two resident workgroups per CU overlap each other's bursts; spreading the instructions gains nothing
+            // small wavefront tiles (and two resident workgroups per CU, which overlap each other's bursts) gain
+            // nothing from spreading the instructions
             MI355_READ_FRAGS(af1, bf1, kt, 1)
             __builtin_amdgcn_sched_barrier(0);
             MI355_MFMA_BLOCK(af0, bf0)
             __builtin_amdgcn_sched_barrier(0);
-            wait_vmcnt_lgkm0<0>();
+            wait_vmcnt_lgkm0<(NS - 2) * LB>();
             __syncthreads();
             issue_a(kt + 2, KT);
             issue_b(kt + NS, KT);
@@ -388,18 +390,41 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     char *stg = lds + wave * (WTM * 16 * ROWB);
     const bool wide = (p.ldc & 7) == 0 && aligned_dev(p.out, 16);
     if (wide) {
+        // The output type, and the common case of a per-token scale with a float bias, are chosen once per
+        // wavefront here and not once per element: a scalar branch per converted pair costs more than the
+        // arithmetic between two of them.
+        auto stage_tile = [&](auto f16_c, auto fast_c) {
+            constexpr bool F16 = decltype(f16_c)::value, FAST = decltype(fast_c)::value;
 #pragma unroll
-        for (int i = 0; i < WTM; i++)
+            for (int i = 0; i < WTM; i++)
 #pragma unroll
-            for (int j = 0; j < WTN; j++) {
-                float f[4];
+                for (int j = 0; j < WTN; j++) {
+                    float f[4];
 #pragma unroll
-                for (int r = 0; r < 4; r++) f[r] = dequant(acc[i][j][r], biv[j][r], psv[i], scv[j][r], bsv[j][r]);
-                u32x2 pk;
-                pk.x = pack2(f[0], f[1]);
-                pk.y = pack2(f[2], f[3]);
-                *reinterpret_cast<u32x2 *>(stg + (i * 16 + mrow) * ROWB + (j * 16 + nquad) * 2) = pk;
-            }
+                    for (int r = 0; r < 4; r++) {
+                        if constexpr (FAST) {
+                            float v = (float)acc[i][j][r];
+                            v = v * psv[i];
+                            v = v * scv[j][r];
+                            f[r] = v + bsv[j][r];
+                        } else {
+                            f[r] = dequant(acc[i][j][r], biv[j][r], psv[i], scv[j][r], bsv[j][r]);
+                        }
+                    }
+                    u32x2 pk;
+                    pk.x = F16 ? pack_f16x2(f[0], f[1]) : pack_bf16x2(f[0], f[1]);
+                    pk.y = F16 ? pack_f16x2(f[2], f[3]) : pack_bf16x2(f[2], f[3]);
+                    *reinterpret_cast<u32x2 *>(stg + (i * 16 + mrow) * ROWB + (j * 16 + nquad) * 2) = pk;
+                }
+        };
+        const bool fast = has_ps && has_bias;                 // a float bias excludes the int32 one
+        using T = std::true_type;
+        using F = std::false_type;
+        if (f16) {
+            if (fast) stage_tile(T{}, T{}); else stage_tile(T{}, F{});
+        } else {
+            if (fast) stage_tile(F{}, T{}); else stage_tile(F{}, F{});
+        }
         const int mw = m0 + wm * WTM * 16, nw = n0 + wn * WTN * 16;
 #pragma unroll
         for (int q0 = 0; q0 < WTM * 16 * CHUNKS; q0 += 64) {
