@@ -41,7 +41,7 @@ def _parse():
     ap.add_argument("--eager", action="store_true",
                     help="launch the timed headline steps one by one instead of from a captured graph (kernel traces:\n"
                          "launches of a graph overlap, which blurs per-kernel durations)")
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c3,c4,a4w4,c5,aq for the 'others' section")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c3,c4,a4w4,c5,aq,qz for the 'others' section")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="launch a 256 MiB device copy and then each main kernel once on fresh buffers (for "
                          "`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: the copy calibrates the counters)")
@@ -455,6 +455,19 @@ def main():
             others.append(hbm_entry(f"npu_anti_quant int{bits}[4096,14336] -> bf16 (per-column float32 scale and offset)", nb, us,
                                     TRAFFIC_BYTES["aq_int8"] if bits == 8 else None))
             del xs, keep
+
+    if want("qz"):
+        # static quantisation of an activation matrix with per-channel scales and zero points: bf16 [2048, 14336] -> int8
+        R, C = 2048, 14336
+        sc_q = torch.rand(C, generator=gen, device=dev) * 0.05 + 0.01
+        zp_q = torch.randint(-8, 8, (C,), generator=gen, device=dev, dtype=torch.int32)
+        nb = R * C * 2 + R * C + 2 * C * 4
+        xs = [(torch.randn(R, C, generator=gen, device=dev)).to(torch.bfloat16) for _ in range(_nsets(nb))]
+        keep = []
+        calls = [(lambda x=x: keep.append(pa.npu_quantize(x, sc_q, zp_q, torch.qint8, -1))) for x in xs] * 2
+        us = _graph_time_us(torch, calls)
+        others.append(hbm_entry("npu_quantize bf16[2048,14336] -> int8 (per-channel float32 scales, int32 zero points)", nb, us, None))
+        del xs, keep
 
     if others:
         result["others"] = others

@@ -38,6 +38,8 @@ typedef enum mi355_status {
 /* 16-bit floating-point element formats of activations. */
 #define MI355_DTYPE_BF16 0
 #define MI355_DTYPE_FP16 1
+#define MI355_DTYPE_FP32 2   /* accepted where a function's comment says so */
+#define MI355_DTYPE_INT32 3  /* likewise */
 
 /* Output formats of mi355_quant_matmul. */
 #define MI355_OUT_BF16 0
@@ -196,6 +198,28 @@ int mi355_swiglu_quant(const void *x_bf16, int activate_left, int8_t *y, float *
 int mi355_anti_quant(const void *x, int x_bits, const float *scale, int64_t scale_len, const float *offset,
                      int64_t offset_len, void *out, int out_dtype, int64_t rows, int64_t cols, int64_t ldx, int64_t ldo,
                      void *stream);
+
+/*
+ * npu_quantize: static quantisation with given scales and zero points along one axis.
+ * Replaces the aclnn Quantize / AscendQuant call behind torch_npu.npu_quantize(inputs, scales, zero_points, dtype, axis,
+ * div_mode=True) (signature test/torch_npu_schema.json:2273-2275, wrapper torch_npu/onnx/wrapper_onnx_ops.py:855-877
+ * and :1278-1279, whose dtype codes name the three output types; the reference tree holds no golden for it, the
+ * formula is the operator's published one).
+ *
+ *   x          contiguous [outer, channels, inner] of in_dtype (MI355_DTYPE_BF16 / FP16 / FP32); channels is the
+ *              size of the quantisation axis, outer / inner the products of the dimensions before / after it
+ *   scale      float32 [scale_len], scale_len == channels or 1;  zero_point [zero_point_len] likewise, of
+ *              zero_point_dtype MI355_DTYPE_FP32 or MI355_DTYPE_INT32 (converted to float32), or NULL
+ *   out        contiguous, same shape, of out_dtype: MI355_Q_INT8 [-128,127], MI355_Q_UINT8 [0,255], MI355_Q_INT32
+ *   div_mode != 0: out = clamp(rint(x / scale[c] + zero_point[c]));  0: out = clamp(rint(x * scale[c] + zero_point[c]))
+ *              every operation rounded to float32, rint = round half to even, NaN -> 0
+ */
+#define MI355_Q_INT8 0
+#define MI355_Q_UINT8 1
+#define MI355_Q_INT32 2
+int mi355_quantize(const void *x, int in_dtype, const float *scale, int64_t scale_len, const void *zero_point,
+                   int zero_point_dtype, int64_t zero_point_len, void *out, int out_dtype, int64_t outer, int64_t channels,
+                   int64_t inner, int div_mode, void *stream);
 
 /*
  * Packed int4 -> int8: widens the A4W4 operands of npu_quant_matmul (both inputs int32, eight int4 values per word:

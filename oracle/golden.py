@@ -218,6 +218,31 @@ def anti_quant(x, scale_f32, offset_f32=None, dst: str = "fp16") -> np.ndarray:
     return f.astype(np.float16).view(np.uint16)          # IEEE round to nearest even
 
 
+def quantize(x_f32, scale_f32, zero_point_f32=None, out: str = "int8", axis: int = -1, div_mode: bool = True) -> np.ndarray:
+    """npu_quantize (signature test/torch_npu_schema.json:2273-2275; output types
+    torch_npu/onnx/wrapper_onnx_ops.py:869-877): q = clamp(rint(x / scale + zero_point)) along ``axis`` (x * scale
+    with div_mode False), every operation rounded to float32, ties to even, NaN -> 0.  ``x_f32`` holds the input
+    values as float32 (bf16 / fp16 inputs converted exactly).  PARITY UNPINNED for the general formula: the reference
+    tree holds no golden or test vector for this operator; the formula is the vendor's published one.  Pinned by the
+    tests where the mathematics fixes it: against torch.quantize_per_channel / quantize_per_tensor for power-of-two
+    scales (where x / scale and x * (1 / scale) agree exactly) and against hand-computed ties."""
+    x = _c(x_f32, np.float32)
+    axis = axis % x.ndim
+    shape = [1] * x.ndim
+    shape[axis] = -1
+    s = _c(scale_f32, np.float32).reshape(-1)
+    s = s.reshape(shape) if s.size > 1 else s.reshape([1] * x.ndim)
+    v = (x / s).astype(np.float32) if div_mode else (x * s).astype(np.float32)
+    if zero_point_f32 is not None:
+        z = _c(zero_point_f32, np.float32).reshape(-1)
+        z = z.reshape(shape) if z.size > 1 else z.reshape([1] * x.ndim)
+        v = (v + z).astype(np.float32)
+    v = np.rint(v)
+    v = np.where(np.isnan(v), np.float32(0), v)
+    lo, hi, dt = {"int8": (-128, 127, np.int8), "uint8": (0, 255, np.uint8), "int32": (-2 ** 31, 2 ** 31 - 1, np.int32)}[out]
+    return np.clip(v.astype(np.float64), lo, hi).astype(dt)
+
+
 def weight_quant_matmul(x_u16, w, scale_u16, off_u16=None, group_size: int = 0, accum: str = "f32", dtype: str = "bf16",
                         bias_u16=None):
     """x bf16 (or, with dtype="fp16", float16) bits [M,K]; w int8 [K,N] (any strides) or int32 [K,N/8] (packed int4);

@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
 EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant",
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
-           "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric")
+           "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize")
 
 _lib = None
 
@@ -49,6 +49,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_anti_quant.argtypes = [vp, i32, vp, i64, vp, i64, vp, i32, i64, i64, i64, i64, vp]
         L.mi355_unpack_int4.argtypes = [vp, vp, i64, i64, i64, i64, vp]
         L.mi355_dynamic_quant_asymmetric.argtypes = [vp, i32, vp, vp, vp, vp, i64, i64, i64, vp]
+        L.mi355_quantize.argtypes = [vp, i32, vp, i64, vp, i32, i64, vp, i32, i64, i64, i64, i32, vp]
         _lib = L
     return _lib
 
@@ -182,6 +183,30 @@ def anti_quant(x, scale, offset=None, dst_dtype=torch.float16):
     _check(lib().mi355_anti_quant(_ptr(x), bits, _ptr(scale), scale.numel(), _ptr(offset), 0 if offset is None else offset.numel(),
                                   _ptr(out), 1 if dst_dtype == torch.float16 else 0, rows, cols, x.stride(0), cols, _stream()),
            "mi355_anti_quant")
+    return out
+
+
+_IN_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+_Q_CODE = {torch.int8: 0, torch.uint8: 1, torch.int32: 2}
+
+
+def quantize(x, scale, zero_point=None, out_dtype=torch.int8, axis=-1, div_mode=True):
+    """x bf16/fp16/fp32 (contiguous, any rank), scale float32, zero_point float32 or int32, [x.shape[axis]] or [1] ->
+    out_dtype tensor of the same shape: clamp(rint(x / scale + zero_point)) (x * scale with div_mode False)."""
+    _need_gpu(x, scale, zero_point)
+    assert x.is_contiguous()
+    axis = axis % x.dim()
+    outer = 1
+    for d in x.shape[:axis]:
+        outer *= d
+    inner = 1
+    for d in x.shape[axis + 1:]:
+        inner *= d
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    zp_code = 3 if zero_point is not None and zero_point.dtype == torch.int32 else 2
+    _check(lib().mi355_quantize(_ptr(x), _IN_CODE[x.dtype], _ptr(scale), scale.numel(), _ptr(zero_point), zp_code,
+                                0 if zero_point is None else zero_point.numel(), _ptr(out), _Q_CODE[out_dtype], outer,
+                                x.shape[axis], inner, 1 if div_mode else 0, _stream()), "mi355_quantize")
     return out
 
 

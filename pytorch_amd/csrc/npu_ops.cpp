@@ -634,6 +634,83 @@ Tensor anti_quant_hip(const Tensor &x, const Tensor &scale, const optional<Tenso
     return out;
 }
 
+
+// ---------------------------------------------------------------- npu_quantize
+// torch_npu.npu_quantize(inputs, scales, zero_points, dtype, axis, div_mode=True)
+// (test/torch_npu_schema.json:2273-2275; torch_npu/onnx/wrapper_onnx_ops.py:855-877 names the output types:
+// torch.qint8 -> int8, torch.quint8 -> uint8, torch.qint32 -> int32)
+
+struct QuantizePlan {
+    at::ScalarType out;
+    int out_code;
+    int64_t axis, outer, channels, inner;
+};
+
+QuantizePlan quantize_check(const Tensor &x, const Tensor &scales, const optional<Tensor> &zero_points, at::ScalarType dtype,
+                            int64_t axis)
+{
+    QuantizePlan pl{};
+    TORCH_CHECK(x.scalar_type() == at::kBFloat16 || x.scalar_type() == at::kHalf || x.scalar_type() == at::kFloat,
+                "npu_quantize: inputs must be float32, float16 or bfloat16, got ", x.scalar_type());
+    if (dtype == at::kQInt8 || dtype == at::kChar) pl.out = at::kChar, pl.out_code = MI355_Q_INT8;
+    else if (dtype == at::kQUInt8 || dtype == at::kByte) pl.out = at::kByte, pl.out_code = MI355_Q_UINT8;
+    else if (dtype == at::kQInt32 || dtype == at::kInt) pl.out = at::kInt, pl.out_code = MI355_Q_INT32;
+    else TORCH_CHECK(false, "npu_quantize: dtype must be torch.qint8, torch.quint8 or torch.qint32, got ", dtype);
+    const int64_t nd = x.dim();
+    TORCH_CHECK(nd >= 1, "npu_quantize: inputs must have at least one dimension");
+    TORCH_CHECK(axis >= -nd && axis < nd, "npu_quantize: axis ", axis, " out of range for ", nd, " dimensions");
+    pl.axis = axis < 0 ? axis + nd : axis;
+    pl.channels = x.size(pl.axis);
+    pl.outer = 1;
+    pl.inner = 1;
+    for (int64_t d = 0; d < pl.axis; d++) pl.outer *= x.size(d);
+    for (int64_t d = pl.axis + 1; d < nd; d++) pl.inner *= x.size(d);
+    TORCH_CHECK(scales.dim() <= 1 && (scales.numel() == 1 || scales.numel() == pl.channels),
+                "npu_quantize: scales must have one element or one per element of dimension ", pl.axis, " (", pl.channels, ")");
+    TORCH_CHECK(at::isFloatingType(scales.scalar_type()), "npu_quantize: scales must be a floating-point tensor");
+    if (const Tensor *z = opt(zero_points)) {
+        TORCH_CHECK(z->dim() <= 1 && (z->numel() == 1 || z->numel() == pl.channels),
+                    "npu_quantize: zero_points must have one element or one per element of dimension ", pl.axis, " (",
+                    pl.channels, ")");
+        TORCH_CHECK(z->scalar_type() != at::kBool && !at::isComplexType(z->scalar_type()),
+                    "npu_quantize: zero_points must be an integer or floating-point tensor");
+    }
+    return pl;
+}
+
+Tensor quantize_meta(const Tensor &x, const Tensor &scales, const optional<Tensor> &zero_points, at::ScalarType dtype,
+                     int64_t axis, bool div_mode)
+{
+    (void)div_mode;
+    const QuantizePlan pl = quantize_check(x, scales, zero_points, dtype, axis);
+    return at::empty(x.sizes(), x.options().dtype(pl.out));
+}
+
+Tensor quantize_hip(const Tensor &x, const Tensor &scales, const optional<Tensor> &zero_points, at::ScalarType dtype,
+                    int64_t axis, bool div_mode)
+{
+    check_same_device("npu_quantize", {&x, &scales, opt(zero_points)});
+    const QuantizePlan pl = quantize_check(x, scales, zero_points, dtype, axis);
+    Tensor out = at::empty(x.sizes(), x.options().dtype(pl.out));
+    if (out.numel() == 0) return out;
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+    Tensor xin = x.contiguous();
+    Tensor sc = scales.to(at::kFloat).contiguous();            // a few hundred to a few thousand elements
+    Tensor zp;                                                 // int32 and float32 zero points go to the kernel as they are
+    if (const Tensor *z = opt(zero_points))
+        zp = (z->scalar_type() == at::kInt || z->scalar_type() == at::kFloat ? *z : z->to(at::kFloat)).contiguous();
+    const int in_code = x.scalar_type() == at::kBFloat16 ? MI355_DTYPE_BF16
+                        : x.scalar_type() == at::kHalf   ? MI355_DTYPE_FP16
+                                                         : MI355_DTYPE_FP32;
+    check_status(mi355_quantize(xin.data_ptr(), in_code, sc.data_ptr<float>(), sc.numel(),
+                                zp.defined() ? zp.data_ptr() : nullptr,
+                                zp.defined() && zp.scalar_type() == at::kInt ? MI355_DTYPE_INT32 : MI355_DTYPE_FP32,
+                                zp.defined() ? zp.numel() : 0, out.data_ptr(),
+                                pl.out_code, pl.outer, pl.channels, pl.inner, div_mode ? 1 : 0, stream_of(x)),
+                 "npu_quantize");
+    return out;
+}
+
 } // namespace
 
 TORCH_LIBRARY_FRAGMENT(npu, m)
@@ -652,6 +729,8 @@ TORCH_LIBRARY_FRAGMENT(npu, m)
           "bool activate_left=False, int quant_mode=0, int group_list_type=0, ScalarType? dst_type=None) -> (Tensor, Tensor)");
     m.def("npu_anti_quant(Tensor x, Tensor scale, *, Tensor? offset=None, ScalarType? dst_dtype=None, "
           "ScalarType? src_dtype=None) -> Tensor");
+    m.def("npu_quantize(Tensor inputs, Tensor scales, Tensor? zero_points, ScalarType dtype, int axis=1, "
+          "bool div_mode=True) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(npu, CUDA, m)
@@ -663,6 +742,7 @@ TORCH_LIBRARY_IMPL(npu, CUDA, m)
     m.impl("npu_swiglu", TORCH_FN(swiglu_hip));
     m.impl("npu_swiglu_quant", TORCH_FN(swiglu_quant_hip));
     m.impl("npu_anti_quant", TORCH_FN(anti_quant_hip));
+    m.impl("npu_quantize", TORCH_FN(quantize_hip));
 }
 
 TORCH_LIBRARY_IMPL(npu, Meta, m)
@@ -674,4 +754,5 @@ TORCH_LIBRARY_IMPL(npu, Meta, m)
     m.impl("npu_swiglu", TORCH_FN(swiglu_meta));
     m.impl("npu_swiglu_quant", TORCH_FN(swiglu_quant_meta));
     m.impl("npu_anti_quant", TORCH_FN(anti_quant_meta));
+    m.impl("npu_quantize", TORCH_FN(quantize_meta));
 }

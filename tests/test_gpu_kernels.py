@@ -590,6 +590,63 @@ def test_anti_quant(capi, golden, rows, cols, packed, dst):
         assert np.array_equal(got, want)
 
 
+QUANTIZE_CASES = [  # shape, axis, number of scales ("c" = one per channel, 1 = single)
+    ((2048, 4096), -1, "c"), ((5, 16, 8), 2, "c"), ((5, 16, 8), 1, "c"), ((3, 7, 5), 0, "c"), ((64, 24), -1, 1),
+    ((33, 1000), -1, "c"), ((4, 12, 16), 1, "c"), ((1, 9), -1, "c"), ((128, 14336), -1, 1)]
+
+
+@pytest.mark.parametrize("shape,axis,nscale", QUANTIZE_CASES)
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_quantize(capi, golden, shape, axis, nscale, in_dtype):
+    """npu_quantize through the C ABI, bit-exact against the oracle: every input and output type, division and
+    multiplication mode, with and without zero points, the vector paths (shared channel / consecutive channels) and the
+    element-wise fallback, values that clamp and exact .5 ties."""
+    g = torch.Generator().manual_seed(sum(shape) + axis)
+    x = (torch.randn(shape, generator=g) * 60).to(in_dtype)
+    flat = x.view(-1)
+    flat[: min(8, flat.numel())] = torch.tensor([0.5, 1.5, 2.5, -0.5, -2.5, 1000.0, -1000.0, 3.5])[: min(8, flat.numel())].to(in_dtype)
+    ch = shape[axis] if nscale == "c" else 1
+    scale = torch.rand(ch, generator=g) * 1.5 + 0.25
+    scale[0] = 1.0
+    zp = torch.randint(-20, 20, (ch,), generator=g).float()
+    xf = x.float().numpy()
+    for out_dtype, name in [(torch.int8, "int8"), (torch.uint8, "uint8"), (torch.int32, "int32")]:
+        for div in (True, False):
+            for z in (zp, None):
+                zc = None if z is None else (z.cuda().to(torch.int32) if div else z.cuda())    # both zero-point types
+                got = capi.quantize(x.cuda(), scale.cuda(), zc, out_dtype, axis, div)
+                want = golden.quantize(xf, scale.numpy(), None if z is None else z.numpy(), name, axis, div)
+                assert got.dtype == out_dtype and got.shape == x.shape
+                assert np.array_equal(got.cpu().numpy(), want), (name, div, z is None)
+
+
+def test_quantize_matches_torch_per_channel(capi):
+    """Independent pin: torch.quantize_per_channel on the CPU for power-of-two scales and even zero points (where its
+    nearbyint(x * (1 / scale)) + zero_point equals rint(x / scale + zero_point))."""
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(6, 32, 10, generator=g) * 50
+    scales = torch.tensor([2.0 ** (i % 6 - 3) for i in range(32)])
+    zps = (torch.arange(32, dtype=torch.int32) - 16) // 2 * 2
+    want = torch.quantize_per_channel(x, scales, zps, axis=1, dtype=torch.qint8).int_repr()
+    got = capi.quantize(x.cuda(), scales.cuda(), zps.float().cuda(), torch.int8, 1, True)
+    assert torch.equal(got.cpu(), want)
+
+
+def test_quantize_bad_arguments(capi):
+    import ctypes
+    L = capi.lib()
+    x = torch.zeros(16, device="cuda")
+    o = torch.zeros(16, dtype=torch.int8, device="cuda")
+    sc = torch.ones(4, device="cuda")
+    call = lambda *a: L.mi355_quantize(*a)
+    vp = ctypes.c_void_p
+    assert call(vp(x.data_ptr()), 2, vp(sc.data_ptr()), 3, None, 2, 0, vp(o.data_ptr()), 0, 1, 4, 4, 1, None) == -1   # scale_len
+    assert call(vp(x.data_ptr()), 7, vp(sc.data_ptr()), 4, None, 2, 0, vp(o.data_ptr()), 0, 1, 4, 4, 1, None) == -1   # in_dtype
+    assert call(vp(x.data_ptr()), 2, vp(sc.data_ptr()), 4, None, 2, 0, vp(o.data_ptr()), 5, 1, 4, 4, 1, None) == -1   # out_dtype
+    assert call(None, 2, vp(sc.data_ptr()), 4, None, 2, 0, vp(o.data_ptr()), 0, 1, 4, 4, 1, None) == -1
+    assert call(None, 2, None, 4, None, 2, 0, None, 0, 0, 4, 4, 1, None) == 0                                        # empty
+
+
 @pytest.mark.parametrize("rows,words,in_pad,out_pad,out_shift", [
     (16, 8, 0, 0, 0), (64, 5, 0, 0, 0), (1024, 512, 0, 0, 0), (4096, 1376, 0, 0, 0),   # 16-byte stores / one odd word count
     (33, 6, 1, 0, 0), (7, 3, 0, 8, 0), (9, 4, 2, 3, 0), (5, 2, 0, 0, 1), (1, 1, 0, 0, 0)])  # pitched and unaligned rows

@@ -305,6 +305,34 @@ def test_anti_quant_operator(pa, golden):
         pa.npu_anti_quant(x.cuda(), scale.cuda(), dst_dtype=torch.float32)
 
 
+def test_npu_quantize_operator(pa, golden):
+    """torch_npu.npu_quantize(inputs, scales, zero_points, dtype, axis, div_mode=True) as the reference's wrapper test
+    calls it (test/onnx/test_wrapper_onnx_ops.py:1444-1452: float32 [5,16,8], eight scales of 0.1, int32 zero points,
+    torch.quint8, axis 2), plus the other output types, a bf16 input with bf16 scales and the multiply mode."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(5, 16, 8, generator=g)
+    scales = torch.tensor([0.1] * 8)
+    zps = torch.tensor([0] * 8, dtype=torch.int32)
+    out = pa.npu_quantize(x.cuda(), scales.cuda(), zps.cuda(), dtype=torch.quint8, axis=2)
+    assert out.dtype == torch.uint8 and out.shape == (5, 16, 8)
+    assert np.array_equal(out.cpu().numpy(), golden.quantize(x.numpy(), scales.numpy(), zps.float().numpy(), "uint8", 2))
+    zps = torch.randint(-5, 5, (16,), generator=g, dtype=torch.int32)
+    sc16 = (torch.rand(16, generator=g) + 0.5).to(torch.bfloat16)
+    xb = (x * 30).to(torch.bfloat16)
+    out = pa.npu_quantize(xb.cuda(), sc16.cuda(), zps.cuda(), torch.qint8, 1)
+    assert out.dtype == torch.int8
+    assert np.array_equal(out.cpu().numpy(), golden.quantize(xb.float().numpy(), sc16.float().numpy(), zps.float().numpy(), "int8", 1))
+    out = pa.npu_quantize(xb.cuda(), sc16.cuda(), None, torch.qint32, 1, False)
+    assert out.dtype == torch.int32
+    assert np.array_equal(out.cpu().numpy(), golden.quantize(xb.float().numpy(), sc16.float().numpy(), None, "int32", 1, False))
+    # a non-contiguous input is quantised by value
+    xt = xb.cuda().transpose(0, 2)
+    out = pa.npu_quantize(xt, sc16.cuda(), None, torch.qint8, 1)
+    assert np.array_equal(out.cpu().numpy(), golden.quantize(xb.float().numpy().transpose(2, 1, 0), sc16.float().numpy(), None, "int8", 1))
+    with pytest.raises(RuntimeError, match="Expected all tensors to be on the same device"):
+        pa.npu_quantize(x.cuda(), scales, None, torch.qint8, 2)
+
+
 def _rand_words(g, *shape):
     return torch.randint(-2 ** 31, 2 ** 31 - 1, shape, generator=g, dtype=torch.int64).to(torch.int32)
 

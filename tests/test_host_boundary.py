@@ -17,7 +17,7 @@ def test_c_abi_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "mi355_quant.h")).read()
     declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", header))
     assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant", "mi355_anti_quant",
-            "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric"} <= declared
+            "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize"} <= declared
     lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_amd", "csrc", "libmi355_quant.so"))
     for name in declared:
         assert hasattr(lib, name), name
@@ -201,6 +201,27 @@ def test_meta_anti_quant(pa):
         pa.npu_anti_quant(_m(4, 8, dtype=torch.int8), _m(7, dtype=torch.float32))
     with pytest.raises(RuntimeError, match="int8 or int32"):
         pa.npu_anti_quant(_m(4, 8, dtype=torch.int16), _m(8, dtype=torch.float32))
+
+
+def test_meta_npu_quantize(pa):
+    """Shapes and output types of npu_quantize (signature test/torch_npu_schema.json:2273-2275; dtype codes
+    torch_npu/onnx/wrapper_onnx_ops.py:869-877) without a GPU."""
+    x = _m(5, 16, 8, dtype=torch.float32)
+    res = pa.npu_quantize(x, _m(8, dtype=torch.float32), _m(8, dtype=torch.int32), torch.quint8, 2)
+    assert res.shape == (5, 16, 8) and res.dtype == torch.uint8
+    res = pa.npu_quantize(_m(4, 6, dtype=torch.bfloat16), _m(1, dtype=torch.float32), None, torch.qint8, -1, False)
+    assert res.dtype == torch.int8
+    assert pa.npu_quantize(_m(4, 6, dtype=torch.float16), _m(4, dtype=torch.float32), None, torch.qint32, 0).dtype == torch.int32
+    s = str(torch.ops.npu.npu_quantize.default._schema)
+    assert "Tensor inputs, Tensor scales, Tensor? zero_points, ScalarType dtype, int axis=1, bool div_mode=True" in s
+    with pytest.raises(RuntimeError, match="scales must have one element or one per element"):
+        pa.npu_quantize(x, _m(7, dtype=torch.float32), None, torch.qint8, 2)
+    with pytest.raises(RuntimeError, match="dtype must be"):
+        pa.npu_quantize(x, _m(8, dtype=torch.float32), None, torch.float16, 2)
+    with pytest.raises(RuntimeError, match="axis"):
+        pa.npu_quantize(x, _m(8, dtype=torch.float32), None, torch.qint8, 3)
+    with pytest.raises(RuntimeError, match="inputs must be"):
+        pa.npu_quantize(_m(4, 4, dtype=torch.int32), _m(4, dtype=torch.float32), None, torch.qint8, 1)
 
 
 def test_meta_swiglu(pa):
