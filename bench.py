@@ -41,7 +41,7 @@ def _parse():
     ap.add_argument("--eager", action="store_true",
                     help="launch the timed headline steps one by one instead of from a captured graph (kernel traces:\n"
                          "launches of a graph overlap, which blurs per-kernel durations)")
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c3,c4,a4w4,c5,aq,qz for the 'others' section")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c2i8,c3,c4,a4w4,c5,aq,qz for the 'others' section")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="launch a 256 MiB device copy and then each main kernel once on fresh buffers (for "
                          "`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: the copy calibrates the counters)")
@@ -381,6 +381,25 @@ def main():
                                     "[N,G]: the module's transposed views)", nb, us, None,
                                     tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2)))
             del wks, keep
+
+    if want("c2i8"):
+        # the headline product with the re-quantised int8 output (packed int64 scale from npu_trans_quant_param, int32 bias)
+        Mx, Kx, Nx = 1024, 4096, 11008
+        nset = _nsets(Mx * Kx + Kx * Nx)
+        xs = [torch.randint(-128, 128, (Mx, Kx), generator=gen, dtype=torch.int8, device=dev) for _ in range(nset)]
+        wsn = [torch.randint(-128, 128, (Nx, Kx), generator=gen, dtype=torch.int8, device=dev).t() for _ in range(nset)]
+        qp = pa.npu_trans_quant_param(torch.rand(Nx, generator=gen, device=dev) * 1e-4 + 1e-4,
+                                      torch.randint(-8, 8, (Nx,), generator=gen, device=dev).float())
+        bi = torch.randint(-1000, 1000, (Nx,), generator=gen, device=dev, dtype=torch.int32)
+        keep = []
+        calls = [(lambda a=a, w=w: keep.append(pa.npu_quant_matmul(a, w, qp, bias=bi, output_dtype=torch.int8)))
+                 for a, w in zip(xs, wsn)] * 4
+        us = _graph_time_us(torch, calls, reps=10)
+        tops = 2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12
+        others.append({"name": "c2 quant_matmul with int8 output (int64 packed scale + offset, int32 bias)", "launch_us": round(us, 3),
+                       "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                                    "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None}})
+        del xs, wsn, keep
 
     if want("a4w4"):
         # both operands packed int4 (A4W4) at the headline shape: the operator widens them to int8 and runs the int8 GEMM

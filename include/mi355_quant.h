@@ -45,6 +45,7 @@ typedef enum mi355_status {
 #define MI355_OUT_BF16 0
 #define MI355_OUT_INT32 1   /* int32 accumulators (plus an int32 bias if given); scales are ignored */
 #define MI355_OUT_FP16 2
+#define MI355_OUT_INT8 3    /* re-quantised output; only mi355_quant_matmul_qparam produces it */
 
 /* bias element types of mi355_quant_matmul */
 #define MI355_BIAS_NONE 0
@@ -119,6 +120,41 @@ int mi355_quant_matmul(const int8_t *a, const int8_t *b,
                        int64_t M, int64_t N, int64_t K,
                        int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                        void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * npu_trans_quant_param: packs a float32 scale (and optional float32 offset) per channel into the 64-bit quantisation
+ * parameter that npu_quant_matmul takes as an int64 `scale`.
+ * Replaces the aclnn TransQuantParam call behind torch_npu.npu_trans_quant_param(scale, offset=None)
+ * (caller torch_npu/contrib/module/linear_quant.py:104-108; shapes and the int64 result type
+ * test/test_fake_tensor.py:1929-1943).  The bit layout is not in the reference tree; it follows the operator's
+ * published description:
+ *   bits 0-31   the float32 bit pattern of scale[i]
+ *   bits 37-45  clamp(rint(offset[i]), -256, 255) as a 9-bit two's-complement integer (zero without an offset)
+ *   bit 46      set
+ * scale_len and offset_len are n or 1 (broadcast); out receives n words.
+ */
+int mi355_trans_quant_param(const float *scale, int64_t scale_len, const float *offset, int64_t offset_len,
+                            uint64_t *out, int64_t n, void *stream);
+
+/*
+ * npu_quant_matmul with the packed 64-bit parameters of mi355_trans_quant_param in place of the float32 scale
+ * (the int64 `scale` of torch_npu.npu_quant_matmul, which LinearQuant passes whenever its scale is float32, there is
+ * no pertoken_scale and the output is int8 or float16: torch_npu/contrib/module/linear_quant.py:104-112).
+ *   qparam    [qparam_len], qparam_len in {1, N}
+ *   bias      int32 [N] (added to the accumulator) or NULL; for the floating-point outputs also float32 / bf16 as in
+ *             mi355_quant_matmul
+ *   out_dtype MI355_OUT_INT8:  out[m*ldc+n] = clamp(rint(float(acc + bias[n]) * scale[n] + offset[n]), -128, 127) as
+ *                              int8 (scale and offset decoded from qparam[n], each operation rounded to float32,
+ *                              rint = round half to even)
+ *             MI355_OUT_FP16 / MI355_OUT_BF16: as mi355_quant_matmul with scale[n] decoded from qparam[n] and no
+ *                              pertoken_scale (the packed offset is ignored)
+ * a, b, strides, M, N, K, workspace: as mi355_quant_matmul (the same mi355_quant_matmul_workspace() query).
+ */
+int mi355_quant_matmul_qparam(const int8_t *a, const int8_t *b, const uint64_t *qparam, int64_t qparam_len,
+                              const void *bias, int bias_dtype, void *out, int out_dtype,
+                              int64_t M, int64_t N, int64_t K,
+                              int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                              void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * npu_weight_quant_batchmatmul, W8A16 per channel and W4A16 per group.

@@ -243,6 +243,43 @@ def quantize(x_f32, scale_f32, zero_point_f32=None, out: str = "int8", axis: int
     return np.clip(v.astype(np.float64), lo, hi).astype(dt)
 
 
+def trans_quant_param(scale_f32, offset_f32=None) -> np.ndarray:
+    """npu_trans_quant_param (caller torch_npu/contrib/module/linear_quant.py:104-108, result type and shapes
+    test/test_fake_tensor.py:1929-1943): int64 words with the float32 bit pattern of the scale in bits 0-31,
+    clamp(rint(offset), -256, 255) as a 9-bit two's-complement field in bits 37-45 and bit 46 set.  PARITY UNPINNED:
+    the bit layout is not in the reference tree (the operator's published description); the tests pin this function
+    by hand-assembled words and by the decode round trip only."""
+    sc = _c(scale_f32, np.float32).reshape(-1)
+    n = sc.size if offset_f32 is None else max(sc.size, np.asarray(offset_f32).size)
+    q = np.broadcast_to(sc.view(np.uint32).astype(np.uint64), (n,)).copy() | np.uint64(1 << 46)
+    if offset_f32 is not None:
+        o = np.clip(np.rint(_c(offset_f32, np.float32).reshape(-1)), -256, 255).astype(np.int64)
+        q |= (np.broadcast_to(o, (n,)) & 0x1FF).astype(np.uint64) << np.uint64(37)
+    return q.view(np.int64)
+
+
+def quant_param_decode(q):
+    """(scale float32, offset float32) carried by the words of trans_quant_param."""
+    u = _c(q, np.int64).reshape(-1).view(np.uint64)
+    scale = (u & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.float32)
+    field = ((u >> np.uint64(37)) & np.uint64(0x1FF)).astype(np.int64)
+    offset = np.where(field >= 256, field - 512, field).astype(np.float32)
+    return scale, offset
+
+
+def quant_matmul_requant(a, b, qparam, bias_i32=None) -> np.ndarray:
+    """npu_quant_matmul with int8 output: clamp(rint(float32(acc + bias) * scale + offset), -128, 127), scale and offset
+    decoded from the packed words, every operation rounded to float32, ties to even.  The int32 product is int8_gemm
+    (pinned); the formula out = (x1 @ x2 + bias) * scale + offset is the operator's published one: PARITY UNPINNED."""
+    acc = int8_gemm(a, b)
+    if bias_i32 is not None:
+        acc = (acc.astype(np.int64) + _c(bias_i32, np.int32).reshape(1, -1)).astype(np.int32)   # wraps like the accumulator
+    scale, offset = quant_param_decode(qparam)
+    v = (acc.astype(np.float32) * scale.reshape(1, -1)).astype(np.float32)
+    v = (v + offset.reshape(1, -1)).astype(np.float32)
+    return np.clip(np.rint(v), -128, 127).astype(np.int8)
+
+
 def weight_quant_matmul(x_u16, w, scale_u16, off_u16=None, group_size: int = 0, accum: str = "f32", dtype: str = "bf16",
                         bias_u16=None):
     """x bf16 (or, with dtype="fp16", float16) bits [M,K]; w int8 [K,N] (any strides) or int32 [K,N/8] (packed int4);

@@ -17,7 +17,8 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
 EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant",
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
-           "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize")
+           "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
+           "mi355_trans_quant_param", "mi355_quant_matmul_qparam")
 
 _lib = None
 
@@ -49,6 +50,8 @@ def lib() -> ctypes.CDLL:
         L.mi355_anti_quant.argtypes = [vp, i32, vp, i64, vp, i64, vp, i32, i64, i64, i64, i64, vp]
         L.mi355_unpack_int4.argtypes = [vp, vp, i64, i64, i64, i64, vp]
         L.mi355_dynamic_quant_asymmetric.argtypes = [vp, i32, vp, vp, vp, vp, i64, i64, i64, vp]
+        L.mi355_trans_quant_param.argtypes = [vp, i64, vp, i64, vp, i64, vp]
+        L.mi355_quant_matmul_qparam.argtypes = [vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
         L.mi355_quantize.argtypes = [vp, i32, vp, i64, vp, i32, i64, vp, i32, i64, i64, i64, i32, vp]
         _lib = L
     return _lib
@@ -107,6 +110,34 @@ def quant_matmul(x1, x2, scale, pertoken_scale=None, bias=None, out_dtype=torch.
                                   M, N, K, x1.stride(0), x2.stride(0), x2.stride(1), out.stride(0), _ptr(workspace),
                                   0 if workspace is None else workspace.numel(), _stream())
     _check(st, "mi355_quant_matmul")
+    return out
+
+
+def trans_quant_param(scale, offset=None):
+    """float32 scale [n] or [1] (and offset likewise) -> int64 [n] packed quantisation parameters."""
+    _need_gpu(scale, offset)
+    n = max(scale.numel(), 1 if offset is None else offset.numel())
+    out = torch.empty((n,), dtype=torch.int64, device=scale.device)
+    _check(lib().mi355_trans_quant_param(_ptr(scale), scale.numel(), _ptr(offset), 0 if offset is None else offset.numel(),
+                                         _ptr(out), n, _stream()), "mi355_trans_quant_param")
+    return out
+
+
+def quant_matmul_qparam(x1, x2, qparam, bias=None, out_dtype=torch.int8, workspace=None):
+    """x1 int8 [M,K]; x2 int8 [K,N] with strides (N,1) or (1,K); qparam int64 [N] or [1] from trans_quant_param."""
+    _need_gpu(x1, x2, qparam, bias)
+    M, K = x1.shape
+    N = x2.shape[1]
+    out = torch.empty((M, N), dtype=out_dtype, device=x1.device)
+    need = lib().mi355_quant_matmul_workspace(M, N, K, x2.stride(0), x2.stride(1))
+    if workspace is None and need:
+        workspace = _wq_workspace(x1.device, need)
+    bias_dtype = 0 if bias is None else {torch.bfloat16: 1, torch.int32: 2, torch.float32: 3}[bias.dtype]
+    out_code = {torch.bfloat16: 0, torch.float16: 2, torch.int8: 3}[out_dtype]
+    st = lib().mi355_quant_matmul_qparam(_ptr(x1), _ptr(x2), _ptr(qparam), qparam.numel(), _ptr(bias), bias_dtype, _ptr(out),
+                                         out_code, M, N, K, x1.stride(0), x2.stride(0), x2.stride(1), out.stride(0),
+                                         _ptr(workspace), 0 if workspace is None else workspace.numel(), _stream())
+    _check(st, "mi355_quant_matmul_qparam")
     return out
 
 

@@ -64,15 +64,11 @@ class _QuantLinearBase(nn.Module):
     def forward(self, linear_quant_input: torch.Tensor) -> torch.Tensor:
         self._check_dtypes(linear_quant_input)
         scale = self.scale
-        needs_packed_scale = (self.pertoken_scale is None and scale.dtype == torch.float32
-                              and self.output_dtype not in (torch.bfloat16, torch.int32, torch.float16))
-        if needs_packed_scale:
-            # the reference converts the float32 scale with npu_trans_quant_param for the int8 output path
-            # (linear_quant.py:104-108); neither that packing nor the int8 output exists in this build.  For
-            # float16 output the packing only re-encodes the same float32 scale, so the scale is passed as it is.
-            raise NotImplementedError("float32 scale without pertoken_scale and output_dtype None/int8 selects the "
-                                      "re-quantised int8 output (npu_trans_quant_param), which is not implemented; "
-                                      "use output_dtype=torch.bfloat16, torch.float16 or torch.int32")
+        # a float32 scale is packed with npu_trans_quant_param when there is no pertoken_scale and the output is int8
+        # (output_dtype None) or float16 (linear_quant.py:104-108)
+        if (self.pertoken_scale is None and scale.dtype == torch.float32
+                and self.output_dtype not in (torch.bfloat16, torch.int32)):
+            scale = torch.ops.npu.npu_trans_quant_param(scale, self.offset)
         return torch.ops.npu.npu_quant_matmul(linear_quant_input, self.weight.transpose(-2, -1), scale,
                                               offset=self.offset, pertoken_scale=self.pertoken_scale, bias=self.bias,
                                               output_dtype=self.output_dtype)

@@ -185,6 +185,43 @@ Tensor zeroed_workspace(const Tensor &like, size_t bytes)
     return ws;
 }
 
+// ---------------------------------------------------------------- npu_trans_quant_param
+// torch_npu.npu_trans_quant_param(scale, offset=None) (linear_quant.py:104-108; shapes test/test_fake_tensor.py:1929-1943:
+// the result is int64 and takes the shape of whichever argument has more elements)
+
+std::vector<int64_t> trans_quant_param_shape(const Tensor &scale, const optional<Tensor> &offset)
+{
+    TORCH_CHECK(scale.scalar_type() == at::kFloat, "npu_trans_quant_param: scale must be float32, got ", scale.scalar_type());
+    TORCH_CHECK(scale.dim() >= 1 && scale.dim() <= 2, "npu_trans_quant_param: scale must have 1 or 2 dimensions");
+    const Tensor *o = opt(offset);
+    if (!o) return scale.sizes().vec();
+    TORCH_CHECK(o->scalar_type() == at::kFloat, "npu_trans_quant_param: offset must be float32, got ", o->scalar_type());
+    TORCH_CHECK(o->dim() >= 1 && o->dim() <= 2, "npu_trans_quant_param: offset must have 1 or 2 dimensions");
+    TORCH_CHECK(scale.numel() == o->numel() || scale.numel() == 1 || o->numel() == 1,
+                "npu_trans_quant_param: scale and offset must have the same number of elements, or one of them a single one");
+    return (o->numel() > scale.numel() ? *o : scale).sizes().vec();
+}
+
+Tensor trans_quant_param_meta(const Tensor &scale, const optional<Tensor> &offset)
+{
+    return at::empty(trans_quant_param_shape(scale, offset), scale.options().dtype(at::kLong));
+}
+
+Tensor trans_quant_param_hip(const Tensor &scale, const optional<Tensor> &offset)
+{
+    check_same_device("npu_trans_quant_param", {&scale, opt(offset)});
+    Tensor out = trans_quant_param_meta(scale, offset);
+    if (out.numel() == 0) return out;
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(scale.device());
+    Tensor sc = scale.contiguous();
+    Tensor of = opt(offset) ? opt(offset)->contiguous() : Tensor();
+    check_status(mi355_trans_quant_param(sc.data_ptr<float>(), sc.numel(), of.defined() ? of.data_ptr<float>() : nullptr,
+                                         of.defined() ? of.numel() : 0, reinterpret_cast<uint64_t *>(out.data_ptr<int64_t>()),
+                                         out.numel(), stream_of(scale)),
+                 "npu_trans_quant_param");
+    return out;
+}
+
 // ---------------------------------------------------------------- npu_quant_matmul
 
 struct QmmPlan {
@@ -194,6 +231,7 @@ struct QmmPlan {
     at::ScalarType out_dtype;
     bool a4w4;                       // both inputs int32 words of eight int4 values
     bool x2_packed_k;                // a4w4: x2 is [K/8, N] (words along K) instead of [K, N/8]
+    bool packed_scale;               // scale is the int64 result of npu_trans_quant_param
 };
 
 QmmPlan quant_matmul_plan(const Tensor &x1, const Tensor &x2, const Tensor &scale, const optional<Tensor> &offset,
@@ -224,19 +262,38 @@ QmmPlan quant_matmul_plan(const Tensor &x1, const Tensor &x2, const Tensor &scal
         TORCH_CHECK(x2.size(-2) == p.K, "npu_quant_matmul: inner dimensions differ: x1 [..., ", p.M, ", ", p.K,
                     "] x2 [..., ", x2.size(-2), ", ", p.N, "]");
     }
-    TORCH_CHECK(output_dtype.has_value(),
-                "npu_quant_matmul: output_dtype=None selects the int8 re-quantised output, which is not supported; "
-                "pass output_dtype=torch.bfloat16, torch.float16 or torch.int32");
-    p.out_dtype = *output_dtype;
-    TORCH_CHECK(p.out_dtype == at::kBFloat16 || p.out_dtype == at::kHalf || p.out_dtype == at::kInt,
-                "npu_quant_matmul: output_dtype must be torch.bfloat16, torch.float16 or torch.int32, got ", p.out_dtype);
-    TORCH_CHECK(!opt(offset), "npu_quant_matmul: offset is only meaningful for int8 output, which is not supported");
+    // output_dtype=None is the re-quantised int8 output (linear_quant.py:60-72)
+    p.out_dtype = output_dtype.value_or(at::kChar);
+    TORCH_CHECK(p.out_dtype == at::kBFloat16 || p.out_dtype == at::kHalf || p.out_dtype == at::kInt || p.out_dtype == at::kChar,
+                "npu_quant_matmul: output_dtype must be torch.int8, torch.bfloat16, torch.float16 or torch.int32, got ", p.out_dtype);
+    p.packed_scale = scale.scalar_type() == at::kLong;        // the result of npu_trans_quant_param
+    if (p.out_dtype == at::kChar) {
+        TORCH_CHECK(p.packed_scale || scale.scalar_type() == at::kFloat,
+                    "npu_quant_matmul: scale must be int64 (npu_trans_quant_param) or float32 for int8 output, got ", scale.scalar_type());
+        TORCH_CHECK(scale.dim() <= 2 && (scale.numel() == 1 || scale.numel() == p.N),
+                    "npu_quant_matmul: scale must have 1 or ", p.N, " elements");
+        TORCH_CHECK(!opt(pertoken_scale), "npu_quant_matmul: pertoken_scale is not applicable to int8 output");
+        if (const Tensor *o = opt(offset)) {
+            TORCH_CHECK(o->scalar_type() == at::kFloat, "npu_quant_matmul: offset must be float32, got ", o->scalar_type());
+            TORCH_CHECK(o->numel() == 1 || o->numel() == p.N, "npu_quant_matmul: offset must have 1 or ", p.N, " elements");
+        }
+        if (const Tensor *b = opt(bias)) {
+            TORCH_CHECK(b->scalar_type() == at::kInt, "npu_quant_matmul: bias must be int32 for int8 output, got ", b->scalar_type());
+            TORCH_CHECK(b->numel() == p.N && b->size(-1) == p.N, "npu_quant_matmul: bias must have shape [", p.N, "]");
+        }
+    } else {
+        TORCH_CHECK(!opt(offset), "npu_quant_matmul: offset is only meaningful for int8 output");
+    }
+    if (p.out_dtype == at::kChar) {
+        // checked above
+    } else
     if (p.out_dtype != at::kInt) {
-        // (an int64 scale is the packed output of npu_trans_quant_param, which is not built)
-        TORCH_CHECK(scale.scalar_type() == at::kFloat || scale.scalar_type() == at::kBFloat16,
-                    "npu_quant_matmul: scale must be float32 or bfloat16 for a floating-point output, got ", scale.scalar_type());
-        TORCH_CHECK(scale.dim() == 1 && (scale.size(0) == 1 || scale.size(0) == p.N),
+        TORCH_CHECK(scale.scalar_type() == at::kFloat || scale.scalar_type() == at::kBFloat16 || p.packed_scale,
+                    "npu_quant_matmul: scale must be float32, bfloat16 or int64 (npu_trans_quant_param) for a floating-point "
+                    "output, got ", scale.scalar_type());
+        TORCH_CHECK((scale.dim() == 1 || (p.packed_scale && scale.dim() == 2)) && (scale.numel() == 1 || scale.numel() == p.N),
                     "npu_quant_matmul: scale must have shape [1] or [", p.N, "]");
+        TORCH_CHECK(!(p.packed_scale && opt(pertoken_scale)), "npu_quant_matmul: an int64 scale excludes pertoken_scale");
         if (const Tensor *ps = opt(pertoken_scale)) {
             TORCH_CHECK(ps->scalar_type() == at::kFloat, "npu_quant_matmul: pertoken_scale must be float32");
             TORCH_CHECK(ps->dim() == 1 && ps->size(0) == p.M, "npu_quant_matmul: pertoken_scale must have shape [", p.M, "]");
@@ -315,9 +372,16 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
         xb = p.x2_packed_k ? unpack_int4_rows(x2.transpose(-2, -1)).transpose(-2, -1)   // stored [..., N, K]
                            : unpack_int4_rows(x2);                              // [..., K, N]
     }
-    const bool bf16 = p.out_dtype != at::kInt;            // a floating-point (dequantised) output
-    Tensor scale_f, ps, b;
-    if (bf16) {
+    const bool i8 = p.out_dtype == at::kChar;
+    const bool bf16 = p.out_dtype != at::kInt && !i8;     // a floating-point (dequantised) output
+    Tensor scale_f, ps, b, qp;
+    if (p.packed_scale) {
+        qp = scale.reshape({-1}).contiguous();            // an int64 scale carries its offset (any `offset` repeats it)
+    } else if (i8) {
+        // float32 scale with int8 output: packed here the way the reference's module does it with
+        // npu_trans_quant_param (linear_quant.py:104-108)
+        qp = trans_quant_param_hip(scale, offset).reshape({-1});
+    } else if (bf16) {
         scale_f = scale.to(at::kFloat).contiguous();
         if (const Tensor *t = opt(pertoken_scale)) ps = t->contiguous();
     }
@@ -325,7 +389,8 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
     const int bias_dtype = !b.defined() ? MI355_BIAS_NONE
                            : b.scalar_type() == at::kInt ? MI355_BIAS_INT32
                            : b.scalar_type() == at::kFloat ? MI355_BIAS_FP32 : MI355_BIAS_BF16;
-    const int out_dtype = p.out_dtype == at::kInt ? MI355_OUT_INT32 : p.out_dtype == at::kHalf ? MI355_OUT_FP16 : MI355_OUT_BF16;
+    const int out_dtype = i8 ? MI355_OUT_INT8
+                          : p.out_dtype == at::kInt ? MI355_OUT_INT32 : p.out_dtype == at::kHalf ? MI355_OUT_FP16 : MI355_OUT_BF16;
     int64_t nb = 1;
     for (auto d : p.batch) nb *= d;
     // x1 with batch dimensions against a single weight matrix is one tall matmul
@@ -353,13 +418,17 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
         const size_t ws_bytes = mi355_quant_matmul_workspace(m, p.N, p.K, w.stride(0), w.stride(1));
         if (ws_bytes) ws = zeroed_workspace(xa, ws_bytes);
         Tensor o = out2d.narrow(0, row0, m);
-        check_status(mi355_quant_matmul(a.data_ptr<int8_t>(), w.data_ptr<int8_t>(), ps.defined() ? ps.data_ptr<float>() : nullptr,
-                                        bf16 ? scale_f.data_ptr<float>() : nullptr, bf16 ? scale_f.numel() : 0,
-                                        b.defined() ? b.data_ptr() : nullptr, bias_dtype, o.data_ptr(), out_dtype, m, p.N, p.K,
-                                        a.stride(0), w.stride(0),
-                                        w.stride(1), o.stride(0), ws.defined() ? ws.data_ptr() : nullptr, ws_bytes,
-                                        stream_of(xa)),
-                     "npu_quant_matmul");
+        const int st = qp.defined()
+            ? mi355_quant_matmul_qparam(a.data_ptr<int8_t>(), w.data_ptr<int8_t>(), reinterpret_cast<const uint64_t *>(qp.data_ptr<int64_t>()),
+                                        qp.numel(), b.defined() ? b.data_ptr() : nullptr, bias_dtype, o.data_ptr(), out_dtype, m, p.N,
+                                        p.K, a.stride(0), w.stride(0), w.stride(1), o.stride(0),
+                                        ws.defined() ? ws.data_ptr() : nullptr, ws_bytes, stream_of(x1))
+            : mi355_quant_matmul(a.data_ptr<int8_t>(), w.data_ptr<int8_t>(), ps.defined() ? ps.data_ptr<float>() : nullptr,
+                                 bf16 ? scale_f.data_ptr<float>() : nullptr, bf16 ? scale_f.numel() : 0,
+                                 b.defined() ? b.data_ptr() : nullptr, bias_dtype, o.data_ptr(), out_dtype, m, p.N, p.K,
+                                 a.stride(0), w.stride(0), w.stride(1), o.stride(0), ws.defined() ? ws.data_ptr() : nullptr,
+                                 ws_bytes, stream_of(x1));
+        check_status(st, "npu_quant_matmul");
         row0 += m;
     }
     return out;
@@ -729,6 +798,7 @@ TORCH_LIBRARY_FRAGMENT(npu, m)
           "bool activate_left=False, int quant_mode=0, int group_list_type=0, ScalarType? dst_type=None) -> (Tensor, Tensor)");
     m.def("npu_anti_quant(Tensor x, Tensor scale, *, Tensor? offset=None, ScalarType? dst_dtype=None, "
           "ScalarType? src_dtype=None) -> Tensor");
+    m.def("npu_trans_quant_param(Tensor scale, Tensor? offset=None) -> Tensor");
     m.def("npu_quantize(Tensor inputs, Tensor scales, Tensor? zero_points, ScalarType dtype, int axis=1, "
           "bool div_mode=True) -> Tensor");
 }
@@ -743,6 +813,7 @@ TORCH_LIBRARY_IMPL(npu, CUDA, m)
     m.impl("npu_swiglu_quant", TORCH_FN(swiglu_quant_hip));
     m.impl("npu_anti_quant", TORCH_FN(anti_quant_hip));
     m.impl("npu_quantize", TORCH_FN(quantize_hip));
+    m.impl("npu_trans_quant_param", TORCH_FN(trans_quant_param_hip));
 }
 
 TORCH_LIBRARY_IMPL(npu, Meta, m)
@@ -755,4 +826,5 @@ TORCH_LIBRARY_IMPL(npu, Meta, m)
     m.impl("npu_swiglu_quant", TORCH_FN(swiglu_quant_meta));
     m.impl("npu_anti_quant", TORCH_FN(anti_quant_meta));
     m.impl("npu_quantize", TORCH_FN(quantize_meta));
+    m.impl("npu_trans_quant_param", TORCH_FN(trans_quant_param_meta));
 }

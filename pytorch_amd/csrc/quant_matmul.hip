@@ -67,11 +67,29 @@ struct QmmArgs {
     int M, N, K;
     int scale_len;
     int out_i32;
+    const uint64_t *qparam;    // packed quantisation parameters [scale_len] (replace `scale`), or null
+    int out_i8;                // re-quantised int8 output (needs qparam)
     int tiles_m, tiles_n, tiles_per_xcd;
     int S;                     // workgroups that share the K range of a tile
     int32_t *partial;          // workspace [tile][chunk][wavefront][accumulator quad][lane] int32x4 (S > 1)
     uint32_t *counter;         // workspace [tile], zero on entry, left zero (S > 1)
 };
+
+// Packed quantisation parameter (the 64-bit words npu_trans_quant_param produces): bits 0-31 the float32 scale,
+// bits 37-45 the offset as a 9-bit two's-complement integer, bit 46 set.
+__device__ __forceinline__ float qparam_scale(uint64_t q) { return __uint_as_float((uint32_t)q); }
+__device__ __forceinline__ float qparam_offset(uint64_t q) { return (float)(((int32_t)((uint32_t)(q >> 37) << 23)) >> 23); }
+
+// out = clamp(rint((acc + int32 bias) * scale + offset)) as int8; each operation rounded to float32
+__device__ __forceinline__ int32_t requant1(int32_t a, int32_t bi, float sc, float off)
+{
+    float v = (float)(int32_t)((uint32_t)a + (uint32_t)bi);
+    v = v * sc;
+    v = v + off;
+    v = rintf(v);
+    v = fminf(fmaxf(v, -128.0f), 127.0f);
+    return (int32_t)v;
+}
 
 // WGM x WGN wavefronts per workgroup, each owning (16*WTM) x (16*WTN) of the output tile.
 template <int WGM, int WGN, int WTM, int WTN, int NS>
@@ -325,6 +343,69 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         }
         return;
     }
+    if (p.out_i8) {
+        // Re-quantised output: a lane owns four consecutive columns of a row in every 16x16 tile, i.e. one 32-bit word
+        // of int8 results.  With aligned output rows the words of the wavefront's tile go through its own LDS region
+        // (the stage buffers are idle after the last barrier) and leave as 16-byte stores over whole tile rows.
+        constexpr int ROWQ = WTN * 16 + 16;                   // padded row pitch in bytes
+        constexpr int CHQ = WTN;                              // 16-byte chunks per row
+        char *stq = lds + wave * (WTM * 16 * ROWQ);
+        const bool wide8 = (p.ldc & 15) == 0 && aligned_dev(p.out, 16);
+        const bool words = (p.ldc & 3) == 0 && aligned_dev(p.out, 4);
+#pragma unroll
+        for (int j = 0; j < WTN; j++) {
+            const int n = n0 + (wn * WTN + j) * 16 + nquad;
+            float sc[4], of[4];
+            int32_t bi[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int nn = min(n + r, p.N - 1);
+                const uint64_t q = p.qparam[p.scale_len == 1 ? 0 : nn];
+                sc[r] = qparam_scale(q);
+                of[r] = qparam_offset(q);
+                bi[r] = p.bias_kind == MI355_BIAS_INT32 ? static_cast<const int32_t *>(p.bias)[nn] : 0;
+            }
+#pragma unroll
+            for (int i = 0; i < WTM; i++) {
+                const int m = m0 + (wm * WTM + i) * 16 + mrow;
+                uint32_t w = 0;
+#pragma unroll
+                for (int r = 0; r < 4; r++) w |= ((uint32_t)requant1(acc[i][j][r], bi[r], sc[r], of[r]) & 0xffu) << (8 * r);
+                if (wide8) {
+                    *reinterpret_cast<uint32_t *>(stq + (i * 16 + mrow) * ROWQ + j * 16 + nquad) = w;
+                    continue;
+                }
+                if (m >= p.M || n >= p.N) continue;
+                int8_t *o = static_cast<int8_t *>(p.out) + (int64_t)m * p.ldc + n;
+                if (words && n + 3 < p.N) {
+                    *reinterpret_cast<uint32_t *>(o) = w;
+                } else {
+                    for (int r = 0; r < 4; r++)
+                        if (n + r < p.N) o[r] = (int8_t)(w >> (8 * r));
+                }
+            }
+        }
+        if (wide8) {
+            const int mw = m0 + wm * WTM * 16, nw = n0 + wn * WTN * 16;
+#pragma unroll
+            for (int q0 = 0; q0 < WTM * 16 * CHQ; q0 += 64) {
+                const int q = q0 + lane;
+                const int row = q / CHQ, ch = q % CHQ;
+                if ((WTM * 16 * CHQ) % 64 != 0 && row >= WTM * 16) continue;
+                const int m = mw + row, n = nw + ch * 16;
+                if (m >= p.M || n >= p.N) continue;
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(stq + row * ROWQ + ch * 16);
+                int8_t *o = static_cast<int8_t *>(p.out) + (int64_t)m * p.ldc + n;
+                if (n + 15 < p.N) {
+                    *reinterpret_cast<u32x4 *>(o) = v;
+                } else {
+                    for (int r = 0; r < 16; r++)
+                        if (n + r < p.N) o[r] = (int8_t)(v[r >> 2] >> ((r & 3) * 8));
+                }
+            }
+        }
+        return;
+    }
     // All dequantisation parameters of this wavefront are fetched in one batch (indices clamped so that every
     // load is in bounds), then every accumulator quad is scaled and rounded.
     float psv[WTM];
@@ -335,11 +416,14 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     }
     f32x4 scv[WTN], bsv[WTN];
     i32x4v biv[WTN];                                          // int32 bias: added to the accumulator before dequantisation
-    const bool quads = (p.N & 3) == 0 && aligned_dev(p.scale, 16) && (!p.bias || aligned_dev(p.bias, 16));
+    const bool quads = (p.N & 3) == 0 && (p.qparam || aligned_dev(p.scale, 16)) && (!p.bias || aligned_dev(p.bias, 16));
 #pragma unroll
     for (int j = 0; j < WTN; j++) {
         const int n = n0 + (wn * WTN + j) * 16 + nquad;
-        if (p.scale_len == 1) {
+        if (p.qparam) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) scv[j][r] = qparam_scale(p.qparam[p.scale_len == 1 ? 0 : min(n + r, p.N - 1)]);
+        } else if (p.scale_len == 1) {
             const float s1 = p.scale[0];
             scv[j] = f32x4{s1, s1, s1, s1};
         } else if (quads) {
@@ -477,7 +561,7 @@ __global__ __launch_bounds__(256) void qmm_generic_kernel(const int8_t *__restri
                                                           const float *__restrict__ pertoken,
                                                           const float *__restrict__ scale, int scale_len,
                                                           const void *__restrict__ bias, int bias_kind, int out_f16, void *out,
-                                                          int out_i32,
+                                                          int out_i32, const uint64_t *__restrict__ qparam, int out_i8,
                                                           int M, int N, int K, int64_t lda, int64_t ldb_k,
                                                           int64_t ldb_n, int64_t ldc)
 {
@@ -486,6 +570,12 @@ __global__ __launch_bounds__(256) void qmm_generic_kernel(const int8_t *__restri
     if (m >= M || n >= N) return;
     int32_t s = 0;
     for (int k = 0; k < K; k++) s += (int32_t)a[(int64_t)m * lda + k] * (int32_t)b[(int64_t)k * ldb_k + (int64_t)n * ldb_n];
+    if (out_i8) {
+        const uint64_t q = qparam[scale_len == 1 ? 0 : n];
+        const int32_t bi = bias_kind == MI355_BIAS_INT32 ? static_cast<const int32_t *>(bias)[n] : 0;
+        static_cast<int8_t *>(out)[(int64_t)m * ldc + n] = (int8_t)requant1(s, bi, qparam_scale(q), qparam_offset(q));
+        return;
+    }
     if (bias_kind == MI355_BIAS_INT32) s = (int32_t)((uint32_t)s + (uint32_t)static_cast<const int32_t *>(bias)[n]);
     if (out_i32) {
         static_cast<int32_t *>(out)[(int64_t)m * ldc + n] = s;
@@ -493,7 +583,7 @@ __global__ __launch_bounds__(256) void qmm_generic_kernel(const int8_t *__restri
     }
     float v = (float)s;
     if (pertoken) v = v * pertoken[m];
-    v = v * scale[scale_len == 1 ? 0 : n];
+    v = v * (qparam ? qparam_scale(qparam[scale_len == 1 ? 0 : n]) : scale[scale_len == 1 ? 0 : n]);
     if (bias_kind == MI355_BIAS_BF16) v = v + bf16_1(static_cast<const uint16_t *>(bias)[n]);
     if (bias_kind == MI355_BIAS_FP32) v = v + static_cast<const float *>(bias)[n];
     static_cast<uint16_t *>(out)[(int64_t)m * ldc + n] = (uint16_t)(out_f16 ? pack_f16x2(v, 0.0f) : pack_bf16x2(v, 0.0f));
@@ -624,21 +714,44 @@ extern "C" size_t mi355_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, 
     return pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes;
 }
 
-extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale,
-                                  int64_t scale_len, const void *bias, int bias_dtype, void *out, int out_dtype, int64_t M,
-                                  int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
-                                  void *workspace, size_t workspace_bytes, void *stream)
+namespace mi355 {
+namespace {
+
+__global__ __launch_bounds__(256) void trans_quant_param_kernel(const float *__restrict__ scale, int scale_one,
+                                                                const float *__restrict__ offset, int offset_one,
+                                                                uint64_t *__restrict__ out, int64_t n)
 {
-    using namespace mi355;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    uint64_t q = (uint64_t)__float_as_uint(scale[scale_one ? 0 : i]) | (1ull << 46);
+    if (offset) {
+        float o = rintf(offset[offset_one ? 0 : i]);
+        o = fminf(fmaxf(o, -256.0f), 255.0f);
+        q |= (uint64_t)((uint32_t)(int32_t)o & 0x1ffu) << 37;
+    }
+    out[i] = q;
+}
+
+// One implementation behind both entry points: `scale` (float32) or `qparam` (packed) carries the per-channel factors.
+int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale, const uint64_t *qparam,
+                     int64_t scale_len, const void *bias, int bias_dtype, void *out, int out_dtype, int64_t M,
+                     int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                     void *workspace, size_t workspace_bytes, void *stream)
+{
     if (M < 0 || N < 0 || K < 0) return MI355_ERR_BAD_ARGUMENT;
-    if (out_dtype != MI355_OUT_BF16 && out_dtype != MI355_OUT_INT32 && out_dtype != MI355_OUT_FP16) return MI355_ERR_BAD_ARGUMENT;
+    if (out_dtype != MI355_OUT_BF16 && out_dtype != MI355_OUT_INT32 && out_dtype != MI355_OUT_FP16 && out_dtype != MI355_OUT_INT8)
+        return MI355_ERR_BAD_ARGUMENT;
+    const int out_i8 = out_dtype == MI355_OUT_INT8;
+    if (out_i8 && (!qparam || pertoken_scale)) return MI355_ERR_BAD_ARGUMENT;
+    if (out_i8 && bias_dtype != MI355_BIAS_NONE && bias_dtype != MI355_BIAS_INT32) return MI355_ERR_UNSUPPORTED;
+    if (qparam && !aligned(qparam, 8)) return MI355_ERR_ALIGNMENT;
     if (bias_dtype < MI355_BIAS_NONE || bias_dtype > MI355_BIAS_FP32) return MI355_ERR_BAD_ARGUMENT;
     if ((bias != nullptr) != (bias_dtype != MI355_BIAS_NONE)) return MI355_ERR_BAD_ARGUMENT;
     if (M == 0 || N == 0) return MI355_OK;
     if (!out || ldc < N) return MI355_ERR_BAD_ARGUMENT;
     if (K > 0 && (!a || !b || lda < K)) return MI355_ERR_BAD_ARGUMENT;
     if (ldb_k != 1 && ldb_n != 1) return MI355_ERR_UNSUPPORTED;
-    if (out_dtype != MI355_OUT_INT32 && (!scale || (scale_len != 1 && scale_len != N))) return MI355_ERR_BAD_ARGUMENT;
+    if (out_dtype != MI355_OUT_INT32 && ((!scale && !qparam) || (scale_len != 1 && scale_len != N))) return MI355_ERR_BAD_ARGUMENT;
     if (out_dtype == MI355_OUT_INT32 && bias_dtype != MI355_BIAS_NONE && bias_dtype != MI355_BIAS_INT32) return MI355_ERR_UNSUPPORTED;
     if (bias && !aligned(bias, bias_dtype == MI355_BIAS_BF16 ? 2 : 4)) return MI355_ERR_ALIGNMENT;
     if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return MI355_ERR_UNSUPPORTED;
@@ -666,7 +779,7 @@ extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float 
     if (!tiled) {
         hipLaunchKernelGGL(qmm_generic_kernel, dim3((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16)), dim3(256), 0, s,
                            a, b, pertoken_scale, scale, (int)scale_len, bias, bias_dtype, out_dtype == MI355_OUT_FP16 ? 1 : 0, out,
-                           out_i32, (int)M, (int)N, (int)K, lda, ldb_k, ldb_n, ldc);
+                           out_i32, qparam, out_i8, (int)M, (int)N, (int)K, lda, ldb_k, ldb_n, ldc);
         return check_launch();
     }
 
@@ -687,6 +800,8 @@ extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float 
     p.K = (int)K;
     p.scale_len = (int)scale_len;
     p.out_i32 = out_i32;
+    p.qparam = qparam;
+    p.out_i8 = out_i8;
     const TileChoice c = pl.tile;
     p.S = pl.S;
     p.counter = pl.S > 1 ? reinterpret_cast<uint32_t *>(ws) : nullptr;
@@ -704,4 +819,42 @@ extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float 
     MI355_QMM_CASE(64, 128, 1, 8)
 #undef MI355_QMM_CASE
     return MI355_ERR_UNSUPPORTED;
+}
+
+} // namespace
+} // namespace mi355
+
+extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale,
+                                  int64_t scale_len, const void *bias, int bias_dtype, void *out, int out_dtype, int64_t M,
+                                  int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                                  void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (out_dtype == MI355_OUT_INT8) return MI355_ERR_BAD_ARGUMENT;          // needs packed parameters
+    return mi355::run_quant_matmul(a, b, pertoken_scale, scale, nullptr, scale_len, bias, bias_dtype, out, out_dtype, M, N, K,
+                                   lda, ldb_k, ldb_n, ldc, workspace, workspace_bytes, stream);
+}
+
+extern "C" int mi355_quant_matmul_qparam(const int8_t *a, const int8_t *b, const uint64_t *qparam, int64_t qparam_len,
+                                         const void *bias, int bias_dtype, void *out, int out_dtype, int64_t M, int64_t N,
+                                         int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc, void *workspace,
+                                         size_t workspace_bytes, void *stream)
+{
+    if (out_dtype == MI355_OUT_INT32) return MI355_ERR_BAD_ARGUMENT;         // an int32 result has no scale
+    if (!qparam && M > 0 && N > 0) return MI355_ERR_BAD_ARGUMENT;
+    return mi355::run_quant_matmul(a, b, nullptr, nullptr, qparam, qparam_len, bias, bias_dtype, out, out_dtype, M, N, K, lda,
+                                   ldb_k, ldb_n, ldc, workspace, workspace_bytes, stream);
+}
+
+extern "C" int mi355_trans_quant_param(const float *scale, int64_t scale_len, const float *offset, int64_t offset_len,
+                                       uint64_t *out, int64_t n, void *stream)
+{
+    using namespace mi355;
+    if (n < 0 || scale_len < 0 || offset_len < 0) return MI355_ERR_BAD_ARGUMENT;
+    if (n == 0) return MI355_OK;
+    if (!scale || !out || (scale_len != 1 && scale_len != n)) return MI355_ERR_BAD_ARGUMENT;
+    if (offset && offset_len != 1 && offset_len != n) return MI355_ERR_BAD_ARGUMENT;
+    if (!aligned(scale, 4) || !aligned(out, 8) || (offset && !aligned(offset, 4))) return MI355_ERR_ALIGNMENT;
+    hipLaunchKernelGGL(trans_quant_param_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), scale, scale_len == 1, offset, offset_len == 1, out, n);
+    return check_launch();
 }

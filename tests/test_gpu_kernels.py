@@ -130,6 +130,56 @@ def test_quant_matmul_bf16(capi, golden, M, K, N, bias):
     assert np.array_equal(_bits(out), want)      # same operation order => bit-identical bf16
 
 
+REQUANT_SHAPES = [(1024, 4096, 11008), (64, 4096, 1024), (48, 256, 192), (130, 384, 1000), (17, 100, 37), (256, 1024, 320)]
+
+
+@pytest.mark.parametrize("M,K,N", REQUANT_SHAPES)
+@pytest.mark.parametrize("weight_nk", [True, False])
+def test_quant_matmul_int8_output(capi, golden, M, K, N, weight_nk):
+    """The re-quantised int8 output through mi355_trans_quant_param + mi355_quant_matmul_qparam, bit-exact against the
+    oracle: tiled kernel (every tile shape these sizes select, split K at M=64), the generic kernel (K=100), with and
+    without an int32 bias, per-channel and single parameters, offsets that clamp and .5 ties."""
+    d = workloads.quant_matmul_inputs(seed=M + N, M=M, K=K, N=N, weight_nk=weight_nk)
+    g = torch.Generator().manual_seed(K)
+    acc_scale = 40.0 / (K ** 0.5 * 74 * 74)                       # spreads the results over the int8 range
+    scale = (torch.rand(N, generator=g) + 0.5) * acc_scale
+    scale[: min(4, N)] = 0.5                                       # exact halves: ties to even
+    offset = torch.randint(-30, 30, (N,), generator=g).float() + torch.rand(N, generator=g)
+    bias = torch.randint(-5000, 5000, (N,), generator=g, dtype=torch.int32)
+    x1, x2 = d["x1"].cuda(), d["x2"].cuda()
+    for sc, of, b in ((scale, offset, bias), (scale, None, None), (scale[:1].clone(), offset[:1].clone(), bias)):
+        qp = capi.trans_quant_param(sc.cuda(), None if of is None else of.cuda())
+        want_q = golden.trans_quant_param(sc.numpy(), None if of is None else of.numpy())
+        assert np.array_equal(qp.cpu().numpy(), want_q)
+        got = capi.quant_matmul_qparam(x1, x2, qp, None if b is None else b.cuda(), torch.int8)
+        qfull = np.repeat(want_q, N) if want_q.size == 1 else want_q
+        want = golden.quant_matmul_requant(d["x1"].numpy(), d["x2"].numpy(), qfull, None if b is None else b.numpy())
+        assert got.dtype == torch.int8
+        assert np.array_equal(got.cpu().numpy(), want)
+        assert np.abs(want.astype(np.int32)).max() > 20           # not everything collapsed to zero
+
+
+def test_quant_matmul_packed_scale_float_outputs(capi, golden):
+    """A packed scale with fp16 / bf16 output equals the float32-scale path bit for bit (the offset field is ignored)."""
+    d = workloads.quant_matmul_inputs(seed=11, M=96, K=512, N=384, weight_nk=True)
+    off = torch.full((384,), 7.0)
+    qp = capi.trans_quant_param(d["scale"].cuda(), off.cuda())
+    for dt in (torch.float16, torch.bfloat16):
+        a = capi.quant_matmul_qparam(d["x1"].cuda(), d["x2"].cuda(), qp, None, dt)
+        b = capi.quant_matmul(d["x1"].cuda(), d["x2"].cuda(), d["scale"].cuda(), None, None, dt)
+        assert torch.equal(a, b)
+    L = capi.lib()
+    import ctypes
+    vp = ctypes.c_void_p
+    x1, x2 = d["x1"].cuda(), d["x2"].cuda()
+    out = torch.empty(96, 384, dtype=torch.int8, device="cuda")
+    # int8 output without packed parameters, and an int32 output through the packed entry point, are refused
+    assert L.mi355_quant_matmul(vp(x1.data_ptr()), vp(x2.data_ptr()), None, vp(d["scale"].cuda().data_ptr()), 384, None, 0,
+                                vp(out.data_ptr()), 3, 96, 384, 512, 512, 1, 512, 384, None, 0, None) == -1
+    assert L.mi355_quant_matmul_qparam(vp(x1.data_ptr()), vp(x2.data_ptr()), vp(qp.data_ptr()), 384, None, 0,
+                                       vp(out.data_ptr()), 1, 96, 384, 512, 512, 1, 512, 384, None, 0, None) == -1
+
+
 def test_quant_matmul_random_shapes(capi, golden):
     """Seeded sweep over shapes (tiled, split over K, generic), weight layouts, bias kinds and output types: int32
     accumulators and rounded outputs bit-identical to the oracle."""

@@ -119,6 +119,41 @@ def test_linear_quant_module_equals_operator(pa):
         assert torch.equal(got, want)
 
 
+def test_quant_matmul_int8_output_operator_and_module(pa, golden):
+    """npu_quant_matmul with output_dtype None / int8 (test/test_fake_tensor.py:1886-1895): a float32 scale is packed
+    like npu_trans_quant_param packs it, an int64 scale is taken as packed; LinearQuant's default configuration
+    (float32 scale, no pertoken_scale, output_dtype None) goes through npu_trans_quant_param like the reference's
+    forward (linear_quant.py:104-112) and equals the direct call."""
+    from pytorch_amd.contrib.module import LinearQuant
+    d = workloads.quant_matmul_inputs(seed=21, M=48, K=256, N=192, weight_nk=True)
+    g = torch.Generator().manual_seed(2)
+    scale = (torch.rand(192, generator=g) + 0.5) * 4e-4
+    offset = torch.randint(-20, 20, (192,), generator=g).float()
+    bias = torch.randint(-3000, 3000, (192,), generator=g, dtype=torch.int32)
+    want = golden.quant_matmul_requant(d["x1"].numpy(), d["x2"].numpy(), golden.trans_quant_param(scale.numpy(), offset.numpy()),
+                                       bias.numpy())
+    x1, x2 = d["x1"].cuda(), d["x2"].cuda()
+    out = pa.npu_quant_matmul(x1, x2, scale.cuda(), offset=offset.cuda(), bias=bias.cuda())
+    assert out.dtype == torch.int8 and np.array_equal(out.cpu().numpy(), want)
+    qp = pa.npu_trans_quant_param(scale.cuda(), offset.cuda())
+    assert qp.dtype == torch.int64 and np.array_equal(qp.cpu().numpy(), golden.trans_quant_param(scale.numpy(), offset.numpy()))
+    out2 = pa.npu_quant_matmul(x1, x2, qp, offset=offset.cuda(), bias=bias.cuda(), output_dtype=torch.int8)
+    assert torch.equal(out, out2)
+    # batched x1 against one weight
+    xb = torch.stack([d["x1"], d["x1"].flip(0)]).cuda()
+    ob = pa.npu_quant_matmul(xb, x2, qp, bias=bias.cuda(), output_dtype=torch.int8)
+    assert ob.shape == (2, 48, 192) and torch.equal(ob[0], out) and torch.equal(ob[1], out.flip(0))
+    m = LinearQuant(256, 192, bias=True, offset=True).cuda()
+    m.weight.data = d["x2"].t().contiguous().cuda()
+    m.scale.data, m.offset.data, m.bias.data = scale.cuda(), offset.cuda(), bias.cuda()
+    assert torch.equal(m(x1), out)
+    # float16 output of the module: packed scale, same numbers as the float32 scale
+    m16 = LinearQuant(256, 192, bias=False, output_dtype=torch.float16).cuda()
+    m16.weight.data = d["x2"].t().contiguous().cuda()
+    m16.scale.data = scale.cuda()
+    assert torch.equal(m16(x1), pa.npu_quant_matmul(x1, x2, scale.cuda(), output_dtype=torch.float16))
+
+
 def test_linear_quant_module_default_int32_bias_and_fp16(pa, golden):
     """LinearQuant as its constructor builds it (int32 bias, linear_quant.py:92) with float16 and bfloat16 outputs,
     against the oracle's statement of the formula."""

@@ -17,7 +17,8 @@ def test_c_abi_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "mi355_quant.h")).read()
     declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", header))
     assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant", "mi355_anti_quant",
-            "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize"} <= declared
+            "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize", "mi355_trans_quant_param",
+            "mi355_quant_matmul_qparam"} <= declared
     lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_amd", "csrc", "libmi355_quant.so"))
     for name in declared:
         assert hasattr(lib, name), name
@@ -101,14 +102,21 @@ def test_meta_quant_matmul(pa):
                             pertoken_scale=_m(16, dtype=torch.float32), output_dtype=torch.bfloat16)
     assert r.shape == (16, 32)
     # unsupported variants raise, never silently ignored
-    with pytest.raises(RuntimeError, match="output_dtype=None"):
-        pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), offset=_m(1, dtype=torch.float32))
+    # output_dtype None is the re-quantised int8 output (test_fake_tensor.py:1886-1895), with a float32 or int64 scale
+    r = pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), offset=_m(1, dtype=torch.float32))
+    assert r.shape == (1, 1, 100) and r.dtype == torch.int8
+    r = pa.npu_quant_matmul(x1, x2, _m(100, dtype=torch.int64), bias=_m(100, dtype=torch.int32), output_dtype=torch.int8)
+    assert r.dtype == torch.int8
+    r = pa.npu_quant_matmul(x1, x2, _m(100, dtype=torch.int64), output_dtype=torch.float16)
+    assert r.dtype == torch.float16
+    with pytest.raises(RuntimeError, match="pertoken_scale is not applicable to int8"):
+        pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), pertoken_scale=_m(1, dtype=torch.float32))
     with pytest.raises(RuntimeError, match="offset"):
         pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), offset=_m(1, dtype=torch.float32), output_dtype=torch.bfloat16)
     r = pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), bias=_m(100, dtype=torch.int32), output_dtype=torch.float16)
     assert r.shape == (1, 1, 100) and r.dtype == torch.float16          # test_fake_tensor.py:1903-1906
     with pytest.raises(RuntimeError, match="output_dtype must be"):
-        pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), output_dtype=torch.int8)
+        pa.npu_quant_matmul(x1, x2, _m(1, dtype=torch.float32), output_dtype=torch.float32)
     # both operands packed int4: last dimension of x2 times 8 (test_fake_tensor.py:1917-1923), or the transposed
     # [N, K/8] weight of the module example (linear_quant.py:40-50)
     r = pa.npu_quant_matmul(_m(16, 8, dtype=torch.int32), _m(64, 5, dtype=torch.int32), _m(1, dtype=torch.float32),
@@ -203,6 +211,19 @@ def test_meta_anti_quant(pa):
         pa.npu_anti_quant(_m(4, 8, dtype=torch.int16), _m(8, dtype=torch.float32))
 
 
+def test_meta_trans_quant_param(pa):
+    """test/test_fake_tensor.py:1929-1943: int64, the shape of the larger argument."""
+    res = pa.npu_trans_quant_param(_m(1, dtype=torch.float32), _m(4, dtype=torch.float32))
+    assert res.shape == (4,) and res.dtype == torch.int64
+    res = pa.npu_trans_quant_param(_m(1, 4, dtype=torch.float32), _m(1, 4, dtype=torch.float32))
+    assert res.shape == (1, 4) and res.dtype == torch.int64
+    assert pa.npu_trans_quant_param(_m(7, dtype=torch.float32)).shape == (7,)
+    with pytest.raises(RuntimeError, match="scale must be float32"):
+        pa.npu_trans_quant_param(_m(4, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="same number of elements"):
+        pa.npu_trans_quant_param(_m(3, dtype=torch.float32), _m(4, dtype=torch.float32))
+
+
 def test_meta_npu_quantize(pa):
     """Shapes and output types of npu_quantize (signature test/torch_npu_schema.json:2273-2275; dtype codes
     torch_npu/onnx/wrapper_onnx_ops.py:869-877) without a GPU."""
@@ -269,11 +290,14 @@ def test_linear_quant_marshalling(pa, monkeypatch):
     assert set(kwargs) == {"offset", "pertoken_scale", "bias", "output_dtype"}
     with pytest.raises(ValueError, match="both torch.int32 or both torch.int8"):
         m(_m(16, 64, dtype=torch.float16))
-    # float32 scale without pertoken_scale and without bf16/int32 output would need npu_trans_quant_param
-    m2 = LinearQuant(64, 32, bias=False).to("meta")
+    # float32 scale without pertoken_scale and without bf16/int32 output goes through npu_trans_quant_param
+    # (linear_quant.py:104-108) and yields the re-quantised int8 output
+    rec2 = _Recorder(monkeypatch, "npu_trans_quant_param")
+    m2 = LinearQuant(64, 32, bias=False, offset=True).to("meta")
     m2.weight.data = _m(32, 64, dtype=torch.int8)
-    with pytest.raises(NotImplementedError, match="npu_trans_quant_param"):
-        m2(_m(16, 64, dtype=torch.int8))
+    out = m2(_m(16, 64, dtype=torch.int8))
+    assert out.dtype == torch.int8 and out.shape == (16, 32)
+    assert len(rec2.calls) == 1 and rec.calls[-1][0][2].dtype == torch.int64
     with pytest.warns(FutureWarning):
         a = LinearA8W8Quant(64, 32, bias=True, output_dtype=torch.bfloat16)
     assert a.bias.dtype == torch.int32

@@ -152,3 +152,33 @@ def test_a4w4_accumulator_is_the_integer_product(golden, words_along_k):
         assert np.array_equal(acc.astype(np.int64), want)
         ref = ((want + bias[None, :]).astype(np.float32) * scale[0]).astype(np.float16).view(np.uint16)
         assert np.array_equal(out, ref)
+
+
+def test_trans_quant_param_words(golden):
+    """Hand-assembled words: scale bits in the low half, a 9-bit two's-complement offset at bit 37, bit 46 set."""
+    q = golden.trans_quant_param(np.float32([1.0, 0.5, -2.0]))
+    assert [hex(int(v)) for v in q.view(np.uint64)] == ["0x40003f800000", "0x40003f000000", "0x4000c0000000"]
+    q = golden.trans_quant_param(np.float32([1.0]), np.float32([3.0, -1.0, 2.5, 3.5, 300.0, -300.0]))
+    fields = [(int(v) >> 37) & 0x1FF for v in q.view(np.uint64)]
+    assert fields == [3, 0x1FF, 2, 4, 255, 256]               # ties to even, clamp to [-256, 255]
+    assert all((int(v) >> 46) & 1 == 1 and int(v) & 0xFFFFFFFF == 0x3F800000 for v in q.view(np.uint64))
+    sc, of = golden.quant_param_decode(q)
+    assert sc.tolist() == [1.0] * 6 and of.tolist() == [3.0, -1.0, 2.0, 4.0, 255.0, -256.0]
+
+
+def test_quant_matmul_requant_against_numpy_int64(golden):
+    rng = np.random.default_rng(3)
+    a = rng.integers(-128, 128, (9, 64), dtype=np.int8)
+    b = rng.integers(-128, 128, (64, 24), dtype=np.int8)
+    bias = rng.integers(-1000, 1000, 24, dtype=np.int32)
+    scale = (rng.random(24, dtype=np.float32) * 4e-3 + 1e-4).astype(np.float32)
+    offset = rng.integers(-20, 20, 24).astype(np.float32)
+    q = golden.trans_quant_param(scale, offset)
+    got = golden.quant_matmul_requant(a, b, q, bias)
+    acc = a.astype(np.int64) @ b.astype(np.int64) + bias
+    want = np.clip(np.rint((acc.astype(np.float32) * scale).astype(np.float32) + offset), -128, 127).astype(np.int8)
+    assert np.array_equal(got, want)
+    # scale 1, offset 0: the clamped accumulator itself
+    one = golden.trans_quant_param(np.float32([1.0]))
+    small = golden.quant_matmul_requant(a[:, :1] // 16, b[:1, :] // 16, np.repeat(one, 24))
+    assert np.array_equal(small, np.clip((a[:, :1] // 16).astype(np.int64) @ (b[:1, :] // 16).astype(np.int64), -128, 127))
