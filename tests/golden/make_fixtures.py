@@ -79,8 +79,30 @@ def write_later_fixtures():
     np.savez_compressed(os.path.join(HERE, "dynamic_quant_asymmetric.npz"), x=bits(x), smooth=bits(sm), y=y, scale=s, offset=o)
 
 
+def write_quantize_fixtures():
+    """Static quantisation and the re-quantised int8 output of quant_matmul (files of their own, see above)."""
+    g = torch.Generator().manual_seed(31)
+    x = (torch.randn(6, 24, 4, generator=g) * 40).to(torch.bfloat16)
+    sc = (torch.rand(24, generator=g) + 0.25).numpy()
+    zp = torch.randint(-10, 10, (24,), generator=g, dtype=torch.int32).numpy()
+    xf = x.float().numpy()
+    np.savez_compressed(os.path.join(HERE, "quantize.npz"), x=bits(x), scale=sc, zero_point=zp,
+                        q_div_i8=golden.quantize(xf, sc, zp.astype(np.float32), "int8", 1, True),
+                        q_mul_u8=golden.quantize(xf, sc, zp.astype(np.float32), "uint8", 1, False))
+    x1 = torch.randint(-128, 128, (20, 256), generator=g, dtype=torch.int8).numpy()
+    x2 = torch.randint(-128, 128, (256, 48), generator=g, dtype=torch.int8).numpy()
+    scale = ((torch.rand(48, generator=g) + 0.5) * 4e-4).numpy()
+    offset = torch.randint(-20, 20, (48,), generator=g).float().numpy()
+    bias = torch.randint(-3000, 3000, (48,), generator=g, dtype=torch.int32).numpy()
+    qp = golden.trans_quant_param(scale, offset)
+    np.savez_compressed(os.path.join(HERE, "quant_matmul_int8.npz"), x1=x1, x2=x2, scale=scale, offset=offset, bias=bias,
+                        qparam=qp, out=golden.quant_matmul_requant(x1, x2, qp, bias))
+
+
 if __name__ == "__main__":
-    if "--later-only" in sys.argv:
+    if "--quantize-only" in sys.argv:
+        write_quantize_fixtures()
+    elif "--later-only" in sys.argv:
         write_later_fixtures()
     else:
         main()

@@ -151,3 +151,29 @@ def test_gpu_reproduces_later_fixtures(capi):
     y, s, o = capi.dynamic_quant_asymmetric(_bf16(f["x"]).cuda(), _bf16(f["smooth"]).cuda())
     assert np.array_equal(y.cpu().numpy(), f["y"]) and np.array_equal(s.cpu().numpy(), f["scale"])
     assert np.array_equal(o.cpu().numpy(), f["offset"])
+
+
+def test_oracle_reproduces_quantize_fixtures(golden):
+    f = _npz("quantize.npz")
+    xf = _bf16(f["x"]).float().numpy()
+    zp = f["zero_point"].astype(np.float32)
+    assert np.array_equal(golden.quantize(xf, f["scale"], zp, "int8", 1, True), f["q_div_i8"])
+    assert np.array_equal(golden.quantize(xf, f["scale"], zp, "uint8", 1, False), f["q_mul_u8"])
+    f = _npz("quant_matmul_int8.npz")
+    assert np.array_equal(golden.trans_quant_param(f["scale"], f["offset"]), f["qparam"])
+    assert np.array_equal(golden.quant_matmul_requant(f["x1"], f["x2"], f["qparam"], f["bias"]), f["out"])
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_quantize_fixtures(capi):
+    import pytorch_amd as pa
+    f = _npz("quantize.npz")
+    x, sc, zp = _bf16(f["x"]).cuda(), torch.from_numpy(f["scale"]).cuda(), torch.from_numpy(f["zero_point"]).cuda()
+    assert np.array_equal(pa.npu_quantize(x, sc, zp, torch.qint8, 1).cpu().numpy(), f["q_div_i8"])
+    assert np.array_equal(pa.npu_quantize(x, sc, zp, torch.quint8, 1, False).cpu().numpy(), f["q_mul_u8"])
+    f = _npz("quant_matmul_int8.npz")
+    x1, x2, scale, offset, bias = (torch.from_numpy(f[k]).cuda() for k in ("x1", "x2", "scale", "offset", "bias"))
+    qp = pa.npu_trans_quant_param(scale, offset)
+    assert np.array_equal(qp.cpu().numpy(), f["qparam"])
+    assert np.array_equal(pa.npu_quant_matmul(x1, x2, qp, bias=bias, output_dtype=torch.int8).cpu().numpy(), f["out"])
+    assert np.array_equal(pa.npu_quant_matmul(x1, x2, scale, offset=offset, bias=bias).cpu().numpy(), f["out"])
