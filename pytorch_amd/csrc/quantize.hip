@@ -187,9 +187,9 @@ int launch_quantize_mode(const QzArgs &p, int vec_mode, hipStream_t s)
     } else if (vec_mode == 2) {
         const int64_t rows = p.total / p.channels;
         const int64_t bx = (p.channels / 8 + 255) / 256;
-        // a block loads its parameters once: give it at least 16 rows (four steps) where that still leaves two
+        // a block loads its parameters once: give it at least 8 rows (two steps) where that still leaves two
         // blocks per CU, and never more blocks than fill the chip several times over
-        int64_t by = (rows + 15) / 16;
+        int64_t by = (rows + 7) / 8;
         const int64_t fill = (512 + bx - 1) / bx, cap = (256 * 16 + bx - 1) / bx;
         if (by < fill) by = std::min<int64_t>(fill, (rows + 3) / 4);
         if (by > cap) by = cap;
