@@ -607,6 +607,42 @@ __global__ __launch_bounds__(256) void transpose_i8_kernel(const int8_t *__restr
     }
 }
 
+// The same for 16-byte aligned rows on both sides: 128x128 byte tiles, 16-byte loads along N and 16-byte stores along K
+// (whole 128-byte lines either way); the transposition itself is done by byte reads from LDS.
+__global__ __launch_bounds__(256) void transpose_i8_wide_kernel(const int8_t *__restrict__ src, int8_t *__restrict__ dst,
+                                                                int K, int N, int64_t ld_src)
+{
+    constexpr int T = 128, PITCH = T + 4;                     // pitch 33 dwords: a column walk changes bank every row
+    __shared__ __attribute__((aligned(16))) int8_t tile[T * PITCH];
+    const int k0 = blockIdx.y * T, n0 = blockIdx.x * T;
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int r = (t >> 3) + 32 * i, c = (t & 7) * 16;    // row k0 + r, bytes n0 + c .. + 15
+        u32x4 v{0u, 0u, 0u, 0u};
+        if (k0 + r < K && n0 + c < N) {                       // N % 16 == 0: a chunk is inside or outside as a whole
+            v = *reinterpret_cast<const u32x4 *>(src + (int64_t)(k0 + r) * ld_src + n0 + c);
+        }
+        uint32_t *d = reinterpret_cast<uint32_t *>(tile + r * PITCH + c);
+        d[0] = v.x, d[1] = v.y, d[2] = v.z, d[3] = v.w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int n = (t >> 3) + 32 * i, kc = (t & 7) * 16;   // output row n0 + n, bytes k0 + kc .. + 15
+        if (n0 + n >= N || k0 + kc >= K) continue;            // K % 16 == 0
+        u32x4 v;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            uint32_t x = 0;
+#pragma unroll
+            for (int b = 0; b < 4; b++) x |= (uint32_t)(uint8_t)tile[(kc + 4 * w + b) * PITCH + n] << (8 * b);
+            v[w] = x;
+        }
+        *reinterpret_cast<u32x4 *>(dst + (int64_t)(n0 + n) * K + k0 + kc) = v;
+    }
+}
+
 template <int WGM, int WGN, int WTM, int WTN>
 int launch_qmm(QmmArgs p, hipStream_t s)
 {
@@ -770,8 +806,12 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     if (tiled && ldb_k != 1) {
         // contiguous [K,N]: transpose once into the workspace
         int8_t *dst = reinterpret_cast<int8_t *>(ws + pl.counter_bytes + pl.partial_bytes);
-        hipLaunchKernelGGL(transpose_i8_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64)), dim3(256), 0,
-                           s, b, dst, (int)K, (int)N, ldb_k);
+        if ((N & 15) == 0 && (K & 15) == 0 && (ldb_k & 15) == 0 && aligned(b, 16) && aligned(dst, 16))
+            hipLaunchKernelGGL(transpose_i8_wide_kernel, dim3((unsigned)((N + 127) / 128), (unsigned)((K + 127) / 128)),
+                               dim3(256), 0, s, b, dst, (int)K, (int)N, ldb_k);
+        else
+            hipLaunchKernelGGL(transpose_i8_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64)), dim3(256), 0,
+                               s, b, dst, (int)K, (int)N, ldb_k);
         bt = dst;
         ldbt = K;
     }
