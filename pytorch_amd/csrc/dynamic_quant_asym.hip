@@ -4,7 +4,8 @@
 // A row whose elements are all equal has scale 0, offset 0 and y 0.
 //
 // One 256-thread block per row, two passes over the row: the first reduces the minimum and the maximum, the second
-// re-reads the row (it is in cache by then: HBM sees it once), divides, adds the offset and stores packed int8.
+// divides, adds the offset and stores packed int8; rows of up to 8192 elements stay in registers between the passes,
+// longer ones are re-read (they are in cache by then: HBM sees them once).
 // The division is IEEE-correct (about a dozen instructions per element), which at [2048, 4096] costs about as much
 // as the memory traffic.
 #include "common.h"
@@ -31,7 +32,8 @@ __device__ __forceinline__ uint32_t quant1(float x, float scale, float offset)
 }
 
 // VEC: cols % 8 == 0, rows (and smooth) 16-byte aligned, y rows 8-byte aligned
-template <bool FP16, bool VEC>
+// REG (with VEC): cols <= 8192, the row stays in registers between the two passes (four 16-byte vectors per thread)
+template <bool FP16, bool VEC, bool REG = false>
 __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ smooth,
                                                       int8_t *__restrict__ y, float *__restrict__ scale_out,
                                                       float *__restrict__ offset_out, int64_t rows, int cols, int64_t row_stride)
@@ -42,9 +44,19 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
         const uint16_t *xr = x + row * row_stride;
         int8_t *yr = y + row * (int64_t)cols;
         float mx = -INFINITY, mn = INFINITY;
+        u32x4 kept[REG ? 4 : 1];
+        if constexpr (REG) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int v = t + 256 * i;
+                kept[i] = v < cols / 8 ? reinterpret_cast<const u32x4 *>(xr)[v] : u32x4{0, 0, 0, 0};
+            }
+        }
         if constexpr (VEC) {
-            for (int v = t; v < cols / 8; v += 256) {
-                const u32x4 a = reinterpret_cast<const u32x4 *>(xr)[v];
+            for (int v = t, it = 0; v < cols / 8; v += 256, it++) {
+                u32x4 a;
+                if constexpr (REG) a = it == 0 ? kept[0] : it == 1 ? kept[1] : it == 2 ? kept[2] : kept[3];
+                else a = reinterpret_cast<const u32x4 *>(xr)[v];
                 u32x4 s = u32x4{0, 0, 0, 0};
                 if (smooth) s = reinterpret_cast<const u32x4 *>(smooth)[v];
 #pragma unroll
@@ -79,8 +91,10 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
         if (flat) scale = 0.0f, offset = 0.0f;
         if (t == 0) scale_out[row] = scale, offset_out[row] = offset;
         if constexpr (VEC) {
-            for (int v = t; v < cols / 8; v += 256) {
-                const u32x4 a = reinterpret_cast<const u32x4 *>(xr)[v];
+            for (int v = t, it = 0; v < cols / 8; v += 256, it++) {
+                u32x4 a;
+                if constexpr (REG) a = it == 0 ? kept[0] : it == 1 ? kept[1] : it == 2 ? kept[2] : kept[3];
+                else a = reinterpret_cast<const u32x4 *>(xr)[v];
                 u32x4 s = u32x4{0, 0, 0, 0};
                 if (smooth) s = reinterpret_cast<const u32x4 *>(smooth)[v];
                 uint32_t q[8];
@@ -124,12 +138,15 @@ extern "C" int mi355_dynamic_quant_asymmetric(const void *x, int in_dtype, const
     hipStream_t s = static_cast<hipStream_t>(stream);
     const unsigned blocks = (unsigned)(rows < 256 * 64 ? rows : 256 * 64);
     const bool f16 = in_dtype == MI355_DTYPE_FP16;
-#define MI355_DQA_LAUNCH(F, V) \
-    hipLaunchKernelGGL((dq_asym_kernel<F, V>), dim3(blocks), dim3(256), 0, s, xp, sp, y, scale, offset, rows, (int)cols, x_row_stride)
-    if (f16 && vec) MI355_DQA_LAUNCH(true, true);
-    else if (f16) MI355_DQA_LAUNCH(true, false);
-    else if (vec) MI355_DQA_LAUNCH(false, true);
-    else MI355_DQA_LAUNCH(false, false);
+#define MI355_DQA_LAUNCH(F, V, R) \
+    hipLaunchKernelGGL((dq_asym_kernel<F, V, R>), dim3(blocks), dim3(256), 0, s, xp, sp, y, scale, offset, rows, (int)cols, x_row_stride)
+    const bool reg = vec && cols <= 8192;
+    if (f16 && reg) MI355_DQA_LAUNCH(true, true, true);
+    else if (f16 && vec) MI355_DQA_LAUNCH(true, true, false);
+    else if (f16) MI355_DQA_LAUNCH(true, false, false);
+    else if (reg) MI355_DQA_LAUNCH(false, true, true);
+    else if (vec) MI355_DQA_LAUNCH(false, true, false);
+    else MI355_DQA_LAUNCH(false, false, false);
 #undef MI355_DQA_LAUNCH
     return check_launch();
 }
