@@ -29,14 +29,62 @@ __device__ __forceinline__ float load1(const void *x, int64_t e)
     else return static_cast<const float *>(x)[e];
 }
 
-template <bool DIV>
-__device__ __forceinline__ float quant1(float x, float sc, float zp, float qmin, float qmax)
+// After the quotient (or product): add the zero point, round half to even, clamp.
+__device__ __forceinline__ float finish1(float v, float zp, float qmin, float qmax)
 {
-    float v = DIV ? x / sc : x * sc;
     v = v + zp;
     v = rintf(v);                                     // ties to even
     v = v == v ? v : 0.0f;                            // NaN quantises to 0
     return fminf(fmaxf(v, qmin), qmax);               // (int32: qmax is 2^31 as a float, see to_i32)
+}
+
+template <bool DIV>
+__device__ __forceinline__ float quant1(float x, float sc, float zp, float qmin, float qmax)
+{
+    return finish1(DIV ? x / sc : x * sc, zp, qmin, qmax);
+}
+
+// Division by a channel's scale with the reciprocal formed once per channel: the operation sequence of the compiler's
+// own float32 division (reciprocal refined once, quotient, two residual corrections with fused multiply-adds) without
+// its range scaling and special-case fix-up, which are the identity while no intermediate leaves the normal range.
+// Used for a group of elements only when every lane of the wavefront has scale and numerators within [2^-60, 2^60]
+// (zero numerators too); otherwise the whole wavefront takes the ordinary division, so there is one scalar branch
+// per group and never both computations.
+__device__ __forceinline__ bool safe_range(float v)
+{
+    const float a = __builtin_fabsf(v);
+    return a >= 0x1p-60f && a <= 0x1p60f;
+}
+__device__ __forceinline__ float refined_rcp(float d)
+{
+    const float r = __builtin_amdgcn_rcpf(d);
+    return __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+}
+__device__ __forceinline__ float div_by_rcp(float x, float d, float r)
+{
+    float q = x * r;
+    q = __builtin_fmaf(__builtin_fmaf(-d, q, x), r, q);
+    q = __builtin_fmaf(__builtin_fmaf(-d, q, x), r, q);
+    return q;
+}
+
+// q[i] = quantised x[i] for eight elements with per-element scale sc[i], reciprocal rc[i] and zero point zp[i]
+template <bool DIV>
+__device__ __forceinline__ void quant8(const float (&x)[8], const float (&sc)[8], const float (&rc)[8], bool scales_safe,
+                                       const float (&zp)[8], float qmin, float qmax, float (&q)[8])
+{
+    if constexpr (DIV) {
+        bool ok = scales_safe;
+#pragma unroll
+        for (int i = 0; i < 8; i++) ok = ok && (safe_range(x[i]) || x[i] == 0.0f);
+        if (__builtin_amdgcn_ballot_w64(!ok) == 0) {          // uniform over the wavefront
+#pragma unroll
+            for (int i = 0; i < 8; i++) q[i] = finish1(div_by_rcp(x[i], sc[i], rc[i]), zp[i], qmin, qmax);
+            return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) q[i] = quant1<DIV>(x[i], sc[i], zp[i], qmin, qmax);
 }
 
 __device__ __forceinline__ float zp_at(const QzArgs &p, int64_t i)
@@ -112,8 +160,10 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(const QzArgs p)
         const int64_t c = single ? 0 : (e / p.inner) % p.channels;
         const float sc = p.scale[p.scale_one ? 0 : c];
         const float zp = p.zp ? zp_at(p, p.zp_one ? 0 : c) : 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) q[i] = quant1<DIV>(x[i], sc, zp, p.qmin, p.qmax);
+        const float r = DIV ? refined_rcp(sc) : 0.0f;
+        const float sc8[8] = {sc, sc, sc, sc, sc, sc, sc, sc}, rc8[8] = {r, r, r, r, r, r, r, r};
+        const float zp8[8] = {zp, zp, zp, zp, zp, zp, zp, zp};
+        quant8<DIV>(x, sc8, rc8, safe_range(sc), zp8, p.qmin, p.qmax, q);
         store8<OUT>(p.out, e, q);
     }
 }
@@ -147,6 +197,13 @@ __global__ __launch_bounds__(256) void quantize_cols_kernel(const QzArgs p)
             zp[4 + i] = p.zp_int ? (float)(int32_t)b[i] : __uint_as_float(b[i]);
         }
     }
+    float rc[8];
+    bool scales_safe = true;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        rc[i] = DIV ? refined_rcp(sc[i]) : 0.0f;
+        scales_safe = scales_safe && safe_range(sc[i]);
+    }
     const int64_t rows = p.total / p.channels;
     constexpr int RU = 4;
     for (int64_t r0 = (int64_t)blockIdx.y * RU; r0 < rows; r0 += (int64_t)gridDim.y * RU) {
@@ -157,8 +214,7 @@ __global__ __launch_bounds__(256) void quantize_cols_kernel(const QzArgs p)
         for (int u = 0; u < RU; u++) {
             if (r0 + u >= rows) break;
             float q[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++) q[i] = quant1<DIV>(x[u][i], sc[i], zp[i], p.qmin, p.qmax);
+            quant8<DIV>(x[u], sc, rc, scales_safe, zp, p.qmin, p.qmax, q);
             store8<OUT>(p.out, (r0 + u) * p.channels + c, q);
         }
     }

@@ -682,6 +682,26 @@ def test_quantize_matches_torch_per_channel(capi):
     assert torch.equal(got.cpu(), want)
 
 
+def test_quantize_extreme_operands(capi, golden):
+    """Operands outside the range where the kernel divides through the channel's reciprocal (tiny, huge, infinite,
+    NaN, denormal numerators; tiny and huge scales): the ordinary division takes over for the whole wavefront, and
+    results stay equal to the oracle element by element."""
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(64, 256, generator=g) * 50
+    special = torch.tensor([1e-30, -1e-30, 1e30, -1e30, float("inf"), float("-inf"), float("nan"), 1e-42, 0.0, -0.0, 3e-20, 7e19])
+    x[::3, :12] = special                                        # some wavefronts see them, others do not
+    scale = torch.rand(256, generator=g) + 0.5
+    scale[5], scale[9], scale[200] = 1e-25, 1e25, 3e-39          # channels with scales outside the range (one denormal)
+    zp = torch.randint(-5, 5, (256,), generator=g).float()
+    with np.errstate(all="ignore"):
+        for name, dt in (("int8", torch.int8), ("int32", torch.int32)):
+            want = golden.quantize(x.numpy(), scale.numpy(), zp.numpy(), name, -1, True)
+            got = capi.quantize(x.cuda(), scale.cuda(), zp.cuda(), dt, -1, True)
+            assert np.array_equal(got.cpu().numpy(), want), name
+        want = golden.quantize(x.numpy(), scale[:1].numpy(), None, "int8", -1, True)
+        assert np.array_equal(capi.quantize(x.cuda(), scale[:1].cuda(), None, torch.int8, -1, True).cpu().numpy(), want)
+
+
 def test_quantize_bad_arguments(capi):
     import ctypes
     L = capi.lib()
