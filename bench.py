@@ -321,6 +321,13 @@ def main():
         calls = [(lambda x=x: keep.append(pa.npu_dynamic_quant_asymmetric(x))) for x in xs] * 2
         us = _graph_time_us(torch, calls)
         others.append(hbm_entry("dynamic_quant_asymmetric bf16[2048,4096] (rotating, > Infinity Cache)", nb + rows * 4, us, None))
+        # SmoothQuant activations: the row is multiplied by per-column smooth scales before it is quantised
+        keep.clear()
+        smq = (torch.rand(xs[0].shape[-1], generator=gen, device=dev) + 0.5).to(torch.bfloat16)
+        calls = [(lambda x=x: keep.append(pa.npu_dynamic_quant(x, smooth_scales=smq))) for x in xs] * 2
+        us = _graph_time_us(torch, calls)
+        others.append(hbm_entry("dynamic_quant with smooth_scales bf16[2048,4096] (rotating, > Infinity Cache)",
+                                nb + xs[0].shape[-1] * 2, us, None))
         del xs, keep
 
     if want("c3"):

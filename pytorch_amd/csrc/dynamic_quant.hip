@@ -223,6 +223,91 @@ __global__ __launch_bounds__(kBlock) void dq_generic_kernel(const uint16_t *__re
     }
 }
 
+// Rows pre-multiplied by smooth scales, cols % 8 == 0 and at most 8192, 16-byte aligned rows and smooth scales: one
+// block per row, the products (arbitrary float32 significands) stay in registers between the maximum and the
+// quantisation.  x / scale uses the row's refined reciprocal with the operation sequence of the compiler's own
+// float32 division (quotient and two residual corrections) whenever every lane of the wavefront has scale and
+// numerators within [2^-60, 2^60] or zero, where that sequence's range scaling and fix-up are the identity; otherwise
+// the wavefront divides the ordinary way.  One scalar branch per eight elements, never both computations.
+template <bool FP16>
+__global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *__restrict__ x,
+                                                                const uint16_t *__restrict__ smooth,
+                                                                int8_t *__restrict__ y, float *__restrict__ scale_out,
+                                                                int cols, int64_t row_stride)
+{
+    constexpr int MAXV = 4;
+    const int64_t row = blockIdx.x;
+    const int t = threadIdx.x, nvec = cols >> 3;
+    const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + row * row_stride);
+    const u32x4 *sr = reinterpret_cast<const u32x4 *>(smooth);
+    float f[MAXV][8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MAXV; i++) {
+        const int idx = t + i * kBlock;
+        u32x4 a{0, 0, 0, 0}, b{0, 0, 0, 0};
+        if (idx < nvec) a = __builtin_nontemporal_load(xr + idx), b = sr[idx];
+        float s8[8];
+        unpack2<FP16>(a.x, f[i][0], f[i][1]);
+        unpack2<FP16>(a.y, f[i][2], f[i][3]);
+        unpack2<FP16>(a.z, f[i][4], f[i][5]);
+        unpack2<FP16>(a.w, f[i][6], f[i][7]);
+        unpack2<FP16>(b.x, s8[0], s8[1]);
+        unpack2<FP16>(b.y, s8[2], s8[3]);
+        unpack2<FP16>(b.z, s8[4], s8[5]);
+        unpack2<FP16>(b.w, s8[6], s8[7]);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            f[i][k] = f[i][k] * s8[k];
+            amax = fmaxf(amax, fabsf(f[i][k]));
+        }
+    }
+    uint32_t mb = wave_max_u32(__float_as_uint(amax));        // non-negative floats order like their bit patterns
+    __shared__ uint32_t part[kBlock / 64];
+    if ((t & 63) == 0) part[t >> 6] = mb;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; w++) mb = part[w] > mb ? part[w] : mb;
+    amax = __uint_as_float(mb);
+    const float scale = amax / 127.0f;
+    if (t == 0) scale_out[row] = scale;
+    u32x2 *yr = reinterpret_cast<u32x2 *>(y + row * (int64_t)cols);
+    const bool zero = !(amax > 0.0f);
+    const bool scale_safe = scale >= 0x1p-60f && scale <= 0x1p60f;
+    float r = __builtin_amdgcn_rcpf(scale);
+    r = __builtin_fmaf(__builtin_fmaf(-scale, r, 1.0f), r, r);
+#pragma unroll
+    for (int i = 0; i < MAXV; i++) {
+        const int idx = t + i * kBlock;
+        uint32_t q[8];
+        bool ok = scale_safe;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float a = fabsf(f[i][k]);
+            ok = ok && ((a >= 0x1p-60f && a <= 0x1p60f) || a == 0.0f);
+        }
+        if (zero) {
+#pragma unroll
+            for (int k = 0; k < 8; k++) q[k] = 0u;
+        } else if (__builtin_amdgcn_ballot_w64(!ok) == 0) {   // uniform over the wavefront
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                float v = f[i][k] * r;
+                v = __builtin_fmaf(__builtin_fmaf(-scale, v, f[i][k]), r, v);
+                v = __builtin_fmaf(__builtin_fmaf(-scale, v, f[i][k]), r, v);
+                v = __builtin_rintf(v);
+                v = v > 127.0f ? 127.0f : v;
+                v = v < -127.0f ? -127.0f : v;
+                q[k] = (uint32_t)(int)v;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) q[k] = quant_exact(f[i][k], scale);
+        }
+        if (idx < nvec) yr[idx] = u32x2{pack4(q[0], q[1], q[2], q[3]), pack4(q[4], q[5], q[6], q[7])};
+    }
+}
+
 template <int TPR, int ITERS>
 void launch_rows(bool fp16, const uint16_t *x, int8_t *y, float *scale, int64_t rows, int cols, int64_t stride,
                  hipStream_t s)
@@ -331,6 +416,15 @@ extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smoo
         else if (nvec <= 256 * 2) launch_rows<256, 2>(fp16, xp, y, scale, rows, c, x_row_stride, s);
         else if (nvec <= 256 * 4) launch_rows<256, 4>(fp16, xp, y, scale, rows, c, x_row_stride, s);
         else launch_rows<256, 8>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+    } else if (smooth && cols > 0 && (cols & 7) == 0 && (x_row_stride & 7) == 0 && aligned(x, 16) && aligned(smooth, 16) &&
+               aligned(y, 8) && nvec <= kBlock * 4) {
+        const uint16_t *sm = static_cast<const uint16_t *>(smooth);
+        if (fp16)
+            hipLaunchKernelGGL((dq_smooth_rows_kernel<true>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale,
+                               (int)cols, x_row_stride);
+        else
+            hipLaunchKernelGGL((dq_smooth_rows_kernel<false>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale,
+                               (int)cols, x_row_stride);
     } else {
         const uint16_t *sm = static_cast<const uint16_t *>(smooth);
         if (fp16)

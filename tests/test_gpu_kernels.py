@@ -104,6 +104,26 @@ def test_dynamic_quant_smooth(capi, golden):
     assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(y.cpu().numpy(), yg)
 
 
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (33, 8192), (7, 24), (64, 14336), (5, 1000), (3, 8200)])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_dynamic_quant_smooth_shapes(capi, golden, rows, cols, dt):
+    """Smooth scales through the register-resident kernel (cols % 8 == 0, up to 8192) and the two-pass one (wider or odd
+    rows), both input types, with rows that hold zeros, a zero row, tiny and huge values (both division paths of the
+    kernel), bit-exact against the oracle."""
+    g = torch.Generator().manual_seed(rows + cols)
+    x = torch.randn(rows, cols, generator=g) * 3
+    x[0] = 0
+    if rows > 2:
+        x[1, :8] = torch.tensor([1e-30, -1e-30, 0.0, 6e4, -6e4, 1e-7, 0.5, -0.5])     # tiny numerators next to a large maximum
+        x[2] = x[2] * 1e-6
+    x = x.to(dt)
+    sm = (torch.rand(cols, generator=g) * 4 + 0.01).to(dt)
+    y, s = capi.dynamic_quant(x.cuda(), sm.cuda())
+    yg, sg = golden.dynamic_quant(_bits(x), "fp16" if dt == torch.float16 else "bf16", _bits(sm))
+    assert np.array_equal(s.cpu().numpy(), sg)
+    assert np.array_equal(y.cpu().numpy(), yg)
+
+
 # ------------------------------------------------------------------ quant_matmul
 
 QMM_SHAPES = [(1024, 4096, 1024), (256, 512, 352), (64, 4096, 512), (100, 256, 200), (1, 128, 16), (300, 1024, 1000),
