@@ -226,9 +226,11 @@ __global__ __launch_bounds__(kBlock) void dq_generic_kernel(const uint16_t *__re
 // Rows pre-multiplied by smooth scales, cols % 8 == 0 and at most 8192, 16-byte aligned rows and smooth scales: one
 // block per row, the products (arbitrary float32 significands) stay in registers between the maximum and the
 // quantisation.  x / scale uses the row's refined reciprocal with the operation sequence of the compiler's own
-// float32 division (quotient and two residual corrections) whenever every lane of the wavefront has scale and
-// numerators within [2^-60, 2^60] or zero, where that sequence's range scaling and fix-up are the identity; otherwise
-// the wavefront divides the ordinary way.  One scalar branch per eight elements, never both computations.
+// float32 division (quotient and two residual corrections) when the scale lies within [2^-60, 2^60]: that sequence's
+// range scaling and fix-up are then the identity for every numerator that matters.  |x| <= 127 * scale, so nothing
+// overflows; a numerator small enough for a residual to leave the normal range has a quotient below 2^-40, which
+// rounds to zero either way; a NaN numerator becomes code 0 on both paths; an infinite one makes the scale infinite.
+// Rows with a scale outside the range divide the ordinary way.
 template <bool FP16>
 __global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *__restrict__ x,
                                                                 const uint16_t *__restrict__ smooth,
@@ -280,16 +282,10 @@ __global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *
     for (int i = 0; i < MAXV; i++) {
         const int idx = t + i * kBlock;
         uint32_t q[8];
-        bool ok = scale_safe;
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const float a = fabsf(f[i][k]);
-            ok = ok && ((a >= 0x1p-60f && a <= 0x1p60f) || a == 0.0f);
-        }
         if (zero) {
 #pragma unroll
             for (int k = 0; k < 8; k++) q[k] = 0u;
-        } else if (__builtin_amdgcn_ballot_w64(!ok) == 0) {   // uniform over the wavefront
+        } else if (scale_safe) {                              // the same for the whole row
 #pragma unroll
             for (int k = 0; k < 8; k++) {
                 float v = f[i][k] * r;

@@ -21,14 +21,29 @@ __device__ __forceinline__ float to_f32(uint16_t h)
     else return bf16_1(h);
 }
 
-__device__ __forceinline__ uint32_t quant1(float x, float scale, float offset)
+__device__ __forceinline__ uint32_t finish1(float q, float offset)
 {
-    float q = x / scale;
     q = q + offset;
     q = __builtin_rintf(q);
     q = q > 127.0f ? 127.0f : q;
     q = q < -128.0f ? -128.0f : q;
     return (uint32_t)(int)q & 0xffu;
+}
+
+__device__ __forceinline__ uint32_t quant1(float x, float scale, float offset) { return finish1(x / scale, offset); }
+
+// x / scale through the row's refined reciprocal `r`: the operation sequence of the compiler's own float32 division
+// (quotient, two residual corrections with fused multiply-adds) without its range scaling and special-case fix-up.
+// Those are the identity when the scale lies within [2^-60, 2^60] and no element of the row exceeds 2^60 (nothing
+// overflows; a numerator small enough for a residual to leave the normal range has a quotient below 2^-40, which the
+// offset absorbs or which rounds to zero either way; NaN becomes code 0 on both paths).  Rows outside that range
+// divide the ordinary way; the choice is the same for a whole row.
+__device__ __forceinline__ uint32_t quant1_rcp(float x, float scale, float r, float offset)
+{
+    float q = x * r;
+    q = __builtin_fmaf(__builtin_fmaf(-scale, q, x), r, q);
+    q = __builtin_fmaf(__builtin_fmaf(-scale, q, x), r, q);
+    return finish1(q, offset);
 }
 
 // VEC: cols % 8 == 0, rows (and smooth) 16-byte aligned, y rows 8-byte aligned
@@ -90,6 +105,10 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
         const bool flat = !(mx > mn);                     // all elements equal (or no finite ordering): zeros
         if (flat) scale = 0.0f, offset = 0.0f;
         if (t == 0) scale_out[row] = scale, offset_out[row] = offset;
+        float rcp = __builtin_amdgcn_rcpf(scale);
+        rcp = __builtin_fmaf(__builtin_fmaf(-scale, rcp, 1.0f), rcp, rcp);
+        const bool fast = __builtin_amdgcn_readfirstlane(
+                              (int)(scale >= 0x1p-60f && scale <= 0x1p60f && fmaxf(fabsf(mx), fabsf(mn)) <= 0x1p60f)) != 0;
         if constexpr (VEC) {
             for (int v = t, it = 0; v < cols / 8; v += 256, it++) {
                 u32x4 a;
@@ -98,11 +117,21 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
                 u32x4 s = u32x4{0, 0, 0, 0};
                 if (smooth) s = reinterpret_cast<const u32x4 *>(smooth)[v];
                 uint32_t q[8];
+                float f8[8];
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
-                    float f = to_f32<FP16>((uint16_t)(a[i / 2] >> (16 * (i & 1))));
-                    if (smooth) f = f * to_f32<FP16>((uint16_t)(s[i / 2] >> (16 * (i & 1))));
-                    q[i] = flat ? 0u : quant1(f, scale, offset);
+                    f8[i] = to_f32<FP16>((uint16_t)(a[i / 2] >> (16 * (i & 1))));
+                    if (smooth) f8[i] = f8[i] * to_f32<FP16>((uint16_t)(s[i / 2] >> (16 * (i & 1))));
+                }
+                if (flat) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) q[i] = 0u;
+                } else if (fast) {                            // one branch: never both divisions
+#pragma unroll
+                    for (int i = 0; i < 8; i++) q[i] = quant1_rcp(f8[i], scale, rcp, offset);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) q[i] = quant1(f8[i], scale, offset);
                 }
                 u32x2 o;
                 o.x = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
@@ -113,7 +142,7 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
             for (int j = t; j < cols; j += 256) {
                 float f = to_f32<FP16>(xr[j]);
                 if (smooth) f = f * to_f32<FP16>(smooth[j]);
-                yr[j] = (int8_t)(flat ? 0u : quant1(f, scale, offset));
+                yr[j] = (int8_t)(flat ? 0u : fast ? quant1_rcp(f, scale, rcp, offset) : quant1(f, scale, offset));
             }
         }
     }

@@ -47,9 +47,10 @@ __device__ __forceinline__ float quant1(float x, float sc, float zp, float qmin,
 // Division by a channel's scale with the reciprocal formed once per channel: the operation sequence of the compiler's
 // own float32 division (reciprocal refined once, quotient, two residual corrections with fused multiply-adds) without
 // its range scaling and special-case fix-up, which are the identity while no intermediate leaves the normal range.
-// Used for a group of elements only when every lane of the wavefront has scale and numerators within [2^-60, 2^60]
-// (zero numerators too); otherwise the whole wavefront takes the ordinary division, so there is one scalar branch
-// per group and never both computations.
+// Used for a group of elements only when every lane of the wavefront has its scales within [2^-60, 2^60] and
+// numerators of at most 2^60 (so nothing overflows; a numerator small enough for a residual to leave the normal
+// range has a quotient below 2^-40, which the zero point absorbs or which rounds to zero either way); otherwise the
+// whole wavefront takes the ordinary division, so there is one scalar branch per group and never both computations.
 __device__ __forceinline__ bool safe_range(float v)
 {
     const float a = __builtin_fabsf(v);
@@ -76,7 +77,7 @@ __device__ __forceinline__ void quant8(const float (&x)[8], const float (&sc)[8]
     if constexpr (DIV) {
         bool ok = scales_safe;
 #pragma unroll
-        for (int i = 0; i < 8; i++) ok = ok && (safe_range(x[i]) || x[i] == 0.0f);
+        for (int i = 0; i < 8; i++) ok = ok && __builtin_fabsf(x[i]) <= 0x1p60f;   // false for NaN and infinity too
         if (__builtin_amdgcn_ballot_w64(!ok) == 0) {          // uniform over the wavefront
 #pragma unroll
             for (int i = 0; i < 8; i++) q[i] = finish1(div_by_rcp(x[i], sc[i], rc[i]), zp[i], qmin, qmax);

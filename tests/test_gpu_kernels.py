@@ -809,6 +809,25 @@ def test_dynamic_quant_asymmetric(capi, golden, rows, cols, f16):
     assert not y[0].any() or sm is not None
 
 
+def test_dynamic_quant_asymmetric_extreme_rows(capi, golden):
+    """Rows that leave the range where the kernel divides through the row's reciprocal (huge elements, a tiny spread, tiny
+    elements next to a normal spread) and rows inside it: bit-identical to the oracle either way."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(12, 512, generator=g) * 2
+    x[1] = x[1] * 1e30                                              # elements above 2^60
+    x[2] = x[2] * 1e-30                                             # scale below 2^-60
+    x[3, :6] = torch.tensor([1e-30, -1e-30, 1e-38, 0.0, -0.0, 3e-20])   # tiny numerators, ordinary scale
+    x[4] = 1000.0 + x[4] * 1e-3                                     # small spread around a large value
+    x[5, 0] = 3e38
+    x = x.to(torch.bfloat16)
+    with np.errstate(all="ignore"):
+        wy, ws, wo = golden.dynamic_quant_asymmetric(_bits(x), "bf16", None)
+    y, s, o = capi.dynamic_quant_asymmetric(x.cuda(), None)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+    assert np.array_equal(o.cpu().numpy().view(np.uint32), wo.view(np.uint32))
+    assert np.array_equal(y.cpu().numpy(), wy)
+
+
 # ------------------------------------------------------------------ error paths (host side, no kernel runs)
 
 @pytest.mark.parametrize("rows,half", [(64, 14336), (2048, 14336), (33, 512), (5, 100), (3, 16384 + 8), (7, 24)])
