@@ -420,8 +420,8 @@ def test_quant_matmul_a4w4_operator(pa, golden):
 def test_graph_replays_match_eager(pa):
     """The operators launched from a captured HIP graph: every replay (with eager launches of the same operators in
     between, which share the per-stream workspaces and their arrival counters) must reproduce the eager bits.  Covers
-    the K-split exchanges of both matmuls, the tiled weight-only kernel with its row-sum pre-kernel and the fused
-    SwiGLU quantisation."""
+    the K-split exchanges of both matmuls (bf16 and re-quantised int8 output), the per-call weight transpose, the tiled
+    weight-only kernel with its row-sum pre-kernel, the fused SwiGLU quantisation, smooth scales and npu_quantize."""
     g = torch.Generator().manual_seed(11)
     d = workloads.mlp_inputs(seed=3, M=64, hidden=1024, inter=4096)
     x = d["x"].cuda()
@@ -431,6 +431,11 @@ def test_graph_replays_match_eager(pa):
     a4 = [d4[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset")]
     a4b = [d4b[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset")]
     act = torch.randn(64, 8192, generator=g).to(torch.bfloat16).cuda()
+    qp = pa.npu_trans_quant_param((torch.rand(1024, generator=g) * 1e-4 + 1e-4).cuda(), torch.randint(-8, 8, (1024,), generator=g).float().cuda())
+    bi = torch.randint(-1000, 1000, (1024,), generator=g, dtype=torch.int32).cuda()
+    wkn = wd.contiguous()                                                          # the same weight stored [K, N]
+    sm = (torch.rand(1024, generator=g) + 0.5).to(torch.bfloat16).cuda()
+    zs, zz = (torch.rand(1024, generator=g) * 0.05 + 0.01).cuda(), torch.randint(-8, 8, (1024,), generator=g, dtype=torch.int32).cuda()
 
     def run():
         q, s = pa.npu_swiglu_quant(act, activate_left=True, quant_mode=1)          # [64, 4096] int8
@@ -438,7 +443,11 @@ def test_graph_replays_match_eager(pa):
         o2 = pa.npu_weight_quant_batchmatmul(*a4, None, None, None, 128)            # streaming kernel, K split
         o3 = pa.npu_weight_quant_batchmatmul(*a4b, None, None, None, 128)           # row sums + tiled kernel, K split
         q1, s1 = pa.npu_dynamic_quant(x)
-        return q, s, o1, o2, o3, q1, s1
+        o4 = pa.npu_quant_matmul(q, wd, qp, bias=bi, output_dtype=torch.int8)      # re-quantised output, K split
+        o5 = pa.npu_quant_matmul(q, wkn, sd, pertoken_scale=s, output_dtype=torch.bfloat16)   # [K,N] weight: transposed per call
+        q2, s2 = pa.npu_dynamic_quant(x, smooth_scales=sm)
+        q3 = pa.npu_quantize(x, zs, zz, torch.qint8, -1)
+        return q, s, o1, o2, o3, q1, s1, o4, o5, q2, s2, q3
 
     want = [t.clone() for t in run()]
     torch.cuda.synchronize()
