@@ -219,6 +219,15 @@ int mi355_swiglu_quant(const void *x_bf16, int activate_left, int8_t *y, float *
                        int64_t rows, int64_t half, int64_t x_row_stride, void *stream);
 
 /*
+ * The same with smooth scales (the smooth_scales argument of torch_npu.npu_swiglu_quant, named in
+ * docs/zh/release_notes.md:303 only): y, scale = dynamic_quant(swiglu(x), smooth) as mi355_dynamic_quant defines it,
+ * i.e. the bf16 SwiGLU value times smooth[j] in float32 before the row maximum and the quantisation.
+ *   smooth_bf16  bf16 [half]
+ */
+int mi355_swiglu_quant_smooth(const void *x_bf16, int activate_left, const void *smooth_bf16, int8_t *y, float *scale,
+                              int64_t rows, int64_t half, int64_t x_row_stride, void *stream);
+
+/*
  * npu_anti_quant: the standalone antiquantisation out = cast((float(x) + offset) * scale).
  * Replaces the aclnn AscendAntiQuant call behind torch_npu.npu_anti_quant (signature test/torch_npu_schema.json:2117-2119,
  * wrapper torch_npu/onnx/wrapper_onnx_ops.py:824-828; CPU golden test/custom_ops/test_npu_anti_quant.py:29-42, int4

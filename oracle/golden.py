@@ -324,14 +324,14 @@ def swiglu(x_u16: np.ndarray) -> np.ndarray:
     return out
 
 
-def swiglu_quant(x_u16: np.ndarray, activate_left: bool = True):
-    """dynamic_quant(swiglu(x)): the composition of the two restatements above (no arithmetic of its own).
+def swiglu_quant(x_u16: np.ndarray, activate_left: bool = True, smooth_u16: np.ndarray | None = None):
+    """dynamic_quant(swiglu(x), smooth): the composition of the two restatements above (no arithmetic of its own).
     activate_left=False activates the right half: silu(x[:, half:]) * x[:, :half]."""
     x = _c(x_u16, np.uint16)
     half = x.shape[1] // 2
     if not activate_left:
         x = np.concatenate([x[:, half:], x[:, :half]], axis=1)
-    return dynamic_quant(swiglu(x))
+    return dynamic_quant(swiglu(x), "bf16", smooth_u16)
 
 
 # ------------------------------------------------------ bit-pattern helpers

@@ -18,7 +18,7 @@ EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quan
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
-           "mi355_trans_quant_param", "mi355_quant_matmul_qparam")
+           "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth")
 
 _lib = None
 
@@ -47,6 +47,7 @@ def lib() -> ctypes.CDLL:
                                                 i64, i64, vp, sz, vp]
         L.mi355_swiglu.argtypes = [vp, vp, i64, i64, i64, vp]
         L.mi355_swiglu_quant.argtypes = [vp, i32, vp, vp, i64, i64, i64, vp]
+        L.mi355_swiglu_quant_smooth.argtypes = [vp, i32, vp, vp, vp, i64, i64, i64, vp]
         L.mi355_anti_quant.argtypes = [vp, i32, vp, i64, vp, i64, vp, i32, i64, i64, i64, i64, vp]
         L.mi355_unpack_int4.argtypes = [vp, vp, i64, i64, i64, i64, vp]
         L.mi355_dynamic_quant_asymmetric.argtypes = [vp, i32, vp, vp, vp, vp, i64, i64, i64, vp]
@@ -193,12 +194,16 @@ def swiglu(x):
     return out
 
 
-def swiglu_quant(x, activate_left: bool = True):
-    """x bf16 [rows, 2*half] -> (int8 [rows, half], float32 [rows]) = dynamic_quant(swiglu(x))."""
-    _need_gpu(x)
+def swiglu_quant(x, activate_left: bool = True, smooth=None):
+    """x bf16 [rows, 2*half] -> (int8 [rows, half], float32 [rows]) = dynamic_quant(swiglu(x), smooth)."""
+    _need_gpu(x, smooth)
     rows, two = x.shape
     y = torch.empty((rows, two // 2), dtype=torch.int8, device=x.device)
     scale = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    if smooth is not None:
+        _check(lib().mi355_swiglu_quant_smooth(_ptr(x), 1 if activate_left else 0, _ptr(smooth), _ptr(y), _ptr(scale), rows,
+                                               two // 2, x.stride(0), _stream()), "mi355_swiglu_quant_smooth")
+        return y, scale
     _check(lib().mi355_swiglu_quant(_ptr(x), 1 if activate_left else 0, _ptr(y), _ptr(scale), rows, two // 2, x.stride(0),
                                     _stream()), "mi355_swiglu_quant")
     return y, scale

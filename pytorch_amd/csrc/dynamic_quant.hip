@@ -231,13 +231,16 @@ __global__ __launch_bounds__(kBlock) void dq_generic_kernel(const uint16_t *__re
 // overflows; a numerator small enough for a residual to leave the normal range has a quotient below 2^-40, which
 // rounds to zero either way; a NaN numerator becomes code 0 on both paths; an infinite one makes the scale infinite.
 // Rows with a scale outside the range divide the ordinary way.
-template <bool FP16>
+// SWIGLU (bf16): the row holds two halves of `cols` elements and the value that is smoothed and quantised is
+// bf16(silu(act half)) * other half, rounded to bf16 like the stand-alone SwiGLU kernel; act_offset / mul_offset are
+// the positions of the two halves in 16-byte vectors.
+template <bool FP16, bool SWIGLU = false, int MAXV = 4>
 __global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *__restrict__ x,
                                                                 const uint16_t *__restrict__ smooth,
                                                                 int8_t *__restrict__ y, float *__restrict__ scale_out,
-                                                                int cols, int64_t row_stride)
+                                                                int cols, int64_t row_stride, int act_offset = 0,
+                                                                int mul_offset = 0)
 {
-    constexpr int MAXV = 4;
     const int64_t row = blockIdx.x;
     const int t = threadIdx.x, nvec = cols >> 3;
     const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + row * row_stride);
@@ -248,7 +251,16 @@ __global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *
     for (int i = 0; i < MAXV; i++) {
         const int idx = t + i * kBlock;
         u32x4 a{0, 0, 0, 0}, b{0, 0, 0, 0};
-        if (idx < nvec) a = __builtin_nontemporal_load(xr + idx), b = sr[idx];
+        if (idx < nvec) {
+            if constexpr (SWIGLU) {
+                const u32x4 g = __builtin_nontemporal_load(xr + act_offset + idx);
+                const u32x4 m = __builtin_nontemporal_load(xr + mul_offset + idx);
+                a = u32x4{swiglu2(g.x, m.x), swiglu2(g.y, m.y), swiglu2(g.z, m.z), swiglu2(g.w, m.w)};
+            } else {
+                a = __builtin_nontemporal_load(xr + idx);
+            }
+            b = sr[idx];
+        }
         float s8[8];
         unpack2<FP16>(a.x, f[i][0], f[i][1]);
         unpack2<FP16>(a.y, f[i][2], f[i][3]);
@@ -331,13 +343,15 @@ void launch_swiglu_rows(const uint16_t *x, int8_t *y, float *scale, int64_t rows
 // Any shape and alignment: one block per row, SwiGLU recomputed in the second pass.
 __global__ __launch_bounds__(kBlock) void swiglu_dq_generic_kernel(const uint16_t *__restrict__ x, int8_t *__restrict__ y,
                                                                   float *__restrict__ scale_out, int64_t half,
-                                                                  int64_t row_stride, int64_t act_off, int64_t mul_off)
+                                                                  int64_t row_stride, int64_t act_off, int64_t mul_off,
+                                                                  const uint16_t *__restrict__ smooth = nullptr)
 {
     const int64_t row = blockIdx.x;
     const uint16_t *xr = x + row * row_stride;
     auto value = [&](int64_t j) {
         const float sl = bf16_1(f32_to_bf16(silu_f32(bf16_1(xr[act_off + j]))));
-        return bf16_1(f32_to_bf16(sl * bf16_1(xr[mul_off + j])));
+        const float v = bf16_1(f32_to_bf16(sl * bf16_1(xr[mul_off + j])));
+        return smooth ? v * bf16_1(smooth[j]) : v;
     };
     float amax = 0.0f;
     for (int64_t j = threadIdx.x; j < half; j += kBlock) amax = fmaxf(amax, fabsf(value(j)));
@@ -357,10 +371,11 @@ __global__ __launch_bounds__(kBlock) void swiglu_dq_generic_kernel(const uint16_
 } // namespace
 } // namespace mi355
 
-extern "C" int mi355_swiglu_quant(const void *x_bf16, int activate_left, int8_t *y, float *scale, int64_t rows, int64_t half,
-                                  int64_t x_row_stride, void *stream)
+namespace mi355 {
+namespace {
+int run_swiglu_quant(const void *x_bf16, int activate_left, const void *smooth, int8_t *y, float *scale, int64_t rows,
+                     int64_t half, int64_t x_row_stride, void *stream)
 {
-    using namespace mi355;
     if (rows < 0 || half < 0) return MI355_ERR_BAD_ARGUMENT;
     if (rows == 0) return MI355_OK;
     if (!scale) return MI355_ERR_BAD_ARGUMENT;
@@ -372,6 +387,23 @@ extern "C" int mi355_swiglu_quant(const void *x_bf16, int activate_left, int8_t 
     const int64_t nvec = half >> 3;
     const bool vec_ok = half > 0 && (half & 7) == 0 && (x_row_stride & 7) == 0 && aligned(xp, 16) && aligned(y, 8) &&
                         nvec <= kBlock * 8;
+    const uint16_t *sm = static_cast<const uint16_t *>(smooth);
+    if (sm) {
+        if (!aligned(sm, 2)) return MI355_ERR_ALIGNMENT;
+        if (vec_ok && aligned(sm, 16)) {
+            const int c = (int)half, ao = (int)(act >> 3), mo = (int)(mul >> 3);
+            if (nvec <= kBlock * 4)
+                hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 4>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y,
+                                   scale, c, x_row_stride, ao, mo);
+            else
+                hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 8>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y,
+                                   scale, c, x_row_stride, ao, mo);
+        } else {
+            hipLaunchKernelGGL(swiglu_dq_generic_kernel, dim3((unsigned)rows), dim3(kBlock), 0, s, xp, y, scale, half,
+                               x_row_stride, act, mul, sm);
+        }
+        return check_launch();
+    }
     if (vec_ok) {
         const int c = (int)half, ao = (int)(act >> 3), mo = (int)(mul >> 3);
         if (nvec <= 64 * 1) launch_swiglu_rows<64, 1>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
@@ -385,6 +417,22 @@ extern "C" int mi355_swiglu_quant(const void *x_bf16, int activate_left, int8_t 
                            act, mul);
     }
     return check_launch();
+}
+
+} // namespace
+} // namespace mi355
+
+extern "C" int mi355_swiglu_quant(const void *x_bf16, int activate_left, int8_t *y, float *scale, int64_t rows, int64_t half,
+                                  int64_t x_row_stride, void *stream)
+{
+    return mi355::run_swiglu_quant(x_bf16, activate_left, nullptr, y, scale, rows, half, x_row_stride, stream);
+}
+
+extern "C" int mi355_swiglu_quant_smooth(const void *x_bf16, int activate_left, const void *smooth_bf16, int8_t *y, float *scale,
+                                         int64_t rows, int64_t half, int64_t x_row_stride, void *stream)
+{
+    if (!smooth_bf16 && rows > 0 && half > 0) return MI355_ERR_BAD_ARGUMENT;
+    return mi355::run_swiglu_quant(x_bf16, activate_left, smooth_bf16, y, scale, rows, half, x_row_stride, stream);
 }
 
 extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth, int8_t *y, float *scale,

@@ -588,14 +588,19 @@ Tensor swiglu_hip(const Tensor &input, int64_t dim)
 
 // The operator is only named in the reference tree (docs/zh/release_notes.md:303); the argument list follows the
 // vendor's published Python signature.  Implemented: dynamic per-token quantisation (quant_mode = 1) of the SwiGLU
-// of the last dimension, without smooth scales, offsets or expert groups.
+// of the last dimension, optionally with one set of smooth scales; no static offsets, no expert groups.
 void swiglu_quant_check(const Tensor &x, const optional<Tensor> &smooth_scales, const optional<Tensor> &offsets,
                         const optional<Tensor> &group_index, int64_t quant_mode, int64_t group_list_type,
                         optional<at::ScalarType> dst_type)
 {
     TORCH_CHECK(x.scalar_type() == at::kBFloat16, "npu_swiglu_quant: only bfloat16 input is supported, got ", x.scalar_type());
     TORCH_CHECK(x.dim() >= 1 && x.size(-1) % 2 == 0, "npu_swiglu_quant: the last dimension must be even");
-    TORCH_CHECK(!opt(smooth_scales), "npu_swiglu_quant: smooth_scales is not supported");
+    if (const Tensor *sm = opt(smooth_scales)) {
+        TORCH_CHECK(sm->scalar_type() == at::kBFloat16, "npu_swiglu_quant: smooth_scales must be bfloat16 like x, got ",
+                    sm->scalar_type());
+        TORCH_CHECK(sm->dim() == 1 && sm->size(0) == x.size(-1) / 2, "npu_swiglu_quant: smooth_scales must have shape [",
+                    x.size(-1) / 2, "] (one per output column; per-expert scales are not supported)");
+    }
     TORCH_CHECK(!opt(offsets), "npu_swiglu_quant: offsets (static quantisation) is not supported");
     TORCH_CHECK(!opt(group_index), "npu_swiglu_quant: group_index is not supported");
     TORCH_CHECK(quant_mode == 1, "npu_swiglu_quant: only quant_mode=1 (dynamic per-token quantisation) is supported, got ",
@@ -629,6 +634,7 @@ std::tuple<Tensor, Tensor> swiglu_quant_hip(const Tensor &x, const optional<Tens
                                             optional<at::ScalarType> dst_type)
 {
     swiglu_quant_check(x, smooth_scales, offsets, group_index, quant_mode, group_list_type, dst_type);
+    check_same_device("npu_swiglu_quant", {&x, opt(smooth_scales)});
     c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
     auto [y, scale] = swiglu_quant_alloc(x);
     const int64_t half = x.size(-1) / 2;
@@ -643,6 +649,13 @@ std::tuple<Tensor, Tensor> swiglu_quant_hip(const Tensor &x, const optional<Tens
         row_stride = xin.stride(0);
     } else if (!xin.is_contiguous()) {
         xin = xin.contiguous();
+    }
+    if (const Tensor *smp = opt(smooth_scales)) {
+        Tensor sm = smp->contiguous();
+        check_status(mi355_swiglu_quant_smooth(xin.data_ptr(), activate_left ? 1 : 0, sm.data_ptr(), y.data_ptr<int8_t>(),
+                                               scale.data_ptr<float>(), rows, half, row_stride, stream_of(x)),
+                     "npu_swiglu_quant");
+        return {y, scale};
     }
     check_status(mi355_swiglu_quant(xin.data_ptr(), activate_left ? 1 : 0, y.data_ptr<int8_t>(), scale.data_ptr<float>(), rows,
                                     half, row_stride, stream_of(x)),

@@ -73,4 +73,4 @@ extern "C" const char *mi355_status_string(int status)
     }
 }
 
-extern "C" int mi355_quant_abi_version(void) { return 2200; }
+extern "C" int mi355_quant_abi_version(void) { return 2300; }

@@ -830,6 +830,24 @@ def test_dynamic_quant_asymmetric_extreme_rows(capi, golden):
 
 # ------------------------------------------------------------------ error paths (host side, no kernel runs)
 
+@pytest.mark.parametrize("rows,half", [(64, 14336), (512, 4096), (33, 512), (5, 100), (3, 16384 + 8), (7, 24)])
+@pytest.mark.parametrize("left", [True, False])
+def test_swiglu_quant_with_smooth_scales(capi, golden, rows, half, left):
+    """Fused SwiGLU + smooth scales + dynamic quantisation equals the oracle's composition bit for bit: the
+    register-resident kernel (four and eight vectors per thread), the two-pass kernel (odd or very wide rows), both
+    orientations, and through the operator."""
+    import pytorch_amd as pa
+    g = torch.Generator().manual_seed(rows + half)
+    x = (torch.randn(rows, 2 * half, generator=g) * 2).to(torch.bfloat16)
+    x[0] = 0
+    sm = (torch.rand(half, generator=g) * 3 + 0.05).to(torch.bfloat16)
+    wy, ws = golden.swiglu_quant(_bits(x), left, _bits(sm))
+    y, s = capi.swiglu_quant(x.cuda(), left, sm.cuda())
+    assert np.array_equal(s.cpu().numpy(), ws) and np.array_equal(y.cpu().numpy(), wy)
+    y2, s2 = pa.npu_swiglu_quant(x.cuda(), smooth_scales=sm.cuda(), activate_left=left, quant_mode=1)
+    assert torch.equal(y2, y) and torch.equal(s2, s)
+
+
 @pytest.mark.parametrize("rows,half", [(64, 14336), (2048, 14336), (33, 512), (5, 100), (3, 16384 + 8), (7, 24)])
 @pytest.mark.parametrize("left", [True, False])
 def test_swiglu_quant_equals_composition(capi, golden, rows, half, left):

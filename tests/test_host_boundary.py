@@ -18,7 +18,7 @@ def test_c_abi_exports_every_declared_symbol():
     declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", header))
     assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant", "mi355_anti_quant",
             "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize", "mi355_trans_quant_param",
-            "mi355_quant_matmul_qparam"} <= declared
+            "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth"} <= declared
     lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_amd", "csrc", "libmi355_quant.so"))
     for name in declared:
         assert hasattr(lib, name), name
@@ -193,8 +193,12 @@ def test_meta_swiglu_quant(pa):
     assert y.shape == (2, 3, 4) and s.shape == (2, 3)
     with pytest.raises(RuntimeError, match="quant_mode"):
         pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16))                      # static quantisation is not built
-    with pytest.raises(RuntimeError, match="smooth_scales"):
-        pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(4, dtype=torch.bfloat16), quant_mode=1)
+    y, s = pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(4, dtype=torch.bfloat16), quant_mode=1)
+    assert y.shape == (4, 4) and s.shape == (4,)
+    with pytest.raises(RuntimeError, match="smooth_scales must have shape"):       # per-expert scales are not built
+        pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(2, 4, dtype=torch.bfloat16), quant_mode=1)
+    with pytest.raises(RuntimeError, match="smooth_scales must be bfloat16"):
+        pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(4, dtype=torch.float32), quant_mode=1)
 
 
 def test_meta_anti_quant(pa):
