@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void dq_generic_kernel(const uint16_t *__re
     }
 }
 
-// Rows pre-multiplied by smooth scales, cols % 8 == 0 and at most 8192, 16-byte aligned rows and smooth scales: one
+// Rows pre-multiplied by smooth scales, cols % 8 == 0 and at most 2048 * MAXV, 16-byte aligned rows and smooth scales: one
 // block per row, the products (arbitrary float32 significands) stay in registers between the maximum and the
 // quantisation.  x / scale uses the row's refined reciprocal with the operation sequence of the compiler's own
 // float32 division (quotient and two residual corrections) when the scale lies within [2^-60, 2^60]: that sequence's
@@ -461,14 +461,19 @@ extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smoo
         else if (nvec <= 256 * 4) launch_rows<256, 4>(fp16, xp, y, scale, rows, c, x_row_stride, s);
         else launch_rows<256, 8>(fp16, xp, y, scale, rows, c, x_row_stride, s);
     } else if (smooth && cols > 0 && (cols & 7) == 0 && (x_row_stride & 7) == 0 && aligned(x, 16) && aligned(smooth, 16) &&
-               aligned(y, 8) && nvec <= kBlock * 4) {
+               aligned(y, 8) && nvec <= kBlock * 8) {
         const uint16_t *sm = static_cast<const uint16_t *>(smooth);
-        if (fp16)
-            hipLaunchKernelGGL((dq_smooth_rows_kernel<true>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale,
-                               (int)cols, x_row_stride);
-        else
-            hipLaunchKernelGGL((dq_smooth_rows_kernel<false>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale,
-                               (int)cols, x_row_stride);
+#define MI355_DQS_LAUNCH(F, V) \
+    hipLaunchKernelGGL((dq_smooth_rows_kernel<F, false, V>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale, (int)cols, \
+                       x_row_stride)
+        if (nvec <= kBlock * 4) {
+            if (fp16) MI355_DQS_LAUNCH(true, 4);
+            else MI355_DQS_LAUNCH(false, 4);
+        } else {
+            if (fp16) MI355_DQS_LAUNCH(true, 8);
+            else MI355_DQS_LAUNCH(false, 8);
+        }
+#undef MI355_DQS_LAUNCH
     } else {
         const uint16_t *sm = static_cast<const uint16_t *>(smooth);
         if (fp16)
