@@ -61,15 +61,35 @@ class _QuantLinearBase(nn.Module):
             raise ValueError("output_dtype should be torch.int8, torch.float16 or torch.bfloat16, "
                              f"but now it is {self.output_dtype}.")
 
+    def prepare_(self) -> "_QuantLinearBase":
+        """One-time widening for inference (optional, A4W4 only): a weight stored as int32 words of eight int4 values is
+        widened to int8 ``[out_features, in_features]`` once, so that a forward pass widens only the activations before
+        the int8 GEMM instead of the weight as well.  The parameter the module exposes (and its state_dict) stays as it
+        is; the widened copy is a plain attribute that costs twice the packed weight's size and must be rebuilt by
+        calling this again after the weight changes."""
+        self._prepared_i8 = None
+        if self.weight.dtype == torch.int32:
+            from ... import _capi
+            self._prepared_i8 = _capi.unpack_int4(self.weight.data)
+        return self
+
     def forward(self, linear_quant_input: torch.Tensor) -> torch.Tensor:
         self._check_dtypes(linear_quant_input)
+        weight = self.weight
+        prepared = getattr(self, "_prepared_i8", None)
+        if prepared is not None and linear_quant_input.dtype == torch.int32:
+            from ... import _capi
+            x = linear_quant_input
+            words = x.shape[-1]
+            linear_quant_input = _capi.unpack_int4(x.reshape(-1, words).contiguous()).view(*x.shape[:-1], words * 8)
+            weight = prepared
         scale = self.scale
         # a float32 scale is packed with npu_trans_quant_param when there is no pertoken_scale and the output is int8
         # (output_dtype None) or float16 (linear_quant.py:104-108)
         if (self.pertoken_scale is None and scale.dtype == torch.float32
                 and self.output_dtype not in (torch.bfloat16, torch.int32)):
             scale = torch.ops.npu.npu_trans_quant_param(scale, self.offset)
-        return torch.ops.npu.npu_quant_matmul(linear_quant_input, self.weight.transpose(-2, -1), scale,
+        return torch.ops.npu.npu_quant_matmul(linear_quant_input, weight.transpose(-2, -1), scale,
                                               offset=self.offset, pertoken_scale=self.pertoken_scale, bias=self.bias,
                                               output_dtype=self.output_dtype)
 

@@ -119,6 +119,29 @@ def test_linear_quant_module_equals_operator(pa):
         assert torch.equal(got, want)
 
 
+def test_linear_quant_a4w4_prepare(pa):
+    """LinearQuant with an int4 weight (int32 words, linear_quant.py:40-50): prepare_() widens the weight once; the
+    forward pass then gives the same bits as the unprepared module, for 2-D and batched int32 activations."""
+    from pytorch_amd.contrib.module import LinearQuant
+    g = torch.Generator().manual_seed(8)
+    rnd = lambda *sh: torch.randint(-2 ** 31, 2 ** 31 - 1, sh, generator=g, dtype=torch.int64).to(torch.int32)  # noqa: E731
+    m = LinearQuant(512, 256, bias=True, pertoken_scale=True, output_dtype=torch.bfloat16).cuda()
+    m.weight.data = rnd(256, 64).cuda()
+    m.scale.data = (torch.rand(256, generator=g) * 1e-2).cuda()
+    m.bias.data = torch.randint(-100, 100, (256,), generator=g, dtype=torch.int32).cuda()
+    x = rnd(48, 64).cuda()
+    m.pertoken_scale.data = (torch.rand(48, generator=g) * 1e-2).cuda()
+    want = m(x)
+    m.prepare_()
+    assert m._prepared_i8.dtype == torch.int8 and m._prepared_i8.shape == (256, 512)
+    assert torch.equal(m(x), want)
+    m2 = LinearQuant(512, 256, bias=False, output_dtype=torch.float16).cuda()
+    m2.weight.data, m2.scale.data = m.weight.data, m.scale.data
+    xb = rnd(2, 3, 64).cuda()
+    want = m2(xb)
+    assert torch.equal(m2.prepare_()(xb), want) and want.shape == (2, 3, 256)
+
+
 def test_quant_matmul_int8_output_operator_and_module(pa, golden):
     """npu_quant_matmul with output_dtype None / int8 (test/test_fake_tensor.py:1886-1895): a float32 scale is packed
     like npu_trans_quant_param packs it, an int64 scale is taken as packed; LinearQuant's default configuration
