@@ -278,6 +278,15 @@ int mi355_quantize(const void *x, int in_dtype, const float *scale, int64_t scal
  */
 int mi355_unpack_int4(const void *x, int8_t *out, int64_t rows, int64_t cols, int64_t ldx, int64_t ldo, void *stream);
 
+/*
+ * Planner knobs for tuning and for tests that must force a particular plan (a given split of K, a tile shape).
+ * No counterpart in the reference: aclnn chooses its tiling inside the closed kernels.  `name` is one of the
+ * names listed in pytorch_amd/csrc/tuning.hip (e.g. "MI355_WQ_SPLIT"); value 0 restores the automatic choice.
+ * A knob's initial value is read once, at load time, from the environment variable of the same name; no launch
+ * reads the environment.  Returns MI355_ERR_BAD_ARGUMENT for an unknown name.  Process-wide, not thread-scoped.
+ */
+int mi355_set_tuning(const char *name, int value);
+
 #ifdef __cplusplus
 }
 #endif

@@ -18,7 +18,7 @@ EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quan
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
-           "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth")
+           "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth", "mi355_set_tuning")
 
 _lib = None
 
@@ -54,8 +54,14 @@ def lib() -> ctypes.CDLL:
         L.mi355_trans_quant_param.argtypes = [vp, i64, vp, i64, vp, i64, vp]
         L.mi355_quant_matmul_qparam.argtypes = [vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
         L.mi355_quantize.argtypes = [vp, i32, vp, i64, vp, i32, i64, vp, i32, i64, i64, i64, i32, vp]
+        L.mi355_set_tuning.argtypes = [ctypes.c_char_p, i32]
         _lib = L
     return _lib
+
+
+def set_tuning(name: str, value: int) -> None:
+    """Set a planner knob (0 = automatic); the knob names are those of ``csrc/tuning.hip``."""
+    _check(lib().mi355_set_tuning(name.encode(), int(value)), "mi355_set_tuning")
 
 
 def _check(status: int, what: str) -> None:
@@ -143,14 +149,20 @@ def quant_matmul_qparam(x1, x2, qparam, bias=None, out_dtype=torch.int8, workspa
 
 
 _wq_workspaces = {}
+_wq_retired = []        # superseded workspaces stay alive: a captured graph may still hold their address
 
 
 def _wq_workspace(device, nbytes: int):
     """Zero-initialised workspace reused across calls on one stream: the kernel needs its counters
-    to start at zero and leaves them at zero."""
+    to start at zero and leaves them at zero.  Never allocated (or filled) while the stream is capturing."""
     key = (device.index, torch.cuda.current_stream().cuda_stream)
     ws = _wq_workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise Mi355Error(f"a {nbytes}-byte zeroed workspace cannot be allocated during stream capture: "
+                             "call once with this shape on this stream before the capture begins")
+        if ws is not None:
+            _wq_retired.append(ws)
         ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.int8, device=device)
         _wq_workspaces[key] = ws
     return ws

@@ -13,11 +13,14 @@ import warnings
 import torch
 from torch import nn
 
+from ._prepared import PreparedCopiesMixin
+
 __all__ = ["LinearQuant", "LinearA8W8Quant"]
 
 
-class _QuantLinearBase(nn.Module):
+class _QuantLinearBase(PreparedCopiesMixin, nn.Module):
     _validate_dtypes = False
+    _prepared_attrs = ("_prepared_i8",)
 
     def __init__(self, in_features: int, out_features: int, *, bias: bool = True, offset: bool = False,
                  pertoken_scale: bool = False, device=None, dtype=None, output_dtype=None) -> None:
@@ -65,8 +68,9 @@ class _QuantLinearBase(nn.Module):
         """One-time widening for inference (optional, A4W4 only): a weight stored as int32 words of eight int4 values is
         widened to int8 ``[out_features, in_features]`` once, so that a forward pass widens only the activations before
         the int8 GEMM instead of the weight as well.  The parameter the module exposes (and its state_dict) stays as it
-        is; the widened copy is a plain attribute that costs twice the packed weight's size and must be rebuilt by
-        calling this again after the weight changes."""
+        is; the widened copy is a plain attribute that costs twice the packed weight's size.  Moving, casting or
+        reloading the module drops the copy (forward then widens per call again); call this again afterwards, and
+        after changing the weight in place."""
         self._prepared_i8 = None
         if self.weight.dtype == torch.int32:
             from ... import _capi

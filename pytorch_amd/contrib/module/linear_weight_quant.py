@@ -14,10 +14,14 @@ from __future__ import annotations
 import torch
 from torch import nn
 
+from ._prepared import PreparedCopiesMixin
+
 __all__ = ["LinearWeightQuant"]
 
 
-class LinearWeightQuant(nn.Module):
+class LinearWeightQuant(PreparedCopiesMixin, nn.Module):
+    _prepared_attrs = ("_prepared",)
+
     def __init__(self, in_features, out_features, bias: bool = True, device=None, dtype=None,
                  antiquant_offset: bool = False, quant_scale: bool = False, quant_offset: bool = False,
                  antiquant_group_size: int = 0, inner_precise: int = 0, weight_dtype=None) -> None:
@@ -40,7 +44,8 @@ class LinearWeightQuant(nn.Module):
         """One-time repack for inference (optional): an int4 weight is rewritten with its words along N and per-group
         parameters are made row-major ``[G, N]``, the layout the decode kernels stream fastest.  The parameters the
         module exposes (and its state_dict) stay as they are; the prepared copies are plain attributes, so they cost
-        the weight's size again and must be rebuilt by calling this again after the parameters change."""
+        the weight's size again.  Moving, casting or reloading the module drops them; call this again afterwards, and
+        after changing a parameter in place."""
         self._prepared = None
         if self.weight.dtype != torch.int32:
             return self

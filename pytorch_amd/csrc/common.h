@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 #include "../../include/mi355_quant.h"
 
 namespace mi355 {
@@ -55,6 +56,12 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
     v[1] = (_Float16)hi;
     return __builtin_bit_cast(uint32_t, v);
 }
+
+// Planner tuning knobs (tuning.hip): 0 = automatic.  Read with knob(); set through mi355_set_tuning() or, once at
+// load time, through the environment variable of the same name.
+enum Knob { kKnobWqSplit, kKnobWqW, kKnobWqgSplit, kKnobWqgBm, kKnobWqGemmOff, kKnobWqkMt, kKnobWqkNw, kKnobWqkKs,
+            kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmStreamKOff, kKnobCount };
+int knob(Knob k);
 
 inline int check_launch()
 {

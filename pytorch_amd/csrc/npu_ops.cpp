@@ -14,6 +14,7 @@
 #include <ATen/ExpandUtils.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <hip/hip_runtime_api.h>
 #include <torch/library.h>
 
 #include <map>
@@ -173,15 +174,30 @@ std::tuple<Tensor, Tensor, Tensor> dynamic_quant_asym_hip(const Tensor &input, c
 // The split-K reductions of the matmul kernels count arrivals in their workspace: the counters must
 // be zero before a launch and the kernels leave them zero.  One zero-initialised buffer per
 // (device, stream) is kept and reused; launches on one stream are ordered, so they never overlap.
+// Lifetime rules, because a captured HIP graph keeps the pointer it was recorded with:
+//   * a buffer that is superseded by a larger one is never released (it stays alive, zeroed, until the process
+//     ends), so a graph recorded earlier replays on valid, quiescent memory;
+//   * nothing is allocated or filled while the stream is capturing: a fill recorded into a graph is not executed
+//     now, and its buffer would belong to the graph's private pool.  The caller gets an error that says what to do
+//     (run the operator once on that stream before the capture begins).
 Tensor zeroed_workspace(const Tensor &like, size_t bytes)
 {
     static std::mutex mu;
     static std::map<std::pair<int, void *>, Tensor> cache;
+    static std::vector<Tensor> *retired = new std::vector<Tensor>();   // intentionally never freed
     std::lock_guard<std::mutex> lock(mu);
     const auto key = std::make_pair((int)like.device().index(), stream_of(like));
     Tensor &ws = cache[key];
-    if (!ws.defined() || (size_t)ws.numel() < bytes)
+    if (!ws.defined() || (size_t)ws.numel() < bytes) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        TORCH_CHECK(hipStreamIsCapturing(static_cast<hipStream_t>(key.second), &capturing) == hipSuccess, "hipStreamIsCapturing failed");
+        TORCH_CHECK(capturing == hipStreamCaptureStatusNone,
+                    "this operator needs a ", bytes, "-byte zero-initialised workspace on this stream, which cannot be "
+                    "allocated while the stream is being captured: call the operator once with this shape (or a larger "
+                    "one) on this stream before the capture begins");
+        if (ws.defined()) retired->push_back(ws);
         ws = at::zeros({(int64_t)std::max<size_t>(bytes, (size_t)1 << 20)}, like.options().dtype(at::kChar));
+    }
     return ws;
 }
 

@@ -684,11 +684,9 @@ constexpr TileChoice kTiles[] = {{256, 256, 256, 60.0, 57.0}, {256, 224, 256, 55
 // Pick the tile shape that minimises (rounds of resident workgroups) x (time per round).
 TileChoice choose_tile(int M, int N)
 {
-    if (const char *e = getenv("MI355_QMM_TILE")) { // debugging aid: "BMxBN"
-        int bm = 0, bn = 0;
-        if (sscanf(e, "%dx%d", &bm, &bn) == 2)
-            for (const TileChoice &c : kTiles)
-                if (c.bm == bm && c.bn == bn) return c;
+    if (const int forced = knob(kKnobQmmTile)) {          // debugging aid: bm * 1000 + bn
+        for (const TileChoice &c : kTiles)
+            if (c.bm == forced / 1000 && c.bn == forced % 1000) return c;
     }
     TileChoice best = kTiles[0];
     double best_cost = 1e300;
@@ -726,10 +724,8 @@ QmmPlan make_qmm_plan(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ld
         if (S > kt / 4) S = kt / 4;
         if (S > 16) S = 16;
         if (S < 1) S = 1;
-        if (const char *e = getenv("MI355_QMM_SPLIT")) { // debugging aid
-            const int f = atoi(e);
+        if (const int f = knob(kKnobQmmSplit))            // debugging aid
             if (f >= 1 && f <= kt) S = f;
-        }
         pl.S = (int)S;
         if (pl.S > 1) pl.partial_bytes = (size_t)tiles * pl.S * pl.tile.bm * pl.tile.bn * 4;   // tiles <= 128 counters
     }

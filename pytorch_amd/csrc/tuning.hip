@@ -1,0 +1,42 @@
+// Tuning knobs of the planners.  A knob is an integer, 0 = let the planner decide.  Each knob takes its initial value
+// from the environment variable of the same name once, when the library is loaded; afterwards only
+// mi355_set_tuning() changes it, so no launch ever reads the environment.
+#include "common.h"
+#include <atomic>
+#include <stdlib.h>
+#include <string.h>
+
+namespace mi355 {
+namespace {
+const char *const kKnobNames[kKnobCount] = {"MI355_WQ_SPLIT", "MI355_WQ_W",    "MI355_WQG_SPLIT", "MI355_WQG_BM",   "MI355_WQ_GEMM_OFF",
+                                            "MI355_WQK_MT",   "MI355_WQK_NW",  "MI355_WQK_KS",    "MI355_QMM_SPLIT", "MI355_QMM_TILE",
+                                            "MI355_WQ_DECODE_OFF", "MI355_QMM_STREAMK_OFF"};
+std::atomic<int> g_knobs[kKnobCount];
+const bool g_knobs_loaded = []() {
+    for (int i = 0; i < kKnobCount; i++) {
+        const char *e = getenv(kKnobNames[i]);
+        int v = 0;
+        if (e) {
+            int bm = 0, bn = 0;
+            v = (i == kKnobQmmTile && sscanf(e, "%dx%d", &bm, &bn) == 2) ? bm * 1000 + bn : atoi(e);
+        }
+        g_knobs[i].store(v, std::memory_order_relaxed);
+    }
+    return true;
+}();
+} // namespace
+
+int knob(Knob k) { return g_knobs[k].load(std::memory_order_relaxed); }
+} // namespace mi355
+
+extern "C" int mi355_set_tuning(const char *name, int value)
+{
+    using namespace mi355;
+    if (!name) return MI355_ERR_BAD_ARGUMENT;
+    for (int i = 0; i < kKnobCount; i++)
+        if (strcmp(name, kKnobNames[i]) == 0) {
+            g_knobs[i].store(value, std::memory_order_relaxed);
+            return MI355_OK;
+        }
+    return MI355_ERR_BAD_ARGUMENT;
+}

@@ -107,11 +107,6 @@ __device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint
 constexpr uint32_t kOutOfRange = 0x80000000u;   // lane offset beyond every buffer size: the load returns zero, no traffic
 constexpr int kNonTemporal = 2;                 // cache-policy bit for data that is read once
 
-inline int env_int(const char *name)
-{
-    const char *e = getenv(name);
-    return e ? atoi(e) : 0;
-}
 
 struct WqArgs {
     const uint16_t *x;              // bf16 [M, K]
@@ -138,7 +133,8 @@ struct WqArgs {
 };
 
 // Output side of a workgroup tile of NBW columns whose partial sums lie in LDS as red[slice][16 rows][NBW].
-// Every thread owns quads of 4 consecutive columns.  Without a split over K the sums go straight to the output.
+// Every thread owns quads of 4 consecutive columns; N must be a multiple of 4 (every planner that uses this requires it),
+// so a quad is either wholly inside the row or skipped.  Without a split over K the sums go straight to the output.
 // With K split over S workgroups every workgroup publishes its partial and the last arrival adds them in chunk
 // order: the exchange uses agent-scope (sc1) write-through stores and cache-bypassing loads, ordered by the
 // wavefronts' own store counters, the workgroup barrier and a relaxed agent-scope counter; a full release/acquire

@@ -498,18 +498,17 @@ WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_
     const int64_t ldw_bytes = w_bits == 4 ? ldw * 4 : ldw;     // bytes between k rows, or (K-major) between columns
     const int64_t group = group_size > 0 ? group_size : K;
     pl.grouped = group_size > 0 && group != K;
-    const char *off_env = getenv("MI355_WQ_GEMM");             // tuning aid: "0" keeps every shape on the streaming kernels
     const bool layout_ok = layout == 1 ? ldw_bytes >= row_bytes && (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 32)
                                        : layout == 2 && w_bits == 8 && ldw >= K && (uint64_t)N * (uint64_t)ldw < (1ull << 32);
     pl.ok = M > 32 && layout_ok && K >= 128 && K % 128 == 0 && group % 128 == 0 && N % 8 == 0 && ldw_bytes % 4 == 0 &&
             ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 4)) &&
             (scale == nullptr || aligned(scale, 4)) && (offset == nullptr || aligned(offset, 4)) &&
             (uint64_t)128 * (uint64_t)ldx * 2 < (1ull << 31) &&
-            (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && !(off_env && off_env[0] == '0');
+            (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && !knob(kKnobWqGemmOff) /* tuning aid: keeps every shape on the streaming kernels */;
     if (!pl.ok) return pl;
     const int bn = w_bits == 4 ? 256 : 128;
     pl.bm = M <= 64 ? 64 : 128;
-    if (const int f = env_int("MI355_WQG_BM"))                 // tuning aid
+    if (const int f = knob(kKnobWqgBm))                 // tuning aid
         if (f == 64 || f == 128) pl.bm = f;
     pl.tiles_m = (int)((M + pl.bm - 1) / pl.bm);
     pl.tiles_n = pl.k_major ? (int)((N + 127) / 128) : (int)((row_bytes + 127) / 128);
@@ -519,7 +518,7 @@ WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_
     int64_t S = tiles < kNumCU ? kNumCU / tiles : 1;
     if (S > pl.n_units) S = pl.n_units;
     if (S > 8) S = 8;
-    if (const int f = env_int("MI355_WQG_SPLIT"))              // tuning aid
+    if (const int f = knob(kKnobWqgSplit))              // tuning aid
         if (f >= 1 && f <= pl.n_units) S = f;
     if (S > 1 && ((uint64_t)S * pl.bm * bn * 4 >= (1ull << 32) || (size_t)tiles * 4 > kWorkspaceCounterBytes)) S = 1;
     pl.S = (int)S;

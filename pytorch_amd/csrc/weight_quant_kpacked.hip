@@ -419,7 +419,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
             (uint64_t)N * (uint64_t)ldw_n * 4 < (1ull << 32) && (uint64_t)M * (uint64_t)ldx * 2 < (1ull << 32);
     if (!pl.ok) return pl;
     pl.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
-    if (const int f = env_int("MI355_WQK_MT"))      // tuning aid
+    if (const int f = knob(kKnobWqkMt))      // tuning aid
         if (f == 1 || f == 2 || f == 4) pl.mt = f;
     pl.mchunks = (int)((M + pl.mt * 16 - 1) / (pl.mt * 16));
     pl.grouped = group_size > 0 && group != K;
@@ -437,7 +437,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     pl.ntw = pl.mt == 4 ? 2 : 1;
     const int tiles8 = (int)((N + 8 * pl.ntw * 16 - 1) / (8 * pl.ntw * 16));
     pl.nw = (int64_t)tiles8 * pl.mchunks >= 200 ? 8 : 4;
-    if (const int f = env_int("MI355_WQK_NW"))      // tuning aid
+    if (const int f = knob(kKnobWqkNw))      // tuning aid
         if (f == 4 || f == 8) pl.nw = f;
     const int wg_cols = pl.nw * pl.ntw * 16;
     pl.tiles = (int)((N + wg_cols - 1) / wg_cols);
@@ -446,7 +446,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     if (S > pl.n_units) S = pl.n_units;
     if (S > 16) S = 16;
     if (S < 1) S = 1;
-    if (const int f = env_int("MI355_WQ_SPLIT"))
+    if (const int f = knob(kKnobWqSplit))
         if (f >= 1 && f <= pl.n_units) S = f;
     if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1;
     if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) S = 1;
@@ -465,7 +465,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     pl.S = S;
     // with four column tiles and at most two m tiles the workgroup's K range is cut into two slices (eight wavefronts,
     // two per SIMD) when it holds at least two units
-    if (pl.nw == 4 && pl.mt <= 2 && (pl.n_units + S - 1) / S >= 2 && env_int("MI355_WQK_KS") != 1) pl.ks = 2;
+    if (pl.nw == 4 && pl.mt <= 2 && (pl.n_units + S - 1) / S >= 2 && knob(kKnobWqkKs) != 1) pl.ks = 2;
     pl.lds_bytes = lds_need(S);
     pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
     pl.counter_bytes = S > 1 ? kWorkspaceCounterBytes : 0;

@@ -331,7 +331,7 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
     const int step0 = u0 * p.unit_steps, nsteps = (u1 - u0) * p.unit_steps;
     const int nchunks = (nsteps + CH - 1) / CH;
 
-    // Weights: this wavefront's 16 rows (rows past N repeat the last valid row; their columns are never stored).
+    // Weights: this wavefront's 16 rows (rows past N repeat the last valid row; N is a multiple of 4, so quads of columns past N are skipped whole).
     // A load instruction fetches whole cache lines - lane l takes 16 bytes of row l/8 (+8 for the second load) - which
     // reads HBM a quarter faster than fetching the MFMA operand layout directly (16 rows x 64 bytes per
     // instruction); the wavefront then turns the step around through a private 2 KiB LDS tile.  The 16-byte chunk a
@@ -572,7 +572,7 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
     // W adjacent strips per workgroup; the remaining wavefronts slice K.  Pairs of strips read DRAM markedly
     // better, but halve the number of tiles: with few strips that means a deeper split of K and a longer exchange.
     pl.w = pl.strips >= 112 ? 2 : 1;
-    if (const int f = env_int("MI355_WQ_W"))      // tuning aid
+    if (const int f = knob(kKnobWqW))      // tuning aid
         if (f == 1 || f == 2) pl.w = f;
     pl.sgroups = (pl.strips + pl.w - 1) / pl.w;
     constexpr int kMaxSlabSteps = (160 * 1024 - 16) / 1024;
@@ -589,14 +589,14 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
         // the activations of a workgroup's K chunk must fit in LDS (1 KiB per step and m tile)
         auto slab_steps = [&](int chunks) { return (pl.n_units + chunks - 1) / chunks * pl.unit_steps * pl.mt; };
         while (slab_steps(S) > kMaxSlabSteps && S < s_max) S++;
-        if (const int f = env_int("MI355_WQ_SPLIT"))  // tuning aid: force the number of K chunks
+        if (const int f = knob(kKnobWqSplit))  // tuning aid: force the number of K chunks
             if (f >= 1 && f <= s_max) S = f;
         if (w_bits == 4 && pl.mt == 2 && grouped && nwv == 8 && pl.bs == 4) {
             // two m tiles of int4 run much better without the running total (eight wavefronts, no spills): split K
             // further, down to one scale group per wavefront, when that stays within 16 chunks (measured at
             // M = 128, K = 4096: 73 us against 92 us)
             const int s_one = (pl.n_units + pl.ks - 1) / pl.ks;
-            if (s_one > S && s_one <= 16 && s_one <= s_max && !env_int("MI355_WQ_SPLIT")) S = s_one;
+            if (s_one > S && s_one <= 16 && s_one <= s_max && !knob(kKnobWqSplit)) S = s_one;
         }
         if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1; // exchange offsets are 32-bit
         pl.S = S;
@@ -668,7 +668,8 @@ WqKmPlan make_kmajor_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, i
 {
     WqKmPlan pl{};
     const int64_t group = group_size > 0 ? group_size : K;
-    pl.fast = K > 0 && K % 128 == 0 && group % 128 == 0 && ldw_n >= K && ldw_n % 16 == 0 && ldx % 8 == 0 &&
+    // N % 4: the output side stores quads of four columns (other N take the generic kernel)
+    pl.fast = K > 0 && K % 128 == 0 && group % 128 == 0 && N % 4 == 0 && ldw_n >= K && ldw_n % 16 == 0 && ldx % 8 == 0 &&
               (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 16)) &&
               (uint64_t)N * (uint64_t)ldw_n < (1ull << 32) && (uint64_t)M * (uint64_t)ldx * 2 < (1ull << 32);
     if (!pl.fast) return pl;
@@ -682,7 +683,7 @@ WqKmPlan make_kmajor_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, i
     if (S > pl.n_units) S = pl.n_units;
     if (S > 16) S = 16;
     if (S < 1) S = 1;
-    if (const int f = env_int("MI355_WQ_SPLIT"))
+    if (const int f = knob(kKnobWqSplit))
         if (f >= 1 && f <= pl.n_units) S = f;
     if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1;
     if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) S = 1;

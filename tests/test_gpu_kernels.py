@@ -320,6 +320,29 @@ def test_w8a16_kmajor_and_no_offset(capi, golden):
     bf16_gate(out, _wq_golden(golden, d2, 0))
 
 
+@pytest.mark.parametrize("M,K,N", [(5, 256, 130), (5, 256, 132), (32, 512, 6), (3, 128, 1)])
+def test_w8a16_kmajor_ragged_columns(capi, golden, M, K, N):
+    """int8 weight stored [N, K] with N not a multiple of 4 (or of 8): the K-major streaming kernel stores quads of
+    columns, so such widths must take a path that writes exactly N columns; the row after the last column and the
+    guard bytes behind the output must stay untouched."""
+    d = workloads.w8a16_inputs(seed=N, M=M, K=K, N=N, weight_nk=True)
+    x, w, sc, of = (d[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset"))
+    want = _wq_golden(golden, d, 0)
+    for _ in range(3):                                   # a race between tiles would not repeat
+        out = capi.weight_quant_matmul(x, w, sc, of)
+        bf16_gate(out, want, floor=True)
+    # output rows inside a wider, pre-filled buffer: nothing outside [M, N] may change
+    wide = torch.full((M + 1, N + 8), 7.0, dtype=torch.bfloat16, device="cuda")
+    view = wide[:M, :N]
+    st = capi.lib().mi355_weight_quant_matmul(x.data_ptr(), 0, w.data_ptr(), 8, sc.data_ptr(), of.data_ptr(), None, view.data_ptr(),
+                                              M, N, K, 0, 0, 1, x.stride(0), w.stride(0), w.stride(1), wide.stride(0), None, 0,
+                                              torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert torch.equal(view, out)
+    assert (wide[:, N:] == 7.0).all() and (wide[M] == 7.0).all()
+
+
 @pytest.mark.parametrize("M", [1, 8, 32, 128])
 def test_w4a16_grouped(capi, golden, M):
     d = workloads.w4a16_inputs(seed=M, M=M, K=4096, N=1024, group_size=128)
@@ -446,13 +469,12 @@ def _tiled_case(capi, golden, bits, M, K, N, gs, f16, with_bias, nk):
     print("tiled", bits, M, K, N, gs, bf16_gate(out, torch.from_numpy(gold)))
     # the split over K must not change a bit of the result, whatever the number of chunks, and repeated launches
     # (which reuse the workspace and its arrival counters) must repeat the result
-    import os
-    for split in ("1", "2"):
-        os.environ["MI355_WQG_SPLIT"] = split
+    for split in (1, 2):
+        capi.set_tuning("MI355_WQG_SPLIT", split)
         try:
             again = capi.weight_quant_matmul(*args, group_size=group, bias=None if bias is None else bias.cuda())
         finally:
-            del os.environ["MI355_WQG_SPLIT"]
+            capi.set_tuning("MI355_WQG_SPLIT", 0)
         bf16_gate(again, torch.from_numpy(gold))
     for _ in range(5):
         assert torch.equal(capi.weight_quant_matmul(*args, group_size=group, bias=None if bias is None else bias.cuda()), out)
@@ -509,13 +531,12 @@ def test_weight_quant_int4_words_along_k(capi, golden, M, K, N, gs, f16, params_
     print("kpacked", M, K, N, gs, bf16_gate(out, torch.from_numpy(gold)))
     for _ in range(3):
         assert torch.equal(call(), out)
-    import os
-    for split in ("1", "2", "3"):
-        os.environ["MI355_WQ_SPLIT"] = split
+    for split in (1, 2, 3):
+        capi.set_tuning("MI355_WQ_SPLIT", split)
         try:
             bf16_gate(call(), torch.from_numpy(gold))
         finally:
-            del os.environ["MI355_WQ_SPLIT"]
+            capi.set_tuning("MI355_WQ_SPLIT", 0)
     assert torch.equal(call(), out)
     out0 = call(None)
     _, gold0 = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(sc), None,

@@ -44,13 +44,13 @@ def test_c2_quant_matmul_full_size(pa, golden, weight_nk):
     # ... and of every output column
     rowsum = d["x1"].to(torch.int64).sum(0)
     assert torch.equal(acc.to(torch.int64).sum(0), rowsum @ d["x2"].to(torch.int64))
-    rows = torch.tensor([0, 1, 255, 256, 511, 640, 1000, 1023])
-    want = golden.int8_gemm(d["x1"][rows].numpy(), d["x2"].numpy())
-    assert np.array_equal(acc[rows].numpy(), want)
+    # every accumulator against the oracle's own integer product (about a second on the host cores)
+    want_acc = golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy())
+    assert np.array_equal(acc.numpy(), want_acc)
     for bias in (d["bias"], None):
         out = pa.npu_quant_matmul(x1, x2, d["scale"].cuda(), pertoken_scale=d["pertoken_scale"].cuda(),
                                   bias=None if bias is None else bias.cuda(), output_dtype=torch.bfloat16)
-        want = golden.quant_matmul_epilogue(acc.numpy(), d["scale"].numpy(), d["pertoken_scale"].numpy(),
+        want = golden.quant_matmul_epilogue(want_acc, d["scale"].numpy(), d["pertoken_scale"].numpy(),
                                             None if bias is None else _bits(bias))
         assert np.array_equal(_bits(out), want)
 
@@ -493,6 +493,70 @@ def test_graph_replays_match_eager(pa):
         torch.cuda.synchronize()
         for got, exp in zip(eager, want):
             assert torch.equal(got, exp)
+
+
+def test_workspace_outlives_growth_after_capture(pa):
+    """A graph captured with a small split-K workspace must replay correctly after an eager call on the same stream
+    needed a larger one: the superseded buffer is kept alive (and zeroed at rest), never handed back to the allocator."""
+    from pytorch_amd import _capi
+    g = torch.Generator().manual_seed(21)
+    M, K, N = 64, 4096, 1024
+    q = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).cuda()
+    w = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).cuda().t()
+    sc, ps = (torch.rand(N, generator=g) * 1e-2).cuda(), (torch.rand(M, generator=g) * 1e-2).cuda()
+    Kb, Nb = 14336, 4096
+    qb = torch.randint(-127, 128, (M, Kb), generator=g, dtype=torch.int8).cuda()
+    wb = torch.randint(-127, 128, (Nb, Kb), generator=g, dtype=torch.int8).cuda().t()
+    scb = (torch.rand(Nb, generator=g) * 1e-2).cuda()
+    small_ws = _capi.lib().mi355_quant_matmul_workspace(M, N, K, 1, K)
+    big_ws = _capi.lib().mi355_quant_matmul_workspace(M, Nb, Kb, 1, Kb)
+    assert 0 < small_ws <= (1 << 20) < big_ws, (small_ws, big_ws)      # the second call must outgrow the first buffer
+    small = lambda: pa.npu_quant_matmul(q, w, sc, pertoken_scale=ps, output_dtype=torch.bfloat16)
+    big = lambda: pa.npu_quant_matmul(qb, wb, scb, pertoken_scale=ps, output_dtype=torch.bfloat16)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        want = small().clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            out = small()
+        want_big = big().clone()                       # eager, same stream: allocates the larger workspace
+        stream.synchronize()
+        for it in range(3):
+            out.zero_()
+            graph.replay()
+            stream.synchronize()
+            assert torch.equal(out, want), f"replay {it} after the workspace grew differs"
+            assert torch.equal(big(), want_big)
+            assert torch.equal(small(), want)
+    torch.cuda.synchronize()
+
+
+def test_capture_without_warmup_is_refused(pa):
+    """A split-K operator whose stream has no workspace yet cannot allocate (and zero) one inside a capture: it raises
+    and says what to do; after one eager call on that stream the same capture works."""
+    g = torch.Generator().manual_seed(22)
+    M, K, N = 64, 4096, 1024
+    q = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).cuda()
+    w = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).cuda().t()
+    sc = (torch.rand(N, generator=g) * 1e-2).cuda()
+    op = lambda: pa.npu_quant_matmul(q, w, sc, output_dtype=torch.bfloat16)
+    want = op().clone()
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()                       # fresh stream: no workspace is cached for it
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="before the capture begins"):
+        with torch.cuda.graph(graph, stream=stream):
+            op()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        op()
+    stream.synchronize()
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph2, stream=stream):
+        out = op()
+    graph2.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
 
 
 def test_c5_mlp_prefill_properties(pa, golden):

@@ -332,6 +332,27 @@ def test_linear_weight_quant_marshalling(pa, monkeypatch):
     assert args[7] == 128 and args[8] == 0 and kwargs == {"weight_dtype": None}
 
 
+def test_prepared_copies_are_dropped_when_the_module_moves_or_reloads(pa):
+    """prepare_() keeps derived weight copies in plain attributes; .to()/.half()/load_state_dict must drop them so that a
+    stale or wrong-device copy can never be used (no kernel runs here: the copies are set by hand)."""
+    from pytorch_amd.contrib.module import LinearQuant, LinearWeightQuant
+    m = LinearQuant(64, 32, bias=False)
+    m._prepared_i8 = torch.zeros(32, 64, dtype=torch.int8)
+    m.to("meta")
+    assert m._prepared_i8 is None
+    m = LinearQuant(64, 32, bias=False)
+    m._prepared_i8 = torch.zeros(32, 64, dtype=torch.int8)
+    m.load_state_dict(LinearQuant(64, 32, bias=False).state_dict())
+    assert m._prepared_i8 is None
+    w = LinearWeightQuant(256, 64, bias=False)
+    w._prepared = (torch.zeros(1), None, None)
+    w.to(torch.device("cpu"), torch.float64)
+    assert w._prepared is None
+    w._prepared = (torch.zeros(1), None, None)
+    w.load_state_dict(LinearWeightQuant(256, 64, bias=False).state_dict())
+    assert w._prepared is None
+
+
 def test_flop_counter_formulas(pa):
     """2*M*K*N for the quantised matmuls, as torch_npu/profiler/_flops_formulas.py:319-329 counts a matmul; counted on
     meta tensors, so no kernel runs."""
