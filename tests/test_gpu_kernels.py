@@ -334,8 +334,11 @@ def test_w8a16_kmajor_ragged_columns(capi, golden, M, K, N):
     # output rows inside a wider, pre-filled buffer: nothing outside [M, N] may change
     wide = torch.full((M + 1, N + 8), 7.0, dtype=torch.bfloat16, device="cuda")
     view = wide[:M, :N]
+    need = capi.lib().mi355_weight_quant_matmul_workspace(M, N, K, 8, 0)
+    ws = capi._wq_workspace(x.device, need) if need else None
     st = capi.lib().mi355_weight_quant_matmul(x.data_ptr(), 0, w.data_ptr(), 8, sc.data_ptr(), of.data_ptr(), None, view.data_ptr(),
-                                              M, N, K, 0, 0, 1, x.stride(0), w.stride(0), w.stride(1), wide.stride(0), None, 0,
+                                              M, N, K, 0, 0, 1, x.stride(0), w.stride(0), w.stride(1), wide.stride(0),
+                                              None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(),
                                               torch.cuda.current_stream().cuda_stream)
     assert st == 0
     torch.cuda.synchronize()
@@ -593,7 +596,9 @@ def test_weight_quant_random_shapes(capi, golden):
         try:
             out = capi.weight_quant_matmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
                                            None if off is None else off.cuda(), group_size=gs)
-            bf16_gate(out, torch.from_numpy(gold))
+            # outputs of a few hundred elements: one element that cancels to almost nothing is already more than
+            # 0.1 % of them, so those are counted with the cancellation floor; larger ones strictly
+            bf16_gate(out, torch.from_numpy(gold), floor=out.numel() < 8192)
         except (AssertionError, capi.Mi355Error) as e:
             raise AssertionError(f"case {case}: bits={bits} M={M} K={K} N={N} gs={gs} nk={nk} f16={f16} offset={with_off}: {e}")
 

@@ -500,7 +500,7 @@ def test_workspace_outlives_growth_after_capture(pa):
     needed a larger one: the superseded buffer is kept alive (and zeroed at rest), never handed back to the allocator."""
     from pytorch_amd import _capi
     g = torch.Generator().manual_seed(21)
-    M, K, N = 64, 4096, 1024
+    M, K, N = 64, 4096, 256
     q = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).cuda()
     w = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).cuda().t()
     sc, ps = (torch.rand(N, generator=g) * 1e-2).cuda(), (torch.rand(M, generator=g) * 1e-2).cuda()
