@@ -157,6 +157,26 @@ int mi355_quant_matmul_qparam(const int8_t *a, const int8_t *b, const uint64_t *
                               void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * mi355_quant_matmul without a workspace argument and without any allocation.  It has no counterpart in the
+ * reference (there the adapter allocates a workspace per call, torch_npu/csrc/framework/utils/OpPreparation.h:130-132);
+ * it exists for callers that cannot allocate or carry a workspace: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Arguments and results are those of mi355_quant_matmul (bit-identical outputs).
+ * The arrival counters, split-K partial sums and the transposed copy of a contiguous [K,N] weight live in a fixed
+ * device array of MI355_NOALLOC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.
+ *   - returns MI355_ERR_WORKSPACE when mi355_quant_matmul_workspace(M, N, K, ldb_k, ldb_n) exceeds that size
+ *     (for example a large weight stored [K,N]: store it [N,K], or use mi355_quant_matmul);
+ *   - calls no hipMalloc / hipFree and no allocating library routine; the first call on a device resolves the
+ *     array's address and clears its counters with a small kernel on `stream`;
+ *   - all calls on one GPU share that GPU's array: calls that may overlap in time (different streams without an
+ *     ordering between them, several host threads) race on it and must be serialised by the caller.
+ */
+#define MI355_NOALLOC_SCRATCH_BYTES ((size_t)16 * 1024 * 1024 + 16384)
+int mi355_quant_matmul_noalloc(const int8_t *a, const int8_t *b, const float *pertoken_scale,
+                               const float *scale, int64_t scale_len, const void *bias, int bias_dtype,
+                               void *out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                               int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc, void *stream);
+
+/*
  * npu_weight_quant_batchmatmul, W8A16 per channel and W4A16 per group.
  * Replaces the aclnn WeightQuantBatchMatmulV2 call behind torch_npu.npu_weight_quant_batchmatmul
  * (caller: torch_npu/contrib/module/linear_weight_quant.py:98-109; CPU golden:

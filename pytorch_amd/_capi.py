@@ -18,7 +18,8 @@ EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quan
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
-           "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth", "mi355_set_tuning")
+           "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth", "mi355_set_tuning",
+           "mi355_quant_matmul_noalloc")
 
 _lib = None
 
@@ -55,6 +56,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_quant_matmul_qparam.argtypes = [vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
         L.mi355_quantize.argtypes = [vp, i32, vp, i64, vp, i32, i64, vp, i32, i64, i64, i64, i32, vp]
         L.mi355_set_tuning.argtypes = [ctypes.c_char_p, i32]
+        L.mi355_quant_matmul_noalloc.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp]
         _lib = L
     return _lib
 

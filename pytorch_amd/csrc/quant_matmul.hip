@@ -24,6 +24,7 @@
 #include <stdio.h>
 #include <type_traits>
 #include <stdlib.h>
+#include <mutex>
 
 namespace mi355 {
 namespace {
@@ -893,4 +894,72 @@ extern "C" int mi355_trans_quant_param(const float *scale, int64_t scale_len, co
     hipLaunchKernelGGL(trans_quant_param_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), scale, scale_len == 1, offset, offset_len == 1, out, n);
     return check_launch();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// mi355_quant_matmul_noalloc: the same product for callers that cannot provide or allocate a workspace (code under
+// HIP graph capture, serving loops and harnesses that forbid hipMalloc).  The workspace the kernels need (arrival
+// counters, split-K partial sums, the transposed copy of a [K,N] weight) lives in a file-scope device array of
+// fixed size; every GPU the library runs on holds its own copy until the process ends.
+namespace mi355 {
+namespace {
+
+constexpr size_t kStaticScratchBytes = MI355_NOALLOC_SCRATCH_BYTES;
+__device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+__global__ __launch_bounds__(256) void scratch_clear_kernel(uint32_t *p, int words)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < words) p[i] = 0u;
+}
+
+constexpr int kMaxDevices = 64;
+struct DeviceScratch {
+    void *ptr = nullptr;        // device address of this GPU's copy of `scratch`
+    bool ready = false;
+};
+DeviceScratch g_scratch[kMaxDevices];
+std::mutex g_scratch_mu;
+
+// Device address of the current device's scratch array; on first use per device the address is resolved and the
+// arrival counters are cleared by a small kernel on the caller's stream (a fill kernel, not a memset node, so that
+// a caller who captures this first call records something that replays correctly).
+int scratch_of_current_device(void **out, hipStream_t s)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MI355_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    DeviceScratch &d = g_scratch[dev];
+    if (!d.ready) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return MI355_ERR_LAUNCH;
+        hipLaunchKernelGGL(scratch_clear_kernel, dim3((unsigned)(kWorkspaceCounterBytes / 4 / 256)), dim3(256), 0, s,
+                           static_cast<uint32_t *>(ptr), (int)(kWorkspaceCounterBytes / 4));
+        if (check_launch() != MI355_OK) return MI355_ERR_LAUNCH;
+        d.ptr = ptr;
+        d.ready = true;
+    }
+    *out = d.ptr;
+    return MI355_OK;
+}
+
+} // namespace
+} // namespace mi355
+
+extern "C" int mi355_quant_matmul_noalloc(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale,
+                                          int64_t scale_len, const void *bias, int bias_dtype, void *out, int out_dtype,
+                                          int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n,
+                                          int64_t ldc, void *stream)
+{
+    using namespace mi355;
+    if (out_dtype == MI355_OUT_INT8) return MI355_ERR_BAD_ARGUMENT;
+    const size_t need = mi355_quant_matmul_workspace(M, N, K, ldb_k, ldb_n);
+    if (need > kStaticScratchBytes) return MI355_ERR_WORKSPACE;      // beyond the fixed scratch: use mi355_quant_matmul
+    void *ws = nullptr;
+    if (need > 0) {
+        const int st = scratch_of_current_device(&ws, static_cast<hipStream_t>(stream));
+        if (st != MI355_OK) return st;
+    }
+    return run_quant_matmul(a, b, pertoken_scale, scale, nullptr, scale_len, bias, bias_dtype, out, out_dtype, M, N, K, lda,
+                            ldb_k, ldb_n, ldc, ws, need > 0 ? kStaticScratchBytes : 0, stream);
 }
