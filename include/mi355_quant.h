@@ -108,10 +108,13 @@ int mi355_dynamic_quant_asymmetric(const void *x, int in_dtype, const void *smoo
  *                 types are rejected)
  *   workspace: at least mi355_quant_matmul_workspace(...) bytes (may be NULL when that is 0), 16-byte aligned.
  *              It holds a transposed copy of a contiguous [K,N] weight and, for narrow outputs with a long K,
- *              the partial sums and arrival counters of a split over K.  The counters lie at its start and
- *              must be zero before the first launch that uses the buffer; every launch leaves them zero, so
- *              one zero-initialised buffer can serve all later launches on the same stream.
+ *              the partial sums and arrival counters of a split over K.  The first MI355_WORKSPACE_ZERO_BYTES of
+ *              every workspace of this library (arrival counters, then a zone for exchanges that recognise data by
+ *              its being non-zero) must be zero before the first launch that uses the buffer; every launch leaves
+ *              them zero and keeps everything else behind them, so one zero-initialised buffer can serve all later
+ *              launches of all operators on the same stream.
  */
+#define MI355_WORKSPACE_ZERO_BYTES ((size_t)16 * 1024 * 1024 + 16384)
 size_t mi355_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n);
 
 int mi355_quant_matmul(const int8_t *a, const int8_t *b,
@@ -163,8 +166,10 @@ int mi355_quant_matmul_qparam(const int8_t *a, const int8_t *b, const uint64_t *
  * harnesses that forbid hipMalloc.  Arguments and results are those of mi355_quant_matmul (bit-identical outputs).
  * The arrival counters, split-K partial sums and the transposed copy of a contiguous [K,N] weight live in a fixed
  * device array of MI355_NOALLOC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.
- *   - returns MI355_ERR_WORKSPACE when mi355_quant_matmul_workspace(M, N, K, ldb_k, ldb_n) exceeds that size
- *     (for example a large weight stored [K,N]: store it [N,K], or use mi355_quant_matmul);
+ *   - the array is private to this operator, so it holds only 16 KiB of counters plus what the problem needs behind
+ *     them: returns MI355_ERR_WORKSPACE when mi355_quant_matmul_workspace(M, N, K, ldb_k, ldb_n) minus the 16 MiB
+ *     exchange zone of the shared workspaces exceeds that size (for example a large weight stored [K,N]: store it
+ *     [N,K], or use mi355_quant_matmul);
  *   - calls no hipMalloc / hipFree and no allocating library routine; the first call on a device resolves the
  *     array's address and clears its counters with a small kernel on `stream`;
  *   - all calls on one GPU share that GPU's array: calls that may overlap in time (different streams without an
@@ -199,12 +204,14 @@ int mi355_quant_matmul_noalloc(const int8_t *a, const int8_t *b, const float *pe
  *   out[m*ldo+n] = round( sum_k float(x[m,k]) * ((float(w[k,n]) + float(offset[g,n])) * float(scale[g,n])) + float(bias[n]) )
  *   group_size: 0 (per channel) or a multiple of 32 that divides K
  *   workspace: at least mi355_weight_quant_matmul_workspace(...) bytes (may be NULL when that is 0), 16-byte aligned.
- *              It holds the arrival counters and partial sums of a split over K.  The counters lie at its start
- *              and must be zero before the first launch that uses the buffer; every launch leaves them zero, so one
- *              zero-initialised buffer can serve all later launches on the same stream.
- *   One kernel launch per call: a weight-streaming kernel for M <= 32 and a tiled GEMM above that; int4 words along
- *   K take a kernel of their own in which a wavefront owns 16 output columns for all of K (no split of K at
- *   decode shapes).
+ *              It holds the arrival counters and partial sums of a split over K; its first
+ *              MI355_WORKSPACE_ZERO_BYTES must be zero before the first launch that uses the buffer and are left
+ *              zero by every launch (see mi355_quant_matmul), so one zero-initialised buffer can serve all later
+ *              launches on the same stream.
+ *   One kernel launch per call: weight-streaming kernels for M <= 32 (for int4 words along N a barrier-free one whose
+ *   workgroups exchange their partial sums through the workspace's zero zone) and a tiled GEMM above that; int4
+ *   words along K take a kernel of their own in which a wavefront owns 16 output columns for all of K (no split of
+ *   K at decode shapes).
  */
 size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size);
 
@@ -306,6 +313,13 @@ int mi355_unpack_int4(const void *x, int8_t *out, int64_t rows, int64_t cols, in
  * reads the environment.  Returns MI355_ERR_BAD_ARGUMENT for an unknown name.  Process-wide, not thread-scoped.
  */
 int mi355_set_tuning(const char *name, int value);
+
+/*
+ * Identifier of the HIP graph capture that `stream` is part of, 0 when the stream is not capturing.  No counterpart in
+ * the reference (aclnn workspaces are allocated per call by the adapter, OpPreparation.h:130-132); a host layer that
+ * caches zeroed workspaces uses it to give every capture a workspace of its own.
+ */
+int mi355_stream_capture_id(void *stream, unsigned long long *id);
 
 #ifdef __cplusplus
 }

@@ -19,7 +19,7 @@ EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quan
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
            "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth", "mi355_set_tuning",
-           "mi355_quant_matmul_noalloc")
+           "mi355_quant_matmul_noalloc", "mi355_stream_capture_id")
 
 _lib = None
 
@@ -56,6 +56,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_quant_matmul_qparam.argtypes = [vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
         L.mi355_quantize.argtypes = [vp, i32, vp, i64, vp, i32, i64, vp, i32, i64, i64, i64, i32, vp]
         L.mi355_set_tuning.argtypes = [ctypes.c_char_p, i32]
+        L.mi355_stream_capture_id.argtypes = [vp, ctypes.POINTER(ctypes.c_ulonglong)]
         L.mi355_quant_matmul_noalloc.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp]
         _lib = L
     return _lib
@@ -151,21 +152,32 @@ def quant_matmul_qparam(x1, x2, qparam, bias=None, out_dtype=torch.int8, workspa
 
 
 _wq_workspaces = {}
+_wq_capture_workspaces = {}
 _wq_retired = []        # superseded workspaces stay alive: a captured graph may still hold their address
+ZERO_AREA_BYTES = (16 << 20) + 16384     # MI355_WORKSPACE_ZERO_BYTES
 
 
 def _wq_workspace(device, nbytes: int):
-    """Zero-initialised workspace reused across calls on one stream: the kernel needs its counters
-    to start at zero and leaves them at zero.  Never allocated (or filled) while the stream is capturing."""
-    key = (device.index, torch.cuda.current_stream().cuda_stream)
+    """Zero-initialised workspace reused across calls on one stream: the kernels need its leading zero area to start
+    at zero and leave it zero.  Calls made while the stream is capturing get one workspace per capture (allocated from
+    the graph's pool, its zero fill recorded into the graph); eager calls never see those."""
+    stream = torch.cuda.current_stream().cuda_stream
+    key = (device.index, stream)
+    want = max(nbytes, ZERO_AREA_BYTES + (1 << 20))
+    cid = ctypes.c_ulonglong(0)
+    _check(lib().mi355_stream_capture_id(ctypes.c_void_p(stream), ctypes.byref(cid)), "mi355_stream_capture_id")
+    if cid.value:
+        ent = _wq_capture_workspaces.get(key)
+        if ent is None or ent[0] != cid.value or ent[1].numel() < nbytes:
+            ent = (cid.value, torch.zeros(want, dtype=torch.int8, device=device))
+            _wq_capture_workspaces[key] = ent
+        return ent[1]
+    _wq_capture_workspaces.pop(key, None)
     ws = _wq_workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        if torch.cuda.is_current_stream_capturing():
-            raise Mi355Error(f"a {nbytes}-byte zeroed workspace cannot be allocated during stream capture: "
-                             "call once with this shape on this stream before the capture begins")
         if ws is not None:
             _wq_retired.append(ws)
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.int8, device=device)
+        ws = torch.zeros(want, dtype=torch.int8, device=device)
         _wq_workspaces[key] = ws
     return ws
 

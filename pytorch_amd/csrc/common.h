@@ -43,10 +43,14 @@ __device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2)
     return pack_bf16x2(s0 * bf16_lo(b2), s1 * bf16_hi(b2));
 }
 
-// Every workspace of this library starts with this many bytes of arrival counters (zero before the first launch,
-// left zero by every launch); whatever else a launch keeps in the workspace lies behind them, so one
-// zero-initialised buffer can be shared by all launches of a stream.
-constexpr size_t kWorkspaceCounterBytes = 16384;
+// Every workspace of this library starts with a zero area: kWorkspaceCounterCapacity bytes of arrival counters followed
+// by kWorkspaceZoneBytes for exchanges that recognise data by its being non-zero (weight_quant_decode.hip).  The area
+// is zero before the first launch and every launch leaves it zero; whatever else a launch keeps in the workspace
+// (split-K partial sums, a transposed weight) lies behind it and needs no initialisation, so one zero-initialised
+// buffer can be shared by all launches of a stream.
+constexpr size_t kWorkspaceCounterCapacity = 16384;
+constexpr size_t kWorkspaceZoneBytes = (size_t)16 << 20;
+constexpr size_t kWorkspaceZeroBytes = kWorkspaceCounterCapacity + kWorkspaceZoneBytes;
 
 __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
 {

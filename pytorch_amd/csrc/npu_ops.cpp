@@ -171,32 +171,47 @@ std::tuple<Tensor, Tensor, Tensor> dynamic_quant_asym_hip(const Tensor &input, c
     return {y, scale, offset};
 }
 
-// The split-K reductions of the matmul kernels count arrivals in their workspace: the counters must
-// be zero before a launch and the kernels leave them zero.  One zero-initialised buffer per
-// (device, stream) is kept and reused; launches on one stream are ordered, so they never overlap.
-// Lifetime rules, because a captured HIP graph keeps the pointer it was recorded with:
-//   * a buffer that is superseded by a larger one is never released (it stays alive, zeroed, until the process
-//     ends), so a graph recorded earlier replays on valid, quiescent memory;
-//   * nothing is allocated or filled while the stream is capturing: a fill recorded into a graph is not executed
-//     now, and its buffer would belong to the graph's private pool.  The caller gets an error that says what to do
-//     (run the operator once on that stream before the capture begins).
+// The matmul kernels exchange split-K partial sums through a workspace whose leading zero area (arrival counters and
+// the exchange zone, MI355_WORKSPACE_ZERO_BYTES) must be zero before a launch; the kernels leave it zero.  One
+// zero-initialised buffer per (device, stream) is kept and reused; launches on one stream are ordered, so they never
+// overlap.  Lifetime rules, because a captured HIP graph keeps the pointer it was recorded with:
+//   * eager calls: a buffer that is superseded by a larger one is never released (it stays alive, zeroed, until the
+//     process ends), so a graph recorded earlier replays on valid, quiescent memory;
+//   * calls made while the stream is capturing get a buffer of their own per capture (keyed by the capture's id): it
+//     comes from the graph's private memory pool and its zero fill is a node of that graph, so every replay starts
+//     from zeros and the memory lives exactly as long as the graph.  It is never handed to an eager call or to another
+//     capture; the cache drops its reference when it sees the next capture (or an eager call) on that stream, which
+//     returns the block to the pool of the graph that owns it.
 Tensor zeroed_workspace(const Tensor &like, size_t bytes)
 {
+    struct Captured {
+        unsigned long long id = 0;
+        Tensor ws;
+    };
     static std::mutex mu;
     static std::map<std::pair<int, void *>, Tensor> cache;
+    static std::map<std::pair<int, void *>, Captured> capture_cache;
     static std::vector<Tensor> *retired = new std::vector<Tensor>();   // intentionally never freed
     std::lock_guard<std::mutex> lock(mu);
     const auto key = std::make_pair((int)like.device().index(), stream_of(like));
+    const int64_t want = (int64_t)std::max<size_t>(bytes, (size_t)MI355_WORKSPACE_ZERO_BYTES + ((size_t)1 << 20));
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    unsigned long long capture_id = 0;
+    TORCH_CHECK(hipStreamGetCaptureInfo(static_cast<hipStream_t>(key.second), &capturing, &capture_id) == hipSuccess,
+                "hipStreamGetCaptureInfo failed");
+    if (capturing != hipStreamCaptureStatusNone) {
+        Captured &c = capture_cache[key];
+        if (!c.ws.defined() || c.id != capture_id || (size_t)c.ws.numel() < bytes) {
+            c.ws = at::zeros({want}, like.options().dtype(at::kChar));      // the fill is recorded into this capture
+            c.id = capture_id;
+        }
+        return c.ws;
+    }
+    capture_cache.erase(key);
     Tensor &ws = cache[key];
     if (!ws.defined() || (size_t)ws.numel() < bytes) {
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        TORCH_CHECK(hipStreamIsCapturing(static_cast<hipStream_t>(key.second), &capturing) == hipSuccess, "hipStreamIsCapturing failed");
-        TORCH_CHECK(capturing == hipStreamCaptureStatusNone,
-                    "this operator needs a ", bytes, "-byte zero-initialised workspace on this stream, which cannot be "
-                    "allocated while the stream is being captured: call the operator once with this shape (or a larger "
-                    "one) on this stream before the capture begins");
         if (ws.defined()) retired->push_back(ws);
-        ws = at::zeros({(int64_t)std::max<size_t>(bytes, (size_t)1 << 20)}, like.options().dtype(at::kChar));
+        ws = at::zeros({want}, like.options().dtype(at::kChar));
     }
     return ws;
 }

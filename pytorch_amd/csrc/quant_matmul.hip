@@ -710,7 +710,9 @@ struct QmmPlan {
     size_t counter_bytes, partial_bytes, transpose_bytes;
 };
 
-QmmPlan make_qmm_plan(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n)
+// `zero_area`: bytes in front of the scratch part of the workspace (the shared zero area, or just the counters when the
+// workspace is private to this operator)
+QmmPlan make_qmm_plan(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n, size_t zero_area = kWorkspaceZeroBytes)
 {
     QmmPlan pl{};
     pl.tile = choose_tile((int)M, (int)N);
@@ -732,7 +734,7 @@ QmmPlan make_qmm_plan(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ld
     }
     // a contiguous [K,N] weight is transposed into the workspace
     pl.transpose_bytes = tiled_shape && ldb_k != 1 && ldb_n == 1 ? (size_t)N * (size_t)K : 0;
-    pl.counter_bytes = pl.partial_bytes + pl.transpose_bytes > 0 ? kWorkspaceCounterBytes : 0;
+    pl.counter_bytes = pl.partial_bytes + pl.transpose_bytes > 0 ? zero_area : 0;
     return pl;
 }
 
@@ -769,7 +771,7 @@ __global__ __launch_bounds__(256) void trans_quant_param_kernel(const float *__r
 int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale, const uint64_t *qparam,
                      int64_t scale_len, const void *bias, int bias_dtype, void *out, int out_dtype, int64_t M,
                      int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
-                     void *workspace, size_t workspace_bytes, void *stream)
+                     void *workspace, size_t workspace_bytes, void *stream, size_t zero_area = kWorkspaceZeroBytes)
 {
     if (M < 0 || N < 0 || K < 0) return MI355_ERR_BAD_ARGUMENT;
     if (out_dtype != MI355_OUT_BF16 && out_dtype != MI355_OUT_INT32 && out_dtype != MI355_OUT_FP16 && out_dtype != MI355_OUT_INT8)
@@ -794,7 +796,7 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     const int8_t *bt = b;
     int64_t ldbt = ldb_n;
     bool tiled = K >= BK && K % BK == 0 && (lda & 15) == 0 && aligned(a, 16);
-    const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n);
+    const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n, zero_area);
     char *ws = static_cast<char *>(workspace);
     if (tiled && pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes > 0) {
         if (!ws || workspace_bytes < pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes) return MI355_ERR_WORKSPACE;
@@ -933,8 +935,8 @@ int scratch_of_current_device(void **out, hipStream_t s)
     if (!d.ready) {
         void *ptr = nullptr;
         if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return MI355_ERR_LAUNCH;
-        hipLaunchKernelGGL(scratch_clear_kernel, dim3((unsigned)(kWorkspaceCounterBytes / 4 / 256)), dim3(256), 0, s,
-                           static_cast<uint32_t *>(ptr), (int)(kWorkspaceCounterBytes / 4));
+        hipLaunchKernelGGL(scratch_clear_kernel, dim3((unsigned)(kWorkspaceCounterCapacity / 4 / 256)), dim3(256), 0, s,
+                           static_cast<uint32_t *>(ptr), (int)(kWorkspaceCounterCapacity / 4));
         if (check_launch() != MI355_OK) return MI355_ERR_LAUNCH;
         d.ptr = ptr;
         d.ready = true;
@@ -953,7 +955,12 @@ extern "C" int mi355_quant_matmul_noalloc(const int8_t *a, const int8_t *b, cons
 {
     using namespace mi355;
     if (out_dtype == MI355_OUT_INT8) return MI355_ERR_BAD_ARGUMENT;
-    const size_t need = mi355_quant_matmul_workspace(M, N, K, ldb_k, ldb_n);
+    if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff)
+        return run_quant_matmul(a, b, pertoken_scale, scale, nullptr, scale_len, bias, bias_dtype, out, out_dtype, M, N, K, lda,
+                                ldb_k, ldb_n, ldc, nullptr, 0, stream);
+    // the scratch array is private to this operator: the arrival counters are followed directly by the partial sums
+    const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n, kWorkspaceCounterCapacity);
+    const size_t need = pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes;
     if (need > kStaticScratchBytes) return MI355_ERR_WORKSPACE;      // beyond the fixed scratch: use mi355_quant_matmul
     void *ws = nullptr;
     if (need > 0) {
@@ -961,5 +968,5 @@ extern "C" int mi355_quant_matmul_noalloc(const int8_t *a, const int8_t *b, cons
         if (st != MI355_OK) return st;
     }
     return run_quant_matmul(a, b, pertoken_scale, scale, nullptr, scale_len, bias, bias_dtype, out, out_dtype, M, N, K, lda,
-                            ldb_k, ldb_n, ldc, ws, need > 0 ? kStaticScratchBytes : 0, stream);
+                            ldb_k, ldb_n, ldc, ws, need > 0 ? kStaticScratchBytes : 0, stream, kWorkspaceCounterCapacity);
 }

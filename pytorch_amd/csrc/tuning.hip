@@ -40,3 +40,15 @@ extern "C" int mi355_set_tuning(const char *name, int value)
         }
     return MI355_ERR_BAD_ARGUMENT;
 }
+
+// Identifier of the capture `stream` is part of (0 when it is not capturing): lets a host layer keep one workspace per
+// capture without reaching into the HIP runtime itself.
+extern "C" int mi355_stream_capture_id(void *stream, unsigned long long *id)
+{
+    if (!id) return MI355_ERR_BAD_ARGUMENT;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long cid = 0;
+    if (hipStreamGetCaptureInfo(static_cast<hipStream_t>(stream), &status, &cid) != hipSuccess) return MI355_ERR_LAUNCH;
+    *id = status == hipStreamCaptureStatusNone ? 0ull : cid;
+    return MI355_OK;
+}

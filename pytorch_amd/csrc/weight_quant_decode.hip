@@ -1,0 +1,321 @@
+// npu_weight_quant_batchmatmul, decode shapes (at most 16 activation rows) with int4 weights packed along N: the job
+// is one pass over the packed weights, and at these sizes (tens of megabytes) the launch is as much a latency
+// problem as a bandwidth problem.  The kernel is therefore built around three rules:
+//   * every byte a wavefront will ever need is requested in its first instructions (its activations, its antiquant
+//     parameters, its whole weight tile) and consumed in arrival order: there is no barrier, no LDS staging and no
+//     dependent load in front of the arithmetic;
+//   * a wavefront's tile is 128 weight rows x one 128-byte strip (256 columns): the rows of one scale group, so the
+//     per-group fold  out += scale * (P + offset * X)  (see weight_quant_matmul.hip) happens once, after the loop;
+//   * the partial sums of the workgroups that share a strip meet without counters or fences: every workgroup but
+//     the one with the highest index stores its partial with agent-scope write-through stores into a region of the
+//     workspace that is zero between launches, mapping a zero sum to -0.0 so that every stored word is non-zero; the
+//     workgroup with the highest index of the strip (dispatched after the others, so those are running or done)
+//     reads the words back with agent-scope loads until none is zero, adds them in chunk order to its own sum,
+//     writes the output and stores the zeros back.  The critical path after the last weight byte is one store, one
+//     load and the output store; the relaxed agent-scope counter it replaces cost an acknowledged store, an atomic
+//     round trip and a load.  The wait is bounded: after kMaxPolls unanswered polls the workgroup gives up (the
+//     output is then wrong, the launch still ends).
+#include "weight_quant_common.h"
+#include "weight_quant_decode.h"
+
+namespace mi355 {
+namespace {
+
+struct WqDecArgs {
+    const uint16_t *x, *scale, *offset, *bias;
+    const void *w;
+    uint16_t *out;
+    uint32_t *zone;                 // [S-1][M][N] float32 bit patterns, zero between launches
+    int64_t ldx, ldo;
+    uint32_t ldw_bytes, row_bytes;
+    int M, N, K;
+    int group_rows;                 // rows of a scale group (K when per channel)
+    int strips, S;
+};
+
+constexpr int kMaxPolls = 1 << 20;
+constexpr int SC1 = 16;             // cache-policy bit: agent scope
+
+template <int ACT, int QPT>
+__global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
+{
+    constexpr int STEPS = 4;                    // 32-row steps of a wavefront's tile
+    constexpr int NT = 16;                      // MFMA column sets per lane = its 16 consecutive columns
+    constexpr int NBW = 256;                    // columns of a strip
+    // QPT: output quads per thread (rows x 64 quads over 512 threads): 1 up to 8 rows, 2 up to 16
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    // Workgroups are dealt round-robin to the 8 XCDs; the last chunk of a strip has the highest index of the strip.
+    const int xcd_slot = blockIdx.x >> 3;
+    const int strip = (blockIdx.x & 7) + 8 * (xcd_slot / p.S), chunk = xcd_slot % p.S;
+    if (strip >= p.strips) return;
+    const int row0 = (chunk * 8 + wave) * (32 * STEPS);
+    const bool wave_live = row0 < p.K;          // K is a multiple of 128: a wavefront's tile is inside K or wholly outside
+    const int rows_valid = min(16, p.M);
+    const int n0 = strip * NBW;
+
+    const bool lane_ok = (uint32_t)strip * 128u + (uint32_t)c * 8u < p.row_bytes;
+    f32x4 tot[NT];
+    if (wave_live) {
+        // ---- requests: activations, parameters, the whole weight tile
+        const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(p.x, (uint32_t)(((int64_t)(p.M - 1) * p.ldx + p.K) * 2));
+        u32x4 xa[STEPS];
+#pragma unroll
+        for (int s = 0; s < STEPS; s++)
+            xa[s] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, c < p.M ? (uint32_t)((c * (int)p.ldx + 8 * g) * 2) : kOutOfRange,
+                                                          (uint32_t)(row0 + 32 * s) * 2u, 0);
+        const bool has_offset = p.offset != nullptr;
+        const int grp = row0 / p.group_rows;
+        const uint32_t param_bytes = (uint32_t)(p.K / p.group_rows) * (uint32_t)p.N * 2u;
+        const __amdgpu_buffer_rsrc_t rsrc_s = make_rsrc(p.scale, param_bytes);
+        const __amdgpu_buffer_rsrc_t rsrc_o = make_rsrc(has_offset ? p.offset : p.scale, param_bytes);
+        const uint32_t voff_p = lane_ok ? (uint32_t)(n0 + 16 * c) * 2u : kOutOfRange;
+        // A lane needs 64 bytes of parameters (16 scales, 16 offsets).  Lane (c, g) fetches the g-th 16-byte quarter
+        // (g = 0, 1: scales, g = 2, 3: offsets; without offsets rsrc_o aliases the scales and the values are dropped at
+        // the fold) so that the instruction carries no duplicate bytes; the four lanes of a column group exchange the
+        // quarters through the LDS crossbar before the fold.
+        const u32x4 pq = __builtin_amdgcn_raw_buffer_load_b128(g < 2 ? rsrc_s : rsrc_o, voff_p + 16u * (g & 1),
+                                                               (uint32_t)grp * (uint32_t)p.N * 2u, 0);
+        const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(p.w, (uint32_t)((uint64_t)(p.K - 1) * p.ldw_bytes + p.row_bytes));
+        const uint32_t voff_w = lane_ok ? (uint32_t)(8 * g) * p.ldw_bytes + (uint32_t)strip * 128u + (uint32_t)c * 8u : kOutOfRange;
+        u32x2 wq[STEPS][8];
+#pragma unroll
+        for (int s = 0; s < STEPS; s++)
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+                wq[s][t] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, voff_w, (uint32_t)(row0 + 32 * s + t) * p.ldw_bytes, kNonTemporal);
+
+        f32x4 P[NT], X = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < NT; i++) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
+        uint32_t magic;
+        asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "n"(kInt4Magic<ACT>));   // opaque to the optimiser: stays in a VGPR
+
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            // a step's arithmetic stays behind the previous step's: otherwise the compiler gathers the unpacking of
+            // all steps in front of the first MFMA, which then waits for the last load
+            __builtin_amdgcn_sched_barrier(0);
+            uint32_t w0[8], w1[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                w0[t] = wq[s][t].x ^ 0x88888888u;
+                w1[t] = wq[s][t].y ^ 0x88888888u;
+            }
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+#pragma unroll
+                for (int jb = 0; jb < 4; jb++) {
+                    u32x4 b0, b1;
+                    expand_pair<4, ACT>(h ? w1 : w0, jb, magic, b0, b1);
+                    P[h * 8 + 2 * jb] = mfma_act<ACT>(xa[s], b0, P[h * 8 + 2 * jb]);
+                    P[h * 8 + 2 * jb + 1] = mfma_act<ACT>(xa[s], b1, P[h * 8 + 2 * jb + 1]);
+                }
+            }
+            X = mfma_act<ACT>(xa[s], ones, X);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        u32x4 sv[2], ov[2];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            sv[0][i] = (uint32_t)__builtin_amdgcn_ds_bpermute(c * 4, (int)pq[i]);
+            sv[1][i] = (uint32_t)__builtin_amdgcn_ds_bpermute((16 + c) * 4, (int)pq[i]);
+            ov[0][i] = (uint32_t)__builtin_amdgcn_ds_bpermute((32 + c) * 4, (int)pq[i]);
+            ov[1][i] = (uint32_t)__builtin_amdgcn_ds_bpermute((48 + c) * 4, (int)pq[i]);
+        }
+        // ---- the single fold: tot = (scale * mul) * (P' + ((offset - bias) / mul) * X), both rescalings exact
+        constexpr float P_MUL = kImageMul<4, ACT>;
+        constexpr float X_BIAS = kImageBias<4>;
+#pragma unroll
+        for (int i = 0; i < NT; i++) {
+            const uint32_t su = sv[i / 8][(i % 8) / 2], ou = ov[i / 8][(i % 8) / 2];
+            const float sc = ((i & 1) ? act_hi<ACT>(su) : act_lo<ACT>(su)) * P_MUL;
+            const float of = ((has_offset ? ((i & 1) ? act_hi<ACT>(ou) : act_lo<ACT>(ou)) : 0.0f) - X_BIAS) * (1.0f / P_MUL);
+#pragma unroll
+            for (int q = 0; q < 4; q++) tot[i][q] = sc * __builtin_fmaf(of, X[q], P[i][q]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < NT; i++) tot[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // ---- the eight wavefronts' sums meet in LDS: red[wave][row][column]
+    float *red = reinterpret_cast<float *>(lds);
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int row = 4 * g + q;
+        if (row < rows_valid) {
+            float *dst = red + ((size_t)wave * rows_valid + row) * NBW + 16 * c;
+#pragma unroll
+            for (int i = 0; i < NT; i += 4) *reinterpret_cast<f32x4 *>(dst + i) = f32x4{tot[i][q], tot[i + 1][q], tot[i + 2][q], tot[i + 3][q]};
+        }
+    }
+    __syncthreads();
+    f32x4 acc[QPT];
+    uint32_t zoff[QPT];
+    bool live[QPT];
+#pragma unroll
+    for (int j = 0; j < QPT; j++) {
+        const int qd = (int)threadIdx.x + 512 * j;
+        const int row = qd / (NBW / 4), nl = (qd % (NBW / 4)) * 4;
+        live[j] = row < rows_valid && n0 + nl < p.N;            // N is a multiple of 8: a quad is inside or outside
+        zoff[j] = live[j] ? (uint32_t)((row * p.N + n0 + nl) * 4) : kOutOfRange;
+        acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (live[j]) {
+#pragma unroll
+            for (int wv = 0; wv < 8; wv++) acc[j] += *reinterpret_cast<const f32x4 *>(red + ((size_t)wv * rows_valid + row) * NBW + nl);
+        }
+    }
+    if (p.S > 1) {
+        const uint32_t zone_chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
+        const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, zone_chunk_bytes * (uint32_t)(p.S - 1));
+        if (chunk < p.S - 1) {
+#pragma unroll
+            for (int j = 0; j < QPT; j++) {
+                u32x4 bits = __builtin_bit_cast(u32x4, acc[j]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) bits[i] = bits[i] == 0u ? 0x80000000u : bits[i];   // +0 travels as -0: no stored word is zero
+                __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_z, zoff[j], (uint32_t)chunk * zone_chunk_bytes, SC1);   // dead quads: out of range
+            }
+            return;
+        }
+        // the strip's last workgroup collects the other chunks in chunk order; all of a thread's requests go out
+        // before the first answer is looked at
+        constexpr int CB = 4;                   // chunks per batch
+        f32x4 sum[QPT];
+#pragma unroll
+        for (int j = 0; j < QPT; j++) sum[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int c0 = 0; c0 < p.S - 1; c0 += CB) {
+            u32x4 v[QPT][CB];
+#pragma unroll
+            for (int j = 0; j < QPT; j++)
+#pragma unroll
+                for (int i = 0; i < CB; i++)
+                    v[j][i] = live[j] && c0 + i < p.S - 1
+                                  ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[j], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1)
+                                  : u32x4{1u, 1u, 1u, 1u};
+            for (int poll = 0; poll < kMaxPolls; poll++) {
+                bool missing = false;
+#pragma unroll
+                for (int j = 0; j < QPT; j++)
+#pragma unroll
+                    for (int i = 0; i < CB; i++)
+                        if (v[j][i][0] == 0u || v[j][i][1] == 0u || v[j][i][2] == 0u || v[j][i][3] == 0u) {
+                            v[j][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[j], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1);
+                            missing = true;
+                        }
+                if (!missing) break;
+            }
+#pragma unroll
+            for (int i = 0; i < CB; i++)
+#pragma unroll
+                for (int j = 0; j < QPT; j++) {
+                    const f32x4 f = __builtin_bit_cast(f32x4, v[j][i]);
+                    sum[j] += live[j] && c0 + i < p.S - 1 ? f : f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < QPT; j++) acc[j] = sum[j] + acc[j];
+    }
+    const bool out_vec = (p.ldo & 3) == 0 && aligned_dev(p.out, 8);
+#pragma unroll
+    for (int j = 0; j < QPT; j++) {
+        if (!live[j]) continue;
+        const int qd = (int)threadIdx.x + 512 * j;
+        const int row = qd / (NBW / 4), nl = (qd % (NBW / 4)) * 4;
+        f32x4 a = acc[j];
+        if (p.bias) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) a[i] = a[i] + act_1<ACT>(p.bias[n0 + nl + i]);
+        }
+        uint16_t *o = p.out + (int64_t)row * p.ldo + n0 + nl;
+        if (out_vec) {
+            u32x2 pk;
+            pk.x = pack_act2<ACT>(a[0], a[1]);
+            pk.y = pack_act2<ACT>(a[2], a[3]);
+            *reinterpret_cast<u32x2 *>(o) = pk;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] = (uint16_t)pack_act2<ACT>(a[i], 0.0f);
+        }
+    }
+    if (p.S > 1) {
+        // the zone goes back to zero for the next launch; no branch around the stores (a dead quad or chunk gets an
+        // out-of-range offset), so nothing waits for their acknowledgements
+        const uint32_t zone_chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
+        const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, zone_chunk_bytes * (uint32_t)(p.S - 1));
+        for (int c0 = 0; c0 < p.S - 1; c0 += 4) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < QPT; j++)
+                    __builtin_amdgcn_raw_buffer_store_b128(u32x4{0u, 0u, 0u, 0u}, rsrc_z, c0 + i < p.S - 1 ? zoff[j] : kOutOfRange,
+                                                           (uint32_t)(c0 + i) * zone_chunk_bytes, SC1);
+        }
+    }
+}
+
+} // namespace
+
+WqDecodePlan make_wq_decode_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size, int64_t ldw_k, int64_t ldx,
+                                 const void *x, const void *w, const void *scale, const void *offset)
+{
+    WqDecodePlan pl{};
+    const int64_t row_bytes = N / 2, ldw_bytes = ldw_k * 4;
+    const int64_t group = group_size > 0 ? group_size : K;
+    pl.grouped = group_size > 0 && group != K;
+    // a wavefront's 128 rows lie inside one scale group; every offset the kernel forms fits in 32 bits
+    pl.ok = !knob(kKnobWqDecodeOff) && w_bits == 4 && M >= 1 && M <= 16 && K >= 128 && K % 128 == 0 && N % 8 == 0 &&
+            (pl.grouped ? group % 128 == 0 : true) && ldw_bytes >= row_bytes && ldw_bytes % 8 == 0 && ldx % 8 == 0 &&
+            (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 8)) && (scale == nullptr || aligned(scale, 16)) &&
+            (offset == nullptr || aligned(offset, 16)) && (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 31) &&
+            (uint64_t)M * (uint64_t)ldx * 2 < (1ull << 31) && (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31);
+    if (!pl.ok) return pl;
+    pl.mt = 1;
+    pl.strips = (int)((row_bytes + 127) / 128);
+    pl.S = (int)((K + 1023) / 1024);
+    pl.zone_bytes = pl.S > 1 ? (size_t)(pl.S - 1) * (size_t)M * (size_t)N * 4 : 0;
+    if (pl.zone_bytes > kWorkspaceZoneBytes || (uint64_t)pl.strips * pl.S > 0x7fffffffu) pl.ok = false;
+    return pl;
+}
+
+int launch_wq_decode(const WqDecodePlan &plan, const void *x, int act_f16, const void *w, const void *scale, const void *offset,
+                     const void *bias, void *out, int64_t M, int64_t N, int64_t K, int64_t group_size, int64_t ldx, int64_t ldw_k,
+                     int64_t ldo, void *workspace, void *stream)
+{
+    WqDecArgs p{};
+    p.x = static_cast<const uint16_t *>(x);
+    p.w = w;
+    p.scale = static_cast<const uint16_t *>(scale);
+    p.offset = static_cast<const uint16_t *>(offset);
+    p.bias = static_cast<const uint16_t *>(bias);
+    p.out = static_cast<uint16_t *>(out);
+    p.zone = plan.S > 1 ? reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kWorkspaceCounterCapacity) : nullptr;
+    p.ldx = ldx;
+    p.ldo = ldo;
+    p.ldw_bytes = (uint32_t)(ldw_k * 4);
+    p.row_bytes = (uint32_t)(N / 2);
+    p.M = (int)M;
+    p.N = (int)N;
+    p.K = (int)K;
+    p.group_rows = (int)(plan.grouped ? group_size : K);
+    p.strips = plan.strips;
+    p.S = plan.S;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int rows = (int)(M < 16 ? M : 16);
+    const size_t lds_bytes = (size_t)8 * rows * 256 * sizeof(float);
+    auto go = [&](auto kern) {
+        static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (attr_status != hipSuccess) return (int)MI355_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, dim3((unsigned)((plan.strips + 7) / 8 * 8 * plan.S)), dim3(512), lds_bytes, s, p);
+        return check_launch();
+    };
+    if (M <= 8) return act_f16 ? go(wq_decode4_kernel<1, 1>) : go(wq_decode4_kernel<0, 1>);
+    return act_f16 ? go(wq_decode4_kernel<1, 2>) : go(wq_decode4_kernel<0, 2>);
+}
+
+} // namespace mi355
+

@@ -449,7 +449,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     if (const int f = knob(kKnobWqSplit))
         if (f >= 1 && f <= pl.n_units) S = f;
     if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1;
-    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) S = 1;
+    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterCapacity) S = 1;
     // the parameter table of a workgroup's K range must fit in LDS beside the activation chunks and turn-around tiles
     auto lds_need = [&](int s) {
         const int64_t units = (pl.n_units + s - 1) / s;
@@ -468,7 +468,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     if (pl.nw == 4 && pl.mt <= 2 && (pl.n_units + S - 1) / S >= 2 && knob(kKnobWqkKs) != 1) pl.ks = 2;
     pl.lds_bytes = lds_need(S);
     pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
-    pl.counter_bytes = S > 1 ? kWorkspaceCounterBytes : 0;
+    pl.counter_bytes = S > 1 ? kWorkspaceZeroBytes : 0;
     return pl;
 }
 

@@ -39,6 +39,7 @@
 #include "weight_quant_common.h"
 #include "weight_quant_gemm.h"
 #include "weight_quant_kpacked.h"
+#include "weight_quant_decode.h"
 #include <type_traits>
 
 namespace mi355 {
@@ -613,11 +614,11 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
     // wavefront that meets a single group)
     if (w_bits == 4 && pl.mt == 2 && pl.w * pl.ks == 4) pl.accum = true;
     pl.partial_bytes = pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0;
-    if (pl.S > 1 && (size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) {
+    if (pl.S > 1 && (size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterCapacity) {
         pl.fast = false;                              // more tiles than arrival counters
         return pl;
     }
-    pl.counter_bytes = pl.S > 1 ? kWorkspaceCounterBytes : 0;
+    pl.counter_bytes = pl.S > 1 ? kWorkspaceZeroBytes : 0;
     return pl;
 }
 
@@ -686,10 +687,10 @@ WqKmPlan make_kmajor_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, i
     if (const int f = knob(kKnobWqSplit))
         if (f >= 1 && f <= pl.n_units) S = f;
     if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1;
-    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) S = 1;
+    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterCapacity) S = 1;
     pl.S = S;
     pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
-    pl.counter_bytes = S > 1 ? kWorkspaceCounterBytes : 0;
+    pl.counter_bytes = S > 1 ? kWorkspaceZeroBytes : 0;
     pl.lds_bytes = 16 + (size_t)2 * 32768 + 8 * 2 * 2048;   // two activation chunks + the turn-around tiles
     return pl;
 }
@@ -742,6 +743,10 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
                                                 nullptr, nullptr, nullptr, nullptr);
         const size_t gneed = gp.counter_bytes + gp.partial_bytes;
         if (gp.ok && gneed > need) need = gneed;
+    }
+    if (w_bits == 4) {                      // decode kernel: its exchange lives in the zero area
+        const WqDecodePlan dp = make_wq_decode_plan(M, N, K, 4, group_size, N / 8, K, nullptr, nullptr, nullptr, nullptr);
+        if (dp.ok && dp.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
     }
     if (w_bits == 4) {                      // words along K
         const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, K / 8, K, nullptr, nullptr);
@@ -848,6 +853,18 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
         }
     }
     const bool n_major = w_bits == 4 || (ldw_n == 1 && ldw_k >= N);
+    if (w_bits == 4) {
+        // at most 32 rows, words along N: the barrier-free decode kernel
+        const WqDecodePlan dp = make_wq_decode_plan(M, N, K, 4, group_size, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
+        if (dp.ok && aligned(out_bf16, 2) && (!bias || aligned(bias, 2))) {
+            if (dp.S > 1) {
+                if (!workspace || workspace_bytes < kWorkspaceZeroBytes) return MI355_ERR_WORKSPACE;
+                if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+            }
+            return launch_wq_decode(dp, x_bf16, f16 ? 1 : 0, w, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, group_size, ldx,
+                                    ldw_k, ldo, workspace, stream);
+        }
+    }
     // more than 32 rows: the tiled kernel decodes every weight once per 64 or 128 rows
     const WqGemmPlan gp = make_wq_gemm_plan(M, N, K, w_bits, group_size, n_major ? 1 : 0, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
     if (gp.ok && aligned(out_bf16, 2) && (!bias || aligned(bias, 2))) {

@@ -510,7 +510,8 @@ def test_workspace_outlives_growth_after_capture(pa):
     scb = (torch.rand(Nb, generator=g) * 1e-2).cuda()
     small_ws = _capi.lib().mi355_quant_matmul_workspace(M, N, K, 1, K)
     big_ws = _capi.lib().mi355_quant_matmul_workspace(M, Nb, Kb, 1, Kb)
-    assert 0 < small_ws <= (1 << 20) < big_ws, (small_ws, big_ws)      # the second call must outgrow the first buffer
+    floor = _capi.ZERO_AREA_BYTES + (1 << 20)          # the smallest buffer the operator layer allocates
+    assert 0 < small_ws <= floor < big_ws, (small_ws, big_ws)          # the second call must outgrow the first buffer
     small = lambda: pa.npu_quant_matmul(q, w, sc, pertoken_scale=ps, output_dtype=torch.bfloat16)
     big = lambda: pa.npu_quant_matmul(qb, wb, scb, pertoken_scale=ps, output_dtype=torch.bfloat16)
     stream = torch.cuda.Stream()
@@ -531,32 +532,37 @@ def test_workspace_outlives_growth_after_capture(pa):
     torch.cuda.synchronize()
 
 
-def test_capture_without_warmup_is_refused(pa):
-    """A split-K operator whose stream has no workspace yet cannot allocate (and zero) one inside a capture: it raises
-    and says what to do; after one eager call on that stream the same capture works."""
+def test_captures_without_warmup_on_their_stream(pa):
+    """The usual capture idiom warms up on one stream and captures on another (torch.cuda.graph picks its own): a
+    split-K operator then meets a stream without a workspace while capturing.  Every capture gets a workspace of its
+    own from the graph's memory pool, zeroed by a node of that graph; two graphs captured one after the other on the
+    same stream, replayed alternately with eager calls in between, must all reproduce the eager bits."""
     g = torch.Generator().manual_seed(22)
-    M, K, N = 64, 4096, 1024
+    M, K = 64, 4096
     q = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).cuda()
-    w = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).cuda().t()
-    sc = (torch.rand(N, generator=g) * 1e-2).cuda()
-    op = lambda: pa.npu_quant_matmul(q, w, sc, output_dtype=torch.bfloat16)
-    want = op().clone()
+    ops, wants = [], []
+    for N in (256, 1024):
+        w = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).cuda().t()
+        sc = (torch.rand(N, generator=g) * 1e-2).cuda()
+        ops.append(lambda w=w, sc=sc: pa.npu_quant_matmul(q, w, sc, output_dtype=torch.bfloat16))
+        wants.append(ops[-1]().clone())                # eager, default stream: also the one-time kernel set-up
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()                       # fresh stream: no workspace is cached for it
-    graph = torch.cuda.CUDAGraph()
-    with pytest.raises(RuntimeError, match="before the capture begins"):
-        with torch.cuda.graph(graph, stream=stream):
-            op()
-    torch.cuda.synchronize()
-    with torch.cuda.stream(stream):
-        op()
-    stream.synchronize()
-    graph2 = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph2, stream=stream):
-        out = op()
-    graph2.replay()
-    torch.cuda.synchronize()
-    assert torch.equal(out, want)
+    graphs, outs = [], []
+    for op in ops:
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=stream):
+            outs.append(op())
+        graphs.append(gr)
+    for it in range(3):
+        for gr, out, want, op in zip(graphs, outs, wants, ops):
+            out.zero_()
+            gr.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want), f"replay {it} differs"
+            with torch.cuda.stream(stream):
+                assert torch.equal(op(), want)         # eager call on the capture stream: its own workspace
+            torch.cuda.synchronize()
 
 
 def test_c5_mlp_prefill_properties(pa, golden):

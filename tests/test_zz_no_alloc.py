@@ -38,7 +38,8 @@ def test_quant_matmul_noalloc_matches_workspace_entry_point():
         ps = (torch.rand(M, generator=g) * 9e-3 + 1e-3).cuda()
         bias = (torch.randn(N, generator=g) * 0.02).to(torch.bfloat16).cuda()
         need = L.mi355_quant_matmul_workspace(M, N, K, x2.stride(0), x2.stride(1))
-        assert 16384 < need <= (16 << 20) + 16384, need
+        zone = 16 << 20                                  # exchange zone of the shared workspaces, absent from the private scratch
+        assert 16384 + zone < need <= (16 << 20) + 16384 + zone, need
         ws = torch.zeros(need, dtype=torch.int8, device="cuda")
         want = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
         assert _call(L, False, x1, x2, scale, ps, bias, want, ws) == 0
