@@ -25,10 +25,32 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA
 BF16_PEAK_TFLOPS = 2500.0    # dense bf16 MFMA
 CACHE_BYTES = 256 << 20      # Infinity Cache
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter
-# reads for a plain 256 MiB copy (factors 2.00 and 1.00); see profiles/hbm_traffic_pmc_all_kernels.txt
-TRAFFIC_BYTES = {"c1": 25296896, "c2": 106379264, "c3": 245574656, "c4_m8": 35894272, "c4_m128": 102222080,
-                 "aq_int8": 176668672}
+TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic_pmc_all_kernels.txt")
+
+
+def _load_traffic():
+    """HBM bytes per launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the same counter
+    reads for a plain 256 MiB copy).  The figures live in the profile summary, one `TRAFFIC tag=... kernel=...
+    hbm_bytes=...` line per kernel and workload; a tag without a line reports traffic null, so a kernel that was
+    replaced after the profile was taken cannot inherit a stale figure (the line names the kernel it was measured on)."""
+    table = {}
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                if not line.startswith("TRAFFIC "):
+                    continue
+                kv = dict(tok.split("=", 1) for tok in line.split()[1:] if "=" in tok)
+                table[kv["tag"]] = {"hbm_bytes": int(kv["hbm_bytes"]), "kernel": kv.get("kernel", "")}
+    except OSError:
+        pass
+    return table
+
+
+TRAFFIC = _load_traffic()
+
+
+def _traffic(tag):
+    return TRAFFIC[tag]["hbm_bytes"] if tag in TRAFFIC else None
 
 
 def _parse():
@@ -69,11 +91,16 @@ def _event_time_ms(torch, fn, iters):
 def _graph_time_us(torch, calls, reps=20):
     """Capture the list of launches in one HIP graph (removes host launch gaps for microsecond-scale
     kernels), replay it `reps` times between two events and return the average time per launch in us."""
-    for c in calls:      # warm-up: lazy one-time initialisation must not happen during capture
-        c()
+    # warm-up on the stream that will capture: one-time initialisation and the per-stream workspace must exist before
+    # the capture, so that the graph holds nothing but the launches
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for c in calls:
+            c()
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
+    with torch.cuda.graph(g, stream=side):
         for c in calls:
             c()
     g.replay()
@@ -160,6 +187,12 @@ def main():
         _pmc_pass(torch, pa, workloads, dev)
         return
 
+    # nominal engine clock from the runtime, and the clock the chip holds while all matrix cores are busy
+    from pytorch_amd import _capi
+    clock_mhz = _capi.device_info()[0]
+    _capi.sustained_mfma_clock_mhz(iters=2000)       # warm-up
+    sustained_mhz = round(_capi.sustained_mfma_clock_mhz(), 1)
+
     # ------------------------------------------------------------------ headline: C2 quant_matmul
     M, K, N = 1024, 4096, 11008
     d0 = workloads.quant_matmul_inputs(seed=0, M=M, K=K, N=N, weight_nk=True, bias=True)
@@ -183,6 +216,9 @@ def main():
         state["i"] += 1
         state["out"] = pa.npu_quant_matmul(x1, w, sc, pertoken_scale=ps, bias=bias, output_dtype=torch.bfloat16)
 
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        step()                                       # one-time set-up on the stream that captures the timed steps
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -192,7 +228,7 @@ def main():
     graph = None
     if not args.eager:
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with torch.cuda.graph(graph, stream=side):
             for _ in range(args.steps):
                 step()
         graph.replay()                               # untimed: first replay of a new graph
@@ -255,10 +291,13 @@ def main():
                                "(stored [N,K], passed as transposed view), pertoken_scale f32[1024], scale f32[11008], "
                                "bias bf16[11008], out bf16[1024,11008]",
                    "rotating_sets": nsets, "launch": "eager" if args.eager else "one captured graph of the timed steps", "device": props.name, "compute_units": props.multi_processor_count,
-                   "clock_mhz": getattr(props, "clock_rate", 0) // 1000},
+                   "clock_mhz": clock_mhz, "sustained_mfma_clock_mhz": sustained_mhz},
         "roofline": {"bound": "mfma", "achieved": round(achieved_tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": round(achieved_tops / INT8_PEAK_TOPS, 4), "traffic": TRAFFIC_BYTES["c2"],
-                     "kernel": "qmm_kernel", "launch_us": round(kern_ms * 1e3, 3)},
+                     "frac": round(achieved_tops / INT8_PEAK_TOPS, 4), "traffic": _traffic("c2"),
+                     "kernel": "qmm_kernel", "launch_us": round(kern_ms * 1e3, 3),
+                     "peak_at_sustained_clock": round(INT8_PEAK_TOPS * sustained_mhz / 2400.0, 1) if sustained_mhz else None,
+                     "frac_at_sustained_clock": round(achieved_tops / (INT8_PEAK_TOPS * sustained_mhz / 2400.0), 4)
+                     if sustained_mhz else None},
         "cpu_baseline": cpu_baseline,
         "parity": parity,
     }
@@ -277,6 +316,31 @@ def main():
                           "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic}}
         e.update(extra)
         return e
+
+    def wq_gate(entry, d, out, group_size, flops):
+        """Oracle leg of a weight-only configuration (untimed): the bf16 gate on every output element and the CPU
+        baseline (the oracle's own float32 evaluation of the golden formula, timed on the host cores)."""
+        if args.skip_cpu:
+            return
+        from oracle import golden
+        from pytorch_amd.testing import bf16_gate
+        c0 = time.perf_counter()
+        _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
+                                             _bits(d["antiquant_offset"]), group_size=group_size)
+        c1 = time.perf_counter()
+        try:
+            st = bf16_gate(out, torch.from_numpy(gold))
+            entry["parity_bf16_gate"] = True
+        except AssertionError as exc:
+            entry["parity_bf16_gate"] = False
+            entry["parity_error"] = str(exc)[:300]
+            st = None
+        if st:
+            entry["within_1ulp_strict"] = round(st["within_1ulp_strict"], 6)
+            entry["bit_identical"] = round(st["bit_identical"], 6)
+            entry["max_ulp"] = st["max_ulp"]
+        entry["cpu_baseline"] = {"value": round(flops / (c1 - c0) / 1e9, 2), "unit": "GFLOP/s", "cores": golden.get_threads(),
+                                 "kind": "port", "sample": f"the full configuration, one pass of the oracle, {c1 - c0:.2f} s"}
 
     if want("c2kn"):
         # same problem with the weight contiguous as [K,N] (transposed into the workspace first)
@@ -302,7 +366,7 @@ def main():
         keep = []
         calls = [(lambda x=x: keep.append(pa.npu_dynamic_quant(x))) for x in xs] * 2
         us = _graph_time_us(torch, calls)
-        e = hbm_entry("c1 dynamic_quant bf16[2048,4096] (rotating, > Infinity Cache)", nb, us, TRAFFIC_BYTES["c1"])
+        e = hbm_entry("c1 dynamic_quant bf16[2048,4096] (rotating, > Infinity Cache)", nb, us, _traffic("c1"))
         keep.clear()
         calls = [(lambda: keep.append(pa.npu_dynamic_quant(xs[0])))] * 8
         e["cache_hot_us"] = round(_graph_time_us(torch, calls), 3)
@@ -340,9 +404,10 @@ def main():
         keep = []
         calls = [(lambda w=w: keep.append(pa.npu_weight_quant_batchmatmul(x, w, s3, o3))) for w in ws] * 4
         us = _graph_time_us(torch, calls, reps=10)
-        others.append(hbm_entry("c3 W8A16 x bf16[16,8192] . int8[8192,28672] (weight contiguous [K,N])", nb, us,
-                                TRAFFIC_BYTES["c3"],
-                                tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2)))
+        e = hbm_entry("c3 W8A16 x bf16[16,8192] . int8[8192,28672] (weight contiguous [K,N])", nb, us,
+                      _traffic("c3"), tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2))
+        wq_gate(e, d3, pa.npu_weight_quant_batchmatmul(x, ws[0], s3, o3), 0, 2.0 * Mx * Kx * Nx)
+        others.append(e)
         del ws, keep
         # the layout torch_npu's LinearWeightQuant passes: weight stored [N, K], given as its transposed view
         ws = [torch.randint(-127, 128, (Nx, Kx), generator=gen, dtype=torch.int8, device=dev).t() for _ in range(2)]
@@ -367,8 +432,9 @@ def main():
                      for w in ws] * 2
             us = _graph_time_us(torch, calls)
             e = hbm_entry(f"c4 W4A16 g128 x bf16[{Mx},4096] . int4[4096,14336]", nb, us,
-                          TRAFFIC_BYTES["c4_m8"] if Mx == 8 else TRAFFIC_BYTES["c4_m128"] if Mx == 128 else None,
+                          _traffic(f"c4_m{Mx}"),
                           tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2))
+            wq_gate(e, d4, pa.npu_weight_quant_batchmatmul(x, ws[0], s4, o4, None, None, None, 128), 128, 2.0 * Mx * Kx * Nx)
             if Mx == 128:
                 tf = 2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12
                 e["roofline_mfma"] = {"bound": "mfma", "achieved": round(tf, 1), "peak": BF16_PEAK_TFLOPS,
@@ -430,37 +496,75 @@ def main():
         for Mx in (64, 2048):
             d5 = workloads.mlp_inputs(seed=0, M=Mx, hidden=H, inter=I)
             x = d5["x"].to(dev)
-            wgu, wd = d5["w_gate_up"].to(dev).t(), d5["w_down"].to(dev).t()
             sgu, sd = d5["scale_gate_up"].to(dev), d5["scale_down"].to(dev)
+            # weight sets: 176 MB each; two sets exceed the 256 MB Infinity Cache, so alternating them keeps every
+            # replay on weights that are not cache-resident (set 0 is the seeded one the oracle checks)
+            wsets = [(d5["w_gate_up"].to(dev).t(), d5["w_down"].to(dev).t())]
+            wsets.append((torch.randint(-127, 128, (2 * I, H), generator=gen, dtype=torch.int8, device=dev).t(),
+                          torch.randint(-127, 128, (H, I), generator=gen, dtype=torch.int8, device=dev).t()))
 
-            def mlp():
+            def mlp(wgu, wd, stages=False):
                 xq, xsc = pa.npu_dynamic_quant(x)
                 gu = pa.npu_quant_matmul(xq, wgu, sgu, pertoken_scale=xsc, output_dtype=torch.bfloat16)
                 act = pa.npu_swiglu(gu)
                 aq, asc = pa.npu_dynamic_quant(act)
-                return pa.npu_quant_matmul(aq, wd, sd, pertoken_scale=asc, output_dtype=torch.bfloat16)
+                out = pa.npu_quant_matmul(aq, wd, sd, pertoken_scale=asc, output_dtype=torch.bfloat16)
+                return (xq, xsc, gu, act, aq, asc, out) if stages else out
 
-            def mlp_fused():
+            def mlp_fused(wgu, wd):
                 xq, xsc = pa.npu_dynamic_quant(x)
                 gu = pa.npu_quant_matmul(xq, wgu, sgu, pertoken_scale=xsc, output_dtype=torch.bfloat16)
                 aq, asc = pa.npu_swiglu_quant(gu, activate_left=True, quant_mode=1)
                 return pa.npu_quant_matmul(aq, wd, sd, pertoken_scale=asc, output_dtype=torch.bfloat16)
 
-            same = bool(torch.equal(mlp(), mlp_fused()))
+            same = bool(torch.equal(mlp(*wsets[0]), mlp_fused(*wsets[0])))
             mops = 2.0 * Mx * H * 2 * I + 2.0 * Mx * I * H
             wbytes = H * 2 * I + I * H
+            # algorithmic bytes of the fused chain: weights, activations in and out of every stage, scales
+            abytes = wbytes + Mx * (H * 2 + H + 4) + Mx * (H + 2 * I * 2) + Mx * (2 * I * 2 + I + 4) + Mx * (I + H * 2) + (2 * I + H) * 4
+            gate, cpu = {}, None
+            if not args.skip_cpu and Mx == 64:
+                # stage-wise gate: every GPU stage against the oracle applied to that stage's actual GPU input
+                from oracle import golden
+                xq, xsc, gu, act, aq, asc, out = mlp(*wsets[0], stages=True)
+                c0 = time.perf_counter()
+                yg, sg = golden.dynamic_quant(_bits(d5["x"]))
+                gate["dynamic_quant_1_bit_exact"] = bool(np.array_equal(xq.cpu().numpy(), yg) and np.array_equal(xsc.cpu().numpy(), sg))
+                want_gu, _ = golden.quant_matmul(xq.cpu().numpy(), d5["w_gate_up"].t().numpy(), d5["scale_gate_up"].numpy(), xsc.cpu().numpy())
+                gate["gate_up_bit_exact"] = bool(np.array_equal(_bits(gu), want_gu))
+                dist = golden.bf16_ulp_distance(_bits(act), golden.swiglu(_bits(gu)))
+                gate["swiglu_within_1ulp"] = bool(dist.max() <= 1)
+                gate["swiglu_bit_identical_frac"] = round(float((dist == 0).mean()), 6)
+                yg2, sg2 = golden.dynamic_quant(_bits(act))
+                gate["dynamic_quant_2_bit_exact"] = bool(np.array_equal(aq.cpu().numpy(), yg2) and np.array_equal(asc.cpu().numpy(), sg2))
+                want_out, _ = golden.quant_matmul(aq.cpu().numpy(), d5["w_down"].t().numpy(), d5["scale_down"].numpy(), asc.cpu().numpy())
+                gate["down_bit_exact"] = bool(np.array_equal(_bits(out), want_out))
+                c1 = time.perf_counter()
+                cpu = {"value": round(mops / (c1 - c0) / 1e12, 5), "unit": "TOP/s", "cores": golden.get_threads(), "kind": "port",
+                       "sample": f"one pass of the oracle over the five stages at M=64 (stage-wise, on the GPU's stage inputs), {c1 - c0:.2f} s"}
             for fn, label in ((mlp, "5 kernels"), (mlp_fused, "4 kernels, fused SwiGLU + dynamic_quant")):
                 keep = []
-                us = _graph_time_us(torch, [lambda: keep.append(fn())] * 4, reps=10)
-                e = {"name": f"c5 Llama-3-8B-shaped W8A8 MLP, M={Mx} ({label}, cache-resident weights)",
-                     "chain_us": round(us, 2), "int8_tops": round(mops / (us * 1e-6) / 1e12, 2),
-                     "weight_gbs": round(wbytes / (us * 1e-6) / 1e9, 1),
-                     "frac_int8_peak": round(mops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4),
-                     "frac_hbm_peak_weights_only": round(wbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+                calls = [(lambda w=w: keep.append(fn(*w))) for w in wsets] * 2
+                us = _graph_time_us(torch, calls, reps=10)
+                keep.clear()
+                hot = _graph_time_us(torch, [lambda: keep.append(fn(*wsets[0]))] * 4, reps=10)
+                e = {"name": f"c5 Llama-3-8B-shaped W8A8 MLP, M={Mx} ({label}; two weight sets alternate, 352 MB > Infinity Cache)",
+                     "chain_us": round(us, 2), "chain_us_cache_resident_weights": round(hot, 2),
+                     "int8_tops": round(mops / (us * 1e-6) / 1e12, 2),
+                     "roofline": ({"bound": "hbm", "achieved": round(abytes / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "frac": round(abytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None} if Mx == 64 else
+                                  {"bound": "mfma", "achieved": round(mops / (us * 1e-6) / 1e12, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                                   "frac": round(mops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None}),
+                     "algorithmic_bytes": int(abytes)}
                 if fn is mlp_fused:
                     e["bit_identical_to_5_kernel_chain"] = same
+                elif gate:
+                    e["parity_stagewise"] = gate
+                    e["parity_all_stages"] = bool(all(v for k, v in gate.items() if k != "swiglu_bit_identical_frac"))
+                    e["cpu_baseline"] = cpu
                 others.append(e)
                 del keep
+            del wsets
 
     if want("aq"):
         # standalone antiquantisation of a decoder-MLP-sized weight: int8 / packed int4 [4096, 14336] -> bf16
@@ -479,7 +583,7 @@ def main():
             calls = [(lambda x=x: keep.append(pa.npu_anti_quant(x, sc_f, offset=of_f, dst_dtype=torch.bfloat16))) for x in xs] * 2
             us = _graph_time_us(torch, calls)
             others.append(hbm_entry(f"npu_anti_quant int{bits}[4096,14336] -> bf16 (per-column float32 scale and offset)", nb, us,
-                                    TRAFFIC_BYTES["aq_int8"] if bits == 8 else None))
+                                    _traffic("aq_int8") if bits == 8 else None))
             del xs, keep
 
     if want("qz"):

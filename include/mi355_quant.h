@@ -321,6 +321,17 @@ int mi355_set_tuning(const char *name, int value);
  */
 int mi355_stream_capture_id(void *stream, unsigned long long *id);
 
+/*
+ * Measurement aid, no counterpart in the reference: keeps `workgroups` x 8 wavefronts issuing dependent int8 MFMAs for
+ * `iters` x 4 instructions each and writes, per workgroup, the elapsed shader-clock cycles and the elapsed ticks of
+ * the constant 100 MHz counter into out[2*w], out[2*w+1]: cycles / ticks x 100 is the clock in MHz that the chip
+ * sustains under matrix-core load.
+ */
+int mi355_probe_clock(unsigned long long *out, int workgroups, int iters, void *stream);
+
+/* Peak engine clock (kHz) and compute-unit count of the current device from the HIP runtime; either pointer may be NULL. */
+int mi355_device_info(int *clock_khz, int *compute_units);
+
 #ifdef __cplusplus
 }
 #endif

@@ -19,7 +19,7 @@ EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quan
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
            "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth", "mi355_set_tuning",
-           "mi355_quant_matmul_noalloc", "mi355_stream_capture_id")
+           "mi355_quant_matmul_noalloc", "mi355_stream_capture_id", "mi355_probe_clock", "mi355_device_info")
 
 _lib = None
 
@@ -56,10 +56,28 @@ def lib() -> ctypes.CDLL:
         L.mi355_quant_matmul_qparam.argtypes = [vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
         L.mi355_quantize.argtypes = [vp, i32, vp, i64, vp, i32, i64, vp, i32, i64, i64, i64, i32, vp]
         L.mi355_set_tuning.argtypes = [ctypes.c_char_p, i32]
+        L.mi355_probe_clock.argtypes = [vp, i32, i32, vp]
+        L.mi355_device_info.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.mi355_stream_capture_id.argtypes = [vp, ctypes.POINTER(ctypes.c_ulonglong)]
         L.mi355_quant_matmul_noalloc.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp]
         _lib = L
     return _lib
+
+
+def device_info():
+    """(peak engine clock in MHz, compute units) of the current device."""
+    khz, cus = ctypes.c_int(0), ctypes.c_int(0)
+    _check(lib().mi355_device_info(ctypes.byref(khz), ctypes.byref(cus)), "mi355_device_info")
+    return khz.value // 1000, cus.value
+
+
+def sustained_mfma_clock_mhz(workgroups: int = 256, iters: int = 20000) -> float:
+    """Shader clock (MHz) the GPU holds while every SIMD issues int8 MFMAs back to back (median over the workgroups)."""
+    out = torch.zeros((workgroups, 2), dtype=torch.int64, device="cuda")
+    _check(lib().mi355_probe_clock(_ptr(out), workgroups, iters, _stream()), "mi355_probe_clock")
+    torch.cuda.synchronize()
+    o = out.cpu().double()
+    return float((o[:, 0] / o[:, 1].clamp(min=1) * 100.0).median())
 
 
 def set_tuning(name: str, value: int) -> None:
@@ -159,14 +177,18 @@ ZERO_AREA_BYTES = (16 << 20) + 16384     # MI355_WORKSPACE_ZERO_BYTES
 
 def _wq_workspace(device, nbytes: int):
     """Zero-initialised workspace reused across calls on one stream: the kernels need its leading zero area to start
-    at zero and leave it zero.  Calls made while the stream is capturing get one workspace per capture (allocated from
-    the graph's pool, its zero fill recorded into the graph); eager calls never see those."""
+    at zero and leave it zero.  A call made while the stream is capturing uses the stream's eager workspace when one
+    exists (the operator ran on this stream before the capture); otherwise the capture gets a workspace of its own
+    (allocated from the graph's pool, its zero fill recorded into the graph), which eager calls never see."""
     stream = torch.cuda.current_stream().cuda_stream
     key = (device.index, stream)
     want = max(nbytes, ZERO_AREA_BYTES + (1 << 20))
     cid = ctypes.c_ulonglong(0)
     _check(lib().mi355_stream_capture_id(ctypes.c_void_p(stream), ctypes.byref(cid)), "mi355_stream_capture_id")
     if cid.value:
+        ws = _wq_workspaces.get(key)
+        if ws is not None and ws.numel() >= nbytes:
+            return ws
         ent = _wq_capture_workspaces.get(key)
         if ent is None or ent[0] != cid.value or ent[1].numel() < nbytes:
             ent = (cid.value, torch.zeros(want, dtype=torch.int8, device=device))

@@ -1,0 +1,50 @@
+// Sustained shader clock under matrix-core load.  The published MFMA peaks assume the peak engine clock; a launch that
+// keeps the matrix cores busy runs below it, so a roofline fraction is easier to read next to the clock the silicon
+// actually held.  The probe keeps every SIMD issuing dependent int8 MFMAs for a few tens of microseconds and records
+// both the shader-clock counter and the constant 100 MHz counter around the loop.
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+typedef int i32x4v __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(512) void clock_probe_kernel(unsigned long long *out, int iters)
+{
+    i32x4v acc[4] = {{0, 0, 0, 0}, {1, 1, 1, 1}, {2, 2, 2, 2}, {3, 3, 3, 3}};
+    const i32x4v a = {(int)threadIdx.x, 1, 2, 3}, b = {4, 5, 6, (int)blockIdx.x};
+    const unsigned long long c0 = __builtin_readcyclecounter(), r0 = wall_clock64();
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[j], 0, 0, 0);
+    }
+    const unsigned long long c1 = __builtin_readcyclecounter(), r1 = wall_clock64();
+    int sink = acc[0][0] ^ acc[1][1] ^ acc[2][2] ^ acc[3][3];
+    if (threadIdx.x == 0) {
+        out[blockIdx.x * 2] = c1 - c0;
+        out[blockIdx.x * 2 + 1] = (r1 - r0) + (sink == 0x7fffffff ? 1 : 0);
+    }
+}
+
+} // namespace
+} // namespace mi355
+
+// out: [workgroups][2] 64-bit counts (shader-clock cycles, ticks of the constant 100 MHz counter) per workgroup.
+extern "C" int mi355_probe_clock(unsigned long long *out, int workgroups, int iters, void *stream)
+{
+    using namespace mi355;
+    if (!out || workgroups <= 0 || iters <= 0) return MI355_ERR_BAD_ARGUMENT;
+    hipLaunchKernelGGL(clock_probe_kernel, dim3((unsigned)workgroups), dim3(512), 0, static_cast<hipStream_t>(stream), out, iters);
+    return check_launch();
+}
+
+// Peak engine clock in kHz and number of compute units of the current device, as the HIP runtime reports them.
+extern "C" int mi355_device_info(int *clock_khz, int *compute_units)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MI355_ERR_LAUNCH;
+    if (clock_khz && hipDeviceGetAttribute(clock_khz, hipDeviceAttributeClockRate, dev) != hipSuccess) return MI355_ERR_LAUNCH;
+    if (compute_units && hipDeviceGetAttribute(compute_units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        return MI355_ERR_LAUNCH;
+    return MI355_OK;
+}

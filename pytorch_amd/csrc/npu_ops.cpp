@@ -177,11 +177,13 @@ std::tuple<Tensor, Tensor, Tensor> dynamic_quant_asym_hip(const Tensor &input, c
 // overlap.  Lifetime rules, because a captured HIP graph keeps the pointer it was recorded with:
 //   * eager calls: a buffer that is superseded by a larger one is never released (it stays alive, zeroed, until the
 //     process ends), so a graph recorded earlier replays on valid, quiescent memory;
-//   * calls made while the stream is capturing get a buffer of their own per capture (keyed by the capture's id): it
-//     comes from the graph's private memory pool and its zero fill is a node of that graph, so every replay starts
-//     from zeros and the memory lives exactly as long as the graph.  It is never handed to an eager call or to another
-//     capture; the cache drops its reference when it sees the next capture (or an eager call) on that stream, which
-//     returns the block to the pool of the graph that owns it.
+//   * a call made while the stream is capturing uses the stream's eager buffer when there is one that is large enough
+//     (the operator was run on this stream before the capture: nothing is allocated or filled inside the graph);
+//     otherwise the capture gets a buffer of its own (keyed by the capture's id): it comes from the graph's private
+//     memory pool and its zero fill is a node of that graph, so every replay starts from zeros and the memory lives
+//     exactly as long as the graph.  Such a buffer is never handed to an eager call or to another capture; the cache
+//     drops its reference when it sees the next capture (or an eager call) on that stream, which returns the block
+//     to the pool of the graph that owns it.
 Tensor zeroed_workspace(const Tensor &like, size_t bytes)
 {
     struct Captured {
@@ -200,6 +202,8 @@ Tensor zeroed_workspace(const Tensor &like, size_t bytes)
     TORCH_CHECK(hipStreamGetCaptureInfo(static_cast<hipStream_t>(key.second), &capturing, &capture_id) == hipSuccess,
                 "hipStreamGetCaptureInfo failed");
     if (capturing != hipStreamCaptureStatusNone) {
+        const auto eager = cache.find(key);
+        if (eager != cache.end() && eager->second.defined() && (size_t)eager->second.numel() >= bytes) return eager->second;
         Captured &c = capture_cache[key];
         if (!c.ws.defined() || c.id != capture_id || (size_t)c.ws.numel() < bytes) {
             c.ws = at::zeros({want}, like.options().dtype(at::kChar));      // the fill is recorded into this capture
