@@ -160,6 +160,15 @@ int mi355_quant_matmul_qparam(const int8_t *a, const int8_t *b, const uint64_t *
                               void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * One-time weight pre-layout for mi355_quant_matmul: src int8 [K,N] (rows ld_src bytes apart) -> dst int8 [N,K]
+ * contiguous, the K-major storage the GEMM reads directly (ldb_k = 1, ldb_n = K); a [K,N] weight passed as it is gets
+ * transposed into the workspace on every call instead.  The counterpart of casting a weight to the device's private
+ * format before deployment (the reference's modules rely on such a cast, e.g.
+ * torch_npu/optim/npu_fused_optim_base.py:49); weights are static, so this runs once per weight.
+ */
+int mi355_transpose_int8(const int8_t *src, int8_t *dst, int64_t K, int64_t N, int64_t ld_src, void *stream);
+
+/*
  * mi355_quant_matmul without a workspace argument and without any allocation.  It has no counterpart in the
  * reference (there the adapter allocates a workspace per call, torch_npu/csrc/framework/utils/OpPreparation.h:130-132);
  * it exists for callers that cannot allocate or carry a workspace: code under HIP graph capture, tight serving loops,

@@ -19,7 +19,7 @@ EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quan
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
            "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth", "mi355_set_tuning",
-           "mi355_quant_matmul_noalloc", "mi355_stream_capture_id", "mi355_probe_clock", "mi355_device_info")
+           "mi355_quant_matmul_noalloc", "mi355_stream_capture_id", "mi355_probe_clock", "mi355_device_info", "mi355_transpose_int8")
 
 _lib = None
 
@@ -57,6 +57,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_quantize.argtypes = [vp, i32, vp, i64, vp, i32, i64, vp, i32, i64, i64, i64, i32, vp]
         L.mi355_set_tuning.argtypes = [ctypes.c_char_p, i32]
         L.mi355_probe_clock.argtypes = [vp, i32, i32, vp]
+        L.mi355_transpose_int8.argtypes = [vp, vp, i64, i64, i64, vp]
         L.mi355_device_info.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.mi355_stream_capture_id.argtypes = [vp, ctypes.POINTER(ctypes.c_ulonglong)]
         L.mi355_quant_matmul_noalloc.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp]
@@ -138,6 +139,16 @@ def quant_matmul(x1, x2, scale, pertoken_scale=None, bias=None, out_dtype=torch.
                                   M, N, K, x1.stride(0), x2.stride(0), x2.stride(1), out.stride(0), _ptr(workspace),
                                   0 if workspace is None else workspace.numel(), _stream())
     _check(st, "mi355_quant_matmul")
+    return out
+
+
+def transpose_int8(w: torch.Tensor) -> torch.Tensor:
+    """w int8 [K, N] with unit column stride -> new int8 [N, K] contiguous (one transposing pass on the GPU)."""
+    _need_gpu(w)
+    assert w.dtype == torch.int8 and w.dim() == 2 and (w.numel() == 0 or w.stride(1) == 1)
+    K, N = w.shape
+    out = torch.empty((N, K), dtype=torch.int8, device=w.device)
+    _check(lib().mi355_transpose_int8(_ptr(w), _ptr(out), K, N, w.stride(0) if K > 1 else max(N, 1), _stream()), "mi355_transpose_int8")
     return out
 
 

@@ -970,3 +970,22 @@ extern "C" int mi355_quant_matmul_noalloc(const int8_t *a, const int8_t *b, cons
     return run_quant_matmul(a, b, pertoken_scale, scale, nullptr, scale_len, bias, bias_dtype, out, out_dtype, M, N, K, lda,
                             ldb_k, ldb_n, ldc, ws, need > 0 ? kStaticScratchBytes : 0, stream, kWorkspaceCounterCapacity);
 }
+
+// One-time weight pre-layout for npu_quant_matmul: a contiguous [K,N] int8 weight is rewritten K-major ([N,K] storage),
+// the layout the GEMM consumes without its per-call transposing pre-pass.
+extern "C" int mi355_transpose_int8(const int8_t *src, int8_t *dst, int64_t K, int64_t N, int64_t ld_src, void *stream)
+{
+    using namespace mi355;
+    if (K < 0 || N < 0 || ld_src < N) return MI355_ERR_BAD_ARGUMENT;
+    if (K == 0 || N == 0) return MI355_OK;
+    if (!src || !dst) return MI355_ERR_BAD_ARGUMENT;
+    if (K > 0x7fffffff || N > 0x7fffffff) return MI355_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if ((N & 15) == 0 && (K & 15) == 0 && (ld_src & 15) == 0 && aligned(src, 16) && aligned(dst, 16))
+        hipLaunchKernelGGL(transpose_i8_wide_kernel, dim3((unsigned)((N + 127) / 128), (unsigned)((K + 127) / 128)), dim3(256), 0, s,
+                           src, dst, (int)K, (int)N, ld_src);
+    else
+        hipLaunchKernelGGL(transpose_i8_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64)), dim3(256), 0, s, src, dst,
+                           (int)K, (int)N, ld_src);
+    return check_launch();
+}

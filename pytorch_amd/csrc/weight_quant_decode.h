@@ -1,4 +1,4 @@
-// Internal interface of the decode-shaped kernel for int4 weights packed along N (at most 16 activation rows); not part
+// Internal interface of the decode-shaped kernel for int4 weights packed along N (at most 32 activation rows); not part
 // of the C ABI.
 #pragma once
 #include <stddef.h>
@@ -8,7 +8,7 @@ namespace mi355 {
 
 struct WqDecodePlan {
     bool ok;                 // the kernel accepts this problem
-    int mt;                  // m tiles (16 rows): always 1
+    int mt;                  // m tiles (16 rows): 1 or 2
     int strips;              // 128-byte strips of a weight row (256 columns each)
     int S;                   // workgroups that share a strip, 1024 weight rows each
     bool grouped;

@@ -1,4 +1,4 @@
-// npu_weight_quant_batchmatmul, decode shapes (at most 16 activation rows) with int4 weights packed along N: the job
+// npu_weight_quant_batchmatmul, decode shapes (at most 32 activation rows) with int4 weights packed along N: the job
 // is one pass over the packed weights, and at these sizes (tens of megabytes) the launch is as much a latency
 // problem as a bandwidth problem.  The kernel is therefore built around three rules:
 //   * every byte a wavefront will ever need is requested in its first instructions (its activations, its antiquant
@@ -36,13 +36,16 @@ struct WqDecArgs {
 constexpr int kMaxPolls = 1 << 20;
 constexpr int SC1 = 16;             // cache-policy bit: agent scope
 
-template <int ACT, int QPT>
+// MT: m tiles of 16 activation rows (1 or 2); QPT: output quads per thread and m tile (rows x 64 quads over 512 threads):
+// 1 up to 8 rows, 2 up to 16.  With two m tiles the accumulators take half of the register file, so the weight tile is
+// requested two steps at a time instead of all at once.
+template <int ACT, int MT, int QPT>
 __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
 {
     constexpr int STEPS = 4;                    // 32-row steps of a wavefront's tile
+    constexpr int PFS = MT == 1 ? 4 : 1;        // steps in flight
     constexpr int NT = 16;                      // MFMA column sets per lane = its 16 consecutive columns
     constexpr int NBW = 256;                    // columns of a strip
-    // QPT: output quads per thread (rows x 64 quads over 512 threads): 1 up to 8 rows, 2 up to 16
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -53,19 +56,24 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
     if (strip >= p.strips) return;
     const int row0 = (chunk * 8 + wave) * (32 * STEPS);
     const bool wave_live = row0 < p.K;          // K is a multiple of 128: a wavefront's tile is inside K or wholly outside
-    const int rows_valid = min(16, p.M);
     const int n0 = strip * NBW;
 
     const bool lane_ok = (uint32_t)strip * 128u + (uint32_t)c * 8u < p.row_bytes;
-    f32x4 tot[NT];
+    f32x4 tot[MT][NT];
     if (wave_live) {
-        // ---- requests: activations, parameters, the whole weight tile
+        // ---- requests: activations, parameters, the weight tile
         const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(p.x, (uint32_t)(((int64_t)(p.M - 1) * p.ldx + p.K) * 2));
-        u32x4 xa[STEPS];
+        u32x4 xa[PFS][MT];
+        auto load_x = [&](int slot, int s) {
 #pragma unroll
-        for (int s = 0; s < STEPS; s++)
-            xa[s] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, c < p.M ? (uint32_t)((c * (int)p.ldx + 8 * g) * 2) : kOutOfRange,
-                                                          (uint32_t)(row0 + 32 * s) * 2u, 0);
+            for (int mt = 0; mt < MT; mt++) {
+                const int m = mt * 16 + c;
+                xa[slot][mt] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, m < p.M ? (uint32_t)((m * (int)p.ldx + 8 * g) * 2) : kOutOfRange,
+                                                                     (uint32_t)(row0 + 32 * s) * 2u, 0);
+            }
+        };
+#pragma unroll
+        for (int s = 0; s < PFS; s++) load_x(s, s);
         const bool has_offset = p.offset != nullptr;
         const int grp = row0 / p.group_rows;
         const uint32_t param_bytes = (uint32_t)(p.K / p.group_rows) * (uint32_t)p.N * 2u;
@@ -80,16 +88,23 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
                                                                (uint32_t)grp * (uint32_t)p.N * 2u, 0);
         const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(p.w, (uint32_t)((uint64_t)(p.K - 1) * p.ldw_bytes + p.row_bytes));
         const uint32_t voff_w = lane_ok ? (uint32_t)(8 * g) * p.ldw_bytes + (uint32_t)strip * 128u + (uint32_t)c * 8u : kOutOfRange;
-        u32x2 wq[STEPS][8];
-#pragma unroll
-        for (int s = 0; s < STEPS; s++)
+        u32x2 wq[PFS][8];
+        auto load_step = [&](int slot, int s) {
 #pragma unroll
             for (int t = 0; t < 8; t++)
-                wq[s][t] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, voff_w, (uint32_t)(row0 + 32 * s + t) * p.ldw_bytes, kNonTemporal);
-
-        f32x4 P[NT], X = f32x4{0.f, 0.f, 0.f, 0.f};
+                wq[slot][t] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, voff_w, (uint32_t)(row0 + 32 * s + t) * p.ldw_bytes,
+                                                                   kNonTemporal);
+        };
 #pragma unroll
-        for (int i = 0; i < NT; i++) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < PFS; s++) load_step(s, s);
+
+        f32x4 P[MT][NT], X[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            X[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < NT; i++) P[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
         const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
         uint32_t magic;
         asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "n"(kInt4Magic<ACT>));   // opaque to the optimiser: stays in a VGPR
@@ -99,11 +114,21 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             // a step's arithmetic stays behind the previous step's: otherwise the compiler gathers the unpacking of
             // all steps in front of the first MFMA, which then waits for the last load
             __builtin_amdgcn_sched_barrier(0);
+            const int slot = s % PFS;
             uint32_t w0[8], w1[8];
 #pragma unroll
             for (int t = 0; t < 8; t++) {
-                w0[t] = wq[s][t].x ^ 0x88888888u;
-                w1[t] = wq[s][t].y ^ 0x88888888u;
+                w0[t] = wq[slot][t].x ^ 0x88888888u;
+                w1[t] = wq[slot][t].y ^ 0x88888888u;
+            }
+            u32x4 xs[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) xs[mt] = xa[slot][mt];
+            if (s + PFS < STEPS) {
+                __builtin_amdgcn_sched_barrier(0);
+                load_x(slot, s + PFS);
+                load_step(slot, s + PFS);
+                __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
             for (int h = 0; h < 2; h++) {
@@ -111,11 +136,15 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
                 for (int jb = 0; jb < 4; jb++) {
                     u32x4 b0, b1;
                     expand_pair<4, ACT>(h ? w1 : w0, jb, magic, b0, b1);
-                    P[h * 8 + 2 * jb] = mfma_act<ACT>(xa[s], b0, P[h * 8 + 2 * jb]);
-                    P[h * 8 + 2 * jb + 1] = mfma_act<ACT>(xa[s], b1, P[h * 8 + 2 * jb + 1]);
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        P[mt][h * 8 + 2 * jb] = mfma_act<ACT>(xs[mt], b0, P[mt][h * 8 + 2 * jb]);
+                        P[mt][h * 8 + 2 * jb + 1] = mfma_act<ACT>(xs[mt], b1, P[mt][h * 8 + 2 * jb + 1]);
+                    }
                 }
             }
-            X = mfma_act<ACT>(xa[s], ones, X);
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) X[mt] = mfma_act<ACT>(xs[mt], ones, X[mt]);
         }
         __builtin_amdgcn_sched_barrier(0);
         u32x4 sv[2], ov[2];
@@ -135,76 +164,88 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             const float sc = ((i & 1) ? act_hi<ACT>(su) : act_lo<ACT>(su)) * P_MUL;
             const float of = ((has_offset ? ((i & 1) ? act_hi<ACT>(ou) : act_lo<ACT>(ou)) : 0.0f) - X_BIAS) * (1.0f / P_MUL);
 #pragma unroll
-            for (int q = 0; q < 4; q++) tot[i][q] = sc * __builtin_fmaf(of, X[q], P[i][q]);
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) tot[mt][i][q] = sc * __builtin_fmaf(of, X[mt][q], P[mt][i][q]);
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < NT; i++) tot[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int i = 0; i < NT; i++) tot[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // ---- the eight wavefronts' sums meet in LDS: red[wave][row][column]
+    // ---- the eight wavefronts' sums meet in LDS, one m tile at a time: red[wave][row][column]
     float *red = reinterpret_cast<float *>(lds);
+    constexpr int NQ = MT * QPT;                 // output quads per thread
+    f32x4 acc[NQ];
+    uint32_t zoff[NQ];
+    bool live[NQ];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int row = 4 * g + q;
-        if (row < rows_valid) {
-            float *dst = red + ((size_t)wave * rows_valid + row) * NBW + 16 * c;
+    for (int mt = 0; mt < MT; mt++) {
+        const int rows_mt = min(16, p.M - mt * 16);
+        if (mt > 0) __syncthreads();             // the previous m tile's sums have been read
 #pragma unroll
-            for (int i = 0; i < NT; i += 4) *reinterpret_cast<f32x4 *>(dst + i) = f32x4{tot[i][q], tot[i + 1][q], tot[i + 2][q], tot[i + 3][q]};
+        for (int q = 0; q < 4; q++) {
+            const int row = 4 * g + q;
+            if (row < rows_mt) {
+                float *dst = red + ((size_t)wave * rows_mt + row) * NBW + 16 * c;
+#pragma unroll
+                for (int i = 0; i < NT; i += 4)
+                    *reinterpret_cast<f32x4 *>(dst + i) = f32x4{tot[mt][i][q], tot[mt][i + 1][q], tot[mt][i + 2][q], tot[mt][i + 3][q]};
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < QPT; j++) {
+            const int qd = (int)threadIdx.x + 512 * j;
+            const int row = qd / (NBW / 4), nl = (qd % (NBW / 4)) * 4;
+            const int e = mt * QPT + j;
+            live[e] = row < rows_mt && n0 + nl < p.N;            // N is a multiple of 8: a quad is inside or outside
+            zoff[e] = live[e] ? (uint32_t)(((mt * 16 + row) * p.N + n0 + nl) * 4) : kOutOfRange;
+            acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (live[e]) {
+#pragma unroll
+                for (int wv = 0; wv < 8; wv++) acc[e] += *reinterpret_cast<const f32x4 *>(red + ((size_t)wv * rows_mt + row) * NBW + nl);
+            }
         }
     }
-    __syncthreads();
-    f32x4 acc[QPT];
-    uint32_t zoff[QPT];
-    bool live[QPT];
-#pragma unroll
-    for (int j = 0; j < QPT; j++) {
-        const int qd = (int)threadIdx.x + 512 * j;
-        const int row = qd / (NBW / 4), nl = (qd % (NBW / 4)) * 4;
-        live[j] = row < rows_valid && n0 + nl < p.N;            // N is a multiple of 8: a quad is inside or outside
-        zoff[j] = live[j] ? (uint32_t)((row * p.N + n0 + nl) * 4) : kOutOfRange;
-        acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (live[j]) {
-#pragma unroll
-            for (int wv = 0; wv < 8; wv++) acc[j] += *reinterpret_cast<const f32x4 *>(red + ((size_t)wv * rows_valid + row) * NBW + nl);
-        }
-    }
+    const uint32_t zone_chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
+    const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, p.S > 1 ? zone_chunk_bytes * (uint32_t)(p.S - 1) : 0u);
     if (p.S > 1) {
-        const uint32_t zone_chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
-        const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, zone_chunk_bytes * (uint32_t)(p.S - 1));
         if (chunk < p.S - 1) {
 #pragma unroll
-            for (int j = 0; j < QPT; j++) {
-                u32x4 bits = __builtin_bit_cast(u32x4, acc[j]);
+            for (int e = 0; e < NQ; e++) {
+                u32x4 bits = __builtin_bit_cast(u32x4, acc[e]);
 #pragma unroll
                 for (int i = 0; i < 4; i++) bits[i] = bits[i] == 0u ? 0x80000000u : bits[i];   // +0 travels as -0: no stored word is zero
-                __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_z, zoff[j], (uint32_t)chunk * zone_chunk_bytes, SC1);   // dead quads: out of range
+                __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_z, zoff[e], (uint32_t)chunk * zone_chunk_bytes, SC1);   // dead quads: out of range
             }
             return;
         }
         // the strip's last workgroup collects the other chunks in chunk order; all of a thread's requests go out
         // before the first answer is looked at
-        constexpr int CB = 4;                   // chunks per batch
-        f32x4 sum[QPT];
+        constexpr int CB = NQ <= 2 ? 4 : 3;     // chunks per batch
+        f32x4 sum[NQ];
 #pragma unroll
-        for (int j = 0; j < QPT; j++) sum[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int e = 0; e < NQ; e++) sum[e] = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int c0 = 0; c0 < p.S - 1; c0 += CB) {
-            u32x4 v[QPT][CB];
+            u32x4 v[NQ][CB];
 #pragma unroll
-            for (int j = 0; j < QPT; j++)
+            for (int e = 0; e < NQ; e++)
 #pragma unroll
                 for (int i = 0; i < CB; i++)
-                    v[j][i] = live[j] && c0 + i < p.S - 1
-                                  ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[j], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1)
+                    v[e][i] = live[e] && c0 + i < p.S - 1
+                                  ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[e], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1)
                                   : u32x4{1u, 1u, 1u, 1u};
             for (int poll = 0; poll < kMaxPolls; poll++) {
                 bool missing = false;
 #pragma unroll
-                for (int j = 0; j < QPT; j++)
+                for (int e = 0; e < NQ; e++)
 #pragma unroll
                     for (int i = 0; i < CB; i++)
-                        if (v[j][i][0] == 0u || v[j][i][1] == 0u || v[j][i][2] == 0u || v[j][i][3] == 0u) {
-                            v[j][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[j], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1);
+                        if (v[e][i][0] == 0u || v[e][i][1] == 0u || v[e][i][2] == 0u || v[e][i][3] == 0u) {
+                            v[e][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[e], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1);
                             missing = true;
                         }
                 if (!missing) break;
@@ -212,21 +253,21 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
 #pragma unroll
             for (int i = 0; i < CB; i++)
 #pragma unroll
-                for (int j = 0; j < QPT; j++) {
-                    const f32x4 f = __builtin_bit_cast(f32x4, v[j][i]);
-                    sum[j] += live[j] && c0 + i < p.S - 1 ? f : f32x4{0.f, 0.f, 0.f, 0.f};
+                for (int e = 0; e < NQ; e++) {
+                    const f32x4 f = __builtin_bit_cast(f32x4, v[e][i]);
+                    sum[e] += live[e] && c0 + i < p.S - 1 ? f : f32x4{0.f, 0.f, 0.f, 0.f};
                 }
         }
 #pragma unroll
-        for (int j = 0; j < QPT; j++) acc[j] = sum[j] + acc[j];
+        for (int e = 0; e < NQ; e++) acc[e] = sum[e] + acc[e];
     }
     const bool out_vec = (p.ldo & 3) == 0 && aligned_dev(p.out, 8);
 #pragma unroll
-    for (int j = 0; j < QPT; j++) {
-        if (!live[j]) continue;
-        const int qd = (int)threadIdx.x + 512 * j;
-        const int row = qd / (NBW / 4), nl = (qd % (NBW / 4)) * 4;
-        f32x4 a = acc[j];
+    for (int e = 0; e < NQ; e++) {
+        if (!live[e]) continue;
+        const int qd = (int)threadIdx.x + 512 * (e % QPT);
+        const int row = (e / QPT) * 16 + qd / (NBW / 4), nl = (qd % (NBW / 4)) * 4;
+        f32x4 a = acc[e];
         if (p.bias) {
 #pragma unroll
             for (int i = 0; i < 4; i++) a[i] = a[i] + act_1<ACT>(p.bias[n0 + nl + i]);
@@ -245,14 +286,12 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
     if (p.S > 1) {
         // the zone goes back to zero for the next launch; no branch around the stores (a dead quad or chunk gets an
         // out-of-range offset), so nothing waits for their acknowledgements
-        const uint32_t zone_chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
-        const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, zone_chunk_bytes * (uint32_t)(p.S - 1));
         for (int c0 = 0; c0 < p.S - 1; c0 += 4) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int j = 0; j < QPT; j++)
-                    __builtin_amdgcn_raw_buffer_store_b128(u32x4{0u, 0u, 0u, 0u}, rsrc_z, c0 + i < p.S - 1 ? zoff[j] : kOutOfRange,
+                for (int e = 0; e < NQ; e++)
+                    __builtin_amdgcn_raw_buffer_store_b128(u32x4{0u, 0u, 0u, 0u}, rsrc_z, c0 + i < p.S - 1 ? zoff[e] : kOutOfRange,
                                                            (uint32_t)(c0 + i) * zone_chunk_bytes, SC1);
         }
     }
@@ -268,13 +307,13 @@ WqDecodePlan make_wq_decode_plan(int64_t M, int64_t N, int64_t K, int w_bits, in
     const int64_t group = group_size > 0 ? group_size : K;
     pl.grouped = group_size > 0 && group != K;
     // a wavefront's 128 rows lie inside one scale group; every offset the kernel forms fits in 32 bits
-    pl.ok = !knob(kKnobWqDecodeOff) && w_bits == 4 && M >= 1 && M <= 16 && K >= 128 && K % 128 == 0 && N % 8 == 0 &&
+    pl.ok = !knob(kKnobWqDecodeOff) && w_bits == 4 && M >= 1 && M <= 32 && K >= 128 && K % 128 == 0 && N % 8 == 0 &&
             (pl.grouped ? group % 128 == 0 : true) && ldw_bytes >= row_bytes && ldw_bytes % 8 == 0 && ldx % 8 == 0 &&
             (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 8)) && (scale == nullptr || aligned(scale, 16)) &&
             (offset == nullptr || aligned(offset, 16)) && (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 31) &&
             (uint64_t)M * (uint64_t)ldx * 2 < (1ull << 31) && (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31);
     if (!pl.ok) return pl;
-    pl.mt = 1;
+    pl.mt = M <= 16 ? 1 : 2;
     pl.strips = (int)((row_bytes + 127) / 128);
     pl.S = (int)((K + 1023) / 1024);
     pl.zone_bytes = pl.S > 1 ? (size_t)(pl.S - 1) * (size_t)M * (size_t)N * 4 : 0;
@@ -313,8 +352,9 @@ int launch_wq_decode(const WqDecodePlan &plan, const void *x, int act_f16, const
         hipLaunchKernelGGL(kern, dim3((unsigned)((plan.strips + 7) / 8 * 8 * plan.S)), dim3(512), lds_bytes, s, p);
         return check_launch();
     };
-    if (M <= 8) return act_f16 ? go(wq_decode4_kernel<1, 1>) : go(wq_decode4_kernel<0, 1>);
-    return act_f16 ? go(wq_decode4_kernel<1, 2>) : go(wq_decode4_kernel<0, 2>);
+    if (M <= 8) return act_f16 ? go(wq_decode4_kernel<1, 1, 1>) : go(wq_decode4_kernel<0, 1, 1>);
+    if (M <= 16) return act_f16 ? go(wq_decode4_kernel<1, 1, 2>) : go(wq_decode4_kernel<0, 1, 2>);
+    return act_f16 ? go(wq_decode4_kernel<1, 2, 2>) : go(wq_decode4_kernel<0, 2, 2>);
 }
 
 } // namespace mi355

@@ -495,6 +495,28 @@ def test_graph_replays_match_eager(pa):
             assert torch.equal(got, exp)
 
 
+def test_prepared_quant_matmul_weight(pa, golden):
+    """prepare_quant_matmul_weight stores a [K,N] weight K-major once: the prepared tensor equals the original, has the
+    strides the GEMM reads directly (no per-call transpose, hence no workspace for it) and gives the same bits."""
+    from pytorch_amd import _capi
+    d = workloads.quant_matmul_inputs(seed=5, M=96, K=512, N=384, weight_nk=False, bias=True)
+    x1, w = d["x1"].cuda(), d["x2"].cuda()
+    assert w.stride() == (384, 1)
+    wp = pa.prepare_quant_matmul_weight(w)
+    assert wp.shape == w.shape and wp.stride() == (1, 512) and torch.equal(wp, w)
+    assert pa.prepare_quant_matmul_weight(wp) is wp                      # already K-major: unchanged
+    L = _capi.lib()
+    assert L.mi355_quant_matmul_workspace(96, 384, 512, *w.stride()) > L.mi355_quant_matmul_workspace(96, 384, 512, *wp.stride())
+    kw = dict(pertoken_scale=d["pertoken_scale"].cuda(), bias=d["bias"].cuda(), output_dtype=torch.bfloat16)
+    a, b = pa.npu_quant_matmul(x1, w, d["scale"].cuda(), **kw), pa.npu_quant_matmul(x1, wp, d["scale"].cuda(), **kw)
+    want, _ = golden.quant_matmul(d["x1"].numpy(), d["x2"].numpy(), d["scale"].numpy(), d["pertoken_scale"].numpy(), _bits(d["bias"]))
+    assert torch.equal(a, b) and np.array_equal(_bits(b), want)
+    # ragged sizes take the byte-wise transposing kernel; a batch of weights keeps its leading dimension
+    wr = torch.randint(-127, 128, (3, 40, 24), dtype=torch.int8, generator=torch.Generator().manual_seed(1)).cuda()
+    wrp = pa.prepare_quant_matmul_weight(wr)
+    assert torch.equal(wrp, wr) and wrp.stride()[-2:] == (1, 40)
+
+
 def test_workspace_outlives_growth_after_capture(pa):
     """A graph captured with a small split-K workspace must replay correctly after an eager call on the same stream
     needed a larger one: the superseded buffer is kept alive (and zeroed at rest), never handed back to the allocator."""
