@@ -370,6 +370,8 @@ def main():
         keep.clear()
         calls = [(lambda: keep.append(pa.npu_dynamic_quant(xs[0])))] * 8
         e["cache_hot_us"] = round(_graph_time_us(torch, calls), 3)
+        # what a launch of this grid costs when the kernel does nothing: the floor under the 3.1 us that 25 MB take at 8 TB/s
+        e["empty_launch_us"] = round(_graph_time_us(torch, [lambda: _capi.empty_launch(2048)] * 16), 3)
         if not args.skip_cpu:
             from oracle import golden
             y, s = pa.npu_dynamic_quant(xs[0])

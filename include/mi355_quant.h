@@ -338,6 +338,9 @@ int mi355_stream_capture_id(void *stream, unsigned long long *id);
  */
 int mi355_probe_clock(unsigned long long *out, int workgroups, int iters, void *stream);
 
+/* Measurement aid: a kernel that does nothing, `workgroups` x 256 threads (the per-launch floor inside a captured graph). */
+int mi355_probe_empty_launch(int workgroups, void *stream);
+
 /* Peak engine clock (kHz) and compute-unit count of the current device from the HIP runtime; either pointer may be NULL. */
 int mi355_device_info(int *clock_khz, int *compute_units);
 

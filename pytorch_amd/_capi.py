@@ -19,7 +19,7 @@ EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quan
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
            "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth", "mi355_set_tuning",
-           "mi355_quant_matmul_noalloc", "mi355_stream_capture_id", "mi355_probe_clock", "mi355_device_info", "mi355_transpose_int8")
+           "mi355_quant_matmul_noalloc", "mi355_stream_capture_id", "mi355_probe_clock", "mi355_device_info", "mi355_transpose_int8", "mi355_probe_empty_launch")
 
 _lib = None
 
@@ -57,12 +57,17 @@ def lib() -> ctypes.CDLL:
         L.mi355_quantize.argtypes = [vp, i32, vp, i64, vp, i32, i64, vp, i32, i64, i64, i64, i32, vp]
         L.mi355_set_tuning.argtypes = [ctypes.c_char_p, i32]
         L.mi355_probe_clock.argtypes = [vp, i32, i32, vp]
+        L.mi355_probe_empty_launch.argtypes = [i32, vp]
         L.mi355_transpose_int8.argtypes = [vp, vp, i64, i64, i64, vp]
         L.mi355_device_info.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.mi355_stream_capture_id.argtypes = [vp, ctypes.POINTER(ctypes.c_ulonglong)]
         L.mi355_quant_matmul_noalloc.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp]
         _lib = L
     return _lib
+
+
+def empty_launch(workgroups: int = 2048) -> None:
+    _check(lib().mi355_probe_empty_launch(workgroups, _stream()), "mi355_probe_empty_launch")
 
 
 def device_info():

@@ -26,8 +26,23 @@ __global__ __launch_bounds__(512) void clock_probe_kernel(unsigned long long *ou
     }
 }
 
+__global__ __launch_bounds__(256) void empty_kernel(int *sink)
+{
+    if (sink && blockIdx.x == 0x7fffffff) sink[0] = 0;
+}
+
 } // namespace
 } // namespace mi355
+
+// Launches a kernel that does nothing (`workgroups` workgroups of 256 threads): timing it from a captured graph gives the
+// per-launch floor that every microsecond-scale kernel of this library sits on.
+extern "C" int mi355_probe_empty_launch(int workgroups, void *stream)
+{
+    using namespace mi355;
+    if (workgroups <= 0) return MI355_ERR_BAD_ARGUMENT;
+    hipLaunchKernelGGL(empty_kernel, dim3((unsigned)workgroups), dim3(256), 0, static_cast<hipStream_t>(stream), nullptr);
+    return check_launch();
+}
 
 // out: [workgroups][2] 64-bit counts (shader-clock cycles, ticks of the constant 100 MHz counter) per workgroup.
 extern "C" int mi355_probe_clock(unsigned long long *out, int workgroups, int iters, void *stream)
