@@ -153,6 +153,14 @@ def _pmc_pass(torch, pa, workloads, dev):
     pa.npu_weight_quant_batchmatmul(g5["x"], g5["weight"], g5["antiquant_scale"], g5["antiquant_offset"], None, None,
                                     None, 128)
     pa.npu_anti_quant(xa, sa, offset=sa, dst_dtype=torch.bfloat16)
+    # the decode kernel at one and at 32 activation rows, each on a weight no kernel has touched
+    for m_rows, seed in ((1, 2), (32, 3)):
+        dm = workloads.w4a16_inputs(seed=seed, M=m_rows)
+        gm = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in dm.items()}
+        flush.fill_(3)
+        torch.cuda.synchronize()
+        pa.npu_weight_quant_batchmatmul(gm["x"], gm["weight"], gm["antiquant_scale"], gm["antiquant_offset"], None, None,
+                                        None, 128)
     # int4 weights with their words along K (the module's layout) at M = 8, and the int4 -> int8 widening of an A4W4
     # weight, on fresh operands
     wk = torch.randint(-2 ** 31, 2 ** 31 - 1, (14336, 512), dtype=torch.int32, device=dev)

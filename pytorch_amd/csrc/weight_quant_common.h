@@ -127,7 +127,6 @@ struct WqArgs {
     int strips;                     // 128-byte strips of a weight row
     int sgroups;                    // workgroup tiles along N: groups of W adjacent strips
     int S;                          // workgroups that share the K range of a tile
-    int skew;                       // streaming kernel: skew of the K slices in units
     // K-packed int4 kernel only
     int unit_sub;                   // sub-steps of 128 k per scale group
     int64_t ld_param_g, ld_param_n; // element strides of scale / offset: element (group, column)

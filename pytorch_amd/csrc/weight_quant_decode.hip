@@ -178,9 +178,30 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
     // ---- the eight wavefronts' sums meet in LDS, one m tile at a time: red[wave][row][column]
     float *red = reinterpret_cast<float *>(lds);
     constexpr int NQ = MT * QPT;                 // output quads per thread
+    constexpr int CB = NQ <= 2 ? 4 : 3;          // chunks collected per batch
     f32x4 acc[NQ];
     uint32_t zoff[NQ];
     bool live[NQ];
+#pragma unroll
+    for (int e = 0; e < NQ; e++) {
+        const int qd = (int)threadIdx.x + 512 * (e % QPT);
+        const int row = qd / (NBW / 4), nl = (qd % (NBW / 4)) * 4, mt = e / QPT;
+        live[e] = row < min(16, p.M - mt * 16) && n0 + nl < p.N;  // N is a multiple of 8: a quad is inside or outside
+        zoff[e] = live[e] ? (uint32_t)(((mt * 16 + row) * p.N + n0 + nl) * 4) : kOutOfRange;
+    }
+    const uint32_t zone_chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
+    const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, p.S > 1 ? zone_chunk_bytes * (uint32_t)(p.S - 1) : 0u);
+    const bool collector = p.S > 1 && chunk == p.S - 1;
+    // The strip's last workgroup asks for the other chunks' sums before it reduces its own: it was dispatched last, so
+    // the others have usually stored theirs by now and the answers arrive while the LDS reduction runs.
+    u32x4 v[NQ][CB];
+#pragma unroll
+    for (int e = 0; e < NQ; e++)
+#pragma unroll
+        for (int i = 0; i < CB; i++)
+            v[e][i] = collector && live[e] && i < p.S - 1
+                          ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[e], (uint32_t)i * zone_chunk_bytes, SC1)
+                          : u32x4{1u, 1u, 1u, 1u};
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
         const int rows_mt = min(16, p.M - mt * 16);
@@ -201,8 +222,6 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             const int qd = (int)threadIdx.x + 512 * j;
             const int row = qd / (NBW / 4), nl = (qd % (NBW / 4)) * 4;
             const int e = mt * QPT + j;
-            live[e] = row < rows_mt && n0 + nl < p.N;            // N is a multiple of 8: a quad is inside or outside
-            zoff[e] = live[e] ? (uint32_t)(((mt * 16 + row) * p.N + n0 + nl) * 4) : kOutOfRange;
             acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
             if (live[e]) {
 #pragma unroll
@@ -210,8 +229,6 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             }
         }
     }
-    const uint32_t zone_chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
-    const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, p.S > 1 ? zone_chunk_bytes * (uint32_t)(p.S - 1) : 0u);
     if (p.S > 1) {
         if (chunk < p.S - 1) {
 #pragma unroll
@@ -225,19 +242,19 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
         }
         // the strip's last workgroup collects the other chunks in chunk order; all of a thread's requests go out
         // before the first answer is looked at
-        constexpr int CB = NQ <= 2 ? 4 : 3;     // chunks per batch
         f32x4 sum[NQ];
 #pragma unroll
         for (int e = 0; e < NQ; e++) sum[e] = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int c0 = 0; c0 < p.S - 1; c0 += CB) {
-            u32x4 v[NQ][CB];
+            if (c0 > 0) {                        // the first batch is already on its way
 #pragma unroll
-            for (int e = 0; e < NQ; e++)
+                for (int e = 0; e < NQ; e++)
 #pragma unroll
-                for (int i = 0; i < CB; i++)
-                    v[e][i] = live[e] && c0 + i < p.S - 1
-                                  ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[e], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1)
-                                  : u32x4{1u, 1u, 1u, 1u};
+                    for (int i = 0; i < CB; i++)
+                        v[e][i] = live[e] && c0 + i < p.S - 1
+                                      ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[e], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1)
+                                      : u32x4{1u, 1u, 1u, 1u};
+            }
             for (int poll = 0; poll < kMaxPolls; poll++) {
                 bool missing = false;
 #pragma unroll

@@ -141,11 +141,7 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
 
     // contiguous range of K units for this (chunk, slice); a wavefront whose strip lies past the row has none
     const int R = p.S * KS, r = chunk * KS + kslice;
-    // The K slices of a workgroup are deliberately uneven: slice s is skewed by p.skew * min(s, KS - s) units, which
-    // gives the first half of the slices (the wavefronts that were placed first on their SIMDs and win its
-    // arbitration) more rows than the second half, so that both wavefronts of a SIMD finish together.
-    const int skew0 = p.skew * min(kslice, KS - kslice), skew1 = p.skew * min(kslice + 1, KS - kslice - 1);
-    const int u0 = (int)((int64_t)p.n_units * r / R) + skew0, u1 = (int)((int64_t)p.n_units * (r + 1) / R) + skew1;
+    const int u0 = (int)((int64_t)p.n_units * r / R), u1 = (int)((int64_t)p.n_units * (r + 1) / R);
     const int step0 = u0 * p.unit_steps;
     const int nsteps = strip < p.strips ? (u1 - u0) * p.unit_steps : 0;
     const int ustep = p.grouped ? p.unit_steps : nsteps;   // steps between folds
@@ -548,7 +544,6 @@ struct WqPlan {
     int strips, sgroups, mchunks, S;
     int unit_steps, n_units;
     int bs;             // steps per loop body of the kernel
-    int skew;           // units by which the K slices of a workgroup are skewed (see the kernel)
     size_t partial_bytes, counter_bytes;
     size_t slab_bytes;  // activations of one K chunk in LDS
 };
@@ -618,15 +613,6 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
     // the four-wavefront int4 kernel for two m tiles exists only with the running total (which also serves a
     // wavefront that meets a single group)
     if (w_bits == 4 && pl.mt == 2 && pl.w * pl.ks == 4) pl.accum = true;
-    {
-        // skew only where every slice keeps at least two units and no slice boundary leaves the chunk
-        // one eighth of a slice (measured on 8192 x 28672 int8, M = 16: 49.2 us even, 46.8 us with 9 + 9 + 7 + 7 units);
-        // the knob forces a value, 100 switches the skew off
-        const int per_slice = pl.n_units / (pl.S * pl.ks);
-        const int forced = knob(kKnobWqSkew);
-        pl.skew = forced == 100 ? 0 : forced != 0 ? forced : per_slice / 8;
-        if (pl.ks < 2 || pl.n_units % (pl.S * pl.ks) != 0 || per_slice - (pl.skew < 0 ? -pl.skew : pl.skew) < 1) pl.skew = 0;
-    }
     pl.partial_bytes = pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0;
     if (pl.S > 1 && (size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterCapacity) {
         pl.fast = false;                              // more tiles than arrival counters
@@ -919,7 +905,6 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
     p.strips = pl.strips;
     p.sgroups = pl.sgroups;
     p.S = pl.S;
-    p.skew = pl.skew;
     if (f16) return w_bits == 4 ? launch_bits<4, 1>(p, pl, s) : launch_bits<8, 1>(p, pl, s);
     return w_bits == 4 ? launch_bits<4, 0>(p, pl, s) : launch_bits<8, 0>(p, pl, s);
 }
