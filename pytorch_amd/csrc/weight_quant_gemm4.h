@@ -1,0 +1,28 @@
+// Internal interface of the tiled kernel for int4 weights packed along N with more than 32 activation rows; not part of
+// the C ABI.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+namespace mi355 {
+
+struct WqGemm4Plan {
+    bool ok;                 // the kernel accepts this problem
+    int bm;                  // activation rows per workgroup tile: 64 or 128
+    int tiles_m, strips;     // workgroup tiles: row blocks x 128-byte strips of the weight rows (256 columns)
+    int S;                   // workgroups that share a tile's K range
+    int gstages;             // 128-row stages per scale group (per channel: all stages of a workgroup)
+    size_t zone_bytes;       // bytes of the workspace's zero area used for the exchange (S > 1)
+};
+
+__attribute__((visibility("hidden"))) WqGemm4Plan make_wq_gemm4_plan(int64_t M, int64_t N, int64_t K, int w_bits,
+                                                                     int64_t group_size, int64_t ldw_k, int64_t ldx,
+                                                                     const void *x, const void *w, const void *scale,
+                                                                     const void *offset);
+
+__attribute__((visibility("hidden"))) int launch_wq_gemm4(const WqGemm4Plan &plan, const void *x, int act_f16, const void *w,
+                                                          const void *scale, const void *offset, const void *bias, void *out,
+                                                          int64_t M, int64_t N, int64_t K, int64_t group_size, int64_t ldx,
+                                                          int64_t ldw_k, int64_t ldo, void *workspace, void *stream);
+
+} // namespace mi355

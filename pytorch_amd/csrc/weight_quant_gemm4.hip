@@ -1,0 +1,500 @@
+// npu_weight_quant_batchmatmul, int4 weights packed along N, more than 32 activation rows: a tiled GEMM in which the
+// packed weights never exist in expanded form outside of registers.
+//
+// A workgroup of four wavefronts owns 64 activation rows x one 128-byte strip of the weight rows (256 columns) and
+// walks its K range in stages of 128 rows.  Per stage the activations (64 x 256 B) and the raw strip (128 x 128 B) are
+// copied global -> LDS by direct loads, three stages ahead (four slots), one barrier per stage.  The strip's 32 dword
+// columns form two spans of 16, a dword's four bytes two byte pairs.  A wavefront owns all 64 rows (four MFMA row
+// tiles) x one span x one byte pair: its lane c reads dword 16h + c of its eight k rows back from LDS (eight 4-byte
+// reads per 32 k) and expands the four nibbles of its byte pair into exact bf16 / fp16 images of the integers, i.e.
+// into the B operands of four MFMA column tiles (tile i = columns 128h + 8c + 4jp + i), each of which meets all four
+// row tiles: 16 MFMAs per step for 4 activation fragments and 8 dwords from LDS and ~40 integer instructions, which
+// is what keeps the matrix pipe, and not LDS or the vector ALU, the busiest unit.  No expanded image ever travels
+// through LDS.  Operands of the next step (also across the stage boundary: a stage is complete in LDS one barrier
+// before it is computed) are requested as soon as the registers they replace are free.
+// Images (bf16): low nibbles stay where they are, as the low mantissa bits of 128.0 (128 + u, u = w + 8); high nibbles
+// move down one bit into the top mantissa bits of 8.0 (8 + u / 2); fp16: both go to the top mantissa bits of 16.0.
+// Per scale group  out += scale * (P + offset * X)  as in the other kernels: a group ends with a stage (or several),
+// the finished sums are folded tile by tile in front of the MFMAs that restart them with a zero accumulator; the row
+// sums X come from one extra MFMA per step (wavefront i takes row tile i) and travel through LDS.
+// K may be split over S workgroups per tile (few tiles): all but the last store their float32 sums in register order
+// into the workspace's zero zone, zero mapped to -0.0; the last one (highest index: dispatched after the others) polls
+// until no word is zero, adds in chunk order, writes the output and restores the zeros (weight_quant_decode.hip).
+#include "weight_quant_common.h"
+#include "weight_quant_gemm4.h"
+
+namespace mi355 {
+namespace {
+
+struct WqGemm4Args {
+    const uint16_t *x, *scale, *offset, *bias;
+    const void *w;
+    uint16_t *out;
+    uint32_t *zone;
+    int64_t ldx, ldo;
+    uint32_t ldw_bytes, row_bytes;
+    int M, N, K;
+    int gstages;                    // stages per scale group
+    int grouped;
+    int tiles_m, strips, S;
+};
+
+constexpr int kMaxPolls4 = 1 << 20;
+constexpr int kMaxRows4 = 384;     // beyond this the kernel that expands the weights once per 256 rows (weight_quant_gemm.hip) is faster
+
+// images of the two nibbles of a byte; t = [byte of row 2v, 0, byte of row 2v + 1, 0].  out = mask ? (t ^ c) : c is one
+// three-input bitwise instruction: c carries the image's exponent bits outside the mask and, inside it, the bit that
+// turns the two's-complement nibble into u = w + 8.
+__device__ __forceinline__ uint32_t bit_blend(uint32_t t, uint32_t mask, uint32_t c)
+{
+    return __builtin_amdgcn_bitop3_b32(t, mask, c, 0x6a);   // truth table of (mask & (t ^ c)) | (~mask & c), t the high index bit
+}
+template <int ACT>
+__device__ __forceinline__ void expand_byte(uint32_t t, uint32_t mask_lo, uint32_t c_lo, uint32_t mask_hi, uint32_t c_hi, uint32_t &lo, uint32_t &hi)
+{
+    if constexpr (ACT == 0) {
+        lo = bit_blend(t, mask_lo, c_lo);
+        hi = bit_blend(t >> 1, mask_hi, c_hi);
+    } else {
+        lo = bit_blend(t << 6, mask_hi, c_hi);
+        hi = bit_blend(t << 2, mask_hi, c_hi);
+    }
+}
+template <int ACT> constexpr uint32_t kMaskLo4 = 0x000f000fu;
+template <int ACT> constexpr uint32_t kBlendLo4 = 0x43004300u | 0x00080008u;
+template <int ACT> constexpr uint32_t kMaskHi4 = ACT == 0 ? 0x00780078u : 0x03c003c0u;
+template <int ACT> constexpr uint32_t kBlendHi4 = ACT == 0 ? (0x41004100u | 0x00400040u) : (0x4c004c00u | 0x02000200u);
+// weight = mul * image - bias, per nibble position
+template <int ACT> constexpr float kMulLo4 = 1.0f;
+template <int ACT> constexpr float kBiasLo4 = ACT == 0 ? 136.0f : 24.0f;
+template <int ACT> constexpr float kMulHi4 = kImageMul<4, ACT>;
+template <int ACT> constexpr float kBiasHi4 = kImageBias<4>;
+
+template <int ACT>
+__global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
+{
+    constexpr int NW = 4, BM = 64, BK = 128, SLOTS = 4;
+    constexpr int A_BYTES = BM * 256, R_BYTES = BK * 128;      // one stage of activations / raw weights
+    constexpr int LA = BM / 4 / NW, LR = 16 / NW;              // 1 KiB load units per wavefront and stage
+    constexpr int LPS = LA + LR;
+    constexpr int PRM_SLOT = 1024;                             // [256 scales | 256 offsets], 16 bits each
+    constexpr int PRM_SLOTS = 8;                               // groups whose parameters are in LDS (+ 1 slot nobody reads)
+    constexpr int SC1 = 16;                                    // cache-policy bit: agent scope
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    char *const raw = lds + SLOTS * A_BYTES;
+    char *const prm = raw + SLOTS * R_BYTES;
+    float *const xsum = reinterpret_cast<float *>(prm + (PRM_SLOTS + 1) * PRM_SLOT);   // [2 slots][BM] row sums
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int h = wave & 1, jp = wave >> 1;
+    // workgroups are dealt round-robin to the 8 XCDs.  The row blocks of a strip and the chunks of a tile sit on one
+    // XCD (they share the strip resp. the activations in its L2); the last chunk has the tile's highest index.
+    const int xcd_slot = blockIdx.x >> 3;
+    const int j = xcd_slot / p.S, chunk = xcd_slot % p.S;
+    const int strip = (blockIdx.x & 7) + 8 * (j / p.tiles_m);
+    if (strip >= p.strips) return;
+    const int mb = j % p.tiles_m;
+    const int tile = strip * p.tiles_m + mb;
+    const int m0 = mb * BM;
+    const int n0 = strip * 256;
+    const int total_stages = p.K / BK;
+    const int units = total_stages / p.gstages;                // K is split in whole scale groups
+    const int u0 = (int)((int64_t)units * chunk / p.S), u1 = (int)((int64_t)units * (chunk + 1) / p.S);
+    const int s0 = u0 * p.gstages, NSTG = (u1 - u0) * p.gstages;
+
+    // ---- global -> LDS.  Activations: unit = 4 rows x 256 B; LDS slot l of a unit is (row l / 16, chunk l % 16) and
+    // holds global chunk (l % 16) ^ (row & 15).  Raw weights: unit = 8 row slots x 128 B; row slot sl holds row
+    // sl ^ ((sl >> 3) & 1) and its chunk slot j' holds chunk j' ^ (4 * ((row >> 4) & 1)): with that the four k octets a
+    // wavefront reads together fall into four different quarters of the banks.
+    const int rows_a = min(BM, p.M - m0);
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.x + (int64_t)m0 * p.ldx, (uint32_t)(((int64_t)(rows_a - 1) * p.ldx + p.K) * 2));
+    const uint32_t strip_valid = min(128u, p.row_bytes - (uint32_t)strip * 128u);
+    const __amdgpu_buffer_rsrc_t rsrc_w =
+        make_rsrc(static_cast<const char *>(p.w) + (size_t)strip * 128, (uint32_t)(p.K - 1) * p.ldw_bytes + strip_valid);
+    // parameters of a scale group (the strip's 256 scales and offsets) travel with the group's first stage, copied
+    // global -> LDS by wavefront 0.  It issues its four parameter loads with every stage (for the other stages of a
+    // group they move no bytes and point at a slot nobody reads), so every wavefront's loads per stage are a constant.
+    const bool has_offset = p.offset != nullptr;
+    const uint32_t param_bytes = (uint32_t)(p.grouped ? units : 1) * (uint32_t)p.N * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc_s = make_rsrc(p.scale, param_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_o = make_rsrc(has_offset ? p.offset : p.scale, param_bytes);
+    int iss_in_group = 0, iss_group = u0;
+    const __amdgpu_buffer_rsrc_t rsrc_none = make_rsrc(p.x, 0);      // every access is out of range: zeros, no traffic
+    auto issue_stage = [&](int s) {
+        const bool live = s < NSTG;
+        const __amdgpu_buffer_rsrc_t ra = live ? rsrc_a : rsrc_none, rw = live ? rsrc_w : rsrc_none;
+        char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
+#pragma unroll
+        for (int i = 0; i < LA; i++) {
+            const int row = 4 * (i * NW + wave) + (lane >> 4);
+            const uint32_t vo = (uint32_t)(row * (int)p.ldx * 2 + (((lane & 15) ^ (row & 15)) * 16));
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void *)(sa + (i * NW + wave) * 1024), 16, vo, (uint32_t)(s0 + s) * 256u, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < LR; i++) {
+            const int sl = 8 * (i * NW + wave) + (lane >> 3);
+            const int row = sl ^ ((sl >> 3) & 1);
+            const uint32_t ch = (uint32_t)((lane & 7) ^ (4 * ((row >> 4) & 1)));
+            const uint32_t vo = ch * 16u < strip_valid ? (uint32_t)row * p.ldw_bytes + ch * 16u : kOutOfRange;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void *)(sr + (i * NW + wave) * 1024), 16, vo,
+                                                     (uint32_t)(s0 + s) * (uint32_t)BK * p.ldw_bytes, 0, kNonTemporal);
+        }
+        if (wave == 0) {
+            const bool first = live && iss_in_group == 0;
+            const uint32_t ro = (uint32_t)(p.grouped ? iss_group : 0) * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
+            char *dst = prm + (first ? (iss_group & (PRM_SLOTS - 1)) : PRM_SLOTS) * PRM_SLOT;
+            const uint32_t vo = first ? (uint32_t)lane * 4u : kOutOfRange;
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_s, (lds_void *)(dst + q * 256), 4, vo, ro + q * 256u, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_o, (lds_void *)(dst + 512 + q * 256), 4, vo, ro + q * 256u, 0, 0);
+            }
+        }
+        if (++iss_in_group == p.gstages) {
+            iss_in_group = 0;
+            iss_group++;
+        }
+    };
+    // everything but the newest stage's loads has landed
+    auto wait_older_stages = [&]() {
+        if (wave == 0) wait_vmcnt<LPS + 4>();
+        else wait_vmcnt<LPS>();
+    };
+
+    // ---- LDS read addresses
+    // raw: dword 16h + c of rows 8g + t; even t and odd t have their own base because odd octets swap row pairs
+    const int jch = (4 * h + (c >> 2)) ^ (4 * ((g >> 1) & 1));
+    const int r_even = (8 * g + (g & 1)) * 128 + jch * 16 + (c & 3) * 4;
+    const int r_odd = (8 * g + 1 - (g & 1)) * 128 + jch * 16 + (c & 3) * 4;
+    // activations: row c of a row tile, chunk 4 ks + g, stored at chunk slot ((ks ^ (c >> 2)) << 2) | (g ^ (c & 3))
+    const int a_lane = c * 256 + ((c >> 2) << 6) + ((g ^ (c & 3)) << 4);   // step ks: a_lane ^ (ks << 6)
+    const int prm_col = (128 * h + 8 * c + 4 * jp) * 2;        // byte offset of this lane's four columns in a parameter slot
+    const uint32_t sel0 = 0x0c000c00u | ((4u + 2u * jp) << 16) | (2u * jp);      // byte 2jp of two rows
+    const uint32_t sel1 = sel0 + 0x00010001u;                                    // byte 2jp + 1
+
+    f32x4 P[4][4], tot[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+            P[i][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+            tot[i][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    f32x4 Xown = f32x4{0.f, 0.f, 0.f, 0.f};                    // row sums of row tile `wave`
+    const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
+    const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+    uint32_t mask_lo, c_lo, mask_hi, c_hi;                     // opaque to the optimiser, which would otherwise undo the blend
+    asm volatile("s_mov_b32 %0, %1" : "=s"(mask_lo) : "n"(kMaskLo4<ACT>));
+    asm volatile("s_mov_b32 %0, %1" : "=s"(mask_hi) : "n"(kMaskHi4<ACT>));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(c_lo) : "n"(kBlendLo4<ACT>));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(c_hi) : "n"(kBlendHi4<ACT>));
+
+    // fold of a finished group into the running total: tot += (scale * mul) * (P' + ((offset - bias) / mul) * X)
+    float scm[4], ofm[4];
+    f32x4 Xg[4];
+    auto fetch_fold_operands = [&](int group) {
+        const int slot = group & 1;
+        const char *pb = prm + (group & (PRM_SLOTS - 1)) * PRM_SLOT + prm_col;
+        const uint32_t sr0 = *reinterpret_cast<const uint32_t *>(pb), sr1 = *reinterpret_cast<const uint32_t *>(pb + 4);
+        const uint32_t or0 = *reinterpret_cast<const uint32_t *>(pb + 512), or1 = *reinterpret_cast<const uint32_t *>(pb + 516);
+        const float *xs = xsum + slot * BM + 4 * g;
+#pragma unroll
+        for (int i = 0; i < 4; i++) Xg[i] = *reinterpret_cast<const f32x4 *>(xs + 16 * i);
+        const float sc[4] = {act_lo<ACT>(sr0), act_hi<ACT>(sr0), act_lo<ACT>(sr1), act_hi<ACT>(sr1)};
+        const float of[4] = {has_offset ? act_lo<ACT>(or0) : 0.f, has_offset ? act_hi<ACT>(or0) : 0.f,
+                             has_offset ? act_lo<ACT>(or1) : 0.f, has_offset ? act_hi<ACT>(or1) : 0.f};
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+            const float mul = (nb & 1) ? kMulHi4<ACT> : kMulLo4<ACT>, bias = (nb & 1) ? kBiasHi4<ACT> : kBiasLo4<ACT>;
+            scm[nb] = sc[nb] * mul;
+            ofm[nb] = (of[nb] - bias) * (1.0f / mul);
+        }
+    };
+    auto fold_tile = [&](int i, int nb) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) tot[i][nb][q] = __builtin_fmaf(scm[nb], __builtin_fmaf(ofm[nb], Xg[i][q], P[i][nb][q]), tot[i][nb][q]);
+    };
+
+    // ---- operands of a step: raw dwords are requested two steps ahead (they are expanded one step ahead, between the
+    // MFMAs of the step before), activation fragments one step ahead, each into the registers of the fragment that
+    // was just used
+    uint32_t w[8];
+    u32x4 AF[4], AX, b[2][4];
+    auto read_w = [&](const char *sr, int ks) {
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+            w[t] = *reinterpret_cast<const uint32_t *>(sr + ks * 4096 + ((t & 1) ? r_odd : r_even) + (t >> 1) * 256);
+    };
+    auto read_a = [&](const char *sa, int ks, int i) { return *reinterpret_cast<const u32x4 *>(sa + i * 4096 + (a_lane ^ (ks << 6))); };
+    auto expand = [&](u32x4 (&bn)[4]) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const uint32_t t0 = __builtin_amdgcn_perm(w[2 * v + 1], w[2 * v], sel0);
+            const uint32_t t1 = __builtin_amdgcn_perm(w[2 * v + 1], w[2 * v], sel1);
+            uint32_t e0, e1, e2, e3;
+            expand_byte<ACT>(t0, mask_lo, c_lo, mask_hi, c_hi, e0, e1);
+            expand_byte<ACT>(t1, mask_lo, c_lo, mask_hi, c_hi, e2, e3);
+            bn[0][v] = e0;
+            bn[1][v] = e1;
+            bn[2][v] = e2;
+            bn[3][v] = e3;
+        }
+    };
+    // one step of 32 k: the MFMAs of step ks with the expansion of step ks + 1 (and, at the start of a group, the fold
+    // of the group before) spread between them
+    auto step = [&](const bool fold, const int ks, const char *sa, const char *sr, const char *sa_next, const char *sr_next) {
+        u32x4(&bc)[4] = b[ks & 1];
+        expand(b[(ks + 1) & 1]);
+        read_w(ks + 2 < 4 ? sr : sr_next, (ks + 2) & 3);
+        const char *na = ks + 1 < 4 ? sa : sa_next;
+        const int nk = (ks + 1) & 3;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++) {
+                if (fold) {
+                    fold_tile(i, nb);
+                    P[i][nb] = mfma_act<ACT>(AF[i], bc[nb], zero4);
+                } else {
+                    P[i][nb] = mfma_act<ACT>(AF[i], bc[nb], P[i][nb]);
+                }
+            }
+            AF[i] = read_a(na, nk, i);
+        }
+        Xown = mfma_act<ACT>(AX, ones, Xown);
+        AX = read_a(na, nk, wave);
+        // interleave: one MFMA, its share of the integer work, one LDS read
+#pragma unroll
+        for (int r = 0; r < 17; r++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (fold) __builtin_amdgcn_sched_group_barrier(0x002, 13, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+
+    // ---- main loop.  Stage s is computed from slot s % 4 while memory is asked for stage s + 3.  Loads are never skipped
+    // (a stage past the end gets an out-of-range lane offset and moves no bytes), so "everything but the newest stage's
+    // loads" at the top means: stage s + 1, whose first operands the last steps of stage s request, is complete behind
+    // the barrier.  The barrier is issued without the fences of __syncthreads(): with direct-to-LDS loads in flight the
+    // compiler puts a full vmcnt(0) in front of a fenced barrier, which would wait for the stage that was requested
+    // last; the explicit waits above it are what the fence would have to do.
+    issue_stage(0);
+    issue_stage(1);
+    wait_older_stages();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();                              // stage 0 is complete in LDS
+    asm volatile("" ::: "memory");
+    issue_stage(2);
+    read_w(raw, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) AF[i] = read_a(lds, 0, i);
+    AX = read_a(lds, 0, wave);
+    expand(b[0]);
+    read_w(raw, 1);
+    bool pending = false;
+    int pending_slot = 0, in_group = 0, group_row = u0;
+    for (int s = 0; s < NSTG; s++) {
+        wait_older_stages();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();                          // stage s + 1 is complete in LDS; everyone is done with stage s - 1
+        asm volatile("" ::: "memory");
+        const bool last_of_group = ++in_group == p.gstages;
+        issue_stage(s + 3);
+
+        const char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
+        const char *sa_next = lds + ((s + 1) & 3) * A_BYTES, *sr_next = raw + ((s + 1) & 3) * R_BYTES;
+        __builtin_amdgcn_sched_barrier(0);
+        if (pending) {
+            fetch_fold_operands(pending_slot);
+            __builtin_amdgcn_sched_barrier(0);                 // requested before anything of the step, not between its MFMAs
+            step(true, 0, sa, sr, sa_next, sr_next);
+        } else {
+            step(false, 0, sa, sr, sa_next, sr_next);
+        }
+#pragma unroll
+        for (int ks = 1; ks < 4; ks++) {
+            __builtin_amdgcn_sched_barrier(0);
+            step(false, ks, sa, sr, sa_next, sr_next);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        pending = last_of_group;
+        pending_slot = group_row;
+        if (last_of_group) {
+            if (c == 0) *reinterpret_cast<f32x4 *>(xsum + (group_row & 1) * BM + wave * 16 + 4 * g) = Xown;   // read after the next barrier
+            Xown = zero4;
+            in_group = 0;
+            group_row++;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the refills past the end (zeros) have landed
+    __syncthreads();
+    if (pending) {
+        fetch_fold_operands(pending_slot);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++) fold_tile(i, nb);
+    }
+
+    // ---- split K: exchange in register order through the zero zone
+    if (p.S > 1) {
+        constexpr uint32_t WAVE_BYTES = 16 * 64 * 16, TILE_BYTES = NW * WAVE_BYTES;
+        const uint32_t tiles = (uint32_t)(p.tiles_m * p.strips);
+        const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, (uint32_t)(p.S - 1) * tiles * TILE_BYTES);
+        const uint32_t lane_off = (uint32_t)tile * TILE_BYTES + (uint32_t)wave * WAVE_BYTES + (uint32_t)lane * 16u;
+        if (chunk < p.S - 1) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                u32x4 bits = __builtin_bit_cast(u32x4, tot[e >> 2][e & 3]);
+#pragma unroll
+                for (int q = 0; q < 4; q++) bits[q] = bits[q] == 0u ? 0x80000000u : bits[q];   // no stored word is zero
+                __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_z, lane_off + e * 1024, (uint32_t)chunk * tiles * TILE_BYTES, SC1);
+            }
+            return;
+        }
+        for (int ch = 0; ch < p.S - 1; ch++) {
+            u32x4 v[16];
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                v[e] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES, SC1);
+            for (int poll = 0; poll < kMaxPolls4; poll++) {
+                bool missing = false;
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    if (v[e][0] == 0u || v[e][1] == 0u || v[e][2] == 0u || v[e][3] == 0u) {
+                        v[e] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES, SC1);
+                        missing = true;
+                    }
+                if (!missing) break;
+            }
+            // chunk order: ((c0 + c1) + ...) + own
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                if (ch == 0) P[e >> 2][e & 3] = __builtin_bit_cast(f32x4, v[e]);
+                else P[e >> 2][e & 3] += __builtin_bit_cast(f32x4, v[e]);
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 16; e++) tot[e >> 2][e & 3] = P[e >> 2][e & 3] + tot[e >> 2][e & 3];
+        // the zone goes back to zero for the next launch (no branches around the stores: nothing waits for them)
+        for (int ch = 0; ch < p.S - 1; ch++)
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                __builtin_amdgcn_raw_buffer_store_b128(u32x4{0u, 0u, 0u, 0u}, rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES, SC1);
+    }
+
+    // ---- output: lane (c, g) holds rows 16 i + 4 g + q, columns 128 h + 8 c + 4 jp .. + 3: 8 bytes per row
+    const int col = n0 + 128 * h + 8 * c + 4 * jp;
+    if (col >= p.N) return;                                    // N is a multiple of 8: the four columns are inside or outside
+    float bv[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) bv[nb] = p.bias ? act_1<ACT>(p.bias[col + nb]) : 0.0f;
+    const bool out_vec = (p.ldo & 3) == 0 && aligned_dev(p.out, 8);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int row = m0 + i * 16 + 4 * g + q;
+            if (row >= p.M) continue;
+            const uint32_t lo = pack_act2<ACT>(tot[i][0][q] + bv[0], tot[i][1][q] + bv[1]);
+            const uint32_t hi = pack_act2<ACT>(tot[i][2][q] + bv[2], tot[i][3][q] + bv[3]);
+            uint16_t *o = p.out + (int64_t)row * p.ldo + col;
+            if (out_vec) {
+                *reinterpret_cast<uint2 *>(o) = uint2{lo, hi};
+            } else {
+                o[0] = (uint16_t)(lo & 0xffffu);
+                o[1] = (uint16_t)(lo >> 16);
+                o[2] = (uint16_t)(hi & 0xffffu);
+                o[3] = (uint16_t)(hi >> 16);
+            }
+        }
+}
+
+template <int ACT>
+int launch4(const WqGemm4Args &p, unsigned grid, hipStream_t s)
+{
+    constexpr size_t lds_bytes = (size_t)4 * 64 * 256 + 4 * 128 * 128 + 9 * 1024 + 2 * 64 * 4;
+    static_assert(lds_bytes <= 160 * 1024, "LDS budget");
+    auto kern = wq_gemm4_kernel<ACT>;
+    static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, s, p);
+    return check_launch();
+}
+
+} // namespace
+
+WqGemm4Plan make_wq_gemm4_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size, int64_t ldw_k, int64_t ldx,
+                               const void *x, const void *w, const void *scale, const void *offset)
+{
+    WqGemm4Plan pl{};
+    const int64_t row_bytes = N / 2, ldw_bytes = ldw_k * 4;
+    const int64_t group = group_size > 0 ? group_size : K;
+    const bool grouped = group_size > 0 && group != K;
+    pl.ok = !knob(kKnobWqGemm4Off) && w_bits == 4 && M > 32 && M <= kMaxRows4 && K >= 128 && K % 128 == 0 && N % 8 == 0 && (!grouped || group % 128 == 0) &&
+            ldw_bytes >= row_bytes && ldw_bytes % 16 == 0 && ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) &&
+            (w == nullptr || aligned(w, 16)) && (scale == nullptr || aligned(scale, 4)) && (offset == nullptr || aligned(offset, 4)) &&
+            (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 31) && (uint64_t)128 * (uint64_t)ldx * 2 + (uint64_t)K * 2 < (1ull << 31) &&
+            (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && M <= 0x7fffffff;
+    if (!pl.ok) return pl;
+    pl.strips = (int)((row_bytes + 127) / 128);
+    const int64_t stages = K / 128;
+    const int64_t units = grouped ? K / group : 1;
+    // few tiles: split K in whole scale groups
+    pl.bm = 64;
+    pl.tiles_m = (int)((M + pl.bm - 1) / pl.bm);
+    const int64_t tiles = (int64_t)pl.tiles_m * pl.strips;
+    int64_t S = tiles < kNumCU ? kNumCU / tiles : 1;
+    if (S > units) S = units;
+    if (S > 8) S = 8;
+    if (const int f = knob(kKnobWqgSplit))
+        if (f >= 1 && f <= units) S = f;
+    auto zone = [&](int64_t s) { return (uint64_t)(s - 1) * (uint64_t)tiles * (uint64_t)pl.bm * 256u * 4u; };
+    while (S > 1 && zone(S) > kWorkspaceZoneBytes) S--;
+    pl.S = (int)S;
+    pl.gstages = (int)(grouped ? group / 128 : stages / S > 0 ? stages : stages);
+    if (!grouped) {
+        // per channel: one fold per workgroup, so a "group" is the workgroup's whole range; K is split in stages
+        if (stages % S != 0) pl.S = 1;
+        pl.gstages = (int)(stages / pl.S);
+    }
+    pl.zone_bytes = pl.S > 1 ? (size_t)zone(pl.S) : 0;
+    if (tiles * pl.S > 0x7fffffff) pl.ok = false;
+    return pl;
+}
+
+int launch_wq_gemm4(const WqGemm4Plan &plan, const void *x, int act_f16, const void *w, const void *scale, const void *offset,
+                    const void *bias, void *out, int64_t M, int64_t N, int64_t K, int64_t group_size, int64_t ldx, int64_t ldw_k,
+                    int64_t ldo, void *workspace, void *stream)
+{
+    WqGemm4Args p{};
+    p.x = static_cast<const uint16_t *>(x);
+    p.w = w;
+    p.scale = static_cast<const uint16_t *>(scale);
+    p.offset = static_cast<const uint16_t *>(offset);
+    p.bias = static_cast<const uint16_t *>(bias);
+    p.out = static_cast<uint16_t *>(out);
+    p.zone = plan.S > 1 ? reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kWorkspaceCounterCapacity) : nullptr;
+    p.ldx = ldx;
+    p.ldo = ldo;
+    p.ldw_bytes = (uint32_t)(ldw_k * 4);
+    p.row_bytes = (uint32_t)(N / 2);
+    p.M = (int)M;
+    p.N = (int)N;
+    p.K = (int)K;
+    p.gstages = plan.gstages;
+    p.grouped = group_size > 0 && group_size != K;
+    p.tiles_m = plan.tiles_m;
+    p.strips = plan.strips;
+    p.S = plan.S;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t tiles = (int64_t)plan.tiles_m * plan.strips;
+    (void)tiles;
+    const unsigned grid = (unsigned)((plan.strips + 7) / 8 * 8 * plan.tiles_m * plan.S);
+    return act_f16 ? launch4<1>(p, grid, s) : launch4<0>(p, grid, s);
+}
+
+} // namespace mi355

@@ -40,6 +40,7 @@
 #include "weight_quant_gemm.h"
 #include "weight_quant_kpacked.h"
 #include "weight_quant_decode.h"
+#include "weight_quant_gemm4.h"
 #include <type_traits>
 
 namespace mi355 {
@@ -747,6 +748,8 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
     if (w_bits == 4) {                      // decode kernel: its exchange lives in the zero area
         const WqDecodePlan dp = make_wq_decode_plan(M, N, K, 4, group_size, N / 8, K, nullptr, nullptr, nullptr, nullptr);
         if (dp.ok && dp.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
+        const WqGemm4Plan g4 = make_wq_gemm4_plan(M, N, K, 4, group_size, N / 8, K, nullptr, nullptr, nullptr, nullptr);
+        if (g4.ok && g4.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
     }
     if (w_bits == 4) {                      // words along K
         const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, K / 8, K, nullptr, nullptr);
@@ -863,6 +866,16 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
             }
             return launch_wq_decode(dp, x_bf16, f16 ? 1 : 0, w, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, group_size, ldx,
                                     ldw_k, ldo, workspace, stream);
+        }
+        // more than 32 rows: the tiled kernel that expands the nibbles in registers
+        const WqGemm4Plan g4 = make_wq_gemm4_plan(M, N, K, 4, group_size, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
+        if (g4.ok && aligned(out_bf16, 2) && (!bias || aligned(bias, 2))) {
+            if (g4.S > 1) {
+                if (!workspace || workspace_bytes < kWorkspaceZeroBytes) return MI355_ERR_WORKSPACE;
+                if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+            }
+            return launch_wq_gemm4(g4, x_bf16, f16 ? 1 : 0, w, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, group_size, ldx, ldw_k,
+                                   ldo, workspace, stream);
         }
     }
     // more than 32 rows: the tiled kernel decodes every weight once per 64 or 128 rows

@@ -430,6 +430,11 @@ TILED_CASES = [  # bits, M, K, N, group, float16, bias
     (4, 100, 1024, 512, 256, True, False),
     (4, 130, 512, 2048, 512, False, False),   # one group = per channel
     (4, 320, 1024, 768, 128, False, False),   # three row tiles
+    (4, 33, 128, 8, 128, False, False),       # one stage, one dword column, one group = per channel
+    (4, 64, 1536, 520, 384, False, True),     # groups of three stages, last strip holds 8 columns
+    (4, 256, 8192, 256, 8192, True, False),   # one strip, four row blocks, per channel with a K split
+    (4, 384, 1024, 512, 128, False, False),   # the most rows the register-expanding kernel takes
+    (4, 400, 1024, 512, 128, False, False),   # beyond it: the kernel that expands weight images into LDS
     # int8 weights stored [N, K] (the transposed view that LinearWeightQuant passes, linear_weight_quant.py:106)
     (8, 40, 1024, 384, 0, False, False, True),
     (8, 128, 2048, 1000, 0, False, True, True),
