@@ -104,6 +104,65 @@ __device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint
     }
 }
 
+// Second expansion of int4 bytes, one instruction shorter per fragment register and without the separate sign flip.
+// t = [byte of row 2v, 0, byte of row 2v + 1, 0] straight from the packed words.  out = mask ? (t ^ c) : c is a single
+// three-input bitwise instruction: c carries the image's exponent bits outside the mask and, inside it, the bit that
+// turns the two's-complement nibble into u = w + 8.  bf16: the low nibble stays where it is, as the low mantissa bits
+// of 128.0 (image 128 + u), the high nibble moves down one bit into the top mantissa bits of 8.0 (image 8 + u / 2);
+// fp16: both go to the top mantissa bits of 16.0 (image 16 + u).  weight = mul * image - bias per nibble position.
+__device__ __forceinline__ uint32_t bit_blend(uint32_t t, uint32_t mask, uint32_t c)
+{
+    return __builtin_amdgcn_bitop3_b32(t, mask, c, 0x6a);   // truth table of (mask & (t ^ c)) | (~mask & c), t the high index bit
+}
+template <int ACT>
+__device__ __forceinline__ void expand_byte(uint32_t t, uint32_t mask_lo, uint32_t c_lo, uint32_t mask_hi, uint32_t c_hi, uint32_t &lo, uint32_t &hi)
+{
+    if constexpr (ACT == 0) {
+        lo = bit_blend(t, mask_lo, c_lo);
+        hi = bit_blend(t >> 1, mask_hi, c_hi);
+    } else {
+        lo = bit_blend(t << 6, mask_hi, c_hi);
+        hi = bit_blend(t << 2, mask_hi, c_hi);
+    }
+}
+template <int ACT> constexpr uint32_t kMaskLo4 = 0x000f000fu;
+template <int ACT> constexpr uint32_t kBlendLo4 = 0x43004300u | 0x00080008u;
+template <int ACT> constexpr uint32_t kMaskHi4 = ACT == 0 ? 0x00780078u : 0x03c003c0u;
+template <int ACT> constexpr uint32_t kBlendHi4 = ACT == 0 ? (0x41004100u | 0x00400040u) : (0x4c004c00u | 0x02000200u);
+template <int ACT> constexpr float kMulLo4 = 1.0f;
+template <int ACT> constexpr float kBiasLo4 = ACT == 0 ? 136.0f : 24.0f;
+template <int ACT> constexpr float kMulHi4 = kImageMul<4, ACT>;
+template <int ACT> constexpr float kBiasHi4 = kImageBias<4>;
+// the blend operands, opaque to the optimiser (which would otherwise split the blend into two instructions again)
+struct BlendRegs {
+    uint32_t mask_lo, c_lo, mask_hi, c_hi;
+};
+template <int ACT>
+__device__ __forceinline__ BlendRegs blend_regs()
+{
+    BlendRegs r;
+    asm volatile("s_mov_b32 %0, %1" : "=s"(r.mask_lo) : "n"(kMaskLo4<ACT>));
+    asm volatile("s_mov_b32 %0, %1" : "=s"(r.mask_hi) : "n"(kMaskHi4<ACT>));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(r.c_lo) : "n"(kBlendLo4<ACT>));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(r.c_hi) : "n"(kBlendHi4<ACT>));
+    return r;
+}
+// B fragments of the two MFMA column tiles that share byte position jb (low nibble -> b0, high nibble -> b1); w holds
+// this lane's dword of its 8 k rows, unmodified
+template <int ACT>
+__device__ __forceinline__ void expand_pair_blend(const uint32_t (&w)[8], int jb, const BlendRegs &r, u32x4 &b0, u32x4 &b1)
+{
+    const uint32_t sel = 0x0c000c00u | ((4u + jb) << 16) | (uint32_t)jb;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const uint32_t t = __builtin_amdgcn_perm(w[2 * v + 1], w[2 * v], sel);
+        uint32_t lo, hi;
+        expand_byte<ACT>(t, r.mask_lo, r.c_lo, r.mask_hi, r.c_hi, lo, hi);
+        b0[v] = lo;
+        b1[v] = hi;
+    }
+}
+
 constexpr uint32_t kOutOfRange = 0x80000000u;   // lane offset beyond every buffer size: the load returns zero, no traffic
 constexpr int kNonTemporal = 2;                 // cache-policy bit for data that is read once
 

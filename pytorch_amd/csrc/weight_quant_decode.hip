@@ -106,8 +106,7 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             for (int i = 0; i < NT; i++) P[mt][i] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
         const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
-        uint32_t magic;
-        asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "n"(kInt4Magic<ACT>));   // opaque to the optimiser: stays in a VGPR
+        const BlendRegs br = blend_regs<ACT>();
 
 #pragma unroll
         for (int s = 0; s < STEPS; s++) {
@@ -118,8 +117,8 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             uint32_t w0[8], w1[8];
 #pragma unroll
             for (int t = 0; t < 8; t++) {
-                w0[t] = wq[slot][t].x ^ 0x88888888u;
-                w1[t] = wq[slot][t].y ^ 0x88888888u;
+                w0[t] = wq[slot][t].x;
+                w1[t] = wq[slot][t].y;
             }
             u32x4 xs[MT];
 #pragma unroll
@@ -135,7 +134,7 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
 #pragma unroll
                 for (int jb = 0; jb < 4; jb++) {
                     u32x4 b0, b1;
-                    expand_pair<4, ACT>(h ? w1 : w0, jb, magic, b0, b1);
+                    expand_pair_blend<ACT>(h ? w1 : w0, jb, br, b0, b1);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         P[mt][h * 8 + 2 * jb] = mfma_act<ACT>(xs[mt], b0, P[mt][h * 8 + 2 * jb]);
@@ -156,10 +155,9 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             ov[1][i] = (uint32_t)__builtin_amdgcn_ds_bpermute((48 + c) * 4, (int)pq[i]);
         }
         // ---- the single fold: tot = (scale * mul) * (P' + ((offset - bias) / mul) * X), both rescalings exact
-        constexpr float P_MUL = kImageMul<4, ACT>;
-        constexpr float X_BIAS = kImageBias<4>;
 #pragma unroll
         for (int i = 0; i < NT; i++) {
+            const float P_MUL = (i & 1) ? kMulHi4<ACT> : kMulLo4<ACT>, X_BIAS = (i & 1) ? kBiasHi4<ACT> : kBiasLo4<ACT>;
             const uint32_t su = sv[i / 8][(i % 8) / 2], ou = ov[i / 8][(i % 8) / 2];
             const float sc = ((i & 1) ? act_hi<ACT>(su) : act_lo<ACT>(su)) * P_MUL;
             const float of = ((has_offset ? ((i & 1) ? act_hi<ACT>(ou) : act_lo<ACT>(ou)) : 0.0f) - X_BIAS) * (1.0f / P_MUL);

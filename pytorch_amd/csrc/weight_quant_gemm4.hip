@@ -42,34 +42,6 @@ struct WqGemm4Args {
 constexpr int kMaxPolls4 = 1 << 20;
 constexpr int kMaxRows4 = 384;     // beyond this the kernel that expands the weights once per 256 rows (weight_quant_gemm.hip) is faster
 
-// images of the two nibbles of a byte; t = [byte of row 2v, 0, byte of row 2v + 1, 0].  out = mask ? (t ^ c) : c is one
-// three-input bitwise instruction: c carries the image's exponent bits outside the mask and, inside it, the bit that
-// turns the two's-complement nibble into u = w + 8.
-__device__ __forceinline__ uint32_t bit_blend(uint32_t t, uint32_t mask, uint32_t c)
-{
-    return __builtin_amdgcn_bitop3_b32(t, mask, c, 0x6a);   // truth table of (mask & (t ^ c)) | (~mask & c), t the high index bit
-}
-template <int ACT>
-__device__ __forceinline__ void expand_byte(uint32_t t, uint32_t mask_lo, uint32_t c_lo, uint32_t mask_hi, uint32_t c_hi, uint32_t &lo, uint32_t &hi)
-{
-    if constexpr (ACT == 0) {
-        lo = bit_blend(t, mask_lo, c_lo);
-        hi = bit_blend(t >> 1, mask_hi, c_hi);
-    } else {
-        lo = bit_blend(t << 6, mask_hi, c_hi);
-        hi = bit_blend(t << 2, mask_hi, c_hi);
-    }
-}
-template <int ACT> constexpr uint32_t kMaskLo4 = 0x000f000fu;
-template <int ACT> constexpr uint32_t kBlendLo4 = 0x43004300u | 0x00080008u;
-template <int ACT> constexpr uint32_t kMaskHi4 = ACT == 0 ? 0x00780078u : 0x03c003c0u;
-template <int ACT> constexpr uint32_t kBlendHi4 = ACT == 0 ? (0x41004100u | 0x00400040u) : (0x4c004c00u | 0x02000200u);
-// weight = mul * image - bias, per nibble position
-template <int ACT> constexpr float kMulLo4 = 1.0f;
-template <int ACT> constexpr float kBiasLo4 = ACT == 0 ? 136.0f : 24.0f;
-template <int ACT> constexpr float kMulHi4 = kImageMul<4, ACT>;
-template <int ACT> constexpr float kBiasHi4 = kImageBias<4>;
-
 template <int ACT>
 __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
 {
@@ -185,11 +157,7 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     f32x4 Xown = f32x4{0.f, 0.f, 0.f, 0.f};                    // row sums of row tile `wave`
     const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
     const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
-    uint32_t mask_lo, c_lo, mask_hi, c_hi;                     // opaque to the optimiser, which would otherwise undo the blend
-    asm volatile("s_mov_b32 %0, %1" : "=s"(mask_lo) : "n"(kMaskLo4<ACT>));
-    asm volatile("s_mov_b32 %0, %1" : "=s"(mask_hi) : "n"(kMaskHi4<ACT>));
-    asm volatile("v_mov_b32 %0, %1" : "=v"(c_lo) : "n"(kBlendLo4<ACT>));
-    asm volatile("v_mov_b32 %0, %1" : "=v"(c_hi) : "n"(kBlendHi4<ACT>));
+    const BlendRegs br = blend_regs<ACT>();
 
     // fold of a finished group into the running total: tot += (scale * mul) * (P' + ((offset - bias) / mul) * X)
     float scm[4], ofm[4];
@@ -234,8 +202,8 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
             const uint32_t t0 = __builtin_amdgcn_perm(w[2 * v + 1], w[2 * v], sel0);
             const uint32_t t1 = __builtin_amdgcn_perm(w[2 * v + 1], w[2 * v], sel1);
             uint32_t e0, e1, e2, e3;
-            expand_byte<ACT>(t0, mask_lo, c_lo, mask_hi, c_hi, e0, e1);
-            expand_byte<ACT>(t1, mask_lo, c_lo, mask_hi, c_hi, e2, e3);
+            expand_byte<ACT>(t0, br.mask_lo, br.c_lo, br.mask_hi, br.c_hi, e0, e1);
+            expand_byte<ACT>(t1, br.mask_lo, br.c_lo, br.mask_hi, br.c_hi, e2, e3);
             bn[0][v] = e0;
             bn[1][v] = e1;
             bn[2][v] = e2;
