@@ -94,18 +94,19 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     const __amdgpu_buffer_rsrc_t rsrc_o = make_rsrc(has_offset ? p.offset : p.scale, param_bytes);
     int iss_in_group = 0, iss_group = u0;
     const __amdgpu_buffer_rsrc_t rsrc_none = make_rsrc(p.x, 0);      // every access is out of range: zeros, no traffic
-    auto issue_stage = [&](int s) {
+    // a stage's loads are issued in four parts (one activation unit and one weight unit per wavefront each; part 0 also
+    // carries wavefront 0's parameter loads), so that the main loop can spread them over the stage's steps: issued back to
+    // back they hold the wavefront, and with it the matrix pipe, until the vector-memory queue has drained
+    auto issue_part = [&](int s, int i) {
         const bool live = s < NSTG;
         const __amdgpu_buffer_rsrc_t ra = live ? rsrc_a : rsrc_none, rw = live ? rsrc_w : rsrc_none;
         char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
-#pragma unroll
-        for (int i = 0; i < LA; i++) {
+        {
             const int row = 4 * (i * NW + wave) + (lane >> 4);
             const uint32_t vo = (uint32_t)(row * (int)p.ldx * 2 + (((lane & 15) ^ (row & 15)) * 16));
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void *)(sa + (i * NW + wave) * 1024), 16, vo, (uint32_t)(s0 + s) * 256u, 0, 0);
         }
-#pragma unroll
-        for (int i = 0; i < LR; i++) {
+        {
             const int sl = 8 * (i * NW + wave) + (lane >> 3);
             const int row = sl ^ ((sl >> 3) & 1);
             const uint32_t ch = (uint32_t)((lane & 7) ^ (4 * ((row >> 4) & 1)));
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void *)(sr + (i * NW + wave) * 1024), 16, vo,
                                                      (uint32_t)(s0 + s) * (uint32_t)BK * p.ldw_bytes, 0, kNonTemporal);
         }
-        if (wave == 0) {
+        if (i == 0 && wave == 0) {
             const bool first = live && iss_in_group == 0;
             const uint32_t ro = (uint32_t)(p.grouped ? iss_group : 0) * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
             char *dst = prm + (first ? (iss_group & (PRM_SLOTS - 1)) : PRM_SLOTS) * PRM_SLOT;
@@ -124,10 +125,14 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_o, (lds_void *)(dst + 512 + q * 256), 4, vo, ro + q * 256u, 0, 0);
             }
         }
-        if (++iss_in_group == p.gstages) {
+        if (i == 3 && ++iss_in_group == p.gstages) {
             iss_in_group = 0;
             iss_group++;
         }
+    };
+    auto issue_stage = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) issue_part(s, i);
     };
     // everything but the newest stage's loads has landed
     auto wait_older_stages = [&]() {
@@ -212,7 +217,7 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     };
     // one step of 32 k: the MFMAs of step ks with the expansion of step ks + 1 (and, at the start of a group, the fold
     // of the group before) spread between them
-    auto step = [&](const bool fold, const int ks, const char *sa, const char *sr, const char *sa_next, const char *sr_next) {
+    auto step = [&](const bool fold, const int ks, const int s_issue, const char *sa, const char *sr, const char *sa_next, const char *sr_next) {
         u32x4(&bc)[4] = b[ks & 1];
         expand(b[(ks + 1) & 1]);
         read_w(ks + 2 < 4 ? sr : sr_next, (ks + 2) & 3);
@@ -233,6 +238,7 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         }
         Xown = mfma_act<ACT>(AX, ones, Xown);
         AX = read_a(na, nk, wave);
+        issue_part(s_issue, ks);                               // behind the step's LDS reads: the compiler keeps that order
         // interleave: one MFMA, its share of the integer work, one LDS read
 #pragma unroll
         for (int r = 0; r < 17; r++) {
@@ -270,7 +276,6 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         __builtin_amdgcn_s_barrier();                          // stage s + 1 is complete in LDS; everyone is done with stage s - 1
         asm volatile("" ::: "memory");
         const bool last_of_group = ++in_group == p.gstages;
-        issue_stage(s + 3);
 
         const char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
         const char *sa_next = lds + ((s + 1) & 3) * A_BYTES, *sr_next = raw + ((s + 1) & 3) * R_BYTES;
@@ -278,14 +283,14 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         if (pending) {
             fetch_fold_operands(pending_slot);
             __builtin_amdgcn_sched_barrier(0);                 // requested before anything of the step, not between its MFMAs
-            step(true, 0, sa, sr, sa_next, sr_next);
+            step(true, 0, s + 3, sa, sr, sa_next, sr_next);
         } else {
-            step(false, 0, sa, sr, sa_next, sr_next);
+            step(false, 0, s + 3, sa, sr, sa_next, sr_next);
         }
 #pragma unroll
         for (int ks = 1; ks < 4; ks++) {
             __builtin_amdgcn_sched_barrier(0);
-            step(false, ks, sa, sr, sa_next, sr_next);
+            step(false, ks, s + 3, sa, sr, sa_next, sr_next);
         }
         __builtin_amdgcn_sched_barrier(0);
         pending = last_of_group;
