@@ -24,14 +24,17 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed-fp32-ops off: packed FP32 instructions are kept out of generated code on this platform.
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
-                "-Wno-pass-failed"]
+                "-Wno-pass-failed",
+                # MFMA accumulators stay in ordinary vector registers.  Left to itself the compiler puts them into the
+                # accumulation registers whenever a kernel may use 512 registers per lane, and then moves them to and
+                # fro around every vector instruction that touches them (the per-group folds) and, for arrays of
+                # accumulators in loops, around the MFMAs themselves (a register-only probe: 27 clocks per MFMA
+                # instead of 17, and scratch spills in four streaming kernels).
+                "-mllvm", "-amdgpu-mfma-vgpr-form"]
 
 
-# Per-file additions.  The kernels that fold their MFMA sums into float32 totals once per scale group keep the
-# accumulators in ordinary vector registers: the compiler's default (accumulation registers) costs a register move
-# per accumulator element and fold in each direction.
-EXTRA_FLAGS = {"weight_quant_kpacked.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
-               "weight_quant_gemm4.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+# Per-file additions (none at present).
+EXTRA_FLAGS = {}
 
 
 def _run(cmd):
