@@ -64,7 +64,7 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
 // Planner tuning knobs (tuning.hip): 0 = automatic.  Read with knob(); set through mi355_set_tuning() or, once at
 // load time, through the environment variable of the same name.
 enum Knob { kKnobWqSplit, kKnobWqW, kKnobWqgSplit, kKnobWqgBm, kKnobWqGemmOff, kKnobWqkMt, kKnobWqkNw, kKnobWqkKs,
-            kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmStreamKOff, kKnobWqGemm4Off, kKnobCount };
+            kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmDeepOff, kKnobWqGemm4Off, kKnobCount };
 int knob(Knob k);
 
 inline int check_launch()

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     constexpr int UNITS_BP = (UNITS_B + NW - 1) / NW * NW;
     constexpr int LA = UNITS_A / NW, LB = UNITS_BP / NW;     // loads of a wavefront per activation / weight stage
     constexpr int A_BYTES = UNITS_A * 1024, B_BYTES = UNITS_BP * 1024;
-    constexpr int NSA = 2;                                   // activation slots; NS weight slots follow them in LDS
+    constexpr int NSA = NS >= 4 ? NS : 2;                    // activation slots; NS weight slots follow them in LDS
     constexpr uint32_t kOutOfRange = 0x80000000u;            // lane offset beyond every buffer: the load writes zeros
     static_assert(UNITS_A % NW == 0, "A units must divide evenly over the wavefronts");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -219,13 +219,25 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     // everything up to the activations of step kt+1 has landed and only the newest weight refill may be in flight.
     // (With NS = 2 the weights of step kt+2 are requested instead and nothing may stay in flight; small tiles
     // use that to keep two workgroups resident per CU.)
-    static_assert(NS == 2 || NS == 3, "weight slots");
+    // (With NS >= 4, for launches of at most one small tile per CU, activations get NS slots as well and whole stages
+    // are requested NS steps ahead: NS-1 stages in flight per CU instead of one is what a weight stream from HBM
+    // needs when no second workgroup shares the CU.)
+    static_assert(NS >= 2 && NS <= 4 && (NS < 4 || WTM * WTN <= 16), "weight slots");
     issue_a(0, KT);
     issue_b(0, KT);
     issue_a(1, KT);
     issue_b(1, KT);
     if constexpr (NS == 3) issue_b(2, KT);
-    wait_vmcnt<LA + (NS - 1) * LB>();                                  // stage 0 has landed
+    if constexpr (NS >= 4) {
+#pragma unroll
+        for (int st = 2; st < NS; st++) {
+            issue_a(st, KT);
+            issue_b(st, KT);
+        }
+        wait_vmcnt<(NS - 1) * (LA + LB)>();                            // stage 0 has landed
+    } else {
+        wait_vmcnt<LA + (NS - 1) * LB>();                              // stage 0 has landed
+    }
     __syncthreads();
     MI355_READ_FRAGS(af0, bf0, 0, 0)
 
@@ -250,9 +262,10 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             __builtin_amdgcn_sched_barrier(0);
             MI355_MFMA_BLOCK(af0, bf0)
             __builtin_amdgcn_sched_barrier(0);
-            wait_vmcnt_lgkm0<(NS - 2) * LB>();
+            if constexpr (NS >= 4) wait_vmcnt_lgkm0<(NS - 2) * (LA + LB)>();   // stage kt+1 has landed, NS-2 more may be in flight
+            else wait_vmcnt_lgkm0<(NS - 2) * LB>();
             __syncthreads();
-            issue_a(kt + 2, KT);
+            issue_a(kt + NSA, KT);
             issue_b(kt + NS, KT);
             MI355_READ_FRAGS(af0, bf0, kt + 1, 0)
             __builtin_amdgcn_sched_barrier(0);
@@ -644,7 +657,7 @@ __global__ __launch_bounds__(256) void transpose_i8_wide_kernel(const int8_t *__
     }
 }
 
-template <int WGM, int WGN, int WTM, int WTN>
+template <int WGM, int WGN, int WTM, int WTN, int DEEP = 0>
 int launch_qmm(QmmArgs p, hipStream_t s)
 {
     constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
@@ -654,8 +667,9 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     // epilogues better than the deeper ring does.
     constexpr size_t a_bytes = (size_t)(BM / 8) * 1024, b_bytes = (size_t)((BN / 8 + NWL - 1) / NWL * NWL) * 1024;
     constexpr size_t staging_bytes = (size_t)BM * WGN * ((BN / WGN) * 2 + 16);   // epilogue: padded bf16 tile rows
-    constexpr int NS = 2 * a_bytes + 2 * b_bytes <= 80 * 1024 && staging_bytes <= 80 * 1024 ? 2 : 3;
-    constexpr size_t stage_bytes = 2 * a_bytes + NS * b_bytes;
+    // DEEP: that many whole stages, one workgroup per CU (for launches that put at most one of these small tiles on a CU)
+    constexpr int NS = DEEP ? DEEP : 2 * a_bytes + 2 * b_bytes <= 80 * 1024 && staging_bytes <= 80 * 1024 ? 2 : 3;
+    constexpr size_t stage_bytes = (DEEP ? DEEP : 2) * a_bytes + NS * b_bytes;
     constexpr size_t lds_bytes = stage_bytes > staging_bytes ? stage_bytes : staging_bytes;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -854,6 +868,14 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     MI355_QMM_CASE(128, 256, 2, 4)
     MI355_QMM_CASE(128, 192, 2, 4)
     MI355_QMM_CASE(128, 128, 2, 4)
+    {
+        // the 64-row tiles normally rely on two resident workgroups per CU to keep loads in flight; when the launch has
+        // no second workgroup for a CU, one workgroup with a four-stage ring streams the weights instead
+        const int64_t wgs = (int64_t)((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn) * p.S;
+        const bool deep = wgs <= 256 && !knob(kKnobQmmDeepOff);
+        if (deep && c.bm == 64 && c.bn == 256) return launch_qmm<1, 8, 4, 2, 3>(p, s);
+        if (deep && c.bm == 64 && c.bn == 128) return launch_qmm<1, 8, 4, 1, 4>(p, s);
+    }
     MI355_QMM_CASE(64, 256, 1, 8)
     MI355_QMM_CASE(64, 128, 1, 8)
 #undef MI355_QMM_CASE
