@@ -43,7 +43,7 @@ template <int ACT, int MT, int QPT>
 __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
 {
     constexpr int STEPS = 4;                    // 32-row steps of a wavefront's tile
-    constexpr int PFS = MT == 1 ? 4 : 1;        // steps in flight
+    constexpr int PFS = MT == 1 ? 4 : 2;        // steps in flight
     constexpr int NT = 16;                      // MFMA column sets per lane = its 16 consecutive columns
     constexpr int NBW = 256;                    // columns of a strip
     extern __shared__ __attribute__((aligned(16))) char lds[];
