@@ -153,7 +153,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     // B units are padded to a multiple of the wavefront count (rows past the tile read as zero), so every
     // wavefront issues the same number of loads per stage
     auto issue_b = [&](int kt, int KT) {
-        char *slot = lds + NSA * A_BYTES + (kt % NS) * B_BYTES;
+        char *slot = lds + NSA * A_BYTES + (kt % (NS > 0 ? NS : 1)) * B_BYTES;
         const uint32_t vo = kt < KT ? voff_b : kOutOfRange;
 #pragma unroll
         for (int i = 0; i < LB; i++) {
@@ -169,6 +169,98 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 #pragma unroll
         for (int j = 0; j < WTN; j++) acc[i][j] = i32x4v{0, 0, 0, 0};
 
+    if constexpr (NS == 0) {
+        // ---- streaming K loop (at most 64 rows, few workgroups per CU: the weights are a pure HBM stream).  No workgroup
+        // ring and no barrier per K step: a wavefront owns its 16 weight rows (= 16 output columns) for the whole K range
+        // of the workgroup, loads 128 bytes of each row per step straight into registers, four steps in flight - whole cache
+        // lines per instruction (lane l: 16 bytes of row l / 8, and of row 8 + l / 8) - and turns each step around through
+        // a private, XOR-swizzled 2 KiB LDS tile into operand order (a wavefront's LDS operations complete in order, so
+        // this needs no barrier).  Activations are staged through LDS in fragment order, four steps at a time, double
+        // buffered: the loads of the next chunk are issued at the top of a chunk and written to LDS at its end, one
+        // barrier per chunk.
+        static_assert(WGM == 1 && WGN == 8 && WTM == 4 && WTN == 1, "streaming loop: eight wavefronts of 64 rows x 16 columns");
+        constexpr int CH = 4;                                   // steps per chunk of activations
+        constexpr int XBUF = CH * WTM * 2048;                   // bytes of one activation chunk: [step][m tile][half][lane] x 16
+        constexpr int TBUF = 2048;
+        constexpr int R = 4;                                    // weight steps in registers per wavefront
+        char *const tbuf = lds + 2 * XBUF + wave * (2 * TBUF);
+        const int c16 = lane & 15, g4 = lane >> 4;
+        uint32_t voff_w[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int rl = 8 * h + (lane >> 3);
+            voff_w[h] = (uint32_t)((wn * 16 + rl) * (int)p.ldbt + (((lane & 7) ^ ((rl >> 1) & 7)) * 16));
+        }
+        const int t_rd = c16 * 128 + ((g4 ^ ((c16 >> 1) & 7)) * 16);   // chunk g of row c; chunk g + 4 is at slot ^ 4
+        i32x4v wq[R][2];
+        auto load_w = [&](int slot, int st) {
+            const bool ok = st < KT;
+            const uint32_t kb = (uint32_t)(kt0 + st) * BK;
+            wq[slot][0] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? voff_w[0] : kOutOfRange, kb, 2));
+            wq[slot][1] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? voff_w[1] : kOutOfRange, kb, 2));
+        };
+        // staging: the chunk is 64 rows x 512 bytes = 2048 pieces of 16 bytes, four per thread
+        i32x4v xst[4];
+        auto stage_load = [&](int ch) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int pid = (int)threadIdx.x + 512 * j;
+                const int row = pid >> 5, q = pid & 31;
+                const bool ok = ch * CH + (q >> 3) < KT;
+                xst[j] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(
+                    rsrc_a, ok ? (uint32_t)(row * (int)p.lda + q * 16) : kOutOfRange, (uint32_t)(kt0 + ch * CH) * BK, 0));
+            }
+        };
+        auto stage_store = [&](int ch) {
+            char *buf = lds + (ch & 1) * XBUF;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int pid = (int)threadIdx.x + 512 * j;
+                const int row = pid >> 5, q = pid & 31;
+                const int step = q >> 3, t = (q >> 2) & 1, gg = q & 3;
+                *reinterpret_cast<i32x4v *>(buf + ((((step * WTM + (row >> 4)) * 2 + t) * 64) + gg * 16 + (row & 15)) * 16) = xst[j];
+            }
+        };
+        stage_load(0);                              // before the weights: loads retire in order, and these come from cache
+#pragma unroll
+        for (int r = 0; r < R; r++) load_w(r, r);
+        stage_store(0);
+        __syncthreads();
+        *reinterpret_cast<i32x4v *>(tbuf + lane * 16) = wq[0][0];
+        *reinterpret_cast<i32x4v *>(tbuf + 1024 + lane * 16) = wq[0][1];
+        const int nchunks = (KT + CH - 1) / CH;
+        for (int ch = 0; ch < nchunks; ch++) {
+            stage_load(ch + 1);                     // past the end: zeros, no memory traffic
+            const char *xb = lds + (ch & 1) * XBUF + lane * 16;
+#pragma unroll
+            for (int j = 0; j < CH; j++) {
+                const int st = ch * CH + j;
+                i32x4v xa[2][WTM];
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                    for (int mt = 0; mt < WTM; mt++) xa[t][mt] = *reinterpret_cast<const i32x4v *>(xb + ((j * WTM + mt) * 2 + t) * 1024);
+                const char *tr = tbuf + (j & 1) * TBUF;
+                const i32x4v w0 = *reinterpret_cast<const i32x4v *>(tr + t_rd);
+                const i32x4v w1 = *reinterpret_cast<const i32x4v *>(tr + (t_rd ^ 64));
+                {
+                    char *tw = tbuf + ((j + 1) & 1) * TBUF + lane * 16;      // the next step's registers take the other half
+                    *reinterpret_cast<i32x4v *>(tw) = wq[(j + 1) % R][0];
+                    *reinterpret_cast<i32x4v *>(tw + 1024) = wq[(j + 1) % R][1];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                load_w(j % R, st + R);                                       // this step's registers are free again
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int mt = 0; mt < WTM; mt++) acc[mt][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, xa[0][mt], acc[mt][0], 0, 0, 0);
+#pragma unroll
+                for (int mt = 0; mt < WTM; mt++) acc[mt][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, xa[1][mt], acc[mt][0], 0, 0, 0);
+            }
+            stage_store(ch + 1);
+            __syncthreads();
+        }
+        __syncthreads();
+    } else {
     // LDS read addressing: lane reads row (lane % 16) of a 16-row tile, 16-byte chunk (ks*4 + lane/16),
     // stored at slot chunk ^ (row % 8).  For ks = 1 the slot is the ks = 0 slot with bit 2 flipped.
     const int frow = lane & 15;
@@ -181,7 +273,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     i32x4v af0[WTM], bf0[WTN], af1[WTM], bf1[WTN];
 #define MI355_READ_FRAGS(AF, BF, KT_, KS)                                                                        \
     {                                                                                                            \
-        const char *sa_ = lds + ((KT_) % NSA) * A_BYTES + a_off, *sb_ = lds + ((KT_) % NS) * B_BYTES + b_off;    \
+        const char *sa_ = lds + ((KT_) % NSA) * A_BYTES + a_off, *sb_ = lds + ((KT_) % (NS > 0 ? NS : 1)) * B_BYTES + b_off; \
         const int sw_ = sw0 ^ ((KS) * 64);                                                                       \
         _Pragma("unroll") for (int i = 0; i < WTM; i++)                                                          \
             AF[i] = *reinterpret_cast<const i32x4v *>(sa_ + i * 16 * BK + sw_);                                  \
@@ -278,6 +370,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 #undef MI355_READ_FRAGS
 #undef MI355_MFMA_BLOCK
 #undef MI355_INTERLEAVE
+    }
 
     if (p.S > 1) {
         // Split K: every workgroup of the tile publishes its int32 partial sums in register order (16 bytes per
@@ -668,8 +761,9 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     constexpr size_t a_bytes = (size_t)(BM / 8) * 1024, b_bytes = (size_t)((BN / 8 + NWL - 1) / NWL * NWL) * 1024;
     constexpr size_t staging_bytes = (size_t)BM * WGN * ((BN / WGN) * 2 + 16);   // epilogue: padded bf16 tile rows
     // DEEP: that many whole stages, one workgroup per CU (for launches that put at most one of these small tiles on a CU)
-    constexpr int NS = DEEP ? DEEP : 2 * a_bytes + 2 * b_bytes <= 80 * 1024 && staging_bytes <= 80 * 1024 ? 2 : 3;
-    constexpr size_t stage_bytes = (DEEP ? DEEP : 2) * a_bytes + NS * b_bytes;
+    constexpr int NS = DEEP < 0 ? 0 : DEEP ? DEEP : 2 * a_bytes + 2 * b_bytes <= 80 * 1024 && staging_bytes <= 80 * 1024 ? 2 : 3;
+    // DEEP < 0: the streaming K loop (two activation chunks of 32 KiB and a 4 KiB turn-around tile per wavefront)
+    constexpr size_t stage_bytes = DEEP < 0 ? (size_t)2 * 32768 + 8 * 4096 : (DEEP ? DEEP : 2) * a_bytes + NS * b_bytes;
     constexpr size_t lds_bytes = stage_bytes > staging_bytes ? stage_bytes : staging_bytes;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -872,9 +966,10 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
         // the 64-row tiles normally rely on two resident workgroups per CU to keep loads in flight; when the launch has
         // no second workgroup for a CU, one workgroup with a four-stage ring streams the weights instead
         const int64_t wgs = (int64_t)((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn) * p.S;
-        const bool deep = wgs <= 256 && !knob(kKnobQmmDeepOff);
+        const int dk = knob(kKnobQmmDeepOff);              // 1: neither; 2: the ring instead of the streaming loop
+        const bool deep = wgs <= 256 && dk != 1;
         if (deep && c.bm == 64 && c.bn == 256) return launch_qmm<1, 8, 4, 2, 3>(p, s);
-        if (deep && c.bm == 64 && c.bn == 128) return launch_qmm<1, 8, 4, 1, 4>(p, s);
+        if (deep && c.bm == 64 && c.bn == 128) return dk == 2 ? launch_qmm<1, 8, 4, 1, 4>(p, s) : launch_qmm<1, 8, 4, 1, -1>(p, s);
     }
     MI355_QMM_CASE(64, 256, 1, 8)
     MI355_QMM_CASE(64, 128, 1, 8)

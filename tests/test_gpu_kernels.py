@@ -278,9 +278,10 @@ def test_quant_matmul_bias_kinds_and_fp16_output(capi, golden, M, K, N):
 @pytest.mark.parametrize("tile", [64128, 64256])
 @pytest.mark.parametrize("M,K,N", [(64, 128, 1000), (33, 384, 520), (64, 4096, 2048), (16, 2048, 8200)])
 def test_quant_matmul_deep_ring_small_tiles(capi, golden, tile, M, K, N):
-    """Launches with at most one 64-row tile per CU use a ring of whole stages several steps ahead instead of relying on a
-    second resident workgroup: fewer K steps than ring slots, ragged columns, with and without a K split; accumulators
-    bit-identical to the oracle and to the shallow-ring kernel."""
+    """Launches with at most one 64-row tile per CU do not rely on a second resident workgroup: the 64x128 tile streams its
+    weight rows straight into registers (no workgroup ring), the 64x256 tile uses a ring of whole stages several steps
+    ahead.  Fewer K steps than ring slots / register steps, ragged columns and rows, with and without a K split;
+    accumulators bit-identical to the oracle and outputs to the shallow-ring kernel."""
     d = workloads.quant_matmul_inputs(seed=M + N, M=M, K=K, N=N, weight_nk=True, bias=True)
     x1, x2 = d["x1"].cuda(), d["x2"].cuda()
     want = golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy())
@@ -291,12 +292,12 @@ def test_quant_matmul_deep_ring_small_tiles(capi, golden, tile, M, K, N):
                 continue
             capi.set_tuning("MI355_QMM_SPLIT", split)
             outs = []
-            for deep_off in (0, 1):
+            for deep_off in (0, 1, 2):      # streaming loop (64x128) / deep ring (64x256); two resident workgroups; deep ring
                 capi.set_tuning("MI355_QMM_DEEP_OFF", deep_off)
                 acc = capi.quant_matmul(x1, x2, None, out_dtype=torch.int32)
                 assert np.array_equal(acc.cpu().numpy(), want), (tile, split, deep_off)
                 outs.append(capi.quant_matmul(x1, x2, d["scale"].cuda(), d["pertoken_scale"].cuda(), d["bias"].cuda()))
-            assert torch.equal(outs[0], outs[1])
+            assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
     finally:
         for k in ("MI355_QMM_TILE", "MI355_QMM_SPLIT", "MI355_QMM_DEEP_OFF"):
             capi.set_tuning(k, 0)
