@@ -903,7 +903,10 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
 
     const int8_t *bt = b;
     int64_t ldbt = ldb_n;
-    bool tiled = K >= BK && K % BK == 0 && (lda & 15) == 0 && aligned(a, 16);
+    // the tiled kernel addresses a tile's rows with 32-bit buffer offsets: 256 rows of either operand must stay below 2^31
+    const bool offsets_fit = (uint64_t)256 * (uint64_t)lda + (uint64_t)K < (1ull << 31) &&
+                             (uint64_t)256 * (uint64_t)(ldb_k != 1 ? K : ldb_n) + (uint64_t)K < (1ull << 31);
+    bool tiled = K >= BK && K % BK == 0 && (lda & 15) == 0 && aligned(a, 16) && offsets_fit;
     const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n, zero_area);
     char *ws = static_cast<char *>(workspace);
     if (tiled && pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes > 0) {

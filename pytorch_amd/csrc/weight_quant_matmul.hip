@@ -736,28 +736,35 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
 {
     using namespace mi355;
     if (M <= 0 || N <= 0 || K <= 0 || (w_bits != 4 && w_bits != 8) || group_size < 0) return 0;
-    // the largest request over the layouts the streaming kernel accepts (row pitch = row length)
-    const WqPlan pl = make_plan(M, N, K, w_bits, group_size, true, w_bits == 4 ? N / 8 : N, K, nullptr, nullptr, nullptr, nullptr);
-    size_t need = pl.fast ? pl.partial_bytes + pl.counter_bytes : 0;
-    for (int layout = 1; layout <= (w_bits == 8 ? 2 : 1); layout++) {
-        const WqGemmPlan gp = make_wq_gemm_plan(M, N, K, w_bits, group_size, layout, layout == 2 ? K : (w_bits == 4 ? N / 8 : N), K,
-                                                nullptr, nullptr, nullptr, nullptr);
-        const size_t gneed = gp.counter_bytes + gp.partial_bytes;
-        if (gp.ok && gneed > need) need = gneed;
-    }
-    if (w_bits == 4) {                      // decode kernel: its exchange lives in the zero area
-        const WqDecodePlan dp = make_wq_decode_plan(M, N, K, 4, group_size, N / 8, K, nullptr, nullptr, nullptr, nullptr);
-        if (dp.ok && dp.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
-        const WqGemm4Plan g4 = make_wq_gemm4_plan(M, N, K, 4, group_size, N / 8, K, nullptr, nullptr, nullptr, nullptr);
-        if (g4.ok && g4.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
-    }
-    if (w_bits == 4) {                      // words along K
-        const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, K / 8, K, nullptr, nullptr);
-        if (kp.ok && kp.partial_bytes + kp.counter_bytes > need) need = kp.partial_bytes + kp.counter_bytes;
-    }
-    if (w_bits == 8) {                      // the K-major layout may split differently
-        const WqKmPlan km = make_kmajor_plan(M, N, K, group_size, K, K, nullptr, nullptr);
-        if (km.fast && km.partial_bytes + km.counter_bytes > need) need = km.partial_bytes + km.counter_bytes;
+    // The query knows neither strides nor alignments, the launch plans with the real ones: the answer is the largest
+    // request over every layout the kernels accept, once with dense rows (pitch = row length) and once with rows padded
+    // to 128 bytes, which is what lets a shape with a ragged row length onto a fast kernel that the dense pitch rules out.
+    auto pad = [](int64_t v, int64_t to) { return (v + to - 1) / to * to; };
+    size_t need = 0;
+    for (int padded = 0; padded < 2; padded++) {
+        const int64_t ldx = padded ? pad(K, 64) : K;                                  // activation pitch, elements
+        const int64_t ldw_n_major = padded ? pad(w_bits == 4 ? N / 8 : N, w_bits == 4 ? 32 : 128) : (w_bits == 4 ? N / 8 : N);
+        const int64_t ldw_k_major = padded ? pad(w_bits == 4 ? K / 8 : K, w_bits == 4 ? 32 : 128) : (w_bits == 4 ? K / 8 : K);
+        const WqPlan pl = make_plan(M, N, K, w_bits, group_size, true, ldw_n_major, ldx, nullptr, nullptr, nullptr, nullptr);
+        if (pl.fast && pl.partial_bytes + pl.counter_bytes > need) need = pl.partial_bytes + pl.counter_bytes;
+        for (int layout = 1; layout <= (w_bits == 8 ? 2 : 1); layout++) {
+            const WqGemmPlan gp = make_wq_gemm_plan(M, N, K, w_bits, group_size, layout, layout == 2 ? ldw_k_major : ldw_n_major, ldx,
+                                                    nullptr, nullptr, nullptr, nullptr);
+            const size_t gneed = gp.counter_bytes + gp.partial_bytes;
+            if (gp.ok && gneed > need) need = gneed;
+        }
+        if (w_bits == 4) {                  // words along N: the decode and register-expanding kernels exchange in the zero area
+            const WqDecodePlan dp = make_wq_decode_plan(M, N, K, 4, group_size, ldw_n_major, ldx, nullptr, nullptr, nullptr, nullptr);
+            if (dp.ok && dp.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
+            const WqGemm4Plan g4 = make_wq_gemm4_plan(M, N, K, 4, group_size, ldw_n_major, ldx, nullptr, nullptr, nullptr, nullptr);
+            if (g4.ok && g4.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
+            // words along K
+            const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, ldw_k_major, ldx, nullptr, nullptr);
+            if (kp.ok && kp.partial_bytes + kp.counter_bytes > need) need = kp.partial_bytes + kp.counter_bytes;
+        } else {                            // the K-major layout may split differently
+            const WqKmPlan km = make_kmajor_plan(M, N, K, group_size, ldw_k_major, ldx, nullptr, nullptr);
+            if (km.fast && km.partial_bytes + km.counter_bytes > need) need = km.partial_bytes + km.counter_bytes;
+        }
     }
     return need;
 }

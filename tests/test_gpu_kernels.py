@@ -938,6 +938,27 @@ def test_c_abi_rejects_bad_arguments(capi):
         capi.quant_matmul(x1, x2, None, out_dtype=torch.int32, workspace=torch.empty(16, dtype=torch.int8, device="cuda"))
 
 
+@pytest.mark.parametrize("bits,N", [(8, 100), (4, 104)])
+def test_weight_quant_padded_rows_get_their_workspace(capi, golden, bits, N):
+    """The workspace query knows no strides: a weight whose rows are padded to 128 bytes is accepted by kernels (with a K
+    split) that the dense row length rules out, so the query must cover that plan as well."""
+    M, K = 8, 4096
+    if bits == 8:
+        d = workloads.w8a16_inputs(seed=N, M=M, K=K, N=N)
+        gs, cols, pitch = 0, N, 128
+    else:
+        d = workloads.w4a16_inputs(seed=N, M=M, K=K, N=N, group_size=128)
+        gs, cols, pitch = 128, N // 8, 32
+    wide = torch.zeros(K, pitch, dtype=d["weight"].dtype)
+    wide[:, :cols] = d["weight"]
+    w = wide.cuda()[:, :cols]
+    assert w.stride(0) == pitch
+    out = capi.weight_quant_matmul(d["x"].cuda(), w, d["antiquant_scale"].cuda(), d["antiquant_offset"].cuda(), group_size=gs)
+    _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
+                                         _bits(d["antiquant_offset"]), group_size=gs)
+    bf16_gate(out, torch.from_numpy(gold), floor=True)
+
+
 def test_w4a16_repeated_launches_reuse_workspace(capi, golden):
     """The split-K exchange reuses one workspace and its arrival counters across launches: alternate two
     problems many times and check every result (a stale partial sum or counter would show up here)."""
