@@ -255,6 +255,9 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             }
             for (int poll = 0; poll < kMaxPolls; poll++) {
                 bool missing = false;
+                // the polls must be real loads: without a compiler barrier a reload with the operands of the first request is
+                // folded into it, and a wavefront that arrived before the data would spin on a stale register until the bound
+                asm volatile("" ::: "memory");
 #pragma unroll
                 for (int e = 0; e < NQ; e++)
 #pragma unroll

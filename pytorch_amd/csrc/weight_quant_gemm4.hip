@@ -335,6 +335,9 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
                 v[e] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES, SC1);
             for (int poll = 0; poll < kMaxPolls4; poll++) {
                 bool missing = false;
+                // the polls must be real loads: without a compiler barrier a reload with the operands of the first request is
+                // folded into it, and a wavefront that arrived before the data would spin on a stale register until the bound
+                asm volatile("" ::: "memory");
 #pragma unroll
                 for (int e = 0; e < 16; e++)
                     if (v[e][0] == 0u || v[e][1] == 0u || v[e][2] == 0u || v[e][3] == 0u) {
