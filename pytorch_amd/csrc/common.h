@@ -12,6 +12,18 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// 16-byte buffer store.  The store reads its data registers a few cycles after it issues, and the compiler keeps the wait
+// states this needs only for stores whose scalar offset is an immediate: with the offset in a register, an instruction that
+// reuses the data registers may follow at once (seen: a lane group's last word replaced by the next value written to the
+// register, on launches in which the store unit was slow).  The empty wait below has the data as an operand, so the
+// registers stay allocated until two wait states have passed.
+template <int AUX>
+__device__ __forceinline__ void buffer_store_b128(u32x4 data, __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_offset, uint32_t scalar_offset)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, lane_offset, scalar_offset, AUX);
+    asm volatile("s_nop 1" ::"v"(data) : "memory");
+}
+
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 __device__ __forceinline__ float bf16_1(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
@@ -63,6 +75,8 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
 
 // Planner tuning knobs (tuning.hip): 0 = automatic.  Read with knob(); set through mi355_set_tuning() or, once at
 // load time, through the environment variable of the same name.
+// MI355_WQ_GEMM4_OFF: 1 = the register-expanding int4 kernel is not used; 2 = only its variant with one set of wavefronts;
+// 3 = its K-split exchange always writes through to memory.
 enum Knob { kKnobWqSplit, kKnobWqW, kKnobWqgSplit, kKnobWqgBm, kKnobWqGemmOff, kKnobWqkMt, kKnobWqkNw, kKnobWqkKs,
             kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmDeepOff, kKnobWqGemm4Off, kKnobCount };
 int knob(Knob k);

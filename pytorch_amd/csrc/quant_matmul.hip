@@ -388,8 +388,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         for (int i = 0; i < WTM; i++)
 #pragma unroll
             for (int j = 0; j < WTN; j++)
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rsrc_p, lane_off + (i * WTN + j) * 1024,
-                                                       (uint32_t)chunk * CHUNK_BYTES, SC1);
+                buffer_store_b128<SC1>(__builtin_bit_cast(u32x4, acc[i][j]), rsrc_p, lane_off + (i * WTN + j) * 1024,
+                                                       (uint32_t)chunk * CHUNK_BYTES);
         wait_vmcnt<0>();                                          // this wavefront's partial sums have reached the coherence point
         __syncthreads();                                          // (also: every wavefront is done with the LDS stages)
         int &is_last = *reinterpret_cast<int *>(lds);

@@ -164,6 +164,9 @@ __device__ __forceinline__ void expand_pair_blend(const uint32_t (&w)[8], int jb
 }
 
 constexpr uint32_t kOutOfRange = 0x80000000u;   // lane offset beyond every buffer size: the load returns zero, no traffic
+// s_getreg operand for the four-bit id of the XCD (accelerator die with its own L2) the wavefront runs on: register 20
+// (XCC_ID), offset 0, width 4
+constexpr int kHwRegXccId = (3 << 11) | (0 << 6) | 20;
 constexpr int kNonTemporal = 2;                 // cache-policy bit for data that is read once
 
 
@@ -248,8 +251,8 @@ struct TileOut {
             if (p.S == 1)
                 store_out(row0 + row, nl, acc);
             else
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), rsrc_p, partial_off(row0 + row, nl),
-                                                       (uint32_t)chunk * chunk_bytes, SC1);
+                buffer_store_b128<SC1>(__builtin_bit_cast(u32x4, acc), rsrc_p, partial_off(row0 + row, nl),
+                                                       (uint32_t)chunk * chunk_bytes);
         }
     }
 

@@ -234,7 +234,7 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
                 u32x4 bits = __builtin_bit_cast(u32x4, acc[e]);
 #pragma unroll
                 for (int i = 0; i < 4; i++) bits[i] = bits[i] == 0u ? 0x80000000u : bits[i];   // +0 travels as -0: no stored word is zero
-                __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_z, zoff[e], (uint32_t)chunk * zone_chunk_bytes, SC1);   // dead quads: out of range
+                buffer_store_b128<SC1>(bits, rsrc_z, zoff[e], (uint32_t)chunk * zone_chunk_bytes);   // dead quads: out of range
             }
             return;
         }
@@ -309,8 +309,8 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int e = 0; e < NQ; e++)
-                    __builtin_amdgcn_raw_buffer_store_b128(u32x4{0u, 0u, 0u, 0u}, rsrc_z, c0 + i < p.S - 1 ? zoff[e] : kOutOfRange,
-                                                           (uint32_t)(c0 + i) * zone_chunk_bytes, SC1);
+                    buffer_store_b128<SC1>(u32x4{0u, 0u, 0u, 0u}, rsrc_z, c0 + i < p.S - 1 ? zoff[e] : kOutOfRange,
+                                                           (uint32_t)(c0 + i) * zone_chunk_bytes);
         }
     }
 }

@@ -1,25 +1,35 @@
 // npu_weight_quant_batchmatmul, int4 weights packed along N, more than 32 activation rows: a tiled GEMM in which the
 // packed weights never exist in expanded form outside of registers.
 //
-// A workgroup of four wavefronts owns 64 activation rows x one 128-byte strip of the weight rows (256 columns) and
-// walks its K range in stages of 128 rows.  Per stage the activations (64 x 256 B) and the raw strip (128 x 128 B) are
-// copied global -> LDS by direct loads, three stages ahead (four slots), one barrier per stage.  The strip's 32 dword
-// columns form two spans of 16, a dword's four bytes two byte pairs.  A wavefront owns all 64 rows (four MFMA row
-// tiles) x one span x one byte pair: its lane c reads dword 16h + c of its eight k rows back from LDS (eight 4-byte
-// reads per 32 k) and expands the four nibbles of its byte pair into exact bf16 / fp16 images of the integers, i.e.
-// into the B operands of four MFMA column tiles (tile i = columns 128h + 8c + 4jp + i), each of which meets all four
-// row tiles: 16 MFMAs per step for 4 activation fragments and 8 dwords from LDS and ~40 integer instructions, which
-// is what keeps the matrix pipe, and not LDS or the vector ALU, the busiest unit.  No expanded image ever travels
-// through LDS.  Operands of the next step (also across the stage boundary: a stage is complete in LDS one barrier
-// before it is computed) are requested as soon as the registers they replace are free.
+// A workgroup owns 64 activation rows x one 128-byte strip of the weight rows (256 columns) and walks its K range in
+// stages of 128 rows.  Per stage the activations (64 x 256 B) and the raw strip (128 x 128 B) are copied global -> LDS by
+// direct loads into one of four slots.  The strip's 32 dword columns form two spans of 16, a dword's four bytes two
+// byte pairs.  A wavefront owns all 64 rows (four MFMA row tiles) x one span x one byte pair: its lane c reads dword
+// 16h + c of its eight k rows back from LDS (eight 4-byte reads per 32 k) and expands the four nibbles of its byte pair
+// into exact bf16 / fp16 images of the integers, i.e. into the B operands of four MFMA column tiles (tile i = columns
+// 128h + 8c + 4jp + i), each of which meets all four row tiles: 16 MFMAs per step for 4 activation fragments and 8
+// dwords from LDS and ~40 integer instructions.  No expanded image ever travels through LDS.
 // Images (bf16): low nibbles stay where they are, as the low mantissa bits of 128.0 (128 + u, u = w + 8); high nibbles
 // move down one bit into the top mantissa bits of 8.0 (8 + u / 2); fp16: both go to the top mantissa bits of 16.0.
-// Per scale group  out += scale * (P + offset * X)  as in the other kernels: a group ends with a stage (or several),
-// the finished sums are folded tile by tile in front of the MFMAs that restart them with a zero accumulator; the row
-// sums X come from one extra MFMA per step (wavefront i takes row tile i) and travel through LDS.
+// Per scale group  out += scale * (P + offset * X)  as in the other kernels; the row sums X come from one extra MFMA
+// per step (wavefront i takes row tile i) and travel through LDS.
+//
+// Three variants (template parameter MODE).  On this chip a SIMD does not issue a wavefront's vector-ALU instructions
+// while its MFMA executes, but it does issue another wavefront's, so two wavefronts per SIMD are worth ~15 %:
+//   MODE 2 (a scale group per stage) and MODE 1 (one group: per channel): eight wavefronts in two sets of four.  The sets
+//     share the tile; set 0 computes the even stages of the K range and set 1 the odd ones, side by side from two slots
+//     while memory is asked for the next two, one barrier per pair.  Each wavefront must fit 256 registers, so nothing
+//     is requested across a stage boundary and a finished group is folded in a block of its own in front of the next
+//     stage (the other wavefront of the SIMD has matrix work meanwhile).  At the end the sets hand each other half of
+//     their totals through LDS, and each finishes 32 of the 64 rows.
+//   MODE 0 (groups of several stages): four wavefronts, one per SIMD, loads three stages ahead, operands of the next
+//     step (also across the stage boundary) requested as soon as their registers are free, the fold of a finished group
+//     spread between the MFMAs that restart its sums.
 // K may be split over S workgroups per tile (few tiles): all but the last store their float32 sums in register order
 // into the workspace's zero zone, zero mapped to -0.0; the last one (highest index: dispatched after the others) polls
 // until no word is zero, adds in chunk order, writes the output and restores the zeros (weight_quant_decode.hip).
+// The chunks of a tile sit on one XCD and the collector says on which (a word per tile behind the sums): a producer
+// that finds itself there leaves its sums in the shared L2 with ordinary stores, any other writes them through to memory.
 #include "weight_quant_common.h"
 #include "weight_quant_gemm4.h"
 
@@ -37,15 +47,17 @@ struct WqGemm4Args {
     int gstages;                    // stages per scale group
     int grouped;
     int tiles_m, strips, S;
+    int l2_exchange;                // producers on the collector's XCD leave their sums in the L2
 };
 
 constexpr int kMaxPolls4 = 1 << 20;
 constexpr int kMaxRows4 = 384;     // beyond this the kernel that expands the weights once per 256 rows (weight_quant_gemm.hip) is faster
 
-template <int ACT>
-__global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
+template <int ACT, int MODE /* 0: one set of wavefronts; 1: two sets, one scale group; 2: two sets, a group per stage */>
+__global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
 {
-    constexpr int NW = 4, BM = 64, BK = 128, SLOTS = 4;
+    constexpr int SETS = MODE ? 2 : 1;
+    constexpr int NW = 4 * SETS, BM = 64, BK = 128, SLOTS = 4;
     constexpr int A_BYTES = BM * 256, R_BYTES = BK * 128;      // one stage of activations / raw weights
     constexpr int LA = BM / 4 / NW, LR = 16 / NW;              // 1 KiB load units per wavefront and stage
     constexpr int LPS = LA + LR;
@@ -55,12 +67,16 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     char *const raw = lds + SLOTS * A_BYTES;
     char *const prm = raw + SLOTS * R_BYTES;
-    float *const xsum = reinterpret_cast<float *>(prm + (PRM_SLOTS + 1) * PRM_SLOT);   // [2 slots][BM] row sums
+    float *const xsum = reinterpret_cast<float *>(prm + (PRM_SLOTS + 1) * PRM_SLOT);   // [SETS][2 slots][BM] row sums
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, g = lane >> 4;
-    const int h = wave & 1, jp = wave >> 1;
+    // SETS == 2: two sets of four wavefronts share the workgroup's tile; set 0 computes the even stages of the K range, set 1
+    // the odd ones, and their totals meet through LDS at the end.  Every SIMD then holds two wavefronts whose vector-ALU
+    // and matrix work overlap.
+    const int set = wave >> 2, ws = wave & 3;
+    const int h = ws & 1, jp = ws >> 1;
     // workgroups are dealt round-robin to the 8 XCDs.  The row blocks of a strip and the chunks of a tile sit on one
     // XCD (they share the strip resp. the activations in its L2); the last chunk has the tile's highest index.
     const int xcd_slot = blockIdx.x >> 3;
@@ -134,6 +150,39 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
 #pragma unroll
         for (int i = 0; i < 4; i++) issue_part(s, i);
     };
+    // SETS == 2: a stage's 32 load units are dealt to the eight wavefronts; the parameters of the stage's group travel with
+    // it (grouped: one group per stage; per channel: the one parameter row once per set), issued by the first wavefront
+    // of the set that computes the stage.  Nothing is issued past the end: the loop waits for vmcnt(0).
+    auto issue_stage_paired = [&](int s) {
+        if (s >= NSTG) return;
+        char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int u = i * NW + wave;
+            {
+                const int row = 4 * u + (lane >> 4);
+                const uint32_t vo = (uint32_t)(row * (int)p.ldx * 2 + (((lane & 15) ^ (row & 15)) * 16));
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void *)(sa + u * 1024), 16, vo, (uint32_t)(s0 + s) * 256u, 0, 0);
+            }
+            {
+                const int sl = 8 * u + (lane >> 3);
+                const int row = sl ^ ((sl >> 3) & 1);
+                const uint32_t ch = (uint32_t)((lane & 7) ^ (4 * ((row >> 4) & 1)));
+                const uint32_t vo = ch * 16u < strip_valid ? (uint32_t)row * p.ldw_bytes + ch * 16u : kOutOfRange;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void *)(sr + u * 1024), 16, vo,
+                                                         (uint32_t)(s0 + s) * (uint32_t)BK * p.ldw_bytes, 0, kNonTemporal);
+            }
+        }
+        if (wave == 4 * (s & 1) && (p.grouped || s < 2)) {
+            const uint32_t ro = (uint32_t)(p.grouped ? u0 + s : 0) * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
+            char *dst = prm + (p.grouped ? (s & (PRM_SLOTS - 1)) : (s & 1)) * PRM_SLOT;
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_s, (lds_void *)(dst + q * 256), 4, (uint32_t)lane * 4u, ro + q * 256u, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_o, (lds_void *)(dst + 512 + q * 256), 4, (uint32_t)lane * 4u, ro + q * 256u, 0, 0);
+            }
+        }
+    };
     // everything but the newest stage's loads has landed
     auto wait_older_stages = [&]() {
         if (wave == 0) wait_vmcnt<LPS + 4>();
@@ -167,12 +216,11 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     // fold of a finished group into the running total: tot += (scale * mul) * (P' + ((offset - bias) / mul) * X)
     float scm[4], ofm[4];
     f32x4 Xg[4];
-    auto fetch_fold_operands = [&](int group) {
-        const int slot = group & 1;
-        const char *pb = prm + (group & (PRM_SLOTS - 1)) * PRM_SLOT + prm_col;
+    auto fetch_fold_operands = [&](int prm_slot, int xsum_slot) {
+        const char *pb = prm + prm_slot * PRM_SLOT + prm_col;
         const uint32_t sr0 = *reinterpret_cast<const uint32_t *>(pb), sr1 = *reinterpret_cast<const uint32_t *>(pb + 4);
         const uint32_t or0 = *reinterpret_cast<const uint32_t *>(pb + 512), or1 = *reinterpret_cast<const uint32_t *>(pb + 516);
-        const float *xs = xsum + slot * BM + 4 * g;
+        const float *xs = xsum + xsum_slot * BM + 4 * g;
 #pragma unroll
         for (int i = 0; i < 4; i++) Xg[i] = *reinterpret_cast<const f32x4 *>(xs + 16 * i);
         const float sc[4] = {act_lo<ACT>(sr0), act_hi<ACT>(sr0), act_lo<ACT>(sr1), act_hi<ACT>(sr1)};
@@ -217,10 +265,13 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     };
     // one step of 32 k: the MFMAs of step ks with the expansion of step ks + 1 (and, at the start of a group, the fold
     // of the group before) spread between them
-    auto step = [&](const bool fold, const int ks, const int s_issue, const char *sa, const char *sr, const char *sa_next, const char *sr_next) {
+    auto step = [&](const int fold /* 1: fold the finished group and restart the sums; 2: restart only */, const int ks, const int s_issue, const char *sa, const char *sr, const char *sa_next, const char *sr_next) {
+        // SETS == 2: a set's next stage is not complete in LDS before the next barrier, so nothing is requested across the
+        // stage boundary (the other wavefront of the SIMD covers the latency at the start of a stage)
+        constexpr bool CROSS = SETS == 1;
         u32x4(&bc)[4] = b[ks & 1];
-        expand(b[(ks + 1) & 1]);
-        read_w(ks + 2 < 4 ? sr : sr_next, (ks + 2) & 3);
+        if (CROSS || ks + 1 < 4) expand(b[(ks + 1) & 1]);
+        if (CROSS || ks + 2 < 4) read_w(ks + 2 < 4 ? sr : sr_next, (ks + 2) & 3);
         const char *na = ks + 1 < 4 ? sa : sa_next;
         const int nk = (ks + 1) & 3;
 #pragma unroll
@@ -228,22 +279,22 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
 #pragma unroll
             for (int nb = 0; nb < 4; nb++) {
                 if (fold) {
-                    fold_tile(i, nb);
+                    if (fold == 1) fold_tile(i, nb);
                     P[i][nb] = mfma_act<ACT>(AF[i], bc[nb], zero4);
                 } else {
                     P[i][nb] = mfma_act<ACT>(AF[i], bc[nb], P[i][nb]);
                 }
             }
-            AF[i] = read_a(na, nk, i);
+            if (CROSS || ks + 1 < 4) AF[i] = read_a(na, nk, i);
         }
         Xown = mfma_act<ACT>(AX, ones, Xown);
-        AX = read_a(na, nk, wave);
-        issue_part(s_issue, ks);                               // behind the step's LDS reads: the compiler keeps that order
+        if (CROSS || ks + 1 < 4) AX = read_a(na, nk, ws);
+        if (CROSS) issue_part(s_issue, ks);                    // behind the step's LDS reads: the compiler keeps that order
         // interleave: one MFMA, its share of the integer work, one LDS read
 #pragma unroll
         for (int r = 0; r < 17; r++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (fold) __builtin_amdgcn_sched_group_barrier(0x002, 13, 0);
+            if (fold == 1) __builtin_amdgcn_sched_group_barrier(0x002, 13, 0);
             else __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
@@ -255,6 +306,21 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     // the barrier.  The barrier is issued without the fences of __syncthreads(): with direct-to-LDS loads in flight the
     // compiler puts a full vmcnt(0) in front of a fenced barrier, which would wait for the stage that was requested
     // last; the explicit waits above it are what the fence would have to do.
+    // split K: the workgroup that collects a tile's sums says at its start on which XCD it runs (a word behind the
+    // exchange area).  A producer on the same XCD shares its L2 and may leave its sums there with ordinary stores, which
+    // are acknowledged in a fifth of the time of stores that write through to memory; the collector's polls bypass the
+    // vector L1 and see either.
+    constexpr uint32_t WAVE_BYTES = 16 * 64 * 16, TILE_BYTES = 4 * WAVE_BYTES;
+    const uint32_t tiles = (uint32_t)(p.tiles_m * p.strips);
+    const uint32_t flag_base = (uint32_t)(p.S - 1) * tiles * TILE_BYTES;
+    const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, p.S > 1 ? flag_base + tiles * 4u : 0u);
+    const uint32_t my_xcd = __builtin_amdgcn_s_getreg(kHwRegXccId) + 1u;
+    if (p.S > 1 && chunk == p.S - 1 && threadIdx.x == 0)
+        __builtin_amdgcn_raw_buffer_store_b32(my_xcd, rsrc_z, (uint32_t)tile * 4u, flag_base, SC1);
+
+    bool pending = false;
+    int pending_prm = 0, pending_x = 0;
+    if constexpr (SETS == 1) {
     issue_stage(0);
     issue_stage(1);
     wait_older_stages();
@@ -265,11 +331,10 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     read_w(raw, 0);
 #pragma unroll
     for (int i = 0; i < 4; i++) AF[i] = read_a(lds, 0, i);
-    AX = read_a(lds, 0, wave);
+    AX = read_a(lds, 0, ws);
     expand(b[0]);
     read_w(raw, 1);
-    bool pending = false;
-    int pending_slot = 0, in_group = 0, group_row = u0;
+    int in_group = 0, group_row = u0;
     for (int s = 0; s < NSTG; s++) {
         wait_older_stages();
         asm volatile("" ::: "memory");
@@ -281,57 +346,144 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         const char *sa_next = lds + ((s + 1) & 3) * A_BYTES, *sr_next = raw + ((s + 1) & 3) * R_BYTES;
         __builtin_amdgcn_sched_barrier(0);
         if (pending) {
-            fetch_fold_operands(pending_slot);
+            fetch_fold_operands(pending_prm, pending_x);
             __builtin_amdgcn_sched_barrier(0);                 // requested before anything of the step, not between its MFMAs
-            step(true, 0, s + 3, sa, sr, sa_next, sr_next);
+            step(1, 0, s + 3, sa, sr, sa_next, sr_next);
         } else {
-            step(false, 0, s + 3, sa, sr, sa_next, sr_next);
+            step(0, 0, s + 3, sa, sr, sa_next, sr_next);
         }
 #pragma unroll
         for (int ks = 1; ks < 4; ks++) {
             __builtin_amdgcn_sched_barrier(0);
-            step(false, ks, s + 3, sa, sr, sa_next, sr_next);
+            step(0, ks, s + 3, sa, sr, sa_next, sr_next);
         }
         __builtin_amdgcn_sched_barrier(0);
         pending = last_of_group;
-        pending_slot = group_row;
+        pending_prm = group_row & (PRM_SLOTS - 1);
+        pending_x = group_row & 1;
         if (last_of_group) {
-            if (c == 0) *reinterpret_cast<f32x4 *>(xsum + (group_row & 1) * BM + wave * 16 + 4 * g) = Xown;   // read after the next barrier
+            if (c == 0) *reinterpret_cast<f32x4 *>(xsum + (group_row & 1) * BM + ws * 16 + 4 * g) = Xown;   // read after the next barrier
             Xown = zero4;
             in_group = 0;
             group_row++;
         }
     }
+    } else {
+        // two sets: stages 2 it and 2 it + 1 are computed side by side from two slots while memory is asked for the next
+        // two; one barrier per pair
+        issue_stage_paired(0);
+        issue_stage_paired(1);
+        int own = 0;
+        for (int it = 0; 2 * it < NSTG; it++) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();                      // this pair is complete in LDS; everyone is done with the pair before
+            asm volatile("" ::: "memory");
+            issue_stage_paired(2 * it + 2);
+            issue_stage_paired(2 * it + 3);
+            const int s = 2 * it + set;
+            if (s >= NSTG) continue;
+            const char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
+            read_w(sr, 0);
+#pragma unroll
+            for (int i = 0; i < 4; i++) AF[i] = read_a(sa, 0, i);
+            AX = read_a(sa, 0, ws);
+            if (MODE == 2 && pending) {
+                // the other wavefront of the SIMD has matrix work for the time of this fold
+                fetch_fold_operands(pending_prm, pending_x);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int nb = 0; nb < 4; nb++) fold_tile(i, nb);
+            }
+            expand(b[0]);
+            read_w(sr, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            // a group per stage: the sums restart from the MFMA's zero operand.  (Compile time: two copies of the step behind
+            // a branch cost a hundred registers.)
+            step(MODE == 2 ? 2 : 0, 0, 0, sa, sr, sa, sr);
+#pragma unroll
+            for (int ks = 1; ks < 4; ks++) {
+                __builtin_amdgcn_sched_barrier(0);
+                step(0, ks, 0, sa, sr, sa, sr);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const bool last_of_group = p.grouped || s + 2 >= NSTG;
+            pending = last_of_group;
+            pending_prm = p.grouped ? (s & (PRM_SLOTS - 1)) : set;
+            pending_x = 2 * set + (own & 1);
+            if (last_of_group) {
+                if (c == 0) *reinterpret_cast<f32x4 *>(xsum + pending_x * BM + ws * 16 + 4 * g) = Xown;   // read after the next barrier
+                Xown = zero4;
+                own++;
+            }
+        }
+    }
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the refills past the end (zeros) have landed
     __syncthreads();
+    uint32_t collector_xcd = 0;
+    if (p.S > 1 && chunk < p.S - 1) collector_xcd = __builtin_amdgcn_raw_buffer_load_b32(rsrc_z, (uint32_t)tile * 4u, flag_base, SC1);   // used after the fold
     if (pending) {
-        fetch_fold_operands(pending_slot);
+        fetch_fold_operands(pending_prm, pending_x);
 #pragma unroll
         for (int i = 0; i < 4; i++)
 #pragma unroll
             for (int nb = 0; nb < 4; nb++) fold_tile(i, nb);
     }
 
+    // each wavefront finishes NE of its 16 register tiles: all of them, or with two sets the half of the rows that the
+    // sets hand each other through LDS (set 1 keeps row tiles 2 and 3 and moves them to the front)
+    constexpr int NE = 16 / SETS, NI = NE / 4;
+    if constexpr (SETS == 2) {
+        // the stage slots are free
+        f32x4 *red = reinterpret_cast<f32x4 *>(lds) + ws * 16 * 64 + lane;
+        if (set == 0) {
+#pragma unroll
+            for (int e = NE; e < 16; e++) red[e * 64] = tot[e >> 2][e & 3];
+        } else {
+#pragma unroll
+            for (int e = 0; e < NE; e++) red[e * 64] = tot[e >> 2][e & 3];
+        }
+        __syncthreads();
+        if (set == 0) {
+#pragma unroll
+            for (int e = 0; e < NE; e++) tot[e >> 2][e & 3] += red[e * 64];
+        } else {
+#pragma unroll
+            for (int e = 0; e < NE; e++) tot[e >> 2][e & 3] = red[(e + NE) * 64] + tot[(e + NE) >> 2][e & 3];
+        }
+    }
+    const int e_first = set * NE;                              // register tile e of this wavefront is tile e_first + e of the 16
+
     // ---- split K: exchange in register order through the zero zone
     if (p.S > 1) {
-        constexpr uint32_t WAVE_BYTES = 16 * 64 * 16, TILE_BYTES = NW * WAVE_BYTES;
-        const uint32_t tiles = (uint32_t)(p.tiles_m * p.strips);
-        const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, (uint32_t)(p.S - 1) * tiles * TILE_BYTES);
-        const uint32_t lane_off = (uint32_t)tile * TILE_BYTES + (uint32_t)wave * WAVE_BYTES + (uint32_t)lane * 16u;
+        const uint32_t lane_off = (uint32_t)tile * TILE_BYTES + (uint32_t)ws * WAVE_BYTES + (uint32_t)e_first * 1024u + (uint32_t)lane * 16u;
         if (chunk < p.S - 1) {
+            const bool same_l2 = p.l2_exchange && __builtin_amdgcn_readfirstlane(collector_xcd) == my_xcd;
+            u32x4 bits[NE];
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                u32x4 bits = __builtin_bit_cast(u32x4, tot[e >> 2][e & 3]);
+            for (int e = 0; e < NE; e++) {
+                bits[e] = __builtin_bit_cast(u32x4, tot[e >> 2][e & 3]);
 #pragma unroll
-                for (int q = 0; q < 4; q++) bits[q] = bits[q] == 0u ? 0x80000000u : bits[q];   // no stored word is zero
-                __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc_z, lane_off + e * 1024, (uint32_t)chunk * tiles * TILE_BYTES, SC1);
+                for (int q = 0; q < 4; q++) bits[e][q] = bits[e][q] == 0u ? 0x80000000u : bits[e][q];   // no stored word is zero
+            }
+            // one branch around all stores, not one per store: a 16-byte store that ends a basic block may be followed, in the
+            // block the code falls into, by an instruction that overwrites its data registers before the store has read them
+            // (the compiler's wait states for that hazard do not reach across the block boundary)
+            if (same_l2) {
+#pragma unroll
+                for (int e = 0; e < NE; e++)
+                    buffer_store_b128<0>(bits[e], rsrc_z, lane_off + e * 1024, (uint32_t)chunk * tiles * TILE_BYTES);
+            } else {
+#pragma unroll
+                for (int e = 0; e < NE; e++)
+                    buffer_store_b128<SC1>(bits[e], rsrc_z, lane_off + e * 1024, (uint32_t)chunk * tiles * TILE_BYTES);
             }
             return;
         }
         for (int ch = 0; ch < p.S - 1; ch++) {
-            u32x4 v[16];
+            u32x4 v[NE];
 #pragma unroll
-            for (int e = 0; e < 16; e++)
+            for (int e = 0; e < NE; e++)
                 v[e] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES, SC1);
             for (int poll = 0; poll < kMaxPolls4; poll++) {
                 bool missing = false;
@@ -339,7 +491,7 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
                 // folded into it, and a wavefront that arrived before the data would spin on a stale register until the bound
                 asm volatile("" ::: "memory");
 #pragma unroll
-                for (int e = 0; e < 16; e++)
+                for (int e = 0; e < NE; e++)
                     if (v[e][0] == 0u || v[e][1] == 0u || v[e][2] == 0u || v[e][3] == 0u) {
                         v[e] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES, SC1);
                         missing = true;
@@ -348,18 +500,21 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
             }
             // chunk order: ((c0 + c1) + ...) + own
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
+            for (int e = 0; e < NE; e++) {
                 if (ch == 0) P[e >> 2][e & 3] = __builtin_bit_cast(f32x4, v[e]);
                 else P[e >> 2][e & 3] += __builtin_bit_cast(f32x4, v[e]);
             }
         }
 #pragma unroll
-        for (int e = 0; e < 16; e++) tot[e >> 2][e & 3] = P[e >> 2][e & 3] + tot[e >> 2][e & 3];
-        // the zone goes back to zero for the next launch (no branches around the stores: nothing waits for them)
+        for (int e = 0; e < NE; e++) tot[e >> 2][e & 3] = P[e >> 2][e & 3] + tot[e >> 2][e & 3];
+        // the zone goes back to zero for the next launch (no branches around the stores: nothing waits for them).  Ordinary
+        // stores: the next launch is what must see them, and a write-through store to a line that a producer left modified
+        // in the L2 takes several times as long
         for (int ch = 0; ch < p.S - 1; ch++)
 #pragma unroll
-            for (int e = 0; e < 16; e++)
-                __builtin_amdgcn_raw_buffer_store_b128(u32x4{0u, 0u, 0u, 0u}, rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES, SC1);
+            for (int e = 0; e < NE; e++)
+                buffer_store_b128<0>(u32x4{0u, 0u, 0u, 0u}, rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES);
+        if (threadIdx.x == 0) __builtin_amdgcn_raw_buffer_store_b32(0u, rsrc_z, (uint32_t)tile * 4u, flag_base, 0);
     }
 
     // ---- output: lane (c, g) holds rows 16 i + 4 g + q, columns 128 h + 8 c + 4 jp .. + 3: 8 bytes per row
@@ -370,10 +525,10 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     for (int nb = 0; nb < 4; nb++) bv[nb] = p.bias ? act_1<ACT>(p.bias[col + nb]) : 0.0f;
     const bool out_vec = (p.ldo & 3) == 0 && aligned_dev(p.out, 8);
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < NI; i++)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            const int row = m0 + i * 16 + 4 * g + q;
+            const int row = m0 + (i + set * NI) * 16 + 4 * g + q;
             if (row >= p.M) continue;
             const uint32_t lo = pack_act2<ACT>(tot[i][0][q] + bv[0], tot[i][1][q] + bv[1]);
             const uint32_t hi = pack_act2<ACT>(tot[i][2][q] + bv[2], tot[i][3][q] + bv[3]);
@@ -389,15 +544,16 @@ __global__ __launch_bounds__(256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         }
 }
 
-template <int ACT>
+template <int ACT, int MODE>
 int launch4(const WqGemm4Args &p, unsigned grid, hipStream_t s)
 {
-    constexpr size_t lds_bytes = (size_t)4 * 64 * 256 + 4 * 128 * 128 + 9 * 1024 + 2 * 64 * 4;
+    constexpr int SETS = MODE ? 2 : 1;
+    constexpr size_t lds_bytes = (size_t)4 * 64 * 256 + 4 * 128 * 128 + 9 * 1024 + SETS * 2 * 64 * 4;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
-    auto kern = wq_gemm4_kernel<ACT>;
+    auto kern = wq_gemm4_kernel<ACT, MODE>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, s, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * SETS), lds_bytes, s, p);
     return check_launch();
 }
 
@@ -410,7 +566,7 @@ WqGemm4Plan make_wq_gemm4_plan(int64_t M, int64_t N, int64_t K, int w_bits, int6
     const int64_t row_bytes = N / 2, ldw_bytes = ldw_k * 4;
     const int64_t group = group_size > 0 ? group_size : K;
     const bool grouped = group_size > 0 && group != K;
-    pl.ok = !knob(kKnobWqGemm4Off) && w_bits == 4 && M > 32 && M <= kMaxRows4 && K >= 128 && K % 128 == 0 && N % 8 == 0 && (!grouped || group % 128 == 0) &&
+    pl.ok = knob(kKnobWqGemm4Off) != 1 && w_bits == 4 && M > 32 && M <= kMaxRows4 && K >= 128 && K % 128 == 0 && N % 8 == 0 && (!grouped || group % 128 == 0) &&
             ldw_bytes >= row_bytes && ldw_bytes % 16 == 0 && ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) &&
             (w == nullptr || aligned(w, 16)) && (scale == nullptr || aligned(scale, 4)) && (offset == nullptr || aligned(offset, 4)) &&
             (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 31) && (uint64_t)128 * (uint64_t)ldx * 2 + (uint64_t)K * 2 < (1ull << 31) &&
@@ -428,7 +584,8 @@ WqGemm4Plan make_wq_gemm4_plan(int64_t M, int64_t N, int64_t K, int w_bits, int6
     if (S > 8) S = 8;
     if (const int f = knob(kKnobWqgSplit))
         if (f >= 1 && f <= units) S = f;
-    auto zone = [&](int64_t s) { return (uint64_t)(s - 1) * (uint64_t)tiles * (uint64_t)pl.bm * 256u * 4u; };
+    // the sums of S - 1 chunks per tile and one word per tile (the XCD of its collector)
+    auto zone = [&](int64_t s) { return (uint64_t)(s - 1) * (uint64_t)tiles * (uint64_t)pl.bm * 256u * 4u + (uint64_t)tiles * 4u; };
     while (S > 1 && zone(S) > kWorkspaceZoneBytes) S--;
     pl.S = (int)S;
     pl.gstages = (int)(grouped ? group / 128 : stages / S > 0 ? stages : stages);
@@ -466,11 +623,16 @@ int launch_wq_gemm4(const WqGemm4Plan &plan, const void *x, int act_f16, const v
     p.tiles_m = plan.tiles_m;
     p.strips = plan.strips;
     p.S = plan.S;
+    p.l2_exchange = knob(kKnobWqGemm4Off) != 3;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t tiles = (int64_t)plan.tiles_m * plan.strips;
     (void)tiles;
     const unsigned grid = (unsigned)((plan.strips + 7) / 8 * 8 * plan.tiles_m * plan.S);
-    return act_f16 ? launch4<1>(p, grid, s) : launch4<0>(p, grid, s);
+    // two sets of wavefronts where a scale group is one stage (or the whole K range)
+    const bool paired = (!p.grouped || plan.gstages == 1) && knob(kKnobWqGemm4Off) != 2;
+    if (paired && p.grouped) return act_f16 ? launch4<1, 2>(p, grid, s) : launch4<0, 2>(p, grid, s);
+    if (paired) return act_f16 ? launch4<1, 1>(p, grid, s) : launch4<0, 1>(p, grid, s);
+    return act_f16 ? launch4<1, 0>(p, grid, s) : launch4<0, 0>(p, grid, s);
 }
 
 } // namespace mi355

@@ -471,6 +471,45 @@ TILED_CASES = [  # bits, M, K, N, group, float16, bias
 ]
 
 
+PAIRED_CASES = [  # M, K, N, group (0: per channel), float16, forced split
+    (64, 128, 256, 128, False, 0),        # one stage: the second set of wavefronts has nothing to compute
+    (64, 640, 512, 128, False, 0),        # five stages: the sets get three and two
+    (128, 640, 520, 128, True, 2),        # chunks of two and three stages, last strip holds 8 columns
+    (96, 1152, 768, 0, False, 0),         # per channel, nine stages
+    (96, 1152, 768, 0, True, 3),          # per channel, chunks of three stages
+    (384, 2048, 1024, 128, False, 4),
+    (200, 4096, 3584, 128, False, 0),     # ragged last row block, several strips per XCD
+]
+
+
+@pytest.mark.parametrize("case", PAIRED_CASES, ids=lambda c: "-".join(str(v) for v in c))
+def test_weight_quant_int4_register_kernel_variants(capi, golden, case):
+    """The register-expanding int4 kernel with two sets of wavefronts per workgroup (a scale group per stage, or one group),
+    with one set, and with the K-split exchange kept out of the L2: all three must meet the gate, and each must repeat
+    its own result bit for bit (the sets and the chunks add in a fixed order)."""
+    M, K, N, gs, f16, split = case
+    d = workloads.w4a16_inputs(seed=M + N + K, M=M, K=K, N=N, group_size=gs if gs else K)
+    bits_of = _bits
+    if f16:
+        d = _to_f16(d)
+        bits_of = _f16_bits
+    args = [d[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset")]
+    _, gold = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(d["antiquant_scale"]),
+                                         bits_of(d["antiquant_offset"]), group_size=gs if gs else K,
+                                         dtype="fp16" if f16 else "bf16")
+    capi.set_tuning("MI355_WQG_SPLIT", split)
+    try:
+        for variant in (0, 2, 3):          # two sets; one set; two sets, exchange through memory
+            capi.set_tuning("MI355_WQ_GEMM4_OFF", variant)
+            out = capi.weight_quant_matmul(*args, group_size=gs if gs else K)
+            bf16_gate(out, torch.from_numpy(gold))
+            for _ in range(2):
+                assert torch.equal(out, capi.weight_quant_matmul(*args, group_size=gs if gs else K))
+    finally:
+        capi.set_tuning("MI355_WQ_GEMM4_OFF", 0)
+        capi.set_tuning("MI355_WQG_SPLIT", 0)
+
+
 @pytest.mark.parametrize("case", TILED_CASES, ids=lambda c: "-".join(str(v) for v in c))
 def test_weight_quant_tiled_kernel(capi, golden, case):
     bits, M, K, N, gs, f16, with_bias = case[:7]
