@@ -75,8 +75,8 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
 
 // Planner tuning knobs (tuning.hip): 0 = automatic.  Read with knob(); set through mi355_set_tuning() or, once at
 // load time, through the environment variable of the same name.
-// MI355_WQ_GEMM4_OFF: 1 = the register-expanding int4 kernel is not used; 2 = only its variant with one set of wavefronts;
-// 3 = its K-split exchange always writes through to memory.
+// MI355_WQ_GEMM4_OFF / MI355_WQ_DECODE_OFF: 1 = the register-expanding int4 GEMM / the int4 decode kernel is not used;
+// 2 = its K-split exchange always writes through to memory.
 enum Knob { kKnobWqSplit, kKnobWqW, kKnobWqgSplit, kKnobWqgBm, kKnobWqGemmOff, kKnobWqkMt, kKnobWqkNw, kKnobWqkKs,
             kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmDeepOff, kKnobWqGemm4Off, kKnobCount };
 int knob(Knob k);

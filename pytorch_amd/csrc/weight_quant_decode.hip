@@ -31,6 +31,7 @@ struct WqDecArgs {
     int M, N, K;
     int group_rows;                 // rows of a scale group (K when per channel)
     int strips, S;
+    int l2_exchange;                // producers on the collector's XCD leave their sums in the L2
 };
 
 constexpr int kMaxPolls = 1 << 20;
@@ -54,6 +55,15 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
     const int xcd_slot = blockIdx.x >> 3;
     const int strip = (blockIdx.x & 7) + 8 * (xcd_slot / p.S), chunk = xcd_slot % p.S;
     if (strip >= p.strips) return;
+    // The chunks of a strip sit on one XCD.  The collector says on which it runs (a word per strip behind the sums); a
+    // producer that finds itself there leaves its sums in the shared L2 with ordinary stores, which the collector's polls
+    // (they bypass the vector L1) see a microsecond before stores that write through to memory.
+    const uint32_t zone_chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
+    const uint32_t flag_base = zone_chunk_bytes * (uint32_t)(p.S - 1);
+    const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, p.S > 1 ? flag_base + (uint32_t)p.strips * 4u : 0u);
+    const bool collector = p.S > 1 && chunk == p.S - 1;
+    const uint32_t my_xcd = __builtin_amdgcn_s_getreg(kHwRegXccId) + 1u;
+    if (collector && threadIdx.x == 0) __builtin_amdgcn_raw_buffer_store_b32(my_xcd, rsrc_z, (uint32_t)strip * 4u, flag_base, SC1);
     const int row0 = (chunk * 8 + wave) * (32 * STEPS);
     const bool wave_live = row0 < p.K;          // K is a multiple of 128: a wavefront's tile is inside K or wholly outside
     const int n0 = strip * NBW;
@@ -187,9 +197,8 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
         live[e] = row < min(16, p.M - mt * 16) && n0 + nl < p.N;  // N is a multiple of 8: a quad is inside or outside
         zoff[e] = live[e] ? (uint32_t)(((mt * 16 + row) * p.N + n0 + nl) * 4) : kOutOfRange;
     }
-    const uint32_t zone_chunk_bytes = (uint32_t)p.M * (uint32_t)p.N * 4u;
-    const __amdgpu_buffer_rsrc_t rsrc_z = make_rsrc(p.zone, p.S > 1 ? zone_chunk_bytes * (uint32_t)(p.S - 1) : 0u);
-    const bool collector = p.S > 1 && chunk == p.S - 1;
+    uint32_t collector_xcd = 0;
+    if (p.S > 1 && !collector) collector_xcd = __builtin_amdgcn_raw_buffer_load_b32(rsrc_z, (uint32_t)strip * 4u, flag_base, SC1);   // used after the reduction
     // The strip's last workgroup asks for the other chunks' sums before it reduces its own: it was dispatched last, so
     // the others have usually stored theirs by now and the answers arrive while the LDS reduction runs.
     u32x4 v[NQ][CB];
@@ -229,12 +238,19 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
     }
     if (p.S > 1) {
         if (chunk < p.S - 1) {
+            u32x4 bits[NQ];
 #pragma unroll
             for (int e = 0; e < NQ; e++) {
-                u32x4 bits = __builtin_bit_cast(u32x4, acc[e]);
+                bits[e] = __builtin_bit_cast(u32x4, acc[e]);
 #pragma unroll
-                for (int i = 0; i < 4; i++) bits[i] = bits[i] == 0u ? 0x80000000u : bits[i];   // +0 travels as -0: no stored word is zero
-                buffer_store_b128<SC1>(bits, rsrc_z, zoff[e], (uint32_t)chunk * zone_chunk_bytes);   // dead quads: out of range
+                for (int i = 0; i < 4; i++) bits[e][i] = bits[e][i] == 0u ? 0x80000000u : bits[e][i];   // +0 travels as -0: no stored word is zero
+            }
+            if (p.l2_exchange && __builtin_amdgcn_readfirstlane(collector_xcd) == my_xcd) {
+#pragma unroll
+                for (int e = 0; e < NQ; e++) buffer_store_b128<0>(bits[e], rsrc_z, zoff[e], (uint32_t)chunk * zone_chunk_bytes);   // dead quads: out of range
+            } else {
+#pragma unroll
+                for (int e = 0; e < NQ; e++) buffer_store_b128<SC1>(bits[e], rsrc_z, zoff[e], (uint32_t)chunk * zone_chunk_bytes);
             }
             return;
         }
@@ -303,15 +319,17 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
     }
     if (p.S > 1) {
         // the zone goes back to zero for the next launch; no branch around the stores (a dead quad or chunk gets an
-        // out-of-range offset), so nothing waits for their acknowledgements
+        // out-of-range offset), so nothing waits for their acknowledgements.  Ordinary stores: the next launch is what must
+        // see them, and a write-through store to a line that a producer left modified in the L2 takes several times as long
         for (int c0 = 0; c0 < p.S - 1; c0 += 4) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int e = 0; e < NQ; e++)
-                    buffer_store_b128<SC1>(u32x4{0u, 0u, 0u, 0u}, rsrc_z, c0 + i < p.S - 1 ? zoff[e] : kOutOfRange,
-                                                           (uint32_t)(c0 + i) * zone_chunk_bytes);
+                    buffer_store_b128<0>(u32x4{0u, 0u, 0u, 0u}, rsrc_z, c0 + i < p.S - 1 ? zoff[e] : kOutOfRange,
+                                         (uint32_t)(c0 + i) * zone_chunk_bytes);
         }
+        if (threadIdx.x == 0) __builtin_amdgcn_raw_buffer_store_b32(0u, rsrc_z, (uint32_t)strip * 4u, flag_base, 0);
     }
 }
 
@@ -325,7 +343,7 @@ WqDecodePlan make_wq_decode_plan(int64_t M, int64_t N, int64_t K, int w_bits, in
     const int64_t group = group_size > 0 ? group_size : K;
     pl.grouped = group_size > 0 && group != K;
     // a wavefront's 128 rows lie inside one scale group; every offset the kernel forms fits in 32 bits
-    pl.ok = !knob(kKnobWqDecodeOff) && w_bits == 4 && M >= 1 && M <= 32 && K >= 128 && K % 128 == 0 && N % 8 == 0 &&
+    pl.ok = knob(kKnobWqDecodeOff) != 1 && w_bits == 4 && M >= 1 && M <= 32 && K >= 128 && K % 128 == 0 && N % 8 == 0 &&
             (pl.grouped ? group % 128 == 0 : true) && ldw_bytes >= row_bytes && ldw_bytes % 8 == 0 && ldx % 8 == 0 &&
             (x == nullptr || aligned(x, 16)) && (w == nullptr || aligned(w, 8)) && (scale == nullptr || aligned(scale, 16)) &&
             (offset == nullptr || aligned(offset, 16)) && (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 31) &&
@@ -334,7 +352,7 @@ WqDecodePlan make_wq_decode_plan(int64_t M, int64_t N, int64_t K, int w_bits, in
     pl.mt = M <= 16 ? 1 : 2;
     pl.strips = (int)((row_bytes + 127) / 128);
     pl.S = (int)((K + 1023) / 1024);
-    pl.zone_bytes = pl.S > 1 ? (size_t)(pl.S - 1) * (size_t)M * (size_t)N * 4 : 0;
+    pl.zone_bytes = pl.S > 1 ? (size_t)(pl.S - 1) * (size_t)M * (size_t)N * 4 + (size_t)pl.strips * 4 : 0;   // sums, and a word per strip
     if (pl.zone_bytes > kWorkspaceZoneBytes || (uint64_t)pl.strips * pl.S > 0x7fffffffu) pl.ok = false;
     return pl;
 }
@@ -361,6 +379,7 @@ int launch_wq_decode(const WqDecodePlan &plan, const void *x, int act_f16, const
     p.group_rows = (int)(plan.grouped ? group_size : K);
     p.strips = plan.strips;
     p.S = plan.S;
+    p.l2_exchange = knob(kKnobWqDecodeOff) != 2;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int rows = (int)(M < 16 ? M : 16);
     const size_t lds_bytes = (size_t)8 * rows * 256 * sizeof(float);

@@ -12,19 +12,16 @@
 // Images (bf16): low nibbles stay where they are, as the low mantissa bits of 128.0 (128 + u, u = w + 8); high nibbles
 // move down one bit into the top mantissa bits of 8.0 (8 + u / 2); fp16: both go to the top mantissa bits of 16.0.
 // Per scale group  out += scale * (P + offset * X)  as in the other kernels; the row sums X come from one extra MFMA
-// per step (wavefront i takes row tile i) and travel through LDS.
+// per step (wavefront i of a set takes row tile i) and travel through LDS.
 //
-// Three variants (template parameter MODE).  On this chip a SIMD does not issue a wavefront's vector-ALU instructions
-// while its MFMA executes, but it does issue another wavefront's, so two wavefronts per SIMD are worth ~15 %:
-//   MODE 2 (a scale group per stage) and MODE 1 (one group: per channel): eight wavefronts in two sets of four.  The sets
-//     share the tile; set 0 computes the even stages of the K range and set 1 the odd ones, side by side from two slots
-//     while memory is asked for the next two, one barrier per pair.  Each wavefront must fit 256 registers, so nothing
-//     is requested across a stage boundary and a finished group is folded in a block of its own in front of the next
-//     stage (the other wavefront of the SIMD has matrix work meanwhile).  At the end the sets hand each other half of
-//     their totals through LDS, and each finishes 32 of the 64 rows.
-//   MODE 0 (groups of several stages): four wavefronts, one per SIMD, loads three stages ahead, operands of the next
-//     step (also across the stage boundary) requested as soon as their registers are free, the fold of a finished group
-//     spread between the MFMAs that restart its sums.
+// A SIMD of this chip does not issue a wavefront's vector-ALU instructions while that wavefront's MFMA executes, but it
+// does issue another wavefront's, so the workgroup has eight wavefronts in two sets of four, two per SIMD.  The sets
+// share the tile; set 0 computes the even stages of the K range and set 1 the odd ones, side by side from two slots
+// while memory is asked for the next two, one barrier per pair.  Both fold their share of a scale group with the
+// group's parameters and their own row sums (the fold is linear).  Each wavefront must fit 256 registers, so nothing is
+// requested across a stage boundary and a finished group is folded in a block of its own in front of the next stage
+// (the other wavefront of the SIMD has matrix work meanwhile).  At the end the sets hand each other half of their totals
+// through LDS, and each finishes 32 of the 64 rows.
 // K may be split over S workgroups per tile (few tiles): all but the last store their float32 sums in register order
 // into the workspace's zero zone, zero mapped to -0.0; the last one (highest index: dispatched after the others) polls
 // until no word is zero, adds in chunk order, writes the output and restores the zeros (weight_quant_decode.hip).
@@ -51,30 +48,24 @@ struct WqGemm4Args {
 };
 
 constexpr int kMaxPolls4 = 1 << 20;
-constexpr int kMaxRows4 = 384;     // beyond this the kernel that expands the weights once per 256 rows (weight_quant_gemm.hip) is faster
 
-template <int ACT, int MODE /* 0: one set of wavefronts; 1: two sets, one scale group; 2: two sets, a group per stage */>
-__global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqGemm4Args p)
+// STAGE_GROUPS: a scale group is one stage, so every stage restarts the group's sums
+template <int ACT, bool STAGE_GROUPS>
+__global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
 {
-    constexpr int SETS = MODE ? 2 : 1;
-    constexpr int NW = 4 * SETS, BM = 64, BK = 128, SLOTS = 4;
+    constexpr int SETS = 2, NW = 4 * SETS, BM = 64, BK = 128, SLOTS = 4;
     constexpr int A_BYTES = BM * 256, R_BYTES = BK * 128;      // one stage of activations / raw weights
-    constexpr int LA = BM / 4 / NW, LR = 16 / NW;              // 1 KiB load units per wavefront and stage
-    constexpr int LPS = LA + LR;
     constexpr int PRM_SLOT = 1024;                             // [256 scales | 256 offsets], 16 bits each
-    constexpr int PRM_SLOTS = 8;                               // groups whose parameters are in LDS (+ 1 slot nobody reads)
+    constexpr int PRM_SLOTS = 8;                               // groups whose parameters are in LDS
     constexpr int SC1 = 16;                                    // cache-policy bit: agent scope
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     char *const raw = lds + SLOTS * A_BYTES;
     char *const prm = raw + SLOTS * R_BYTES;
-    float *const xsum = reinterpret_cast<float *>(prm + (PRM_SLOTS + 1) * PRM_SLOT);   // [SETS][2 slots][BM] row sums
+    float *const xsum = reinterpret_cast<float *>(prm + PRM_SLOTS * PRM_SLOT);   // [SETS][2 slots][BM] row sums
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, g = lane >> 4;
-    // SETS == 2: two sets of four wavefronts share the workgroup's tile; set 0 computes the even stages of the K range, set 1
-    // the odd ones, and their totals meet through LDS at the end.  Every SIMD then holds two wavefronts whose vector-ALU
-    // and matrix work overlap.
     const int set = wave >> 2, ws = wave & 3;
     const int h = ws & 1, jp = ws >> 1;
     // workgroups are dealt round-robin to the 8 XCDs.  The row blocks of a strip and the chunks of a tile sit on one
@@ -101,59 +92,14 @@ __global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqG
     const uint32_t strip_valid = min(128u, p.row_bytes - (uint32_t)strip * 128u);
     const __amdgpu_buffer_rsrc_t rsrc_w =
         make_rsrc(static_cast<const char *>(p.w) + (size_t)strip * 128, (uint32_t)(p.K - 1) * p.ldw_bytes + strip_valid);
-    // parameters of a scale group (the strip's 256 scales and offsets) travel with the group's first stage, copied
-    // global -> LDS by wavefront 0.  It issues its four parameter loads with every stage (for the other stages of a
-    // group they move no bytes and point at a slot nobody reads), so every wavefront's loads per stage are a constant.
     const bool has_offset = p.offset != nullptr;
     const uint32_t param_bytes = (uint32_t)(p.grouped ? units : 1) * (uint32_t)p.N * 2u;
     const __amdgpu_buffer_rsrc_t rsrc_s = make_rsrc(p.scale, param_bytes);
     const __amdgpu_buffer_rsrc_t rsrc_o = make_rsrc(has_offset ? p.offset : p.scale, param_bytes);
-    int iss_in_group = 0, iss_group = u0;
-    const __amdgpu_buffer_rsrc_t rsrc_none = make_rsrc(p.x, 0);      // every access is out of range: zeros, no traffic
-    // a stage's loads are issued in four parts (one activation unit and one weight unit per wavefront each; part 0 also
-    // carries wavefront 0's parameter loads), so that the main loop can spread them over the stage's steps: issued back to
-    // back they hold the wavefront, and with it the matrix pipe, until the vector-memory queue has drained
-    auto issue_part = [&](int s, int i) {
-        const bool live = s < NSTG;
-        const __amdgpu_buffer_rsrc_t ra = live ? rsrc_a : rsrc_none, rw = live ? rsrc_w : rsrc_none;
-        char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
-        {
-            const int row = 4 * (i * NW + wave) + (lane >> 4);
-            const uint32_t vo = (uint32_t)(row * (int)p.ldx * 2 + (((lane & 15) ^ (row & 15)) * 16));
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void *)(sa + (i * NW + wave) * 1024), 16, vo, (uint32_t)(s0 + s) * 256u, 0, 0);
-        }
-        {
-            const int sl = 8 * (i * NW + wave) + (lane >> 3);
-            const int row = sl ^ ((sl >> 3) & 1);
-            const uint32_t ch = (uint32_t)((lane & 7) ^ (4 * ((row >> 4) & 1)));
-            const uint32_t vo = ch * 16u < strip_valid ? (uint32_t)row * p.ldw_bytes + ch * 16u : kOutOfRange;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void *)(sr + (i * NW + wave) * 1024), 16, vo,
-                                                     (uint32_t)(s0 + s) * (uint32_t)BK * p.ldw_bytes, 0, kNonTemporal);
-        }
-        if (i == 0 && wave == 0) {
-            const bool first = live && iss_in_group == 0;
-            const uint32_t ro = (uint32_t)(p.grouped ? iss_group : 0) * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
-            char *dst = prm + (first ? (iss_group & (PRM_SLOTS - 1)) : PRM_SLOTS) * PRM_SLOT;
-            const uint32_t vo = first ? (uint32_t)lane * 4u : kOutOfRange;
-#pragma unroll
-            for (int q = 0; q < 2; q++) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_s, (lds_void *)(dst + q * 256), 4, vo, ro + q * 256u, 0, 0);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_o, (lds_void *)(dst + 512 + q * 256), 4, vo, ro + q * 256u, 0, 0);
-            }
-        }
-        if (i == 3 && ++iss_in_group == p.gstages) {
-            iss_in_group = 0;
-            iss_group++;
-        }
-    };
+    // a stage's 32 load units are dealt to the eight wavefronts; the parameters of a scale group (the strip's 256 scales
+    // and offsets) travel with its first stage, issued by the first wavefront of the set that computes that stage.
+    // Nothing is issued past the end: the loop waits for vmcnt(0).
     auto issue_stage = [&](int s) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) issue_part(s, i);
-    };
-    // SETS == 2: a stage's 32 load units are dealt to the eight wavefronts; the parameters of the stage's group travel with
-    // it (grouped: one group per stage; per channel: the one parameter row once per set), issued by the first wavefront
-    // of the set that computes the stage.  Nothing is issued past the end: the loop waits for vmcnt(0).
-    auto issue_stage_paired = [&](int s) {
         if (s >= NSTG) return;
         char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
 #pragma unroll
@@ -173,20 +119,16 @@ __global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqG
                                                          (uint32_t)(s0 + s) * (uint32_t)BK * p.ldw_bytes, 0, kNonTemporal);
             }
         }
-        if (wave == 4 * (s & 1) && (p.grouped || s < 2)) {
-            const uint32_t ro = (uint32_t)(p.grouped ? u0 + s : 0) * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
-            char *dst = prm + (p.grouped ? (s & (PRM_SLOTS - 1)) : (s & 1)) * PRM_SLOT;
+        const int grp = s / p.gstages;
+        if (wave == 4 * (s & 1) && s == grp * p.gstages) {
+            const uint32_t ro = (uint32_t)(p.grouped ? u0 + grp : 0) * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
+            char *dst = prm + (grp & (PRM_SLOTS - 1)) * PRM_SLOT;
 #pragma unroll
             for (int q = 0; q < 2; q++) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_s, (lds_void *)(dst + q * 256), 4, (uint32_t)lane * 4u, ro + q * 256u, 0, 0);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_o, (lds_void *)(dst + 512 + q * 256), 4, (uint32_t)lane * 4u, ro + q * 256u, 0, 0);
             }
         }
-    };
-    // everything but the newest stage's loads has landed
-    auto wait_older_stages = [&]() {
-        if (wave == 0) wait_vmcnt<LPS + 4>();
-        else wait_vmcnt<LPS>();
     };
 
     // ---- LDS read addresses
@@ -208,7 +150,7 @@ __global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqG
             P[i][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
             tot[i][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-    f32x4 Xown = f32x4{0.f, 0.f, 0.f, 0.f};                    // row sums of row tile `wave`
+    f32x4 Xown = f32x4{0.f, 0.f, 0.f, 0.f};                    // row sums of row tile `ws`
     const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
     const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
     const BlendRegs br = blend_regs<ACT>();
@@ -238,9 +180,10 @@ __global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqG
         for (int q = 0; q < 4; q++) tot[i][nb][q] = __builtin_fmaf(scm[nb], __builtin_fmaf(ofm[nb], Xg[i][q], P[i][nb][q]), tot[i][nb][q]);
     };
 
-    // ---- operands of a step: raw dwords are requested two steps ahead (they are expanded one step ahead, between the
-    // MFMAs of the step before), activation fragments one step ahead, each into the registers of the fragment that
-    // was just used
+    // ---- operands of a step, all from the stage's own slots (a set's next stage is not complete in LDS before the next
+    // barrier; the other wavefront of the SIMD covers the latency at the start of a stage): raw dwords are requested two
+    // steps ahead (they are expanded one step ahead, between the MFMAs of the step before), activation fragments one
+    // step ahead, each into the registers of the fragment that was just used
     uint32_t w[8];
     u32x4 AF[4], AX, b[2][4];
     auto read_w = [&](const char *sr, int ks) {
@@ -263,49 +206,28 @@ __global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqG
             bn[3][v] = e3;
         }
     };
-    // one step of 32 k: the MFMAs of step ks with the expansion of step ks + 1 (and, at the start of a group, the fold
-    // of the group before) spread between them
-    auto step = [&](const int fold /* 1: fold the finished group and restart the sums; 2: restart only */, const int ks, const int s_issue, const char *sa, const char *sr, const char *sa_next, const char *sr_next) {
-        // SETS == 2: a set's next stage is not complete in LDS before the next barrier, so nothing is requested across the
-        // stage boundary (the other wavefront of the SIMD covers the latency at the start of a stage)
-        constexpr bool CROSS = SETS == 1;
+    // one step of 32 k: the MFMAs of step ks with the expansion of step ks + 1 spread between them
+    auto step = [&](const bool restart /* the sums start from the MFMA's zero operand */, const int ks, const char *sa, const char *sr) {
         u32x4(&bc)[4] = b[ks & 1];
-        if (CROSS || ks + 1 < 4) expand(b[(ks + 1) & 1]);
-        if (CROSS || ks + 2 < 4) read_w(ks + 2 < 4 ? sr : sr_next, (ks + 2) & 3);
-        const char *na = ks + 1 < 4 ? sa : sa_next;
-        const int nk = (ks + 1) & 3;
+        if (ks + 1 < 4) expand(b[(ks + 1) & 1]);
+        if (ks + 2 < 4) read_w(sr, ks + 2);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
 #pragma unroll
-            for (int nb = 0; nb < 4; nb++) {
-                if (fold) {
-                    if (fold == 1) fold_tile(i, nb);
-                    P[i][nb] = mfma_act<ACT>(AF[i], bc[nb], zero4);
-                } else {
-                    P[i][nb] = mfma_act<ACT>(AF[i], bc[nb], P[i][nb]);
-                }
-            }
-            if (CROSS || ks + 1 < 4) AF[i] = read_a(na, nk, i);
+            for (int nb = 0; nb < 4; nb++) P[i][nb] = mfma_act<ACT>(AF[i], bc[nb], restart ? zero4 : P[i][nb]);
+            if (ks + 1 < 4) AF[i] = read_a(sa, ks + 1, i);
         }
         Xown = mfma_act<ACT>(AX, ones, Xown);
-        if (CROSS || ks + 1 < 4) AX = read_a(na, nk, ws);
-        if (CROSS) issue_part(s_issue, ks);                    // behind the step's LDS reads: the compiler keeps that order
+        if (ks + 1 < 4) AX = read_a(sa, ks + 1, ws);
         // interleave: one MFMA, its share of the integer work, one LDS read
 #pragma unroll
         for (int r = 0; r < 17; r++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (fold == 1) __builtin_amdgcn_sched_group_barrier(0x002, 13, 0);
-            else __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
     };
 
-    // ---- main loop.  Stage s is computed from slot s % 4 while memory is asked for stage s + 3.  Loads are never skipped
-    // (a stage past the end gets an out-of-range lane offset and moves no bytes), so "everything but the newest stage's
-    // loads" at the top means: stage s + 1, whose first operands the last steps of stage s request, is complete behind
-    // the barrier.  The barrier is issued without the fences of __syncthreads(): with direct-to-LDS loads in flight the
-    // compiler puts a full vmcnt(0) in front of a fenced barrier, which would wait for the stage that was requested
-    // last; the explicit waits above it are what the fence would have to do.
     // split K: the workgroup that collects a tile's sums says at its start on which XCD it runs (a word behind the
     // exchange area).  A producer on the same XCD shares its L2 and may leave its sums there with ordinary stores, which
     // are acknowledged in a fifth of the time of stores that write through to memory; the collector's polls bypass the
@@ -318,107 +240,63 @@ __global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqG
     if (p.S > 1 && chunk == p.S - 1 && threadIdx.x == 0)
         __builtin_amdgcn_raw_buffer_store_b32(my_xcd, rsrc_z, (uint32_t)tile * 4u, flag_base, SC1);
 
+    // ---- main loop: stages 2 it and 2 it + 1 are computed side by side from two slots while memory is asked for the
+    // next two; one barrier per pair.  The barrier is issued without the fences of __syncthreads(): the explicit wait
+    // above it is what the fence would have to do.
     bool pending = false;
     int pending_prm = 0, pending_x = 0;
-    if constexpr (SETS == 1) {
     issue_stage(0);
     issue_stage(1);
-    wait_older_stages();
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();                              // stage 0 is complete in LDS
-    asm volatile("" ::: "memory");
-    issue_stage(2);
-    read_w(raw, 0);
-#pragma unroll
-    for (int i = 0; i < 4; i++) AF[i] = read_a(lds, 0, i);
-    AX = read_a(lds, 0, ws);
-    expand(b[0]);
-    read_w(raw, 1);
-    int in_group = 0, group_row = u0;
-    for (int s = 0; s < NSTG; s++) {
-        wait_older_stages();
+    int own = 0;
+    for (int it = 0; 2 * it < NSTG; it++) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                          // this pair is complete in LDS; everyone is done with the pair before
         asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_barrier();                          // stage s + 1 is complete in LDS; everyone is done with stage s - 1
-        asm volatile("" ::: "memory");
-        const bool last_of_group = ++in_group == p.gstages;
-
+        issue_stage(2 * it + 2);
+        issue_stage(2 * it + 3);
+        const int s = 2 * it + set;
+        if (s >= NSTG) continue;
+        const int grp = s / p.gstages;
         const char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
-        const char *sa_next = lds + ((s + 1) & 3) * A_BYTES, *sr_next = raw + ((s + 1) & 3) * R_BYTES;
-        __builtin_amdgcn_sched_barrier(0);
+        read_w(sr, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) AF[i] = read_a(sa, 0, i);
+        AX = read_a(sa, 0, ws);
         if (pending) {
+            // the other wavefront of the SIMD has matrix work for the time of this fold
             fetch_fold_operands(pending_prm, pending_x);
-            __builtin_amdgcn_sched_barrier(0);                 // requested before anything of the step, not between its MFMAs
-            step(1, 0, s + 3, sa, sr, sa_next, sr_next);
-        } else {
-            step(0, 0, s + 3, sa, sr, sa_next, sr_next);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++) {
+                    fold_tile(i, nb);
+                    if (!STAGE_GROUPS) P[i][nb] = zero4;       // otherwise the next step restarts the sums
+                }
         }
+        expand(b[0]);
+        read_w(sr, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        // Compile time, not a branch: two copies of the step behind a branch cost a hundred registers, so groups of several
+        // stages clear the sums after the fold instead.
+        step(STAGE_GROUPS, 0, sa, sr);
 #pragma unroll
         for (int ks = 1; ks < 4; ks++) {
             __builtin_amdgcn_sched_barrier(0);
-            step(0, ks, s + 3, sa, sr, sa_next, sr_next);
+            step(false, ks, sa, sr);
         }
         __builtin_amdgcn_sched_barrier(0);
+        // the set's share of a group ends with its last stage inside the group
+        const bool last_of_group = s + 2 >= NSTG || (s + 2) / p.gstages != grp;
         pending = last_of_group;
-        pending_prm = group_row & (PRM_SLOTS - 1);
-        pending_x = group_row & 1;
+        pending_prm = grp & (PRM_SLOTS - 1);
+        pending_x = 2 * set + (own & 1);
         if (last_of_group) {
-            if (c == 0) *reinterpret_cast<f32x4 *>(xsum + (group_row & 1) * BM + ws * 16 + 4 * g) = Xown;   // read after the next barrier
+            if (c == 0) *reinterpret_cast<f32x4 *>(xsum + pending_x * BM + ws * 16 + 4 * g) = Xown;   // read after the next barrier
             Xown = zero4;
-            in_group = 0;
-            group_row++;
+            own++;
         }
     }
-    } else {
-        // two sets: stages 2 it and 2 it + 1 are computed side by side from two slots while memory is asked for the next
-        // two; one barrier per pair
-        issue_stage_paired(0);
-        issue_stage_paired(1);
-        int own = 0;
-        for (int it = 0; 2 * it < NSTG; it++) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __builtin_amdgcn_s_barrier();                      // this pair is complete in LDS; everyone is done with the pair before
-            asm volatile("" ::: "memory");
-            issue_stage_paired(2 * it + 2);
-            issue_stage_paired(2 * it + 3);
-            const int s = 2 * it + set;
-            if (s >= NSTG) continue;
-            const char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
-            read_w(sr, 0);
-#pragma unroll
-            for (int i = 0; i < 4; i++) AF[i] = read_a(sa, 0, i);
-            AX = read_a(sa, 0, ws);
-            if (MODE == 2 && pending) {
-                // the other wavefront of the SIMD has matrix work for the time of this fold
-                fetch_fold_operands(pending_prm, pending_x);
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-#pragma unroll
-                    for (int nb = 0; nb < 4; nb++) fold_tile(i, nb);
-            }
-            expand(b[0]);
-            read_w(sr, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            // a group per stage: the sums restart from the MFMA's zero operand.  (Compile time: two copies of the step behind
-            // a branch cost a hundred registers.)
-            step(MODE == 2 ? 2 : 0, 0, 0, sa, sr, sa, sr);
-#pragma unroll
-            for (int ks = 1; ks < 4; ks++) {
-                __builtin_amdgcn_sched_barrier(0);
-                step(0, ks, 0, sa, sr, sa, sr);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            const bool last_of_group = p.grouped || s + 2 >= NSTG;
-            pending = last_of_group;
-            pending_prm = p.grouped ? (s & (PRM_SLOTS - 1)) : set;
-            pending_x = 2 * set + (own & 1);
-            if (last_of_group) {
-                if (c == 0) *reinterpret_cast<f32x4 *>(xsum + pending_x * BM + ws * 16 + 4 * g) = Xown;   // read after the next barrier
-                Xown = zero4;
-                own++;
-            }
-        }
-    }
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the refills past the end (zeros) have landed
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
     uint32_t collector_xcd = 0;
     if (p.S > 1 && chunk < p.S - 1) collector_xcd = __builtin_amdgcn_raw_buffer_load_b32(rsrc_z, (uint32_t)tile * 4u, flag_base, SC1);   // used after the fold
@@ -430,10 +308,10 @@ __global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqG
             for (int nb = 0; nb < 4; nb++) fold_tile(i, nb);
     }
 
-    // each wavefront finishes NE of its 16 register tiles: all of them, or with two sets the half of the rows that the
-    // sets hand each other through LDS (set 1 keeps row tiles 2 and 3 and moves them to the front)
+    // each wavefront finishes NE = 8 of its 16 register tiles: the half of the rows that the sets hand each other through
+    // LDS (set 1 keeps row tiles 2 and 3 and moves them to the front)
     constexpr int NE = 16 / SETS, NI = NE / 4;
-    if constexpr (SETS == 2) {
+    {
         // the stage slots are free
         f32x4 *red = reinterpret_cast<f32x4 *>(lds) + ws * 16 * 64 + lane;
         if (set == 0) {
@@ -480,29 +358,41 @@ __global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqG
             }
             return;
         }
-        for (int ch = 0; ch < p.S - 1; ch++) {
-            u32x4 v[NE];
+        // the sums of up to CB chunks are asked for together and added in chunk order: ((c0 + c1) + ...) + own
+        constexpr int CB = 3;
+        bool first = true;
+        for (int c0 = 0; c0 < p.S - 1; c0 += CB) {
+            u32x4 v[CB][NE];
 #pragma unroll
-            for (int e = 0; e < NE; e++)
-                v[e] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES, SC1);
+            for (int i = 0; i < CB; i++)
+#pragma unroll
+                for (int e = 0; e < NE; e++)
+                    v[i][e] = c0 + i < p.S - 1 ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)(c0 + i) * tiles * TILE_BYTES, SC1)
+                                               : u32x4{1u, 1u, 1u, 1u};
             for (int poll = 0; poll < kMaxPolls4; poll++) {
                 bool missing = false;
                 // the polls must be real loads: without a compiler barrier a reload with the operands of the first request is
                 // folded into it, and a wavefront that arrived before the data would spin on a stale register until the bound
                 asm volatile("" ::: "memory");
 #pragma unroll
-                for (int e = 0; e < NE; e++)
-                    if (v[e][0] == 0u || v[e][1] == 0u || v[e][2] == 0u || v[e][3] == 0u) {
-                        v[e] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)ch * tiles * TILE_BYTES, SC1);
-                        missing = true;
-                    }
+                for (int i = 0; i < CB; i++)
+#pragma unroll
+                    for (int e = 0; e < NE; e++)
+                        if (v[i][e][0] == 0u || v[i][e][1] == 0u || v[i][e][2] == 0u || v[i][e][3] == 0u) {
+                            v[i][e] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)(c0 + i) * tiles * TILE_BYTES, SC1);
+                            missing = true;
+                        }
                 if (!missing) break;
             }
-            // chunk order: ((c0 + c1) + ...) + own
 #pragma unroll
-            for (int e = 0; e < NE; e++) {
-                if (ch == 0) P[e >> 2][e & 3] = __builtin_bit_cast(f32x4, v[e]);
-                else P[e >> 2][e & 3] += __builtin_bit_cast(f32x4, v[e]);
+            for (int i = 0; i < CB; i++) {
+                if (c0 + i >= p.S - 1) break;
+#pragma unroll
+                for (int e = 0; e < NE; e++) {
+                    if (first) P[e >> 2][e & 3] = __builtin_bit_cast(f32x4, v[i][e]);
+                    else P[e >> 2][e & 3] += __builtin_bit_cast(f32x4, v[i][e]);
+                }
+                first = false;
             }
         }
 #pragma unroll
@@ -544,16 +434,15 @@ __global__ __launch_bounds__(MODE ? 512 : 256, 1) void wq_gemm4_kernel(const WqG
         }
 }
 
-template <int ACT, int MODE>
+template <int ACT, bool STAGE_GROUPS>
 int launch4(const WqGemm4Args &p, unsigned grid, hipStream_t s)
 {
-    constexpr int SETS = MODE ? 2 : 1;
-    constexpr size_t lds_bytes = (size_t)4 * 64 * 256 + 4 * 128 * 128 + 9 * 1024 + SETS * 2 * 64 * 4;
+    constexpr size_t lds_bytes = (size_t)4 * 64 * 256 + 4 * 128 * 128 + 8 * 1024 + 2 * 2 * 64 * 4;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
-    auto kern = wq_gemm4_kernel<ACT, MODE>;
+    auto kern = wq_gemm4_kernel<ACT, STAGE_GROUPS>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * SETS), lds_bytes, s, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, s, p);
     return check_launch();
 }
 
@@ -566,7 +455,7 @@ WqGemm4Plan make_wq_gemm4_plan(int64_t M, int64_t N, int64_t K, int w_bits, int6
     const int64_t row_bytes = N / 2, ldw_bytes = ldw_k * 4;
     const int64_t group = group_size > 0 ? group_size : K;
     const bool grouped = group_size > 0 && group != K;
-    pl.ok = knob(kKnobWqGemm4Off) != 1 && w_bits == 4 && M > 32 && M <= kMaxRows4 && K >= 128 && K % 128 == 0 && N % 8 == 0 && (!grouped || group % 128 == 0) &&
+    pl.ok = knob(kKnobWqGemm4Off) != 1 && w_bits == 4 && M > 32 && K >= 128 && K % 128 == 0 && N % 8 == 0 && (!grouped || group % 128 == 0) &&
             ldw_bytes >= row_bytes && ldw_bytes % 16 == 0 && ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) &&
             (w == nullptr || aligned(w, 16)) && (scale == nullptr || aligned(scale, 4)) && (offset == nullptr || aligned(offset, 4)) &&
             (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 31) && (uint64_t)128 * (uint64_t)ldx * 2 + (uint64_t)K * 2 < (1ull << 31) &&
@@ -574,8 +463,8 @@ WqGemm4Plan make_wq_gemm4_plan(int64_t M, int64_t N, int64_t K, int w_bits, int6
     if (!pl.ok) return pl;
     pl.strips = (int)((row_bytes + 127) / 128);
     const int64_t stages = K / 128;
-    const int64_t units = grouped ? K / group : 1;
-    // few tiles: split K in whole scale groups
+    const int64_t units = grouped ? K / group : stages;
+    // few tiles: split K in whole scale groups (per channel: in equal numbers of stages)
     pl.bm = 64;
     pl.tiles_m = (int)((M + pl.bm - 1) / pl.bm);
     const int64_t tiles = (int64_t)pl.tiles_m * pl.strips;
@@ -586,14 +475,10 @@ WqGemm4Plan make_wq_gemm4_plan(int64_t M, int64_t N, int64_t K, int w_bits, int6
         if (f >= 1 && f <= units) S = f;
     // the sums of S - 1 chunks per tile and one word per tile (the XCD of its collector)
     auto zone = [&](int64_t s) { return (uint64_t)(s - 1) * (uint64_t)tiles * (uint64_t)pl.bm * 256u * 4u + (uint64_t)tiles * 4u; };
-    while (S > 1 && zone(S) > kWorkspaceZoneBytes) S--;
+    while (S > 1 && (zone(S) > kWorkspaceZoneBytes || (!grouped && stages % S != 0))) S--;
     pl.S = (int)S;
-    pl.gstages = (int)(grouped ? group / 128 : stages / S > 0 ? stages : stages);
-    if (!grouped) {
-        // per channel: one fold per workgroup, so a "group" is the workgroup's whole range; K is split in stages
-        if (stages % S != 0) pl.S = 1;
-        pl.gstages = (int)(stages / pl.S);
-    }
+    // per channel: one fold per workgroup, so a "group" is the workgroup's whole range
+    pl.gstages = (int)(grouped ? group / 128 : stages / S);
     pl.zone_bytes = pl.S > 1 ? (size_t)zone(pl.S) : 0;
     if (tiles * pl.S > 0x7fffffff) pl.ok = false;
     return pl;
@@ -623,16 +508,14 @@ int launch_wq_gemm4(const WqGemm4Plan &plan, const void *x, int act_f16, const v
     p.tiles_m = plan.tiles_m;
     p.strips = plan.strips;
     p.S = plan.S;
-    p.l2_exchange = knob(kKnobWqGemm4Off) != 3;
+    p.l2_exchange = knob(kKnobWqGemm4Off) != 2;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t tiles = (int64_t)plan.tiles_m * plan.strips;
     (void)tiles;
     const unsigned grid = (unsigned)((plan.strips + 7) / 8 * 8 * plan.tiles_m * plan.S);
-    // two sets of wavefronts where a scale group is one stage (or the whole K range)
-    const bool paired = (!p.grouped || plan.gstages == 1) && knob(kKnobWqGemm4Off) != 2;
-    if (paired && p.grouped) return act_f16 ? launch4<1, 2>(p, grid, s) : launch4<0, 2>(p, grid, s);
-    if (paired) return act_f16 ? launch4<1, 1>(p, grid, s) : launch4<0, 1>(p, grid, s);
-    return act_f16 ? launch4<1, 0>(p, grid, s) : launch4<0, 0>(p, grid, s);
+    // a variant of its own where a scale group is one stage
+    if (p.grouped && plan.gstages == 1) return act_f16 ? launch4<1, true>(p, grid, s) : launch4<0, true>(p, grid, s);
+    return act_f16 ? launch4<1, false>(p, grid, s) : launch4<0, false>(p, grid, s);
 }
 
 } // namespace mi355

@@ -461,8 +461,8 @@ TILED_CASES = [  # bits, M, K, N, group, float16, bias
     (4, 33, 128, 8, 128, False, False),       # one stage, one dword column, one group = per channel
     (4, 64, 1536, 520, 384, False, True),     # groups of three stages, last strip holds 8 columns
     (4, 256, 8192, 256, 8192, True, False),   # one strip, four row blocks, per channel with a K split
-    (4, 384, 1024, 512, 128, False, False),   # the most rows the register-expanding kernel takes
-    (4, 400, 1024, 512, 128, False, False),   # beyond it: the kernel that expands weight images into LDS
+    (4, 384, 1024, 512, 128, False, False),
+    (4, 400, 1024, 512, 128, False, False),   # ragged seventh row block
     # int8 weights stored [N, K] (the transposed view that LinearWeightQuant passes, linear_weight_quant.py:106)
     (8, 40, 1024, 384, 0, False, False, True),
     (8, 128, 2048, 1000, 0, False, True, True),
@@ -479,14 +479,17 @@ PAIRED_CASES = [  # M, K, N, group (0: per channel), float16, forced split
     (96, 1152, 768, 0, True, 3),          # per channel, chunks of three stages
     (384, 2048, 1024, 128, False, 4),
     (200, 4096, 3584, 128, False, 0),     # ragged last row block, several strips per XCD
+    (128, 1536, 512, 256, False, 3),      # groups of two stages, chunks of two groups: each set has one stage per group
+    (72, 2304, 264, 384, True, 2),        # groups of three stages: the sets alternate two and one
+    (1100, 512, 1024, 128, False, 0),     # many row blocks per strip
 ]
 
 
 @pytest.mark.parametrize("case", PAIRED_CASES, ids=lambda c: "-".join(str(v) for v in c))
 def test_weight_quant_int4_register_kernel_variants(capi, golden, case):
-    """The register-expanding int4 kernel with two sets of wavefronts per workgroup (a scale group per stage, or one group),
-    with one set, and with the K-split exchange kept out of the L2: all three must meet the gate, and each must repeat
-    its own result bit for bit (the sets and the chunks add in a fixed order)."""
+    """The register-expanding int4 kernel (a scale group per stage, groups of several stages, or one group), with its
+    K-split exchange through the L2 and through memory: both must meet the gate, and each must repeat its own result bit
+    for bit (the sets of wavefronts and the chunks add in a fixed order)."""
     M, K, N, gs, f16, split = case
     d = workloads.w4a16_inputs(seed=M + N + K, M=M, K=K, N=N, group_size=gs if gs else K)
     bits_of = _bits
@@ -499,7 +502,7 @@ def test_weight_quant_int4_register_kernel_variants(capi, golden, case):
                                          dtype="fp16" if f16 else "bf16")
     capi.set_tuning("MI355_WQG_SPLIT", split)
     try:
-        for variant in (0, 2, 3):          # two sets; one set; two sets, exchange through memory
+        for variant in (0, 2):             # exchange through the L2 where the XCD allows; through memory
             capi.set_tuning("MI355_WQ_GEMM4_OFF", variant)
             out = capi.weight_quant_matmul(*args, group_size=gs if gs else K)
             bf16_gate(out, torch.from_numpy(gold))
