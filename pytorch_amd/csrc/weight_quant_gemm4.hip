@@ -98,7 +98,9 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     const __amdgpu_buffer_rsrc_t rsrc_o = make_rsrc(has_offset ? p.offset : p.scale, param_bytes);
     // a stage's 32 load units are dealt to the eight wavefronts; the parameters of a scale group (the strip's 256 scales
     // and offsets) travel with its first stage, issued by the first wavefront of the set that computes that stage.
-    // Nothing is issued past the end: the loop waits for vmcnt(0).
+    // Nothing is issued past the end: the loop waits for vmcnt(0).  Stages are issued in order, so the group of the next
+    // stage and its place in the group are counted along.
+    int iss_grp = 0, iss_in = 0;
     auto issue_stage = [&](int s) {
         if (s >= NSTG) return;
         char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
@@ -119,15 +121,18 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
                                                          (uint32_t)(s0 + s) * (uint32_t)BK * p.ldw_bytes, 0, kNonTemporal);
             }
         }
-        const int grp = s / p.gstages;
-        if (wave == 4 * (s & 1) && s == grp * p.gstages) {
-            const uint32_t ro = (uint32_t)(p.grouped ? u0 + grp : 0) * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
-            char *dst = prm + (grp & (PRM_SLOTS - 1)) * PRM_SLOT;
+        if (wave == 4 * (s & 1) && iss_in == 0) {
+            const uint32_t ro = (uint32_t)(p.grouped ? u0 + iss_grp : 0) * (uint32_t)p.N * 2u + (uint32_t)n0 * 2u;
+            char *dst = prm + (iss_grp & (PRM_SLOTS - 1)) * PRM_SLOT;
 #pragma unroll
             for (int q = 0; q < 2; q++) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_s, (lds_void *)(dst + q * 256), 4, (uint32_t)lane * 4u, ro + q * 256u, 0, 0);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_o, (lds_void *)(dst + 512 + q * 256), 4, (uint32_t)lane * 4u, ro + q * 256u, 0, 0);
             }
+        }
+        if (++iss_in == p.gstages) {
+            iss_in = 0;
+            iss_grp++;
         }
     };
 
@@ -248,6 +253,8 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     issue_stage(0);
     issue_stage(1);
     int own = 0;
+    // group of the set's current stage and the stage's place in it (no divisions in the loop)
+    int grp = STAGE_GROUPS ? set : set / p.gstages, in_grp = STAGE_GROUPS ? 0 : set - grp * p.gstages;
     for (int it = 0; 2 * it < NSTG; it++) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();                          // this pair is complete in LDS; everyone is done with the pair before
@@ -256,7 +263,6 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         issue_stage(2 * it + 3);
         const int s = 2 * it + set;
         if (s >= NSTG) continue;
-        const int grp = s / p.gstages;
         const char *sa = lds + (s & 3) * A_BYTES, *sr = raw + (s & 3) * R_BYTES;
         read_w(sr, 0);
 #pragma unroll
@@ -286,9 +292,18 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         }
         __builtin_amdgcn_sched_barrier(0);
         // the set's share of a group ends with its last stage inside the group
-        const bool last_of_group = s + 2 >= NSTG || (s + 2) / p.gstages != grp;
+        int next_grp = grp + (STAGE_GROUPS ? 2 : 0), next_in = in_grp + (STAGE_GROUPS ? 0 : 2);
+        if (!STAGE_GROUPS)
+            for (int r = 0; r < 2; r++)
+                if (next_in >= p.gstages) {
+                    next_in -= p.gstages;
+                    next_grp++;
+                }
+        const bool last_of_group = s + 2 >= NSTG || next_grp != grp;
         pending = last_of_group;
         pending_prm = grp & (PRM_SLOTS - 1);
+        grp = next_grp;
+        in_grp = next_in;
         pending_x = 2 * set + (own & 1);
         if (last_of_group) {
             if (c == 0) *reinterpret_cast<f32x4 *>(xsum + pending_x * BM + ws * 16 + 4 * g) = Xown;   // read after the next barrier
