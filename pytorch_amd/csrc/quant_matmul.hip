@@ -401,14 +401,25 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         const bool last = is_last != 0;
         __syncthreads();                                          // the flag's LDS word is reused by the epilogue
         if (!last) return;
-        for (int ch = 0; ch < p.S; ch++) {
-            if (ch == chunk) continue;
+        // the other chunks' sums are asked for CB chunks at a time (as many as the registers hold): one round trip to the
+        // coherence point per batch instead of one per chunk.  The own chunk and chunks past the end get an out-of-range
+        // lane offset, i.e. zeros.
+        constexpr int TL = WTM * WTN;
+        constexpr int CB = TL <= 4 ? 8 : TL <= 8 ? 4 : TL <= 16 ? 2 : 1;
+        for (int c0 = 0; c0 < p.S; c0 += CB) {
+            u32x4 v[CB][TL];
 #pragma unroll
-            for (int i = 0; i < WTM; i++)
+            for (int b = 0; b < CB; b++) {
+                const int ch = c0 + b;
+                const uint32_t lo = ch < p.S && ch != chunk ? lane_off : kOutOfRange;
 #pragma unroll
-                for (int j = 0; j < WTN; j++)
-                    acc[i][j] += __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(
-                        rsrc_p, lane_off + (i * WTN + j) * 1024, (uint32_t)ch * CHUNK_BYTES, SC1));
+                for (int t = 0; t < TL; t++)
+                    v[b][t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, lo + t * 1024, (uint32_t)min(ch, p.S - 1) * CHUNK_BYTES, SC1);
+            }
+#pragma unroll
+            for (int b = 0; b < CB; b++)
+#pragma unroll
+                for (int t = 0; t < TL; t++) acc[t / WTN][t % WTN] += __builtin_bit_cast(i32x4v, v[b][t]);
         }
         if (threadIdx.x == 0) __hip_atomic_store(p.counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
