@@ -220,7 +220,9 @@ int mi355_quant_matmul_noalloc(const int8_t *a, const int8_t *b, const float *pe
  *   One kernel launch per call: weight-streaming kernels for M <= 32 (for int4 words along N a barrier-free one whose
  *   workgroups exchange their partial sums through the workspace's zero zone) and a tiled GEMM above that; int4
  *   words along K take a kernel of their own in which a wavefront owns 16 output columns for all of K (no split of
- *   K at decode shapes).
+ *   K at decode shapes); from 256 rows up they are first rewritten into the workspace with their words along N (the
+ *   tiled GEMM for that layout is faster by more than the rewrite costs: three small launches in front of it), which
+ *   is what the workspace query asks room for at those sizes.
  */
 size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size);
 

@@ -41,6 +41,7 @@
 #include "weight_quant_kpacked.h"
 #include "weight_quant_decode.h"
 #include "weight_quant_gemm4.h"
+#include "weight_quant_repack.h"
 #include <type_traits>
 
 namespace mi355 {
@@ -732,6 +733,44 @@ int launch_kmajor_any(const WqArgs &p, const WqKmPlan &km, hipStream_t s)
 } // namespace
 } // namespace mi355
 
+namespace mi355 {
+namespace {
+// Which kernel a launch with rows along N takes when every pointer is aligned, in the order of the launch: the int4 decode
+// kernel, the int4 register-expanding GEMM, the tiled GEMM through LDS images, the streaming kernel.
+enum { kPreferDecode, kPreferGemm4, kPreferGemm, kPreferStream };
+
+// int4 words along K, many rows: the weight is rewritten into the workspace with its words along N (and the parameters
+// gathered into row-major [G, N]) for the register-expanding GEMM.  Layout of the workspace: the zero area, the weight
+// ([K, repack_pitch_words(N)] words), scales, offsets.
+constexpr int64_t kRepackRows = 256;
+int64_t repack_pitch_words(int64_t N) { return (N / 8 + 3) / 4 * 4; }
+size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+size_t repack_weight_bytes(int64_t N, int64_t K) { return align256((size_t)K * (size_t)repack_pitch_words(N) * 4); }
+size_t repack_param_bytes(int64_t N, int64_t K, int64_t group_size)
+{
+    return align256((size_t)(group_size > 0 ? K / group_size : 1) * (size_t)N * 2);
+}
+size_t repack_workspace_bytes(int64_t N, int64_t K, int64_t group_size)
+{
+    return kWorkspaceZeroBytes + repack_weight_bytes(N, K) + 2 * repack_param_bytes(N, K, group_size);
+}
+bool repack_applies(int64_t M, int64_t N, int64_t K, int64_t group_size, int64_t ldx, const void *x)
+{
+    return M >= kRepackRows && N % 8 == 0 && K % 128 == 0 &&
+           make_wq_gemm4_plan(M, N, K, 4, group_size, repack_pitch_words(N), ldx, x, nullptr, nullptr, nullptr).ok;
+}
+int preferred_n_major_kernel(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size, int64_t ldw_k, int64_t ldx)
+{
+    if (w_bits == 4) {
+        if (make_wq_decode_plan(M, N, K, 4, group_size, ldw_k, ldx, nullptr, nullptr, nullptr, nullptr).ok) return kPreferDecode;
+        if (make_wq_gemm4_plan(M, N, K, 4, group_size, ldw_k, ldx, nullptr, nullptr, nullptr, nullptr).ok) return kPreferGemm4;
+    }
+    if (make_wq_gemm_plan(M, N, K, w_bits, group_size, 1, ldw_k, ldx, nullptr, nullptr, nullptr, nullptr).ok) return kPreferGemm;
+    return kPreferStream;
+}
+} // namespace
+} // namespace mi355
+
 extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size)
 {
     using namespace mi355;
@@ -739,15 +778,22 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
     // The query knows neither strides nor alignments, the launch plans with the real ones: the answer is the largest
     // request over every layout the kernels accept, once with dense rows (pitch = row length) and once with rows padded
     // to 128 bytes, which is what lets a shape with a ragged row length onto a fast kernel that the dense pitch rules out.
+    // Per layout it asks for the kernel the launch prefers (preferred_n_major_kernel); a kernel further down the order, which
+    // only runs when a pointer is misaligned, falls through to the generic kernel if its own request is not met (the
+    // streaming kernel would ask for S x M x N x 4 bytes at large M: hundreds of MiB that no launch of a sane caller uses).
     auto pad = [](int64_t v, int64_t to) { return (v + to - 1) / to * to; };
     size_t need = 0;
     for (int padded = 0; padded < 2; padded++) {
         const int64_t ldx = padded ? pad(K, 64) : K;                                  // activation pitch, elements
         const int64_t ldw_n_major = padded ? pad(w_bits == 4 ? N / 8 : N, w_bits == 4 ? 32 : 128) : (w_bits == 4 ? N / 8 : N);
         const int64_t ldw_k_major = padded ? pad(w_bits == 4 ? K / 8 : K, w_bits == 4 ? 32 : 128) : (w_bits == 4 ? K / 8 : K);
-        const WqPlan pl = make_plan(M, N, K, w_bits, group_size, true, ldw_n_major, ldx, nullptr, nullptr, nullptr, nullptr);
-        if (pl.fast && pl.partial_bytes + pl.counter_bytes > need) need = pl.partial_bytes + pl.counter_bytes;
+        const int preferred = preferred_n_major_kernel(M, N, K, w_bits, group_size, ldw_n_major, ldx);
+        if (preferred == kPreferStream) {
+            const WqPlan pl = make_plan(M, N, K, w_bits, group_size, true, ldw_n_major, ldx, nullptr, nullptr, nullptr, nullptr);
+            if (pl.fast && pl.partial_bytes + pl.counter_bytes > need) need = pl.partial_bytes + pl.counter_bytes;
+        }
         for (int layout = 1; layout <= (w_bits == 8 ? 2 : 1); layout++) {
+            if (layout == 1 && preferred != kPreferGemm) continue;
             const WqGemmPlan gp = make_wq_gemm_plan(M, N, K, w_bits, group_size, layout, layout == 2 ? ldw_k_major : ldw_n_major, ldx,
                                                     nullptr, nullptr, nullptr, nullptr);
             const size_t gneed = gp.counter_bytes + gp.partial_bytes;
@@ -758,9 +804,13 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
             if (dp.ok && dp.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
             const WqGemm4Plan g4 = make_wq_gemm4_plan(M, N, K, 4, group_size, ldw_n_major, ldx, nullptr, nullptr, nullptr, nullptr);
             if (g4.ok && g4.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
-            // words along K
-            const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, ldw_k_major, ldx, nullptr, nullptr);
-            if (kp.ok && kp.partial_bytes + kp.counter_bytes > need) need = kp.partial_bytes + kp.counter_bytes;
+            // words along K: rewritten per call from kRepackRows rows up, a kernel of their own below
+            if (repack_applies(M, N, K, group_size, ldx, nullptr)) {
+                if (repack_workspace_bytes(N, K, group_size) > need) need = repack_workspace_bytes(N, K, group_size);
+            } else {
+                const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, ldw_k_major, ldx, nullptr, nullptr);
+                if (kp.ok && kp.partial_bytes + kp.counter_bytes > need) need = kp.partial_bytes + kp.counter_bytes;
+            }
         } else {                            // the K-major layout may split differently
             const WqKmPlan km = make_kmajor_plan(M, N, K, group_size, ldw_k_major, ldx, nullptr, nullptr);
             if (km.fast && km.partial_bytes + km.counter_bytes > need) need = km.partial_bytes + km.counter_bytes;
@@ -807,6 +857,24 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
         return check_launch();
     };
     if (kpacked) {
+        if (repack_applies(M, N, K, group_size, ldx, x_bf16) && ldw_n % 4 == 0 && aligned(w, 16) && aligned(scale_bf16, 2) &&
+            (!offset_bf16 || aligned(offset_bf16, 2)) && aligned(out_bf16, 2) && (!bias || aligned(bias, 2)) && workspace &&
+            aligned(workspace, 256) && workspace_bytes >= repack_workspace_bytes(N, K, group_size)) {
+            char *ws = static_cast<char *>(workspace);
+            void *w_kn = ws + kWorkspaceZeroBytes;
+            void *scale_gn = ws + kWorkspaceZeroBytes + repack_weight_bytes(N, K);
+            void *offset_gn = offset_bf16 ? static_cast<char *>(scale_gn) + repack_param_bytes(N, K, group_size) : nullptr;
+            const int64_t pitch = repack_pitch_words(N);
+            int st = launch_repack_int4_k_to_n(w, ldw_n, w_kn, pitch, N, K, stream);
+            if (st == MI355_OK) st = launch_gather_params_u16(scale_bf16, ld_param_g, ld_param_n, scale_gn, n_groups, N, stream);
+            if (st == MI355_OK && offset_bf16)
+                st = launch_gather_params_u16(offset_bf16, ld_param_g, ld_param_n, offset_gn, n_groups, N, stream);
+            if (st != MI355_OK) return st;
+            const WqGemm4Plan g4 = make_wq_gemm4_plan(M, N, K, 4, group_size, pitch, ldx, x_bf16, w_kn, scale_gn, offset_gn);
+            if (!g4.ok) return MI355_ERR_LAUNCH;       // planned with these strides a few lines up
+            return launch_wq_gemm4(g4, x_bf16, f16 ? 1 : 0, w_kn, scale_gn, offset_gn, bias, out_bf16, M, N, K, group_size, ldx, pitch,
+                                   ldo, workspace, stream);
+        }
         const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, ldw_n, ldx, x_bf16, w);
         const bool ptrs_ok = aligned(scale_bf16, 2) && (!offset_bf16 || aligned(offset_bf16, 2)) && aligned(out_bf16, 2) &&
                              (!bias || aligned(bias, 2));
@@ -886,8 +954,13 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
         }
     }
     // more than 32 rows: the tiled kernel decodes every weight once per 64 or 128 rows
+    // A kernel that the workspace query did not plan for (it only runs because a pointer kept the preferred one away) goes
+    // on to the next one when its own request is not met; the preferred one reports the missing workspace.
+    const int preferred = n_major ? preferred_n_major_kernel(M, N, K, w_bits, group_size, ldw_k, ldx) : kPreferStream;
+    const auto workspace_holds = [&](size_t bytes) { return workspace && workspace_bytes >= bytes && aligned(workspace, 16); };
     const WqGemmPlan gp = make_wq_gemm_plan(M, N, K, w_bits, group_size, n_major ? 1 : 0, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
-    if (gp.ok && aligned(out_bf16, 2) && (!bias || aligned(bias, 2))) {
+    if (gp.ok && aligned(out_bf16, 2) && (!bias || aligned(bias, 2)) &&
+        (gp.S == 1 || preferred >= kPreferGemm || workspace_holds(gp.counter_bytes + gp.partial_bytes))) {
         if (gp.S > 1) {
             if (!workspace || workspace_bytes < gp.counter_bytes + gp.partial_bytes) return MI355_ERR_WORKSPACE;
             if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
@@ -898,6 +971,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
     const WqPlan pl = make_plan(M, N, K, w_bits, group_size, n_major, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
     if (!pl.fast) return generic();
     if (pl.S > 1) {
+        if (preferred != kPreferStream && !workspace_holds(pl.partial_bytes + pl.counter_bytes)) return generic();
         if (!workspace || workspace_bytes < pl.partial_bytes + pl.counter_bytes) return MI355_ERR_WORKSPACE;
         if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
     }

@@ -575,6 +575,11 @@ KPACKED_CASES = [
     (3, 2048, 4096, 0, False, False, True),         # per channel, 1-D parameters
     (70, 14336, 4096, 128, False, True, False),     # long K: K is split between workgroups, 112 groups
     (16, 256, 16, 128, True, True, False),          # a single step, a single wavefront's worth of columns
+    # from 256 rows up the weight is rewritten per call with its words along N (weight_quant_repack.hip)
+    (256, 512, 1000, 128, False, True, True),       # ragged columns: 125 words per row, the last tile partly valid
+    (300, 1024, 520, 256, True, True, False),       # ragged rows, groups of two stages, fp16
+    (257, 640, 264, 0, False, False, False),        # per channel, K / 8 = 80 words: a partly valid tile along K
+    (512, 4096, 14336, 128, False, True, False),    # the W4A16 configuration at prefill size, module layout
 ]
 
 

@@ -370,3 +370,23 @@ def test_flop_counter_formulas(pa):
         pa.npu_quant_matmul(_m(3, 16, 256, dtype=torch.int8), _m(256, 64, dtype=torch.int8), _m(64, dtype=torch.float32),
                             output_dtype=torch.bfloat16)
     assert fc.get_total_flops() == 2 * 3 * 16 * 256 * 64
+
+
+def test_weight_quant_workspace_query_follows_the_preferred_kernel():
+    """Host logic of mi355_weight_quant_matmul_workspace (no GPU needed): the request is that of the kernel a launch with
+    aligned pointers takes, not of a kernel further down the order.  int4 with K split between workgroups asks for the
+    zero area; int4 at prefill sizes asks for the zero area plus the rewritten weight and parameters (words along K are
+    rewritten per call from 256 rows up) and no longer for S x M x N x 4 bytes of partial sums; per-channel int4 splits
+    K like the grouped case."""
+    from pytorch_amd import _capi
+    L = _capi.lib()
+    zero_area = 16 * 1024 * 1024 + 16384
+    q = L.mi355_weight_quant_matmul_workspace
+    assert q(1, 14336, 4096, 4, 128) == zero_area            # decode kernel, four chunks of K
+    assert q(128, 14336, 4096, 4, 128) == zero_area          # register-expanding GEMM, two chunks of K
+    assert q(128, 14336, 4096, 4, 0) == zero_area            # per channel: the same split
+    repack = zero_area + 4096 * (14336 // 8) * 4 + 2 * (4096 // 128) * 14336 * 2
+    for rows in (256, 2048, 8192):
+        assert q(rows, 14336, 4096, 4, 128) == repack
+        assert q(rows, 14336, 4096, 8, 0) == 0                # int8 tiled GEMM with enough tiles: no split, no workspace
+    assert q(0, 14336, 4096, 4, 128) == 0 and q(16, 14336, 4096, 5, 128) == 0
