@@ -690,7 +690,7 @@ def test_weight_quant_int4_words_along_k_random_shapes(capi, golden):
     import os
     rng = np.random.default_rng(4242)
     for case in range(int(os.environ.get("MI355_SWEEP_CASES", "64"))):
-        M = int(rng.choice([1, 2, 15, 16, 17, 32, 33, 63, 64, 65, 100, 130]))
+        M = int(rng.choice([1, 2, 15, 16, 17, 32, 33, 63, 64, 65, 100, 130, 256, 300]))
         K = int(rng.choice([128, 256, 512, 768, 1024, 1280, 2048, 3072]))
         N = int(rng.choice([8, 16, 24, 64, 72, 128, 136, 200, 256, 1000, 2048]))
         gs = int(rng.choice([g for g in (0, 32, 64, 128, 256, 384, 512, 1024) if g == 0 or K % g == 0]))
@@ -711,7 +711,8 @@ def test_weight_quant_int4_words_along_k_random_shapes(capi, golden):
         dev = lambda t: None if t is None else (t.t().contiguous().cuda().t() if params_ng and t.dim() == 2 else t.cuda())  # noqa: E731
         try:
             out = capi.weight_quant_matmul(d["x"].cuda(), w_nk.cuda().t(), dev(sc), dev(of), group_size=gs)
-            bf16_gate(out, torch.from_numpy(gold))
+            # small outputs are counted with the cancellation floor, as in the sweep above
+            bf16_gate(out, torch.from_numpy(gold), floor=out.numel() < 8192)
         except (AssertionError, capi.Mi355Error) as e:
             raise AssertionError(f"case {case}: M={M} K={K} N={N} gs={gs} f16={f16} offset={with_off} params_ng={params_ng}: {e}")
 
