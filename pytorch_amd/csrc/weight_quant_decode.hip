@@ -217,10 +217,13 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
         for (int q = 0; q < 4; q++) {
             const int row = 4 * g + q;
             if (row < rows_mt) {
+                // a lane's four 16-byte pieces are rotated by its column group: with the pieces of neighbouring lanes 64 bytes
+                // apart, unrotated stores would meet in two groups of banks
                 float *dst = red + ((size_t)wave * rows_mt + row) * NBW + 16 * c;
 #pragma unroll
                 for (int i = 0; i < NT; i += 4)
-                    *reinterpret_cast<f32x4 *>(dst + i) = f32x4{tot[mt][i][q], tot[mt][i + 1][q], tot[mt][i + 2][q], tot[mt][i + 3][q]};
+                    *reinterpret_cast<f32x4 *>(dst + 4 * ((i / 4 + c) & 3)) =
+                        f32x4{tot[mt][i][q], tot[mt][i + 1][q], tot[mt][i + 2][q], tot[mt][i + 3][q]};
             }
         }
         __syncthreads();
@@ -231,8 +234,9 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
             const int e = mt * QPT + j;
             acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
             if (live[e]) {
+                const int piece = nl >> 2, nl_rot = (piece & ~3) * 4 + 4 * ((piece + (piece >> 2)) & 3);   // where the stores put it
 #pragma unroll
-                for (int wv = 0; wv < 8; wv++) acc[e] += *reinterpret_cast<const f32x4 *>(red + ((size_t)wv * rows_mt + row) * NBW + nl);
+                for (int wv = 0; wv < 8; wv++) acc[e] += *reinterpret_cast<const f32x4 *>(red + ((size_t)wv * rows_mt + row) * NBW + nl_rot);
             }
         }
     }
