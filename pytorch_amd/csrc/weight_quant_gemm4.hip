@@ -1,5 +1,6 @@
-// npu_weight_quant_batchmatmul, int4 weights packed along N, more than 32 activation rows: a tiled GEMM in which the
-// packed weights never exist in expanded form outside of registers.
+// npu_weight_quant_batchmatmul, int4 weights packed along N (and int8 weights [K, N], see the kernel's template
+// parameters), more than 32 activation rows: a tiled GEMM in which the packed weights never exist in expanded form outside
+// of registers.  The description is that of the int4 case.
 //
 // A workgroup owns 64 activation rows x one 128-byte strip of the weight rows (256 columns) and walks its K range in
 // stages of 128 rows.  Per stage the activations (64 x 256 B) and the raw strip (128 x 128 B) are copied global -> LDS by
@@ -49,12 +50,18 @@ struct WqGemm4Args {
 
 constexpr int kMaxPolls4 = 1 << 20;
 
-// STAGE_GROUPS: a scale group is one stage, so every stage restarts the group's sums
-template <int ACT, bool STAGE_GROUPS>
+// STAGE_GROUPS: a scale group is one stage, so every stage restarts the group's sums.
+// WBITS == 8: the same kernel for int8 weights [K, N].  A weight row of the tile is then 256 bytes (256 columns), a stage
+// 64 rows (two steps), and a wavefront owns one 128-byte half of the rows x one span of 16 dwords with all four bytes
+// of its dwords: again four column tiles per lane (columns 128 s2 + 64 h + 4 c .. + 3), expanded with a byte-to-float
+// conversion and a packing conversion per pair of weights (image u = w + 128).
+template <int ACT, bool STAGE_GROUPS, int WBITS = 4>
 __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
 {
-    constexpr int SETS = 2, NW = 4 * SETS, BM = 64, BK = 128, SLOTS = 4;
-    constexpr int A_BYTES = BM * 256, R_BYTES = BK * 128;      // one stage of activations / raw weights
+    constexpr int SETS = 2, NW = 4 * SETS, BM = 64, BK = WBITS == 4 ? 128 : 64, SLOTS = 4;
+    constexpr int STEPS = BK / 32;                             // MFMA steps of a stage
+    constexpr int ROW_B = WBITS == 4 ? 128 : 256;              // bytes of a weight row inside the tile
+    constexpr int A_BYTES = BM * BK * 2, R_BYTES = BK * ROW_B; // one stage of activations / raw weights
     constexpr int PRM_SLOT = 1024;                             // [256 scales | 256 offsets], 16 bits each
     constexpr int PRM_SLOTS = 8;                               // groups whose parameters are in LDS
     constexpr int SC1 = 16;                                    // cache-policy bit: agent scope
@@ -87,11 +94,13 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     // holds global chunk (l % 16) ^ (row & 15).  Raw weights: unit = 8 row slots x 128 B; row slot sl holds row
     // sl ^ ((sl >> 3) & 1) and its chunk slot j' holds chunk j' ^ (4 * ((row >> 4) & 1)): with that the four k octets a
     // wavefront reads together fall into four different quarters of the banks.
+    // (int8: activation unit = 8 rows x 128 B, chunk slot l % 8 holds chunk (l % 8) ^ (row & 7); weight unit = 4 rows x
+    // 256 B, chunk slot j' holds chunk j' ^ (4 * ((row >> 3) & 1)).)
     const int rows_a = min(BM, p.M - m0);
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.x + (int64_t)m0 * p.ldx, (uint32_t)(((int64_t)(rows_a - 1) * p.ldx + p.K) * 2));
-    const uint32_t strip_valid = min(128u, p.row_bytes - (uint32_t)strip * 128u);
+    const uint32_t strip_valid = min((uint32_t)ROW_B, p.row_bytes - (uint32_t)strip * (uint32_t)ROW_B);
     const __amdgpu_buffer_rsrc_t rsrc_w =
-        make_rsrc(static_cast<const char *>(p.w) + (size_t)strip * 128, (uint32_t)(p.K - 1) * p.ldw_bytes + strip_valid);
+        make_rsrc(static_cast<const char *>(p.w) + (size_t)strip * ROW_B, (uint32_t)(p.K - 1) * p.ldw_bytes + strip_valid);
     const bool has_offset = p.offset != nullptr;
     const uint32_t param_bytes = (uint32_t)(p.grouped ? units : 1) * (uint32_t)p.N * 2u;
     const __amdgpu_buffer_rsrc_t rsrc_s = make_rsrc(p.scale, param_bytes);
@@ -107,15 +116,22 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             const int u = i * NW + wave;
-            {
-                const int row = 4 * u + (lane >> 4);
-                const uint32_t vo = (uint32_t)(row * (int)p.ldx * 2 + (((lane & 15) ^ (row & 15)) * 16));
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void *)(sa + u * 1024), 16, vo, (uint32_t)(s0 + s) * 256u, 0, 0);
+            if (WBITS == 4 || i == 0) {                        // int8: eight units of activations, one per wavefront
+                const int row = WBITS == 4 ? 4 * u + (lane >> 4) : 8 * u + (lane >> 3);
+                const uint32_t vo = WBITS == 4 ? (uint32_t)(row * (int)p.ldx * 2 + (((lane & 15) ^ (row & 15)) * 16))
+                                               : (uint32_t)(row * (int)p.ldx * 2 + (((lane & 7) ^ (row & 7)) * 16));
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void *)(sa + u * 1024), 16, vo, (uint32_t)(s0 + s) * (uint32_t)(BK * 2), 0, 0);
             }
-            {
+            if constexpr (WBITS == 4) {
                 const int sl = 8 * u + (lane >> 3);
                 const int row = sl ^ ((sl >> 3) & 1);
                 const uint32_t ch = (uint32_t)((lane & 7) ^ (4 * ((row >> 4) & 1)));
+                const uint32_t vo = ch * 16u < strip_valid ? (uint32_t)row * p.ldw_bytes + ch * 16u : kOutOfRange;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void *)(sr + u * 1024), 16, vo,
+                                                         (uint32_t)(s0 + s) * (uint32_t)BK * p.ldw_bytes, 0, kNonTemporal);
+            } else {
+                const int row = 4 * u + (lane >> 4);
+                const uint32_t ch = (uint32_t)((lane & 15) ^ (4 * ((row >> 3) & 1)));
                 const uint32_t vo = ch * 16u < strip_valid ? (uint32_t)row * p.ldw_bytes + ch * 16u : kOutOfRange;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void *)(sr + u * 1024), 16, vo,
                                                          (uint32_t)(s0 + s) * (uint32_t)BK * p.ldw_bytes, 0, kNonTemporal);
@@ -138,12 +154,18 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
 
     // ---- LDS read addresses
     // raw: dword 16h + c of rows 8g + t; even t and odd t have their own base because odd octets swap row pairs
-    const int jch = (4 * h + (c >> 2)) ^ (4 * ((g >> 1) & 1));
-    const int r_even = (8 * g + (g & 1)) * 128 + jch * 16 + (c & 3) * 4;
-    const int r_odd = (8 * g + 1 - (g & 1)) * 128 + jch * 16 + (c & 3) * 4;
+    // (int8: dword 32 s2 + 16 h + c of rows 8g + t, s2 = jp; rows of one parity of g share their banks: a two-way conflict
+    // on reads that are a small part of the step)
+    const int jch = WBITS == 4 ? (4 * h + (c >> 2)) ^ (4 * ((g >> 1) & 1)) : (8 * jp + 4 * h + (c >> 2)) ^ (4 * (g & 1));
+    const int r_even = WBITS == 4 ? (8 * g + (g & 1)) * 128 + jch * 16 + (c & 3) * 4 : 8 * g * 256 + jch * 16 + (c & 3) * 4;
+    const int r_odd = WBITS == 4 ? (8 * g + 1 - (g & 1)) * 128 + jch * 16 + (c & 3) * 4 : r_even + 256;
     // activations: row c of a row tile, chunk 4 ks + g, stored at chunk slot ((ks ^ (c >> 2)) << 2) | (g ^ (c & 3))
-    const int a_lane = c * 256 + ((c >> 2) << 6) + ((g ^ (c & 3)) << 4);   // step ks: a_lane ^ (ks << 6)
-    const int prm_col = (128 * h + 8 * c + 4 * jp) * 2;        // byte offset of this lane's four columns in a parameter slot
+    // (int8: rows of 128 bytes, chunk slot (4 ks + g) ^ (c & 7))
+    const int a_lane = WBITS == 4 ? c * 256 + ((c >> 2) << 6) + ((g ^ (c & 3)) << 4)
+                                  : c * 128 + (((c >> 2) & 1) << 6) + ((g ^ (c & 3)) << 4);   // step ks: a_lane ^ (ks << 6)
+    constexpr int A_TILE = 16 * BK * 2;                        // bytes of a row tile in a stage
+    // byte offset of this lane's four columns in a parameter slot
+    const int prm_col = WBITS == 4 ? (128 * h + 8 * c + 4 * jp) * 2 : (128 * jp + 64 * h + 4 * c) * 2;
     const uint32_t sel0 = 0x0c000c00u | ((4u + 2u * jp) << 16) | (2u * jp);      // byte 2jp of two rows
     const uint32_t sel1 = sel0 + 0x00010001u;                                    // byte 2jp + 1
 
@@ -175,7 +197,8 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
                              has_offset ? act_lo<ACT>(or1) : 0.f, has_offset ? act_hi<ACT>(or1) : 0.f};
 #pragma unroll
         for (int nb = 0; nb < 4; nb++) {
-            const float mul = (nb & 1) ? kMulHi4<ACT> : kMulLo4<ACT>, bias = (nb & 1) ? kBiasHi4<ACT> : kBiasLo4<ACT>;
+            const float mul = WBITS == 8 ? 1.0f : (nb & 1) ? kMulHi4<ACT> : kMulLo4<ACT>;
+            const float bias = WBITS == 8 ? kImageBias<8> : (nb & 1) ? kBiasHi4<ACT> : kBiasLo4<ACT>;
             scm[nb] = sc[nb] * mul;
             ofm[nb] = (of[nb] - bias) * (1.0f / mul);
         }
@@ -194,10 +217,20 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     auto read_w = [&](const char *sr, int ks) {
 #pragma unroll
         for (int t = 0; t < 8; t++)
-            w[t] = *reinterpret_cast<const uint32_t *>(sr + ks * 4096 + ((t & 1) ? r_odd : r_even) + (t >> 1) * 256);
+            w[t] = *reinterpret_cast<const uint32_t *>(sr + ks * (32 * ROW_B) + ((t & 1) ? r_odd : r_even) + (t >> 1) * (2 * ROW_B));
     };
-    auto read_a = [&](const char *sa, int ks, int i) { return *reinterpret_cast<const u32x4 *>(sa + i * 4096 + (a_lane ^ (ks << 6))); };
+    auto read_a = [&](const char *sa, int ks, int i) { return *reinterpret_cast<const u32x4 *>(sa + i * A_TILE + (a_lane ^ (ks << 6))); };
     auto expand = [&](u32x4 (&bn)[4]) {
+        if constexpr (WBITS == 8) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const uint32_t wa = w[2 * v] ^ 0x80808080u, wb = w[2 * v + 1] ^ 0x80808080u;
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++)
+                    bn[nb][v] = pack_act2<ACT>((float)((wa >> (8 * nb)) & 0xffu), (float)((wb >> (8 * nb)) & 0xffu));
+            }
+            return;
+        }
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const uint32_t t0 = __builtin_amdgcn_perm(w[2 * v + 1], w[2 * v], sel0);
@@ -214,16 +247,16 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     // one step of 32 k: the MFMAs of step ks with the expansion of step ks + 1 spread between them
     auto step = [&](const bool restart /* the sums start from the MFMA's zero operand */, const int ks, const char *sa, const char *sr) {
         u32x4(&bc)[4] = b[ks & 1];
-        if (ks + 1 < 4) expand(b[(ks + 1) & 1]);
-        if (ks + 2 < 4) read_w(sr, ks + 2);
+        if (ks + 1 < STEPS) expand(b[(ks + 1) & 1]);
+        if (ks + 2 < STEPS) read_w(sr, ks + 2);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
 #pragma unroll
             for (int nb = 0; nb < 4; nb++) P[i][nb] = mfma_act<ACT>(AF[i], bc[nb], restart ? zero4 : P[i][nb]);
-            if (ks + 1 < 4) AF[i] = read_a(sa, ks + 1, i);
+            if (ks + 1 < STEPS) AF[i] = read_a(sa, ks + 1, i);
         }
         Xown = mfma_act<ACT>(AX, ones, Xown);
-        if (ks + 1 < 4) AX = read_a(sa, ks + 1, ws);
+        if (ks + 1 < STEPS) AX = read_a(sa, ks + 1, ws);
         // interleave: one MFMA, its share of the integer work, one LDS read
 #pragma unroll
         for (int r = 0; r < 17; r++) {
@@ -280,13 +313,13 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
                 }
         }
         expand(b[0]);
-        read_w(sr, 1);
+        if (STEPS > 1) read_w(sr, 1);
         __builtin_amdgcn_sched_barrier(0);
         // Compile time, not a branch: two copies of the step behind a branch cost a hundred registers, so groups of several
         // stages clear the sums after the fold instead.
         step(STAGE_GROUPS, 0, sa, sr);
 #pragma unroll
-        for (int ks = 1; ks < 4; ks++) {
+        for (int ks = 1; ks < STEPS; ks++) {
             __builtin_amdgcn_sched_barrier(0);
             step(false, ks, sa, sr);
         }
@@ -423,8 +456,8 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     }
 
     // ---- output: lane (c, g) holds rows 16 i + 4 g + q, columns 128 h + 8 c + 4 jp .. + 3: 8 bytes per row
-    const int col = n0 + 128 * h + 8 * c + 4 * jp;
-    if (col >= p.N) return;                                    // N is a multiple of 8: the four columns are inside or outside
+    const int col = WBITS == 4 ? n0 + 128 * h + 8 * c + 4 * jp : n0 + 128 * jp + 64 * h + 4 * c;
+    if (col >= p.N) return;                                    // N is a multiple of 8 (int8: of 4): the four columns are inside or outside
     float bv[4];
 #pragma unroll
     for (int nb = 0; nb < 4; nb++) bv[nb] = p.bias ? act_1<ACT>(p.bias[col + nb]) : 0.0f;
@@ -449,12 +482,13 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         }
 }
 
-template <int ACT, bool STAGE_GROUPS>
+template <int ACT, bool STAGE_GROUPS, int WBITS>
 int launch4(const WqGemm4Args &p, unsigned grid, hipStream_t s)
 {
-    constexpr size_t lds_bytes = (size_t)4 * 64 * 256 + 4 * 128 * 128 + 8 * 1024 + 2 * 2 * 64 * 4;
+    // four slots of activations (64 rows x 128 / 64 k) and raw weights (16 KiB either way), parameters, row sums
+    constexpr size_t lds_bytes = (size_t)4 * 64 * (WBITS == 4 ? 256 : 128) + 4 * 16384 + 8 * 1024 + 2 * 2 * 64 * 4;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
-    auto kern = wq_gemm4_kernel<ACT, STAGE_GROUPS>;
+    auto kern = wq_gemm4_kernel<ACT, STAGE_GROUPS, WBITS>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, s, p);
@@ -467,17 +501,20 @@ WqGemm4Plan make_wq_gemm4_plan(int64_t M, int64_t N, int64_t K, int w_bits, int6
                                const void *x, const void *w, const void *scale, const void *offset)
 {
     WqGemm4Plan pl{};
-    const int64_t row_bytes = N / 2, ldw_bytes = ldw_k * 4;
+    // int4: rows of N / 8 words, 128-row stages, 128-byte strips; int8: rows of N bytes, 64-row stages, 256-byte strips
+    const int64_t row_bytes = w_bits == 4 ? N / 2 : N, ldw_bytes = w_bits == 4 ? ldw_k * 4 : ldw_k;
+    const int64_t bk = w_bits == 4 ? 128 : 64, strip_bytes = w_bits == 4 ? 128 : 256;
     const int64_t group = group_size > 0 ? group_size : K;
     const bool grouped = group_size > 0 && group != K;
-    pl.ok = knob(kKnobWqGemm4Off) != 1 && w_bits == 4 && M > 32 && K >= 128 && K % 128 == 0 && N % 8 == 0 && (!grouped || group % 128 == 0) &&
+    pl.ok = knob(kKnobWqGemm4Off) != 1 && (w_bits == 4 || w_bits == 8) && M > 32 && K >= 128 && K % 128 == 0 &&
+            N % (w_bits == 4 ? 8 : 4) == 0 && (!grouped || group % bk == 0) &&
             ldw_bytes >= row_bytes && ldw_bytes % 16 == 0 && ldx % 8 == 0 && (x == nullptr || aligned(x, 16)) &&
             (w == nullptr || aligned(w, 16)) && (scale == nullptr || aligned(scale, 4)) && (offset == nullptr || aligned(offset, 4)) &&
             (uint64_t)K * (uint64_t)ldw_bytes < (1ull << 31) && (uint64_t)128 * (uint64_t)ldx * 2 + (uint64_t)K * 2 < (1ull << 31) &&
             (uint64_t)(K / group) * (uint64_t)N * 2 < (1ull << 31) && M <= 0x7fffffff;
     if (!pl.ok) return pl;
-    pl.strips = (int)((row_bytes + 127) / 128);
-    const int64_t stages = K / 128;
+    pl.strips = (int)((row_bytes + strip_bytes - 1) / strip_bytes);
+    const int64_t stages = K / bk;
     const int64_t units = grouped ? K / group : stages;
     // few tiles: split K in whole scale groups (per channel: in equal numbers of stages)
     pl.bm = 64;
@@ -493,15 +530,15 @@ WqGemm4Plan make_wq_gemm4_plan(int64_t M, int64_t N, int64_t K, int w_bits, int6
     while (S > 1 && (zone(S) > kWorkspaceZoneBytes || (!grouped && stages % S != 0))) S--;
     pl.S = (int)S;
     // per channel: one fold per workgroup, so a "group" is the workgroup's whole range
-    pl.gstages = (int)(grouped ? group / 128 : stages / S);
+    pl.gstages = (int)(grouped ? group / bk : stages / S);
     pl.zone_bytes = pl.S > 1 ? (size_t)zone(pl.S) : 0;
     if (tiles * pl.S > 0x7fffffff) pl.ok = false;
     return pl;
 }
 
-int launch_wq_gemm4(const WqGemm4Plan &plan, const void *x, int act_f16, const void *w, const void *scale, const void *offset,
-                    const void *bias, void *out, int64_t M, int64_t N, int64_t K, int64_t group_size, int64_t ldx, int64_t ldw_k,
-                    int64_t ldo, void *workspace, void *stream)
+int launch_wq_gemm4(const WqGemm4Plan &plan, const void *x, int act_f16, const void *w, int w_bits, const void *scale,
+                    const void *offset, const void *bias, void *out, int64_t M, int64_t N, int64_t K, int64_t group_size, int64_t ldx,
+                    int64_t ldw_k, int64_t ldo, void *workspace, void *stream)
 {
     WqGemm4Args p{};
     p.x = static_cast<const uint16_t *>(x);
@@ -513,8 +550,8 @@ int launch_wq_gemm4(const WqGemm4Plan &plan, const void *x, int act_f16, const v
     p.zone = plan.S > 1 ? reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kWorkspaceCounterCapacity) : nullptr;
     p.ldx = ldx;
     p.ldo = ldo;
-    p.ldw_bytes = (uint32_t)(ldw_k * 4);
-    p.row_bytes = (uint32_t)(N / 2);
+    p.ldw_bytes = (uint32_t)(w_bits == 4 ? ldw_k * 4 : ldw_k);
+    p.row_bytes = (uint32_t)(w_bits == 4 ? N / 2 : N);
     p.M = (int)M;
     p.N = (int)N;
     p.K = (int)K;
@@ -528,9 +565,10 @@ int launch_wq_gemm4(const WqGemm4Plan &plan, const void *x, int act_f16, const v
     const int64_t tiles = (int64_t)plan.tiles_m * plan.strips;
     (void)tiles;
     const unsigned grid = (unsigned)((plan.strips + 7) / 8 * 8 * plan.tiles_m * plan.S);
-    // a variant of its own where a scale group is one stage
-    if (p.grouped && plan.gstages == 1) return act_f16 ? launch4<1, true>(p, grid, s) : launch4<0, true>(p, grid, s);
-    return act_f16 ? launch4<1, false>(p, grid, s) : launch4<0, false>(p, grid, s);
+    if (w_bits == 8) return act_f16 ? launch4<1, false, 8>(p, grid, s) : launch4<0, false, 8>(p, grid, s);
+    // int4: a variant of its own where a scale group is one stage
+    if (p.grouped && plan.gstages == 1) return act_f16 ? launch4<1, true, 4>(p, grid, s) : launch4<0, true, 4>(p, grid, s);
+    return act_f16 ? launch4<1, false, 4>(p, grid, s) : launch4<0, false, 4>(p, grid, s);
 }
 
 } // namespace mi355

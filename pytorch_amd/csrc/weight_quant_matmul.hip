@@ -761,10 +761,8 @@ bool repack_applies(int64_t M, int64_t N, int64_t K, int64_t group_size, int64_t
 }
 int preferred_n_major_kernel(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size, int64_t ldw_k, int64_t ldx)
 {
-    if (w_bits == 4) {
-        if (make_wq_decode_plan(M, N, K, 4, group_size, ldw_k, ldx, nullptr, nullptr, nullptr, nullptr).ok) return kPreferDecode;
-        if (make_wq_gemm4_plan(M, N, K, 4, group_size, ldw_k, ldx, nullptr, nullptr, nullptr, nullptr).ok) return kPreferGemm4;
-    }
+    if (w_bits == 4 && make_wq_decode_plan(M, N, K, 4, group_size, ldw_k, ldx, nullptr, nullptr, nullptr, nullptr).ok) return kPreferDecode;
+    if (make_wq_gemm4_plan(M, N, K, w_bits, group_size, ldw_k, ldx, nullptr, nullptr, nullptr, nullptr).ok) return kPreferGemm4;
     if (make_wq_gemm_plan(M, N, K, w_bits, group_size, 1, ldw_k, ldx, nullptr, nullptr, nullptr, nullptr).ok) return kPreferGemm;
     return kPreferStream;
 }
@@ -812,6 +810,8 @@ extern "C" size_t mi355_weight_quant_matmul_workspace(int64_t M, int64_t N, int6
                 if (kp.ok && kp.partial_bytes + kp.counter_bytes > need) need = kp.partial_bytes + kp.counter_bytes;
             }
         } else {                            // the K-major layout may split differently
+            const WqGemm4Plan g8 = make_wq_gemm4_plan(M, N, K, 8, group_size, ldw_n_major, ldx, nullptr, nullptr, nullptr, nullptr);
+            if (g8.ok && g8.S > 1 && kWorkspaceZeroBytes > need) need = kWorkspaceZeroBytes;
             const WqKmPlan km = make_kmajor_plan(M, N, K, group_size, ldw_k_major, ldx, nullptr, nullptr);
             if (km.fast && km.partial_bytes + km.counter_bytes > need) need = km.partial_bytes + km.counter_bytes;
         }
@@ -872,7 +872,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
             if (st != MI355_OK) return st;
             const WqGemm4Plan g4 = make_wq_gemm4_plan(M, N, K, 4, group_size, pitch, ldx, x_bf16, w_kn, scale_gn, offset_gn);
             if (!g4.ok) return MI355_ERR_LAUNCH;       // planned with these strides a few lines up
-            return launch_wq_gemm4(g4, x_bf16, f16 ? 1 : 0, w_kn, scale_gn, offset_gn, bias, out_bf16, M, N, K, group_size, ldx, pitch,
+            return launch_wq_gemm4(g4, x_bf16, f16 ? 1 : 0, w_kn, 4, scale_gn, offset_gn, bias, out_bf16, M, N, K, group_size, ldx, pitch,
                                    ldo, workspace, stream);
         }
         const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, ldw_n, ldx, x_bf16, w);
@@ -949,7 +949,19 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
                 if (!workspace || workspace_bytes < kWorkspaceZeroBytes) return MI355_ERR_WORKSPACE;
                 if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
             }
-            return launch_wq_gemm4(g4, x_bf16, f16 ? 1 : 0, w, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, group_size, ldx, ldw_k,
+            return launch_wq_gemm4(g4, x_bf16, f16 ? 1 : 0, w, 4, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, group_size, ldx, ldw_k,
+                                   ldo, workspace, stream);
+        }
+    }
+    if (w_bits == 8 && n_major) {
+        // int8 [K, N], more than 32 rows: the same register-expanding kernel
+        const WqGemm4Plan g8 = make_wq_gemm4_plan(M, N, K, 8, group_size, ldw_k, ldx, x_bf16, w, scale_bf16, offset_bf16);
+        if (g8.ok && aligned(out_bf16, 2) && (!bias || aligned(bias, 2))) {
+            if (g8.S > 1) {
+                if (!workspace || workspace_bytes < kWorkspaceZeroBytes) return MI355_ERR_WORKSPACE;
+                if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;
+            }
+            return launch_wq_gemm4(g8, x_bf16, f16 ? 1 : 0, w, 8, scale_bf16, offset_bf16, bias, out_bf16, M, N, K, group_size, ldx, ldw_k,
                                    ldo, workspace, stream);
         }
     }

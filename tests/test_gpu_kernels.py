@@ -513,6 +513,46 @@ def test_weight_quant_int4_register_kernel_variants(capi, golden, case):
         capi.set_tuning("MI355_WQG_SPLIT", 0)
 
 
+INT8_REGISTER_CASES = [  # M, K, N, group (0: per channel), float16, forced split
+    (64, 128, 256, 0, False, 0),          # two stages of 64 rows: one per set of wavefronts
+    (100, 640, 1000, 64, False, 0),       # a scale group per stage, ragged rows, last strip holds 232 columns
+    (128, 768, 516, 192, True, 2),        # groups of three stages, two chunks of two groups, last strip holds 4 columns
+    (256, 4096, 512, 0, False, 4),        # per channel, four chunks of K
+    (72, 1024, 260, 128, False, 3),       # groups of two stages, uneven chunks
+]
+
+
+@pytest.mark.parametrize("case", INT8_REGISTER_CASES, ids=lambda c: "-".join(str(v) for v in c))
+def test_weight_quant_int8_register_kernel_variants(capi, golden, case):
+    """int8 weights [K, N] with more than 32 rows take the register-expanding kernel too (64-row stages, 256-byte
+    strips): group sizes of one, two and three stages and per channel, K splits, exchange through the L2 and through
+    memory; each variant repeats its own result bit for bit."""
+    M, K, N, gs, f16, split = case
+    d = workloads.w8a16_inputs(seed=M + N + K, M=M, K=K, N=N)
+    if gs:
+        g = torch.Generator().manual_seed(7)
+        d["antiquant_scale"] = (torch.rand(K // gs, N, generator=g) * 9e-3 + 1e-3).to(torch.bfloat16)
+        d["antiquant_offset"] = (torch.rand(K // gs, N, generator=g) * 8 - 4).to(torch.bfloat16)
+    bits_of = _bits
+    if f16:
+        d = _to_f16(d)
+        bits_of = _f16_bits
+    args = [d[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset")]
+    _, gold = golden.weight_quant_matmul(bits_of(d["x"]), d["weight"].numpy(), bits_of(d["antiquant_scale"]),
+                                         bits_of(d["antiquant_offset"]), group_size=gs, dtype="fp16" if f16 else "bf16")
+    capi.set_tuning("MI355_WQG_SPLIT", split)
+    try:
+        for variant in (0, 2):             # exchange through the L2 where the XCD allows; through memory
+            capi.set_tuning("MI355_WQ_GEMM4_OFF", variant)
+            out = capi.weight_quant_matmul(*args, group_size=gs)
+            bf16_gate(out, torch.from_numpy(gold))
+            for _ in range(2):
+                assert torch.equal(out, capi.weight_quant_matmul(*args, group_size=gs))
+    finally:
+        capi.set_tuning("MI355_WQ_GEMM4_OFF", 0)
+        capi.set_tuning("MI355_WQG_SPLIT", 0)
+
+
 @pytest.mark.parametrize("case", TILED_CASES, ids=lambda c: "-".join(str(v) for v in c))
 def test_weight_quant_tiled_kernel(capi, golden, case):
     bits, M, K, N, gs, f16, with_bias = case[:7]
