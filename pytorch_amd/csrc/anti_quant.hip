@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void anti_quant_vec_kernel(const AqArgs p)
             o.y = pack2<OUT_F16>(antiquant1(v[2], of[2], sc[2]), antiquant1(v[3], of[3], sc[3]));
             o.z = pack2<OUT_F16>(antiquant1(v[4], of[4], sc[4]), antiquant1(v[5], of[5], sc[5]));
             o.w = pack2<OUT_F16>(antiquant1(v[6], of[6], sc[6]), antiquant1(v[7], of[7], sc[7]));
-            *reinterpret_cast<u32x4 *>(p.out + (r0 + u) * p.ldo + c) = o;
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(p.out + (r0 + u) * p.ldo + c));
         }
     }
 }

@@ -312,7 +312,7 @@ __global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *
 #pragma unroll
             for (int k = 0; k < 8; k++) q[k] = quant_exact(f[i][k], scale);
         }
-        if (idx < nvec) yr[idx] = u32x2{pack4(q[0], q[1], q[2], q[3]), pack4(q[4], q[5], q[6], q[7])};
+        if (idx < nvec) __builtin_nontemporal_store(u32x2{pack4(q[0], q[1], q[2], q[3]), pack4(q[4], q[5], q[6], q[7])}, yr + idx);
     }
 }
 

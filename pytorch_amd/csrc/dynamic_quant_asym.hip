@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int v = t + 256 * i;
-                kept[i] = v < cols / 8 ? reinterpret_cast<const u32x4 *>(xr)[v] : u32x4{0, 0, 0, 0};
+                kept[i] = v < cols / 8 ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xr) + v) : u32x4{0, 0, 0, 0};
             }
         }
         if constexpr (VEC) {
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
                 u32x2 o;
                 o.x = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
                 o.y = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
-                reinterpret_cast<u32x2 *>(yr)[v] = o;
+                __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(yr) + v);
             }
         } else {
             for (int j = t; j < cols; j += 256) {

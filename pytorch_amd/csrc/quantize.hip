@@ -113,7 +113,7 @@ __device__ __forceinline__ void load8(const void *x, int64_t e, float (&v)[8])
 #pragma unroll
         for (int i = 0; i < 4; i++) v[i] = a[i], v[4 + i] = b[i];
     } else {
-        const u32x4 w = *reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(x) + e);
+        const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(x) + e));
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t u = w[i];
@@ -144,7 +144,7 @@ __device__ __forceinline__ void store8(void *out, int64_t e, const float (&q)[8]
             o.x |= ((uint32_t)(int)q[i] & 0xffu) << (8 * i);
             o.y |= ((uint32_t)(int)q[4 + i] & 0xffu) << (8 * i);
         }
-        *reinterpret_cast<u32x2 *>(static_cast<uint8_t *>(out) + e) = o;
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(static_cast<uint8_t *>(out) + e));
     }
 }
 

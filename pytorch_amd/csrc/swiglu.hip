@@ -15,13 +15,13 @@ __global__ __launch_bounds__(256) void swiglu_vec_kernel(const uint16_t *__restr
         const int64_t r = e / half_vec;
         const int v = (int)(e % half_vec);
         const u32x4 *a = reinterpret_cast<const u32x4 *>(x + r * ldx) + v;
-        const u32x4 av = *a, bv = a[half_vec];
+        const u32x4 av = __builtin_nontemporal_load(a), bv = __builtin_nontemporal_load(a + half_vec);
         u32x4 o;
         o.x = swiglu2(av.x, bv.x);
         o.y = swiglu2(av.y, bv.y);
         o.z = swiglu2(av.z, bv.z);
         o.w = swiglu2(av.w, bv.w);
-        reinterpret_cast<u32x4 *>(out)[e] = o;
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(out) + e);
     }
 }
 
