@@ -85,17 +85,17 @@ __device__ __forceinline__ uint32_t pack4(uint32_t a, uint32_t b, uint32_t c, ui
     return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
 }
 
-// TPR threads cooperate on one row (64 = one wavefront, no barrier; 256 = whole block);
+// TPR threads cooperate on one row (64 = one wavefront, no barrier; more = the whole block of BLOCK threads);
 // each thread holds ITERS vectors of 8 elements.
 // SWIGLU: the input row holds two halves of `cols` elements each and the quantised row is
 // bf16(silu(act half)) * other half (rounded to bf16 like the stand-alone SwiGLU kernel): the fused
 // SwiGLU + dynamic_quant of an MLP, which saves writing and re-reading the bf16 activation.
-template <int TPR, int ITERS, bool FP16, bool SWIGLU = false>
-__global__ __launch_bounds__(kBlock) void dq_rows_kernel(const uint16_t *__restrict__ x, int8_t *__restrict__ y,
+template <int TPR, int ITERS, bool FP16, bool SWIGLU = false, int BLOCK = kBlock>
+__global__ __launch_bounds__(BLOCK) void dq_rows_kernel(const uint16_t *__restrict__ x, int8_t *__restrict__ y,
                                                          float *__restrict__ scale_out, int64_t rows, int cols,
                                                          int64_t row_stride, int act_offset = 0, int mul_offset = 0)
 {
-    constexpr int RPB = kBlock / TPR;
+    constexpr int RPB = BLOCK / TPR;
     const int t = threadIdx.x % TPR;
     const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
     const bool live = row < rows;
@@ -131,11 +131,11 @@ __global__ __launch_bounds__(kBlock) void dq_rows_kernel(const uint16_t *__restr
     uint32_t m16 = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
     m16 = wave_max_u32(m16);
     if constexpr (TPR > 64) {
-        __shared__ uint32_t part[kBlock / 64];
+        __shared__ uint32_t part[BLOCK / 64];
         if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m16;
         __syncthreads();
 #pragma unroll
-        for (int w = 0; w < kBlock / 64; w++) m16 = part[w] > m16 ? part[w] : m16;
+        for (int w = 0; w < BLOCK / 64; w++) m16 = part[w] > m16 ? part[w] : m16;
     }
     if (!live) return;
 
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void dq_generic_kernel(const uint16_t *__re
     }
 }
 
-// Rows pre-multiplied by smooth scales, cols % 8 == 0 and at most 2048 * MAXV, 16-byte aligned rows and smooth scales: one
+// Rows pre-multiplied by smooth scales, cols % 8 == 0 and at most 8 * BLOCK * MAXV, 16-byte aligned rows and smooth scales: one
 // block per row, the products (arbitrary float32 significands) stay in registers between the maximum and the
 // quantisation.  x / scale uses the row's refined reciprocal with the operation sequence of the compiler's own
 // float32 division (quotient and two residual corrections) when the scale lies within [2^-60, 2^60]: that sequence's
@@ -234,8 +234,8 @@ __global__ __launch_bounds__(kBlock) void dq_generic_kernel(const uint16_t *__re
 // SWIGLU (bf16): the row holds two halves of `cols` elements and the value that is smoothed and quantised is
 // bf16(silu(act half)) * other half, rounded to bf16 like the stand-alone SwiGLU kernel; act_offset / mul_offset are
 // the positions of the two halves in 16-byte vectors.
-template <bool FP16, bool SWIGLU = false, int MAXV = 4>
-__global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *__restrict__ x,
+template <bool FP16, bool SWIGLU = false, int MAXV = 4, int BLOCK = kBlock>
+__global__ __launch_bounds__(BLOCK) void dq_smooth_rows_kernel(const uint16_t *__restrict__ x,
                                                                 const uint16_t *__restrict__ smooth,
                                                                 int8_t *__restrict__ y, float *__restrict__ scale_out,
                                                                 int cols, int64_t row_stride, int act_offset = 0,
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < MAXV; i++) {
-        const int idx = t + i * kBlock;
+        const int idx = t + i * BLOCK;
         u32x4 a{0, 0, 0, 0}, b{0, 0, 0, 0};
         if (idx < nvec) {
             if constexpr (SWIGLU) {
@@ -277,11 +277,11 @@ __global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *
         }
     }
     uint32_t mb = wave_max_u32(__float_as_uint(amax));        // non-negative floats order like their bit patterns
-    __shared__ uint32_t part[kBlock / 64];
+    __shared__ uint32_t part[BLOCK / 64];
     if ((t & 63) == 0) part[t >> 6] = mb;
     __syncthreads();
 #pragma unroll
-    for (int w = 0; w < kBlock / 64; w++) mb = part[w] > mb ? part[w] : mb;
+    for (int w = 0; w < BLOCK / 64; w++) mb = part[w] > mb ? part[w] : mb;
     amax = __uint_as_float(mb);
     const float scale = amax / 127.0f;
     if (t == 0) scale_out[row] = scale;
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *
     r = __builtin_fmaf(__builtin_fmaf(-scale, r, 1.0f), r, r);
 #pragma unroll
     for (int i = 0; i < MAXV; i++) {
-        const int idx = t + i * kBlock;
+        const int idx = t + i * BLOCK;
         uint32_t q[8];
         if (zero) {
 #pragma unroll
@@ -316,27 +316,27 @@ __global__ __launch_bounds__(kBlock) void dq_smooth_rows_kernel(const uint16_t *
     }
 }
 
-template <int TPR, int ITERS>
+template <int TPR, int ITERS, int BLOCK = kBlock>
 void launch_rows(bool fp16, const uint16_t *x, int8_t *y, float *scale, int64_t rows, int cols, int64_t stride,
                  hipStream_t s)
 {
-    constexpr int RPB = kBlock / TPR;
+    constexpr int RPB = BLOCK / TPR;
     const unsigned grid = (unsigned)((rows + RPB - 1) / RPB);
     if (fp16)
-        hipLaunchKernelGGL((dq_rows_kernel<TPR, ITERS, true>), dim3(grid), dim3(kBlock), 0, s, x, y, scale, rows, cols,
-                           stride);
+        hipLaunchKernelGGL((dq_rows_kernel<TPR, ITERS, true, false, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, x, y, scale, rows,
+                           cols, stride);
     else
-        hipLaunchKernelGGL((dq_rows_kernel<TPR, ITERS, false>), dim3(grid), dim3(kBlock), 0, s, x, y, scale, rows,
+        hipLaunchKernelGGL((dq_rows_kernel<TPR, ITERS, false, false, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, x, y, scale, rows,
                            cols, stride);
 }
 
-template <int TPR, int ITERS>
+template <int TPR, int ITERS, int BLOCK = kBlock>
 void launch_swiglu_rows(const uint16_t *x, int8_t *y, float *scale, int64_t rows, int cols, int64_t stride, int act_off,
                         int mul_off, hipStream_t s)
 {
-    constexpr int RPB = kBlock / TPR;
+    constexpr int RPB = BLOCK / TPR;
     const unsigned grid = (unsigned)((rows + RPB - 1) / RPB);
-    hipLaunchKernelGGL((dq_rows_kernel<TPR, ITERS, false, true>), dim3(grid), dim3(kBlock), 0, s, x, y, scale, rows, cols,
+    hipLaunchKernelGGL((dq_rows_kernel<TPR, ITERS, false, true, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, x, y, scale, rows, cols,
                        stride, act_off, mul_off);
 }
 
@@ -386,7 +386,7 @@ int run_swiglu_quant(const void *x_bf16, int activate_left, const void *smooth, 
     const int64_t act = activate_left ? 0 : half, mul = activate_left ? half : 0;
     const int64_t nvec = half >> 3;
     const bool vec_ok = half > 0 && (half & 7) == 0 && (x_row_stride & 7) == 0 && aligned(xp, 16) && aligned(y, 8) &&
-                        nvec <= kBlock * 8;
+                        nvec <= 1024 * 8;       // halves of up to 16384 elements on 256 threads, up to 65536 on 1024
     const uint16_t *sm = static_cast<const uint16_t *>(smooth);
     if (sm) {
         if (!aligned(sm, 2)) return MI355_ERR_ALIGNMENT;
@@ -395,9 +395,15 @@ int run_swiglu_quant(const void *x_bf16, int activate_left, const void *smooth, 
             if (nvec <= kBlock * 4)
                 hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 4>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y,
                                    scale, c, x_row_stride, ao, mo);
-            else
+            else if (nvec <= kBlock * 8)
                 hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 8>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y,
                                    scale, c, x_row_stride, ao, mo);
+            else if (nvec <= 1024 * 4)
+                hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 4, 1024>), dim3((unsigned)rows), dim3(1024), 0, s, xp, sm,
+                                   y, scale, c, x_row_stride, ao, mo);
+            else
+                hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 8, 1024>), dim3((unsigned)rows), dim3(1024), 0, s, xp, sm,
+                                   y, scale, c, x_row_stride, ao, mo);
         } else {
             hipLaunchKernelGGL(swiglu_dq_generic_kernel, dim3((unsigned)rows), dim3(kBlock), 0, s, xp, y, scale, half,
                                x_row_stride, act, mul, sm);
@@ -411,7 +417,9 @@ int run_swiglu_quant(const void *x_bf16, int activate_left, const void *smooth, 
         else if (nvec <= 64 * 4) launch_swiglu_rows<64, 4>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
         else if (nvec <= 256 * 2) launch_swiglu_rows<256, 2>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
         else if (nvec <= 256 * 4) launch_swiglu_rows<256, 4>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
-        else launch_swiglu_rows<256, 8>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
+        else if (nvec <= 256 * 8) launch_swiglu_rows<256, 8>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
+        else if (nvec <= 1024 * 4) launch_swiglu_rows<1024, 4, 1024>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
+        else launch_swiglu_rows<1024, 8, 1024>(xp, y, scale, rows, c, x_row_stride, ao, mo, s);
     } else {
         hipLaunchKernelGGL(swiglu_dq_generic_kernel, dim3((unsigned)rows), dim3(kBlock), 0, s, xp, y, scale, half, x_row_stride,
                            act, mul);
@@ -450,8 +458,9 @@ extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smoo
     const uint16_t *xp = static_cast<const uint16_t *>(x);
 
     const int64_t nvec = cols >> 3;
+    // rows of up to 16384 elements on 256 threads, up to 65536 on 1024 (eight 16-byte vectors per thread at most)
     const bool vec_ok = !smooth && cols > 0 && (cols & 7) == 0 && (x_row_stride & 7) == 0 && aligned(x, 16) &&
-                        aligned(y, 8) && nvec <= kBlock * 8;
+                        aligned(y, 8) && nvec <= 1024 * 8;
     if (vec_ok) {
         const int c = (int)cols;
         if (nvec <= 64 * 1) launch_rows<64, 1>(fp16, xp, y, scale, rows, c, x_row_stride, s);
@@ -459,19 +468,27 @@ extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smoo
         else if (nvec <= 64 * 4) launch_rows<64, 4>(fp16, xp, y, scale, rows, c, x_row_stride, s);
         else if (nvec <= 256 * 2) launch_rows<256, 2>(fp16, xp, y, scale, rows, c, x_row_stride, s);
         else if (nvec <= 256 * 4) launch_rows<256, 4>(fp16, xp, y, scale, rows, c, x_row_stride, s);
-        else launch_rows<256, 8>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+        else if (nvec <= 256 * 8) launch_rows<256, 8>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+        else if (nvec <= 1024 * 4) launch_rows<1024, 4, 1024>(fp16, xp, y, scale, rows, c, x_row_stride, s);
+        else launch_rows<1024, 8, 1024>(fp16, xp, y, scale, rows, c, x_row_stride, s);
     } else if (smooth && cols > 0 && (cols & 7) == 0 && (x_row_stride & 7) == 0 && aligned(x, 16) && aligned(smooth, 16) &&
-               aligned(y, 8) && nvec <= kBlock * 8) {
+               aligned(y, 8) && nvec <= 1024 * 8) {
         const uint16_t *sm = static_cast<const uint16_t *>(smooth);
-#define MI355_DQS_LAUNCH(F, V) \
-    hipLaunchKernelGGL((dq_smooth_rows_kernel<F, false, V>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale, (int)cols, \
+#define MI355_DQS_LAUNCH(F, V, B) \
+    hipLaunchKernelGGL((dq_smooth_rows_kernel<F, false, V, B>), dim3((unsigned)rows), dim3(B), 0, s, xp, sm, y, scale, (int)cols, \
                        x_row_stride)
         if (nvec <= kBlock * 4) {
-            if (fp16) MI355_DQS_LAUNCH(true, 4);
-            else MI355_DQS_LAUNCH(false, 4);
+            if (fp16) MI355_DQS_LAUNCH(true, 4, kBlock);
+            else MI355_DQS_LAUNCH(false, 4, kBlock);
+        } else if (nvec <= kBlock * 8) {
+            if (fp16) MI355_DQS_LAUNCH(true, 8, kBlock);
+            else MI355_DQS_LAUNCH(false, 8, kBlock);
+        } else if (nvec <= 1024 * 4) {
+            if (fp16) MI355_DQS_LAUNCH(true, 4, 1024);
+            else MI355_DQS_LAUNCH(false, 4, 1024);
         } else {
-            if (fp16) MI355_DQS_LAUNCH(true, 8);
-            else MI355_DQS_LAUNCH(false, 8);
+            if (fp16) MI355_DQS_LAUNCH(true, 8, 1024);
+            else MI355_DQS_LAUNCH(false, 8, 1024);
         }
 #undef MI355_DQS_LAUNCH
     } else {

@@ -27,7 +27,8 @@ def _bits(t):
 # ------------------------------------------------------------------ dynamic_quant
 
 @pytest.mark.parametrize("rows,cols", [(2048, 4096), (64, 14336), (7, 512), (33, 1024), (5, 8), (3, 40), (2, 16384),
-                                       (2, 20000), (9, 100), (1, 1)])
+                                       (2, 20000), (9, 100), (1, 1), (5, 28672), (3, 32776), (2, 65536), (2, 65544),
+                                       (3, 16388)])
 def test_dynamic_quant_bit_exact(capi, golden, rows, cols):
     x = workloads.dynamic_quant_input(seed=rows + cols, rows=rows, cols=cols)
     y, s = capi.dynamic_quant(x.cuda())
@@ -104,10 +105,11 @@ def test_dynamic_quant_smooth(capi, golden):
     assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(y.cpu().numpy(), yg)
 
 
-@pytest.mark.parametrize("rows,cols", [(2048, 4096), (33, 8192), (7, 24), (64, 14336), (5, 1000), (3, 8200)])
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (33, 8192), (7, 24), (64, 14336), (5, 1000), (3, 8200), (5, 28672),
+                                       (3, 65536), (3, 65544)])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 def test_dynamic_quant_smooth_shapes(capi, golden, rows, cols, dt):
-    """Smooth scales through the register-resident kernel (cols % 8 == 0, up to 8192) and the two-pass one (wider or odd
+    """Smooth scales through the register-resident kernels (cols % 8 == 0, up to 65536) and the two-pass one (wider or odd
     rows), both input types, with rows that hold zeros, a zero row, tiny and huge values (both division paths of the
     kernel), bit-exact against the oracle."""
     g = torch.Generator().manual_seed(rows + cols)
@@ -977,7 +979,8 @@ def test_dynamic_quant_asymmetric_extreme_rows(capi, golden):
 
 # ------------------------------------------------------------------ error paths (host side, no kernel runs)
 
-@pytest.mark.parametrize("rows,half", [(64, 14336), (512, 4096), (33, 512), (5, 100), (3, 16384 + 8), (7, 24)])
+@pytest.mark.parametrize("rows,half", [(64, 14336), (512, 4096), (33, 512), (5, 100), (3, 16384 + 8), (7, 24), (5, 28672),
+                                       (2, 65536), (2, 65536 + 8)])
 @pytest.mark.parametrize("left", [True, False])
 def test_swiglu_quant_with_smooth_scales(capi, golden, rows, half, left):
     """Fused SwiGLU + smooth scales + dynamic quantisation equals the oracle's composition bit for bit: the
@@ -995,7 +998,8 @@ def test_swiglu_quant_with_smooth_scales(capi, golden, rows, half, left):
     assert torch.equal(y2, y) and torch.equal(s2, s)
 
 
-@pytest.mark.parametrize("rows,half", [(64, 14336), (2048, 14336), (33, 512), (5, 100), (3, 16384 + 8), (7, 24)])
+@pytest.mark.parametrize("rows,half", [(64, 14336), (2048, 14336), (33, 512), (5, 100), (3, 16384 + 8), (7, 24), (5, 28672),
+                                       (2, 65536), (2, 65536 + 8)])
 @pytest.mark.parametrize("left", [True, False])
 def test_swiglu_quant_equals_composition(capi, golden, rows, half, left):
     g = torch.Generator().manual_seed(rows + half)
