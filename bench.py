@@ -503,7 +503,7 @@ def main():
 
     if want("c5"):
         H, I = 4096, 14336
-        for Mx in (64, 2048):
+        for Mx in (16, 64, 2048):
             d5 = workloads.mlp_inputs(seed=0, M=Mx, hidden=H, inter=I)
             x = d5["x"].to(dev)
             sgu, sd = d5["scale_gate_up"].to(dev), d5["scale_down"].to(dev)
@@ -562,7 +562,7 @@ def main():
                      "chain_us": round(us, 2), "chain_us_cache_resident_weights": round(hot, 2),
                      "int8_tops": round(mops / (us * 1e-6) / 1e12, 2),
                      "roofline": ({"bound": "hbm", "achieved": round(abytes / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                   "frac": round(abytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None} if Mx == 64 else
+                                   "frac": round(abytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None} if Mx <= 64 else
                                   {"bound": "mfma", "achieved": round(mops / (us * 1e-6) / 1e12, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                                    "frac": round(mops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None}),
                      "algorithmic_bytes": int(abytes)}

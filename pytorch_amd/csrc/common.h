@@ -77,8 +77,10 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
 // load time, through the environment variable of the same name.
 // MI355_WQ_GEMM4_OFF / MI355_WQ_DECODE_OFF: 1 = the register-expanding int4 GEMM / the int4 decode kernel is not used;
 // 2 = its K-split exchange always writes through to memory.
+// MI355_QMM_DECODE_OFF: 1 = quant_matmul with at most 64 rows takes the tiled kernel instead of the decode kernel.
 enum Knob { kKnobWqSplit, kKnobWqW, kKnobWqgSplit, kKnobWqgBm, kKnobWqGemmOff, kKnobWqkMt, kKnobWqkNw, kKnobWqkKs,
-            kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmDeepOff, kKnobWqGemm4Off, kKnobCount };
+            kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmDeepOff, kKnobWqGemm4Off, kKnobQmmDecodeOff,
+            kKnobCount };
 int knob(Knob k);
 
 inline int check_launch()

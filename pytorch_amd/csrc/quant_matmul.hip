@@ -21,6 +21,7 @@
 // evaluates ((float(acc) * pertoken[m]) * scale[n]) + bias[n] with separately rounded binary32
 // operations (contraction is disabled for this library) and rounds once to bf16.
 #include "common.h"
+#include "quant_matmul_decode.h"
 #include <stdio.h>
 #include <type_traits>
 #include <stdlib.h>
@@ -846,6 +847,7 @@ QmmPlan make_qmm_plan(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ld
         if (S > kt / 4) S = kt / 4;
         if (S > 16) S = 16;
         if (S < 1) S = 1;
+        if (qmm_decode_shape(M, N, K)) S = 1;             // the decode kernel splits K inside its workgroups
         if (const int f = knob(kKnobQmmSplit))            // debugging aid
             if (f >= 1 && f <= kt) S = f;
         pl.S = (int)S;
@@ -937,6 +939,27 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
         ldbt = K;
     }
     tiled = tiled && (ldbt & 15) == 0 && aligned(bt, 16);
+    if (tiled && !out_i32 && !out_i8 && !qparam && knob(kKnobQmmSplit) == 0 && knob(kKnobQmmTile) == 0) {
+        // at most 64 rows: the barrier-free kernel that splits K inside the workgroup (quant_matmul_decode.hip)
+        QmmDecodeArgs d;
+        d.a = a;
+        d.bt = bt;
+        d.pertoken = pertoken_scale;
+        d.scale = scale;
+        d.bias = bias;
+        d.bias_kind = bias_dtype;
+        d.out_f16 = out_dtype == MI355_OUT_FP16;
+        d.out = out;
+        d.lda = lda;
+        d.ldbt = ldbt;
+        d.ldc = ldc;
+        d.M = (int)M;
+        d.N = (int)N;
+        d.K = (int)K;
+        d.scale_len = (int)scale_len;
+        const int st = launch_qmm_decode(d, s);
+        if (st != MI355_ERR_UNSUPPORTED) return st;
+    }
     if (!tiled) {
         hipLaunchKernelGGL(qmm_generic_kernel, dim3((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16)), dim3(256), 0, s,
                            a, b, pertoken_scale, scale, (int)scale_len, bias, bias_dtype, out_dtype == MI355_OUT_FP16 ? 1 : 0, out,

@@ -321,6 +321,46 @@ def test_quant_matmul_split_k_repeated_launches(capi, golden):
         assert np.array_equal(_bits(out), want)
 
 
+QMM_DECODE_CASES = [(1, 4096, 4096), (7, 1024, 2048), (16, 1152, 2056), (5, 14336, 4096), (3, 11008, 2048), (16, 16384, 2048),
+                    (1, 1024, 8200), (17, 4096, 6144), (32, 8192, 2048), (30, 2176, 4100), (33, 4096, 4104), (64, 2048, 5120),
+                    (48, 1024, 16384)]
+
+
+@pytest.mark.parametrize("M,K,N", QMM_DECODE_CASES)
+def test_quant_matmul_decode_kernel(capi, golden, M, K, N):
+    """At most 64 rows and a weight stored [N, K]: the kernel that splits K over the wavefronts of a workgroup and walks
+    over strips of 16 columns (one, two and four tiles of 16 rows; 1 to 16 steps per wavefront, even and uneven; strips
+    that end past N; more strips than workgroups).  Outputs bit-identical to the oracle for every bias kind, both output
+    types, with and without per-token scales, a single scale, pitched activations; and to the tiled kernel."""
+    d = workloads.quant_matmul_inputs(seed=M + K + N, M=M, K=K, N=N, weight_nk=True, bias=True)
+    g = torch.Generator().manual_seed(M + N)
+    bias_i32 = torch.randint(-(1 << 20), 1 << 20, (N,), generator=g, dtype=torch.int32)
+    bias_f32 = torch.randn(N, generator=g)
+    x1, x2, sc, ps = d["x1"].cuda(), d["x2"].cuda(), d["scale"].cuda(), d["pertoken_scale"].cuda()
+    assert capi.lib().mi355_quant_matmul_workspace(M, N, K, 1, K) == 0          # no split of K over workgroups
+    acc = golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy())
+    cases = [(d["bias"], torch.bfloat16, "bf16", True), (bias_i32, torch.bfloat16, "bf16", True), (bias_f32, torch.float16, "fp16", True),
+             (None, torch.float16, "fp16", True), (None, torch.bfloat16, "bf16", False), (bias_f32, torch.bfloat16, "bf16", False)]
+    for bias, dt, name, with_ps in cases:
+        out = capi.quant_matmul(x1, x2, sc, ps if with_ps else None, None if bias is None else bias.cuda(), out_dtype=dt)
+        bias_np = None if bias is None else (_bits(bias) if bias.dtype == torch.bfloat16 else bias.numpy())
+        want = golden.quant_matmul_epilogue_ex(acc, d["scale"].numpy(), d["pertoken_scale"].numpy() if with_ps else None, bias_np, out=name)
+        assert np.array_equal(out.cpu().view(torch.int16).numpy().view(np.uint16), want), (name, with_ps, None if bias is None else bias.dtype)
+    # one scale for all columns; activations that are a view of a wider matrix
+    one = capi.quant_matmul(x1, x2, sc[:1].contiguous(), ps, d["bias"].cuda())
+    want = golden.quant_matmul_epilogue_ex(acc, d["scale"].numpy()[:1], d["pertoken_scale"].numpy(), _bits(d["bias"]), out="bf16")
+    assert np.array_equal(_bits(one), want)
+    wide = torch.zeros(M, K + 64, dtype=torch.int8, device="cuda")
+    wide[:, :K] = x1
+    ref = capi.quant_matmul(x1, x2, sc, ps, d["bias"].cuda())
+    assert torch.equal(capi.quant_matmul(wide[:, :K], x2, sc, ps, d["bias"].cuda()), ref)
+    capi.set_tuning("MI355_QMM_DECODE_OFF", 1)
+    try:
+        assert torch.equal(capi.quant_matmul(x1, x2, sc, ps, d["bias"].cuda()), ref)
+    finally:
+        capi.set_tuning("MI355_QMM_DECODE_OFF", 0)
+
+
 # ------------------------------------------------------------------ weight-quant matmul
 
 def _wq_golden(golden, d, group):
