@@ -802,27 +802,6 @@ constexpr TileChoice kTiles[] = {{256, 256, 256, 60.0, 57.0}, {256, 224, 256, 55
                                  {128, 320, 256, 48.0, 43.0}, {128, 256, 256, 40.0, 45.6}, {128, 192, 512, 55.8, 58.8},
                                  {128, 128, 512, 40.0, 43.3}, {64, 256, 512, 40.0, 52.6},  {64, 128, 512, 24.0, 30.0}};
 
-// Pick the tile shape that minimises (rounds of resident workgroups) x (time per round).
-TileChoice choose_tile(int M, int N)
-{
-    if (const int forced = knob(kKnobQmmTile)) {          // debugging aid: bm * 1000 + bn
-        for (const TileChoice &c : kTiles)
-            if (c.bm == forced / 1000 && c.bn == forced % 1000) return c;
-    }
-    TileChoice best = kTiles[0];
-    double best_cost = 1e300;
-    for (const TileChoice &c : kTiles) {
-        const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
-        const long rounds = (tiles + c.slots - 1) / c.slots;
-        const double cost = rounds == 1 ? c.single_us : (double)rounds * c.round_us;
-        if (cost < best_cost) {
-            best_cost = cost;
-            best = c;
-        }
-    }
-    return best;
-}
-
 // Workspace layout: [arrival counters | split-K partial sums | transposed weight].
 struct QmmPlan {
     TileChoice tile;
@@ -830,28 +809,65 @@ struct QmmPlan {
     size_t counter_bytes, partial_bytes, transpose_bytes;
 };
 
+// Pick the tile shape and the split of K with the smallest estimated time.  The table above gives a launch at K = 4096
+// without a split; other depths scale the part of it that is the K loop (`kBaseUs` is what a launch costs around the
+// loop).  Two terms that the table does not hold are added: every tile reads (bm + bn) x K bytes through the L2, which
+// bounds small tiles on a long K (64x128 tiles on 1024x14336x4096: 1.4 GB, 107 us), and a split of K moves
+// wgs x bm x bn x 4 bytes of partial sums out and in again, the S - 1 foreign chunks of a tile through the one workgroup
+// that collects them (128x256 tiles split twelve ways: 39 us where a four-way split of 64x128 tiles takes 25).
+// Constants fitted to sweeps over tile x split on M = 128 .. 2048, K = 8192 .. 28672 (the estimate's choice is the
+// measured best on nine of ten shapes and 16 % off on the tenth; at K = 4096 without a split the estimate is the table
+// itself).
+constexpr double kBaseUs = 6.0, kL2BytesPerUs = 12e6, kExchangeUs = 1.0, kExchangeBytesPerUs = 12e6, kCollectorBytesPerUs = 100e3;
+
+void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, TileChoice *tile, int *split)
+{
+    const int forced_tile = knob(kKnobQmmTile);             // debugging aids: bm * 1000 + bn, and the split
+    const int forced_split = knob(kKnobQmmSplit);
+    const int64_t kt = K / BK;
+    double best_cost = 1e300;
+    *tile = kTiles[0];
+    *split = 1;
+    for (const TileChoice &c : kTiles) {
+        if (forced_tile && (c.bm != forced_tile / 1000 || c.bn != forced_tile % 1000)) continue;
+        const int64_t tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+        for (const int S : {1, 2, 3, 4, 6, 8, 12, 16}) {
+            if (forced_split >= 1 && forced_split <= kt && may_split) {
+                if (S != 1) continue;                       // one candidate per tile: the forced split
+            } else if (S > 1 && (!may_split || tiles > 128 || kt / S < 4)) {
+                continue;                                   // few tiles and at least four K steps per workgroup
+            }
+            const int s_eff = forced_split >= 1 && forced_split <= kt && may_split ? forced_split : S;
+            const int64_t wgs = tiles * s_eff;
+            const int64_t rounds = (wgs + c.slots - 1) / c.slots;
+            const double at_4096 = rounds == 1 ? c.single_us : (double)rounds * c.round_us;
+            double cost = kBaseUs + (at_4096 - kBaseUs) * ((double)kt / s_eff) / 32.0;
+            const double l2 = kBaseUs + (double)tiles * (c.bm + c.bn) * (double)K / kL2BytesPerUs;
+            if (l2 > cost) cost = l2;
+            if (s_eff > 1)
+                cost += kExchangeUs + (double)wgs * c.bm * c.bn * 8.0 / kExchangeBytesPerUs +
+                        (double)(s_eff - 1) * c.bm * c.bn * 4.0 / kCollectorBytesPerUs;
+            if (cost < best_cost) {
+                best_cost = cost;
+                *tile = c;
+                *split = s_eff;
+            }
+        }
+    }
+}
+
 // `zero_area`: bytes in front of the scratch part of the workspace (the shared zero area, or just the counters when the
 // workspace is private to this operator)
 QmmPlan make_qmm_plan(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n, size_t zero_area = kWorkspaceZeroBytes)
 {
     QmmPlan pl{};
-    pl.tile = choose_tile((int)M, (int)N);
-    pl.S = 1;
     const bool tiled_shape = K >= BK && K % BK == 0;
-    if (tiled_shape) {
-        // Few tiles and a long K (the narrow GEMMs of small batches): split K until the CUs are busy, keeping at
-        // least four K steps per workgroup.
+    // the decode kernel splits K inside its workgroups (it is not used while a tile or a split is forced)
+    const bool decode = qmm_decode_shape(M, N, K) && knob(kKnobQmmSplit) == 0 && knob(kKnobQmmTile) == 0;
+    choose_tile_and_split(M, N, K, tiled_shape && !decode, &pl.tile, &pl.S);
+    if (tiled_shape && pl.S > 1) {
         const int64_t tiles = ((M + pl.tile.bm - 1) / pl.tile.bm) * ((N + pl.tile.bn - 1) / pl.tile.bn);
-        const int64_t kt = K / BK;
-        int64_t S = tiles <= 128 ? 256 / tiles : 1;
-        if (S > kt / 4) S = kt / 4;
-        if (S > 16) S = 16;
-        if (S < 1) S = 1;
-        if (qmm_decode_shape(M, N, K)) S = 1;             // the decode kernel splits K inside its workgroups
-        if (const int f = knob(kKnobQmmSplit))            // debugging aid
-            if (f >= 1 && f <= kt) S = f;
-        pl.S = (int)S;
-        if (pl.S > 1) pl.partial_bytes = (size_t)tiles * pl.S * pl.tile.bm * pl.tile.bn * 4;   // tiles <= 128 counters
+        pl.partial_bytes = (size_t)tiles * pl.S * pl.tile.bm * pl.tile.bn * 4;   // tiles <= 128 counters
     }
     // a contiguous [K,N] weight is transposed into the workspace
     pl.transpose_bytes = tiled_shape && ldb_k != 1 && ldb_n == 1 ? (size_t)N * (size_t)K : 0;
