@@ -63,7 +63,7 @@ def _parse():
     ap.add_argument("--eager", action="store_true",
                     help="launch the timed headline steps one by one instead of from a captured graph (kernel traces:\n"
                          "launches of a graph overlap, which blurs per-kernel durations)")
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c2i8,c3,c4,a4w4,c5,aq,qz for the 'others' section")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c2i8,c3,c4,qd,a4w4,c5,aq,qz for the 'others' section")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="launch a 256 MiB device copy and then each main kernel once on fresh buffers (for "
                          "`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: the copy calibrates the counters)")
@@ -171,6 +171,16 @@ def _pmc_pass(torch, pa, workloads, dev):
     torch.cuda.synchronize()
     pa.npu_weight_quant_batchmatmul(g4["x"], wk.t(), s4t, o4t, None, None, None, 128)
     pa.npu_quant_matmul(xa4, wa.t(), g["scale"], pertoken_scale=g["pertoken_scale"], output_dtype=torch.bfloat16)
+    # the decode kernel of quant_matmul: the two projections of the MLP at 16 rows, weights no kernel has touched
+    wgu = torch.randint(-128, 128, (28672, 4096), dtype=torch.int8, device=dev)
+    wdn = torch.randint(-128, 128, (4096, 14336), dtype=torch.int8, device=dev)
+    xq1 = torch.randint(-128, 128, (16, 4096), dtype=torch.int8, device=dev)
+    xq2 = torch.randint(-128, 128, (16, 14336), dtype=torch.int8, device=dev)
+    sgu, sdn, ps16 = torch.rand(28672, device=dev), torch.rand(4096, device=dev), torch.rand(16, device=dev)
+    flush.fill_(4)
+    torch.cuda.synchronize()
+    pa.npu_quant_matmul(xq1, wgu.t(), sgu, pertoken_scale=ps16, output_dtype=torch.bfloat16)
+    pa.npu_quant_matmul(xq2, wdn.t(), sdn, pertoken_scale=ps16, output_dtype=torch.bfloat16)
     torch.cuda.synchronize()
     print(json.dumps({"pmc_pass": "done"}))
 
@@ -483,6 +493,29 @@ def main():
                        "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                                     "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None}})
         del xs, wsn, keep
+
+    if want("qd"):
+        # W8A8 projections of a Llama-3-8B-shaped layer at decode batch sizes (weights [N,K], rotated so that none is
+        # cache-resident): the decode kernel of quant_matmul
+        for (Kx, Nx) in ((4096, 6144), (4096, 4096), (4096, 28672), (14336, 4096)):
+            nset = _nsets(Kx * Nx)
+            wsn = [torch.randint(-128, 128, (Nx, Kx), generator=gen, dtype=torch.int8, device=dev).t() for _ in range(nset)]
+            sc = torch.rand(Nx, generator=gen, device=dev) * 1e-2
+            for Mx in (1, 16):
+                xs = [torch.randint(-128, 128, (Mx, Kx), generator=gen, dtype=torch.int8, device=dev) for _ in range(nset)]
+                ps = torch.rand(Mx, generator=gen, device=dev) * 1e-2
+                keep = []
+                calls = [(lambda a=a, w=w: keep.append(pa.npu_quant_matmul(a, w, sc, pertoken_scale=ps, output_dtype=torch.bfloat16)))
+                         for a, w in zip(xs, wsn)] * 2
+                us = _graph_time_us(torch, calls, reps=10)
+                nb = Kx * Nx + Mx * Kx + Mx * Nx * 2 + Nx * 4 + Mx * 4
+                others.append({"name": f"quant_matmul decode int8[{Mx},{Kx}] . int8 stored [{Nx},{Kx}] -> bf16", "launch_us": round(us, 3),
+                               "roofline": {"bound": "hbm", "achieved": round(nb / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                                            "unit": "GB/s", "frac": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                                            "traffic": _traffic(f"qd_{Kx}x{Nx}_m{Mx}")},
+                               "algorithmic_bytes": int(nb)})
+                del xs, keep
+            del wsn
 
     if want("a4w4"):
         # both operands packed int4 (A4W4) at the headline shape: the operator widens them to int8 and runs the int8 GEMM
