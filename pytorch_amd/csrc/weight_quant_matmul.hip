@@ -36,6 +36,7 @@
 // (to occupy all CUs when there are few strips) each workgroup writes its float32 partial to the
 // workspace and the workgroup that arrives last at a per-tile counter adds them in chunk order,
 // which keeps the result independent of scheduling.
+#include "weight_quant_kmajor_decode.h"
 #include "weight_quant_common.h"
 #include "weight_quant_gemm.h"
 #include "weight_quant_kpacked.h"
@@ -372,13 +373,14 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
     // staging: 16-byte piece q of a row's chunk (8 consecutive k) belongs to step q/16, sub-step t and lane group g with
     // q % 16 = 8 * (t / 2) + 2 * g + (t % 2); it goes to fragment (step, m tile, t) at lane (g, row % 16)
     constexpr int XR = (MT * 16 + 7) / 8;          // rows per wavefront
-    u32x4 xst[XR][2];
+    constexpr int XH = CH * 16 / 64;               // a row's chunk is CH * 16 pieces, 64 per load instruction
+    u32x4 xst[XR][XH];
     auto stage_load = [&](int ch) {
 #pragma unroll
         for (int i = 0; i < XR; i++) {
             const int r = wave + 8 * i;
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
+            for (int h = 0; h < XH; h++) {
                 const int q = lane + 64 * h;
                 const int st = ch * CH + (q >> 4);
                 const bool ok = r < rows_valid && st < nsteps;
@@ -395,7 +397,7 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
             const int r = wave + 8 * i;
             if (r >= MT * 16) continue;
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
+            for (int h = 0; h < XH; h++) {
                 const int q = lane + 64 * h;
                 const int sl = q >> 4, rr = q & 15;
                 const int t = 2 * (rr >> 3) + (rr & 1), gg = (rr & 7) >> 1;
@@ -690,6 +692,7 @@ WqKmPlan make_kmajor_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, i
         if (f >= 1 && f <= pl.n_units) S = f;
     if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1;
     if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterCapacity) S = 1;
+    if (wq_kmajor_decode_shape(M, N, K, group_size)) S = 1;   // the decode kernel splits K inside its workgroups
     pl.S = S;
     pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
     pl.counter_bytes = S > 1 ? kWorkspaceZeroBytes : 0;
@@ -901,6 +904,24 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
         const WqKmPlan km = make_kmajor_plan(M, N, K, group_size, ldw_n, ldx, x_bf16, w);
         const bool params_ok = aligned(scale_bf16, 2) && (!offset_bf16 || aligned(offset_bf16, 2));
         if (km.fast && params_ok) {
+            if (wq_kmajor_decode_shape(M, N, K, group_size)) {
+                // at most 32 rows, one scale per column: the barrier-free kernel that splits K inside the workgroup
+                WqKmDecodeArgs d;
+                d.x = static_cast<const uint16_t *>(x_bf16);
+                d.w = static_cast<const int8_t *>(w);
+                d.scale = static_cast<const uint16_t *>(scale_bf16);
+                d.offset = static_cast<const uint16_t *>(offset_bf16);
+                d.bias = static_cast<const uint16_t *>(bias);
+                d.out = static_cast<uint16_t *>(out_bf16);
+                d.ldx = ldx;
+                d.ldw = ldw_n;
+                d.ldo = ldo;
+                d.M = (int)M;
+                d.N = (int)N;
+                d.K = (int)K;
+                const int st = launch_wq_kmajor_decode(d, f16 ? 1 : 0, s);
+                if (st != MI355_ERR_UNSUPPORTED) return st;
+            }
             if (km.S > 1) {
                 if (!workspace || workspace_bytes < km.partial_bytes + km.counter_bytes) return MI355_ERR_WORKSPACE;
                 if (!aligned(workspace, 16)) return MI355_ERR_ALIGNMENT;

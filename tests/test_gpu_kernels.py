@@ -390,6 +390,38 @@ def test_w8a16_kmajor_and_no_offset(capi, golden):
     bf16_gate(out, _wq_golden(golden, d2, 0))
 
 
+@pytest.mark.parametrize("M,K,N,f16", [(1, 4096, 4096, False), (16, 8192, 2048, False), (7, 1152, 2052, True), (16, 2176, 4104, False),
+                                       (17, 4096, 2048, False), (32, 3072, 6144, True), (3, 1024, 8200, False)])
+def test_w8a16_kmajor_decode_kernel(capi, golden, M, K, N, f16):
+    """int8 weight stored [N, K], one scale per column, at most 32 rows: the kernel that splits K over the wavefronts of a
+    workgroup and walks over strips of 16 columns (one and two tiles of 16 rows, 1 to 8 steps per wavefront, even and
+    uneven, strips that end past N, more strips than workgroups; both activation types; with and without offset and bias;
+    pitched activations).  No workspace; within the gate of the oracle, and of the tiled K-major kernel's own result."""
+    d = workloads.w8a16_inputs(seed=M + K + N, M=M, K=K, N=N, weight_nk=True)
+    g = torch.Generator().manual_seed(N)
+    dt = torch.float16 if f16 else torch.bfloat16
+    bits = _f16_bits if f16 else _bits
+    x, sc, of = d["x"].to(dt), d["antiquant_scale"].to(dt), d["antiquant_offset"].to(dt)
+    bias = torch.randn(N, generator=g).to(dt)
+    w = d["weight"]
+    assert capi.lib().mi355_weight_quant_matmul_workspace(M, N, K, 8, 0) >= 0
+    for use_of, use_bias in ((True, True), (False, False), (True, False)):
+        out = capi.weight_quant_matmul(x.cuda(), w.cuda(), sc.cuda(), of.cuda() if use_of else None, 0, bias.cuda() if use_bias else None)
+        _, want = golden.weight_quant_matmul(bits(x), w.numpy(), bits(sc), bits(of) if use_of else None, group_size=0,
+                                             bias_u16=bits(bias) if use_bias else None, dtype="fp16" if f16 else "bf16")
+        bf16_gate(out, torch.from_numpy(want), floor=out.numel() < 8192)
+    wide = torch.zeros(M, K + 64, dtype=dt, device="cuda")
+    wide[:, :K] = x.cuda()
+    ref = capi.weight_quant_matmul(x.cuda(), w.cuda(), sc.cuda(), of.cuda(), 0, bias.cuda())
+    assert torch.equal(capi.weight_quant_matmul(wide[:, :K], w.cuda(), sc.cuda(), of.cuda(), 0, bias.cuda()), ref)
+    capi.set_tuning("MI355_WQ_DECODE_OFF", 1)
+    try:
+        tiled = capi.weight_quant_matmul(x.cuda(), w.cuda(), sc.cuda(), of.cuda(), 0, bias.cuda())
+    finally:
+        capi.set_tuning("MI355_WQ_DECODE_OFF", 0)
+    bf16_gate(ref, tiled.float().cpu(), floor=ref.numel() < 8192)
+
+
 @pytest.mark.parametrize("M,K,N", [(5, 256, 130), (5, 256, 132), (32, 512, 6), (3, 128, 1)])
 def test_w8a16_kmajor_ragged_columns(capi, golden, M, K, N):
     """int8 weight stored [N, K] with N not a multiple of 4 (or of 8): the K-major streaming kernel stores quads of
