@@ -321,6 +321,26 @@ def test_quant_matmul_split_k_repeated_launches(capi, golden):
         assert np.array_equal(_bits(out), want)
 
 
+@pytest.mark.parametrize("M,K,N", [(512, 14336, 4096), (1024, 14336, 4096), (256, 8192, 8192), (128, 4096, 28672), (304, 5120, 1000)])
+def test_quant_matmul_long_k_plans(capi, M, K, N):
+    """Shapes on which the planner picks large tiles with a split of K (256x256 four ways, 128x256 four ways and two ways):
+    accumulators against an exact float64 evaluation on the GPU (products and partial sums of 4096 terms are exact in
+    float64), outputs against the same formula in separately rounded float32 tensor operations."""
+    g = torch.Generator(device="cuda").manual_seed(M + K + N)
+    x = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8, device="cuda")
+    w = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8, device="cuda")
+    ps = torch.rand(M, device="cuda", generator=g) * 1e-2
+    sc = torch.rand(N, device="cuda", generator=g) * 1e-2
+    bias = torch.randn(N, device="cuda", generator=g).to(torch.bfloat16)
+    acc = torch.zeros(M, N, dtype=torch.float64, device="cuda")
+    for k0 in range(0, K, 4096):
+        acc += x[:, k0:k0 + 4096].double() @ w[:, k0:k0 + 4096].double().t()
+    acc = acc.to(torch.int64).to(torch.int32)
+    assert torch.equal(capi.quant_matmul(x, w.t(), None, out_dtype=torch.int32), acc)
+    want = (((acc.float() * ps[:, None]) * sc[None, :]) + bias.float()[None, :]).to(torch.bfloat16)
+    assert torch.equal(capi.quant_matmul(x, w.t(), sc, ps, bias).view(torch.int16), want.view(torch.int16))
+
+
 QMM_DECODE_CASES = [(1, 4096, 4096), (7, 1024, 2048), (16, 1152, 2056), (5, 14336, 4096), (3, 11008, 2048), (16, 16384, 2048),
                     (1, 1024, 8200), (17, 4096, 6144), (32, 8192, 2048), (30, 2176, 4100), (33, 4096, 4104), (64, 2048, 5120),
                     (48, 1024, 16384)]
