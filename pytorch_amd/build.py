@@ -17,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 KERNEL_LIB = os.path.join(CSRC, "libmi355_quant.so")
 OPS_LIB = os.path.join(CSRC, "libmi355_npu_ops.so")
-KERNEL_SOURCES = ["dynamic_quant.hip", "dynamic_quant_asym.hip", "quant_matmul.hip", "quant_matmul_decode.hip", "weight_quant_matmul.hip", "weight_quant_gemm.hip", "weight_quant_kpacked.hip", "weight_quant_kmajor_decode.hip", "weight_quant_decode.hip", "weight_quant_gemm4.hip", "weight_quant_repack.hip", "swiglu.hip", "anti_quant.hip", "unpack_int4.hip", "quantize.hip", "tuning.hip", "device_probe.hip"]
+KERNEL_SOURCES = ["dynamic_quant.hip", "dynamic_quant_asym.hip", "quant_matmul.hip", "quant_matmul_decode.hip", "weight_quant_matmul.hip", "weight_quant_gemm.hip", "weight_quant_kpacked.hip", "weight_quant_kpacked_decode.hip", "weight_quant_kmajor_decode.hip", "weight_quant_decode.hip", "weight_quant_gemm4.hip", "weight_quant_repack.hip", "swiglu.hip", "anti_quant.hip", "unpack_int4.hip", "quantize.hip", "tuning.hip", "device_probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -ffp-contract=off: the dequantising epilogues must round every operation separately.

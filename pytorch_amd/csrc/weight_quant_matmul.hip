@@ -40,6 +40,7 @@
 #include "weight_quant_common.h"
 #include "weight_quant_gemm.h"
 #include "weight_quant_kpacked.h"
+#include "weight_quant_kpacked_decode.h"
 #include "weight_quant_decode.h"
 #include "weight_quant_gemm4.h"
 #include "weight_quant_repack.h"
@@ -877,6 +878,26 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
             if (!g4.ok) return MI355_ERR_LAUNCH;       // planned with these strides a few lines up
             return launch_wq_gemm4(g4, x_bf16, f16 ? 1 : 0, w_kn, 4, scale_gn, offset_gn, bias, out_bf16, M, N, K, group_size, ldx, pitch,
                                    ldo, workspace, stream);
+        }
+        if (wq_kpacked_decode_shape(M, N, K, group_size) && ldw_n < (1ll << 29)) {
+            // at most 16 rows, groups of 128: the barrier-free kernel that splits K inside the workgroup
+            WqKpDecodeArgs d;
+            d.x = static_cast<const uint16_t *>(x_bf16);
+            d.w = w;
+            d.scale = static_cast<const uint16_t *>(scale_bf16);
+            d.offset = static_cast<const uint16_t *>(offset_bf16);
+            d.bias = static_cast<const uint16_t *>(bias);
+            d.out = static_cast<uint16_t *>(out_bf16);
+            d.ldx = ldx;
+            d.ldo = ldo;
+            d.ld_param_g = ld_param_g;
+            d.ld_param_n = ld_param_n;
+            d.ldw_bytes = (uint32_t)(ldw_n * 4);
+            d.M = (int)M;
+            d.N = (int)N;
+            d.K = (int)K;
+            const int st = launch_wq_kpacked_decode(d, f16 ? 1 : 0, static_cast<hipStream_t>(stream));
+            if (st != MI355_ERR_UNSUPPORTED) return st;
         }
         const WqKpackedPlan kp = make_wq_kpacked_plan(M, N, K, group_size, ldw_n, ldx, x_bf16, w);
         const bool ptrs_ok = aligned(scale_bf16, 2) && (!offset_bf16 || aligned(offset_bf16, 2)) && aligned(out_bf16, 2) &&
