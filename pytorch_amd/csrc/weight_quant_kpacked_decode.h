@@ -1,5 +1,5 @@
 // Internal interface of the decode-shaped kernel for int4 weights packed along K (storage [N, K/8]) with scale groups of
-// 128 (at most 16 activation rows); not part of the C ABI.
+// 128 (at most 32 activation rows); not part of the C ABI.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stddef.h>

@@ -1,6 +1,6 @@
 // npu_weight_quant_batchmatmul for decode-sized batches of int4 weights packed along K (storage [N, K/8] int32, the
 // layout torch_npu's LinearWeightQuant passes as a transposed view, torch_npu/contrib/module/linear_weight_quant.py:71,106)
-// with scale groups of 128, at most 16 activation rows.
+// with scale groups of 128, at most 32 activation rows.
 //
 // The structure is that of the other decode kernels (quant_matmul_decode.hip, weight_quant_kmajor_decode.hip): a
 // workgroup of eight wavefronts owns strips of weight rows (= output columns) over the whole of K, wavefront w the w-th
@@ -56,13 +56,13 @@ __device__ __forceinline__ u32x4 even_odd(u32x4 v)
     return r;
 }
 
-// NS steps per wavefront and column tile, NT column tiles of 16 per strip (NS * NT steps per strip, four in flight);
-// ACT 0 bf16, 1 fp16.  One tile of 16 activation rows.
-template <int NS, int NT, int ACT>
+// MT tiles of 16 activation rows; NS steps per wavefront and column tile, NT column tiles of 16 per strip (NS * NT steps
+// per strip), PF steps in flight; ACT 0 bf16, 1 fp16.
+template <int MT, int NS, int NT, int PF, int ACT>
 __global__ __launch_bounds__(512) void wq_kpacked_decode_kernel(const WqKpDecodeArgs p)
 {
-    constexpr int PF = 4, FS = NS * NT;                                   // flat steps per strip
-    static_assert(FS % PF == 0, "static ring slots and LDS buffer parities");
+    constexpr int FS = NS * NT;                                           // flat steps per strip
+    static_assert(FS % PF == 0 && PF % 2 == 0, "static ring slots and LDS buffer parities");
     constexpr int NG = 2 * NS;                                            // scale groups of a wavefront
     static_assert(NG == 4 || NG == 8, "parameters travel in lane groups of four");
     constexpr float P_MUL = kImageMul<4, ACT>, X_BIAS = kImageBias<4>;
@@ -96,17 +96,19 @@ __global__ __launch_bounds__(512) void wq_kpacked_decode_kernel(const WqKpDecode
     // The wavefront's slice of the activations, once: a step is 16 rows x 512 bytes; an instruction loads two whole rows
     // (lane l: 16 bytes of row 2 i + l / 32), the step goes through LDS, and lane (c, g) reads for MFMA d of half h the
     // 8 k at 128 h + 32 g + 8 d of row c, even elements first.
-    u32x4 xf[NS][2][4];
-    f32x4 Xg[NS][2];
+    u32x4 xf[NS][MT][2][4];
+    f32x4 Xg[NS][MT][2];
     const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
     {
         char *xb = shared + wave * 8192;
 #pragma unroll
-        for (int j = 0; j < NS; j++) {
+        for (int j = 0; j < NS; j++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
             u32x4 xl[8];
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const int row = 2 * i + (lane >> 5);
+                const int row = mt * 16 + 2 * i + (lane >> 5);
                 xl[i] = __builtin_amdgcn_raw_buffer_load_b128(
                     rsrc_x, j < ns && row < p.M ? (uint32_t)((row * (int)p.ldx) * 2 + (lane & 31) * 16) : kOutOfRange,
                     (uint32_t)(s0 + j) * (4 * kStep), 0);
@@ -115,11 +117,11 @@ __global__ __launch_bounds__(512) void wq_kpacked_decode_kernel(const WqKpDecode
             for (int i = 0; i < 8; i++) *reinterpret_cast<u32x4 *>(xb + i * 1024 + lane * 16) = xl[i];
 #pragma unroll
             for (int h = 0; h < 2; h++) {
-                Xg[j][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+                Xg[j][mt][h] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
-                    xf[j][h][d] = even_odd(*reinterpret_cast<const u32x4 *>(xb + c * 512 + (16 * h + 4 * g + d) * 16));
-                    Xg[j][h] = mfma_act<ACT>(xf[j][h][d], ones, Xg[j][h]);
+                    xf[j][mt][h][d] = even_odd(*reinterpret_cast<const u32x4 *>(xb + c * 512 + (16 * h + 4 * g + d) * 16));
+                    Xg[j][mt][h] = mfma_act<ACT>(xf[j][mt][h][d], ones, Xg[j][mt][h]);
                 }
             }
         }
@@ -160,9 +162,12 @@ __global__ __launch_bounds__(512) void wq_kpacked_decode_kernel(const WqKpDecode
     uint32_t prm_next[NT][NG / 4];
     load_params(0, prm_next);
 
-    // wavefront f < NT finishes column tile f of every strip: lane l writes row l / 4, columns 4 (l % 4) .. + 3
-    const bool finisher = wave < NT;
+    // wavefront f < NT * MT finishes tile (column tile f / MT, row tile f % MT) of every strip: lane l writes row l / 4,
+    // columns 4 (l % 4) .. + 3
+    const bool finisher = wave < NT * MT;
+    const int fnt = wave / MT, fmt = wave % MT;
     const int er = lane >> 2, ec = (lane & 3) * 4;
+    const int em = fmt * 16 + er;
     const int e_idx = (16 * (er >> 2)) * 4 + (er & 3);                    // accumulator element (row, column 0) of a tile
 
     __syncthreads();                                                      // every wavefront is done with its activation tile
@@ -174,14 +179,17 @@ __global__ __launch_bounds__(512) void wq_kpacked_decode_kernel(const WqKpDecode
 #pragma unroll
             for (int r = 0; r < NG / 4; r++) prm[nt][r] = prm_next[nt][r];
         load_params(t + 1, prm_next);
-        const int en = (((int)blockIdx.x + t * (int)gridDim.x) * NT + wave) * 16 + ec;
+        const int en = (((int)blockIdx.x + t * (int)gridDim.x) * NT + fnt) * 16 + ec;
         const u32x2 bq = __builtin_amdgcn_raw_buffer_load_b64(rsrc_bias, finisher && en < p.N ? (uint32_t)en * 2u : kOutOfRange, 0, 0);
 
-        f32x4 tot[NT];
+        f32x4 tot[NT][MT];
 #pragma unroll
         for (int f = 0; f < FS; f++) {
             const int nt = f / NS, j = f % NS;
-            if (j == 0) tot[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (j == 0) {
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) tot[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
             const char *src = tb + (f & 1) * 2048;
             const u32x4 w0 = *reinterpret_cast<const u32x4 *>(src + t_rd) ^ 0x88888888u;          // nibbles u = w + 8
             const u32x4 w1 = *reinterpret_cast<const u32x4 *>(src + (t_rd ^ 64)) ^ 0x88888888u;
@@ -191,29 +199,39 @@ __global__ __launch_bounds__(512) void wq_kpacked_decode_kernel(const WqKpDecode
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int h = 0; h < 2; h++) {
-                f32x4 P = f32x4{0.f, 0.f, 0.f, 0.f};
+                f32x4 P[MT];
 #pragma unroll
-                for (int d = 0; d < 4; d++) P = mfma_act<ACT>(xf[j][h][d], expand_word<ACT>(h ? w1[d] : w0[d]), P);
+                for (int mt = 0; mt < MT; mt++) P[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    const u32x4 b = expand_word<ACT>(h ? w1[d] : w0[d]);
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) P[mt] = mfma_act<ACT>(xf[j][mt][h][d], b, P[mt]);
+                }
                 const int gl = 2 * j + h;                                 // group of this half among the wavefront's
                 const uint32_t pr = (uint32_t)__builtin_amdgcn_ds_bpermute((c + 16 * (gl & 3)) * 4, (int)prm[nt][gl >> 2]);
                 const float sc = act_lo<ACT>(pr) * P_MUL;
                 const float of = ((p.offset ? act_hi<ACT>(pr) : 0.0f) - X_BIAS) * (1.0f / P_MUL);
 #pragma unroll
-                for (int q = 0; q < 4; q++) tot[nt][q] = __builtin_fmaf(sc, __builtin_fmaf(of, Xg[j][h][q], P[q]), tot[nt][q]);
+                for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) tot[nt][mt][q] = __builtin_fmaf(sc, __builtin_fmaf(of, Xg[j][mt][h][q], P[mt][q]), tot[nt][mt][q]);
             }
         }
 
-        float *const rd = red + (t & 1) * (8 * NT * 256);
+        float *const rd = red + (t & 1) * (8 * NT * MT * 256);
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) *reinterpret_cast<f32x4 *>(rd + ((wave * NT + nt) * 64 + lane) * 4) = tot[nt];
+        for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) *reinterpret_cast<f32x4 *>(rd + (((wave * NT + nt) * MT + mt) * 64 + lane) * 4) = tot[nt][mt];
         __syncthreads();
         if (finisher) {
             float sum[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int w = 0; w < 8; w++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) sum[i] += rd[(w * NT + wave) * 256 + e_idx + 4 * (ec + i)];
-            if (er < p.M && en < p.N) {
+                for (int i = 0; i < 4; i++) sum[i] += rd[(w * NT * MT + wave) * 256 + e_idx + 4 * (ec + i)];
+            if (em < p.M && en < p.N) {
                 if (p.bias) {
 #pragma unroll
                     for (int i = 0; i < 4; i++) sum[i] = sum[i] + ((i & 1) ? act_hi<ACT>(bq[i >> 1]) : act_lo<ACT>(bq[i >> 1]));
@@ -221,18 +239,18 @@ __global__ __launch_bounds__(512) void wq_kpacked_decode_kernel(const WqKpDecode
                 u32x2 pk;
                 pk.x = pack_act2<ACT>(sum[0], sum[1]);
                 pk.y = pack_act2<ACT>(sum[2], sum[3]);
-                *reinterpret_cast<u32x2 *>(p.out + (int64_t)er * p.ldo + en) = pk;
+                *reinterpret_cast<u32x2 *>(p.out + (int64_t)em * p.ldo + en) = pk;
             }
         }
     }
 }
 
-template <int NS, int NT, int ACT>
+template <int MT, int NS, int NT, int PF, int ACT>
 int launch(const WqKpDecodeArgs &p, hipStream_t s)
 {
     constexpr int lds_bytes = 8 * 4096 + 8 * 8192;                        // weight tiles, activation tiles (later: the sums)
-    static_assert(2 * 8 * NT * 1024 <= 8 * 8192, "the sums fit where the activation tiles were");
-    auto kern = wq_kpacked_decode_kernel<NS, NT, ACT>;
+    static_assert(2 * 8 * NT * MT * 1024 <= 8 * 8192, "the sums fit where the activation tiles were");
+    auto kern = wq_kpacked_decode_kernel<MT, NS, NT, PF, ACT>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
     const int strips = (p.N + 16 * NT - 1) / (16 * NT);
@@ -244,7 +262,8 @@ template <int ACT>
 int launch_act(const WqKpDecodeArgs &p, hipStream_t s)
 {
     const int ns = (p.K / (2 * kStep) + 7) / 8;
-    return ns <= 2 ? launch<2, 2, ACT>(p, s) : launch<4, 1, ACT>(p, s);
+    if (p.M > 16) return launch<2, 2, 1, 2, ACT>(p, s);
+    return ns <= 2 ? launch<1, 2, 2, 4, ACT>(p, s) : launch<1, 4, 1, 4, ACT>(p, s);
 }
 
 } // namespace
@@ -253,9 +272,10 @@ bool wq_kpacked_decode_shape(int64_t M, int64_t N, int64_t K, int64_t group_size
 {
     if (knob(kKnobWqDecodeOff) == 1 || knob(kKnobWqSplit) != 0) return false;
     if (group_size != 128) return false;
-    if (M < 1 || M > 16 || K % (2 * kStep) != 0 || K < 8 * 2 * kStep || N < 2048 || N % 4 != 0) return false;
-    // the activations of a wavefront's eighth of K stay in registers: at most four steps of 256 k
-    return (K / (2 * kStep) + 7) / 8 <= 4;
+    if (M < 1 || M > 32 || K % (2 * kStep) != 0 || K < 8 * 2 * kStep || N < 2048 || N % 4 != 0) return false;
+    // the activations of a wavefront's eighth of K stay in registers: at most four steps of 256 k with one tile of 16
+    // rows, two with two
+    return (K / (2 * kStep) + 7) / 8 <= (M <= 16 ? 4 : 2);
 }
 
 int launch_wq_kpacked_decode(const WqKpDecodeArgs &p, int act_f16, hipStream_t s)

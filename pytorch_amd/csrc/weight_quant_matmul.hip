@@ -880,7 +880,7 @@ extern "C" int mi355_weight_quant_matmul(const void *x_bf16, int act_dtype, cons
                                    ldo, workspace, stream);
         }
         if (wq_kpacked_decode_shape(M, N, K, group_size) && ldw_n < (1ll << 29)) {
-            // at most 16 rows, groups of 128: the barrier-free kernel that splits K inside the workgroup
+            // at most 32 rows, groups of 128: the barrier-free kernel that splits K inside the workgroup
             WqKpDecodeArgs d;
             d.x = static_cast<const uint16_t *>(x_bf16);
             d.w = w;

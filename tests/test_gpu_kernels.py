@@ -709,12 +709,14 @@ KPACKED_CASES = [
     (3, 2048, 4096, 0, False, False, True),         # per channel, 1-D parameters
     (70, 14336, 4096, 128, False, True, False),     # long K: K is split between workgroups, 112 groups
     (16, 256, 16, 128, True, True, False),          # a single step, a single wavefront's worth of columns
-    # at most 16 rows, groups of 128, at least 2048 columns and k: the decode kernel (weight_quant_kpacked_decode.hip), as
+    # at most 32 rows, groups of 128, at least 2048 columns and k: the decode kernel (weight_quant_kpacked_decode.hip), as
     # are the first two cases above
     (16, 2048, 2048, 128, True, True, True),        # one step per wavefront of the two the kernel is built for
     (9, 5120, 2056, 128, False, False, True),       # two or three steps per wavefront, a strip that ends past N
     (4, 8192, 4096, 128, False, True, False),       # four steps per wavefront, one column tile per strip
     (16, 3072, 8224, 128, True, True, True),        # more strips than workgroups, uneven steps, fp16
+    (17, 4096, 2048, 128, False, True, True),       # two tiles of rows (at most two steps per wavefront)
+    (32, 3072, 4104, 128, True, False, False),      # the same, uneven steps, a strip that ends past N, fp16
     # from 256 rows up the weight is rewritten per call with its words along N (weight_quant_repack.hip)
     (256, 512, 1000, 128, False, True, True),       # ragged columns: 125 words per row, the last tile partly valid
     (300, 1024, 520, 256, True, True, False),       # ragged rows, groups of two stages, fp16
