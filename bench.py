@@ -171,6 +171,11 @@ def _pmc_pass(torch, pa, workloads, dev):
     torch.cuda.synchronize()
     pa.npu_weight_quant_batchmatmul(g4["x"], wk.t(), s4t, o4t, None, None, None, 128)
     pa.npu_quant_matmul(xa4, wa.t(), g["scale"], pertoken_scale=g["pertoken_scale"], output_dtype=torch.bfloat16)
+    # configuration 3 with the weight stored [N, K] (the contrib module's layout), on a weight no kernel has touched
+    w3nk = torch.randint(-127, 128, (28672, 8192), dtype=torch.int8, device=dev)
+    flush.fill_(5)
+    torch.cuda.synchronize()
+    pa.npu_weight_quant_batchmatmul(g3["x"], w3nk.t(), g3["antiquant_scale"], g3["antiquant_offset"])
     # the decode kernel of quant_matmul: the two projections of the MLP at 16 rows, weights no kernel has touched
     wgu = torch.randint(-128, 128, (28672, 4096), dtype=torch.int8, device=dev)
     wdn = torch.randint(-128, 128, (4096, 14336), dtype=torch.int8, device=dev)
@@ -429,13 +434,16 @@ def main():
         wq_gate(e, d3, pa.npu_weight_quant_batchmatmul(x, ws[0], s3, o3), 0, 2.0 * Mx * Kx * Nx)
         others.append(e)
         del ws, keep
-        # the layout torch_npu's LinearWeightQuant passes: weight stored [N, K], given as its transposed view
-        ws = [torch.randint(-127, 128, (Nx, Kx), generator=gen, dtype=torch.int8, device=dev).t() for _ in range(2)]
+        # the layout torch_npu's LinearWeightQuant passes (linear_weight_quant.py:71,106): weight stored [N, K], given as its
+        # transposed view; set 0 holds the seeded values the oracle checks
+        ws = [d3["weight"].t().contiguous().to(dev).t()] + [torch.randint(-127, 128, (Nx, Kx), generator=gen, dtype=torch.int8, device=dev).t()]
         keep = []
         calls = [(lambda w=w: keep.append(pa.npu_weight_quant_batchmatmul(x, w, s3, o3))) for w in ws] * 4
         us = _graph_time_us(torch, calls, reps=10)
-        others.append(hbm_entry("c3 W8A16 x bf16[16,8192] . int8[8192,28672] (weight stored [N,K], transposed view)", nb, us,
-                                None, tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2)))
+        e = hbm_entry("c3 W8A16 x bf16[16,8192] . int8[8192,28672] (weight stored [N,K] and passed as its transposed view: the contrib module's layout)",
+                      nb, us, _traffic("c3_nk"), tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2))
+        wq_gate(e, d3, pa.npu_weight_quant_batchmatmul(x, ws[0], s3, o3), 0, 2.0 * Mx * Kx * Nx)
+        others.append(e)
         del ws, keep
 
     if want("c4"):
