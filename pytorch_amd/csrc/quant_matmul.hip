@@ -820,7 +820,7 @@ struct QmmPlan {
 // itself).
 constexpr double kBaseUs = 6.0, kL2BytesPerUs = 12e6, kExchangeUs = 1.0, kExchangeBytesPerUs = 12e6, kCollectorBytesPerUs = 100e3;
 
-void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, TileChoice *tile, int *split)
+void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size_t partial_cap, TileChoice *tile, int *split)
 {
     const int forced_tile = knob(kKnobQmmTile);             // debugging aids: bm * 1000 + bn, and the split
     const int forced_split = knob(kKnobQmmSplit);
@@ -839,6 +839,8 @@ void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, Tile
             }
             const int s_eff = forced_split >= 1 && forced_split <= kt && may_split ? forced_split : S;
             const int64_t wgs = tiles * s_eff;
+            // a caller with a fixed scratch area (mi355_quant_matmul_noalloc) only gets splits whose partial sums fit it
+            if (s_eff > 1 && s_eff == S && (uint64_t)wgs * c.bm * c.bn * 4 > partial_cap) continue;
             const int64_t rounds = (wgs + c.slots - 1) / c.slots;
             const double at_4096 = rounds == 1 ? c.single_us : (double)rounds * c.round_us;
             double cost = kBaseUs + (at_4096 - kBaseUs) * ((double)kt / s_eff) / 32.0;
@@ -858,19 +860,21 @@ void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, Tile
 
 // `zero_area`: bytes in front of the scratch part of the workspace (the shared zero area, or just the counters when the
 // workspace is private to this operator)
-QmmPlan make_qmm_plan(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n, size_t zero_area = kWorkspaceZeroBytes)
+QmmPlan make_qmm_plan(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n, size_t zero_area = kWorkspaceZeroBytes,
+                      size_t scratch_cap = ~(size_t)0)
 {
     QmmPlan pl{};
     const bool tiled_shape = K >= BK && K % BK == 0;
     // the decode kernel splits K inside its workgroups (it is not used while a tile or a split is forced)
     const bool decode = qmm_decode_shape(M, N, K) && knob(kKnobQmmSplit) == 0 && knob(kKnobQmmTile) == 0;
-    choose_tile_and_split(M, N, K, tiled_shape && !decode, &pl.tile, &pl.S);
+    // a contiguous [K,N] weight is transposed into the workspace
+    pl.transpose_bytes = tiled_shape && ldb_k != 1 && ldb_n == 1 ? (size_t)N * (size_t)K : 0;
+    const size_t fixed = zero_area + pl.transpose_bytes;
+    choose_tile_and_split(M, N, K, tiled_shape && !decode, scratch_cap > fixed ? scratch_cap - fixed : 0, &pl.tile, &pl.S);
     if (tiled_shape && pl.S > 1) {
         const int64_t tiles = ((M + pl.tile.bm - 1) / pl.tile.bm) * ((N + pl.tile.bn - 1) / pl.tile.bn);
         pl.partial_bytes = (size_t)tiles * pl.S * pl.tile.bm * pl.tile.bn * 4;   // tiles <= 128 counters
     }
-    // a contiguous [K,N] weight is transposed into the workspace
-    pl.transpose_bytes = tiled_shape && ldb_k != 1 && ldb_n == 1 ? (size_t)N * (size_t)K : 0;
     pl.counter_bytes = pl.partial_bytes + pl.transpose_bytes > 0 ? zero_area : 0;
     return pl;
 }
@@ -908,7 +912,8 @@ __global__ __launch_bounds__(256) void trans_quant_param_kernel(const float *__r
 int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale, const uint64_t *qparam,
                      int64_t scale_len, const void *bias, int bias_dtype, void *out, int out_dtype, int64_t M,
                      int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
-                     void *workspace, size_t workspace_bytes, void *stream, size_t zero_area = kWorkspaceZeroBytes)
+                     void *workspace, size_t workspace_bytes, void *stream, size_t zero_area = kWorkspaceZeroBytes,
+                     size_t scratch_cap = ~(size_t)0)
 {
     if (M < 0 || N < 0 || K < 0) return MI355_ERR_BAD_ARGUMENT;
     if (out_dtype != MI355_OUT_BF16 && out_dtype != MI355_OUT_INT32 && out_dtype != MI355_OUT_FP16 && out_dtype != MI355_OUT_INT8)
@@ -936,7 +941,7 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     const bool offsets_fit = (uint64_t)256 * (uint64_t)lda + (uint64_t)K < (1ull << 31) &&
                              (uint64_t)256 * (uint64_t)(ldb_k != 1 ? K : ldb_n) + (uint64_t)K < (1ull << 31);
     bool tiled = K >= BK && K % BK == 0 && (lda & 15) == 0 && aligned(a, 16) && offsets_fit;
-    const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n, zero_area);
+    const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n, zero_area, scratch_cap);
     char *ws = static_cast<char *>(workspace);
     if (tiled && pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes > 0) {
         if (!ws || workspace_bytes < pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes) return MI355_ERR_WORKSPACE;
@@ -1129,7 +1134,7 @@ extern "C" int mi355_quant_matmul_noalloc(const int8_t *a, const int8_t *b, cons
         return run_quant_matmul(a, b, pertoken_scale, scale, nullptr, scale_len, bias, bias_dtype, out, out_dtype, M, N, K, lda,
                                 ldb_k, ldb_n, ldc, nullptr, 0, stream);
     // the scratch array is private to this operator: the arrival counters are followed directly by the partial sums
-    const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n, kWorkspaceCounterCapacity);
+    const QmmPlan pl = make_qmm_plan(M, N, K, ldb_k, ldb_n, kWorkspaceCounterCapacity, kStaticScratchBytes);
     const size_t need = pl.counter_bytes + pl.partial_bytes + pl.transpose_bytes;
     if (need > kStaticScratchBytes) return MI355_ERR_WORKSPACE;      // beyond the fixed scratch: use mi355_quant_matmul
     void *ws = nullptr;
@@ -1138,7 +1143,7 @@ extern "C" int mi355_quant_matmul_noalloc(const int8_t *a, const int8_t *b, cons
         if (st != MI355_OK) return st;
     }
     return run_quant_matmul(a, b, pertoken_scale, scale, nullptr, scale_len, bias, bias_dtype, out, out_dtype, M, N, K, lda,
-                            ldb_k, ldb_n, ldc, ws, need > 0 ? kStaticScratchBytes : 0, stream, kWorkspaceCounterCapacity);
+                            ldb_k, ldb_n, ldc, ws, need > 0 ? kStaticScratchBytes : 0, stream, kWorkspaceCounterCapacity, kStaticScratchBytes);
 }
 
 // One-time weight pre-layout for npu_quant_matmul: a contiguous [K,N] int8 weight is rewritten K-major ([N,K] storage),

@@ -60,6 +60,23 @@ def test_quant_matmul_noalloc_matches_workspace_entry_point():
         assert _call(L, True, x1, x2, scale, ps, bias, got) == 0
         torch.cuda.synchronize()
         assert torch.equal(got, want)
+    # a shape whose preferred plan (large tiles, K split four ways: 64 MiB of partial sums) does not fit the scratch: the
+    # entry point plans within its scratch instead of refusing, and integer sums make the result the same bit for bit
+    M, K, N = 1024, 14336, 4096
+    x1 = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).cuda()
+    x2 = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).cuda().t()
+    scale = (torch.rand(N, generator=g) * 9e-3 + 1e-3).cuda()
+    ps = (torch.rand(M, generator=g) * 9e-3 + 1e-3).cuda()
+    bias = (torch.randn(N, generator=g) * 0.02).to(torch.bfloat16).cuda()
+    need = L.mi355_quant_matmul_workspace(M, N, K, x2.stride(0), x2.stride(1))
+    assert need > (32 << 20) + 16384, need
+    ws = torch.zeros(need, dtype=torch.int8, device="cuda")
+    want = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    got = torch.full((M, N), 3.0, dtype=torch.bfloat16, device="cuda")
+    assert _call(L, False, x1, x2, scale, ps, bias, want, ws) == 0
+    assert _call(L, True, x1, x2, scale, ps, bias, got) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
     # a request beyond the fixed scratch is refused with the workspace status, nothing is launched
     M, K, N = 16, 8192, 8192                          # [K,N] weight: 64 MiB transposed copy
     x1 = torch.zeros((M, K), dtype=torch.int8, device="cuda")
