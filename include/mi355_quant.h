@@ -176,9 +176,9 @@ int mi355_transpose_int8(const int8_t *src, int8_t *dst, int64_t K, int64_t N, i
  * The arrival counters, split-K partial sums and the transposed copy of a contiguous [K,N] weight live in a fixed
  * device array of MI355_NOALLOC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.
  *   - the array is private to this operator, so it holds only 16 KiB of counters plus what the problem needs behind
- *     them: returns MI355_ERR_WORKSPACE when mi355_quant_matmul_workspace(M, N, K, ldb_k, ldb_n) minus the 16 MiB
- *     exchange zone of the shared workspaces exceeds that size (for example a large weight stored [K,N]: store it
- *     [N,K], or use mi355_quant_matmul);
+ *     them.  A split of K is planned so that its partial sums fit (mi355_quant_matmul may prefer a split with more of
+ *     them; integer sums make the results identical); returns MI355_ERR_WORKSPACE when the transposed copy of a
+ *     weight stored [K,N] does not fit (store it [N,K], or use mi355_quant_matmul);
  *   - calls no hipMalloc / hipFree and no allocating library routine; the first call on a device resolves the
  *     array's address and clears its counters with a small kernel on `stream`;
  *   - all calls on one GPU share that GPU's array: calls that may overlap in time (different streams without an
