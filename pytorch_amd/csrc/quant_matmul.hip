@@ -818,6 +818,7 @@ struct QmmPlan {
 // Constants fitted to sweeps over tile x split on M = 128 .. 2048, K = 8192 .. 28672 (the estimate's choice is the
 // measured best on nine of ten shapes and 16 % off on the tenth; at K = 4096 without a split the estimate is the table
 // itself).
+constexpr size_t kMaxPartialBytes = (size_t)128 << 20;
 constexpr double kBaseUs = 6.0, kL2BytesPerUs = 12e6, kExchangeUs = 1.0, kExchangeBytesPerUs = 12e6, kCollectorBytesPerUs = 100e3;
 
 void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size_t partial_cap, TileChoice *tile, int *split)
@@ -840,7 +841,8 @@ void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size
             const int s_eff = forced_split >= 1 && forced_split <= kt && may_split ? forced_split : S;
             const int64_t wgs = tiles * s_eff;
             // a caller with a fixed scratch area (mi355_quant_matmul_noalloc) only gets splits whose partial sums fit it
-            if (s_eff > 1 && s_eff == S && (uint64_t)wgs * c.bm * c.bn * 4 > partial_cap) continue;
+            // ... and nobody gets more than 128 MiB of them
+            if (s_eff > 1 && s_eff == S && (uint64_t)wgs * c.bm * c.bn * 4 > (partial_cap < kMaxPartialBytes ? partial_cap : kMaxPartialBytes)) continue;
             const int64_t rounds = (wgs + c.slots - 1) / c.slots;
             const double at_4096 = rounds == 1 ? c.single_us : (double)rounds * c.round_us;
             double cost = kBaseUs + (at_4096 - kBaseUs) * ((double)kt / s_eff) / 32.0;
