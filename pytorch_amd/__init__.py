@@ -43,4 +43,4 @@ _export_npu_ops()
 
 from . import contrib  # noqa: E402,F401
 from . import flops  # noqa: E402,F401  (registers the FLOP formulas of the matmul operators)
-from .prepare import prepare_quant_matmul_weight  # noqa: E402,F401
+from .prepare import prepare_quant_matmul_weight, prepare_weight_quant_weight  # noqa: E402,F401

@@ -6,7 +6,7 @@ import torch
 
 from . import _capi
 
-__all__ = ["prepare_quant_matmul_weight"]
+__all__ = ["prepare_quant_matmul_weight", "prepare_weight_quant_weight"]
 
 
 def prepare_quant_matmul_weight(x2: torch.Tensor) -> torch.Tensor:
@@ -26,3 +26,21 @@ def prepare_quant_matmul_weight(x2: torch.Tensor) -> torch.Tensor:
     out = torch.stack([_capi.transpose_int8(flat[b]) for b in range(flat.shape[0])]) if flat.shape[0] != 1 else \
         _capi.transpose_int8(flat[0]).unsqueeze(0)
     return out.reshape(*x2.shape[:-2], N, K).transpose(-1, -2)
+
+
+def prepare_weight_quant_weight(weight: torch.Tensor) -> torch.Tensor:
+    """Return a tensor equal to the int8 ``weight`` (logical ``[K, N]``) of ``npu_weight_quant_batchmatmul`` whose storage
+    is ``[N, K]`` contiguous (strides ``(1, K)``): the layout ``LinearWeightQuant`` keeps and passes as a transposed view
+    (torch_npu/contrib/module/linear_weight_quant.py:71,106).  With at most 32 activation rows and one scale per column
+    that layout takes the decode kernel that splits K inside a workgroup (configuration 3: 41-45 us against 48-50 for a
+    weight contiguous along N).  Weights already stored that way, and int32 words of int4 values, are returned
+    unchanged."""
+    if weight.dim() != 2:
+        raise ValueError(f"prepare_weight_quant_weight expects a two-dimensional weight, got {tuple(weight.shape)}")
+    if weight.dtype != torch.int8:
+        return weight
+    K, N = weight.shape
+    if weight.stride(0) == 1 and weight.stride(1) == K:
+        return weight
+    src = weight if weight.stride(1) == 1 else weight.contiguous()
+    return _capi.transpose_int8(src).t()

@@ -596,3 +596,21 @@ def test_c5_mlp_prefill_properties(pa, golden):
     sub["x"] = d["x"][rows]
     part = _mlp_gpu(pa, sub)[-1]
     assert torch.equal(full[rows.cuda()], part)
+
+
+def test_prepare_weight_quant_weight(pa):
+    """An int8 weight contiguous along N is rewritten once into the contrib module's storage ([N, K], passed as its
+    transposed view): equal values, strides (1, K), the operator's result within the gate of the unprepared call's;
+    weights already stored that way and int4 words come back unchanged."""
+    from pytorch_amd.testing import workloads, bf16_gate
+    d = workloads.w8a16_inputs(seed=5, M=16, K=4096, N=2304)
+    w = d["weight"].cuda()
+    wp = pa.prepare_weight_quant_weight(w)
+    assert wp.shape == w.shape and wp.stride() == (1, 4096) and torch.equal(wp, w)
+    assert pa.prepare_weight_quant_weight(wp) is wp
+    words = torch.zeros(64, 8, dtype=torch.int32, device="cuda")
+    assert pa.prepare_weight_quant_weight(words) is words
+    x, sc, of = d["x"].cuda(), d["antiquant_scale"].cuda(), d["antiquant_offset"].cuda()
+    ref = pa.npu_weight_quant_batchmatmul(x, w, sc, of)
+    out = pa.npu_weight_quant_batchmatmul(x, wp, sc, of)
+    bf16_gate(out, ref.float().cpu())
