@@ -517,7 +517,13 @@ def main():
                          for a, w in zip(xs, wsn)] * 2
                 us = _graph_time_us(torch, calls, reps=10)
                 nb = Kx * Nx + Mx * Kx + Mx * Nx * 2 + Nx * 4 + Mx * 4
-                others.append({"name": f"quant_matmul decode int8[{Mx},{Kx}] . int8 stored [{Nx},{Kx}] -> bf16", "launch_us": round(us, 3),
+                gate = {}
+                if not args.skip_cpu and Mx == 16:
+                    from oracle import golden
+                    gold, _ = golden.quant_matmul(xs[0].cpu().numpy(), wsn[0].cpu().numpy(), sc.cpu().numpy(), ps.cpu().numpy())
+                    got = pa.npu_quant_matmul(xs[0], wsn[0], sc, pertoken_scale=ps, output_dtype=torch.bfloat16)
+                    gate = {"parity_bit_exact": bool(np.array_equal(_bits(got), gold))}
+                others.append({"name": f"quant_matmul decode int8[{Mx},{Kx}] . int8 stored [{Nx},{Kx}] -> bf16", "launch_us": round(us, 3), **gate,
                                "roofline": {"bound": "hbm", "achieved": round(nb / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
                                             "unit": "GB/s", "frac": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                                             "traffic": _traffic(f"qd_{Kx}x{Nx}_m{Mx}")},
