@@ -381,6 +381,25 @@ def test_quant_matmul_decode_kernel(capi, golden, M, K, N):
         capi.set_tuning("MI355_QMM_DECODE_OFF", 0)
 
 
+@pytest.mark.parametrize("M,K,N,pad", [(8, 1024, 2049, 0), (16, 4096, 2054, 0), (5, 2048, 4096, 8), (64, 4096, 2049, 0)])
+def test_quant_matmul_decode_shapes_that_fall_back(capi, M, K, N, pad):
+    """Decode-sized problems the decode kernel declines (N not a multiple of 4, activation rows whose pitch is not a
+    multiple of 16, a scale pointer that is not 16-byte aligned): the planner has already dropped the K split for them,
+    and the kernels behind give the same bits as the formula in float32 tensor operations."""
+    g = torch.Generator(device="cuda").manual_seed(M + N)
+    xw = torch.randint(-128, 128, (M, K + pad), generator=g, dtype=torch.int8, device="cuda")
+    x = xw[:, :K]
+    w = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8, device="cuda")
+    ps = torch.rand(M, device="cuda", generator=g) * 1e-2
+    sc = torch.rand(N + 1, device="cuda", generator=g) * 1e-2
+    bias = torch.randn(N, device="cuda", generator=g).to(torch.bfloat16)
+    acc = (x.double() @ w.double().t()).to(torch.int64).to(torch.int32)
+    for scale in (sc[:N], sc[1:]):
+        want = (((acc.float() * ps[:, None]) * scale[None, :]) + bias.float()[None, :]).to(torch.bfloat16)
+        out = capi.quant_matmul(x, w.t(), scale, ps, bias)
+        assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
 # ------------------------------------------------------------------ weight-quant matmul
 
 def _wq_golden(golden, d, group):
