@@ -845,7 +845,11 @@ void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size
             if (s_eff > 1 && s_eff == S && (uint64_t)wgs * c.bm * c.bn * 4 > (partial_cap < kMaxPartialBytes ? partial_cap : kMaxPartialBytes)) continue;
             const int64_t rounds = (wgs + c.slots - 1) / c.slots;
             const double at_4096 = rounds == 1 ? c.single_us : (double)rounds * c.round_us;
-            double cost = kBaseUs + (at_4096 - kBaseUs) * ((double)kt / s_eff) / 32.0;
+            double loop_us = (at_4096 - kBaseUs) * ((double)kt / s_eff) / 32.0;
+            // tiles that run two to a CU: with more than 256 and fewer than 512 workgroups the CUs that hold two set the
+            // time, as if all did (128x128 split six ways, 384 workgroups: 42 us where eight ways, 512, take 38)
+            if (c.slots == 512 && rounds == 1 && wgs > 256) loop_us *= 512.0 / (double)wgs;
+            double cost = kBaseUs + loop_us;
             const double l2 = kBaseUs + (double)tiles * (c.bm + c.bn) * (double)K / kL2BytesPerUs;
             if (l2 > cost) cost = l2;
             if (s_eff > 1)
