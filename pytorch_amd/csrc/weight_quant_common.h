@@ -73,8 +73,13 @@ template <int ACT>
 constexpr uint32_t kInt4Magic = ACT == 0 ? 0x41004100u : 0x4c004c00u;
 template <int WBITS, int ACT>
 constexpr float kImageMul = (WBITS == 4 && ACT == 0) ? 2.0f : 1.0f;    // weight = kImageMul * image - kImageBias
+// int8 image: the weight itself (every integer up to 256 is a bf16 / fp16 number).  Byte i of a word is converted with its
+// sign in one instruction (v_cvt_f32_i32 with a sign-extending byte select), so no bias has to be removed afterwards: an
+// image w + 128 made the sum of products 128 X + sum(x w) and its float32 rounding, 2^-24 of 128 X, the error floor of
+// small outputs.
 template <int WBITS>
-constexpr float kImageBias = WBITS == 4 ? 24.0f : 128.0f;
+constexpr float kImageBias = WBITS == 4 ? 24.0f : 0.0f;
+__device__ __forceinline__ float sbyte_f32(uint32_t w, int i) { return (float)(int8_t)((w >> (8 * i)) & 0xffu); }
 
 template <int WBITS, int ACT>
 __device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint32_t magic, u32x4 &b0, u32x4 &b1)
@@ -97,9 +102,8 @@ __device__ __forceinline__ void expand_pair(const uint32_t (&w)[8], int jb, uint
         (void)magic;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            b0[v] = pack_act2<ACT>((float)((w[2 * v] >> (16 * jb)) & 0xffu), (float)((w[2 * v + 1] >> (16 * jb)) & 0xffu));
-            b1[v] = pack_act2<ACT>((float)((w[2 * v] >> (16 * jb + 8)) & 0xffu),
-                                (float)((w[2 * v + 1] >> (16 * jb + 8)) & 0xffu));
+            b0[v] = pack_act2<ACT>(sbyte_f32(w[2 * v], 2 * jb), sbyte_f32(w[2 * v + 1], 2 * jb));
+            b1[v] = pack_act2<ACT>(sbyte_f32(w[2 * v], 2 * jb + 1), sbyte_f32(w[2 * v + 1], 2 * jb + 1));
         }
     }
 }

@@ -142,10 +142,10 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
     };
     uint32_t magic;
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "n"(kInt4Magic<ACT>));   // opaque to the optimiser: stays in a VGPR
-    // two's complement -> offset binary (w + 128 / nibble + 8), then the 16-bit images -> LDS
+    // int4: two's complement -> offset binary (nibble + 8); then the 16-bit images -> LDS
     auto flip_w = [&](uint32_t (&wx)[8], const uint32_t (&wr)[8]) {
 #pragma unroll
-        for (int t = 0; t < (KM ? 4 : 8); t++) wx[t] = wr[t] ^ (KM ? 0x80808080u : WBITS == 4 ? 0x8888u : 0x8080u);
+        for (int t = 0; t < (KM ? 4 : 8); t++) wx[t] = wr[t] ^ (WBITS == 4 ? 0x8888u : 0u);   // int8 converts signed
     };
     // registers -> LDS, one piece: column n, k octet o -> chunk slot o ^ ((n >> 1) & 7) of row n
     auto expand_piece = [&](const uint32_t (&wx)[8], int piece, int s) {
@@ -155,10 +155,10 @@ __global__ __launch_bounds__(512, 1) void wq_gemm_kernel(const WqGemmArgs p)
             const int n = c >> 3, o = c & 7;
             const uint32_t lo = wx[2 * piece], hi = wx[2 * piece + 1];
             u32x4 b;
-            b[0] = pack_act2<ACT>((float)(lo & 0xffu), (float)((lo >> 8) & 0xffu));
-            b[1] = pack_act2<ACT>((float)((lo >> 16) & 0xffu), (float)(lo >> 24));
-            b[2] = pack_act2<ACT>((float)(hi & 0xffu), (float)((hi >> 8) & 0xffu));
-            b[3] = pack_act2<ACT>((float)((hi >> 16) & 0xffu), (float)(hi >> 24));
+            b[0] = pack_act2<ACT>(sbyte_f32(lo, 0), sbyte_f32(lo, 1));
+            b[1] = pack_act2<ACT>(sbyte_f32(lo, 2), sbyte_f32(lo, 3));
+            b[2] = pack_act2<ACT>(sbyte_f32(hi, 0), sbyte_f32(hi, 1));
+            b[3] = pack_act2<ACT>(sbyte_f32(hi, 2), sbyte_f32(hi, 3));
             *reinterpret_cast<u32x4 *>(bs + n * PITCH + ((o ^ ((n >> 1) & 7)) * 16)) = b;
         } else {
             u32x4 b0, b1;

@@ -224,10 +224,10 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         if constexpr (WBITS == 8) {
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const uint32_t wa = w[2 * v] ^ 0x80808080u, wb = w[2 * v + 1] ^ 0x80808080u;
+                const uint32_t wa = w[2 * v], wb = w[2 * v + 1];
 #pragma unroll
                 for (int nb = 0; nb < 4; nb++)
-                    bn[nb][v] = pack_act2<ACT>((float)((wa >> (8 * nb)) & 0xffu), (float)((wb >> (8 * nb)) & 0xffu));
+                    bn[nb][v] = pack_act2<ACT>(sbyte_f32(wa, nb), sbyte_f32(wb, nb));
             }
             return;
         }

@@ -11,9 +11,9 @@
 // a strip meet in LDS (two areas in turn, one barrier per strip) and the first wavefronts write it out while the others go
 // on.  No split of K over workgroups, no workspace, no barrier in front of the data.
 //
-// Arithmetic as in the other weight-only kernels: the MFMA multiplies the activations by the exact bf16 / fp16 image
-// w + 128 of the integer weight, and  out = scale * (P + (offset - 128) * X) + bias  in float32 with P the sum of products
-// and X the sum of the row's activations (formed once per launch: it does not depend on the strip), then one rounding.
+// Arithmetic as in the other weight-only kernels: the MFMA multiplies the activations by the integer weight, which is an
+// exact bf16 / fp16 number, and  out = scale * (P + offset * X) + bias  in float32 with P the sum of products and X the
+// sum of the row's activations (formed once per launch: it does not depend on the strip), then one rounding.
 #include "weight_quant_common.h"
 #include "weight_quant_kmajor_decode.h"
 
@@ -134,8 +134,8 @@ __global__ __launch_bounds__(512) void wq_kmajor_decode_kernel(const WqKmDecodeA
 #pragma unroll
         for (int j = 0; j < NS; j++) {
             const char *src = tb + (j & 1) * 2048;
-            const u32x4 w0 = *reinterpret_cast<const u32x4 *>(src + t_rd) ^ 0x80808080u;          // w + 128 as unsigned bytes
-            const u32x4 w1 = *reinterpret_cast<const u32x4 *>(src + (t_rd ^ 64)) ^ 0x80808080u;
+            const u32x4 w0 = *reinterpret_cast<const u32x4 *>(src + t_rd);
+            const u32x4 w1 = *reinterpret_cast<const u32x4 *>(src + (t_rd ^ 64));
             to_lds_w((j + 1) % PF, (j + 1) & 1);                          // the next step's registers take the other buffer
             __builtin_amdgcn_sched_barrier(0);
             load_w(j % PF, t + (j + PF) / NS, (j + PF) % NS);             // this step's registers are free again
@@ -144,10 +144,10 @@ __global__ __launch_bounds__(512) void wq_kmajor_decode_kernel(const WqKmDecodeA
             for (int q = 0; q < 4; q++) {
                 const uint32_t lo = q < 2 ? w0[2 * (q & 1)] : w1[2 * (q & 1)], hi = q < 2 ? w0[2 * (q & 1) + 1] : w1[2 * (q & 1) + 1];
                 u32x4 b;
-                b[0] = pack_act2<ACT>((float)(lo & 0xffu), (float)((lo >> 8) & 0xffu));
-                b[1] = pack_act2<ACT>((float)((lo >> 16) & 0xffu), (float)(lo >> 24));
-                b[2] = pack_act2<ACT>((float)(hi & 0xffu), (float)((hi >> 8) & 0xffu));
-                b[3] = pack_act2<ACT>((float)((hi >> 16) & 0xffu), (float)(hi >> 24));
+                b[0] = pack_act2<ACT>(sbyte_f32(lo, 0), sbyte_f32(lo, 1));
+                b[1] = pack_act2<ACT>(sbyte_f32(lo, 2), sbyte_f32(lo, 3));
+                b[2] = pack_act2<ACT>(sbyte_f32(hi, 0), sbyte_f32(hi, 1));
+                b[3] = pack_act2<ACT>(sbyte_f32(hi, 2), sbyte_f32(hi, 3));
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) P[mt] = mfma_act<ACT>(xf[j][mt][q], b, P[mt]);
             }
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(512) void wq_kmajor_decode_kernel(const WqKmDecodeA
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float sc = (i & 1) ? act_hi<ACT>(scq[i >> 1]) : act_lo<ACT>(scq[i >> 1]);
-                    const float of = (p.offset ? ((i & 1) ? act_hi<ACT>(ofq[i >> 1]) : act_lo<ACT>(ofq[i >> 1])) : 0.0f) - 128.0f;
+                    const float of = p.offset ? ((i & 1) ? act_hi<ACT>(ofq[i >> 1]) : act_lo<ACT>(ofq[i >> 1])) : 0.0f;
                     float v = sc * __builtin_fmaf(of, xtot, sum[i]);
                     if (p.bias) v = v + ((i & 1) ? act_hi<ACT>(bq[i >> 1]) : act_lo<ACT>(bq[i >> 1]));
                     f[i] = v;

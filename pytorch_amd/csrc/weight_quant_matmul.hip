@@ -12,8 +12,8 @@
 // (X_g comes from one extra MFMA against a vector of ones).
 //
 // Weight images (chosen so the expansion is a few bit operations per pair of weights):
-//   int8 : u = w ^ 0x80 = w + 128 in [0,255], converted with v_cvt_f32_ubyteN and packed to
-//          bf16 (exact: 8 significant bits);  P = P' - 128 X.
+//   int8 : the weight itself, byte i of a word converted with its sign in one instruction (v_cvt_f32_i32 with a
+//          sign-extending byte select) and packed to bf16 (exact: 8 significant bits);  P = P'.
 //   int4 : nibble ^ 8 = w + 8 = u in [0,15] is placed in mantissa bits 3..6 of the bf16
 //          pattern 0x4100, i.e. the value 8 + u/2 = (w + 24) / 2;  P = 2 P' - 24 X.
 //
@@ -231,8 +231,8 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
             uint32_t w0[8], w1[8];
 #pragma unroll
             for (int t = 0; t < 8; t++) {
-                w0[t] = wq[slot][t].x ^ (WBITS == 4 ? 0x88888888u : 0x80808080u);
-                w1[t] = wq[slot][t].y ^ (WBITS == 4 ? 0x88888888u : 0x80808080u);
+                w0[t] = wq[slot][t].x ^ (WBITS == 4 ? 0x88888888u : 0u);      // int4: nibbles u = w + 8; int8 converts signed
+                w1[t] = wq[slot][t].y ^ (WBITS == 4 ? 0x88888888u : 0u);
             }
             u32x4 xa[MT];
 #pragma unroll
@@ -308,7 +308,7 @@ __global__ __launch_bounds__(W * KS * 64) void wq_stream_kernel(const WqArgs p)
 // (two 16-byte loads) and feeds four MFMAs with the 8-byte halves; the activation fragments are laid out to match.
 // Activations are staged through LDS in chunks of 8 steps, already in fragment order, double buffered: the loads of
 // the next chunk are issued at the top of a chunk, written to LDS at its end, one barrier per chunk.
-// Per group:  out = sum_g scale_g * (P'_g + (offset_g - 128) * X_g)  with the int8 image w + 128 (see the top of the file).
+// Per group:  out = sum_g scale_g * (P_g + offset_g * X_g)  with the weight as its own image (see the top of the file).
 template <int MT, bool GROUPED, int ACT>
 __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
 {
@@ -413,7 +413,7 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
     const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
     auto fold = [&](int grp) {
         const float sc = act_1<ACT>(p.scale[(int64_t)grp * p.N + pcol]);
-        const float of = (has_offset ? act_1<ACT>(p.offset[(int64_t)grp * p.N + pcol]) : 0.0f) - 128.0f;
+        const float of = has_offset ? act_1<ACT>(p.offset[(int64_t)grp * p.N + pcol]) : 0.0f;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
@@ -448,8 +448,8 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
             // this step's weights in operand order (written during the previous step), then the next step's
             // registers take their place in the other half of the tile
             const char *tr = tbuf + (j & 1) * TBUF + t_rd;
-            u32x4 w0 = *reinterpret_cast<const u32x4 *>(tr) ^ 0x80808080u;
-            u32x4 w1 = *reinterpret_cast<const u32x4 *>(tbuf + (j & 1) * TBUF + (t_rd ^ 64)) ^ 0x80808080u;
+            u32x4 w0 = *reinterpret_cast<const u32x4 *>(tr);
+            u32x4 w1 = *reinterpret_cast<const u32x4 *>(tbuf + (j & 1) * TBUF + (t_rd ^ 64));
             {
                 const int sn = ((j + 1) / BODY) & 1, jsn = (j + 1) % BODY;
                 char *tw = tbuf + ((j + 1) & 1) * TBUF + lane * 16;
@@ -465,10 +465,10 @@ __global__ __launch_bounds__(512) void wq_kmajor_kernel(const WqArgs p)
             for (int t = 0; t < 4; t++) {
                 const uint32_t lo = t < 2 ? w0[2 * (t & 1)] : w1[2 * (t & 1)], hi = t < 2 ? w0[2 * (t & 1) + 1] : w1[2 * (t & 1) + 1];
                 u32x4 b;
-                b[0] = pack_act2<ACT>((float)(lo & 0xffu), (float)((lo >> 8) & 0xffu));
-                b[1] = pack_act2<ACT>((float)((lo >> 16) & 0xffu), (float)(lo >> 24));
-                b[2] = pack_act2<ACT>((float)(hi & 0xffu), (float)((hi >> 8) & 0xffu));
-                b[3] = pack_act2<ACT>((float)((hi >> 16) & 0xffu), (float)(hi >> 24));
+                b[0] = pack_act2<ACT>(sbyte_f32(lo, 0), sbyte_f32(lo, 1));
+                b[1] = pack_act2<ACT>(sbyte_f32(lo, 2), sbyte_f32(lo, 3));
+                b[2] = pack_act2<ACT>(sbyte_f32(hi, 0), sbyte_f32(hi, 1));
+                b[3] = pack_act2<ACT>(sbyte_f32(hi, 2), sbyte_f32(hi, 3));
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) {
                     P[mt] = mfma_act<ACT>(xa[t][mt], b, P[mt]);

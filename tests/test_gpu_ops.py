@@ -614,3 +614,38 @@ def test_prepare_weight_quant_weight(pa):
     ref = pa.npu_weight_quant_batchmatmul(x, w, sc, of)
     out = pa.npu_weight_quant_batchmatmul(x, wp, sc, of)
     bf16_gate(out, ref.float().cpu())
+
+
+def test_linear_weight_quant_reference_test_shape(pa):
+    """test/contrib/test_linear_weight_quant.py:53-73 as it stands: m, k, n = 1024, 11264, 1664, float16 activations,
+    an int8 weight drawn as randn().to(int8) and kept [n, k] by the module, per-channel float16 scale and offset drawn
+    from randn().  Two goldens: the formula with float32 arithmetic for (w + offset) * scale, which is this build's
+    contract (compared the way assertRtolEqual compares float16 arrays, testcase.py:158-227: at most 0.1 % of the
+    elements off by more than 1e-3), and the test's own CPU formula (:20-28), which rounds the sum and the product to
+    float16 before the float32 matmul.  Against the latter the exact antiquantisation differs by a few 1e-4 of a
+    column's typical magnitude, which is more than 1e-3 of the smaller outputs: the comparison holds at the 0.01 the
+    reference's call names, not at the 1e-3 that assertRtolEqual applies to float16 arrays."""
+    from pytorch_amd.contrib.module import LinearWeightQuant
+    from pytorch_amd.testing.compare import rtol_failures
+    m, k, n = 1024, 11264, 1664
+    g = torch.Generator().manual_seed(0)
+    x_cpu = torch.randn((m, k), generator=g, dtype=torch.float32).to(torch.float16)
+    weight_cpu = torch.randn((n, k), generator=g, dtype=torch.float32).to(torch.float16).to(torch.int8).to(torch.float16)
+    scale_cpu = torch.randn((n,), generator=g, dtype=torch.float32).to(torch.float16)
+    offset_cpu = torch.randn((n,), generator=g, dtype=torch.float32).to(torch.float16)
+    model = LinearWeightQuant(k, n, bias=False, dtype=torch.float16, antiquant_offset=True, quant_scale=False, quant_offset=False,
+                              antiquant_group_size=0).cuda()
+    model.weight.data = weight_cpu.to(torch.int8).cuda()
+    model.antiquant_scale.data = scale_cpu.cuda()
+    model.antiquant_offset.data = offset_cpu.cuda()
+    out = model(x_cpu.cuda()).cpu()
+    assert out.dtype == torch.float16 and out.shape == (m, n)
+    w = weight_cpu.transpose(0, 1)
+    x32 = x_cpu.to(torch.float32)
+    exact = torch.matmul(x32, (w.float() + offset_cpu.float()) * scale_cpu.float()).numpy().astype("float16")
+    assert_rtol_equal(exact, out.numpy(), 0.01)                                  # float16 arrays: 1e-3, 0.1 % of the elements
+    rounded = torch.matmul(x32, ((w + offset_cpu) * scale_cpu).to(torch.float32)).numpy().astype("float16")
+    assert_rtol_equal(rounded, out.numpy(), 0.01, prec16=0.01)
+    frac = rtol_failures(rounded, out.numpy(), 1e-3) / out.numel()
+    print("reference shape: fraction beyond 1e-3 of the float16-rounded golden", round(frac, 4))
+    assert frac < 0.25
