@@ -54,7 +54,7 @@ constexpr int kMaxPolls4 = 1 << 20;
 // WBITS == 8: the same kernel for int8 weights [K, N].  A weight row of the tile is then 256 bytes (256 columns), a stage
 // 64 rows (two steps), and a wavefront owns one 128-byte half of the rows x one span of 16 dwords with all four bytes
 // of its dwords: again four column tiles per lane (columns 128 s2 + 64 h + 4 c .. + 3), expanded with a byte-to-float
-// conversion and a packing conversion per pair of weights (image u = w + 128).
+// conversion and a packing conversion per pair of weights (the weight is its own image, converted with its sign).
 template <int ACT, bool STAGE_GROUPS, int WBITS = 4>
 __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
 {
