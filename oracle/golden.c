@@ -370,6 +370,11 @@ void orc_antiquant(const int8_t *w, const float *scale, const float *offset,
  * wf[k,n]  = (float32(w[k,n]) + float32(off[g,n])) * float32(scale[g,n]),  g = k / group_size
  * (group_size 0 = per channel: g = 0).  Follows cpu_linear_weight_quant in
  * test/contrib/test_linear_weight_quant.py:20-28 with bf16 parameters and float32 arithmetic.
+ * That test evaluates w + offset and * scale in the tensors' own type (float16 there), i.e. it
+ * rounds the antiquantised weight twice before its float32 matmul; the benchmark's gate is stated
+ * against the float32 formula, which is what this function restates.  The difference between the
+ * two on the reference test's own data is measured by
+ * tests/test_gpu_ops.py::test_linear_weight_quant_reference_test_shape.
  *
  * w_bits 8: w is int8 addressed as w[k*ldw_k + n*ldw_n].
  * w_bits 4: w is int32 [K, N/8] row-major, packed as described at orc_unpack_int4.
