@@ -11,7 +11,8 @@ struct QmmDecodeArgs {
     const int8_t *a;           // [M, K], row pitch lda
     const int8_t *bt;          // [N, K], row pitch ldbt
     const float *pertoken;     // [M] or null
-    const float *scale;        // [scale_len]
+    const float *scale;        // [scale_len], or null when qparam is given
+    const uint64_t *qparam;    // [scale_len] packed quantisation parameters (bits 0-31: the float32 scale), or null
     const void *bias;          // [N] of bias_kind, or null
     int bias_kind;             // MI355_BIAS_*
     int out_f16;               // round to fp16 instead of bf16

@@ -49,7 +49,9 @@ __global__ __launch_bounds__(512) void qmm_decode_kernel(const QmmDecodeArgs p)
 
     const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(p.bt, (uint32_t)((int64_t)(p.N - 1) * p.ldbt + p.K));
     const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(p.a, (uint32_t)((int64_t)(p.M - 1) * p.lda + p.K));
-    const __amdgpu_buffer_rsrc_t rsrc_sc = make_rsrc(p.scale, (uint32_t)p.scale_len * 4u);
+    // per-channel factors: float32 words, or the low halves of 64-bit packed parameters
+    const uint32_t sc_elem = p.qparam ? 8u : 4u;
+    const __amdgpu_buffer_rsrc_t rsrc_sc = make_rsrc(p.qparam ? static_cast<const void *>(p.qparam) : static_cast<const void *>(p.scale), (uint32_t)p.scale_len * sc_elem);
     const uint32_t bias_elem = p.bias_kind == MI355_BIAS_BF16 ? 2u : 4u;
     const __amdgpu_buffer_rsrc_t rsrc_bias = make_rsrc(p.bias, p.bias ? (uint32_t)p.N * bias_elem : 0u);
     // lane l of half h loads row 8 h + l / 8, and the 16-byte piece that belongs in slot l % 8 of that row's swizzled
@@ -101,7 +103,7 @@ __global__ __launch_bounds__(512) void qmm_decode_kernel(const QmmDecodeArgs p)
     const bool finisher = wave < MT;
     const int em = wave * 16 + c;
     const float ps = p.pertoken && finisher ? p.pertoken[min(em, p.M - 1)] : 1.0f;
-    const float sc_one = p.scale_len == 1 ? p.scale[0] : 0.0f;
+    const float sc_one = p.scale_len != 1 ? 0.0f : p.qparam ? __uint_as_float((uint32_t)p.qparam[0]) : p.scale[0];
 
     // turn the activation fragments around (a wavefront's LDS operations complete in order)
 #pragma unroll
@@ -124,7 +126,12 @@ __global__ __launch_bounds__(512) void qmm_decode_kernel(const QmmDecodeArgs p)
         // dequantisation parameters of this strip, requested before its last weights are (wavefronts that finish no tile
         // get an out-of-range offset: no branch around loads)
         const uint32_t pn = finisher && en < p.N ? (uint32_t)en : kOutOfRange / 4;
-        const u32x4 scq = __builtin_amdgcn_raw_buffer_load_b128(rsrc_sc, p.scale_len == 1 ? kOutOfRange : pn * 4u, 0, 0);
+        const uint32_t sc_off = p.scale_len == 1 || pn >= kOutOfRange / 4 ? kOutOfRange : pn * sc_elem;
+        u32x4 scq = __builtin_amdgcn_raw_buffer_load_b128(rsrc_sc, sc_off, 0, 0);
+        if (p.qparam) {                                                   // columns 0, 1 | 2, 3: keep the low words
+            const u32x4 hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc_sc, sc_off == kOutOfRange ? kOutOfRange : sc_off + 16u, 0, 0);
+            scq = u32x4{scq[0], scq[2], hi[0], hi[2]};
+        }
         const u32x4 bq = __builtin_amdgcn_raw_buffer_load_b128(rsrc_bias, bias_elem == 4u ? pn * 4u : kOutOfRange, 0, 0);
         const u32x2 bh = __builtin_amdgcn_raw_buffer_load_b64(rsrc_bias, bias_elem == 2u ? pn * 2u : kOutOfRange, 0, 0);
 
@@ -209,7 +216,7 @@ int launch_qmm_decode(const QmmDecodeArgs &p, hipStream_t s)
     if ((p.lda & 15) != 0 || (p.ldbt & 15) != 0 || !aligned(p.a, 16) || !aligned(p.bt, 16) || p.ldbt < p.K)
         return MI355_ERR_UNSUPPORTED;
     // dequantisation parameters and results in pieces of four columns
-    if ((p.N & 3) != 0 || (p.ldc & 3) != 0 || !aligned(p.out, 8) || !aligned(p.scale, 16) ||
+    if ((p.N & 3) != 0 || (p.ldc & 3) != 0 || !aligned(p.out, 8) || !aligned(p.qparam ? static_cast<const void *>(p.qparam) : static_cast<const void *>(p.scale), 16) ||
         (p.bias && !aligned(p.bias, p.bias_kind == MI355_BIAS_BF16 ? 8 : 16)))
         return MI355_ERR_UNSUPPORTED;
     // 32-bit buffer offsets over the whole weight and all activation rows

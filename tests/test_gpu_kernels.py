@@ -374,6 +374,14 @@ def test_quant_matmul_decode_kernel(capi, golden, M, K, N):
     wide[:, :K] = x1
     ref = capi.quant_matmul(x1, x2, sc, ps, d["bias"].cuda())
     assert torch.equal(capi.quant_matmul(wide[:, :K], x2, sc, ps, d["bias"].cuda()), ref)
+    # the scale as packed 64-bit parameters (what LinearQuant hands over for a float16 output, linear_quant.py:104-108):
+    # the same bits as with the float32 scale, per channel and single
+    for scale in (sc, sc[:1].contiguous()):
+        qp = capi.trans_quant_param(scale)
+        for dt, name in ((torch.float16, "fp16"), (torch.bfloat16, "bf16")):
+            got = capi.quant_matmul_qparam(x1, x2, qp, bias_i32.cuda(), out_dtype=dt)
+            want = golden.quant_matmul_epilogue_ex(acc, scale.cpu().numpy(), None, bias_i32.numpy(), out=name)
+            assert np.array_equal(got.cpu().view(torch.int16).numpy().view(np.uint16), want), (name, scale.numel())
     capi.set_tuning("MI355_QMM_DECODE_OFF", 1)
     try:
         assert torch.equal(capi.quant_matmul(x1, x2, sc, ps, d["bias"].cuda()), ref)
