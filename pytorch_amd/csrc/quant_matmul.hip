@@ -966,7 +966,7 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
         ldbt = K;
     }
     tiled = tiled && (ldbt & 15) == 0 && aligned(bt, 16);
-    if (tiled && !out_i32 && !out_i8 && knob(kKnobQmmSplit) == 0 && knob(kKnobQmmTile) == 0) {
+    if (tiled && !out_i32 && knob(kKnobQmmSplit) == 0 && knob(kKnobQmmTile) == 0) {
         // at most 64 rows: the barrier-free kernel that splits K inside the workgroup (quant_matmul_decode.hip)
         QmmDecodeArgs d;
         d.a = a;
@@ -977,6 +977,7 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
         d.bias = bias;
         d.bias_kind = bias_dtype;
         d.out_f16 = out_dtype == MI355_OUT_FP16;
+        d.out_i8 = out_i8;
         d.out = out;
         d.lda = lda;
         d.ldbt = ldbt;

@@ -16,7 +16,8 @@ struct QmmDecodeArgs {
     const void *bias;          // [N] of bias_kind, or null
     int bias_kind;             // MI355_BIAS_*
     int out_f16;               // round to fp16 instead of bf16
-    void *out;                 // [M, N] 16-bit floats, row pitch ldc
+    int out_i8;                // re-quantise to int8 with the scale and offset of qparam (no pertoken, bias none or int32)
+    void *out;                 // [M, N] 16-bit floats or int8, row pitch ldc in elements
     int64_t lda, ldbt, ldc;
     int M, N, K;
     int scale_len;             // 1 or N

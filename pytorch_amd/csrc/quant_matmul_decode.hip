@@ -1,4 +1,4 @@
-// npu_quant_matmul for decode-sized batches on gfx950: int8 [M,K] x int8 weight stored [N,K], few rows, bf16 / fp16 output.
+// npu_quant_matmul for decode-sized batches on gfx950: int8 [M,K] x int8 weight stored [N,K], few rows; bf16, fp16 or re-quantised int8 output.
 //
 // With so few rows the operator is a stream of the weight from HBM, and what the tiled kernel spends around that stream
 // (an activation staging barrier before the first weight byte is used, a split of K over workgroups with partial sums and
@@ -17,7 +17,7 @@
 //   * dequantisation parameters are requested before the weights and wait in registers.
 // Integer accumulation makes the result independent of the split; the epilogue is the tiled kernel's, operation for
 // operation: ((float(acc + int32 bias) * pertoken[m]) * scale[n]) + bias[n], each operation rounded to float32, then one
-// rounding to the output type.
+// rounding to the output type; or clamp(rint((acc + int32 bias) * scale[n] + offset[n])) for an int8 output.
 #include "common.h"
 #include "quant_matmul_decode.h"
 
@@ -33,6 +33,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, ui
 {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
 }
+
+// The offset of a packed quantisation parameter, from its high word: bits 37-45 of the 64, a 9-bit two's-complement integer.
+__device__ __forceinline__ float qparam_hi_offset(uint32_t hi) { return (float)(((int32_t)((hi >> 5) << 23)) >> 23); }
 
 // MT tiles of 16 activation rows; NS (even) steps of 128 bytes of K per wavefront and strip, PF of them in flight.
 template <int MT, int NS, int PF>
@@ -117,6 +120,7 @@ __global__ __launch_bounds__(512) void qmm_decode_kernel(const QmmDecodeArgs p)
             for (int h = 0; h < 2; h++) xf[j][mt][h] = *reinterpret_cast<const i32x4v *>(xb + (t_rd ^ (64 * h)));
         }
 
+    const uint32_t of_one = p.scale_len == 1 && p.qparam ? (uint32_t)(p.qparam[0] >> 32) : 0u;
     const bool has_ps = p.pertoken != nullptr;
     const bool has_bias = p.bias_kind == MI355_BIAS_BF16 || p.bias_kind == MI355_BIAS_FP32;
     to_lds_w(0, 0);
@@ -128,8 +132,10 @@ __global__ __launch_bounds__(512) void qmm_decode_kernel(const QmmDecodeArgs p)
         const uint32_t pn = finisher && en < p.N ? (uint32_t)en : kOutOfRange / 4;
         const uint32_t sc_off = p.scale_len == 1 || pn >= kOutOfRange / 4 ? kOutOfRange : pn * sc_elem;
         u32x4 scq = __builtin_amdgcn_raw_buffer_load_b128(rsrc_sc, sc_off, 0, 0);
-        if (p.qparam) {                                                   // columns 0, 1 | 2, 3: keep the low words
+        u32x4 ofq = u32x4{0u, 0u, 0u, 0u};                                // the high words: the offset of an int8 output
+        if (p.qparam) {                                                   // columns 0, 1 | 2, 3: low words apart from high
             const u32x4 hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc_sc, sc_off == kOutOfRange ? kOutOfRange : sc_off + 16u, 0, 0);
+            ofq = u32x4{scq[1], scq[3], hi[1], hi[3]};
             scq = u32x4{scq[0], scq[2], hi[0], hi[2]};
         }
         const u32x4 bq = __builtin_amdgcn_raw_buffer_load_b128(rsrc_bias, bias_elem == 4u ? pn * 4u : kOutOfRange, 0, 0);
@@ -164,7 +170,20 @@ __global__ __launch_bounds__(512) void qmm_decode_kernel(const QmmDecodeArgs p)
             i32x4v sum = rd[wave * 64 + lane];
 #pragma unroll
             for (int w = 1; w < 8; w++) sum += rd[(w * MT + wave) * 64 + lane];
-            if (em < p.M && en < p.N) {
+            if (em < p.M && en < p.N && p.out_i8) {
+                // clamp(rint((sum + int32 bias) * scale + offset)): each operation rounded to float32
+                uint32_t w = 0;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int32_t bi = p.bias_kind == MI355_BIAS_INT32 ? (int32_t)bq[r] : 0;
+                    float v = (float)(int32_t)((uint32_t)sum[r] + (uint32_t)bi);
+                    v = v * (p.scale_len == 1 ? sc_one : __uint_as_float(scq[r]));
+                    v = v + qparam_hi_offset(p.scale_len == 1 ? of_one : ofq[r]);
+                    v = fminf(fmaxf(rintf(v), -128.0f), 127.0f);
+                    w |= ((uint32_t)(int32_t)v & 0xffu) << (8 * r);
+                }
+                *reinterpret_cast<uint32_t *>(static_cast<int8_t *>(p.out) + (int64_t)em * p.ldc + en) = w;
+            } else if (em < p.M && en < p.N) {
                 float f[4];
 #pragma unroll
                 for (int r = 0; r < 4; r++) {

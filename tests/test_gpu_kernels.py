@@ -152,15 +152,17 @@ def test_quant_matmul_bf16(capi, golden, M, K, N, bias):
     assert np.array_equal(_bits(out), want)      # same operation order => bit-identical bf16
 
 
-REQUANT_SHAPES = [(1024, 4096, 11008), (64, 4096, 1024), (48, 256, 192), (130, 384, 1000), (17, 100, 37), (256, 1024, 320)]
+REQUANT_SHAPES = [(1024, 4096, 11008), (64, 4096, 1024), (48, 256, 192), (130, 384, 1000), (17, 100, 37), (256, 1024, 320),
+                  (1, 4096, 4096), (16, 1152, 2056), (33, 2048, 4104), (5, 14336, 4096)]
 
 
 @pytest.mark.parametrize("M,K,N", REQUANT_SHAPES)
 @pytest.mark.parametrize("weight_nk", [True, False])
 def test_quant_matmul_int8_output(capi, golden, M, K, N, weight_nk):
     """The re-quantised int8 output through mi355_trans_quant_param + mi355_quant_matmul_qparam, bit-exact against the
-    oracle: tiled kernel (every tile shape these sizes select, split K at M=64), the generic kernel (K=100), with and
-    without an int32 bias, per-channel and single parameters, offsets that clamp and .5 ties."""
+    oracle: tiled kernel (every tile shape these sizes select, split K at M=64), the generic kernel (K=100), the decode
+    kernel (the last four shapes with the weight stored [N, K]), with and without an int32 bias, per-channel and single
+    parameters, offsets that clamp and .5 ties."""
     d = workloads.quant_matmul_inputs(seed=M + N, M=M, K=K, N=N, weight_nk=weight_nk)
     g = torch.Generator().manual_seed(K)
     acc_scale = 40.0 / (K ** 0.5 * 74 * 74)                       # spreads the results over the int8 range
