@@ -966,18 +966,19 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
         ldbt = K;
     }
     tiled = tiled && (ldbt & 15) == 0 && aligned(bt, 16);
-    if (tiled && !out_i32 && knob(kKnobQmmSplit) == 0 && knob(kKnobQmmTile) == 0) {
+    if (tiled && knob(kKnobQmmSplit) == 0 && knob(kKnobQmmTile) == 0) {
         // at most 64 rows: the barrier-free kernel that splits K inside the workgroup (quant_matmul_decode.hip)
         QmmDecodeArgs d;
         d.a = a;
         d.bt = bt;
-        d.pertoken = pertoken_scale;
-        d.scale = scale;
-        d.qparam = qparam;
+        d.pertoken = out_i32 ? nullptr : pertoken_scale;
+        d.scale = out_i32 ? nullptr : scale;             // an int32 output takes no scales: empty descriptors
+        d.qparam = out_i32 ? nullptr : qparam;
         d.bias = bias;
         d.bias_kind = bias_dtype;
         d.out_f16 = out_dtype == MI355_OUT_FP16;
         d.out_i8 = out_i8;
+        d.out_i32 = out_i32;
         d.out = out;
         d.lda = lda;
         d.ldbt = ldbt;
@@ -985,7 +986,7 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
         d.M = (int)M;
         d.N = (int)N;
         d.K = (int)K;
-        d.scale_len = (int)scale_len;
+        d.scale_len = out_i32 ? 0 : (int)scale_len;
         const int st = launch_qmm_decode(d, s);
         if (st != MI355_ERR_UNSUPPORTED) return st;
     }

@@ -11,13 +11,14 @@ struct QmmDecodeArgs {
     const int8_t *a;           // [M, K], row pitch lda
     const int8_t *bt;          // [N, K], row pitch ldbt
     const float *pertoken;     // [M] or null
-    const float *scale;        // [scale_len], or null when qparam is given
+    const float *scale;        // [scale_len], or null when qparam is given or the output is int32
     const uint64_t *qparam;    // [scale_len] packed quantisation parameters (bits 0-31: the float32 scale), or null
     const void *bias;          // [N] of bias_kind, or null
     int bias_kind;             // MI355_BIAS_*
     int out_f16;               // round to fp16 instead of bf16
     int out_i8;                // re-quantise to int8 with the scale and offset of qparam (no pertoken, bias none or int32)
-    void *out;                 // [M, N] 16-bit floats or int8, row pitch ldc in elements
+    int out_i32;               // the int32 accumulator (plus an int32 bias) itself: no scales
+    void *out;                 // [M, N] 16-bit floats, int8 or int32, row pitch ldc in elements
     int64_t lda, ldbt, ldc;
     int M, N, K;
     int scale_len;             // 1 or N

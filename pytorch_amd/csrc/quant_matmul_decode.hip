@@ -1,4 +1,4 @@
-// npu_quant_matmul for decode-sized batches on gfx950: int8 [M,K] x int8 weight stored [N,K], few rows; bf16, fp16 or re-quantised int8 output.
+// npu_quant_matmul for decode-sized batches on gfx950: int8 [M,K] x int8 weight stored [N,K], few rows; bf16, fp16, re-quantised int8 or int32 output.
 //
 // With so few rows the operator is a stream of the weight from HBM, and what the tiled kernel spends around that stream
 // (an activation staging barrier before the first weight byte is used, a split of K over workgroups with partial sums and
@@ -17,7 +17,7 @@
 //   * dequantisation parameters are requested before the weights and wait in registers.
 // Integer accumulation makes the result independent of the split; the epilogue is the tiled kernel's, operation for
 // operation: ((float(acc + int32 bias) * pertoken[m]) * scale[n]) + bias[n], each operation rounded to float32, then one
-// rounding to the output type; or clamp(rint((acc + int32 bias) * scale[n] + offset[n])) for an int8 output.
+// rounding to the output type; or clamp(rint((acc + int32 bias) * scale[n] + offset[n])) for an int8 output, acc + int32 bias for an int32 one.
 #include "common.h"
 #include "quant_matmul_decode.h"
 
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(512) void qmm_decode_kernel(const QmmDecodeArgs p)
     const bool finisher = wave < MT;
     const int em = wave * 16 + c;
     const float ps = p.pertoken && finisher ? p.pertoken[min(em, p.M - 1)] : 1.0f;
-    const float sc_one = p.scale_len != 1 ? 0.0f : p.qparam ? __uint_as_float((uint32_t)p.qparam[0]) : p.scale[0];
+    const float sc_one = p.scale_len != 1 ? 0.0f : p.qparam ? __uint_as_float((uint32_t)p.qparam[0]) : p.scale ? p.scale[0] : 0.0f;
 
     // turn the activation fragments around (a wavefront's LDS operations complete in order)
 #pragma unroll
@@ -170,7 +170,13 @@ __global__ __launch_bounds__(512) void qmm_decode_kernel(const QmmDecodeArgs p)
             i32x4v sum = rd[wave * 64 + lane];
 #pragma unroll
             for (int w = 1; w < 8; w++) sum += rd[(w * MT + wave) * 64 + lane];
-            if (em < p.M && en < p.N && p.out_i8) {
+            if (em < p.M && en < p.N && p.out_i32) {
+                i32x4v o = sum;                                           // the accumulator itself, plus an int32 bias
+                if (p.bias_kind == MI355_BIAS_INT32)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) o[r] = (int32_t)((uint32_t)sum[r] + bq[r]);
+                *reinterpret_cast<i32x4v *>(static_cast<int32_t *>(p.out) + (int64_t)em * p.ldc + en) = o;
+            } else if (em < p.M && en < p.N && p.out_i8) {
                 // clamp(rint((sum + int32 bias) * scale + offset)): each operation rounded to float32
                 uint32_t w = 0;
 #pragma unroll
@@ -235,7 +241,7 @@ int launch_qmm_decode(const QmmDecodeArgs &p, hipStream_t s)
     if ((p.lda & 15) != 0 || (p.ldbt & 15) != 0 || !aligned(p.a, 16) || !aligned(p.bt, 16) || p.ldbt < p.K)
         return MI355_ERR_UNSUPPORTED;
     // dequantisation parameters and results in pieces of four columns
-    if ((p.N & 3) != 0 || (p.ldc & 3) != 0 || !aligned(p.out, 8) || !aligned(p.qparam ? static_cast<const void *>(p.qparam) : static_cast<const void *>(p.scale), 16) ||
+    if ((p.N & 3) != 0 || (p.ldc & 3) != 0 || !aligned(p.out, p.out_i32 ? 16 : 8) || !aligned(p.qparam ? static_cast<const void *>(p.qparam) : static_cast<const void *>(p.scale), 16) ||
         (p.bias && !aligned(p.bias, p.bias_kind == MI355_BIAS_BF16 ? 8 : 16)))
         return MI355_ERR_UNSUPPORTED;
     // 32-bit buffer offsets over the whole weight and all activation rows

@@ -384,9 +384,15 @@ def test_quant_matmul_decode_kernel(capi, golden, M, K, N):
             got = capi.quant_matmul_qparam(x1, x2, qp, bias_i32.cuda(), out_dtype=dt)
             want = golden.quant_matmul_epilogue_ex(acc, scale.cpu().numpy(), None, bias_i32.numpy(), out=name)
             assert np.array_equal(got.cpu().view(torch.int16).numpy().view(np.uint16), want), (name, scale.numel())
+    # the int32 accumulator itself (LinearQuant with output_dtype=torch.int32), with and without the int32 bias; a scale
+    # passed along is ignored
+    assert np.array_equal(capi.quant_matmul(x1, x2, None, out_dtype=torch.int32).cpu().numpy(), acc)
+    got = capi.quant_matmul(x1, x2, sc, ps, bias_i32.cuda(), out_dtype=torch.int32)
+    assert np.array_equal(got.cpu().numpy(), (acc.astype(np.int64) + bias_i32.numpy().astype(np.int64)).astype(np.int32))
     capi.set_tuning("MI355_QMM_DECODE_OFF", 1)
     try:
         assert torch.equal(capi.quant_matmul(x1, x2, sc, ps, d["bias"].cuda()), ref)
+        assert torch.equal(capi.quant_matmul(x1, x2, sc, ps, bias_i32.cuda(), out_dtype=torch.int32), got)
     finally:
         capi.set_tuning("MI355_QMM_DECODE_OFF", 0)
 
