@@ -95,37 +95,20 @@ __global__ __launch_bounds__(512) void wq_kpacked_decode_kernel(const WqKpDecode
 
     // The wavefront's slice of the activations, once: a step is 16 rows x 512 bytes; an instruction loads two whole rows
     // (lane l: 16 bytes of row 2 i + l / 32), the step goes through LDS, and lane (c, g) reads for MFMA d of half h the
-    // 8 k at 128 h + 32 g + 8 d of row c, even elements first.
-    u32x4 xf[NS][MT][2][4];
-    f32x4 Xg[NS][MT][2];
-    const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
-    {
-        char *xb = shared + wave * 8192;
+    // 8 k at 128 h + 32 g + 8 d of row c, even elements first.  All of the loads are requested before the first weights,
+    // so one memory round trip covers both (the counter of outstanding loads runs in order).
+    u32x4 xl[NS][MT][8];
 #pragma unroll
-        for (int j = 0; j < NS; j++)
+    for (int j = 0; j < NS; j++)
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            u32x4 xl[8];
+        for (int mt = 0; mt < MT; mt++)
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 const int row = mt * 16 + 2 * i + (lane >> 5);
-                xl[i] = __builtin_amdgcn_raw_buffer_load_b128(
+                xl[j][mt][i] = __builtin_amdgcn_raw_buffer_load_b128(
                     rsrc_x, j < ns && row < p.M ? (uint32_t)((row * (int)p.ldx) * 2 + (lane & 31) * 16) : kOutOfRange,
                     (uint32_t)(s0 + j) * (4 * kStep), 0);
             }
-#pragma unroll
-            for (int i = 0; i < 8; i++) *reinterpret_cast<u32x4 *>(xb + i * 1024 + lane * 16) = xl[i];
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-                Xg[j][mt][h] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int d = 0; d < 4; d++) {
-                    xf[j][mt][h][d] = even_odd(*reinterpret_cast<const u32x4 *>(xb + c * 512 + (16 * h + 4 * g + d) * 16));
-                    Xg[j][mt][h] = mfma_act<ACT>(xf[j][mt][h][d], ones, Xg[j][mt][h]);
-                }
-            }
-        }
-    }
 
     // weights: flat step f = strip index * FS + column tile * NS + step; ring slot f % PF, LDS buffer f % 2
     u32x4 wr[PF][2];
@@ -161,6 +144,31 @@ __global__ __launch_bounds__(512) void wq_kpacked_decode_kernel(const WqKpDecode
     for (int r = 0; r < PF; r++) load_w(r, r / FS, r % FS);
     uint32_t prm_next[NT][NG / 4];
     load_params(0, prm_next);
+
+    // turn the activations around while the first weights are on their way
+    u32x4 xf[NS][MT][2][4];
+    f32x4 Xg[NS][MT][2];
+    const u32x4 ones = u32x4{kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>, kOnes2<ACT>};
+    {
+        char *xb = shared + wave * 8192;
+#pragma unroll
+        for (int j = 0; j < NS; j++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) *reinterpret_cast<u32x4 *>(xb + i * 1024 + lane * 16) = xl[j][mt][i];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                Xg[j][mt][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    xf[j][mt][h][d] = even_odd(*reinterpret_cast<const u32x4 *>(xb + c * 512 + (16 * h + 4 * g + d) * 16));
+                    Xg[j][mt][h] = mfma_act<ACT>(xf[j][mt][h][d], ones, Xg[j][mt][h]);
+                }
+            }
+        }
+    }
+
 
     // wavefront f < NT * MT finishes tile (column tile f / MT, row tile f % MT) of every strip: lane l writes row l / 4,
     // columns 4 (l % 4) .. + 3
@@ -263,7 +271,11 @@ int launch_act(const WqKpDecodeArgs &p, hipStream_t s)
 {
     const int ns = (p.K / (2 * kStep) + 7) / 8;
     if (p.M > 16) return launch<2, 2, 1, 2, ACT>(p, s);
-    return ns <= 2 ? launch<1, 2, 2, 4, ACT>(p, s) : launch<1, 4, 1, 4, ACT>(p, s);
+    if (ns > 2) return launch<1, 4, 1, 4, ACT>(p, s);
+    // strips of 32 columns keep four steps in flight across strips; when strips of 16 give every workgroup at most one,
+    // they fill twice as many CUs (4096 x 4096 at one row: 7.5 -> 6.4 us; with several strips per workgroup the deeper
+    // ring wins: 4096 x 28672 16.1 against 18.9 us)
+    return p.N <= 16 * kMaxWorkgroups ? launch<1, 2, 1, 2, ACT>(p, s) : launch<1, 2, 2, 4, ACT>(p, s);
 }
 
 } // namespace

@@ -747,6 +747,7 @@ KPACKED_CASES = [
     # at most 32 rows, groups of 128, at least 2048 columns and k: the decode kernel (weight_quant_kpacked_decode.hip), as
     # are the first two cases above
     (16, 2048, 2048, 128, True, True, True),        # one step per wavefront of the two the kernel is built for
+    (3, 4096, 4088, 128, False, False, True),       # at most 4096 columns: strips of 16 columns, the last partly valid
     (9, 5120, 2056, 128, False, False, True),       # two or three steps per wavefront, a strip that ends past N
     (4, 8192, 4096, 128, False, True, False),       # four steps per wavefront, one column tile per strip
     (16, 3072, 8224, 128, True, True, True),        # more strips than workgroups, uneven steps, fp16
