@@ -815,11 +815,12 @@ struct QmmPlan {
 // bounds small tiles on a long K (64x128 tiles on 1024x14336x4096: 1.4 GB, 107 us), and a split of K moves
 // wgs x bm x bn x 4 bytes of partial sums out and in again, the S - 1 foreign chunks of a tile through the one workgroup
 // that collects them (128x256 tiles split twelve ways: 39 us where a four-way split of 64x128 tiles takes 25).
-// Constants fitted to sweeps over tile x split on M = 128 .. 2048, K = 8192 .. 28672 (the estimate's choice is the
-// measured best on nine of ten shapes and 16 % off on the tenth; at K = 4096 without a split the estimate is the table
-// itself).
+// Constants fitted to sweeps over tile x split on M = 128 .. 2048, K = 8192 .. 28672 and on M = 80 .. 512 over the
+// projections of transformer layers with K = 4096 .. 14336 (46 shapes: the estimate's choice is 0.7 % slower than the
+// measured best on average and 8 % at worst; at K = 4096 without a split the estimate is the table itself).
 constexpr size_t kMaxPartialBytes = (size_t)128 << 20;
-constexpr double kBaseUs = 6.0, kL2BytesPerUs = 12e6, kExchangeUs = 1.0, kExchangeBytesPerUs = 12e6, kCollectorBytesPerUs = 100e3;
+constexpr double kBaseUs = 6.0, kL2BytesPerUs = 12e6, kExchangeUs = 1.0, kExchangeBytesPerUs = 10e6, kCollectorBytesPerUs = 100e3;
+constexpr double kAloneOnCu = 0.85;
 
 void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size_t partial_cap, TileChoice *tile, int *split)
 {
@@ -849,6 +850,8 @@ void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size
             // tiles that run two to a CU: with more than 256 and fewer than 512 workgroups the CUs that hold two set the
             // time, as if all did (128x128 split six ways, 384 workgroups: 42 us where eight ways, 512, take 38)
             if (c.slots == 512 && rounds == 1 && wgs > 256) loop_us *= 512.0 / (double)wgs;
+            // ... and with at most 256 every workgroup has a CU to itself
+            if (c.slots == 512 && wgs <= 256) loop_us *= kAloneOnCu;
             double cost = kBaseUs + loop_us;
             const double l2 = kBaseUs + (double)tiles * (c.bm + c.bn) * (double)K / kL2BytesPerUs;
             if (l2 > cost) cost = l2;
