@@ -509,7 +509,8 @@ def main():
             nset = _nsets(Kx * Nx)
             wsn = [torch.randint(-128, 128, (Nx, Kx), generator=gen, dtype=torch.int8, device=dev).t() for _ in range(nset)]
             sc = torch.rand(Nx, generator=gen, device=dev) * 1e-2
-            for Mx in (1, 16):
+            # 128 rows on two of them: past the decode kernel's 64 rows, the tiled kernel with the planner's tile and split
+            for Mx in (1, 16) + ((128,) if (Kx, Nx) in ((4096, 6144), (14336, 4096)) else ()):
                 xs = [torch.randint(-128, 128, (Mx, Kx), generator=gen, dtype=torch.int8, device=dev) for _ in range(nset)]
                 ps = torch.rand(Mx, generator=gen, device=dev) * 1e-2
                 keep = []
@@ -518,12 +519,12 @@ def main():
                 us = _graph_time_us(torch, calls, reps=10)
                 nb = Kx * Nx + Mx * Kx + Mx * Nx * 2 + Nx * 4 + Mx * 4
                 gate = {}
-                if not args.skip_cpu and Mx == 16:
+                if not args.skip_cpu and Mx >= 16:
                     from oracle import golden
                     gold, _ = golden.quant_matmul(xs[0].cpu().numpy(), wsn[0].cpu().numpy(), sc.cpu().numpy(), ps.cpu().numpy())
                     got = pa.npu_quant_matmul(xs[0], wsn[0], sc, pertoken_scale=ps, output_dtype=torch.bfloat16)
                     gate = {"parity_bit_exact": bool(np.array_equal(_bits(got), gold))}
-                others.append({"name": f"quant_matmul decode int8[{Mx},{Kx}] . int8 stored [{Nx},{Kx}] -> bf16", "launch_us": round(us, 3), **gate,
+                others.append({"name": f"quant_matmul {'decode ' if Mx <= 64 else ''}int8[{Mx},{Kx}] . int8 stored [{Nx},{Kx}] -> bf16", "launch_us": round(us, 3), **gate,
                                "roofline": {"bound": "hbm", "achieved": round(nb / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
                                             "unit": "GB/s", "frac": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                                             "traffic": _traffic(f"qd_{Kx}x{Nx}_m{Mx}")},
