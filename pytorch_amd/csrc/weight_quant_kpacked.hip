@@ -432,11 +432,20 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
         pl.unit_steps = (int)(K / 256);
         pl.n_units = 1;
     }
-    // eight wavefronts per workgroup when that still gives every CU a workgroup, else four; with four m tiles a
+    // eight wavefronts per workgroup when that still gives (nearly) every CU a workgroup, else four; with four m tiles a
     // wavefront owns two column tiles
     pl.ntw = pl.mt == 4 ? 2 : 1;
     const int tiles8 = (int)((N + 8 * pl.ntw * 16 - 1) / (8 * pl.ntw * 16));
-    pl.nw = (int64_t)tiles8 * pl.mchunks >= 200 ? 8 : 4;
+    const int64_t wgs8 = (int64_t)tiles8 * pl.mchunks;
+    bool eight = wgs8 >= 200;
+    if (pl.mt == 4 && !eight) {
+        // ... or, with four m tiles, when a split of K of at most eight fills the CUs with them (measured on layer
+        // projections at 48-192 rows: 14336x4096 at 128 rows 47.4 -> 40.4 us, 8192x8192 47.6 -> 38.3, 4096x14336 at 48
+        // rows 27.5 -> 24.2; a sixteen-way split of eight-wavefront workgroups loses to an eight-way one of four)
+        const int64_t s8 = kNumCU / wgs8;
+        eight = wgs8 >= 160 || (s8 <= 8 && s8 <= pl.n_units && wgs8 * s8 >= 224);
+    }
+    pl.nw = eight ? 8 : 4;
     if (const int f = knob(kKnobWqkNw))      // tuning aid
         if (f == 4 || f == 8) pl.nw = f;
     const int wg_cols = pl.nw * pl.ntw * 16;
