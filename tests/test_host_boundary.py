@@ -383,8 +383,11 @@ def test_weight_quant_workspace_query_follows_the_preferred_kernel():
     zero_area = 16 * 1024 * 1024 + 16384
     q = L.mi355_weight_quant_matmul_workspace
     assert q(1, 14336, 4096, 4, 128) == zero_area            # decode kernel, four chunks of K
-    assert q(128, 14336, 4096, 4, 128) == zero_area          # register-expanding GEMM, two chunks of K
-    assert q(128, 14336, 4096, 4, 0) == zero_area            # per channel: the same split
+    # 128 rows: the register-expanding GEMM (words along N, two chunks of K) needs the zero area alone; with the words along
+    # K the launch takes workgroups of eight wavefronts with K split two ways, so the request covers its partial sums
+    two_chunks = zero_area + 2 * 128 * 14336 * 4
+    assert q(128, 14336, 4096, 4, 128) == two_chunks
+    assert q(128, 14336, 4096, 4, 0) == two_chunks           # per channel: the same split
     repack = zero_area + 4096 * (14336 // 8) * 4 + 2 * (4096 // 128) * 14336 * 2
     for rows in (256, 2048, 8192):
         assert q(rows, 14336, 4096, 4, 128) == repack
