@@ -80,7 +80,7 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
 // MI355_QMM_DECODE_OFF: 1 = quant_matmul with at most 64 rows takes the tiled kernel instead of the decode kernel.
 enum Knob { kKnobWqSplit, kKnobWqW, kKnobWqgSplit, kKnobWqgBm, kKnobWqGemmOff, kKnobWqkMt, kKnobWqkNw, kKnobWqkKs,
             kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmDeepOff, kKnobWqGemm4Off, kKnobQmmDecodeOff,
-            kKnobCount };
+            kKnobQmmLoop, kKnobCount };
 int knob(Knob k);
 
 inline int check_launch()

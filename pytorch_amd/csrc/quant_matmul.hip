@@ -22,6 +22,7 @@
 // operations (contraction is disabled for this library) and rounds once to bf16.
 #include "common.h"
 #include "quant_matmul_decode.h"
+#include "quant_matmul_wide.h"
 #include <stdio.h>
 #include <type_traits>
 #include <stdlib.h>
@@ -94,7 +95,9 @@ __device__ __forceinline__ int32_t requant1(int32_t a, int32_t bi, float sc, flo
 }
 
 // WGM x WGN wavefronts per workgroup, each owning (16*WTM) x (16*WTN) of the output tile.
-template <int WGM, int WGN, int WTM, int WTN, int NS>
+// LOOP 0: the generic K loop below; 1 / 2: the loop of quant_matmul_wide.h (4 x 2 wavefronts of 64 rows, weights requested
+// right behind the barrier / half a step later)
+template <int WGM, int WGN, int WTM, int WTN, int NS, int LOOP = 0>
 __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 {
     constexpr int NW = WGM * WGN;
@@ -170,7 +173,43 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 #pragma unroll
         for (int j = 0; j < WTN; j++) acc[i][j] = i32x4v{0, 0, 0, 0};
 
-    if constexpr (NS == 0) {
+    if constexpr (LOOP != 0) {
+        static_assert(WGM == 4 && WGN == 2 && WTM == 4 && NS == 3, "wide loop: 4 x 2 wavefronts of 64 rows");
+        using G = wide::Geometry<WTN>;
+        if (threadIdx.x < 16) reinterpret_cast<uint32_t *>(lds + G::FLAG_BASE)[threadIdx.x] = 0u;
+        const int frow = lane & 15;
+        const uint32_t sw0 = (uint32_t)(((lane >> 4) ^ ((frow >> 1) & 7)) * 16);
+        wide::LoopState st;
+        st.va0 = (uint32_t)((wm * 64 + frow) * BK) + sw0;
+        st.va1 = (uint32_t)((wm * 64 + frow) * BK) + (sw0 ^ 64u);
+        st.vb0 = (uint32_t)(G::B_BASE + (wn * WTN * 16 + frow) * BK) + sw0;
+        st.vb1 = (uint32_t)(G::B_BASE + (wn * WTN * 16 + frow) * BK) + (sw0 ^ 64u);
+        st.flag = (uint32_t)(G::FLAG_BASE + wm * 4);
+        st.KT = KT;
+        // unit u of a stage holds rows 8u .. 8u+7; lane l fills row l / 8, 16-byte slot l % 8 with the row's chunk
+        // (l % 8) ^ ((row >> 1) & 7), and (row >> 1) & 7 = 4 * (u & 1) + (l / 8) / 2
+        auto lane_off = [&](int par, int64_t ld) { return (uint32_t)(rr * (int)ld + (((lane & 7) ^ ((par << 2) | (rr >> 1))) * 16)); };
+        if (wn == 0) {
+            const int u0 = wm * wide::LAW;                                // its own 64 activation rows
+            st.rsrc = rsrc_a;
+            st.voff0 = lane_off(0, p.lda);
+            st.voff1 = lane_off(1, p.lda);
+            st.unit_stride = unit_stride_a;
+            st.sbase = (uint32_t)u0 * unit_stride_a + (uint32_t)kt0 * BK;
+            st.dst0 = (uint32_t)u0 * 1024u;
+            wide::k_loop<WTN, 0, LOOP - 1>(acc, lds, st);
+        } else {
+            const int u0 = wm * G::LBW;                                   // a quarter of the weight rows
+            st.rsrc = rsrc_b;
+            st.voff0 = lane_off(u0 & 1, p.ldbt);
+            st.voff1 = lane_off((u0 & 1) ^ 1, p.ldbt);
+            st.unit_stride = unit_stride_b;
+            st.sbase = (uint32_t)u0 * unit_stride_b + (uint32_t)kt0 * BK;
+            st.dst0 = (uint32_t)u0 * 1024u;
+            wide::k_loop<WTN, 1, LOOP - 1>(acc, lds, st);
+        }
+        __syncthreads();
+    } else if constexpr (NS == 0) {
         // ---- streaming K loop (at most 64 rows, few workgroups per CU: the weights are a pure HBM stream).  No workgroup
         // ring and no barrier per K step: a wavefront owns its 16 weight rows (= 16 output columns) for the whole K range
         // of the workgroup, loads 128 bytes of each row per step straight into registers, four steps in flight - whole cache
@@ -762,7 +801,7 @@ __global__ __launch_bounds__(256) void transpose_i8_wide_kernel(const int8_t *__
     }
 }
 
-template <int WGM, int WGN, int WTM, int WTN, int DEEP = 0>
+template <int WGM, int WGN, int WTM, int WTN, int DEEP = 0, int LOOP = 0>
 int launch_qmm(QmmArgs p, hipStream_t s)
 {
     constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
@@ -776,14 +815,15 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     constexpr int NS = DEEP < 0 ? 0 : DEEP ? DEEP : 2 * a_bytes + 2 * b_bytes <= 80 * 1024 && staging_bytes <= 80 * 1024 ? 2 : 3;
     // DEEP < 0: the streaming K loop (two activation chunks of 32 KiB and a 4 KiB turn-around tile per wavefront)
     constexpr size_t stage_bytes = DEEP < 0 ? (size_t)2 * 32768 + 8 * 4096 : (DEEP ? DEEP : 2) * a_bytes + NS * b_bytes;
-    constexpr size_t lds_bytes = stage_bytes > staging_bytes ? stage_bytes : staging_bytes;
+    constexpr size_t ring_bytes = LOOP != 0 ? (size_t)wide::Geometry<WTN>::LDS_BYTES : stage_bytes;
+    constexpr size_t lds_bytes = ring_bytes > staging_bytes ? ring_bytes : staging_bytes;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
     if (p.S > 1 && (uint64_t)p.S * BM * BN * 4 >= (1ull << 32)) return MI355_ERR_UNSUPPORTED;
-    auto kern = qmm_kernel<WGM, WGN, WTM, WTN, NS>;
+    auto kern = qmm_kernel<WGM, WGN, WTM, WTN, NS, LOOP>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
@@ -1026,6 +1066,13 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
 #define MI355_QMM_CASE(bm_, bn_, wgm_, wgn_)  \
     if (c.bm == bm_ && c.bn == bn_) return launch_qmm<wgm_, wgn_, bm_ / (16 * wgm_), bn_ / (16 * wgn_)>(p, s);
     MI355_QMM_CASE(256, 256, 2, 4)
+    {
+        const int lk = knob(kKnobQmmLoop);                 // 0: automatic; 1: the generic loop; 2, 3: the wide loop's variants
+        if (lk == 2 || lk == 3) {
+            if (c.bm == 256 && c.bn == 224) return lk == 2 ? launch_qmm<4, 2, 4, 7, 0, 1>(p, s) : launch_qmm<4, 2, 4, 7, 0, 2>(p, s);
+            if (c.bm == 256 && c.bn == 192) return lk == 2 ? launch_qmm<4, 2, 4, 6, 0, 1>(p, s) : launch_qmm<4, 2, 4, 6, 0, 2>(p, s);
+        }
+    }
     MI355_QMM_CASE(256, 224, 4, 2)
     MI355_QMM_CASE(256, 192, 4, 2)
     MI355_QMM_CASE(128, 320, 2, 4)
