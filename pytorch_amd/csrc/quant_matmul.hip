@@ -76,7 +76,16 @@ struct QmmArgs {
     int S;                     // workgroups that share the K range of a tile
     int32_t *partial;          // workspace [tile][chunk][wavefront][accumulator quad][lane] int32x4 (S > 1)
     uint32_t *counter;         // workspace [tile], zero on entry, left zero (S > 1)
+#ifdef MI355_QMM_TS
+    unsigned long long *ts;    // debugging aid: [workgroup][wavefront][64] cycle counter stamps
+#endif
 };
+
+#ifdef MI355_QMM_TS
+#define MI355_TS(IDX) if (p.ts && lane == 0) p.ts[((size_t)blockIdx.x * 8 + wave) * 128 + (IDX)] = __builtin_readcyclecounter();
+#else
+#define MI355_TS(IDX)
+#endif
 
 // Packed quantisation parameter (the 64-bit words npu_trans_quant_param produces): bits 0-31 the float32 scale,
 // bits 37-45 the offset as a 9-bit two's-complement integer, bit 46 set.
@@ -95,8 +104,8 @@ __device__ __forceinline__ int32_t requant1(int32_t a, int32_t bi, float sc, flo
 }
 
 // WGM x WGN wavefronts per workgroup, each owning (16*WTM) x (16*WTN) of the output tile.
-// LOOP 0: the generic K loop below; 1 / 2: the loop of quant_matmul_wide.h (4 x 2 wavefronts of 64 rows, weights requested
-// right behind the barrier / half a step later)
+// LOOP 0: the generic K loop below; 1, 2: the loop of quant_matmul_wide.h (4 x 2 wavefronts of 64 rows) with its
+// instruction order 0 (refills in a block) or 1 (refills spread over the step)
 template <int WGM, int WGN, int WTM, int WTN, int NS, int LOOP = 0>
 __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 {
@@ -124,6 +133,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    MI355_TS(0)
     const int wm = wave / WGN, wn = wave % WGN;
     const int kt0 = (int)((int64_t)(p.K / BK) * chunk / p.S);            // first K step of this workgroup
     const int KT = (int)((int64_t)(p.K / BK) * (chunk + 1) / p.S) - kt0;  // its number of K steps
@@ -173,10 +183,19 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 #pragma unroll
         for (int j = 0; j < WTN; j++) acc[i][j] = i32x4v{0, 0, 0, 0};
 
+    // the wide loop's epilogue for the common case takes its parameters from LDS (quant_matmul_wide.h)
+    const bool fast_epilogue = LOOP != 0 && !p.out_i32 && !p.out_i8 && !p.qparam && p.pertoken && p.scale_len == p.N &&
+                               (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_BF16) && (p.ldc & 7) == 0 &&
+                               aligned_dev(p.out, 16) && aligned_dev(p.pertoken, 16) && aligned_dev(p.scale, 16) &&
+                               (!p.bias || aligned_dev(p.bias, 16));
+
     if constexpr (LOOP != 0) {
         static_assert(WGM == 4 && WGN == 2 && WTM == 4 && NS == 3, "wide loop: 4 x 2 wavefronts of 64 rows");
         using G = wide::Geometry<WTN>;
         if (threadIdx.x < 16) reinterpret_cast<uint32_t *>(lds + G::FLAG_BASE)[threadIdx.x] = 0u;
+        if (fast_epilogue && wave == 0)
+            wide::request_params(lds, G::PARAM_BASE, p.pertoken, p.scale, p.bias_kind == MI355_BIAS_BF16 ? p.bias : nullptr, m0, n0,
+                                 rows_a, rows_b, lane);
         const int frow = lane & 15;
         const uint32_t sw0 = (uint32_t)(((lane >> 4) ^ ((frow >> 1) & 7)) * 16);
         wide::LoopState st;
@@ -186,6 +205,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         st.vb1 = (uint32_t)(G::B_BASE + (wn * WTN * 16 + frow) * BK) + (sw0 ^ 64u);
         st.flag = (uint32_t)(G::FLAG_BASE + wm * 4);
         st.KT = KT;
+#ifdef MI355_QMM_TS
+        st.ts = p.ts ? p.ts + ((size_t)blockIdx.x * 8 + wave) * 128 : nullptr;
+#endif
         // unit u of a stage holds rows 8u .. 8u+7; lane l fills row l / 8, 16-byte slot l % 8 with the row's chunk
         // (l % 8) ^ ((row >> 1) & 7), and (row >> 1) & 7 = 4 * (u & 1) + (l / 8) / 2
         auto lane_off = [&](int par, int64_t ld) { return (uint32_t)(rr * (int)ld + (((lane & 7) ^ ((par << 2) | (rr >> 1))) * 16)); };
@@ -208,7 +230,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             st.dst0 = (uint32_t)u0 * 1024u;
             wide::k_loop<WTN, 1, LOOP - 1>(acc, lds, st);
         }
+        MI355_TS(2)
         __syncthreads();
+        MI355_TS(3)
     } else if constexpr (NS == 0) {
         // ---- streaming K loop (at most 64 rows, few workgroups per CU: the weights are a pure HBM stream).  No workgroup
         // ring and no barrier per K step: a wavefront owns its 16 weight rows (= 16 output columns) for the whole K range
@@ -464,6 +488,22 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         if (threadIdx.x == 0) __hip_atomic_store(p.counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
+    if constexpr (LOOP != 0) {
+        if (fast_epilogue) {
+            wide::EpilogueArgs e;
+            e.out = p.out;
+            e.ldc = p.ldc;
+            e.M = p.M;
+            e.N = p.N;
+            e.m0 = m0;
+            e.n0 = n0;
+            e.has_bias = p.bias_kind == MI355_BIAS_BF16;
+            e.out_f16 = p.out_f16;
+            wide::epilogue_fast<WTN>(acc, lds, e, wave, lane);
+            MI355_TS(4)
+            return;
+        }
+    }
     // Epilogue.  The weight fragment was the first MFMA operand, so
     // acc[i][j][r] = C[m = tile row (lane % 16)][n = 4 * (lane / 16) + r].
     const int mrow = lane & 15;
@@ -957,6 +997,10 @@ __global__ __launch_bounds__(256) void trans_quant_param_kernel(const float *__r
     out[i] = q;
 }
 
+#ifdef MI355_QMM_TS
+unsigned long long *g_dbg_ts = nullptr;
+#endif
+
 // One implementation behind both entry points: `scale` (float32) or `qparam` (packed) carries the per-channel factors.
 int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale, const uint64_t *qparam,
                      int64_t scale_len, const void *bias, int bias_dtype, void *out, int out_dtype, int64_t M,
@@ -1063,14 +1107,17 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     p.S = pl.S;
     p.counter = pl.S > 1 ? reinterpret_cast<uint32_t *>(ws) : nullptr;
     p.partial = pl.S > 1 ? reinterpret_cast<int32_t *>(ws + pl.counter_bytes) : nullptr;
+#ifdef MI355_QMM_TS
+    p.ts = g_dbg_ts;
+#endif
 #define MI355_QMM_CASE(bm_, bn_, wgm_, wgn_)  \
     if (c.bm == bm_ && c.bn == bn_) return launch_qmm<wgm_, wgn_, bm_ / (16 * wgm_), bn_ / (16 * wgn_)>(p, s);
     MI355_QMM_CASE(256, 256, 2, 4)
     {
-        const int lk = knob(kKnobQmmLoop);                 // 0: automatic; 1: the generic loop; 2, 3: the wide loop's variants
-        if (lk == 2 || lk == 3) {
-            if (c.bm == 256 && c.bn == 224) return lk == 2 ? launch_qmm<4, 2, 4, 7, 0, 1>(p, s) : launch_qmm<4, 2, 4, 7, 0, 2>(p, s);
-            if (c.bm == 256 && c.bn == 192) return lk == 2 ? launch_qmm<4, 2, 4, 6, 0, 1>(p, s) : launch_qmm<4, 2, 4, 6, 0, 2>(p, s);
+        const int lk = knob(kKnobQmmLoop);                 // 0: automatic; 1: the generic loop; 2, 3: the wide loop's instruction orders
+        if (lk != 1) {
+            if (c.bm == 256 && c.bn == 224) return lk == 3 ? launch_qmm<4, 2, 4, 7, 0, 2>(p, s) : launch_qmm<4, 2, 4, 7, 0, 1>(p, s);
+            if (c.bm == 256 && c.bn == 192) return lk == 3 ? launch_qmm<4, 2, 4, 6, 0, 2>(p, s) : launch_qmm<4, 2, 4, 6, 0, 1>(p, s);
         }
     }
     MI355_QMM_CASE(256, 224, 4, 2)
@@ -1096,6 +1143,10 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
 
 } // namespace
 } // namespace mi355
+
+#ifdef MI355_QMM_TS
+extern "C" void mi355_dbg_set_ts(unsigned long long *p) { mi355::g_dbg_ts = p; }
+#endif
 
 extern "C" int mi355_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_scale, const float *scale,
                                   int64_t scale_len, const void *bias, int bias_dtype, void *out, int out_dtype, int64_t M,

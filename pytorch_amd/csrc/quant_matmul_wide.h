@@ -16,6 +16,11 @@
 //    ALU instructions per step besides the MFMAs.
 #pragma once
 #include "common.h"
+#include <utility>
+
+#ifndef MI355_WIDE_ABL
+#define MI355_WIDE_ABL 0       // compile-time ablations for timing experiments (wrong results): 1 no refill traffic, 2 no fragment reads, 4 no MFMAs, 8 no handshake, 16 no barrier
+#endif
 
 namespace mi355 {
 namespace wide {
@@ -34,8 +39,8 @@ struct Geometry {
     static constexpr int B_BYTES = LBW * 4 * 1024;           // one weight slot
     static constexpr int B_BASE = 2 * A_BYTES;
     static constexpr int FLAG_BASE = B_BASE + 3 * B_BYTES;   // four flag words, one per pair of wavefronts
-    static constexpr int PARAM_BASE = FLAG_BASE + 64;        // epilogue parameters (filled during the prologue)
-    static constexpr int LDS_BYTES = PARAM_BASE + 4096;
+    static constexpr int PARAM_BASE = FLAG_BASE + 64;        // epilogue parameters (filled during the prologue): 2.5 KiB
+    static constexpr int LDS_BYTES = PARAM_BASE + 2560;
 };
 
 // s_waitcnt vmcnt(VM) lgkmcnt(0) as the builtin, so that the compiler's own bookkeeping of outstanding LDS reads sees it
@@ -65,7 +70,8 @@ __device__ __forceinline__ void mfma_range(i32x4v (&acc)[4][WTN], const i32x4v (
 #pragma unroll
     for (int t = FROM; t < TO; t++) {
         const int i = t / WTN, j = t % WTN;
-        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
+        if constexpr (MI355_WIDE_ABL & 4) asm volatile("" ::"v"(bf[j]), "v"(af[i]));
+        else acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
     }
 }
 
@@ -91,57 +97,197 @@ struct LoopState {
     uint32_t va0, va1, vb0, vb1;       // LDS byte offsets of the lane's fragment rows (first / second 64 bytes of a K step)
     uint32_t flag;                     // LDS byte offset of the pair's flag word
     int KT;                            // K steps of this workgroup
+#ifdef MI355_QMM_TS
+    unsigned long long *ts;
+#endif
 };
+
+#ifdef MI355_QMM_TS
+#define MI355_WIDE_TS(IDX) if (st.ts && (threadIdx.x & 63) == 0 && (IDX) < 128) st.ts[(IDX)] = __builtin_readcyclecounter();
+#else
+#define MI355_WIDE_TS(IDX)
+#endif
+
+// ---------------------------------------------------------------------------------------------------------------
+// Instruction order.  A part of a K step is written as a string, one character per instruction, and emitted in exactly
+// that order (every instruction is pinned by a scheduling group of its own):
+//   M  the next MFMA of the half step (activation fragment outer, weight fragment inner)
+//   a  the next activation fragment read (first the four fragments of the first 64 bytes of K, then the second four)
+//   b  the next weight fragment read
+//   D  the next refill (1 KiB direct-to-LDS load) of this wavefront
+// Every wavefront issues, per K step, the second half "S" (behind the barrier in the middle of the step; split into the
+// part before the release of the activation slot, S1, and the part after it, S2) and the first half "F" of the next step.
+// The refills of one stage may be spread over S2 and the following F: they all precede the next barrier, so the number
+// of loads that may be outstanding there does not change.
+template <int V, int WTN, int ROLE, int PART>
+struct Order {
+    static constexpr const char *str()
+    {
+        if constexpr (WTN == 6) {
+            if constexpr (V == 0) {
+                if constexpr (PART == 0) return "aMaMaMaMaMaMaMaMbMbMbMbMbMbM";
+                if constexpr (PART == 1) return ROLE == 0 ? "DMDMDMDMDMDMDMDMMM" : "DMDMDMDMDMDMMMMM";
+                if constexpr (PART == 2) return "bMMbMMbMMbMMbMMbMMMMMMMMMMMMMM";
+            }
+            if constexpr (V == 1) {
+                if constexpr (PART == 0) return "aMaMaMaMaMaMaMaMbMbMbMbMbMbM";
+                if constexpr (PART == 1) return "DMMMDMMMDMMMM";
+                if constexpr (PART == 2) return ROLE == 0 ? "bMMDMbMMMbDMMMbMDMMbMMDMbMMMDMMMMMM" : "bMMMbMDMMbMMMbMDMMbMMMbMDMMMMMMMM";
+            }
+        } else if constexpr (WTN == 7) {
+            if constexpr (V == 0) {
+                if constexpr (PART == 0) return "aMaMaMaMaMaMaMaMbMbMbMbMbMbMbM";
+                if constexpr (PART == 1) return ROLE == 0 ? "DMDMDMDMDMDMDMDMMMMMM" : "DMDMDMDMDMDMDMMMMMMM";
+                if constexpr (PART == 2) return "bMMbMMbMMbMMbMMbMMbMMMMMMMMMMMMMMMM";
+            }
+            if constexpr (V == 1) {
+                if constexpr (PART == 0) return "aMaMaMaMaMaMaMaMbMbMbMbMbMbMbM";
+                if constexpr (PART == 1) return "DMMMDMMMDMMMMMMM";
+                if constexpr (PART == 2) return ROLE == 0 ? "bMMDMbMMMbDMMMbMDMMbMMDMbMMMbDMMMMMMMMMM" : "bMMMbMDMMbMMMbMDMMbMMMbMDMMbMMMMDMMMMMM";
+            }
+        }
+        return "";
+    }
+    static constexpr int length()
+    {
+        int n = 0;
+        while (str()[n]) n++;
+        return n;
+    }
+    static constexpr char at(int i) { return str()[i]; }
+    static constexpr int count(char c, int upto = length())
+    {
+        int n = 0;
+        for (int i = 0; i < upto; i++) n += str()[i] == c;
+        return n;
+    }
+    // weight fragment reads behind the last activation fragment read (what may still be in flight when the slot is released)
+    static constexpr int b_after_last_a()
+    {
+        int n = 0;
+        for (int i = 0; i < length(); i++) {
+            if (str()[i] == 'a') n = 0;
+            if (str()[i] == 'b') n++;
+        }
+        return n;
+    }
+};
+
+// refill number i of a stage: 1 KiB, eight rows of 128 bytes
+__device__ __forceinline__ void issue_unit(const LoopState &st, char *lds, uint32_t dst, uint32_t soff, int i)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(st.rsrc, (lds_void *)(lds + dst + i * 1024), 16, (i & 1) ? st.voff1 : st.voff0,
+                                             soff + (uint32_t)i * st.unit_stride, 0, 0);
+}
+
+template <int WTN>
+struct PartCtx {
+    i32x4v (&acc)[4][WTN];
+    const i32x4v (&ma)[4];             // MFMA operands of this part
+    const i32x4v (&mb)[WTN];
+    i32x4v (&ra0)[4];                  // destinations of the fragment reads
+    i32x4v (&ra1)[4];
+    i32x4v (&rb)[WTN];
+    char *lds;
+    uint32_t a0, a1, b;                // LDS byte offsets the fragments are read from
+    const LoopState &st;
+    uint32_t dst, soff;                // refills: LDS byte offset and scalar offset of the wavefront's first unit
+};
+
+template <char C, int IDX, int M0, int A0, int B0, int D0, int WTN>
+__device__ __forceinline__ void emit_one(PartCtx<WTN> &c)
+{
+    if constexpr (C == 'M') {
+        constexpr int t = M0 + IDX, i = t / WTN, j = t % WTN;
+        if constexpr (MI355_WIDE_ABL & 4) asm volatile("" ::"v"(c.mb[j]), "v"(c.ma[i]));
+        else c.acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(c.mb[j], c.ma[i], c.acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    } else if constexpr (C == 'a') {
+        constexpr int r = A0 + IDX;
+        if constexpr (!(MI355_WIDE_ABL & 2)) {
+            if constexpr (r < 4) c.ra0[r] = *reinterpret_cast<const i32x4v *>(c.lds + c.a0 + r * 2048);
+            else c.ra1[r - 4] = *reinterpret_cast<const i32x4v *>(c.lds + c.a1 + (r - 4) * 2048);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    } else if constexpr (C == 'b') {
+        constexpr int r = B0 + IDX;
+        if constexpr (!(MI355_WIDE_ABL & 2)) {
+            c.rb[r] = *reinterpret_cast<const i32x4v *>(c.lds + c.b + r * 2048);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    } else {
+        static_assert(C == 'D', "unknown instruction class");
+        issue_unit(c.st, c.lds, c.dst, c.soff, D0 + IDX);
+        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+    }
+}
+
+// emits the instructions of Order O; M0 / A0 / B0 / D0: how many of each class the earlier parts of the half step held
+template <class O, int M0, int A0, int B0, int D0, int WTN, int... I>
+__device__ __forceinline__ void emit_part(PartCtx<WTN> &c, std::integer_sequence<int, I...>)
+{
+    (emit_one<O::at(I), O::count(O::at(I), I), M0, A0, B0, D0, WTN>(c), ...);
+}
 
 template <int NL>
 __device__ __forceinline__ void issue_units(const LoopState &st, char *lds, uint32_t dst, uint32_t soff)
 {
 #pragma unroll
-    for (int i = 0; i < NL; i++)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(st.rsrc, (lds_void *)(lds + dst + i * 1024), 16, (i & 1) ? st.voff1 : st.voff0,
-                                                 soff + (uint32_t)i * st.unit_stride, 0, 0);
+    for (int i = 0; i < NL; i++) issue_unit(st, lds, dst, soff, i);
 }
 
-// ROLE 0: refills activations (two slots); ROLE 1: refills weights (three slots).
-// BPOS 0: weights are requested right behind the barrier that releases their slot (two steps of lead);
-// BPOS 1: half a step later, in the first half of the next step, so that the two roles' requests alternate.
-template <int WTN, int ROLE, int BPOS>
+// ROLE 0: refills activations (two slots); ROLE 1: refills weights (three slots).  V: instruction order (Order).
+template <int WTN, int ROLE, int V>
 __device__ __forceinline__ void k_loop(i32x4v (&acc)[4][WTN], char *lds, const LoopState st)
 {
     using G = Geometry<WTN>;
     constexpr int LBW = G::LBW, B_BYTES = G::B_BYTES, B_BASE = G::B_BASE;
     constexpr int NL = ROLE == 0 ? LAW : LBW;                  // refills of this wavefront per stage
     constexpr int HALF = 4 * WTN;                              // MFMAs per half step
-    static_assert(HALF - 8 - WTN >= (ROLE == 0 ? LAW : (BPOS == 0 ? LBW : 0)), "refills need MFMAs to hide behind");
+    using S1 = Order<V, WTN, ROLE, 0>;
+    using S2 = Order<V, WTN, ROLE, 1>;
+    using F = Order<V, WTN, ROLE, 2>;
+    constexpr int DS1 = S1::count('D'), DS = DS1 + S2::count('D');   // refills issued in S; the rest follow in F
+    static_assert(S1::count('M') + S2::count('M') == HALF && F::count('M') == HALF, "MFMAs per half step");
+    static_assert(S1::count('a') == 8 && S2::count('a') == 0 && F::count('a') == 0, "activation fragments are read before the release");
+    static_assert(S1::count('b') + S2::count('b') == WTN && F::count('b') == WTN, "weight fragment reads");
+    static_assert(DS + F::count('D') == NL, "refills per stage");
+    static_assert(ROLE == 1 || DS1 == 0, "activation refills follow the release");
     const int KT = st.KT;
-    auto k_off = [&](int stage) { return stage < KT ? st.sbase + (uint32_t)stage * BK : kPastEnd; };
+    auto k_off = [&](int stage) { return stage < KT && !(MI355_WIDE_ABL & 1) ? st.sbase + (uint32_t)stage * BK : kPastEnd; };
     typedef __attribute__((address_space(3))) volatile uint32_t lds_flag_t;
     lds_flag_t *flag = (lds_flag_t *)(lds + st.flag);
 
     i32x4v ap[4], aq0[4], aq1[4], bf0[WTN], bf1[WTN];
 
-#define MI355_WIDE_READ_A(P_, Q_, SLOT_)                                                                             \
-    _Pragma("unroll") for (int i = 0; i < 4; i++)                                                                    \
-        P_[i] = *reinterpret_cast<const i32x4v *>(lds + st.va0 + (SLOT_) * A_BYTES + i * 2048);                      \
-    _Pragma("unroll") for (int i = 0; i < 4; i++)                                                                    \
-        Q_[i] = *reinterpret_cast<const i32x4v *>(lds + st.va1 + (SLOT_) * A_BYTES + i * 2048);
-#define MI355_WIDE_READ_B(BF_, VB_, SB_)                                                                             \
-    _Pragma("unroll") for (int j = 0; j < WTN; j++)                                                                  \
-        BF_[j] = *reinterpret_cast<const i32x4v *>(lds + (VB_) + (SB_) + j * 2048);
-    // release of the activation slot just read: the reader publishes, the loader waits for it
+    // release of the activation slot just read: the reader publishes the step, the loader waits for it
 #define MI355_WIDE_PUBLISH(VAL_)                                                                                     \
-    {                                                                                                                \
-        /* the eight activation reads are older than the WTN weight reads; one lane stores the flag */             \
+    if constexpr (!(MI355_WIDE_ABL & 8)) {                                                                           \
+        /* LDS reads return in order: at most the weight fragment reads behind the last activation read may be     \
+           outstanding; one lane stores the flag */                                                                 \
         asm volatile("s_waitcnt lgkmcnt(%2)\n\ts_mov_b64 exec, 1\n\tds_write_b32 %0, %1\n\ts_mov_b64 exec, -1"           \
-                     ::"v"(st.flag), "v"((uint32_t)(VAL_)), "n"(WTN) : "memory");                                    \
+                     ::"v"(st.flag), "v"((uint32_t)(VAL_)), "n"(S1::b_after_last_a()) : "memory");                   \
     }
 #define MI355_WIDE_AWAIT(VAL_)                                                                                       \
-    {                                                                                                                \
+    if constexpr (!(MI355_WIDE_ABL & 8)) {                                                                           \
+        /* like the barrier, this wait ends because the other wavefront of the pair runs the same steps */          \
         uint32_t f_;                                                                                                 \
-        int spins_ = 0;                                                                                              \
         do {                                                                                                         \
             f_ = __builtin_amdgcn_readfirstlane(*flag);                                                              \
-        } while (f_ < (VAL_) && ++spins_ < (1 << 16));                                                               \
+        } while (f_ < (VAL_));                                                                                       \
+    }
+    // the second half of step KT_ (KT_ = -1: what precedes the loop): fragments of stage KT_ + 1, refills of stage KT_ + 3
+#define MI355_WIDE_SECOND(KT_, Q_, QN_, ASLOT_, MFMA_)                                                               \
+    {                                                                                                                \
+        PartCtx<WTN> c_{acc, Q_, bf1, ap, QN_, bf0, lds, st.va0 + (ASLOT_) * A_BYTES, st.va1 + (ASLOT_) * A_BYTES,   \
+                        st.vb0 + sb_rd, st, ROLE == 0 ? st.dst0 + (ASLOT_) * A_BYTES : B_BASE + st.dst0 + sb_wr,     \
+                        k_off((KT_) + 3)};                                                   \
+        emit_part<S1, 0, 0, 0, 0>(c_, std::make_integer_sequence<int, S1::length()>{});                              \
+        __builtin_amdgcn_sched_barrier(0);                                                                           \
+        if constexpr (ROLE == 1) { MI355_WIDE_PUBLISH((uint32_t)((KT_) + 2)) } else { MI355_WIDE_AWAIT((uint32_t)((KT_) + 2)) } \
+        __builtin_amdgcn_sched_barrier(0);                                                                           \
+        emit_part<S2, S1::count('M'), 8, S1::count('b'), DS1>(c_, std::make_integer_sequence<int, S2::length()>{});  \
+        __builtin_amdgcn_sched_barrier(0);                                                                           \
     }
 
     // prologue: stages 0 and 1 are requested, stage 0 has landed behind the barrier
@@ -152,28 +298,27 @@ __device__ __forceinline__ void k_loop(i32x4v (&acc)[4][WTN], char *lds, const L
         issue_units<NL>(st, lds, B_BASE + st.dst0, k_off(0));
         issue_units<NL>(st, lds, B_BASE + st.dst0 + B_BYTES, k_off(1));
     }
-    wait_vmcnt_lgkm0<NL>();                 // (also the caller's LDS stores: the cleared flags)
+    wait_vmcnt_lgkm0<NL>();                  // stage 0 (also the caller's LDS stores: the cleared flags)
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
+    MI355_WIDE_TS(1)
 
     uint32_t sb_rd = 0;                      // byte offset of the weight slot that is read
-    uint32_t sb_wr = 2 * B_BYTES;            // ... of the weight slot refilled next
-    // what follows the barrier of "step -1": fragments of stage 0, release and refill of its activation slot
+    uint32_t sb_wr = 2 * B_BYTES;            // ... of the weight slot being refilled
     {
-        MI355_WIDE_READ_A(ap, aq0, 0)
-        __builtin_amdgcn_sched_barrier(0);   // the order of the reads matters to the publishing wait below
-        MI355_WIDE_READ_B(bf0, st.vb0, sb_rd)
+        // what precedes the loop is the second half of "step -1" without MFMAs: fragments of stage 0, release of its
+        // activation slot, the first refills of stage 2
+#pragma unroll
+        for (int i = 0; i < 4; i++) ap[i] = *reinterpret_cast<const i32x4v *>(lds + st.va0 + i * 2048);
+#pragma unroll
+        for (int i = 0; i < 4; i++) aq0[i] = *reinterpret_cast<const i32x4v *>(lds + st.va1 + i * 2048);
+        __builtin_amdgcn_sched_barrier(0);   // the order of the reads matters to the publishing wait
+#pragma unroll
+        for (int j = 0; j < WTN; j++) bf0[j] = *reinterpret_cast<const i32x4v *>(lds + st.vb0 + j * 2048);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (ROLE == 1) {
-            MI355_WIDE_PUBLISH(1u)
-            if constexpr (BPOS == 0) {
-                issue_units<NL>(st, lds, B_BASE + st.dst0 + sb_wr, k_off(2));
-                sb_wr = 0;
-            }
-        } else {
-            MI355_WIDE_AWAIT(1u)
-            issue_units<NL>(st, lds, st.dst0, k_off(2));
-        }
+        if constexpr (ROLE == 1) { MI355_WIDE_PUBLISH(1u) } else { MI355_WIDE_AWAIT(1u) }
+        __builtin_amdgcn_sched_barrier(0);
+        issue_units<DS>(st, lds, ROLE == 0 ? st.dst0 : B_BASE + st.dst0 + sb_wr, k_off(2));
         __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -181,46 +326,24 @@ __device__ __forceinline__ void k_loop(i32x4v (&acc)[4][WTN], char *lds, const L
     // step; ASLOT_ is the activation slot of the next step (compile time: the loop is unrolled by two).
 #define MI355_WIDE_STEP(KT_, Q_, QN_, ASLOT_)                                                                        \
     {                                                                                                                \
-        /* first half: the weights of the second 64 bytes of K arrive while the first 64 are multiplied */         \
-        MI355_WIDE_READ_B(bf1, st.vb1, sb_rd)                                                                        \
-        if constexpr (ROLE == 1 && BPOS == 1) issue_units<NL>(st, lds, B_BASE + st.dst0 + sb_wr, k_off((KT_) + 2)); \
-        mfma_range<WTN, 0, HALF>(acc, ap, bf0);                                                                      \
-        interleave<0x100, WTN, 2>();                                                                                 \
-        if constexpr (ROLE == 1 && BPOS == 1) interleave<0x010, NL, 1>();                                            \
-        __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);                                                        \
+        /* first half: the weights of the second 64 bytes of K arrive while the first 64 are multiplied; the      \
+           remaining refills of stage KT_ + 2 */                                                                    \
+        {                                                                                                            \
+            PartCtx<WTN> c_{acc, ap, bf0, ap, ap, bf1, lds, 0u, 0u, st.vb1 + sb_rd, st,                              \
+                            ROLE == 0 ? st.dst0 + (1 - (ASLOT_)) * A_BYTES : B_BASE + st.dst0 + sb_wr, k_off((KT_) + 2)}; \
+            emit_part<F, 0, 0, 0, DS>(c_, std::make_integer_sequence<int, F::length()>{});                           \
+        }                                                                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                                           \
         /* stage KT_ + 1 has landed (only this wavefront's newest refill may be in flight) and this wavefront is   \
            done reading the weights of stage KT_ */                                                                 \
+        MI355_WIDE_TS(8 + 2 * (KT_))                                                                                 \
         wait_vmcnt_lgkm0<NL>();                                                                                      \
-        __builtin_amdgcn_s_barrier();                                                                                \
+        MI355_WIDE_TS(9 + 2 * (KT_))                                                                                 \
+        if constexpr (!(MI355_WIDE_ABL & 16)) __builtin_amdgcn_s_barrier();                                          \
         __builtin_amdgcn_sched_barrier(0);                                                                           \
         sb_rd = sb_rd == 2 * B_BYTES ? 0u : sb_rd + B_BYTES;                                                         \
-        /* second half: all activation fragments of the next step first, then its first weights */                 \
-        MI355_WIDE_READ_A(ap, QN_, ASLOT_)                                                                           \
-        mfma_range<WTN, 0, 8>(acc, Q_, bf1);                                                                         \
-        interleave<0x100, 8, 1>();                                                                                   \
-        __builtin_amdgcn_sched_barrier(0);                                                                           \
-        MI355_WIDE_READ_B(bf0, st.vb0, sb_rd)                                                                        \
-        mfma_range<WTN, 8, 8 + WTN>(acc, Q_, bf1);                                                                   \
-        interleave<0x100, WTN, 1>();                                                                                 \
-        __builtin_amdgcn_sched_barrier(0);                                                                           \
-        if constexpr (ROLE == 1) {                                                                                   \
-            MI355_WIDE_PUBLISH((uint32_t)(KT_) + 2u)                                                                 \
-            __builtin_amdgcn_sched_barrier(0);                                                                       \
-            if constexpr (BPOS == 0) issue_units<NL>(st, lds, B_BASE + st.dst0 + sb_wr, k_off((KT_) + 3));           \
-            mfma_range<WTN, 8 + WTN, HALF>(acc, Q_, bf1);                                                            \
-            if constexpr (BPOS == 0) interleave<0x010, NL, 1>();                                                     \
-            __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);                                                    \
-        } else {                                                                                                     \
-            MI355_WIDE_AWAIT((uint32_t)(KT_) + 2u)                                                                   \
-            __builtin_amdgcn_sched_barrier(0);                                                                       \
-            issue_units<NL>(st, lds, st.dst0 + (ASLOT_) * A_BYTES, k_off((KT_) + 3));                                \
-            mfma_range<WTN, 8 + WTN, HALF>(acc, Q_, bf1);                                                            \
-            interleave<0x010, NL, 1>();                                                                              \
-            __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);                                                    \
-        }                                                                                                            \
         sb_wr = sb_wr == 2 * B_BYTES ? 0u : sb_wr + B_BYTES;                                                         \
-        __builtin_amdgcn_sched_barrier(0);                                                                           \
+        MI355_WIDE_SECOND(KT_, Q_, QN_, ASLOT_, 1)                                                                   \
     }
 
     for (int kt = 0; kt < KT; kt += 2) {
@@ -229,11 +352,118 @@ __device__ __forceinline__ void k_loop(i32x4v (&acc)[4][WTN], char *lds, const L
         MI355_WIDE_STEP(kt + 1, aq1, aq0, 0)
     }
 #undef MI355_WIDE_STEP
-#undef MI355_WIDE_READ_A
-#undef MI355_WIDE_READ_B
+#undef MI355_WIDE_SECOND
 #undef MI355_WIDE_PUBLISH
 #undef MI355_WIDE_AWAIT
     wait_vmcnt_only<0>();                    // the refills past the end must not land in the epilogue's LDS
+}
+
+
+// ---------------------------------------------------------------------------------------------------------------
+// Epilogue for the common case: per-token scale, one float32 scale per column, optional bf16 bias, bf16 / fp16 output
+// with 16-byte aligned rows.  The three parameter vectors of the tile were requested into LDS (PARAM_BASE) before the
+// first K step, so nothing here waits for global memory.  Per block of 16 rows a wavefront converts its WTN accumulator
+// tiles, stages them in its own LDS rows and stores whole rows of the wavefront tile (16 bytes per lane) right away, so
+// the stores of one block leave while the next block is converted.
+//   ((float(acc) * pertoken[m]) * scale[n]) + bias[n], every operation rounded to binary32, one rounding to 16 bits.
+struct EpilogueArgs {
+    void *out;
+    int64_t ldc;
+    int M, N;
+    int m0, n0;                        // first row / column of the workgroup tile
+    int has_bias, out_f16;
+};
+
+constexpr int PARAM_PS = 0, PARAM_SCALE = 1024, PARAM_BIAS = 2048;
+
+// issued by one wavefront in front of its first stage requests (loads retire in order, so they have landed when
+// stage 0 has); rows / columns past the matrix read as zero
+__device__ __forceinline__ void request_params(char *lds, int param_base, const float *pertoken, const float *scale, const void *bias,
+                                                int m0, int n0, int rows, int cols, int lane)
+{
+    const __amdgpu_buffer_rsrc_t r_ps = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(pertoken + m0), 0, rows * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t r_sc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(scale + n0), 0, cols * 4, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r_ps, (lds_void *)(lds + param_base + PARAM_PS), 16, (uint32_t)lane * 16u, 0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r_sc, (lds_void *)(lds + param_base + PARAM_SCALE), 16, (uint32_t)lane * 16u, 0, 0, 0);
+    if (bias) {
+        const __amdgpu_buffer_rsrc_t r_b =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(static_cast<const uint16_t *>(bias) + n0), 0, cols * 2, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r_b, (lds_void *)(lds + param_base + PARAM_BIAS), 16, (uint32_t)lane * 16u, 0, 0, 0);
+    }
+}
+
+template <int WTN, bool F16, bool BIAS>
+__device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
+{
+    using G = Geometry<WTN>;
+    constexpr int ROWB = WTN * 32 + 16;                       // padded pitch of a staged row: spreads rows over the banks
+    constexpr int CHUNKS = WTN * 2;                           // 16-byte chunks per row of the wavefront tile
+    const int wm = wave >> 1, wn = wave & 1;
+    const int mrow = lane & 15, nquad = (lane >> 4) * 4;
+    const char *par = lds + G::PARAM_BASE;
+    float ps[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) ps[i] = *reinterpret_cast<const float *>(par + PARAM_PS + (wm * 64 + i * 16 + mrow) * 4);
+    f32x4 sc[WTN], bs[WTN];
+#pragma unroll
+    for (int j = 0; j < WTN; j++) {
+        const int c = wn * WTN * 16 + j * 16 + nquad;
+        sc[j] = *reinterpret_cast<const f32x4 *>(par + PARAM_SCALE + c * 4);
+        if constexpr (BIAS) {
+            const u32x2 b2 = *reinterpret_cast<const u32x2 *>(par + PARAM_BIAS + c * 2);
+            bs[j] = f32x4{bf16_lo(b2.x), bf16_hi(b2.x), bf16_lo(b2.y), bf16_hi(b2.y)};
+        }
+    }
+    char *stg = lds + wave * (16 * ROWB);
+    const int mw = e.m0 + wm * 64, nw = e.n0 + wn * WTN * 16;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < WTN; j++) {
+            float f[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float v = (float)acc[i][j][r];
+                v = v * ps[i];
+                v = v * sc[j][r];
+                if constexpr (BIAS) v = v + bs[j][r];
+                f[r] = v;
+            }
+            u32x2 pk;
+            pk.x = F16 ? pack_f16x2(f[0], f[1]) : pack_bf16x2(f[0], f[1]);
+            pk.y = F16 ? pack_f16x2(f[2], f[3]) : pack_bf16x2(f[2], f[3]);
+            *reinterpret_cast<u32x2 *>(stg + mrow * ROWB + (j * 16 + nquad) * 2) = pk;
+        }
+#pragma unroll
+        for (int q0 = 0; q0 < 16 * CHUNKS; q0 += 64) {
+            const int q = q0 + lane;
+            const int row = q / CHUNKS, ch = q % CHUNKS;
+            if ((16 * CHUNKS) % 64 != 0 && row >= 16) continue;
+            const int m = mw + i * 16 + row, n = nw + ch * 8;
+            if (m >= e.M || n >= e.N) continue;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(stg + row * ROWB + ch * 16);
+            uint16_t *o = static_cast<uint16_t *>(e.out) + (int64_t)m * e.ldc + n;
+            if (n + 7 < e.N) {
+                *reinterpret_cast<u32x4 *>(o) = v;
+            } else {
+                for (int r = 0; r < 8; r++)
+                    if (n + r < e.N) o[r] = (uint16_t)(v[r >> 1] >> ((r & 1) * 16));
+            }
+        }
+    }
+}
+
+template <int WTN>
+__device__ __forceinline__ void epilogue_fast(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
+{
+    // output type and bias presence are resolved once per wavefront
+    if (e.out_f16) {
+        if (e.has_bias) epilogue_rows<WTN, true, true>(acc, lds, e, wave, lane);
+        else epilogue_rows<WTN, true, false>(acc, lds, e, wave, lane);
+    } else {
+        if (e.has_bias) epilogue_rows<WTN, false, true>(acc, lds, e, wave, lane);
+        else epilogue_rows<WTN, false, false>(acc, lds, e, wave, lane);
+    }
 }
 
 } // namespace wide

@@ -177,3 +177,37 @@ def test_gpu_reproduces_quantize_fixtures(capi):
     assert np.array_equal(qp.cpu().numpy(), f["qparam"])
     assert np.array_equal(pa.npu_quant_matmul(x1, x2, qp, bias=bias, output_dtype=torch.int8).cpu().numpy(), f["out"])
     assert np.array_equal(pa.npu_quant_matmul(x1, x2, scale, offset=offset, bias=bias).cpu().numpy(), f["out"])
+
+
+# The one part of npu_trans_quant_param's result that the reference tree does hold: the offset is a signed 9-bit
+# integer obtained by rounding (ties to even, numpy's round) and clipping to [-256, 255] -- the helper f32_2_s9 of
+# test/contrib/test_linear_weight_quant.py:13-16.  Inputs and the values that helper yields, typed by hand:
+_S9_IN = [0.0, 0.4, 0.5, 0.6, 1.5, 2.5, -0.5, -1.5, -2.5, 3.49, -3.51, 127.0, 128.0, 254.5, 255.0, 255.4, 255.5, 256.0, 300.0,
+          1e9, -255.5, -256.0, -256.5, -257.0, -300.0, -1e9, 7.0, -8.0]
+_S9_OUT = [0, 0, 0, 1, 2, 2, 0, -2, -2, 3, -4, 127, 128, 254, 255, 255, 255, 255, 255,
+           255, -256, -256, -256, -256, -256, -256, 7, -8]
+
+
+def test_trans_quant_param_offset_field_follows_f32_2_s9(golden):
+    """Pins the offset field of the packed parameter (rounding and range; the bit positions stay unpinned): decoding the
+    oracle's words gives f32_2_s9 of the offsets, and the field occupies nine bits."""
+    off = np.array(_S9_IN, dtype=np.float32)
+    want = np.array(_S9_OUT, dtype=np.float32)
+    q = golden.trans_quant_param(np.full(off.size, 0.5, dtype=np.float32), off)
+    scale, got = golden.quant_param_decode(q)
+    assert np.array_equal(got, want)
+    assert np.array_equal(scale, np.full(off.size, 0.5, dtype=np.float32))
+    # a second scale does not disturb the field, and without an offset the field is zero
+    assert np.array_equal(golden.quant_param_decode(golden.trans_quant_param(np.full(off.size, 3e-4, dtype=np.float32), off))[1], want)
+    assert np.array_equal(golden.quant_param_decode(golden.trans_quant_param(np.float32([0.5, 2.0])))[1], np.float32([0, 0]))
+    # nine bits: the extremes differ from each other only inside a 9-bit window
+    lo, hi = golden.trans_quant_param(np.float32([1.0]), np.float32([-256.0])), golden.trans_quant_param(np.float32([1.0]), np.float32([255.0]))
+    diff = int(lo.view(np.uint64)[0] ^ hi.view(np.uint64)[0])
+    assert diff != 0 and (diff >> (diff.bit_length() - 9)) == 0x1FF and diff.bit_length() - 9 == (diff & -diff).bit_length() - 1
+
+
+@pytest.mark.gpu
+def test_gpu_trans_quant_param_offset_field_follows_f32_2_s9(capi, golden):
+    off = torch.tensor(_S9_IN, dtype=torch.float32)
+    qp = capi.trans_quant_param(torch.full((off.numel(),), 0.5).cuda(), off.cuda()).cpu().numpy()
+    assert np.array_equal(golden.quant_param_decode(qp)[1], np.array(_S9_OUT, dtype=np.float32))

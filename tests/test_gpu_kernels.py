@@ -307,6 +307,80 @@ def test_quant_matmul_deep_ring_small_tiles(capi, golden, tile, M, K, N):
             capi.set_tuning(k, 0)
 
 
+@pytest.mark.parametrize("tile", [256192, 256224])
+@pytest.mark.parametrize("M,K,N", [(256, 128, 192), (300, 640, 500), (512, 4224, 1000), (1024, 1152, 2300), (255, 2048, 8 * 97)])
+def test_quant_matmul_wide_loop_tiles(capi, golden, tile, M, K, N):
+    """The 256-row tiles run the K loop with loader roles (activation slots released by an LDS flag between the two
+    wavefronts that read them).  One K step, odd and even step counts, ragged rows and columns, with and without a split of
+    K, both instruction orders: int32 accumulators bit-identical to the oracle, every epilogue (the LDS-parameter one for
+    per-token scale + bf16 bias / no bias in bf16 and fp16, and the general one for the other bias kinds, a single scale,
+    no per-token scale, int32 and re-quantised int8 outputs) bit-identical to the generic loop and to the oracle."""
+    d = workloads.quant_matmul_inputs(seed=M + N + K, M=M, K=K, N=N, weight_nk=True, bias=True)
+    g = torch.Generator().manual_seed(M + K)
+    x1, x2, sc, ps, bias = (d[k].cuda() for k in ("x1", "x2", "scale", "pertoken_scale", "bias"))
+    bias_i32 = torch.randint(-(1 << 20), 1 << 20, (N,), generator=g, dtype=torch.int32).cuda()
+    bias_f32 = torch.randn(N, generator=g).cuda()
+    one = torch.tensor([3e-3], device="cuda")
+    off = torch.randint(-20, 20, (N,), generator=g).float()
+    qp = capi.trans_quant_param((d["scale"] * 1e-2).cuda(), off.cuda())
+    acc_want = golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy())
+    want_bf16, _ = golden.quant_matmul(d["x1"].numpy(), d["x2"].numpy(), d["scale"].numpy(), d["pertoken_scale"].numpy(), _bits(d["bias"]))
+    want_i8 = golden.quant_matmul_requant(d["x1"].numpy(), d["x2"].numpy(), golden.trans_quant_param((d["scale"] * 1e-2).numpy(), off.numpy()),
+                                          bias_i32.cpu().numpy())
+
+    def run_all():
+        return [capi.quant_matmul(x1, x2, None, out_dtype=torch.int32),
+                capi.quant_matmul(x1, x2, sc, ps, bias),
+                capi.quant_matmul(x1, x2, sc, ps, None),
+                capi.quant_matmul(x1, x2, sc, ps, bias, out_dtype=torch.float16),
+                capi.quant_matmul(x1, x2, sc, ps, None, out_dtype=torch.float16),
+                capi.quant_matmul(x1, x2, sc, ps, bias_f32),
+                capi.quant_matmul(x1, x2, sc, ps, bias_i32),
+                capi.quant_matmul(x1, x2, sc, None, bias),
+                capi.quant_matmul(x1, x2, one, ps, bias),
+                capi.quant_matmul(x1, x2, None, None, bias_i32, out_dtype=torch.int32),
+                capi.quant_matmul_qparam(x1, x2, qp, bias_i32),
+                capi.quant_matmul_qparam(x1, x2, qp, None, out_dtype=torch.bfloat16)]
+
+    capi.set_tuning("MI355_QMM_TILE", tile)
+    try:
+        for split in (0, 2, 3):
+            if split and K // 128 < split:
+                continue
+            capi.set_tuning("MI355_QMM_SPLIT", split)
+            capi.set_tuning("MI355_QMM_LOOP", 1)            # the generic loop on the same tile
+            ref = run_all()
+            assert np.array_equal(ref[0].cpu().numpy(), acc_want), (tile, split)
+            assert np.array_equal(_bits(ref[1]), want_bf16), (tile, split)
+            assert np.array_equal(ref[10].cpu().numpy(), want_i8), (tile, split)
+            for order in (2, 3):
+                capi.set_tuning("MI355_QMM_LOOP", order)
+                got = run_all()
+                for i, (a, b) in enumerate(zip(got, ref)):
+                    assert torch.equal(a, b), (tile, split, order, i)
+    finally:
+        for k in ("MI355_QMM_TILE", "MI355_QMM_SPLIT", "MI355_QMM_LOOP"):
+            capi.set_tuning(k, 0)
+
+
+def test_quant_matmul_wide_loop_strided_operands(capi, golden):
+    """Row pitches larger than the rows (views into wider buffers) and an output view whose rows are not 16-byte aligned
+    (the general epilogue): the wide loop addresses rows through the pitches only."""
+    M, K, N = 512, 1024, 384
+    d = workloads.quant_matmul_inputs(seed=5, M=M, K=K, N=N, weight_nk=True, bias=True)
+    xa = torch.zeros((M, K + 256), dtype=torch.int8, device="cuda")
+    xa[:, :K] = d["x1"].cuda()
+    wb = torch.zeros((N, K + 128), dtype=torch.int8, device="cuda")
+    wb[:, :K] = d["x2"].t().cuda()
+    want, _ = golden.quant_matmul(d["x1"].numpy(), d["x2"].numpy(), d["scale"].numpy(), d["pertoken_scale"].numpy(), _bits(d["bias"]))
+    capi.set_tuning("MI355_QMM_TILE", 256192)
+    try:
+        out = capi.quant_matmul(xa[:, :K], wb[:, :K].t(), d["scale"].cuda(), d["pertoken_scale"].cuda(), d["bias"].cuda())
+        assert np.array_equal(_bits(out), want)
+    finally:
+        capi.set_tuning("MI355_QMM_TILE", 0)
+
+
 def test_quant_matmul_split_k_repeated_launches(capi, golden):
     """A narrow output with a long K is split over K (workgroups meet at counters in the shared workspace): the
     down-projection shape of the MLP configuration, launched repeatedly on the same zero-initialised workspace."""

@@ -598,6 +598,26 @@ def test_c5_mlp_prefill_properties(pa, golden):
     assert torch.equal(full[rows.cuda()], part)
 
 
+def test_c5_mlp_prefill_stagewise_oracle(pa, golden):
+    """M = 2048 against the oracle: every stage works row by row, so the oracle is applied, stage by stage, to a sample of
+    128 rows of the GPU's own stage inputs that touches every 256-row tile (the plans this size selects: the 256x224 tile
+    for gate|up, a 256x256 tile with K split in two for the down projection).  Quantisations and both GEMMs bit-exact,
+    SwiGLU within one bf16 ulp."""
+    d = workloads.mlp_inputs(seed=1, M=2048)
+    rows = torch.cat([torch.arange(0, 2048, 32) + 3, torch.arange(0, 2048, 32) + 29]).sort().values
+    xq, xs, gu, act, aq, as_, out = (t.cpu()[rows] for t in _mlp_gpu(pa, d))
+    yg, sg = golden.dynamic_quant(_bits(d["x"][rows]))
+    assert np.array_equal(xq.numpy(), yg) and np.array_equal(xs.numpy(), sg)
+    want, _ = golden.quant_matmul(xq.numpy(), d["w_gate_up"].t().numpy(), d["scale_gate_up"].numpy(), xs.numpy())
+    assert np.array_equal(_bits(gu), want)
+    dist = golden.bf16_ulp_distance(_bits(act), golden.swiglu(_bits(gu)))
+    assert dist.max() <= 1 and (dist == 0).mean() > 0.995
+    yg, sg = golden.dynamic_quant(_bits(act))
+    assert np.array_equal(aq.numpy(), yg) and np.array_equal(as_.numpy(), sg)
+    want, _ = golden.quant_matmul(aq.numpy(), d["w_down"].t().numpy(), d["scale_down"].numpy(), as_.numpy())
+    assert np.array_equal(_bits(out), want)
+
+
 def test_prepare_weight_quant_weight(pa):
     """An int8 weight contiguous along N is rewritten once into the contrib module's storage ([N, K], passed as its
     transposed view): equal values, strides (1, K), the operator's result within the gate of the unprepared call's;
