@@ -13,7 +13,9 @@
  *     arguments on the host, enqueues kernels on `stream` (a hipStream_t passed as void*,
  *     NULL = the default stream) and returns;
  *   - return value: MI355_OK (0) or a negative mi355_status; mi355_status_string() names it;
- *   - re-entrant; no mutable global state.
+ *   - launches are re-entrant and keep no state between calls, with three documented exceptions: the planner knobs of
+ *     mi355_set_tuning() are process-wide, mi355_quant_matmul_noalloc() works on one scratch array per GPU, and
+ *     mi355_workspace_status() is a query that synchronises the stream it is given.
  *   - strides ("ld*", "*_stride") are in ELEMENTS of the respective array.
  */
 #ifndef MI355_QUANT_H
@@ -32,7 +34,8 @@ typedef enum mi355_status {
     MI355_ERR_UNSUPPORTED = -2,    /* valid request outside what the kernels implement     */
     MI355_ERR_ALIGNMENT = -3,      /* pointer / stride alignment the kernels cannot handle */
     MI355_ERR_WORKSPACE = -4,      /* workspace missing or smaller than *_workspace() says */
-    MI355_ERR_LAUNCH = -5          /* hipGetLastError() != hipSuccess after the launch     */
+    MI355_ERR_LAUNCH = -5,         /* hipGetLastError() != hipSuccess after the launch     */
+    MI355_ERR_DEVICE = -6          /* a kernel reported a failure through the workspace's status word (mi355_workspace_status) */
 } mi355_status;
 
 /* 16-bit floating-point element formats of activations. */
@@ -115,6 +118,26 @@ int mi355_dynamic_quant_asymmetric(const void *x, int in_dtype, const void *smoo
  *              launches of all operators on the same stream.
  */
 #define MI355_WORKSPACE_ZERO_BYTES ((size_t)16 * 1024 * 1024 + 16384)
+/* The same number as a query, for hosts that bind the library without this header. */
+size_t mi355_workspace_zero_bytes(void);
+
+/*
+ * Device-side failures.  The reference reports a failed device task to the caller at the next synchronisation
+ * (torch_npu/csrc/framework/OpParamMaker.cpp:541-571); here the only failure a kernel can detect is a bounded wait
+ * running out: the int4 kernels of mi355_weight_quant_matmul exchange split-K partial sums through the workspace's
+ * zero zone, and the workgroup that collects them polls a bounded number of times.  When the bound is hit the kernel
+ * writes NaN where the missing sums would have gone and stores a non-zero code in the workspace's sticky status word
+ * (4 bytes at MI355_WORKSPACE_STATUS_OFFSET, inside the zero area); later stores of the late producers may leave
+ * non-zero words in the zone, so the zone must be cleared before the workspace is used again.
+ *
+ * mi355_workspace_status waits for `stream`, reads the status word and returns MI355_OK when it is zero, MI355_ERR_DEVICE
+ * otherwise.  With `reset` non-zero a failed workspace is made usable again: its whole zero area, the status word
+ * included, is cleared on `stream` before the call returns.  Unlike the launchers this call synchronises; call it where
+ * the caller synchronises anyway, or before a workspace is retired.
+ */
+#define MI355_WORKSPACE_STATUS_OFFSET ((size_t)16384 - 16)
+int mi355_workspace_status(void *workspace, size_t workspace_bytes, int reset, void *stream);
+
 size_t mi355_quant_matmul_workspace(int64_t M, int64_t N, int64_t K, int64_t ldb_k, int64_t ldb_n);
 
 int mi355_quant_matmul(const int8_t *a, const int8_t *b,
@@ -180,7 +203,10 @@ int mi355_transpose_int8(const int8_t *src, int8_t *dst, int64_t K, int64_t N, i
  *     them; integer sums make the results identical); returns MI355_ERR_WORKSPACE when the transposed copy of a
  *     weight stored [K,N] does not fit (store it [N,K], or use mi355_quant_matmul);
  *   - calls no hipMalloc / hipFree and no allocating library routine; the first call on a device resolves the
- *     array's address and clears its counters with a small kernel on `stream`;
+ *     array's address and clears its counters with a small kernel on `stream` (recorded again by every capturing call
+ *     until a call outside a capture has enqueued it);
+ *   - the array belongs to the current device: `stream` must be NULL or a stream of the current device
+ *     (MI355_ERR_BAD_ARGUMENT otherwise);
  *   - all calls on one GPU share that GPU's array: calls that may overlap in time (different streams without an
  *     ordering between them, several host threads) race on it and must be serialised by the caller.
  */

@@ -44,3 +44,19 @@ _export_npu_ops()
 from . import contrib  # noqa: E402,F401
 from . import flops  # noqa: E402,F401  (registers the FLOP formulas of the matmul operators)
 from .prepare import prepare_quant_matmul_weight, prepare_weight_quant_weight  # noqa: E402,F401
+
+
+def check_device_status() -> None:
+    """Waits for the streams the operators have launched on and raises RuntimeError if a kernel reported a failure
+    through the status word of its workspace (a bounded wait for another workgroup's partial sums ran out; the outputs of
+    that launch hold NaN).  The workspaces concerned are cleared, so the operators can be used again afterwards.  The
+    reference reports device-side failures the same way, at the caller's next synchronisation
+    (torch_npu/csrc/framework/OpParamMaker.cpp:541-571)."""
+    import ctypes as _ctypes
+    failures = _ctypes.CDLL(OPS_LIBRARY).mi355_npu_check_workspaces()
+    if failures:
+        raise RuntimeError(f"mi355: {failures} workspace(s) hold a device-side failure report (a bounded wait for split-K "
+                           "partial sums ran out; the outputs of that launch hold NaN); the workspaces have been cleared")
+
+
+__all__.append("check_device_status")

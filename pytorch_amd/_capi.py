@@ -19,7 +19,8 @@ EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quan
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
            "mi355_trans_quant_param", "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth", "mi355_set_tuning",
-           "mi355_quant_matmul_noalloc", "mi355_stream_capture_id", "mi355_probe_clock", "mi355_device_info", "mi355_transpose_int8", "mi355_probe_empty_launch")
+           "mi355_quant_matmul_noalloc", "mi355_stream_capture_id", "mi355_probe_clock", "mi355_device_info", "mi355_transpose_int8", "mi355_probe_empty_launch",
+           "mi355_workspace_status", "mi355_workspace_zero_bytes")
 
 _lib = None
 
@@ -62,6 +63,8 @@ def lib() -> ctypes.CDLL:
         L.mi355_device_info.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.mi355_stream_capture_id.argtypes = [vp, ctypes.POINTER(ctypes.c_ulonglong)]
         L.mi355_quant_matmul_noalloc.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp]
+        L.mi355_workspace_status.argtypes = [vp, sz, i32, vp]
+        L.mi355_workspace_zero_bytes.restype = sz
         _lib = L
     return _lib
 
@@ -188,7 +191,21 @@ def quant_matmul_qparam(x1, x2, qparam, bias=None, out_dtype=torch.int8, workspa
 _wq_workspaces = {}
 _wq_capture_workspaces = {}
 _wq_retired = []        # superseded workspaces stay alive: a captured graph may still hold their address
-ZERO_AREA_BYTES = (16 << 20) + 16384     # MI355_WORKSPACE_ZERO_BYTES
+ZERO_AREA_BYTES = (16 << 20) + 16384     # MI355_WORKSPACE_ZERO_BYTES (checked against the library when it loads a workspace)
+
+
+def workspace_status(ws, reset: bool = True) -> None:
+    """Waits for the current stream and raises Mi355Error if a kernel reported a failure through the sticky status word
+    of workspace `ws` (a bounded wait for split-K partial sums ran out; the affected outputs hold NaN).  With `reset` the
+    workspace's zero area is cleared so that it can be used again."""
+    _check(lib().mi355_workspace_status(_ptr(ws), ws.numel(), 1 if reset else 0, _stream()), "mi355_workspace_status")
+
+
+def check_workspaces(reset: bool = True) -> None:
+    """workspace_status() for every workspace this module keeps for eager calls (one per device and stream)."""
+    for ws in list(_wq_workspaces.values()) + list(_wq_retired):
+        with torch.cuda.device(ws.device):
+            workspace_status(ws, reset)
 
 
 def _wq_workspace(device, nbytes: int):
@@ -214,7 +231,10 @@ def _wq_workspace(device, nbytes: int):
     ws = _wq_workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         if ws is not None:
+            workspace_status(ws)                   # a failure reported into the outgrown buffer must not be lost
             _wq_retired.append(ws)
+            want = max(want, 2 * ws.numel())       # geometric growth: a stream retires a bounded number of buffers
+        assert lib().mi355_workspace_zero_bytes() == ZERO_AREA_BYTES
         ws = torch.zeros(want, dtype=torch.int8, device=device)
         _wq_workspaces[key] = ws
     return ws

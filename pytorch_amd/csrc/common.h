@@ -61,6 +61,12 @@ __device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2)
 // (split-K partial sums, a transposed weight) lies behind it and needs no initialisation, so one zero-initialised
 // buffer can be shared by all launches of a stream.
 constexpr size_t kWorkspaceCounterCapacity = 16384;
+// The last 16 bytes of the counter part are not counters: the first word of them is the workspace's sticky status word
+// (MI355_WORKSPACE_STATUS_OFFSET).  A kernel whose bounded wait for another workgroup's partial sums ran out stores a
+// non-zero code there (and NaNs where its sums should be); mi355_workspace_status() reads and clears it.
+constexpr size_t kWorkspaceStatusOffset = kWorkspaceCounterCapacity - 16;
+constexpr size_t kWorkspaceCounterBytes = kWorkspaceStatusOffset;      // what planners may fill with arrival counters
+constexpr uint32_t kStatusExchangeTimeout = 1;
 constexpr size_t kWorkspaceZoneBytes = (size_t)16 << 20;
 constexpr size_t kWorkspaceZeroBytes = kWorkspaceCounterCapacity + kWorkspaceZoneBytes;
 
@@ -78,9 +84,12 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
 // MI355_WQ_GEMM4_OFF / MI355_WQ_DECODE_OFF: 1 = the register-expanding int4 GEMM / the int4 decode kernel is not used;
 // 2 = its K-split exchange always writes through to memory.
 // MI355_QMM_DECODE_OFF: 1 = quant_matmul with at most 64 rows takes the tiled kernel instead of the decode kernel.
+// MI355_WQ_MAX_POLLS: bound of the int4 kernels' wait for the other workgroups' partial sums (0 = 2^20 polls);
+// MI355_WQ_ONLY_CHUNK: c + 1 = only the workgroups of K chunk c do anything, -1 = only the collecting chunk (with a small MI355_WQ_MAX_POLLS this drives
+// a collector into its give-up path from the host, every kernel still ending normally: tests of the error reporting).
 enum Knob { kKnobWqSplit, kKnobWqW, kKnobWqgSplit, kKnobWqgBm, kKnobWqGemmOff, kKnobWqkMt, kKnobWqkNw, kKnobWqkKs,
             kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmDeepOff, kKnobWqGemm4Off, kKnobQmmDecodeOff,
-            kKnobQmmLoop, kKnobCount };
+            kKnobQmmLoop, kKnobWqMaxPolls, kKnobWqOnlyChunk, kKnobCount };
 int knob(Knob k);
 
 inline int check_launch()

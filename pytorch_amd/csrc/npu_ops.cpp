@@ -184,38 +184,67 @@ std::tuple<Tensor, Tensor, Tensor> dynamic_quant_asym_hip(const Tensor &input, c
 //     exactly as long as the graph.  Such a buffer is never handed to an eager call or to another capture; the cache
 //     drops its reference when it sees the next capture (or an eager call) on that stream, which returns the block
 //     to the pool of the graph that owns it.
-Tensor zeroed_workspace(const Tensor &like, size_t bytes)
-{
+struct WorkspaceCache {
     struct Captured {
         unsigned long long id = 0;
         Tensor ws;
     };
-    static std::mutex mu;
-    static std::map<std::pair<int, void *>, Tensor> cache;
-    static std::map<std::pair<int, void *>, Captured> capture_cache;
-    static std::vector<Tensor> *retired = new std::vector<Tensor>();   // intentionally never freed
-    std::lock_guard<std::mutex> lock(mu);
+    std::mutex mu;
+    std::map<std::pair<int, void *>, Tensor> eager;
+    std::map<std::pair<int, void *>, Captured> captured;
+    std::vector<std::pair<std::pair<int, void *>, Tensor>> retired;       // never freed: an earlier graph may point into them
+};
+
+WorkspaceCache &workspace_cache()
+{
+    static WorkspaceCache *c = new WorkspaceCache();                      // intentionally never destroyed
+    return *c;
+}
+
+// A kernel that gave up waiting for partial sums has said so in the workspace's status word (and put NaN where the sums
+// belonged).  Reading the word needs the stream to drain, so it is read where that costs nothing extra: before a
+// workspace is retired, and on request (mi355_npu_check_workspaces, pytorch_amd.check_device_status()), the way the
+// reference reports a failed device task at the caller's next synchronisation (OpParamMaker.cpp:541-571).
+void check_workspace(const Tensor &ws, void *stream, const char *when)
+{
+    const int st = mi355_workspace_status(ws.data_ptr(), (size_t)ws.numel(), 1, stream);
+    TORCH_CHECK(st == MI355_OK, "mi355: ", mi355_status_string(st), " (found ", when,
+                "; the outputs of that launch hold NaN, the workspace has been cleared and is usable again)");
+}
+
+Tensor zeroed_workspace(const Tensor &like, size_t bytes)
+{
+    WorkspaceCache &wc = workspace_cache();
+    std::lock_guard<std::mutex> lock(wc.mu);
     const auto key = std::make_pair((int)like.device().index(), stream_of(like));
-    const int64_t want = (int64_t)std::max<size_t>(bytes, (size_t)MI355_WORKSPACE_ZERO_BYTES + ((size_t)1 << 20));
+    int64_t want = (int64_t)std::max<size_t>(bytes, (size_t)MI355_WORKSPACE_ZERO_BYTES + ((size_t)1 << 20));
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     unsigned long long capture_id = 0;
     TORCH_CHECK(hipStreamGetCaptureInfo(static_cast<hipStream_t>(key.second), &capturing, &capture_id) == hipSuccess,
                 "hipStreamGetCaptureInfo failed");
     if (capturing != hipStreamCaptureStatusNone) {
-        const auto eager = cache.find(key);
-        if (eager != cache.end() && eager->second.defined() && (size_t)eager->second.numel() >= bytes) return eager->second;
-        Captured &c = capture_cache[key];
+        const auto eager = wc.eager.find(key);
+        if (eager != wc.eager.end() && eager->second.defined() && (size_t)eager->second.numel() >= bytes) return eager->second;
+        WorkspaceCache::Captured &c = wc.captured[key];
         if (!c.ws.defined() || c.id != capture_id || (size_t)c.ws.numel() < bytes) {
             c.ws = at::zeros({want}, like.options().dtype(at::kChar));      // the fill is recorded into this capture
             c.id = capture_id;
         }
         return c.ws;
     }
-    capture_cache.erase(key);
-    Tensor &ws = cache[key];
+    wc.captured.erase(key);
+    Tensor &ws = wc.eager[key];
     if (!ws.defined() || (size_t)ws.numel() < bytes) {
-        if (ws.defined()) retired->push_back(ws);
-        ws = at::zeros({want}, like.options().dtype(at::kChar));
+        if (ws.defined()) {
+            // geometric growth bounds the buffers a stream can retire (a handful between 17 MiB and the largest problem)
+            want = std::max<int64_t>(want, 2 * ws.numel());
+            Tensor old = ws;
+            wc.retired.emplace_back(key, old);
+            ws = at::zeros({want}, like.options().dtype(at::kChar));
+            check_workspace(old, key.second, "when its workspace was outgrown");
+        } else {
+            ws = at::zeros({want}, like.options().dtype(at::kChar));
+        }
     }
     return ws;
 }
@@ -875,4 +904,24 @@ TORCH_LIBRARY_IMPL(npu, Meta, m)
     m.impl("npu_anti_quant", TORCH_FN(anti_quant_meta));
     m.impl("npu_quantize", TORCH_FN(quantize_meta));
     m.impl("npu_trans_quant_param", TORCH_FN(trans_quant_param_meta));
+}
+
+// Reads the status word of every workspace kept for eager launches (synchronises their streams); throws c10::Error if a
+// kernel reported a failure.  Exported with C linkage for the Python package (pytorch_amd.check_device_status()).
+extern "C" int mi355_npu_check_workspaces(void)
+{
+    WorkspaceCache &wc = workspace_cache();
+    std::vector<std::pair<std::pair<int, void *>, Tensor>> all;
+    {
+        std::lock_guard<std::mutex> lock(wc.mu);
+        for (auto &kv : wc.eager)
+            if (kv.second.defined()) all.emplace_back(kv.first, kv.second);
+        for (auto &kv : wc.retired) all.push_back(kv);
+    }
+    int failures = 0;
+    for (auto &kv : all) {
+        c10::hip::HIPGuardMasqueradingAsCUDA guard(kv.second.device());
+        if (mi355_workspace_status(kv.second.data_ptr(), (size_t)kv.second.numel(), 1, kv.first.second) != MI355_OK) failures++;
+    }
+    return failures;
 }

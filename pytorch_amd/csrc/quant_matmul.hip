@@ -923,7 +923,12 @@ void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size
             const int64_t wgs = tiles * s_eff;
             // a caller with a fixed scratch area (mi355_quant_matmul_noalloc) only gets splits whose partial sums fit it
             // ... and nobody gets more than 128 MiB of them
-            if (s_eff > 1 && s_eff == S && (uint64_t)wgs * c.bm * c.bn * 4 > (partial_cap < kMaxPartialBytes ? partial_cap : kMaxPartialBytes)) continue;
+            // (a split forced through the knob is bound by a fixed scratch area too, and no split may need more arrival
+            // counters than the workspace holds)
+            if (s_eff > 1 && (s_eff == S || partial_cap < kMaxPartialBytes) &&
+                (uint64_t)wgs * c.bm * c.bn * 4 > (partial_cap < kMaxPartialBytes ? partial_cap : kMaxPartialBytes))
+                continue;
+            if (s_eff > 1 && (uint64_t)tiles * 4 > kWorkspaceCounterBytes) continue;
             const int64_t rounds = (wgs + c.slots - 1) / c.slots;
             const double at_4096 = rounds == 1 ? c.single_us : (double)rounds * c.round_us;
             double loop_us = (at_4096 - kBaseUs) * ((double)kt / s_eff) / 32.0;
@@ -1114,10 +1119,10 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     if (c.bm == bm_ && c.bn == bn_) return launch_qmm<wgm_, wgn_, bm_ / (16 * wgm_), bn_ / (16 * wgn_)>(p, s);
     MI355_QMM_CASE(256, 256, 2, 4)
     {
-        const int lk = knob(kKnobQmmLoop);                 // 0: automatic; 1: the generic loop; 2, 3: the wide loop's instruction orders
+        const int lk = knob(kKnobQmmLoop);                 // 0: automatic; 1: the generic loop; 2, 3: the wide loop with refills in a block / spread
         if (lk != 1) {
-            if (c.bm == 256 && c.bn == 224) return lk == 3 ? launch_qmm<4, 2, 4, 7, 0, 2>(p, s) : launch_qmm<4, 2, 4, 7, 0, 1>(p, s);
-            if (c.bm == 256 && c.bn == 192) return lk == 3 ? launch_qmm<4, 2, 4, 6, 0, 2>(p, s) : launch_qmm<4, 2, 4, 6, 0, 1>(p, s);
+            if (c.bm == 256 && c.bn == 224) return lk == 2 ? launch_qmm<4, 2, 4, 7, 0, 1>(p, s) : launch_qmm<4, 2, 4, 7, 0, 2>(p, s);
+            if (c.bm == 256 && c.bn == 192) return lk == 2 ? launch_qmm<4, 2, 4, 6, 0, 1>(p, s) : launch_qmm<4, 2, 4, 6, 0, 2>(p, s);
         }
     }
     MI355_QMM_CASE(256, 224, 4, 2)
@@ -1215,16 +1220,29 @@ int scratch_of_current_device(void **out, hipStream_t s)
 {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MI355_ERR_LAUNCH;
+    // the array's address is resolved for the current device: a stream of another device cannot use it
+    if (s) {
+        int sdev = -1;
+        if (hipStreamGetDevice(s, &sdev) != hipSuccess) return MI355_ERR_LAUNCH;
+        if (sdev != dev) return MI355_ERR_BAD_ARGUMENT;
+    }
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     DeviceScratch &d = g_scratch[dev];
-    if (!d.ready) {
+    if (!d.ptr) {
         void *ptr = nullptr;
         if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return MI355_ERR_LAUNCH;
-        hipLaunchKernelGGL(scratch_clear_kernel, dim3((unsigned)(kWorkspaceCounterCapacity / 4 / 256)), dim3(256), 0, s,
-                           static_cast<uint32_t *>(ptr), (int)(kWorkspaceCounterCapacity / 4));
-        if (check_launch() != MI355_OK) return MI355_ERR_LAUNCH;
         d.ptr = ptr;
-        d.ready = true;
+    }
+    if (!d.ready) {
+        // A __device__ array starts out zeroed and every launch leaves the counters zero, so this clear only guards
+        // against a process that wrote to the array by other means.  While the stream is capturing the kernel is merely
+        // recorded, so the array does not count as cleared until a call outside a capture has enqueued the clear.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &capturing) != hipSuccess) return MI355_ERR_LAUNCH;
+        hipLaunchKernelGGL(scratch_clear_kernel, dim3((unsigned)(kWorkspaceCounterCapacity / 4 / 256)), dim3(256), 0, s,
+                           static_cast<uint32_t *>(d.ptr), (int)(kWorkspaceCounterCapacity / 4));
+        if (check_launch() != MI355_OK) return MI355_ERR_LAUNCH;
+        if (capturing == hipStreamCaptureStatusNone) d.ready = true;
     }
     *out = d.ptr;
     return MI355_OK;

@@ -69,8 +69,9 @@ extern "C" const char *mi355_status_string(int status)
     case MI355_ERR_ALIGNMENT: return "pointer or stride alignment not supported";
     case MI355_ERR_WORKSPACE: return "workspace missing or too small";
     case MI355_ERR_LAUNCH: return "kernel launch failed";
+    case MI355_ERR_DEVICE: return "a kernel reported a failure through the workspace status word (a bounded wait for partial sums ran out)";
     default: return "unknown status";
     }
 }
 
-extern "C" int mi355_quant_abi_version(void) { return 2300; }
+extern "C" int mi355_quant_abi_version(void) { return 3000; }

@@ -11,7 +11,7 @@ namespace {
 const char *const kKnobNames[kKnobCount] = {"MI355_WQ_SPLIT", "MI355_WQ_W",    "MI355_WQG_SPLIT", "MI355_WQG_BM",   "MI355_WQ_GEMM_OFF",
                                             "MI355_WQK_MT",   "MI355_WQK_NW",  "MI355_WQK_KS",    "MI355_QMM_SPLIT", "MI355_QMM_TILE",
                                             "MI355_WQ_DECODE_OFF", "MI355_QMM_DEEP_OFF", "MI355_WQ_GEMM4_OFF",
-                                            "MI355_QMM_DECODE_OFF", "MI355_QMM_LOOP"};
+                                            "MI355_QMM_DECODE_OFF", "MI355_QMM_LOOP", "MI355_WQ_MAX_POLLS", "MI355_WQ_ONLY_CHUNK"};
 std::atomic<int> g_knobs[kKnobCount];
 const bool g_knobs_loaded = []() {
     for (int i = 0; i < kKnobCount; i++) {
@@ -52,4 +52,26 @@ extern "C" int mi355_stream_capture_id(void *stream, unsigned long long *id)
     if (hipStreamGetCaptureInfo(static_cast<hipStream_t>(stream), &status, &cid) != hipSuccess) return MI355_ERR_LAUNCH;
     *id = status == hipStreamCaptureStatusNone ? 0ull : cid;
     return MI355_OK;
+}
+
+extern "C" size_t mi355_workspace_zero_bytes(void) { return mi355::kWorkspaceZeroBytes; }
+
+// The sticky status word of a workspace (common.h): read it once the stream has drained; with `reset`, clear the whole zero
+// area of a workspace that reported a failure, because late stores of the producers the collector gave up on may have
+// left non-zero words in the exchange zone.
+extern "C" int mi355_workspace_status(void *workspace, size_t workspace_bytes, int reset, void *stream)
+{
+    using namespace mi355;
+    if (!workspace || workspace_bytes < kWorkspaceCounterCapacity) return MI355_ERR_BAD_ARGUMENT;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint32_t word = 0;
+    if (hipMemcpyAsync(&word, static_cast<char *>(workspace) + kWorkspaceStatusOffset, sizeof(word), hipMemcpyDeviceToHost, s) != hipSuccess)
+        return MI355_ERR_LAUNCH;
+    if (hipStreamSynchronize(s) != hipSuccess) return MI355_ERR_LAUNCH;
+    if (word == 0) return MI355_OK;
+    if (reset) {
+        const size_t n = workspace_bytes < kWorkspaceZeroBytes ? workspace_bytes : kWorkspaceZeroBytes;
+        if (hipMemsetAsync(workspace, 0, n, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess) return MI355_ERR_LAUNCH;
+    }
+    return MI355_ERR_DEVICE;
 }

@@ -13,8 +13,10 @@
 //     reads the words back with agent-scope loads until none is zero, adds them in chunk order to its own sum,
 //     writes the output and stores the zeros back.  The critical path after the last weight byte is one store, one
 //     load and the output store; the relaxed agent-scope counter it replaces cost an acknowledged store, an atomic
-//     round trip and a load.  The wait is bounded: after kMaxPolls unanswered polls the workgroup gives up (the
-//     output is then wrong, the launch still ends).
+//     round trip and a load.  The wait is bounded: after max_polls unanswered polls a thread gives up, stores NaN where
+//     its sums should be and sets the workspace's sticky status word, which mi355_workspace_status() reports to the host
+//     (the launch still ends).  The order of dispatch that the scheme leans on - a strip's highest workgroup index
+//     starts last - is what the hardware does today, not a guarantee; the bound and the status word are the net.
 #include "weight_quant_common.h"
 #include "weight_quant_decode.h"
 
@@ -32,6 +34,9 @@ struct WqDecArgs {
     int group_rows;                 // rows of a scale group (K when per channel)
     int strips, S;
     int l2_exchange;                // producers on the collector's XCD leave their sums in the L2
+    int max_polls;                  // bound of the collector's wait
+    int only_chunk;                 // testing aid: c + 1 = only the workgroups of chunk c run
+    uint32_t *status;               // the workspace's sticky status word
 };
 
 constexpr int kMaxPolls = 1 << 20;
@@ -55,6 +60,7 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
     const int xcd_slot = blockIdx.x >> 3;
     const int strip = (blockIdx.x & 7) + 8 * (xcd_slot / p.S), chunk = xcd_slot % p.S;
     if (strip >= p.strips) return;
+    if (p.only_chunk && chunk != (p.only_chunk < 0 ? p.S - 1 : p.only_chunk - 1)) return;      // testing aid (host-driven give-up of the collector)
     // The chunks of a strip sit on one XCD.  The collector says on which it runs (a word per strip behind the sums); a
     // producer that finds itself there leaves its sums in the shared L2 with ordinary stores, which the collector's polls
     // (they bypass the vector L1) see a microsecond before stores that write through to memory.
@@ -261,6 +267,7 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
         // the strip's last workgroup collects the other chunks in chunk order; all of a thread's requests go out
         // before the first answer is looked at
         f32x4 sum[NQ];
+        bool gave_up = false;
 #pragma unroll
         for (int e = 0; e < NQ; e++) sum[e] = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int c0 = 0; c0 < p.S - 1; c0 += CB) {
@@ -273,8 +280,9 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
                                       ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[e], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1)
                                       : u32x4{1u, 1u, 1u, 1u};
             }
-            for (int poll = 0; poll < kMaxPolls; poll++) {
-                bool missing = false;
+            bool missing = true;
+            for (int poll = 0; poll < p.max_polls && missing; poll++) {
+                missing = false;
                 // the polls must be real loads: without a compiler barrier a reload with the operands of the first request is
                 // folded into it, and a wavefront that arrived before the data would spin on a stale register until the bound
                 asm volatile("" ::: "memory");
@@ -286,8 +294,8 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
                             v[e][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, zoff[e], (uint32_t)(c0 + i) * zone_chunk_bytes, SC1);
                             missing = true;
                         }
-                if (!missing) break;
             }
+            gave_up = gave_up || missing;
 #pragma unroll
             for (int i = 0; i < CB; i++)
 #pragma unroll
@@ -298,6 +306,13 @@ __global__ __launch_bounds__(512) void wq_decode4_kernel(const WqDecArgs p)
         }
 #pragma unroll
         for (int e = 0; e < NQ; e++) acc[e] = sum[e] + acc[e];
+        if (gave_up) {
+            // some partial sums never came: the result is marked (NaN), not guessed, and the host is told
+            const float nan = __uint_as_float(0x7fc00000u);
+#pragma unroll
+            for (int e = 0; e < NQ; e++) acc[e] = f32x4{nan, nan, nan, nan};
+            *p.status = kStatusExchangeTimeout;
+        }
     }
     const bool out_vec = (p.ldo & 3) == 0 && aligned_dev(p.out, 8);
 #pragma unroll
@@ -384,6 +399,9 @@ int launch_wq_decode(const WqDecodePlan &plan, const void *x, int act_f16, const
     p.strips = plan.strips;
     p.S = plan.S;
     p.l2_exchange = knob(kKnobWqDecodeOff) != 2;
+    p.max_polls = knob(kKnobWqMaxPolls) > 0 ? knob(kKnobWqMaxPolls) : kMaxPolls;
+    p.only_chunk = knob(kKnobWqOnlyChunk);
+    p.status = plan.S > 1 ? reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kWorkspaceStatusOffset) : nullptr;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int rows = (int)(M < 16 ? M : 16);
     const size_t lds_bytes = (size_t)8 * rows * 256 * sizeof(float);

@@ -520,7 +520,7 @@ WqGemmPlan make_wq_gemm_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_
     if (S > 8) S = 8;
     if (const int f = knob(kKnobWqgSplit))              // tuning aid
         if (f >= 1 && f <= pl.n_units) S = f;
-    if (S > 1 && ((uint64_t)S * pl.bm * bn * 4 >= (1ull << 32) || (size_t)tiles * 4 > kWorkspaceCounterCapacity)) S = 1;
+    if (S > 1 && ((uint64_t)S * pl.bm * bn * 4 >= (1ull << 32) || (size_t)tiles * 4 > kWorkspaceCounterBytes)) S = 1;
     pl.S = (int)S;
     pl.accum = pl.grouped && (pl.n_units + pl.S - 1) / pl.S > 1;
     pl.partial_bytes = pl.S > 1 ? (size_t)tiles * pl.S * pl.bm * bn * 4 : 0;

@@ -46,6 +46,9 @@ struct WqGemm4Args {
     int grouped;
     int tiles_m, strips, S;
     int l2_exchange;                // producers on the collector's XCD leave their sums in the L2
+    int max_polls;                  // bound of the collector's wait
+    int only_chunk;                 // testing aid: c + 1 = only the workgroups of chunk c run
+    uint32_t *status;               // the workspace's sticky status word
 };
 
 constexpr int kMaxPolls4 = 1 << 20;
@@ -81,6 +84,7 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
     const int j = xcd_slot / p.S, chunk = xcd_slot % p.S;
     const int strip = (blockIdx.x & 7) + 8 * (j / p.tiles_m);
     if (strip >= p.strips) return;
+    if (p.only_chunk && chunk != (p.only_chunk < 0 ? p.S - 1 : p.only_chunk - 1)) return;      // testing aid (host-driven give-up of the collector)
     const int mb = j % p.tiles_m;
     const int tile = strip * p.tiles_m + mb;
     const int m0 = mb * BM;
@@ -408,7 +412,7 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         }
         // the sums of up to CB chunks are asked for together and added in chunk order: ((c0 + c1) + ...) + own
         constexpr int CB = 3;
-        bool first = true;
+        bool first = true, gave_up = false;
         for (int c0 = 0; c0 < p.S - 1; c0 += CB) {
             u32x4 v[CB][NE];
 #pragma unroll
@@ -417,8 +421,9 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
                 for (int e = 0; e < NE; e++)
                     v[i][e] = c0 + i < p.S - 1 ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)(c0 + i) * tiles * TILE_BYTES, SC1)
                                                : u32x4{1u, 1u, 1u, 1u};
-            for (int poll = 0; poll < kMaxPolls4; poll++) {
-                bool missing = false;
+            bool missing = true;
+            for (int poll = 0; poll < p.max_polls && missing; poll++) {
+                missing = false;
                 // the polls must be real loads: without a compiler barrier a reload with the operands of the first request is
                 // folded into it, and a wavefront that arrived before the data would spin on a stale register until the bound
                 asm volatile("" ::: "memory");
@@ -430,8 +435,8 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
                             v[i][e] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_z, lane_off + e * 1024, (uint32_t)(c0 + i) * tiles * TILE_BYTES, SC1);
                             missing = true;
                         }
-                if (!missing) break;
             }
+            gave_up = gave_up || missing;
 #pragma unroll
             for (int i = 0; i < CB; i++) {
                 if (c0 + i >= p.S - 1) break;
@@ -445,6 +450,14 @@ __global__ __launch_bounds__(512, 1) void wq_gemm4_kernel(const WqGemm4Args p)
         }
 #pragma unroll
         for (int e = 0; e < NE; e++) tot[e >> 2][e & 3] = P[e >> 2][e & 3] + tot[e >> 2][e & 3];
+        if (gave_up) {
+            // the wait for the other chunks ran out: the result is marked (NaN), not guessed, and the host is told through
+            // the workspace's sticky status word (mi355_workspace_status)
+            const float nan = __uint_as_float(0x7fc00000u);
+#pragma unroll
+            for (int e = 0; e < NE; e++) tot[e >> 2][e & 3] = f32x4{nan, nan, nan, nan};
+            *p.status = kStatusExchangeTimeout;
+        }
         // the zone goes back to zero for the next launch (no branches around the stores: nothing waits for them).  Ordinary
         // stores: the next launch is what must see them, and a write-through store to a line that a producer left modified
         // in the L2 takes several times as long
@@ -561,6 +574,9 @@ int launch_wq_gemm4(const WqGemm4Plan &plan, const void *x, int act_f16, const v
     p.strips = plan.strips;
     p.S = plan.S;
     p.l2_exchange = knob(kKnobWqGemm4Off) != 2;
+    p.max_polls = knob(kKnobWqMaxPolls) > 0 ? knob(kKnobWqMaxPolls) : kMaxPolls4;
+    p.only_chunk = knob(kKnobWqOnlyChunk);
+    p.status = plan.S > 1 ? reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kWorkspaceStatusOffset) : nullptr;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t tiles = (int64_t)plan.tiles_m * plan.strips;
     (void)tiles;

@@ -458,7 +458,7 @@ WqKpackedPlan make_wq_kpacked_plan(int64_t M, int64_t N, int64_t K, int64_t grou
     if (const int f = knob(kKnobWqSplit))
         if (f >= 1 && f <= pl.n_units) S = f;
     if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1;
-    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterCapacity) S = 1;
+    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) S = 1;
     // the parameter table of a workgroup's K range must fit in LDS beside the activation chunks and turn-around tiles
     auto lds_need = [&](int s) {
         const int64_t units = (pl.n_units + s - 1) / s;

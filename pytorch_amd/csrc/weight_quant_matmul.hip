@@ -619,7 +619,7 @@ WqPlan make_plan(int64_t M, int64_t N, int64_t K, int w_bits, int64_t group_size
     // wavefront that meets a single group)
     if (w_bits == 4 && pl.mt == 2 && pl.w * pl.ks == 4) pl.accum = true;
     pl.partial_bytes = pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0;
-    if (pl.S > 1 && (size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterCapacity) {
+    if (pl.S > 1 && (size_t)pl.sgroups * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) {
         pl.fast = false;                              // more tiles than arrival counters
         return pl;
     }
@@ -692,7 +692,7 @@ WqKmPlan make_kmajor_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, i
     if (const int f = knob(kKnobWqSplit))
         if (f >= 1 && f <= pl.n_units) S = f;
     if ((uint64_t)S * (uint64_t)M * (uint64_t)N * 4 >= (1ull << 32)) S = 1;
-    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterCapacity) S = 1;
+    if (S > 1 && (size_t)pl.tiles * pl.mchunks * sizeof(uint32_t) > kWorkspaceCounterBytes) S = 1;
     if (wq_kmajor_decode_shape(M, N, K, group_size)) S = 1;   // the decode kernel splits K inside its workgroups
     pl.S = S;
     pl.partial_bytes = S > 1 ? (size_t)S * M * N * sizeof(float) : 0;

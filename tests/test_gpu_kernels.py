@@ -307,14 +307,15 @@ def test_quant_matmul_deep_ring_small_tiles(capi, golden, tile, M, K, N):
             capi.set_tuning(k, 0)
 
 
-@pytest.mark.parametrize("tile", [256192, 256224])
+@pytest.mark.parametrize("tile", [256192, 256224, 256256])
 @pytest.mark.parametrize("M,K,N", [(256, 128, 192), (300, 640, 500), (512, 4224, 1000), (1024, 1152, 2300), (255, 2048, 8 * 97)])
 def test_quant_matmul_wide_loop_tiles(capi, golden, tile, M, K, N):
     """The 256-row tiles run the K loop with loader roles (activation slots released by an LDS flag between the two
     wavefronts that read them).  One K step, odd and even step counts, ragged rows and columns, with and without a split of
     K, both instruction orders: int32 accumulators bit-identical to the oracle, every epilogue (the LDS-parameter one for
     per-token scale + bf16 bias / no bias in bf16 and fp16, and the general one for the other bias kinds, a single scale,
-    no per-token scale, int32 and re-quantised int8 outputs) bit-identical to the generic loop and to the oracle."""
+    no per-token scale, int32 and re-quantised int8 outputs) bit-identical to the generic loop and to the oracle.  (The
+    256x256 tile, which only has the generic loop, runs through the same cases against the oracle.)"""
     d = workloads.quant_matmul_inputs(seed=M + N + K, M=M, K=K, N=N, weight_nk=True, bias=True)
     g = torch.Generator().manual_seed(M + K)
     x1, x2, sc, ps, bias = (d[k].cuda() for k in ("x1", "x2", "scale", "pertoken_scale", "bias"))
@@ -1279,3 +1280,35 @@ def test_w4a16_repeated_launches_reuse_workspace(capi, golden):
             first[it % 2] = out.clone()
         else:
             assert torch.equal(out, first[it % 2]), f"launch {it} differs from the first launch of the same problem"
+
+
+@pytest.mark.parametrize("M", [8, 128])
+def test_weight_quant_exchange_timeout_is_reported(capi, golden, M):
+    """The int4 kernels' collecting workgroup waits a bounded number of polls for the other K chunks' partial sums.  The
+    give-up path is driven from the host so that every kernel still ends normally: a knob lets only the collecting chunk
+    run and shortens the bound to four polls.  The launch then reports MI355_OK (it was enqueued), its outputs hold NaN
+    instead of a wrong sum, the workspace's sticky status word makes mi355_workspace_status fail once and clears the
+    zero area, and the next ordinary launch on the same workspace is right again (M = 8: the decode kernel, M = 128: the
+    register-expanding tiled kernel)."""
+    d = workloads.w4a16_inputs(seed=3, M=M)
+    x, w, sc, of = (d[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset"))
+    need = capi.lib().mi355_weight_quant_matmul_workspace(M, 14336, 4096, 4, 128)
+    assert need > 0
+    ws = capi._wq_workspace(x.device, need)
+    good = capi.weight_quant_matmul(x, w, sc, of, group_size=128)
+    capi.workspace_status(ws)                                   # nothing to report
+    capi.set_tuning("MI355_WQ_MAX_POLLS", 4)
+    capi.set_tuning("MI355_WQ_ONLY_CHUNK", -1)
+    try:
+        bad = capi.weight_quant_matmul(x, w, sc, of, group_size=128)
+    finally:
+        capi.set_tuning("MI355_WQ_MAX_POLLS", 0)
+        capi.set_tuning("MI355_WQ_ONLY_CHUNK", 0)
+    torch.cuda.synchronize()
+    assert torch.isnan(bad.float()).all(), "the collector must mark what it could not sum"
+    with pytest.raises(capi.Mi355Error, match="status word"):
+        capi.workspace_status(ws)
+    capi.workspace_status(ws)                                   # reported once, then cleared
+    assert int(ws[:capi.ZERO_AREA_BYTES].count_nonzero()) == 0
+    again = capi.weight_quant_matmul(x, w, sc, of, group_size=128)
+    assert torch.equal(again, good)

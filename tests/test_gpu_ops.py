@@ -669,3 +669,26 @@ def test_linear_weight_quant_reference_test_shape(pa):
     frac = rtol_failures(rounded, out.numpy(), 1e-3) / out.numel()
     print("reference shape: fraction beyond 1e-3 of the float16-rounded golden", round(frac, 4))
     assert frac < 0.25
+
+
+def test_device_failure_report_reaches_the_operator_layer(pa):
+    """torch.ops.npu path of the same report: after a launch whose collector gave up (driven from the host, every kernel
+    ends normally), pytorch_amd.check_device_status() raises once, clears the workspace, and the operator works again."""
+    from pytorch_amd import _capi
+    d = workloads.w4a16_inputs(seed=4, M=8)
+    args = [d[k].cuda() for k in ("x", "weight", "antiquant_scale", "antiquant_offset")] + [None, None, None, 128]
+    good = pa.npu_weight_quant_batchmatmul(*args)
+    pa.check_device_status()
+    _capi.set_tuning("MI355_WQ_MAX_POLLS", 4)
+    _capi.set_tuning("MI355_WQ_ONLY_CHUNK", -1)
+    try:
+        bad = pa.npu_weight_quant_batchmatmul(*args)
+    finally:
+        _capi.set_tuning("MI355_WQ_MAX_POLLS", 0)
+        _capi.set_tuning("MI355_WQ_ONLY_CHUNK", 0)
+    torch.cuda.synchronize()
+    assert torch.isnan(bad.float()).all()
+    with pytest.raises(RuntimeError, match="device-side failure"):
+        pa.check_device_status()
+    pa.check_device_status()
+    assert torch.equal(pa.npu_weight_quant_batchmatmul(*args), good)

@@ -17,7 +17,7 @@ def test_c_abi_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "mi355_quant.h")).read()
     declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", header))
     assert {"mi355_dynamic_quant", "mi355_quant_matmul", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant", "mi355_anti_quant",
-            "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize", "mi355_trans_quant_param",
+            "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize", "mi355_trans_quant_param", "mi355_workspace_status", "mi355_workspace_zero_bytes",
             "mi355_quant_matmul_qparam", "mi355_swiglu_quant_smooth"} <= declared
     lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_amd", "csrc", "libmi355_quant.so"))
     for name in declared:

@@ -84,3 +84,76 @@ def test_quant_matmul_noalloc_matches_workspace_entry_point():
     out = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
     sc = torch.ones(N, device="cuda")
     assert _call(L, True, x1, x2, sc, None, None, out) == -4
+
+
+def test_quant_matmul_noalloc_under_graph_capture():
+    """The entry point exists for callers that cannot allocate, graph capture among them: two calls (a split-K shape and
+    a smaller one) are captured on a fresh stream and replayed three times with eager work and synchronisations between
+    the replays; every replay reproduces the bits of mi355_quant_matmul with a caller workspace."""
+    from pytorch_amd import _capi
+    L = _capi.lib()
+    g = torch.Generator().manual_seed(9)
+    cases = []
+    for (M, K, N) in [(64, 14336, 4096), (40, 4096, 512)]:
+        x1 = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).cuda()
+        x2 = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).cuda().t()
+        scale = (torch.rand(N, generator=g) * 9e-3 + 1e-3).cuda()
+        ps = (torch.rand(M, generator=g) * 9e-3 + 1e-3).cuda()
+        bias = (torch.randn(N, generator=g) * 0.02).to(torch.bfloat16).cuda()
+        need = L.mi355_quant_matmul_workspace(M, N, K, x2.stride(0), x2.stride(1))
+        ws = torch.zeros(max(need, 16), dtype=torch.int8, device="cuda")
+        want = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        assert _call(L, False, x1, x2, scale, ps, bias, want, ws if need else None) == 0
+        got = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        cases.append((x1, x2, scale, ps, bias, want, got))
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        for (x1, x2, scale, ps, bias, want, got) in cases:
+            assert _call(L, True, x1, x2, scale, ps, bias, got) == 0
+    for it in range(3):
+        for c in cases:
+            c[6].fill_(1.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        for c in cases:
+            assert torch.equal(c[6], c[5]), f"replay {it}"
+        # eager work of the same entry point between the replays
+        x1, x2, scale, ps, bias, want, got = cases[it % 2]
+        eager = torch.zeros_like(want)
+        assert _call(L, True, x1, x2, scale, ps, bias, eager) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(eager, want)
+
+
+def test_quant_matmul_noalloc_int32_output_and_forced_split():
+    """An int32 output (raw accumulators) through the scratch array, and a split of K forced through the tuning knob: the
+    forced split is held to the scratch's capacity like a planned one (here it fits), results equal to the ordinary entry
+    point's."""
+    from pytorch_amd import _capi
+    L = _capi.lib()
+    g = torch.Generator().manual_seed(11)
+    M, K, N = 96, 8192, 1024
+    x1 = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).cuda()
+    x2 = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).cuda().t()
+    p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ref = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    need = L.mi355_quant_matmul_workspace(M, N, K, x2.stride(0), x2.stride(1))
+    ws = torch.zeros(max(need, 16), dtype=torch.int8, device="cuda")
+    args = (p(x1), p(x2), None, None, 0, None, 0)
+    tail = (1, M, N, K, x1.stride(0), x2.stride(0), x2.stride(1), N)
+    assert L.mi355_quant_matmul(*args, p(ref), *tail, p(ws), ws.numel(), stream) == 0
+    for split in (0, 4):
+        _capi.set_tuning("MI355_QMM_SPLIT", split)
+        try:
+            got = torch.full((M, N), 7, dtype=torch.int32, device="cuda")
+            assert L.mi355_quant_matmul_noalloc(*args, p(got), *tail, stream) == 0
+            torch.cuda.synchronize()
+            assert torch.equal(got, ref), split
+        finally:
+            _capi.set_tuning("MI355_QMM_SPLIT", 0)
+    import numpy as np
+    from oracle import golden
+    assert np.array_equal(ref.cpu().numpy(), golden.int8_gemm(x1.cpu().numpy(), x2.cpu().numpy()))
