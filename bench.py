@@ -64,6 +64,8 @@ def _parse():
                     help="launch the timed headline steps from one captured HIP graph instead of one by one")
     ap.add_argument("--eager", action="store_true", help="accepted for compatibility: one-by-one launches are the default")
     ap.add_argument("--only", default="", help="comma-separated subset of: c1,c2kn,c2i8,c3,c4,qd,a4w4,c5,aq,qz for the 'others' section")
+    ap.add_argument("--pmc-summarize", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="print the TRAFFIC lines from the output directories of the two rocprofv3 --pmc runs of --pmc-pass")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="launch a 256 MiB device copy and then each main kernel once on fresh buffers (for "
                          "`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: the copy calibrates the counters)")
@@ -120,78 +122,145 @@ def _nsets(bytes_per_set):
 
 
 def _pmc_pass(torch, pa, workloads, dev):
-    """One launch of every main kernel on buffers that no earlier kernel of this process touched, preceded by a
-    plain device copy of known size (268,435,456 bytes read and written) that calibrates FETCH_SIZE / WRITE_SIZE."""
-    src = torch.empty(256 << 20, dtype=torch.int8, device=dev)
+    """One launch of every benchmarked kernel (or chain of kernels) on operands that no earlier kernel of this process
+    touched, for `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs.  Every item is preceded by a 1 GiB fill that
+    pushes earlier data out of the caches; an empty kernel whose workgroup count is 1000 + index opens the item and one
+    with 999 workgroups closes it.  Item 0 is a plain device copy of known size that calibrates the two counters.
+    `bench.py --pmc-summarize <dir of the FETCH_SIZE run> <dir of the WRITE_SIZE run>` turns the two counter files into
+    the TRAFFIC lines of profiles/hbm_traffic_pmc_all_kernels.txt."""
+    from pytorch_amd import _capi
+    gen = torch.Generator(device=dev).manual_seed(7)
+    ri8 = lambda *sh: torch.randint(-127, 128, sh, generator=gen, dtype=torch.int8, device=dev)  # noqa: E731
+    ri32 = lambda *sh: torch.randint(-2 ** 31, 2 ** 31 - 1, sh, generator=gen, dtype=torch.int32, device=dev)  # noqa: E731
+    up = lambda d: {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d.items()}  # noqa: E731
+    items = []
+
+    # one-time set-up (per-stream workspaces, function attributes) on small shapes: no big traffic, no allocation later
+    w0 = up(workloads.w4a16_inputs(seed=9, M=8, K=1024, N=512))
+    pa.npu_weight_quant_batchmatmul(w0["x"], w0["weight"], w0["antiquant_scale"], w0["antiquant_offset"], None, None, None, 128)
+    pa.npu_quant_matmul(ri8(64, 14336), ri8(256, 14336).t(), torch.rand(256, device=dev), output_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+
+    src = torch.empty(256 << 20, dtype=torch.int8, device=dev).fill_(1)
     dst = torch.empty_like(src)
-    src.fill_(1)
-    torch.cuda.synchronize()
-    dst.copy_(src)                                   # calibration kernel
+    items.append(("copy", lambda: dst.copy_(src)))
     d1 = workloads.dynamic_quant_input(seed=0).to(dev)
-    d2 = workloads.quant_matmul_inputs(seed=0, weight_nk=True)
-    d3 = workloads.w8a16_inputs(seed=0)
-    d4 = workloads.w4a16_inputs(seed=0, M=8)
-    g = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d2.items()}
-    g3 = {k: v.to(dev) for k, v in d3.items()}
-    g4 = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d4.items()}
+    items.append(("c1", lambda: pa.npu_dynamic_quant(d1)))
+    g2 = up(workloads.quant_matmul_inputs(seed=0, weight_nk=True))
+    items.append(("c2", lambda: pa.npu_quant_matmul(g2["x1"], g2["x2"], g2["scale"], pertoken_scale=g2["pertoken_scale"], bias=g2["bias"],
+                                                    output_dtype=torch.bfloat16)))
+    w2kn = ri8(4096, 11008)
+    items.append(("c2_kn", lambda: pa.npu_quant_matmul(g2["x1"], w2kn, g2["scale"], pertoken_scale=g2["pertoken_scale"], bias=g2["bias"],
+                                                       output_dtype=torch.bfloat16)))
+    qp = pa.npu_trans_quant_param(torch.rand(11008, device=dev) * 1e-4 + 1e-4, torch.randint(-8, 8, (11008,), device=dev).float())
+    bi = torch.randint(-1000, 1000, (11008,), device=dev, dtype=torch.int32)
+    x2i8, w2i8 = ri8(1024, 4096), ri8(11008, 4096).t()
+    items.append(("c2_i8", lambda: pa.npu_quant_matmul(x2i8, w2i8, qp, bias=bi, output_dtype=torch.int8)))
+    xa4, wa4 = ri32(1024, 512), ri32(11008, 512).t()
+    items.append(("a4w4", lambda: pa.npu_quant_matmul(xa4, wa4, g2["scale"], pertoken_scale=g2["pertoken_scale"], output_dtype=torch.bfloat16)))
+    g3 = up(workloads.w8a16_inputs(seed=0))
+    items.append(("c3", lambda: pa.npu_weight_quant_batchmatmul(g3["x"], g3["weight"], g3["antiquant_scale"], g3["antiquant_offset"])))
+    w3nk = ri8(28672, 8192).t()
+    items.append(("c3_nk", lambda: pa.npu_weight_quant_batchmatmul(g3["x"], w3nk, g3["antiquant_scale"], g3["antiquant_offset"])))
+    for m_rows in (1, 8, 32, 128):
+        g4 = up(workloads.w4a16_inputs(seed=m_rows, M=m_rows))
+        items.append((f"c4_m{m_rows}", lambda g4=g4: pa.npu_weight_quant_batchmatmul(g4["x"], g4["weight"], g4["antiquant_scale"],
+                                                                                      g4["antiquant_offset"], None, None, None, 128)))
+        wk = ri32(14336, 512).t()
+        s4t, o4t = g4["antiquant_scale"].t().contiguous().t(), g4["antiquant_offset"].t().contiguous().t()
+        items.append((f"c4k_m{m_rows}", lambda g4=g4, wk=wk, s4t=s4t, o4t=o4t: pa.npu_weight_quant_batchmatmul(
+            g4["x"], wk, s4t, o4t, None, None, None, 128)))
+    xa, sa = torch.randint(-128, 128, (4096, 14336), dtype=torch.int8, device=dev), torch.rand(14336, device=dev) + 0.5
+    items.append(("aq_int8", lambda: pa.npu_anti_quant(xa, sa, offset=sa, dst_dtype=torch.bfloat16)))
+    for (Kx, Nx) in ((4096, 28672), (14336, 4096)):
+        wq, xq = ri8(Nx, Kx).t(), ri8(16, Kx)
+        sq, pq = torch.rand(Nx, device=dev), torch.rand(16, device=dev)
+        items.append((f"qd_{Kx}x{Nx}_m16", lambda wq=wq, xq=xq, sq=sq, pq=pq: pa.npu_quant_matmul(xq, wq, sq, pertoken_scale=pq,
+                                                                                                  output_dtype=torch.bfloat16)))
+    H, I = 4096, 14336
+    for Mx in (16, 64, 2048):
+        x5 = torch.randn(Mx, H, device=dev).to(torch.bfloat16)
+        wgu, wd = ri8(2 * I, H).t(), ri8(H, I).t()
+        sgu, sd = torch.rand(2 * I, device=dev) * 1e-2, torch.rand(H, device=dev) * 1e-2
+
+        def mlp(x5=x5, wgu=wgu, wd=wd, sgu=sgu, sd=sd):
+            xq, xsc = pa.npu_dynamic_quant(x5)
+            gu = pa.npu_quant_matmul(xq, wgu, sgu, pertoken_scale=xsc, output_dtype=torch.bfloat16)
+            aq, asc = pa.npu_swiglu_quant(gu, activate_left=True, quant_mode=1)
+            return pa.npu_quant_matmul(aq, wd, sd, pertoken_scale=asc, output_dtype=torch.bfloat16)
+        items.append((f"c5_m{Mx}", mlp))
+
     flush = torch.empty(1 << 30, dtype=torch.int8, device=dev)
-    flush.fill_(0)                                   # push the freshly uploaded operands out of the caches
-    torch.cuda.synchronize()
-    pa.npu_dynamic_quant(d1)
-    pa.npu_quant_matmul(g["x1"], g["x2"], g["scale"], pertoken_scale=g["pertoken_scale"], bias=g["bias"],
-                        output_dtype=torch.bfloat16)
-    pa.npu_weight_quant_batchmatmul(g3["x"], g3["weight"], g3["antiquant_scale"], g3["antiquant_offset"])
-    pa.npu_weight_quant_batchmatmul(g4["x"], g4["weight"], g4["antiquant_scale"], g4["antiquant_offset"], None, None,
-                                    None, 128)
-    # the tiled weight-only kernel (configuration 4 at M = 128) and the standalone antiquantisation, on fresh operands
-    d5 = workloads.w4a16_inputs(seed=1, M=128)
-    g5 = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d5.items()}
-    xa = torch.randint(-128, 128, (4096, 14336), dtype=torch.int8, device=dev)
-    sa = torch.rand(14336, device=dev) + 0.5
-    flush.fill_(1)
-    torch.cuda.synchronize()
-    pa.npu_weight_quant_batchmatmul(g5["x"], g5["weight"], g5["antiquant_scale"], g5["antiquant_offset"], None, None,
-                                    None, 128)
-    pa.npu_anti_quant(xa, sa, offset=sa, dst_dtype=torch.bfloat16)
-    # the decode kernel at one and at 32 activation rows, each on a weight no kernel has touched
-    for m_rows, seed in ((1, 2), (32, 3)):
-        dm = workloads.w4a16_inputs(seed=seed, M=m_rows)
-        gm = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in dm.items()}
-        flush.fill_(3)
+    keep = []
+    for idx, (tag, fn) in enumerate(items):
+        flush.fill_(idx & 127)
         torch.cuda.synchronize()
-        pa.npu_weight_quant_batchmatmul(gm["x"], gm["weight"], gm["antiquant_scale"], gm["antiquant_offset"], None, None,
-                                        None, 128)
-    # int4 weights with their words along K (the module's layout) at M = 8, and the int4 -> int8 widening of an A4W4
-    # weight, on fresh operands
-    wk = torch.randint(-2 ** 31, 2 ** 31 - 1, (14336, 512), dtype=torch.int32, device=dev)
-    wa = torch.randint(-2 ** 31, 2 ** 31 - 1, (11008, 512), dtype=torch.int32, device=dev)
-    xa4 = torch.randint(-2 ** 31, 2 ** 31 - 1, (1024, 512), dtype=torch.int32, device=dev)
-    s4t, o4t = g4["antiquant_scale"].t().contiguous().t(), g4["antiquant_offset"].t().contiguous().t()
-    flush.fill_(2)
-    torch.cuda.synchronize()
-    pa.npu_weight_quant_batchmatmul(g4["x"], wk.t(), s4t, o4t, None, None, None, 128)
-    pa.npu_quant_matmul(xa4, wa.t(), g["scale"], pertoken_scale=g["pertoken_scale"], output_dtype=torch.bfloat16)
-    # configuration 3 with the weight stored [N, K] (the contrib module's layout), on a weight no kernel has touched
-    w3nk = torch.randint(-127, 128, (28672, 8192), dtype=torch.int8, device=dev)
-    flush.fill_(5)
-    torch.cuda.synchronize()
-    pa.npu_weight_quant_batchmatmul(g3["x"], w3nk.t(), g3["antiquant_scale"], g3["antiquant_offset"])
-    # the decode kernel of quant_matmul: the two projections of the MLP at 16 rows, weights no kernel has touched
-    wgu = torch.randint(-128, 128, (28672, 4096), dtype=torch.int8, device=dev)
-    wdn = torch.randint(-128, 128, (4096, 14336), dtype=torch.int8, device=dev)
-    xq1 = torch.randint(-128, 128, (16, 4096), dtype=torch.int8, device=dev)
-    xq2 = torch.randint(-128, 128, (16, 14336), dtype=torch.int8, device=dev)
-    sgu, sdn, ps16 = torch.rand(28672, device=dev), torch.rand(4096, device=dev), torch.rand(16, device=dev)
-    flush.fill_(4)
-    torch.cuda.synchronize()
-    pa.npu_quant_matmul(xq1, wgu.t(), sgu, pertoken_scale=ps16, output_dtype=torch.bfloat16)
-    pa.npu_quant_matmul(xq2, wdn.t(), sdn, pertoken_scale=ps16, output_dtype=torch.bfloat16)
-    torch.cuda.synchronize()
-    print(json.dumps({"pmc_pass": "done"}))
+        _capi.empty_launch(1000 + idx)                 # opens item idx
+        keep.append(fn())
+        _capi.empty_launch(999)                        # closes it
+        torch.cuda.synchronize()
+    print(json.dumps({"pmc_pass": [t for t, _ in items]}))
+
+
+_PMC_TAGS = ["copy", "c1", "c2", "c2_kn", "c2_i8", "a4w4", "c3", "c3_nk", "c4_m1", "c4k_m1", "c4_m8", "c4k_m8", "c4_m32", "c4k_m32",
+             "c4_m128", "c4k_m128", "aq_int8", "qd_4096x28672_m16", "qd_14336x4096_m16", "c5_m16", "c5_m64", "c5_m2048"]
+
+
+def _pmc_summarize(fetch_dir, write_dir):
+    """Reads the counter files of the two `rocprofv3 --pmc` runs of `bench.py --pmc-pass` and prints, per item, the
+    kernels it launched and its HBM bytes (FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for the 256 MiB copy)."""
+    import csv
+    import glob
+    import re
+
+    def load(d, counter):
+        files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            raise SystemExit(f"no *counter_collection.csv under {d}")
+        rows = []
+        for f in files:
+            with open(f, newline="") as fh:
+                for r in csv.DictReader(fh):
+                    if r.get("Counter_Name") == counter:
+                        rows.append((int(r["Dispatch_Id"]), r["Kernel_Name"], int(r["Grid_Size"]) // max(int(r["Workgroup_Size"]), 1),
+                                     float(r["Counter_Value"])))
+        rows.sort()
+        segs, cur = {}, None
+        for _, name, wgs, val in rows:
+            if "empty_kernel" in name:
+                cur = wgs - 1000 if wgs >= 1000 else None
+                continue
+            if cur is not None:
+                segs.setdefault(cur, []).append((name, val))
+        return segs
+
+    fetch, write = load(fetch_dir, "FETCH_SIZE"), load(write_dir, "WRITE_SIZE")
+    kib = 256 * 1024.0
+    f_scale = kib / sum(v for _, v in fetch[0])
+    w_scale = kib / sum(v for _, v in write[0])
+    print(f"calibration (plain copy, 262,144 KiB read and written): FETCH_SIZE reads {sum(v for _, v in fetch[0]):,.0f} -> factor {f_scale:.3f}; "
+          f"WRITE_SIZE reads {sum(v for _, v in write[0]):,.0f} -> factor {w_scale:.3f}")
+    for idx, tag in enumerate(_PMC_TAGS):
+        if idx == 0 or idx not in fetch:
+            continue
+        # zero fills and small copies are the host layer growing a workspace on first use, not the operator's traffic
+        own = lambda seg: [(n, v) for n, v in seg if "FillFunctor" not in n and "copyBuffer" not in n]  # noqa: E731
+        fk = sum(v for _, v in own(fetch[idx])) * f_scale
+        wk = sum(v for _, v in own(write.get(idx, []))) * w_scale
+        names = []
+        for n, _ in own(fetch[idx]):
+            m = re.search(r"([A-Za-z_0-9]+_kernel[A-Za-z_0-9]*|copyBuffer)(<[^()]*>)?", n.replace("(anonymous namespace)::", ""))
+            short = (m.group(1) + (m.group(2) or "")) if m else n[:40]
+            if short not in names:
+                names.append(short)
+        print(f"TRAFFIC tag={tag} kernel={'+'.join(names).replace(' ', '')} hbm_bytes={int((fk + wk) * 1024)} fetch_kib={fk:.0f} write_kib={wk:.0f}")
 
 
 def main():
     args = _parse()
+    if args.pmc_summarize:
+        _pmc_summarize(*args.pmc_summarize)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this operator path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
@@ -347,11 +416,28 @@ def main():
     def want(tag):
         return not args.skip_others and (not only or tag in only)
 
+    copy_cache = {}
+
+    def copy_ceiling_us(nbytes):
+        """Time of a plain device-to-device copy that moves `nbytes` in all (half read, half written), launched the same
+        way (captured graph, buffers rotated past the Infinity Cache): what a launch of this size can reach on this chip,
+        next to which the microsecond-scale kernels are to be read (an empty launch alone takes about 2 us)."""
+        half = max(int(nbytes) // 2 // 4096 * 4096, 4096)
+        if half not in copy_cache:
+            ns = _nsets(2 * half)
+            src = [torch.empty(half, dtype=torch.int8, device=dev).fill_(1) for _ in range(ns)]
+            dst = [torch.empty(half, dtype=torch.int8, device=dev) for _ in range(ns)]
+            calls = [(lambda a=a, b=b: b.copy_(a)) for a, b in zip(src, dst)] * 2
+            copy_cache[half] = round(_graph_time_us(torch, calls), 3)
+            del src, dst
+        return copy_cache[half]
+
     def hbm_entry(name, bytes_per_launch, us, traffic=None, **extra):
         gbs = bytes_per_launch / (us * 1e-6) / 1e9
         e = {"name": name, "launch_us": round(us, 3), "bytes": int(bytes_per_launch),
              "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic}}
+                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                          "copy_ceiling_us": copy_ceiling_us(bytes_per_launch)}}
         e.update(extra)
         return e
 
@@ -391,7 +477,7 @@ def main():
         others.append({"name": "c2 quant_matmul, weight contiguous [K,N]", "launch_us": round(ms * 1e3, 2),
                        "roofline": {"bound": "mfma", "achieved": round(ops / (ms * 1e-3) / 1e12, 2), "peak": INT8_PEAK_TOPS,
                                     "unit": "TOP/s", "frac": round(ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
-                                    "traffic": None}})
+                                    "traffic": _traffic("c2_kn")}})
         del w_kn
 
     if want("c1"):
@@ -494,7 +580,7 @@ def main():
                      for w in wks] * 2
             us = _graph_time_us(torch, calls)
             others.append(hbm_entry(f"c4 W4A16 g128 x bf16[{Mx},4096] . int4 stored [14336,4096/8] (words along K, parameters "
-                                    "[N,G]: the module's transposed views)", nb, us, None,
+                                    "[N,G]: the module's transposed views)", nb, us, _traffic(f"c4k_m{Mx}"),
                                     tflops=round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2)))
             del wks, keep
 
@@ -514,7 +600,7 @@ def main():
         tops = 2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12
         others.append({"name": "c2 quant_matmul with int8 output (int64 packed scale + offset, int32 bias)", "launch_us": round(us, 3),
                        "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                                    "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None}})
+                                    "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": _traffic("c2_i8")}})
         del xs, wsn, keep
 
     if want("qd"):
@@ -542,7 +628,7 @@ def main():
                 others.append({"name": f"quant_matmul {'decode ' if Mx <= 64 else ''}int8[{Mx},{Kx}] . int8 stored [{Nx},{Kx}] -> bf16", "launch_us": round(us, 3), **gate,
                                "roofline": {"bound": "hbm", "achieved": round(nb / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
                                             "unit": "GB/s", "frac": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                                            "traffic": _traffic(f"qd_{Kx}x{Nx}_m{Mx}")},
+                                            "traffic": _traffic(f"qd_{Kx}x{Nx}_m{Mx}"), "copy_ceiling_us": copy_ceiling_us(nb)},
                                "algorithmic_bytes": int(nb)})
                 del xs, keep
             del wsn
@@ -561,7 +647,10 @@ def main():
         us = _graph_time_us(torch, calls, reps=10)
         others.append({"name": "a4w4 quant_matmul int4[1024,4096] . int4 stored [11008,4096/8] -> bf16 (unpack kernels + int8 GEMM)",
                        "us": round(us, 2), "tops": round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 1),
-                       "frac_int8_peak": round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4)})
+                       "frac_int8_peak": round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4),
+                       "roofline": {"bound": "mfma", "achieved": round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12, 2), "peak": INT8_PEAK_TOPS,
+                                    "unit": "TOP/s", "frac": round(2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4),
+                                    "traffic": _traffic("a4w4")}, "algorithmic_bytes": int(nb)})
         del xs, wsk, keep
 
     if want("c5"):
@@ -628,9 +717,11 @@ def main():
                      "chain_us": round(us, 2), "chain_us_cache_resident_weights": round(hot, 2),
                      "int8_tops": round(mops / (us * 1e-6) / 1e12, 2),
                      "roofline": ({"bound": "hbm", "achieved": round(abytes / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                   "frac": round(abytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None} if Mx <= 64 else
+                                   "frac": round(abytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                                   "traffic": _traffic(f"c5_m{Mx}") if fn is mlp_fused else None, "copy_ceiling_us": copy_ceiling_us(abytes)} if Mx <= 64 else
                                   {"bound": "mfma", "achieved": round(mops / (us * 1e-6) / 1e12, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                                   "frac": round(mops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None}),
+                                   "frac": round(mops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4),
+                                   "traffic": _traffic(f"c5_m{Mx}") if fn is mlp_fused else None}),
                      "algorithmic_bytes": int(abytes)}
                 if fn is mlp_fused:
                     e["bit_identical_to_5_kernel_chain"] = same
