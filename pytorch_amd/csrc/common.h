@@ -89,7 +89,7 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
 // a collector into its give-up path from the host, every kernel still ending normally: tests of the error reporting).
 enum Knob { kKnobWqSplit, kKnobWqW, kKnobWqgSplit, kKnobWqgBm, kKnobWqGemmOff, kKnobWqkMt, kKnobWqkNw, kKnobWqkKs,
             kKnobQmmSplit, kKnobQmmTile /* bm * 1000 + bn */, kKnobWqDecodeOff, kKnobQmmDeepOff, kKnobWqGemm4Off, kKnobQmmDecodeOff,
-            kKnobQmmLoop, kKnobWqMaxPolls, kKnobWqOnlyChunk, kKnobCount };
+            kKnobQmmLoop, kKnobWqMaxPolls, kKnobWqOnlyChunk, kKnobQmmStreamOut, kKnobCount };
 int knob(Knob k);
 
 inline int check_launch()

@@ -72,6 +72,7 @@ struct QmmArgs {
     int out_i32;
     const uint64_t *qparam;    // packed quantisation parameters [scale_len] (replace `scale`), or null
     int out_i8;                // re-quantised int8 output (needs qparam)
+    int stream_out;            // 256-row tiles, 16-bit output: non-temporal row stores (chosen by the launcher)
     int tiles_m, tiles_n, tiles_per_xcd;
     int S;                     // workgroups that share the K range of a tile
     int32_t *partial;          // workspace [tile][chunk][wavefront][accumulator quad][lane] int32x4 (S > 1)
@@ -499,6 +500,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             e.n0 = n0;
             e.has_bias = p.bias_kind == MI355_BIAS_BF16;
             e.out_f16 = p.out_f16;
+            e.stream_out = p.stream_out;
             wide::epilogue_fast<WTN>(acc, lds, e, wave, lane);
             MI355_TS(4)
             return;
@@ -899,6 +901,7 @@ struct QmmPlan {
 // projections of transformer layers with K = 4096 .. 14336 (46 shapes: the estimate's choice is 0.7 % slower than the
 // measured best on average and 8 % at worst; at K = 4096 without a split the estimate is the table itself).
 constexpr size_t kMaxPartialBytes = (size_t)128 << 20;
+constexpr uint64_t kStreamOutMaxBytes = (uint64_t)32 << 20;     // the L2s of the eight XCDs together
 constexpr double kBaseUs = 6.0, kL2BytesPerUs = 12e6, kExchangeUs = 1.0, kExchangeBytesPerUs = 10e6, kCollectorBytesPerUs = 100e3;
 constexpr double kAloneOnCu = 0.85;
 
@@ -1108,6 +1111,17 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     p.out_i32 = out_i32;
     p.qparam = qparam;
     p.out_i8 = out_i8;
+    // An output that the L2s could hold (8 x 4 MiB) would leave them only in the write-back at the end of the kernel, a
+    // burst that nothing overlaps; streaming the rows out while other tiles still compute makes the launch 2.5 us
+    // (1024x4096x11008) shorter and costs the next reader nothing (product + dynamic_quant of it: 60.1 -> 58.5 us).  A
+    // larger output spills into the Infinity Cache during the kernel anyway, and a reader finds it there: non-temporal
+    // stores would take that away (2048x4096x28672 followed by the fused SwiGLU + quantisation: +11 us), so it keeps
+    // ordinary stores.  MI355_QMM_STREAM_OUT: 1 never, 2 always.
+    {
+        const int so = knob(kKnobQmmStreamOut);
+        const uint64_t out_bytes = (uint64_t)M * (uint64_t)N * 2u;
+        p.stream_out = so == 2 || (so != 1 && out_bytes <= kStreamOutMaxBytes);
+    }
     const TileChoice c = pl.tile;
     p.S = pl.S;
     p.counter = pl.S > 1 ? reinterpret_cast<uint32_t *>(ws) : nullptr;

@@ -372,6 +372,7 @@ struct EpilogueArgs {
     int M, N;
     int m0, n0;                        // first row / column of the workgroup tile
     int has_bias, out_f16;
+    int stream_out;                    // store the rows with non-temporal stores (see the launcher's choice)
 };
 
 constexpr int PARAM_PS = 0, PARAM_SCALE = 1024, PARAM_BIAS = 2048;
@@ -392,7 +393,7 @@ __device__ __forceinline__ void request_params(char *lds, int param_base, const 
     }
 }
 
-template <int WTN, bool F16, bool BIAS>
+template <int WTN, bool F16, bool BIAS, bool NT>
 __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
 {
     using G = Geometry<WTN>;
@@ -444,7 +445,8 @@ __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, 
             const u32x4 v = *reinterpret_cast<const u32x4 *>(stg + row * ROWB + ch * 16);
             uint16_t *o = static_cast<uint16_t *>(e.out) + (int64_t)m * e.ldc + n;
             if (n + 7 < e.N) {
-                *reinterpret_cast<u32x4 *>(o) = v;
+                if constexpr (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(o));
+                else *reinterpret_cast<u32x4 *>(o) = v;
             } else {
                 for (int r = 0; r < 8; r++)
                     if (n + r < e.N) o[r] = (uint16_t)(v[r >> 1] >> ((r & 1) * 16));
@@ -456,13 +458,19 @@ __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, 
 template <int WTN>
 __device__ __forceinline__ void epilogue_fast(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
 {
-    // output type and bias presence are resolved once per wavefront
+    // output type, bias presence and the kind of store are resolved once per wavefront
+    auto go = [&](auto f16, auto bias) {
+        if (e.stream_out) epilogue_rows<WTN, decltype(f16)::value, decltype(bias)::value, true>(acc, lds, e, wave, lane);
+        else epilogue_rows<WTN, decltype(f16)::value, decltype(bias)::value, false>(acc, lds, e, wave, lane);
+    };
+    using T = std::true_type;
+    using F = std::false_type;
     if (e.out_f16) {
-        if (e.has_bias) epilogue_rows<WTN, true, true>(acc, lds, e, wave, lane);
-        else epilogue_rows<WTN, true, false>(acc, lds, e, wave, lane);
+        if (e.has_bias) go(T{}, T{});
+        else go(T{}, F{});
     } else {
-        if (e.has_bias) epilogue_rows<WTN, false, true>(acc, lds, e, wave, lane);
-        else epilogue_rows<WTN, false, false>(acc, lds, e, wave, lane);
+        if (e.has_bias) go(F{}, T{});
+        else go(F{}, F{});
     }
 }
 

@@ -11,7 +11,8 @@ namespace {
 const char *const kKnobNames[kKnobCount] = {"MI355_WQ_SPLIT", "MI355_WQ_W",    "MI355_WQG_SPLIT", "MI355_WQG_BM",   "MI355_WQ_GEMM_OFF",
                                             "MI355_WQK_MT",   "MI355_WQK_NW",  "MI355_WQK_KS",    "MI355_QMM_SPLIT", "MI355_QMM_TILE",
                                             "MI355_WQ_DECODE_OFF", "MI355_QMM_DEEP_OFF", "MI355_WQ_GEMM4_OFF",
-                                            "MI355_QMM_DECODE_OFF", "MI355_QMM_LOOP", "MI355_WQ_MAX_POLLS", "MI355_WQ_ONLY_CHUNK"};
+                                            "MI355_QMM_DECODE_OFF", "MI355_QMM_LOOP", "MI355_WQ_MAX_POLLS", "MI355_WQ_ONLY_CHUNK",
+                                            "MI355_QMM_STREAM_OUT"};
 std::atomic<int> g_knobs[kKnobCount];
 const bool g_knobs_loaded = []() {
     for (int i = 0; i < kKnobCount; i++) {

@@ -356,11 +356,14 @@ def test_quant_matmul_wide_loop_tiles(capi, golden, tile, M, K, N):
             assert np.array_equal(ref[10].cpu().numpy(), want_i8), (tile, split)
             for order in (2, 3):
                 capi.set_tuning("MI355_QMM_LOOP", order)
-                got = run_all()
-                for i, (a, b) in enumerate(zip(got, ref)):
-                    assert torch.equal(a, b), (tile, split, order, i)
+                for stream_out in (1, 2):                   # ordinary / non-temporal row stores of the 16-bit epilogue
+                    capi.set_tuning("MI355_QMM_STREAM_OUT", stream_out)
+                    got = run_all()
+                    for i, (a, b) in enumerate(zip(got, ref)):
+                        assert torch.equal(a, b), (tile, split, order, stream_out, i)
+                capi.set_tuning("MI355_QMM_STREAM_OUT", 0)
     finally:
-        for k in ("MI355_QMM_TILE", "MI355_QMM_SPLIT", "MI355_QMM_LOOP"):
+        for k in ("MI355_QMM_TILE", "MI355_QMM_SPLIT", "MI355_QMM_LOOP", "MI355_QMM_STREAM_OUT"):
             capi.set_tuning(k, 0)
 
 
