@@ -475,6 +475,44 @@ def test_quant_matmul_decode_kernel(capi, golden, M, K, N):
         capi.set_tuning("MI355_QMM_DECODE_OFF", 0)
 
 
+QMM_MID_ROWS = [33, 64, 65, 128, 192, 256]
+QMM_MID_PROJECTIONS = [(4096, 6144), (4096, 11008), (11008, 4096)]
+
+
+@pytest.mark.parametrize("K,N", QMM_MID_PROJECTIONS)
+@pytest.mark.parametrize("M", QMM_MID_ROWS)
+def test_quant_matmul_mid_rows(capi, golden, M, K, N):
+    """33 to 256 rows on the projections of a transformer layer, with whatever kernel, tile and split of K the planner
+    picks for them (the decode kernel up to 64 rows where the activations fit its registers, the streaming loop of the
+    64x128 tile, larger tiles with K split over workgroups): accumulators, the bf16 and fp16 epilogues with every bias
+    kind, and the re-quantised int8 output, bit-identical to the oracle."""
+    d = workloads.quant_matmul_inputs(seed=3 * M + K + N, M=M, K=K, N=N, weight_nk=True, bias=True)
+    g = torch.Generator().manual_seed(M + K)
+    bias_i32 = torch.randint(-(1 << 20), 1 << 20, (N,), generator=g, dtype=torch.int32)
+    bias_f32 = torch.randn(N, generator=g)
+    offset = torch.randint(-40, 40, (N,), generator=g).float()
+    x1, x2, sc, ps = d["x1"].cuda(), d["x2"].cuda(), d["scale"].cuda(), d["pertoken_scale"].cuda()
+    acc = golden.int8_gemm(d["x1"].numpy(), d["x2"].numpy())
+    assert np.array_equal(capi.quant_matmul(x1, x2, None, out_dtype=torch.int32).cpu().numpy(), acc)
+    for bias, dt, name, with_ps in [(d["bias"], torch.bfloat16, "bf16", True), (bias_i32, torch.bfloat16, "bf16", True),
+                                    (bias_f32, torch.float16, "fp16", True), (None, torch.bfloat16, "bf16", False)]:
+        out = capi.quant_matmul(x1, x2, sc, ps if with_ps else None, None if bias is None else bias.cuda(), out_dtype=dt)
+        bias_np = None if bias is None else (_bits(bias) if bias.dtype == torch.bfloat16 else bias.numpy())
+        want = golden.quant_matmul_epilogue_ex(acc, d["scale"].numpy(), d["pertoken_scale"].numpy() if with_ps else None, bias_np, out=name)
+        assert np.array_equal(out.cpu().view(torch.int16).numpy().view(np.uint16), want), (name, with_ps)
+    rq_scale = (torch.rand(N, generator=g) + 0.5) * (40.0 / (K ** 0.5 * 74 * 74))     # spreads the results over the int8 range
+    qp = capi.trans_quant_param(rq_scale.cuda(), offset.cuda())
+    got = capi.quant_matmul_qparam(x1, x2, qp, bias_i32.cuda())
+    want = golden.quant_matmul_requant(d["x1"].numpy(), d["x2"].numpy(), golden.trans_quant_param(rq_scale.numpy(), offset.numpy()),
+                                       bias_i32.numpy())
+    assert np.array_equal(got.cpu().numpy(), want)
+    assert np.abs(want.astype(np.int32)).max() > 20 and (np.abs(want.astype(np.int32)) < 127).mean() > 0.5
+    # a second launch on the same workspace (the first must have left its counters and exchange area clean)
+    again = capi.quant_matmul(x1, x2, sc, ps, d["bias"].cuda())
+    want = golden.quant_matmul_epilogue_ex(acc, d["scale"].numpy(), d["pertoken_scale"].numpy(), _bits(d["bias"]), out="bf16")
+    assert np.array_equal(_bits(again), want)
+
+
 @pytest.mark.parametrize("M,K,N,pad", [(8, 1024, 2049, 0), (16, 4096, 2054, 0), (5, 2048, 4096, 8), (64, 4096, 2049, 0)])
 def test_quant_matmul_decode_shapes_that_fall_back(capi, M, K, N, pad):
     """Decode-sized problems the decode kernel declines (N not a multiple of 4, activation rows whose pitch is not a
