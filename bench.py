@@ -768,6 +768,13 @@ def main():
 
     if others:
         result["others"] = others
+        # the same lines in short, inside `config` (a consumer that keeps only the contract's keys still sees them):
+        # [us per launch or chain, fraction of the bounding peak, us of a plain copy of the same bytes, oracle gate]
+        def gate(e):
+            flags = [v for k, v in e.items() if k.startswith("parity") and isinstance(v, bool)]
+            return all(flags) if flags else None
+        result["config"]["lines"] = {e["name"][:64]: [e.get("launch_us", e.get("chain_us", e.get("us"))), e.get("roofline", {}).get("frac"),
+                                                       e.get("roofline", {}).get("copy_ceiling_us"), gate(e)] for e in others}
     print(json.dumps(result))
 
 
