@@ -189,6 +189,10 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
                                (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_BF16) && (p.ldc & 7) == 0 &&
                                aligned_dev(p.out, 16) && aligned_dev(p.pertoken, 16) && aligned_dev(p.scale, 16) &&
                                (!p.bias || aligned_dev(p.bias, 16));
+    // ... and so does the one for the re-quantised int8 output with per-channel parameter words
+    const bool fast_epilogue_i8 = LOOP != 0 && p.out_i8 && p.qparam && p.scale_len == p.N &&
+                                  (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_INT32) && (p.ldc & 15) == 0 &&
+                                  aligned_dev(p.out, 16) && aligned_dev(p.qparam, 16) && (!p.bias || aligned_dev(p.bias, 16));
 
     if constexpr (LOOP != 0) {
         static_assert(WGM == 4 && WGN == 2 && WTM == 4 && NS == 3, "wide loop: 4 x 2 wavefronts of 64 rows");
@@ -197,6 +201,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         if (fast_epilogue && wave == 0)
             wide::request_params(lds, G::PARAM_BASE, p.pertoken, p.scale, p.bias_kind == MI355_BIAS_BF16 ? p.bias : nullptr, m0, n0,
                                  rows_a, rows_b, lane);
+        if (fast_epilogue_i8 && wave == 0)
+            wide::request_params_i8(lds, G::PARAM_BASE, p.qparam, p.bias_kind == MI355_BIAS_INT32 ? p.bias : nullptr, n0, rows_b, lane);
         const int frow = lane & 15;
         const uint32_t sw0 = (uint32_t)(((lane >> 4) ^ ((frow >> 1) & 7)) * 16);
         wide::LoopState st;
@@ -490,6 +496,20 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     }
 
     if constexpr (LOOP != 0) {
+        if (fast_epilogue_i8) {
+            wide::EpilogueArgs e;
+            e.out = p.out;
+            e.ldc = p.ldc;
+            e.M = p.M;
+            e.N = p.N;
+            e.m0 = m0;
+            e.n0 = n0;
+            e.has_bias = p.bias_kind == MI355_BIAS_INT32;
+            e.out_f16 = 0;
+            e.stream_out = p.stream_out;
+            wide::epilogue_fast_i8<WTN>(acc, lds, e, wave, lane);
+            return;
+        }
         if (fast_epilogue) {
             wide::EpilogueArgs e;
             e.out = p.out;
@@ -1119,7 +1139,7 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     // ordinary stores.  MI355_QMM_STREAM_OUT: 1 never, 2 always.
     {
         const int so = knob(kKnobQmmStreamOut);
-        const uint64_t out_bytes = (uint64_t)M * (uint64_t)N * 2u;
+        const uint64_t out_bytes = (uint64_t)M * (uint64_t)N * (out_i8 ? 1u : 2u);
         p.stream_out = so == 2 || (so != 1 && out_bytes <= kStreamOutMaxBytes);
     }
     const TileChoice c = pl.tile;

@@ -40,7 +40,7 @@ struct Geometry {
     static constexpr int B_BASE = 2 * A_BYTES;
     static constexpr int FLAG_BASE = B_BASE + 3 * B_BYTES;   // four flag words, one per pair of wavefronts
     static constexpr int PARAM_BASE = FLAG_BASE + 64;        // epilogue parameters (filled during the prologue): 2.5 KiB
-    static constexpr int LDS_BYTES = PARAM_BASE + 2560;
+    static constexpr int LDS_BYTES = PARAM_BASE + 3072;
 };
 
 // s_waitcnt vmcnt(VM) lgkmcnt(0) as the builtin, so that the compiler's own bookkeeping of outstanding LDS reads sees it
@@ -471,6 +471,94 @@ __device__ __forceinline__ void epilogue_fast(i32x4v (&acc)[4][WTN], char *lds, 
     } else {
         if (e.has_bias) go(F{}, T{});
         else go(F{}, F{});
+    }
+}
+
+// ---- the same for the re-quantised int8 output: clamp(rint(float(acc + int32 bias) * scale + offset)), scale and the
+// 9-bit offset from the packed 64-bit parameter words, each operation rounded to binary32.  The parameter words of the
+// tile's columns (2 KiB) and the int32 bias (1 KiB) are requested into LDS in front of the first K step; a wavefront
+// stages its whole tile (a lane owns one 32-bit word of four columns per 16x16 tile) and stores 16 bytes per lane.
+constexpr int PARAM_QP = 0, PARAM_BIAS32 = 2048;
+
+__device__ __forceinline__ void request_params_i8(char *lds, int param_base, const uint64_t *qparam, const void *bias_i32, int n0,
+                                                   int cols, int lane)
+{
+    const __amdgpu_buffer_rsrc_t r_q = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint64_t *>(qparam + n0), 0, cols * 8, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r_q, (lds_void *)(lds + param_base + PARAM_QP), 16, (uint32_t)lane * 16u, 0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r_q, (lds_void *)(lds + param_base + PARAM_QP + 1024), 16, (uint32_t)lane * 16u, 1024, 0, 0);
+    if (bias_i32) {
+        const __amdgpu_buffer_rsrc_t r_b = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<int32_t *>(static_cast<const int32_t *>(bias_i32) + n0), 0, cols * 4, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r_b, (lds_void *)(lds + param_base + PARAM_BIAS32), 16, (uint32_t)lane * 16u, 0, 0, 0);
+    }
+}
+
+template <int WTN, bool BIAS, bool NT>
+__device__ __forceinline__ void epilogue_rows_i8(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
+{
+    using G = Geometry<WTN>;
+    constexpr int ROWQ = WTN * 16 + 16;                       // padded pitch of a staged row of the wavefront tile
+    constexpr int CHQ = WTN;                                  // 16-byte chunks per row
+    const int wm = wave >> 1, wn = wave & 1;
+    const int mrow = lane & 15, nquad = (lane >> 4) * 4;
+    const char *par = lds + G::PARAM_BASE;
+    char *stq = lds + wave * (64 * ROWQ);
+#pragma unroll
+    for (int j = 0; j < WTN; j++) {
+        const int c = wn * WTN * 16 + j * 16 + nquad;
+        const u32x4 q01 = *reinterpret_cast<const u32x4 *>(par + PARAM_QP + c * 8);        // low, high words of columns c, c + 1
+        const u32x4 q23 = *reinterpret_cast<const u32x4 *>(par + PARAM_QP + c * 8 + 16);
+        const uint32_t lo[4] = {q01.x, q01.z, q23.x, q23.z}, hi[4] = {q01.y, q01.w, q23.y, q23.w};
+        i32x4v bi = i32x4v{0, 0, 0, 0};
+        if constexpr (BIAS) bi = *reinterpret_cast<const i32x4v *>(par + PARAM_BIAS32 + c * 4);
+        float sc[4], of[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            sc[r] = __uint_as_float(lo[r]);
+            of[r] = (float)(((int32_t)((hi[r] >> 5) << 23)) >> 23);                        // bits 37-45 of the 64: a 9-bit integer
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float v = (float)(int32_t)((uint32_t)acc[i][j][r] + (uint32_t)bi[r]);      // wraps like the accumulator
+                v = v * sc[r];
+                v = v + of[r];
+                v = fminf(fmaxf(rintf(v), -128.0f), 127.0f);
+                w |= ((uint32_t)(int32_t)v & 0xffu) << (8 * r);
+            }
+            *reinterpret_cast<uint32_t *>(stq + (i * 16 + mrow) * ROWQ + j * 16 + nquad) = w;
+        }
+    }
+    const int mw = e.m0 + wm * 64, nw = e.n0 + wn * WTN * 16;
+#pragma unroll
+    for (int q0 = 0; q0 < 64 * CHQ; q0 += 64) {
+        const int q = q0 + lane;
+        const int row = q / CHQ, ch = q % CHQ;
+        const int m = mw + row, n = nw + ch * 16;
+        if (m >= e.M || n >= e.N) continue;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(stq + row * ROWQ + ch * 16);
+        int8_t *o = static_cast<int8_t *>(e.out) + (int64_t)m * e.ldc + n;
+        if (n + 15 < e.N) {
+            if constexpr (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(o));
+            else *reinterpret_cast<u32x4 *>(o) = v;
+        } else {
+            for (int r = 0; r < 16; r++)
+                if (n + r < e.N) o[r] = (int8_t)(v[r >> 2] >> ((r & 3) * 8));
+        }
+    }
+}
+
+template <int WTN>
+__device__ __forceinline__ void epilogue_fast_i8(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
+{
+    if (e.has_bias) {
+        if (e.stream_out) epilogue_rows_i8<WTN, true, true>(acc, lds, e, wave, lane);
+        else epilogue_rows_i8<WTN, true, false>(acc, lds, e, wave, lane);
+    } else {
+        if (e.stream_out) epilogue_rows_i8<WTN, false, true>(acc, lds, e, wave, lane);
+        else epilogue_rows_i8<WTN, false, false>(acc, lds, e, wave, lane);
     }
 }
 

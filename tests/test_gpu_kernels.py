@@ -308,13 +308,15 @@ def test_quant_matmul_deep_ring_small_tiles(capi, golden, tile, M, K, N):
 
 
 @pytest.mark.parametrize("tile", [256192, 256224, 256256])
-@pytest.mark.parametrize("M,K,N", [(256, 128, 192), (300, 640, 500), (512, 4224, 1000), (1024, 1152, 2300), (255, 2048, 8 * 97)])
+@pytest.mark.parametrize("M,K,N", [(256, 128, 192), (300, 640, 500), (512, 4224, 1000), (1024, 1152, 2300), (255, 2048, 8 * 97),
+                                   (520, 1152, 16 * 129)])
 def test_quant_matmul_wide_loop_tiles(capi, golden, tile, M, K, N):
     """The 256-row tiles run the K loop with loader roles (activation slots released by an LDS flag between the two
     wavefronts that read them).  One K step, odd and even step counts, ragged rows and columns, with and without a split of
     K, both instruction orders: int32 accumulators bit-identical to the oracle, every epilogue (the LDS-parameter one for
-    per-token scale + bf16 bias / no bias in bf16 and fp16, and the general one for the other bias kinds, a single scale,
-    no per-token scale, int32 and re-quantised int8 outputs) bit-identical to the generic loop and to the oracle.  (The
+    per-token scale + bf16 bias / no bias in bf16 and fp16, the LDS-parameter one for the re-quantised int8 output when the
+    output rows are 16-byte aligned, and the general one for the other bias kinds, a single scale, no per-token scale, int32
+    and unaligned int8 outputs) bit-identical to the generic loop and to the oracle.  (The
     256x256 tile, which only has the generic loop, runs through the same cases against the oracle.)"""
     d = workloads.quant_matmul_inputs(seed=M + N + K, M=M, K=K, N=N, weight_nk=True, bias=True)
     g = torch.Generator().manual_seed(M + K)
@@ -341,7 +343,8 @@ def test_quant_matmul_wide_loop_tiles(capi, golden, tile, M, K, N):
                 capi.quant_matmul(x1, x2, one, ps, bias),
                 capi.quant_matmul(x1, x2, None, None, bias_i32, out_dtype=torch.int32),
                 capi.quant_matmul_qparam(x1, x2, qp, bias_i32),
-                capi.quant_matmul_qparam(x1, x2, qp, None, out_dtype=torch.bfloat16)]
+                capi.quant_matmul_qparam(x1, x2, qp, None, out_dtype=torch.bfloat16),
+                capi.quant_matmul_qparam(x1, x2, qp, None)]
 
     capi.set_tuning("MI355_QMM_TILE", tile)
     try:
