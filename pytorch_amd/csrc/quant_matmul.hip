@@ -72,7 +72,7 @@ struct QmmArgs {
     int out_i32;
     const uint64_t *qparam;    // packed quantisation parameters [scale_len] (replace `scale`), or null
     int out_i8;                // re-quantised int8 output (needs qparam)
-    int stream_out;            // 256-row tiles, 16-bit output: non-temporal row stores (chosen by the launcher)
+    int stream_out;            // 16-bit and int8 outputs with aligned rows: non-temporal row stores (chosen by the launcher)
     int tiles_m, tiles_n, tiles_per_xcd;
     int S;                     // workgroups that share the K range of a tile
     int32_t *partial;          // workspace [tile][chunk][wavefront][accumulator quad][lane] int32x4 (S > 1)
@@ -730,24 +730,27 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             if (fast) stage_tile(F{}, T{}); else stage_tile(F{}, F{});
         }
         const int mw = m0 + wm * WTM * 16, nw = n0 + wn * WTN * 16;
+        // the kind of store is a compile-time choice (a run-time choice between the two is merged into ordinary stores)
+        auto store_rows = [&](auto nt_c) {
 #pragma unroll
-        for (int q0 = 0; q0 < WTM * 16 * CHUNKS; q0 += 64) {
-            const int q = q0 + lane;
-            const int row = q / CHUNKS, ch = q % CHUNKS;
-            if ((WTM * 16 * CHUNKS) % 64 != 0 && row >= WTM * 16) continue;
-            const int m = mw + row, n = nw + ch * 8;
-            if (m >= p.M || n >= p.N) continue;
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(stg + row * ROWB + ch * 16);
-            uint16_t *o = static_cast<uint16_t *>(p.out) + (int64_t)m * p.ldc + n;
-            if (n + 7 < p.N) {
-                *reinterpret_cast<u32x4 *>(o) = v;
-            } else {
-                const uint16_t *e = reinterpret_cast<const uint16_t *>(&v);
-                for (int r = 0; r < 8; r++)
-                    if (n + r < p.N) o[r] = (uint16_t)(v[r >> 1] >> ((r & 1) * 16));
-                (void)e;
+            for (int q0 = 0; q0 < WTM * 16 * CHUNKS; q0 += 64) {
+                const int q = q0 + lane;
+                const int row = q / CHUNKS, ch = q % CHUNKS;
+                if ((WTM * 16 * CHUNKS) % 64 != 0 && row >= WTM * 16) continue;
+                const int m = mw + row, n = nw + ch * 8;
+                if (m >= p.M || n >= p.N) continue;
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(stg + row * ROWB + ch * 16);
+                uint16_t *o = static_cast<uint16_t *>(p.out) + (int64_t)m * p.ldc + n;
+                if (n + 7 < p.N) {
+                    if constexpr (decltype(nt_c)::value) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(o));
+                    else *reinterpret_cast<u32x4 *>(o) = v;
+                } else {
+                    for (int r = 0; r < 8; r++)
+                        if (n + r < p.N) o[r] = (uint16_t)(v[r >> 1] >> ((r & 1) * 16));
+                }
             }
-        }
+        };
+        if (p.stream_out) store_rows(T{}); else store_rows(F{});
         return;
     }
     const bool vec = (p.ldc & 3) == 0 && aligned_dev(p.out, 8);
