@@ -630,6 +630,19 @@ def main():
                                             "unit": "GB/s", "frac": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                                             "traffic": _traffic(f"qd_{Kx}x{Nx}_m{Mx}"), "copy_ceiling_us": copy_ceiling_us(nb)},
                                "algorithmic_bytes": int(nb)})
+                if Kx == 4096 and Mx == 16:
+                    # the same launch on weights prepared once (pytorch_amd.prepare_quant_matmul_weight: rows of 4096
+                    # bytes get a pitch of 4224)
+                    wsp = [pa.prepare_quant_matmul_weight(w) for w in wsn]
+                    keep = []
+                    calls = [(lambda a=a, w=w: keep.append(pa.npu_quant_matmul(a, w, sc, pertoken_scale=ps, output_dtype=torch.bfloat16)))
+                             for a, w in zip(xs, wsp)] * 2
+                    usp = _graph_time_us(torch, calls, reps=10)
+                    same = bool(torch.equal(pa.npu_quant_matmul(xs[0], wsp[0], sc, pertoken_scale=ps, output_dtype=torch.bfloat16),
+                                            pa.npu_quant_matmul(xs[0], wsn[0], sc, pertoken_scale=ps, output_dtype=torch.bfloat16)))
+                    others[-1]["prepared_weight_us"] = round(usp, 3)
+                    others[-1]["prepared_weight_bit_identical"] = same
+                    del wsp
                 del xs, keep
             del wsn
 

@@ -65,16 +65,22 @@ class _QuantLinearBase(PreparedCopiesMixin, nn.Module):
                              f"but now it is {self.output_dtype}.")
 
     def prepare_(self) -> "_QuantLinearBase":
-        """One-time widening for inference (optional, A4W4 only): a weight stored as int32 words of eight int4 values is
+        """One-time pre-layout for inference (optional).  A4W4: a weight stored as int32 words of eight int4 values is
         widened to int8 ``[out_features, in_features]`` once, so that a forward pass widens only the activations before
-        the int8 GEMM instead of the weight as well.  The parameter the module exposes (and its state_dict) stays as it
-        is; the widened copy is a plain attribute that costs twice the packed weight's size.  Moving, casting or
-        reloading the module drops the copy (forward then widens per call again); call this again afterwards, and
-        after changing the weight in place."""
+        the int8 GEMM instead of the weight as well.  W8A8 with ``in_features`` = 4096: the weight is copied into rows
+        with a padded pitch (``pytorch_amd.prepare.padded_row_bytes``), which the decode kernels read 8-15 % faster.
+        The parameter the module exposes (and its state_dict) stays as it is; the copy is a plain attribute that costs
+        the int8 weight's size.  Moving, casting or reloading the module drops the copy; call this again afterwards,
+        and after changing the weight in place."""
         self._prepared_i8 = None
+        from ...prepare import prepare_quant_matmul_weight
         if self.weight.dtype == torch.int32:
             from ... import _capi
-            self._prepared_i8 = _capi.unpack_int4(self.weight.data)
+            self._prepared_i8 = prepare_quant_matmul_weight(_capi.unpack_int4(self.weight.data).t()).t()
+        elif self.weight.dtype == torch.int8:
+            prepared = prepare_quant_matmul_weight(self.weight.data.t()).t()
+            if prepared.data_ptr() != self.weight.data_ptr():
+                self._prepared_i8 = prepared
         return self
 
     def forward(self, linear_quant_input: torch.Tensor) -> torch.Tensor:
@@ -86,6 +92,8 @@ class _QuantLinearBase(PreparedCopiesMixin, nn.Module):
             x = linear_quant_input
             words = x.shape[-1]
             linear_quant_input = _capi.unpack_int4(x.reshape(-1, words).contiguous()).view(*x.shape[:-1], words * 8)
+            weight = prepared
+        elif prepared is not None and linear_quant_input.dtype == torch.int8 and self.weight.dtype == torch.int8:
             weight = prepared
         scale = self.scale
         # a float32 scale is packed with npu_trans_quant_param when there is no pertoken_scale and the output is int8

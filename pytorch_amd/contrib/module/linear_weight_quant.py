@@ -42,11 +42,19 @@ class LinearWeightQuant(PreparedCopiesMixin, nn.Module):
     @torch.no_grad()
     def prepare_(self) -> "LinearWeightQuant":
         """One-time repack for inference (optional): an int4 weight is rewritten with its words along N and per-group
-        parameters are made row-major ``[G, N]``, the layout the decode kernels stream fastest.  The parameters the
+        parameters are made row-major ``[G, N]``, the layout the decode kernels stream fastest; an int8 weight with
+        ``in_features`` = 4096 is copied into rows with a padded pitch.  The parameters the
         module exposes (and its state_dict) stay as they are; the prepared copies are plain attributes, so they cost
         the weight's size again.  Moving, casting or reloading the module drops them; call this again afterwards, and
         after changing a parameter in place."""
         self._prepared = None
+        if self.weight.dtype == torch.int8:
+            # rows of 4096 bytes get a padded pitch (pytorch_amd.prepare.padded_row_bytes); other weights stay as they are
+            from ...prepare import prepare_weight_quant_weight
+            kn = prepare_weight_quant_weight(self.weight.data.t())
+            if kn.data_ptr() != self.weight.data_ptr():
+                self._prepared = (kn, self._as_group_major(self.antiquant_scale), self._as_group_major(self.antiquant_offset))
+            return self
         if self.weight.dtype != torch.int32:
             return self
         w = self.weight                                             # [N, K/8], word j of a row holds k = 8j..8j+7

@@ -517,6 +517,52 @@ def test_prepared_quant_matmul_weight(pa, golden):
     assert torch.equal(wrp, wr) and wrp.stride()[-2:] == (1, 40)
 
 
+@pytest.mark.parametrize("M", [1, 16, 64, 128, 1024])
+def test_prepared_weights_with_padded_row_pitch(pa, golden, M):
+    """Weights whose rows are 4096 bytes are prepared with a row pitch of 4224: every kernel that a row count selects
+    (decode, streaming loop, 256-row tiles) reads them through the pitch and returns the bits of the unprepared call,
+    which equal the oracle's; the modules keep such a copy after prepare_()."""
+    from pytorch_amd.contrib.module import LinearQuant, LinearWeightQuant
+    from pytorch_amd.testing import workloads
+    K, N = 4096, 1536
+    d = workloads.quant_matmul_inputs(seed=M, M=M, K=K, N=N, weight_nk=True, bias=True)
+    x1, w = d["x1"].cuda(), d["x2"].cuda()
+    wp = pa.prepare_quant_matmul_weight(w)
+    assert wp.stride() == (1, 4224) and torch.equal(wp, w) and pa.prepare_quant_matmul_weight(wp) is wp
+    assert pa.prepare_quant_matmul_weight(w, row_pad=False) is w
+    kw = dict(pertoken_scale=d["pertoken_scale"].cuda(), bias=d["bias"].cuda(), output_dtype=torch.bfloat16)
+    out = pa.npu_quant_matmul(x1, wp, d["scale"].cuda(), **kw)
+    want, _ = golden.quant_matmul(d["x1"].numpy(), d["x2"].numpy(), d["scale"].numpy(), d["pertoken_scale"].numpy(), _bits(d["bias"]))
+    assert np.array_equal(_bits(out), want)
+    assert torch.equal(pa.npu_quant_matmul(x1, wp, None, output_dtype=torch.int32), pa.npu_quant_matmul(x1, w, None, output_dtype=torch.int32))
+    # a contiguous [K, N] weight: transposed and padded in one preparation
+    wkn = w.contiguous()
+    wkp = pa.prepare_quant_matmul_weight(wkn)
+    assert wkp.stride() == (1, 4224) and torch.equal(wkp, wkn)
+    assert torch.equal(pa.npu_quant_matmul(x1, wkp, d["scale"].cuda(), **kw), out)
+    # the module keeps the padded copy and gives the same result with and without it
+    m = LinearQuant(K, N, bias=True, pertoken_scale=True, output_dtype=torch.bfloat16).cuda()
+    m.weight.data = w.t().contiguous()
+    m.scale.data = d["scale"].cuda()
+    m.pertoken_scale.data = d["pertoken_scale"].cuda()
+    m.bias.data = d["bias"].cuda()
+    ref = m(x1)
+    assert torch.equal(ref, out)
+    m.prepare_()
+    assert m._prepared_i8 is not None and m._prepared_i8.stride() == (4224, 1)
+    assert torch.equal(m(x1), ref)
+    if M <= 64:
+        dw = workloads.w8a16_inputs(seed=M, M=M, K=K, N=N)
+        lw = LinearWeightQuant(K, N, bias=False, antiquant_offset=True)
+        lw.weight.data = dw["weight"].t().contiguous()
+        lw.antiquant_scale.data, lw.antiquant_offset.data = dw["antiquant_scale"], dw["antiquant_offset"]
+        lw = lw.cuda()
+        ref = lw(dw["x"].cuda())
+        lw.prepare_()
+        assert lw._prepared is not None and lw._prepared[0].stride() == (1, 4224)
+        assert torch.equal(lw(dw["x"].cuda()), ref)
+
+
 def test_workspace_outlives_growth_after_capture(pa):
     """A graph captured with a small split-K workspace must replay correctly after an eager call on the same stream
     needed a larger one: the superseded buffer is kept alive (and zeroed at rest), never handed back to the allocator."""
@@ -625,15 +671,19 @@ def test_prepare_weight_quant_weight(pa):
     from pytorch_amd.testing import workloads, bf16_gate
     d = workloads.w8a16_inputs(seed=5, M=16, K=4096, N=2304)
     w = d["weight"].cuda()
-    wp = pa.prepare_weight_quant_weight(w)
+    wp = pa.prepare_weight_quant_weight(w, row_pad=False)
     assert wp.shape == w.shape and wp.stride() == (1, 4096) and torch.equal(wp, w)
-    assert pa.prepare_weight_quant_weight(wp) is wp
+    assert pa.prepare_weight_quant_weight(wp, row_pad=False) is wp
+    wpp = pa.prepare_weight_quant_weight(w)                              # rows of 4096 bytes: padded pitch by default
+    assert wpp.stride() == (1, 4224) and torch.equal(wpp, w) and pa.prepare_weight_quant_weight(wpp) is wpp
+    assert torch.equal(pa.prepare_weight_quant_weight(wp), w) and pa.prepare_weight_quant_weight(wp).stride() == (1, 4224)
     words = torch.zeros(64, 8, dtype=torch.int32, device="cuda")
     assert pa.prepare_weight_quant_weight(words) is words
     x, sc, of = d["x"].cuda(), d["antiquant_scale"].cuda(), d["antiquant_offset"].cuda()
     ref = pa.npu_weight_quant_batchmatmul(x, w, sc, of)
     out = pa.npu_weight_quant_batchmatmul(x, wp, sc, of)
     bf16_gate(out, ref.float().cpu())
+    assert torch.equal(pa.npu_weight_quant_batchmatmul(x, wpp, sc, of), out)     # the pitch changes no bit
 
 
 def test_linear_weight_quant_reference_test_shape(pa):
