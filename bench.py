@@ -738,6 +738,14 @@ def main():
                      "algorithmic_bytes": int(abytes)}
                 if fn is mlp_fused:
                     e["bit_identical_to_5_kernel_chain"] = same
+                    if Mx <= 64:
+                        # the same chain on weights prepared once (rows of 4096 bytes get a padded pitch)
+                        wprep = [(pa.prepare_quant_matmul_weight(wg), wdn) for wg, wdn in wsets]
+                        keep.clear()
+                        e["chain_us_prepared_weights"] = round(_graph_time_us(
+                            torch, [(lambda w=w: keep.append(fn(*w))) for w in wprep] * 2, reps=10), 2)
+                        e["prepared_weights_bit_identical"] = bool(torch.equal(fn(*wprep[0]), fn(*wsets[0])))
+                        del wprep
                 elif gate:
                     e["parity_stagewise"] = gate
                     e["parity_all_stages"] = bool(all(v for k, v in gate.items() if k not in ("swiglu_bit_identical_frac", "rows_checked")))
