@@ -568,8 +568,16 @@ def main():
                 tf = 2.0 * Mx * Kx * Nx / (us * 1e-6) / 1e12
                 e["roofline_mfma"] = {"bound": "mfma", "achieved": round(tf, 1), "peak": BF16_PEAK_TFLOPS,
                                       "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4), "traffic": None}
+            # the same launches on weights prepared once (pytorch_amd.prepare_weight_quant_weight: rows of 7168 bytes get a
+            # padded pitch; values and layout are unchanged)
+            wsp = [pa.prepare_weight_quant_weight(w) for w in ws]
+            keep.clear()
+            e["prepared_weight_us"] = round(_graph_time_us(
+                torch, [(lambda w=w: keep.append(pa.npu_weight_quant_batchmatmul(x, w, s4, o4, None, None, None, 128))) for w in wsp] * 2), 3)
+            e["prepared_weight_bit_identical"] = bool(torch.equal(pa.npu_weight_quant_batchmatmul(x, wsp[0], s4, o4, None, None, None, 128),
+                                                                  pa.npu_weight_quant_batchmatmul(x, ws[0], s4, o4, None, None, None, 128)))
             others.append(e)
-            del ws, keep
+            del ws, wsp, keep
             # the layout torch_npu's LinearWeightQuant passes: weight stored [N, K/8] (words along K), per-group
             # parameters stored [N, G], all three given as transposed views
             wks = [torch.randint(-2 ** 31, 2 ** 31 - 1, (Nx, Kx // 8), generator=gen, dtype=torch.int32, device=dev).t()

@@ -63,6 +63,8 @@ class LinearWeightQuant(PreparedCopiesMixin, nn.Module):
         kn = nib.reshape(w.shape[0], -1).t().contiguous()           # [K, N]
         words = (kn.reshape(kn.shape[0], -1, 8) << shifts).sum(-1)  # [K, N/8]: word j of a row holds n = 8j..8j+7
         prepared_w = words.to(torch.int32)                          # wraps modulo 2**32: bit 31 becomes the sign
+        from ...prepare import prepare_weight_quant_weight
+        prepared_w = prepare_weight_quant_weight(prepared_w)        # row padding where the pitch calls for it
         group_major = lambda t: None if t is None else self._as_group_major(t).contiguous()  # noqa: E731
         self._prepared = (prepared_w, group_major(self.antiquant_scale), group_major(self.antiquant_offset))
         return self
