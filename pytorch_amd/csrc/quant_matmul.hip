@@ -105,7 +105,8 @@ __device__ __forceinline__ int32_t requant1(int32_t a, int32_t bi, float sc, flo
 }
 
 // WGM x WGN wavefronts per workgroup, each owning (16*WTM) x (16*WTN) of the output tile.
-// LOOP 0: the generic K loop below; 1, 2: the loop of quant_matmul_wide.h (4 x 2 wavefronts of 64 rows) with its
+// LOOP 0: the generic K loop below; 3: the same with as many activation slots as weight slots (whole stages requested
+// NS steps ahead); 1, 2: the loop of quant_matmul_wide.h (4 x 2 wavefronts of 64 rows) with its
 // instruction order 0 (refills in a block) or 1 (refills spread over the step)
 template <int WGM, int WGN, int WTM, int WTN, int NS, int LOOP = 0>
 __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
@@ -116,7 +117,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     constexpr int UNITS_BP = (UNITS_B + NW - 1) / NW * NW;
     constexpr int LA = UNITS_A / NW, LB = UNITS_BP / NW;     // loads of a wavefront per activation / weight stage
     constexpr int A_BYTES = UNITS_A * 1024, B_BYTES = UNITS_BP * 1024;
-    constexpr int NSA = NS >= 4 ? NS : 2;                    // activation slots; NS weight slots follow them in LDS
+    constexpr bool WIDE = LOOP == 1 || LOOP == 2;
+    constexpr bool WHOLE = NS >= 4 || LOOP == 3;             // whole stages: activations get NS slots as well
+    constexpr int NSA = WHOLE ? NS : 2;                      // activation slots; NS weight slots follow them in LDS
     constexpr uint32_t kOutOfRange = 0x80000000u;            // lane offset beyond every buffer: the load writes zeros
     static_assert(UNITS_A % NW == 0, "A units must divide evenly over the wavefronts");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -185,16 +188,16 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         for (int j = 0; j < WTN; j++) acc[i][j] = i32x4v{0, 0, 0, 0};
 
     // the wide loop's epilogue for the common case takes its parameters from LDS (quant_matmul_wide.h)
-    const bool fast_epilogue = LOOP != 0 && !p.out_i32 && !p.out_i8 && !p.qparam && p.pertoken && p.scale_len == p.N &&
+    const bool fast_epilogue = WIDE && !p.out_i32 && !p.out_i8 && !p.qparam && p.pertoken && p.scale_len == p.N &&
                                (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_BF16) && (p.ldc & 7) == 0 &&
                                aligned_dev(p.out, 16) && aligned_dev(p.pertoken, 16) && aligned_dev(p.scale, 16) &&
                                (!p.bias || aligned_dev(p.bias, 16));
     // ... and so does the one for the re-quantised int8 output with per-channel parameter words
-    const bool fast_epilogue_i8 = LOOP != 0 && p.out_i8 && p.qparam && p.scale_len == p.N &&
+    const bool fast_epilogue_i8 = WIDE && p.out_i8 && p.qparam && p.scale_len == p.N &&
                                   (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_INT32) && (p.ldc & 15) == 0 &&
                                   aligned_dev(p.out, 16) && aligned_dev(p.qparam, 16) && (!p.bias || aligned_dev(p.bias, 16));
 
-    if constexpr (LOOP != 0) {
+    if constexpr (WIDE) {
         static_assert(WGM == 4 && WGN == 2 && WTM == 4 && NS == 3, "wide loop: 4 x 2 wavefronts of 64 rows");
         using G = wide::Geometry<WTN>;
         if (threadIdx.x < 16) reinterpret_cast<uint32_t *>(lds + G::FLAG_BASE)[threadIdx.x] = 0u;
@@ -390,8 +393,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     issue_b(0, KT);
     issue_a(1, KT);
     issue_b(1, KT);
-    if constexpr (NS == 3) issue_b(2, KT);
-    if constexpr (NS >= 4) {
+    if constexpr (NS == 3 && !WHOLE) issue_b(2, KT);
+    if constexpr (WHOLE) {
 #pragma unroll
         for (int st = 2; st < NS; st++) {
             issue_a(st, KT);
@@ -405,7 +408,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     MI355_READ_FRAGS(af0, bf0, 0, 0)
 
     for (int kt = 0; kt < KT; kt++) {
-        if constexpr (NS == 3 && WTM * WTN > 16) {
+        if constexpr (NS == 3 && WTM * WTN > 16 && !WHOLE) {
             MI355_READ_FRAGS(af1, bf1, kt, 1)
             MI355_MFMA_BLOCK(af0, bf0)
             MI355_INTERLEAVE(0, 2)
@@ -425,7 +428,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             __builtin_amdgcn_sched_barrier(0);
             MI355_MFMA_BLOCK(af0, bf0)
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (NS >= 4) wait_vmcnt_lgkm0<(NS - 2) * (LA + LB)>();   // stage kt+1 has landed, NS-2 more may be in flight
+            if constexpr (WHOLE) wait_vmcnt_lgkm0<(NS - 2) * (LA + LB)>();     // stage kt+1 has landed, NS-2 more may be in flight
             else wait_vmcnt_lgkm0<(NS - 2) * LB>();
             __syncthreads();
             issue_a(kt + NSA, KT);
@@ -495,7 +498,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         if (threadIdx.x == 0) __hip_atomic_store(p.counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
-    if constexpr (LOOP != 0) {
+    if constexpr (WIDE) {
         if (fast_epilogue_i8) {
             wide::EpilogueArgs e;
             e.out = p.out;
@@ -880,7 +883,7 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     constexpr int NS = DEEP < 0 ? 0 : DEEP ? DEEP : 2 * a_bytes + 2 * b_bytes <= 80 * 1024 && staging_bytes <= 80 * 1024 ? 2 : 3;
     // DEEP < 0: the streaming K loop (two activation chunks of 32 KiB and a 4 KiB turn-around tile per wavefront)
     constexpr size_t stage_bytes = DEEP < 0 ? (size_t)2 * 32768 + 8 * 4096 : (DEEP ? DEEP : 2) * a_bytes + NS * b_bytes;
-    constexpr size_t ring_bytes = LOOP != 0 ? (size_t)wide::Geometry<WTN>::LDS_BYTES : stage_bytes;
+    constexpr size_t ring_bytes = LOOP == 1 || LOOP == 2 ? (size_t)wide::Geometry<WTN>::LDS_BYTES : stage_bytes;
     constexpr size_t lds_bytes = ring_bytes > staging_bytes ? ring_bytes : staging_bytes;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -899,13 +902,18 @@ int launch_qmm(QmmArgs p, hipStream_t s)
 // Tile shapes (rows x columns of the workgroup tile) the library instantiates, with measured times at K = 4096
 // on operands that are not cache resident: `slots` workgroups are resident at once (256 CUs x 1 or 2), a launch
 // that fits in one round of them takes `single_us` in all, longer launches take `round_us` per round.
+// `whole`: the variant of a 128-row tile that keeps three whole stages (as many activation slots as weight slots) and
+// has a CU to itself: its activation refills get two K steps to land instead of one, which is what a tile needs when no
+// second workgroup on the CU covers the wait (128x192 at K = 4096: 37.2 -> 31.6 us per round, 128x128: 33.0 -> 24.7).
 struct TileChoice {
     int bm, bn, slots;
     double single_us, round_us;
+    int whole;
 };
-constexpr TileChoice kTiles[] = {{256, 256, 256, 60.0, 57.0}, {256, 224, 256, 55.5, 55.5}, {256, 192, 256, 51.5, 52.5},
-                                 {128, 320, 256, 48.0, 43.0}, {128, 256, 256, 40.0, 45.6}, {128, 192, 512, 55.8, 58.8},
-                                 {128, 128, 512, 40.0, 43.3}, {64, 256, 512, 40.0, 52.6},  {64, 128, 512, 24.0, 30.0}};
+constexpr TileChoice kTiles[] = {{256, 256, 256, 58.0, 59.0, 0}, {256, 224, 256, 52.5, 52.0, 0}, {256, 192, 256, 44.5, 45.5, 0},
+                                 {128, 320, 256, 48.0, 43.0, 0}, {128, 256, 256, 40.0, 45.6, 0}, {128, 192, 512, 55.8, 58.8, 0},
+                                 {128, 128, 512, 40.0, 43.3, 0}, {64, 256, 512, 40.0, 52.6, 0},  {64, 128, 512, 24.0, 30.0, 0},
+                                 {128, 192, 256, 32.0, 32.0, 1}, {128, 128, 256, 24.0, 24.8, 1}};
 
 // Workspace layout: [arrival counters | split-K partial sums | transposed weight].
 struct QmmPlan {
@@ -927,6 +935,9 @@ constexpr size_t kMaxPartialBytes = (size_t)128 << 20;
 constexpr uint64_t kStreamOutMaxBytes = (uint64_t)32 << 20;     // the L2s of the eight XCDs together
 constexpr double kBaseUs = 6.0, kL2BytesPerUs = 12e6, kExchangeUs = 1.0, kExchangeBytesPerUs = 10e6, kCollectorBytesPerUs = 100e3;
 constexpr double kAloneOnCu = 0.85;
+// a split of a whole-stage tile measured 2-4 us above what the terms below give (its partial sums are 64-96 KiB per
+// workgroup); and of two plans with the same estimate the one that leaves fewer CUs idle is the faster one
+constexpr double kWholeSplitUs = 3.0, kIdleCuUs = 2.0;
 
 void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size_t partial_cap, TileChoice *tile, int *split)
 {
@@ -938,6 +949,8 @@ void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size
     *split = 1;
     for (const TileChoice &c : kTiles) {
         if (forced_tile && (c.bm != forced_tile / 1000 || c.bn != forced_tile % 1000)) continue;
+        if (c.whole && knob(kKnobQmmLoop) == 1) continue;   // MI355_QMM_LOOP = 1: only the generic loop with its usual rings
+        if (!c.whole && knob(kKnobQmmLoop) == 4 && c.bm == 128 && (c.bn == 128 || c.bn == 192)) continue;   // 4: only their whole-stage variants
         const int64_t tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
         for (const int S : {1, 2, 3, 4, 6, 8, 12, 16}) {
             if (forced_split >= 1 && forced_split <= kt && may_split) {
@@ -968,7 +981,8 @@ void choose_tile_and_split(int64_t M, int64_t N, int64_t K, bool may_split, size
             if (l2 > cost) cost = l2;
             if (s_eff > 1)
                 cost += kExchangeUs + (double)wgs * c.bm * c.bn * 8.0 / kExchangeBytesPerUs +
-                        (double)(s_eff - 1) * c.bm * c.bn * 4.0 / kCollectorBytesPerUs;
+                        (double)(s_eff - 1) * c.bm * c.bn * 4.0 / kCollectorBytesPerUs + (c.whole ? kWholeSplitUs : 0.0);
+            if (wgs < 256) cost += kIdleCuUs * (1.0 - (double)wgs / 256.0);
             if (cost < best_cost) {
                 best_cost = cost;
                 *tile = c;
@@ -1156,7 +1170,7 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     if (c.bm == bm_ && c.bn == bn_) return launch_qmm<wgm_, wgn_, bm_ / (16 * wgm_), bn_ / (16 * wgn_)>(p, s);
     MI355_QMM_CASE(256, 256, 2, 4)
     {
-        const int lk = knob(kKnobQmmLoop);                 // 0: automatic; 1: the generic loop; 2, 3: the wide loop with refills in a block / spread
+        const int lk = knob(kKnobQmmLoop);                 // 0: automatic; 1: the generic loop; 2, 3: the wide loop with refills in a block / spread; 4: see the planner
         if (lk != 1) {
             if (c.bm == 256 && c.bn == 224) return lk == 2 ? launch_qmm<4, 2, 4, 7, 0, 1>(p, s) : launch_qmm<4, 2, 4, 7, 0, 2>(p, s);
             if (c.bm == 256 && c.bn == 192) return lk == 2 ? launch_qmm<4, 2, 4, 6, 0, 1>(p, s) : launch_qmm<4, 2, 4, 6, 0, 2>(p, s);
@@ -1164,6 +1178,11 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     }
     MI355_QMM_CASE(256, 224, 4, 2)
     MI355_QMM_CASE(256, 192, 4, 2)
+    if (c.whole) {
+        if (c.bm == 128 && c.bn == 192) return launch_qmm<2, 4, 4, 3, 3, 3>(p, s);
+        if (c.bm == 128 && c.bn == 128) return launch_qmm<2, 4, 4, 2, 3, 3>(p, s);
+        return MI355_ERR_UNSUPPORTED;
+    }
     MI355_QMM_CASE(128, 320, 2, 4)
     MI355_QMM_CASE(128, 256, 2, 4)
     MI355_QMM_CASE(128, 192, 2, 4)

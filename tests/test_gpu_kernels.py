@@ -307,7 +307,7 @@ def test_quant_matmul_deep_ring_small_tiles(capi, golden, tile, M, K, N):
             capi.set_tuning(k, 0)
 
 
-@pytest.mark.parametrize("tile", [256192, 256224, 256256])
+@pytest.mark.parametrize("tile", [256192, 256224, 256256, 128128, 128192])
 @pytest.mark.parametrize("M,K,N", [(256, 128, 192), (300, 640, 500), (512, 4224, 1000), (1024, 1152, 2300), (255, 2048, 8 * 97),
                                    (520, 1152, 16 * 129)])
 def test_quant_matmul_wide_loop_tiles(capi, golden, tile, M, K, N):
@@ -317,7 +317,8 @@ def test_quant_matmul_wide_loop_tiles(capi, golden, tile, M, K, N):
     per-token scale + bf16 bias / no bias in bf16 and fp16, the LDS-parameter one for the re-quantised int8 output when the
     output rows are 16-byte aligned, and the general one for the other bias kinds, a single scale, no per-token scale, int32
     and unaligned int8 outputs) bit-identical to the generic loop and to the oracle.  (The
-    256x256 tile, which only has the generic loop, runs through the same cases against the oracle.)"""
+    256x256 tile, which only has the generic loop, runs through the same cases against the oracle; the 128x128 and 128x192
+    tiles run their variant with three whole stages, MI355_QMM_LOOP = 4, against their usual rings.)"""
     d = workloads.quant_matmul_inputs(seed=M + N + K, M=M, K=K, N=N, weight_nk=True, bias=True)
     g = torch.Generator().manual_seed(M + K)
     x1, x2, sc, ps, bias = (d[k].cuda() for k in ("x1", "x2", "scale", "pertoken_scale", "bias"))
@@ -357,7 +358,7 @@ def test_quant_matmul_wide_loop_tiles(capi, golden, tile, M, K, N):
             assert np.array_equal(ref[0].cpu().numpy(), acc_want), (tile, split)
             assert np.array_equal(_bits(ref[1]), want_bf16), (tile, split)
             assert np.array_equal(ref[10].cpu().numpy(), want_i8), (tile, split)
-            for order in (2, 3):
+            for order in ((2, 3) if tile >= 256000 else (4,)):
                 capi.set_tuning("MI355_QMM_LOOP", order)
                 for stream_out in (1, 2):                   # ordinary / non-temporal row stores of the 16-bit epilogue
                     capi.set_tuning("MI355_QMM_STREAM_OUT", stream_out)
