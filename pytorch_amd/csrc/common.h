@@ -48,10 +48,25 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 // float32, result = bf16(float(s) * float(b)).
 __device__ __forceinline__ float silu_f32(float a) { return a / (1.0f + expf(-a)); }
 
+// bf16(silu(a)) for an `a` that is itself a bf16 value, returned as a float.  Exponential and division through the
+// hardware's exp2 and reciprocal are a few units in the last place of binary32 off, which changes the bf16 result only
+// when the value lies next to a rounding boundary of bf16: those (lower 16 bits within 16 of 0x8000: one value in 2048),
+// arguments beyond +-8 (the rounding error of a * log2(e) grows with |a|, and far below zero the reciprocal leaves the
+// normal range) and NaN take the exact formula.  There are only 65536 arguments: tests compare all of them with the
+// exact formula and with the oracle.
+__device__ __forceinline__ float silu_bf16(float a)
+{
+    const float e = __builtin_amdgcn_exp2f(a * -1.44269504088896340736f);
+    float s = a * __builtin_amdgcn_rcpf(1.0f + e);
+    const uint32_t lo = __float_as_uint(s) & 0xffffu;
+    if (__builtin_expect((lo - 0x7ff0u) < 0x20u || !(fabsf(a) <= 8.0f), 0)) s = silu_f32(a);
+    return bf16_1(f32_to_bf16(s));
+}
+
 __device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2)
 {
-    const float s0 = bf16_1(f32_to_bf16(silu_f32(bf16_lo(a2))));
-    const float s1 = bf16_1(f32_to_bf16(silu_f32(bf16_hi(a2))));
+    const float s0 = silu_bf16(bf16_lo(a2));
+    const float s1 = silu_bf16(bf16_hi(a2));
     return pack_bf16x2(s0 * bf16_lo(b2), s1 * bf16_hi(b2));
 }
 

@@ -353,7 +353,7 @@ __global__ __launch_bounds__(kBlock) void swiglu_dq_generic_kernel(const uint16_
     const int64_t row = blockIdx.x;
     const uint16_t *xr = x + row * row_stride;
     auto value = [&](int64_t j) {
-        const float sl = bf16_1(f32_to_bf16(silu_f32(bf16_1(xr[act_off + j]))));
+        const float sl = silu_bf16(bf16_1(xr[act_off + j]));
         const float v = bf16_1(f32_to_bf16(sl * bf16_1(xr[mul_off + j])));
         return smooth ? v * bf16_1(smooth[j]) : v;
     };

@@ -32,7 +32,7 @@ __global__ __launch_bounds__(256) void swiglu_scalar_kernel(const uint16_t *__re
     for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
         const int64_t r = e / half, j = e % half;
         const float a = bf16_1(x[r * ldx + j]), b = bf16_1(x[r * ldx + half + j]);
-        const float s = bf16_1(f32_to_bf16(silu_f32(a)));
+        const float s = silu_bf16(a);
         out[e] = f32_to_bf16(s * b);
     }
 }

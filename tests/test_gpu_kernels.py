@@ -1042,6 +1042,35 @@ def test_swiglu(capi, golden):
         assert dist.max() <= 1 and (dist == 0).mean() > 0.995   # device expf vs libm expf
 
 
+def test_swiglu_every_bf16_argument(capi, golden):
+    """silu is evaluated on bf16 arguments and rounded to bf16, so there are 65536 cases: all of them (every bit pattern
+    as the activated half, multiplied by 1 and by 3), through the vector kernel, the scalar kernel (odd width) and the
+    fused SwiGLU + quantisation.  The kernels take hardware exp2 / reciprocal and fall back to the exact formula next to
+    bf16 rounding boundaries; the results must be those of the exact formula as the oracle evaluates it (libm expf and
+    IEEE division) wherever that is a number."""
+    a = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    for mul in (1.0, 3.0):
+        x = torch.cat([a.view(256, 256), torch.full((256, 256), mul, dtype=torch.bfloat16)], dim=1).contiguous()
+        want = golden.swiglu(_bits(x))
+        nan = np.isnan(golden.bf16_bits_to_f32(want))
+        got = _bits(capi.swiglu(x.cuda()))
+        assert np.array_equal(got[~nan], want[~nan]), int((got[~nan] != want[~nan]).sum())
+        assert np.isnan(golden.bf16_bits_to_f32(got[nan])).all()
+        # odd width: the scalar kernel
+        xo = torch.cat([a.view(256, 256)[:, :255], torch.full((256, 255), mul, dtype=torch.bfloat16)], dim=1).contiguous()
+        wo = golden.swiglu(_bits(xo))
+        go = _bits(capi.swiglu(xo.cuda()))
+        ok = ~np.isnan(golden.bf16_bits_to_f32(wo))
+        assert np.array_equal(go[ok], wo[ok])
+    # fused with the quantisation: rows of finite arguments only (a NaN or an infinity would own its row's scale)
+    fin = a[torch.isfinite(a.float())]
+    fin = fin[: fin.numel() // 256 * 256].view(-1, 256)
+    xf = torch.cat([fin, torch.full(fin.shape, 1.0, dtype=torch.bfloat16)], dim=1).contiguous()
+    y, s = capi.swiglu_quant(xf.cuda(), activate_left=True)
+    wy, ws = golden.swiglu_quant(_bits(xf), activate_left=True)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), ws.view(np.uint32)) and np.array_equal(y.cpu().numpy(), wy)
+
+
 # ------------------------------------------------------------------ anti_quant
 
 @pytest.mark.parametrize("rows,cols,packed", [(10, 100, False), (10, 200, True), (4096, 14336, False), (512, 4096, True),
