@@ -107,6 +107,14 @@ def _graph_time_us(torch, calls, reps=20):
             c()
     g.replay()
     torch.cuda.synchronize()
+    # after an idle period the chip needs about 30 ms of continuous work to reach the clocks it then holds (the headline
+    # launch: 45 us for the first twenty launches, 47-54 us for the next few hundred, 43.5-44.5 us from about the 700th on):
+    # replay untimed for that long, so that every line is measured in the settled state
+    w0 = time.perf_counter()
+    while time.perf_counter() - w0 < 0.03:
+        for _ in range(4):
+            g.replay()
+        torch.cuda.synchronize()
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     start.record()
@@ -352,6 +360,17 @@ def main():
     ev3.record()
     torch.cuda.synchronize()
     long_run_us = ev2.elapsed_time(ev3) * 1e3 / 200
+    # ... and once the clocks have settled under continuous load (about 30 ms after an idle period: launches 1500-1700)
+    for _ in range(1300):
+        step()
+    ev4 = torch.cuda.Event(enable_timing=True)
+    ev5 = torch.cuda.Event(enable_timing=True)
+    ev4.record()
+    for _ in range(200):
+        step()
+    ev5.record()
+    torch.cuda.synchronize()
+    settled_us = ev4.elapsed_time(ev5) * 1e3 / 200
     # the clock the chip holds while all matrix cores are busy (measured after the headline: the probe saturates every
     # SIMD for about a millisecond)
     _capi.sustained_mfma_clock_mhz(iters=2000)       # warm-up
@@ -401,6 +420,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved_tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": round(achieved_tops / INT8_PEAK_TOPS, 4), "traffic": _traffic("c2"),
                      "kernel": "qmm_kernel", "launch_us": round(kern_ms * 1e3, 3), "launch_us_over_200_launches": round(long_run_us, 3),
+                     "launch_us_settled": round(settled_us, 3),
                      "bit_identical_to_oracle": parity.get("c2_bit_identical_to_oracle"),
                      "peak_at_sustained_clock": round(INT8_PEAK_TOPS * sustained_mhz / 2400.0, 1) if sustained_mhz else None,
                      "frac_at_sustained_clock": round(achieved_tops / (INT8_PEAK_TOPS * sustained_mhz / 2400.0), 4)
