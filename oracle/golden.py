@@ -243,6 +243,22 @@ def quantize(x_f32, scale_f32, zero_point_f32=None, out: str = "int8", axis: int
     return np.clip(v.astype(np.float64), lo, hi).astype(dt)
 
 
+def weight_quant_requant(out_u16, quant_scale_f32, quant_offset_f32=None, dtype: str = "bf16") -> np.ndarray:
+    """int8 output of npu_weight_quant_batchmatmul with quant_scale / quant_offset (the arguments
+    torch_npu/contrib/module/linear_weight_quant.py:79-87,106-109 constructs and passes): the product rounded to the
+    dtype of x (``out_u16``: its bit patterns), times quant_scale[n], plus the offset brought to the 9-bit integer range
+    of the packed parameter words (round, clip to [-256, 255]: f32_2_s9, test/contrib/test_linear_weight_quant.py:13-16),
+    rounded half to even and clamped to int8; every operation rounded to float32.  PARITY UNPINNED: the reference tree
+    holds no golden or test vector for this output (its test builds the module with quant_scale=False); this is the
+    re-quantisation of npu_quant_matmul's int8 output applied to the rounded product."""
+    u = np.ascontiguousarray(out_u16, dtype=np.uint16)
+    x = u.view(np.float16).astype(np.float32) if dtype == "fp16" else bf16_bits_to_f32(u)
+    off = None
+    if quant_offset_f32 is not None:
+        off = np.clip(np.rint(_c(quant_offset_f32, np.float32)), -256, 255).astype(np.float32)
+    return quantize(x, quant_scale_f32, off, out="int8", axis=-1, div_mode=False)
+
+
 def trans_quant_param(scale_f32, offset_f32=None) -> np.ndarray:
     """npu_trans_quant_param (caller torch_npu/contrib/module/linear_quant.py:104-108, result type and shapes
     test/test_fake_tensor.py:1929-1943): int64 words with the float32 bit pattern of the scale in bits 0-31,

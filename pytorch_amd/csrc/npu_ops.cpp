@@ -518,7 +518,7 @@ WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &an
     TORCH_CHECK(weight.scalar_type() == at::kChar || weight.scalar_type() == at::kInt, op,
                 ": weight must be int8, or int32 holding 8 int4 values per word, got ", weight.scalar_type());
     TORCH_CHECK(x.dim() >= 2 && weight.dim() == 2, op, ": x must be [..., K] with at least 2 dimensions and weight 2-D");
-    TORCH_CHECK(!opt(quant_scale) && !opt(quant_offset), op, ": quant_scale / quant_offset (int8 output) are not supported");
+    TORCH_CHECK(opt(quant_scale) || !opt(quant_offset), op, ": quant_offset needs quant_scale");
     TORCH_CHECK(inner_precise == 0, op, ": inner_precise must be 0");
     TORCH_CHECK(!weight_dtype.has_value(), op, ": weight_dtype is not supported");
     WqPlan p;
@@ -551,6 +551,21 @@ WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &an
                     b->scalar_type());
         TORCH_CHECK(b->numel() == p.N && b->size(-1) == p.N, op, ": bias must have shape [", p.N, "]");
     }
+    // quant_scale (float32, or the int64 words of npu_trans_quant_param, which hold the offset as well) and quant_offset
+    // (float32): one value or one per output column; they turn the output into int8
+    auto check_requant = [&](const Tensor &t, const char *name, bool may_be_packed) {
+        TORCH_CHECK(t.scalar_type() == at::kFloat || (may_be_packed && t.scalar_type() == at::kLong), op, ": ", name, " must be float32",
+                    may_be_packed ? " or int64 (npu_trans_quant_param)" : "", ", got ", t.scalar_type());
+        TORCH_CHECK((t.dim() == 1 || (t.dim() == 2 && t.size(0) == 1)) && (t.size(-1) == p.N || t.size(-1) == 1), op, ": ", name,
+                    " must have shape [", p.N, "], [1, ", p.N, "] or one element, got ", t.sizes());
+    };
+    if (const Tensor *q = opt(quant_scale)) {
+        check_requant(*q, "quant_scale", true);
+        if (const Tensor *o = opt(quant_offset)) {
+            TORCH_CHECK(q->scalar_type() == at::kFloat, op, ": an int64 quant_scale already holds the offset; pass quant_offset=None");
+            check_requant(*o, "quant_offset", false);
+        }
+    }
     p.out_shape = x.sizes().vec();
     p.out_shape.back() = p.N;
     return p;
@@ -563,7 +578,7 @@ Tensor weight_quant_meta(const Tensor &x, const Tensor &weight, const Tensor &an
 {
     WqPlan p = weight_quant_plan(x, weight, antiquant_scale, antiquant_offset, quant_scale, quant_offset, bias, group_size,
                                  inner_precise, weight_dtype);
-    return at::empty(p.out_shape, x.options());
+    return at::empty(p.out_shape, opt(quant_scale) ? x.options().dtype(at::kChar) : x.options());
 }
 
 Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &antiquant_scale,
@@ -573,7 +588,8 @@ Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &ant
 {
     WqPlan p = weight_quant_plan(x, weight, antiquant_scale, antiquant_offset, quant_scale, quant_offset, bias, group_size,
                                  inner_precise, weight_dtype);
-    check_same_device("npu_weight_quant_batchmatmul", {&x, &weight, &antiquant_scale, opt(antiquant_offset), opt(bias)});
+    check_same_device("npu_weight_quant_batchmatmul",
+                      {&x, &weight, &antiquant_scale, opt(antiquant_offset), opt(quant_scale), opt(quant_offset), opt(bias)});
     c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
     Tensor out = at::empty(p.out_shape, x.options());
     if (out.numel() == 0) return out;
@@ -616,7 +632,30 @@ Tensor weight_quant_hip(const Tensor &x, const Tensor &weight, const Tensor &ant
                                            ws.defined() ? ws.data_ptr() : nullptr, ws.defined() ? (size_t)ws.numel() : 0,
                                            stream_of(x)),
                  "npu_weight_quant_batchmatmul");
-    return out;
+    const Tensor *qs = opt(quant_scale);
+    if (!qs) return out;
+    // int8 output: y = clamp(rint(float(out) * quant_scale[n] + quant_offset[n]), -128, 127), the product rounded to the
+    // dtype of x first (it is the operator's result without quant_scale), every later operation rounded to float32, and
+    // the offset brought to the 9-bit integer range that the packed parameter words hold (round, clip to [-256, 255]: the
+    // reference's own test helper f32_2_s9, test/contrib/test_linear_weight_quant.py:13-16).  The reference tree holds no
+    // golden for this output; the formula is the re-quantisation of npu_quant_matmul's int8 output applied to the
+    // rounded product.
+    Tensor scale_f, offset_f;
+    if (qs->scalar_type() == at::kLong) {
+        const Tensor q = qs->reshape({-1});
+        scale_f = q.bitwise_and((int64_t)0xffffffffLL).bitwise_xor((int64_t)0x80000000LL).sub((int64_t)0x80000000LL).to(at::kInt).view(at::kFloat);
+        offset_f = q.bitwise_right_shift(37).bitwise_and(0x1ff).bitwise_xor(256).sub(256).to(at::kFloat);
+    } else {
+        scale_f = qs->reshape({-1}).contiguous();
+        if (const Tensor *qo = opt(quant_offset)) offset_f = at::clamp(at::round(qo->reshape({-1})), -256.0, 255.0).contiguous();
+    }
+    Tensor out8 = at::empty(p.out_shape, x.options().dtype(at::kChar));
+    check_status(mi355_quantize(out2d.data_ptr(), x.scalar_type() == at::kHalf ? MI355_DTYPE_FP16 : MI355_DTYPE_BF16,
+                                scale_f.data_ptr<float>(), scale_f.numel(), offset_f.defined() ? offset_f.data_ptr() : nullptr,
+                                MI355_DTYPE_FP32, offset_f.defined() ? offset_f.numel() : 0, out8.data_ptr(), MI355_Q_INT8, p.M, p.N, 1,
+                                0, stream_of(x)),
+                 "npu_weight_quant_batchmatmul (quant_scale)");
+    return out8;
 }
 
 // ---------------------------------------------------------------- npu_swiglu

@@ -138,17 +138,21 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     MI355_TS(0)
-    const int wm = wave / WGN, wn = wave % WGN;
+    // Wavefronts w and w + 4 of a workgroup share a SIMD.  In the wide loop the two wavefronts of a SIMD take different
+    // roles (one refills activations, one weights): wn = 0, 1, 0, 1, 1, 0, 1, 0 for wavefronts 0 .. 7.
+    const int wm = LOOP == 1 || LOOP == 2 ? ((wave & 3) >> 1) + 2 * (wave >> 2) : wave / WGN;
+    const int wn = LOOP == 1 || LOOP == 2 ? ((wave >> 2) ^ wave) & 1 : wave % WGN;
     const int kt0 = (int)((int64_t)(p.K / BK) * chunk / p.S);            // first K step of this workgroup
     const int KT = (int)((int64_t)(p.K / BK) * (chunk + 1) / p.S) - kt0;  // its number of K steps
 
     // Global -> LDS addressing.  Lane l of a unit fills LDS slot l (16 B): row l/8, chunk slot l%8,
     // which must hold global chunk (l%8) ^ (l/8) of that row (XOR swizzle).
     const int rows_a = min(BM, p.M - m0), rows_b = min(BN, p.N - n0);
+    // (timing ablations 32 / 64: every tile reads the activation rows / weight columns of the first tile)
     const __amdgpu_buffer_rsrc_t rsrc_a =
-        make_rsrc(p.a + (int64_t)m0 * p.lda, (uint32_t)((int64_t)(rows_a - 1) * p.lda + p.K));
+        make_rsrc(p.a + (int64_t)((MI355_WIDE_ABL & 32) ? 0 : m0) * p.lda, (uint32_t)((int64_t)(rows_a - 1) * p.lda + p.K));
     const __amdgpu_buffer_rsrc_t rsrc_b =
-        make_rsrc(p.bt + (int64_t)n0 * p.ldbt, (uint32_t)((int64_t)(rows_b - 1) * p.ldbt + p.K));
+        make_rsrc(p.bt + (int64_t)((MI355_WIDE_ABL & 64) ? 0 : n0) * p.ldbt, (uint32_t)((int64_t)(rows_b - 1) * p.ldbt + p.K));
     const int rr = lane >> 3;
     // row of the tile = 8 * unit + rr and unit = i * NW + wave with NW even: (row >> 1) & 7 = 4 * (wave & 1) + rr / 2
     const int gchunk = ((lane & 7) ^ (((wave & 1) << 2) | (rr >> 1))) * 16;
@@ -510,6 +514,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             e.has_bias = p.bias_kind == MI355_BIAS_INT32;
             e.out_f16 = 0;
             e.stream_out = p.stream_out;
+            e.wm = wm;
+            e.wn = wn;
             wide::epilogue_fast_i8<WTN>(acc, lds, e, wave, lane);
             return;
         }
@@ -524,6 +530,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             e.has_bias = p.bias_kind == MI355_BIAS_BF16;
             e.out_f16 = p.out_f16;
             e.stream_out = p.stream_out;
+            e.wm = wm;
+            e.wn = wn;
             wide::epilogue_fast<WTN>(acc, lds, e, wave, lane);
             MI355_TS(4)
             return;

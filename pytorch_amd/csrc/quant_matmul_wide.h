@@ -19,7 +19,7 @@
 #include <utility>
 
 #ifndef MI355_WIDE_ABL
-#define MI355_WIDE_ABL 0       // compile-time ablations for timing experiments (wrong results): 1 no refill traffic, 2 no fragment reads, 4 no MFMAs, 8 no handshake, 16 no barrier
+#define MI355_WIDE_ABL 0       // compile-time ablations for timing experiments (wrong results): 1 no refill traffic, 2 no fragment reads, 4 no MFMAs, 8 no handshake, 16 no barrier, 32 / 64 all tiles read the first tile's activation rows / weight columns
 #endif
 
 namespace mi355 {
@@ -60,30 +60,6 @@ template <int LG>
 __device__ __forceinline__ void wait_lgkmcnt()
 {
     asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(LG) : "memory");
-}
-
-// MFMAs FROM .. TO-1 of a half step (activation fragment outer, weight fragment inner).  The weight fragment is the
-// first operand: a lane ends up with four consecutive output columns of one row.
-template <int WTN, int FROM, int TO>
-__device__ __forceinline__ void mfma_range(i32x4v (&acc)[4][WTN], const i32x4v (&af)[4], const i32x4v (&bf)[WTN])
-{
-#pragma unroll
-    for (int t = FROM; t < TO; t++) {
-        const int i = t / WTN, j = t % WTN;
-        if constexpr (MI355_WIDE_ABL & 4) asm volatile("" ::"v"(bf[j]), "v"(af[i]));
-        else acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
-    }
-}
-
-// N groups of (one instruction of class MASK, then PER MFMAs) for the scheduler
-template <int MASK, int N, int PER>
-__device__ __forceinline__ void interleave()
-{
-#pragma unroll
-    for (int q = 0; q < N; q++) {
-        __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
-    }
 }
 
 struct LoopState {
@@ -373,6 +349,7 @@ struct EpilogueArgs {
     int m0, n0;                        // first row / column of the workgroup tile
     int has_bias, out_f16;
     int stream_out;                    // store the rows with non-temporal stores (see the launcher's choice)
+    int wm, wn;                        // position of the wavefront's 64 x 16 * WTN share in the workgroup tile
 };
 
 constexpr int PARAM_PS = 0, PARAM_SCALE = 1024, PARAM_BIAS = 2048;
@@ -399,7 +376,7 @@ __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, 
     using G = Geometry<WTN>;
     constexpr int ROWB = WTN * 32 + 16;                       // padded pitch of a staged row: spreads rows over the banks
     constexpr int CHUNKS = WTN * 2;                           // 16-byte chunks per row of the wavefront tile
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = e.wm, wn = e.wn;
     const int mrow = lane & 15, nquad = (lane >> 4) * 4;
     const char *par = lds + G::PARAM_BASE;
     float ps[4];
@@ -499,7 +476,7 @@ __device__ __forceinline__ void epilogue_rows_i8(i32x4v (&acc)[4][WTN], char *ld
     using G = Geometry<WTN>;
     constexpr int ROWQ = WTN * 16 + 16;                       // padded pitch of a staged row of the wavefront tile
     constexpr int CHQ = WTN;                                  // 16-byte chunks per row
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = e.wm, wn = e.wn;
     const int mrow = lane & 15, nquad = (lane >> 4) * 4;
     const char *par = lds + G::PARAM_BASE;
     char *stq = lds + wave * (64 * ROWQ);

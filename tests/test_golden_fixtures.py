@@ -206,6 +206,22 @@ def test_trans_quant_param_offset_field_follows_f32_2_s9(golden):
     assert diff != 0 and (diff >> (diff.bit_length() - 9)) == 0x1FF and diff.bit_length() - 9 == (diff & -diff).bit_length() - 1
 
 
+def test_weight_quant_requant_hand_computed(golden):
+    """The int8 output of npu_weight_quant_batchmatmul with quant_scale / quant_offset as the oracle states it, on values
+    typed by hand: the offset goes through f32_2_s9 (0.4 -> 0, 300 -> 255, -300 -> -256, 2.5 -> 2), products and sums are
+    rounded to float32, ties go to even, the result saturates at the int8 range."""
+    import torch
+    out = torch.tensor([[1.5, 2.5, -3.0, 100.0, -0.5, 7.0]], dtype=torch.bfloat16)
+    bits = out.view(torch.int16).numpy().view(np.uint16)
+    scale = np.float32([1.0, 1.0, 2.0, 1.0, 1.0, 0.5])
+    off = np.float32([0.4, 300.0, -300.0, 2.5, 0.0, 0.0])
+    #            1.5+0 -> 2   2.5+255 -> 127   -6-256 -> -128   100+2 -> 102   -0.5 -> -0   3.5 -> 4
+    assert golden.weight_quant_requant(bits, scale, off).tolist() == [[2, 127, -128, 102, 0, 4]]
+    assert golden.weight_quant_requant(bits, scale, None).tolist() == [[2, 2, -6, 100, 0, 4]]
+    h = out.to(torch.float16).view(torch.int16).numpy().view(np.uint16)
+    assert golden.weight_quant_requant(h, scale, off, dtype="fp16").tolist() == [[2, 127, -128, 102, 0, 4]]
+
+
 @pytest.mark.gpu
 def test_gpu_trans_quant_param_offset_field_follows_f32_2_s9(capi, golden):
     off = torch.tensor(_S9_IN, dtype=torch.float32)

@@ -742,3 +742,56 @@ def test_device_failure_report_reaches_the_operator_layer(pa):
         pa.check_device_status()
     pa.check_device_status()
     assert torch.equal(pa.npu_weight_quant_batchmatmul(*args), good)
+
+
+@pytest.mark.gpu
+def test_weight_quant_batchmatmul_int8_output(pa, golden):
+    """quant_scale / quant_offset of npu_weight_quant_batchmatmul (what LinearWeightQuant constructs and passes,
+    torch_npu/contrib/module/linear_weight_quant.py:79-87,106-109): int8 = clamp(rint(out * quant_scale + s9(quant_offset))).
+    Against the oracle applied to the operator's own 16-bit result (which other tests compare with the oracle), for
+    float32 parameters, for the packed int64 words of npu_trans_quant_param, through the module, and for float16.
+    The formula itself has no pin in the reference tree (parity unpinned); the offset's 9-bit range is the reference's
+    f32_2_s9 helper (test/contrib/test_linear_weight_quant.py:13-16)."""
+    from pytorch_amd.contrib.module import LinearWeightQuant
+    g = torch.Generator().manual_seed(11)
+    for (dt, name, M, K, N, bits) in [(torch.bfloat16, "bf16", 32, 1024, 256, 8), (torch.float16, "fp16", 5, 512, 384, 8),
+                                      (torch.bfloat16, "bf16", 8, 1024, 512, 4)]:
+        if bits == 8:
+            d = workloads.w8a16_inputs(seed=M, M=M, K=K, N=N, weight_nk=True)
+            gs = 0
+        else:
+            d = workloads.w4a16_inputs(seed=M, M=M, K=K, N=N, group_size=128)
+            gs = 128
+        x, sc, of = d["x"].to(dt).cuda(), d["antiquant_scale"].to(dt).cuda(), d["antiquant_offset"].to(dt).cuda()
+        w = d["weight"].cuda()
+        plain = pa.npu_weight_quant_batchmatmul(x, w, sc, of, None, None, None, gs)
+        # scales that spread the results over the int8 range and beyond it, offsets beyond the 9-bit range
+        qs = (torch.rand(N, generator=g) * 0.5 + 0.05) * (100.0 / max(float(plain.float().abs().max()), 1e-6))
+        qo = torch.randn(N, generator=g) * 40.0
+        qo[:4] = torch.tensor([300.0, -300.0, 0.5, 1.5])
+        want = golden.weight_quant_requant(golden.bits_of(plain), qs.numpy(), qo.numpy(), dtype=name)
+        got = pa.npu_weight_quant_batchmatmul(x, w, sc, of, qs.cuda(), qo.cuda(), None, gs)
+        assert got.dtype == torch.int8 and got.shape == plain.shape
+        assert np.array_equal(got.cpu().numpy(), want)
+        assert len(np.unique(want)) > 100 and want.min() == -128 and want.max() == 127
+        # no offset, and [1, N] parameters
+        want0 = golden.weight_quant_requant(golden.bits_of(plain), qs.numpy(), None, dtype=name)
+        got0 = pa.npu_weight_quant_batchmatmul(x, w, sc, of, qs.cuda().view(1, N), None, None, gs)
+        assert np.array_equal(got0.cpu().numpy(), want0)
+        # the packed words hold the same scale and the same 9-bit offset
+        packed = pa.npu_trans_quant_param(qs.cuda(), qo.cuda())
+        assert packed.dtype == torch.int64
+        gotp = pa.npu_weight_quant_batchmatmul(x, w, sc, of, packed, None, None, gs)
+        assert torch.equal(gotp, got)
+        if bits == 8:
+            m = LinearWeightQuant(K, N, bias=False, antiquant_offset=True, quant_scale=True, quant_offset=True, dtype=dt).cuda()
+            m.weight.data = d["weight"].t().contiguous().cuda()
+            m.antiquant_scale.data, m.antiquant_offset.data = sc, of
+            m.quant_scale.data, m.quant_offset.data = qs.cuda(), qo.cuda()
+            assert torch.equal(m(x), got)
+    with pytest.raises(RuntimeError, match="quant_offset needs quant_scale"):
+        pa.npu_weight_quant_batchmatmul(x, w, sc, of, None, qo.cuda(), None, gs)
+    with pytest.raises(RuntimeError, match="already holds the offset"):
+        pa.npu_weight_quant_batchmatmul(x, w, sc, of, packed, qo.cuda(), None, gs)
+    with pytest.raises(RuntimeError, match="quant_scale must be float32"):
+        pa.npu_weight_quant_batchmatmul(x, w, sc, of, qs.to(torch.bfloat16).cuda(), None, None, gs)

@@ -167,7 +167,17 @@ def test_meta_weight_quant_batchmatmul(pa):
         pa.npu_weight_quant_batchmatmul(_m(3, 4096, dtype=torch.bfloat16), _m(500, 14336, dtype=torch.int32), sg, og, None, None,
                                         None, 128)
     xs = _m(1, 4096, dtype=torch.bfloat16)
-    for kwargs, pat in [(dict(quant_scale=_m(14336, dtype=torch.float32)), "quant_scale"),
+    # quant_scale turns the output into int8 (float32 values, or the int64 words of npu_trans_quant_param)
+    for qs in (_m(14336, dtype=torch.float32), _m(1, 14336, dtype=torch.int64), _m(1, dtype=torch.float32)):
+        r = pa.npu_weight_quant_batchmatmul(xs, w4, sg, og, qs, None, None, 128)
+        assert r.dtype == torch.int8 and r.shape == (1, 14336)
+    r = pa.npu_weight_quant_batchmatmul(xs, w4, sg, og, _m(14336, dtype=torch.float32), _m(14336, dtype=torch.float32), None, 128)
+    assert r.dtype == torch.int8
+    for kwargs, pat in [(dict(quant_offset=_m(14336, dtype=torch.float32)), "quant_offset needs quant_scale"),
+                        (dict(quant_scale=_m(14336, dtype=torch.bfloat16)), "quant_scale must be float32"),
+                        (dict(quant_scale=_m(100, dtype=torch.float32)), "quant_scale must have shape"),
+                        (dict(quant_scale=_m(14336, dtype=torch.int64), quant_offset=_m(14336, dtype=torch.float32)),
+                         "already holds the offset"),
                         (dict(bias=_m(14336, dtype=torch.float16)), "bias must have the dtype of x"),
                         (dict(inner_precise=1), "inner_precise"),
                         (dict(weight_dtype=torch.int8), "weight_dtype")]:
