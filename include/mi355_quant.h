@@ -78,6 +78,20 @@ int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth,
                         int64_t rows, int64_t cols, int64_t x_row_stride, void *stream);
 
 /*
+ * npu_dynamic_quant with per-expert smooth scales (the `group_index` argument of torch_npu.npu_dynamic_quant,
+ * signature test/test_fake_tensor.py:1670-1687, test/torch_npu_schema.json:2144-2146; the reference tree holds no call
+ * that passes it, the meaning is the operator's published one).
+ *   smooth       [groups, cols] in_dtype, contiguous
+ *   group_index  [groups] int32 on the device, non-decreasing running totals of the rows of each expert: row r is
+ *                multiplied by smooth[e] for the first e with r < group_index[e]; rows past the last total take the
+ *                last expert.  NULL: as mi355_dynamic_quant (smooth is then [cols] or NULL)
+ * Everything else as mi355_dynamic_quant.
+ */
+int mi355_dynamic_quant_grouped(const void *x, int in_dtype, const void *smooth, const int32_t *group_index,
+                                int64_t groups, int8_t *y, float *scale,
+                                int64_t rows, int64_t cols, int64_t x_row_stride, void *stream);
+
+/*
  * npu_dynamic_quant_asymmetric, per-token asymmetric int8.
  * Replaces the aclnn DynamicQuantV2 call behind torch_npu.npu_dynamic_quant_asymmetric (signature and output
  * shapes: test/test_fake_tensor.py:1689-1709, test/torch_npu_schema.json:2147-2149).  The arithmetic is not in the

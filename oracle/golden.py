@@ -91,6 +91,29 @@ def dynamic_quant(x_u16: np.ndarray, in_dtype: str = "bf16", smooth_u16: np.ndar
     return y, scale
 
 
+def dynamic_quant_grouped(x_u16: np.ndarray, smooth_u16: np.ndarray, group_index, in_dtype: str = "bf16"):
+    """npu_dynamic_quant with per-expert smooth scales (``group_index`` of the operator's signature,
+    test/test_fake_tensor.py:1670-1687; no call in the reference tree passes it): ``smooth_u16`` [E, cols],
+    ``group_index`` [E] the running totals of the rows of each expert; rows group_index[e-1] .. group_index[e]-1 are
+    quantised as dynamic_quant does with smooth_u16[e], rows past the last total with the last expert's scales.
+    PARITY UNPINNED for the meaning of group_index (the operator's published description); the arithmetic is
+    dynamic_quant's."""
+    x = _c(x_u16, np.uint16)
+    x2 = x.reshape(-1, x.shape[-1])
+    sm = _c(smooth_u16, np.uint16)
+    gi = [int(v) for v in np.asarray(group_index).reshape(-1)]
+    assert sm.ndim == 2 and sm.shape[0] == len(gi) and sm.shape[1] == x.shape[-1]
+    y = np.empty(x2.shape, dtype=np.int8)
+    scale = np.empty(x2.shape[0], dtype=np.float32)
+    lo = 0
+    for e, hi in enumerate(gi):
+        hi = x2.shape[0] if e == len(gi) - 1 else min(max(hi, lo), x2.shape[0])
+        if hi > lo:
+            y[lo:hi], scale[lo:hi] = dynamic_quant(x2[lo:hi], in_dtype, sm[e])
+        lo = max(lo, hi)
+    return y.reshape(x.shape), scale.reshape(x.shape[:-1])
+
+
 def dynamic_quant_asymmetric(x_u16: np.ndarray, in_dtype: str = "bf16", smooth_u16: np.ndarray | None = None):
     """x: uint16 bit patterns [..., cols] -> (y int8 same shape, scale float32 [...], offset float32 [...])."""
     x = _c(x_u16, np.uint16)

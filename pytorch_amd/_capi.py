@@ -14,7 +14,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
 
-EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant",
+EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant", "mi355_dynamic_quant_grouped",
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
@@ -40,6 +40,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_status_string.argtypes = [i32]
         L.mi355_quant_abi_version.restype = i32
         L.mi355_dynamic_quant.argtypes = [vp, i32, vp, vp, vp, i64, i64, i64, vp]
+        L.mi355_dynamic_quant_grouped.argtypes = [vp, i32, vp, vp, i64, vp, vp, i64, i64, i64, vp]
         L.mi355_quant_matmul_workspace.restype = sz
         L.mi355_quant_matmul_workspace.argtypes = [i64, i64, i64, i64, i64]
         L.mi355_quant_matmul.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
@@ -113,9 +114,11 @@ def _need_gpu(*ts):
             raise Mi355Error("the C ABI takes device pointers: tensors must live on the GPU")
 
 
-def dynamic_quant(x: torch.Tensor, smooth: torch.Tensor | None = None):
+def dynamic_quant(x: torch.Tensor, smooth: torch.Tensor | None = None, group_index: torch.Tensor | None = None):
+    """smooth [cols], or with group_index (int32 [E], running row totals per expert) [E, cols]."""
     _need_gpu(x, smooth)
     assert x.dtype in (torch.bfloat16, torch.float16)
+    assert group_index is None or (group_index.dtype == torch.int32 and group_index.is_cuda and smooth.is_contiguous())
     if x.numel() and x.stride(-1) != 1:
         x = x.contiguous()
     cols = x.shape[-1]
@@ -125,6 +128,12 @@ def dynamic_quant(x: torch.Tensor, smooth: torch.Tensor | None = None):
     rows = x2.shape[0]
     y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
     scale = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    if group_index is not None:
+        st = lib().mi355_dynamic_quant_grouped(_ptr(x2), 0 if x.dtype == torch.bfloat16 else 1, _ptr(smooth), _ptr(group_index),
+                                               group_index.numel(), _ptr(y), _ptr(scale), rows, cols,
+                                               x2.stride(0) if rows > 1 else max(cols, 1), _stream())
+        _check(st, "mi355_dynamic_quant_grouped")
+        return y, scale
     st = lib().mi355_dynamic_quant(_ptr(x2), 0 if x.dtype == torch.bfloat16 else 1, _ptr(smooth), _ptr(y), _ptr(scale),
                                    rows, cols, x2.stride(0) if rows > 1 else max(cols, 1), _stream())
     _check(st, "mi355_dynamic_quant")

@@ -193,16 +193,30 @@ __global__ __launch_bounds__(BLOCK) void dq_rows_kernel(const uint16_t *__restri
     }
 }
 
+// Per-expert smooth scales (npu_dynamic_quant with group_index): `group_index` holds the running totals of the rows of
+// each expert, so row r belongs to the first expert e with r < group_index[e] (rows past the last total take the last
+// expert); returns the first element of that expert's scales.
+__device__ __forceinline__ const uint16_t *expert_scales(const uint16_t *smooth, const int32_t *group_index, int groups, int64_t row,
+                                                         int64_t cols)
+{
+    if (!group_index) return smooth;
+    int e = 0;
+    while (e < groups - 1 && row >= (int64_t)group_index[e]) e++;
+    return smooth + (int64_t)e * cols;
+}
+
 // Any shape, stride and alignment; optional smooth scales.  One block per row, two passes
 // over the row (the second one hits in cache), IEEE division per element.
 template <bool FP16>
 __global__ __launch_bounds__(kBlock) void dq_generic_kernel(const uint16_t *__restrict__ x,
                                                             const uint16_t *__restrict__ smooth,
                                                             int8_t *__restrict__ y, float *__restrict__ scale_out,
-                                                            int64_t cols, int64_t row_stride)
+                                                            int64_t cols, int64_t row_stride,
+                                                            const int32_t *__restrict__ group_index = nullptr, int groups = 0)
 {
     const int64_t row = blockIdx.x;
     const uint16_t *xr = x + row * row_stride;
+    if (smooth) smooth = expert_scales(smooth, group_index, groups, row, cols);
     float amax = 0.0f;
     for (int64_t j = threadIdx.x; j < cols; j += kBlock) {
         float v = cvt1<FP16>(xr[j]);
@@ -243,12 +257,13 @@ __global__ __launch_bounds__(BLOCK) void dq_smooth_rows_kernel(const uint16_t *_
                                                                 const uint16_t *__restrict__ smooth,
                                                                 int8_t *__restrict__ y, float *__restrict__ scale_out,
                                                                 int cols, int64_t row_stride, int act_offset = 0,
-                                                                int mul_offset = 0)
+                                                                int mul_offset = 0,
+                                                                const int32_t *__restrict__ group_index = nullptr, int groups = 0)
 {
     const int64_t row = blockIdx.x;
     const int t = threadIdx.x, nvec = cols >> 3;
     const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + row * row_stride);
-    const u32x4 *sr = reinterpret_cast<const u32x4 *>(smooth);
+    const u32x4 *sr = reinterpret_cast<const u32x4 *>(expert_scales(smooth, group_index, groups, row, cols));
     float f[MAXV][8];
     float amax = 0.0f;
 #pragma unroll
@@ -455,8 +470,18 @@ extern "C" int mi355_swiglu_quant_smooth(const void *x_bf16, int activate_left, 
 extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth, int8_t *y, float *scale,
                                    int64_t rows, int64_t cols, int64_t x_row_stride, void *stream)
 {
+    return mi355_dynamic_quant_grouped(x, in_dtype, smooth, nullptr, 0, y, scale, rows, cols, x_row_stride, stream);
+}
+
+extern "C" int mi355_dynamic_quant_grouped(const void *x, int in_dtype, const void *smooth, const int32_t *group_index,
+                                           int64_t groups, int8_t *y, float *scale, int64_t rows, int64_t cols,
+                                           int64_t x_row_stride, void *stream)
+{
     using namespace mi355;
     if (rows < 0 || cols < 0) return MI355_ERR_BAD_ARGUMENT;
+    if (group_index && (!smooth || groups < 1 || groups > 0x7fffffff)) return MI355_ERR_BAD_ARGUMENT;
+    if (group_index && !aligned(group_index, 4)) return MI355_ERR_ALIGNMENT;
+    const int ng = group_index ? (int)groups : 0;
     if (in_dtype != MI355_DTYPE_BF16 && in_dtype != MI355_DTYPE_FP16) return MI355_ERR_BAD_ARGUMENT;
     if (rows == 0) return MI355_OK;
     if (!scale) return MI355_ERR_BAD_ARGUMENT;
@@ -486,7 +511,7 @@ extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smoo
         const uint16_t *sm = static_cast<const uint16_t *>(smooth);
 #define MI355_DQS_LAUNCH(F, V, B) \
     hipLaunchKernelGGL((dq_smooth_rows_kernel<F, false, V, B>), dim3((unsigned)rows), dim3(B), 0, s, xp, sm, y, scale, (int)cols, \
-                       x_row_stride)
+                       x_row_stride, 0, 0, group_index, ng)
         if (nvec <= kBlock * 4) {
             if (fp16) MI355_DQS_LAUNCH(true, 4, kBlock);
             else MI355_DQS_LAUNCH(false, 4, kBlock);
@@ -505,10 +530,10 @@ extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smoo
         const uint16_t *sm = static_cast<const uint16_t *>(smooth);
         if (fp16)
             hipLaunchKernelGGL((dq_generic_kernel<true>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale,
-                               cols, x_row_stride);
+                               cols, x_row_stride, group_index, ng);
         else
             hipLaunchKernelGGL((dq_generic_kernel<false>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y, scale,
-                               cols, x_row_stride);
+                               cols, x_row_stride, group_index, ng);
     }
     return check_launch();
 }

@@ -59,16 +59,28 @@ void *stream_of(const Tensor &t)
 
 // ---------------------------------------------------------------- npu_dynamic_quant
 
+// `grouped_ok`: the operator takes per-expert smooth scales (smooth_scales [E, H] with group_index [E], the running
+// totals of the rows of each expert)
 void dynamic_quant_check(const Tensor &input, const optional<Tensor> &smooth_scales, const optional<Tensor> &group_index,
-                         optional<at::ScalarType> dst_type)
+                         optional<at::ScalarType> dst_type, bool grouped_ok = false)
 {
     TORCH_CHECK(input.scalar_type() == at::kBFloat16 || input.scalar_type() == at::kHalf,
                 "npu_dynamic_quant: input must be bfloat16 or float16, got ", input.scalar_type());
     TORCH_CHECK(input.dim() >= 1, "npu_dynamic_quant: input must have at least one dimension");
-    TORCH_CHECK(!opt(group_index), "npu_dynamic_quant: group_index (per-expert smooth scales) is not supported");
+    TORCH_CHECK(grouped_ok || !opt(group_index), "npu_dynamic_quant: group_index (per-expert smooth scales) is not supported");
     TORCH_CHECK(!dst_type.has_value() || *dst_type == at::kChar,
                 "npu_dynamic_quant: only dst_type=torch.int8 is supported, got ", *dst_type);
-    if (const Tensor *s = opt(smooth_scales)) {
+    if (const Tensor *g = opt(group_index)) {
+        const Tensor *s = opt(smooth_scales);
+        TORCH_CHECK(s, "npu_dynamic_quant: group_index needs smooth_scales of shape [experts, ", input.size(-1), "]");
+        TORCH_CHECK(g->scalar_type() == at::kInt || g->scalar_type() == at::kLong,
+                    "npu_dynamic_quant: group_index must be int32 or int64, got ", g->scalar_type());
+        TORCH_CHECK(g->dim() == 1 && g->size(0) >= 1, "npu_dynamic_quant: group_index must have shape [experts]");
+        TORCH_CHECK(s->scalar_type() == input.scalar_type(), "npu_dynamic_quant: smooth_scales must have the dtype of input");
+        TORCH_CHECK(s->dim() == 2 && s->size(0) == g->size(0) && s->size(1) == input.size(-1),
+                    "npu_dynamic_quant: with group_index, smooth_scales must have shape [", g->size(0), ", ", input.size(-1), "], got ",
+                    s->sizes());
+    } else if (const Tensor *s = opt(smooth_scales)) {
         TORCH_CHECK(s->scalar_type() == input.scalar_type(), "npu_dynamic_quant: smooth_scales must have the dtype of input");
         TORCH_CHECK(s->dim() == 1 && s->size(0) == input.size(-1),
                     "npu_dynamic_quant: smooth_scales must have shape [", input.size(-1), "]");
@@ -86,15 +98,15 @@ std::tuple<Tensor, Tensor> dynamic_quant_alloc(const Tensor &input)
 std::tuple<Tensor, Tensor> dynamic_quant_meta(const Tensor &input, const optional<Tensor> &smooth_scales,
                                               const optional<Tensor> &group_index, optional<at::ScalarType> dst_type)
 {
-    dynamic_quant_check(input, smooth_scales, group_index, dst_type);
+    dynamic_quant_check(input, smooth_scales, group_index, dst_type, true);
     return dynamic_quant_alloc(input);
 }
 
 std::tuple<Tensor, Tensor> dynamic_quant_hip(const Tensor &input, const optional<Tensor> &smooth_scales,
                                              const optional<Tensor> &group_index, optional<at::ScalarType> dst_type)
 {
-    dynamic_quant_check(input, smooth_scales, group_index, dst_type);
-    check_same_device("npu_dynamic_quant", {&input, opt(smooth_scales)});
+    dynamic_quant_check(input, smooth_scales, group_index, dst_type, true);
+    check_same_device("npu_dynamic_quant", {&input, opt(smooth_scales), opt(group_index)});
     c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     auto [y, scale] = dynamic_quant_alloc(input);
     const int64_t cols = input.size(-1);
@@ -113,9 +125,13 @@ std::tuple<Tensor, Tensor> dynamic_quant_hip(const Tensor &input, const optional
     }
     Tensor smooth;
     if (const Tensor *s = opt(smooth_scales)) smooth = s->contiguous();
-    check_status(mi355_dynamic_quant(x.data_ptr(), x.scalar_type() == at::kBFloat16 ? MI355_DTYPE_BF16 : MI355_DTYPE_FP16,
-                                     smooth.defined() ? smooth.data_ptr() : nullptr, y.data_ptr<int8_t>(),
-                                     scale.data_ptr<float>(), rows, cols, row_stride, stream_of(input)),
+    Tensor gi;                                             // a handful of totals: int64 ones are narrowed on the device
+    if (const Tensor *g = opt(group_index)) gi = g->to(at::kInt).contiguous();
+    check_status(mi355_dynamic_quant_grouped(x.data_ptr(), x.scalar_type() == at::kBFloat16 ? MI355_DTYPE_BF16 : MI355_DTYPE_FP16,
+                                             smooth.defined() ? smooth.data_ptr() : nullptr,
+                                             gi.defined() ? gi.data_ptr<int32_t>() : nullptr, gi.defined() ? gi.numel() : 0,
+                                             y.data_ptr<int8_t>(), scale.data_ptr<float>(), rows, cols, row_stride,
+                                             stream_of(input)),
                  "npu_dynamic_quant");
     return {y, scale};
 }

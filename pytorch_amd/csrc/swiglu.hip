@@ -74,4 +74,4 @@ extern "C" const char *mi355_status_string(int status)
     }
 }
 
-extern "C" int mi355_quant_abi_version(void) { return 3000; }
+extern "C" int mi355_quant_abi_version(void) { return 3001; }

@@ -126,6 +126,28 @@ def test_dynamic_quant_smooth_shapes(capi, golden, rows, cols, dt):
     assert np.array_equal(y.cpu().numpy(), yg)
 
 
+@pytest.mark.parametrize("rows,cols,totals", [(64, 4096, [10, 10, 37, 64]), (33, 1000, [0, 33]), (20, 8200, [5, 9, 12]),
+                                              (128, 14336, [1, 2, 3, 4, 100, 128]), (7, 512, [7])])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_dynamic_quant_per_expert_smooth_scales(capi, golden, rows, cols, totals, dt):
+    """group_index of npu_dynamic_quant (signature test/test_fake_tensor.py:1670-1687): smooth_scales [E, cols], the
+    running row totals per expert select a row's scales.  Empty experts, totals short of the row count (the rest takes the
+    last expert) and a single expert; register-resident and two-pass kernels; bit-exact against the oracle, which
+    quantises every expert's rows separately with dynamic_quant."""
+    g = torch.Generator().manual_seed(rows + cols)
+    x = (torch.randn(rows, cols, generator=g) * 3).to(dt)
+    sm = (torch.rand(len(totals), cols, generator=g) * 4 + 0.01).to(dt)
+    gi = torch.tensor(totals, dtype=torch.int32)
+    y, s = capi.dynamic_quant(x.cuda(), sm.cuda(), gi.cuda())
+    yg, sg = golden.dynamic_quant_grouped(_bits(x), _bits(sm), totals, "fp16" if dt == torch.float16 else "bf16")
+    assert np.array_equal(s.cpu().numpy(), sg)
+    assert np.array_equal(y.cpu().numpy(), yg)
+    # one expert = the plain smooth-scale call
+    y1, s1 = capi.dynamic_quant(x.cuda(), sm[:1].contiguous().cuda(), torch.tensor([rows], dtype=torch.int32).cuda())
+    y0, s0 = capi.dynamic_quant(x.cuda(), sm[0].contiguous().cuda())
+    assert torch.equal(y1, y0) and torch.equal(s1, s0)
+
+
 # ------------------------------------------------------------------ quant_matmul
 
 QMM_SHAPES = [(1024, 4096, 1024), (256, 512, 352), (64, 4096, 512), (100, 256, 200), (1, 128, 16), (300, 1024, 1000),

@@ -795,3 +795,16 @@ def test_weight_quant_batchmatmul_int8_output(pa, golden):
         pa.npu_weight_quant_batchmatmul(x, w, sc, of, packed, qo.cuda(), None, gs)
     with pytest.raises(RuntimeError, match="quant_scale must be float32"):
         pa.npu_weight_quant_batchmatmul(x, w, sc, of, qs.to(torch.bfloat16).cuda(), None, None, gs)
+
+
+@pytest.mark.gpu
+def test_npu_dynamic_quant_group_index_operator(pa, golden):
+    """torch.ops.npu.npu_dynamic_quant with per-expert smooth scales: 3-D input, int64 totals."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(2, 24, 1024, generator=g).to(torch.bfloat16)
+    sm = (torch.rand(3, 1024, generator=g) + 0.5).to(torch.bfloat16)
+    totals = [16, 16, 48]
+    y, s = pa.npu_dynamic_quant(x.cuda(), smooth_scales=sm.cuda(), group_index=torch.tensor(totals).cuda())
+    yg, sg = golden.dynamic_quant_grouped(golden.bits_of(x), golden.bits_of(sm), totals)
+    assert y.shape == x.shape and s.shape == x.shape[:-1]
+    assert np.array_equal(y.cpu().numpy(), yg) and np.array_equal(s.cpu().numpy(), sg)

@@ -69,8 +69,15 @@ def test_meta_dynamic_quant(pa):
     assert s.shape == (4, 2048) and s.dtype == torch.float32
     y, s = pa.npu_dynamic_quant(_m(7, 64, dtype=torch.bfloat16), dst_type=torch.int8)
     assert y.shape == (7, 64) and s.shape == (7,)
-    with pytest.raises(RuntimeError, match="group_index"):
+    # per-expert smooth scales: smooth_scales [E, H] with group_index [E]
+    y, s = pa.npu_dynamic_quant(x, smooth_scales=_m(4, 1024, dtype=torch.float16), group_index=_m(4, dtype=torch.int32))
+    assert y.shape == (4, 2048, 1024) and s.shape == (4, 2048)
+    with pytest.raises(RuntimeError, match="group_index needs smooth_scales"):
         pa.npu_dynamic_quant(x, group_index=_m(4, dtype=torch.int32))
+    with pytest.raises(RuntimeError, match="with group_index, smooth_scales must have shape"):
+        pa.npu_dynamic_quant(x, smooth_scales=sm, group_index=_m(4, dtype=torch.int32))
+    with pytest.raises(RuntimeError, match="group_index must be int32 or int64"):
+        pa.npu_dynamic_quant(x, smooth_scales=_m(4, 1024, dtype=torch.float16), group_index=_m(4, dtype=torch.float32))
     with pytest.raises(RuntimeError, match="dst_type"):
         pa.npu_dynamic_quant(x, dst_type=torch.quint4x2)
     with pytest.raises(RuntimeError, match="bfloat16 or float16"):

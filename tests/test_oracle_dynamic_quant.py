@@ -128,6 +128,20 @@ def test_smooth_scales(golden):
     assert np.array_equal(y, torch.round(xf / scale[:, None]).clamp(-127, 127).to(torch.int8).numpy())
 
 
+def test_per_expert_smooth_scales(golden):
+    """group_index: rows below a running total take that expert's scales.  Checked against a torch float32 evaluation
+    with the scales gathered per row, with an empty expert, and with totals that stop short of the row count."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(12, 128, generator=g).to(torch.bfloat16)
+    sm = (torch.rand(4, 128, generator=g) + 0.5).to(torch.bfloat16)
+    for totals, expert_of_row in [([3, 3, 8, 12], [0] * 3 + [2] * 5 + [3] * 4), ([5, 7, 9, 10], [0] * 5 + [1] * 2 + [2] * 2 + [3] * 3)]:
+        y, s = golden.dynamic_quant_grouped(_bits(x), _bits(sm), totals)
+        xf = x.float() * sm.float()[torch.tensor(expert_of_row)]
+        scale = xf.abs().amax(-1) / 127.0
+        assert np.array_equal(s, scale.numpy())
+        assert np.array_equal(y, torch.round(xf / scale[:, None]).clamp(-127, 127).to(torch.int8).numpy())
+
+
 # ------------------------------------------------------------------ asymmetric variant
 
 def _asym_numpy(xf):
