@@ -92,6 +92,19 @@ int mi355_dynamic_quant_grouped(const void *x, int in_dtype, const void *smooth,
                                 int64_t rows, int64_t cols, int64_t x_row_stride, void *stream);
 
 /*
+ * npu_dynamic_quant with dst_type=torch.quint4x2: per-token symmetric int4 (the `dst_type` argument of the operator's
+ * signature, test/test_fake_tensor.py:1670-1687; the reference tree holds no call or golden for it, the meaning is the
+ * operator's published one: an int32 result whose last dimension is an eighth of the input's).
+ *   y_words  [rows, cols / 8] int32, contiguous; word j of a row holds the codes of columns 8j .. 8j+7, column 8j in
+ *            bits 0-3 (the nibble order of mi355_unpack_int4); cols must be a multiple of 8
+ *   scale    [rows] float32:  scale = max_j |x| / 7,  code = rint_half_even(x / scale) in [-7, 7]
+ * x, smooth, group_index, groups, rows, cols, x_row_stride as in mi355_dynamic_quant_grouped (group_index may be NULL).
+ */
+int mi355_dynamic_quant_int4(const void *x, int in_dtype, const void *smooth, const int32_t *group_index,
+                             int64_t groups, void *y_words, float *scale,
+                             int64_t rows, int64_t cols, int64_t x_row_stride, void *stream);
+
+/*
  * npu_dynamic_quant_asymmetric, per-token asymmetric int8.
  * Replaces the aclnn DynamicQuantV2 call behind torch_npu.npu_dynamic_quant_asymmetric (signature and output
  * shapes: test/test_fake_tensor.py:1689-1709, test/torch_npu_schema.json:2147-2149).  The arithmetic is not in the

@@ -114,6 +114,25 @@ def dynamic_quant_grouped(x_u16: np.ndarray, smooth_u16: np.ndarray, group_index
     return y.reshape(x.shape), scale.reshape(x.shape[:-1])
 
 
+def dynamic_quant_int4(x_u16: np.ndarray, in_dtype: str = "bf16", smooth_u16: np.ndarray | None = None):
+    """npu_dynamic_quant with dst_type=torch.quint4x2 (the argument is in the operator's signature,
+    test/test_fake_tensor.py:1670-1687; no call or golden in the reference tree): per row scale = max|x| / 7 and codes
+    rint(x / scale) in [-7, 7] (float32 operations, ties to even, a zero row gives scale 0 and codes 0), packed eight to
+    an int32 word, first column in the low nibble (the order pinned by test/custom_ops/test_npu_anti_quant.py:12-24).
+    Returns (int32 [..., cols / 8], scale float32 [...]).  PARITY UNPINNED: the operator's published description."""
+    u = _c(x_u16, np.uint16)
+    x = u.view(np.float16).astype(np.float32) if in_dtype == "fp16" else bf16_bits_to_f32(u)
+    if smooth_u16 is not None:
+        sm = _c(smooth_u16, np.uint16)
+        x = (x * (sm.view(np.float16).astype(np.float32) if in_dtype == "fp16" else bf16_bits_to_f32(sm))).astype(np.float32)
+    amax = np.abs(x).max(axis=-1, keepdims=True).astype(np.float32)
+    scale = (amax / np.float32(7.0)).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.rint((x / scale).astype(np.float32))
+    q = np.where(amax > 0, np.clip(np.nan_to_num(q, nan=0.0), -7, 7), 0).astype(np.int8)
+    return pack_int4(q), scale[..., 0]
+
+
 def dynamic_quant_asymmetric(x_u16: np.ndarray, in_dtype: str = "bf16", smooth_u16: np.ndarray | None = None):
     """x: uint16 bit patterns [..., cols] -> (y int8 same shape, scale float32 [...], offset float32 [...])."""
     x = _c(x_u16, np.uint16)

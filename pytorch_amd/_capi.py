@@ -14,7 +14,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
 
-EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant", "mi355_dynamic_quant_grouped",
+EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant", "mi355_dynamic_quant_grouped", "mi355_dynamic_quant_int4",
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
@@ -41,6 +41,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_quant_abi_version.restype = i32
         L.mi355_dynamic_quant.argtypes = [vp, i32, vp, vp, vp, i64, i64, i64, vp]
         L.mi355_dynamic_quant_grouped.argtypes = [vp, i32, vp, vp, i64, vp, vp, i64, i64, i64, vp]
+        L.mi355_dynamic_quant_int4.argtypes = [vp, i32, vp, vp, i64, vp, vp, i64, i64, i64, vp]
         L.mi355_quant_matmul_workspace.restype = sz
         L.mi355_quant_matmul_workspace.argtypes = [i64, i64, i64, i64, i64]
         L.mi355_quant_matmul.argtypes = [vp, vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
@@ -349,6 +350,20 @@ def unpack_int4(x, out=None):
     _check(lib().mi355_unpack_int4(_ptr(x), _ptr(out), rows, words * 8, x.stride(0), out.stride(0), _stream()),
            "mi355_unpack_int4")
     return out
+
+
+def dynamic_quant_int4(x: torch.Tensor, smooth: torch.Tensor | None = None, group_index: torch.Tensor | None = None):
+    """x bf16/fp16 [rows, cols] (cols % 8 == 0) -> (int32 [rows, cols / 8] of eight int4 codes each, scale float32 [rows])."""
+    _need_gpu(x, smooth)
+    assert x.dim() == 2 and (x.numel() == 0 or x.stride(1) == 1) and x.shape[1] % 8 == 0
+    rows, cols = x.shape
+    y = torch.empty((rows, cols // 8), dtype=torch.int32, device=x.device)
+    scale = torch.zeros((rows,), dtype=torch.float32, device=x.device)
+    _check(lib().mi355_dynamic_quant_int4(_ptr(x), 1 if x.dtype == torch.float16 else 0, _ptr(smooth), _ptr(group_index),
+                                          0 if group_index is None else group_index.numel(), _ptr(y), _ptr(scale), rows, cols,
+                                          x.stride(0) if rows > 1 else max(cols, 1), _stream()),
+           "mi355_dynamic_quant_int4")
+    return y, scale
 
 
 def dynamic_quant_asymmetric(x: torch.Tensor, smooth: torch.Tensor | None = None):

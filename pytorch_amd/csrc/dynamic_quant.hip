@@ -241,6 +241,50 @@ __global__ __launch_bounds__(kBlock) void dq_generic_kernel(const uint16_t *__re
     }
 }
 
+// int4 output (dst_type torch.quint4x2): scale = max|x| / 7, codes rint(x / scale) in [-7, 7], eight codes per int32
+// word with the first column in the low nibble (the order of mi355_unpack_int4 and mi355_anti_quant).  One block per
+// row, two passes like dq_generic_kernel; cols is a multiple of 8 and a thread packs whole words.
+template <bool FP16>
+__global__ __launch_bounds__(kBlock) void dq_int4_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ smooth,
+                                                         uint32_t *__restrict__ y, float *__restrict__ scale_out,
+                                                         int64_t cols, int64_t row_stride,
+                                                         const int32_t *__restrict__ group_index, int groups)
+{
+    const int64_t row = blockIdx.x;
+    const uint16_t *xr = x + row * row_stride;
+    if (smooth) smooth = expert_scales(smooth, group_index, groups, row, cols);
+    float amax = 0.0f;
+    for (int64_t j = threadIdx.x; j < cols; j += kBlock) {
+        float v = cvt1<FP16>(xr[j]);
+        if (smooth) v = v * cvt1<FP16>(smooth[j]);
+        amax = fmaxf(amax, fabsf(v));
+    }
+    uint32_t mb = wave_max_u32(__float_as_uint(amax));
+    __shared__ uint32_t part[kBlock / 64];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = mb;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; w++) mb = part[w] > mb ? part[w] : mb;
+    amax = __uint_as_float(mb);
+    const float scale = amax / 7.0f;
+    if (threadIdx.x == 0) scale_out[row] = scale;
+    uint32_t *yr = y + row * (cols >> 3);
+    const bool zero = !(amax > 0.0f);
+    for (int64_t w = threadIdx.x; w < (cols >> 3); w += kBlock) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float v = cvt1<FP16>(xr[8 * w + i]);
+            if (smooth) v = v * cvt1<FP16>(smooth[8 * w + i]);
+            float q = __builtin_rintf(v / scale);
+            q = q > 7.0f ? 7.0f : q;
+            q = q < -7.0f ? -7.0f : q;                       // NaN falls through both tests and converts to 0
+            word |= ((uint32_t)(int)q & 0xfu) << (4 * i);
+        }
+        yr[w] = zero ? 0u : word;
+    }
+}
+
 // Rows pre-multiplied by smooth scales, cols % 8 == 0 and at most 8 * BLOCK * MAXV, 16-byte aligned rows and smooth scales: one
 // block per row, the products (arbitrary float32 significands) stay in registers between the maximum and the
 // quantisation.  x / scale uses the row's refined reciprocal with the operation sequence of the compiler's own
@@ -471,6 +515,32 @@ extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smoo
                                    int64_t rows, int64_t cols, int64_t x_row_stride, void *stream)
 {
     return mi355_dynamic_quant_grouped(x, in_dtype, smooth, nullptr, 0, y, scale, rows, cols, x_row_stride, stream);
+}
+
+extern "C" int mi355_dynamic_quant_int4(const void *x, int in_dtype, const void *smooth, const int32_t *group_index,
+                                        int64_t groups, void *y_words, float *scale, int64_t rows, int64_t cols,
+                                        int64_t x_row_stride, void *stream)
+{
+    using namespace mi355;
+    if (rows < 0 || cols < 0 || (cols & 7) != 0) return MI355_ERR_BAD_ARGUMENT;
+    if (in_dtype != MI355_DTYPE_BF16 && in_dtype != MI355_DTYPE_FP16) return MI355_ERR_BAD_ARGUMENT;
+    if (group_index && (!smooth || groups < 1 || groups > 0x7fffffff)) return MI355_ERR_BAD_ARGUMENT;
+    if (group_index && !aligned(group_index, 4)) return MI355_ERR_ALIGNMENT;
+    if (rows == 0) return MI355_OK;
+    if (!scale) return MI355_ERR_BAD_ARGUMENT;
+    if (cols > 0 && (!x || !y_words || x_row_stride < cols)) return MI355_ERR_BAD_ARGUMENT;
+    if (y_words && !aligned(y_words, 4)) return MI355_ERR_ALIGNMENT;
+    if (rows > 0x7fffffff) return MI355_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint16_t *xp = static_cast<const uint16_t *>(x), *sm = static_cast<const uint16_t *>(smooth);
+    const int ng = group_index ? (int)groups : 0;
+    if (in_dtype == MI355_DTYPE_FP16)
+        hipLaunchKernelGGL((dq_int4_kernel<true>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, static_cast<uint32_t *>(y_words),
+                           scale, cols, x_row_stride, group_index, ng);
+    else
+        hipLaunchKernelGGL((dq_int4_kernel<false>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, static_cast<uint32_t *>(y_words),
+                           scale, cols, x_row_stride, group_index, ng);
+    return check_launch();
 }
 
 extern "C" int mi355_dynamic_quant_grouped(const void *x, int in_dtype, const void *smooth, const int32_t *group_index,

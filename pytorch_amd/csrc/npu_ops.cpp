@@ -68,8 +68,11 @@ void dynamic_quant_check(const Tensor &input, const optional<Tensor> &smooth_sca
                 "npu_dynamic_quant: input must be bfloat16 or float16, got ", input.scalar_type());
     TORCH_CHECK(input.dim() >= 1, "npu_dynamic_quant: input must have at least one dimension");
     TORCH_CHECK(grouped_ok || !opt(group_index), "npu_dynamic_quant: group_index (per-expert smooth scales) is not supported");
-    TORCH_CHECK(!dst_type.has_value() || *dst_type == at::kChar,
-                "npu_dynamic_quant: only dst_type=torch.int8 is supported, got ", *dst_type);
+    TORCH_CHECK(!dst_type.has_value() || *dst_type == at::kChar || (grouped_ok && *dst_type == at::kQUInt4x2),
+                "npu_dynamic_quant: dst_type must be torch.int8", grouped_ok ? " or torch.quint4x2" : "", ", got ", *dst_type);
+    if (dst_type.has_value() && *dst_type == at::kQUInt4x2)
+        TORCH_CHECK(input.size(-1) % 8 == 0, "npu_dynamic_quant: dst_type=torch.quint4x2 packs eight values per int32 word: the last "
+                    "dimension must be a multiple of 8, got ", input.size(-1));
     if (const Tensor *g = opt(group_index)) {
         const Tensor *s = opt(smooth_scales);
         TORCH_CHECK(s, "npu_dynamic_quant: group_index needs smooth_scales of shape [experts, ", input.size(-1), "]");
@@ -87,11 +90,14 @@ void dynamic_quant_check(const Tensor &input, const optional<Tensor> &smooth_sca
     }
 }
 
-std::tuple<Tensor, Tensor> dynamic_quant_alloc(const Tensor &input)
+// int4: an int32 result whose last dimension is an eighth of the input's
+std::tuple<Tensor, Tensor> dynamic_quant_alloc(const Tensor &input, bool int4 = false)
 {
     auto scale_shape = input.sizes().vec();
     scale_shape.pop_back();
-    return {at::empty(input.sizes(), input.options().dtype(at::kChar)),
+    auto y_shape = input.sizes().vec();
+    if (int4) y_shape.back() /= 8;
+    return {at::empty(y_shape, input.options().dtype(int4 ? at::kInt : at::kChar)),
             at::empty(scale_shape, input.options().dtype(at::kFloat))};
 }
 
@@ -99,7 +105,7 @@ std::tuple<Tensor, Tensor> dynamic_quant_meta(const Tensor &input, const optiona
                                               const optional<Tensor> &group_index, optional<at::ScalarType> dst_type)
 {
     dynamic_quant_check(input, smooth_scales, group_index, dst_type, true);
-    return dynamic_quant_alloc(input);
+    return dynamic_quant_alloc(input, dst_type.has_value() && *dst_type == at::kQUInt4x2);
 }
 
 std::tuple<Tensor, Tensor> dynamic_quant_hip(const Tensor &input, const optional<Tensor> &smooth_scales,
@@ -108,7 +114,8 @@ std::tuple<Tensor, Tensor> dynamic_quant_hip(const Tensor &input, const optional
     dynamic_quant_check(input, smooth_scales, group_index, dst_type, true);
     check_same_device("npu_dynamic_quant", {&input, opt(smooth_scales), opt(group_index)});
     c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
-    auto [y, scale] = dynamic_quant_alloc(input);
+    const bool int4 = dst_type.has_value() && *dst_type == at::kQUInt4x2;
+    auto [y, scale] = dynamic_quant_alloc(input, int4);
     const int64_t cols = input.size(-1);
     const int64_t rows = cols ? input.numel() / cols : 0;
     if (rows == 0 || cols == 0) {
@@ -127,6 +134,14 @@ std::tuple<Tensor, Tensor> dynamic_quant_hip(const Tensor &input, const optional
     if (const Tensor *s = opt(smooth_scales)) smooth = s->contiguous();
     Tensor gi;                                             // a handful of totals: int64 ones are narrowed on the device
     if (const Tensor *g = opt(group_index)) gi = g->to(at::kInt).contiguous();
+    if (int4) {
+        check_status(mi355_dynamic_quant_int4(x.data_ptr(), x.scalar_type() == at::kBFloat16 ? MI355_DTYPE_BF16 : MI355_DTYPE_FP16,
+                                              smooth.defined() ? smooth.data_ptr() : nullptr,
+                                              gi.defined() ? gi.data_ptr<int32_t>() : nullptr, gi.defined() ? gi.numel() : 0,
+                                              y.data_ptr(), scale.data_ptr<float>(), rows, cols, row_stride, stream_of(input)),
+                     "npu_dynamic_quant");
+        return {y, scale};
+    }
     check_status(mi355_dynamic_quant_grouped(x.data_ptr(), x.scalar_type() == at::kBFloat16 ? MI355_DTYPE_BF16 : MI355_DTYPE_FP16,
                                              smooth.defined() ? smooth.data_ptr() : nullptr,
                                              gi.defined() ? gi.data_ptr<int32_t>() : nullptr, gi.defined() ? gi.numel() : 0,

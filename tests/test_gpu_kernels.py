@@ -148,6 +148,33 @@ def test_dynamic_quant_per_expert_smooth_scales(capi, golden, rows, cols, totals
     assert torch.equal(y1, y0) and torch.equal(s1, s0)
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 4096), (5, 1000), (3, 24), (33, 14336)])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_dynamic_quant_int4_output(capi, golden, rows, cols, dt):
+    """dst_type=torch.quint4x2 through the C ABI: packed int4 codes and scales bit-exact against the oracle, plain, with
+    smooth scales and with per-expert smooth scales; a zero row, tiny values, rows that use every code."""
+    name = "fp16" if dt == torch.float16 else "bf16"
+    g = torch.Generator().manual_seed(rows * 7 + cols)
+    x = torch.randn(rows, cols, generator=g) * 3
+    x[0] = 0
+    x[1] = x[1] * 1e-6
+    x = x.to(dt)
+    y, s = capi.dynamic_quant_int4(x.cuda())
+    yg, sg = golden.dynamic_quant_int4(_bits(x), name)
+    assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(y.cpu().numpy(), yg)
+    codes = golden.unpack_int4(yg)
+    assert codes.min() == -7 and codes.max() == 7
+    sm = (torch.rand(2, cols, generator=g) * 4 + 0.01).to(dt)
+    y, s = capi.dynamic_quant_int4(x.cuda(), sm[0].contiguous().cuda())
+    yg, sg = golden.dynamic_quant_int4(_bits(x), name, _bits(sm[0]))
+    assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(y.cpu().numpy(), yg)
+    cut = rows // 2
+    y, s = capi.dynamic_quant_int4(x.cuda(), sm.cuda(), torch.tensor([cut, rows], dtype=torch.int32).cuda())
+    for lo, hi, e in ((0, cut, 0), (cut, rows, 1)):
+        yg, sg = golden.dynamic_quant_int4(_bits(x[lo:hi]), name, _bits(sm[e]))
+        assert np.array_equal(s[lo:hi].cpu().numpy(), sg) and np.array_equal(y[lo:hi].cpu().numpy(), yg)
+
+
 # ------------------------------------------------------------------ quant_matmul
 
 QMM_SHAPES = [(1024, 4096, 1024), (256, 512, 352), (64, 4096, 512), (100, 256, 200), (1, 128, 16), (300, 1024, 1000),

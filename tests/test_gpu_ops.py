@@ -808,3 +808,17 @@ def test_npu_dynamic_quant_group_index_operator(pa, golden):
     yg, sg = golden.dynamic_quant_grouped(golden.bits_of(x), golden.bits_of(sm), totals)
     assert y.shape == x.shape and s.shape == x.shape[:-1]
     assert np.array_equal(y.cpu().numpy(), yg) and np.array_equal(s.cpu().numpy(), sg)
+
+
+@pytest.mark.gpu
+def test_npu_dynamic_quant_int4_operator(pa, golden):
+    """torch.ops.npu.npu_dynamic_quant(dst_type=torch.quint4x2): int32 words, last dimension an eighth; the words feed
+    npu_anti_quant (int4 source) back to values within half a scale step of the input."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 10, 512, generator=g).to(torch.bfloat16)
+    y, s = pa.npu_dynamic_quant(x.cuda(), dst_type=torch.quint4x2)
+    yg, sg = golden.dynamic_quant_int4(golden.bits_of(x))
+    assert y.dtype == torch.int32 and y.shape == (3, 10, 64) and s.shape == (3, 10)
+    assert np.array_equal(y.cpu().numpy(), yg) and np.array_equal(s.cpu().numpy(), sg)
+    codes = torch.from_numpy(golden.unpack_int4(yg)).float()
+    assert float(((codes * torch.from_numpy(sg)[..., None]) - x.float()).abs().max()) <= 0.5 * float(sg.max()) * 1.001

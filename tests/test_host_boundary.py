@@ -78,8 +78,13 @@ def test_meta_dynamic_quant(pa):
         pa.npu_dynamic_quant(x, smooth_scales=sm, group_index=_m(4, dtype=torch.int32))
     with pytest.raises(RuntimeError, match="group_index must be int32 or int64"):
         pa.npu_dynamic_quant(x, smooth_scales=_m(4, 1024, dtype=torch.float16), group_index=_m(4, dtype=torch.float32))
-    with pytest.raises(RuntimeError, match="dst_type"):
-        pa.npu_dynamic_quant(x, dst_type=torch.quint4x2)
+    # int4 codes: eight to an int32 word
+    y, s = pa.npu_dynamic_quant(x, dst_type=torch.quint4x2)
+    assert y.shape == (4, 2048, 128) and y.dtype == torch.int32 and s.shape == (4, 2048)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        pa.npu_dynamic_quant(_m(4, 12, dtype=torch.float16), dst_type=torch.quint4x2)
+    with pytest.raises(RuntimeError, match="dst_type must be"):
+        pa.npu_dynamic_quant(x, dst_type=torch.uint8)
     with pytest.raises(RuntimeError, match="bfloat16 or float16"):
         pa.npu_dynamic_quant(_m(4, 8, dtype=torch.float32))
     with pytest.raises(RuntimeError, match="smooth_scales"):

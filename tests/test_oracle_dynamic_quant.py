@@ -142,6 +142,27 @@ def test_per_expert_smooth_scales(golden):
         assert np.array_equal(y, torch.round(xf / scale[:, None]).clamp(-127, 127).to(torch.int8).numpy())
 
 
+def test_int4_output_hand_computed_and_torch(golden):
+    """dst_type=torch.quint4x2: scale = max|x| / 7, codes rint(x / scale), eight to a word with the first column in the
+    low nibble.  A row typed by hand (scale 1; ties 3.5 -> 4, 2.5 -> 2, +-0.5 -> 0; -7 is nibble 9) and a torch float32
+    evaluation unpacked with the oracle's own unpack_int4 (whose nibble order the reference pins)."""
+    row = torch.tensor([[7.0, -7.0, 3.5, 2.5, 0.5, -0.5, 1.0, 0.0]], dtype=torch.bfloat16)
+    y, s = golden.dynamic_quant_int4(_bits(row))
+    assert s.tolist() == [1.0] and y.dtype == np.int32 and y.shape == (1, 1)
+    assert int(y.view(np.uint32)[0, 0]) == 0x01002497
+    g = torch.Generator().manual_seed(8)
+    x = (torch.randn(16, 256, generator=g) * 2).to(torch.bfloat16)
+    x[3] = 0
+    sm = (torch.rand(256, generator=g) + 0.5).to(torch.bfloat16)
+    for smooth in (None, sm):
+        y, s = golden.dynamic_quant_int4(_bits(x), smooth_u16=None if smooth is None else _bits(smooth))
+        xf = x.float() if smooth is None else x.float() * smooth.float()
+        scale = xf.abs().amax(-1) / 7.0
+        assert np.array_equal(s, scale.numpy())
+        want = torch.where(scale[:, None] > 0, torch.round(xf / scale[:, None]), torch.zeros(())).to(torch.int8).numpy()
+        assert np.array_equal(golden.unpack_int4(y), want) and want.min() == -7 and want.max() == 7
+
+
 # ------------------------------------------------------------------ asymmetric variant
 
 def _asym_numpy(xf):
