@@ -120,6 +120,14 @@ int mi355_dynamic_quant_asymmetric(const void *x, int in_dtype, const void *smoo
                                    int64_t rows, int64_t cols, int64_t x_row_stride, void *stream);
 
 /*
+ * npu_dynamic_quant_asymmetric with per-expert smooth scales (`group_index`): smooth [groups, cols], group_index as in
+ * mi355_dynamic_quant_grouped (NULL: as mi355_dynamic_quant_asymmetric); everything else as mi355_dynamic_quant_asymmetric.
+ */
+int mi355_dynamic_quant_asymmetric_grouped(const void *x, int in_dtype, const void *smooth, const int32_t *group_index,
+                                           int64_t groups, int8_t *y, float *scale, float *offset,
+                                           int64_t rows, int64_t cols, int64_t x_row_stride, void *stream);
+
+/*
  * npu_quant_matmul, W8A8 with int32 accumulation and fused dequantisation.
  * Replaces the aclnn QuantMatmul call behind torch_npu.npu_quant_matmul
  * (callers: torch_npu/contrib/module/linear_quant.py:96-112, linear_a8w8_quant.py:87-120;

@@ -148,6 +148,25 @@ def dynamic_quant_asymmetric(x_u16: np.ndarray, in_dtype: str = "bf16", smooth_u
     return y, scale, offset
 
 
+def dynamic_quant_asymmetric_grouped(x_u16: np.ndarray, smooth_u16: np.ndarray, group_index, in_dtype: str = "bf16"):
+    """npu_dynamic_quant_asymmetric with per-expert smooth scales: dynamic_quant_asymmetric applied to every expert's rows
+    with that expert's scales (group_index as in dynamic_quant_grouped; PARITY UNPINNED likewise)."""
+    x = _c(x_u16, np.uint16)
+    x2 = x.reshape(-1, x.shape[-1])
+    sm = _c(smooth_u16, np.uint16)
+    gi = [int(v) for v in np.asarray(group_index).reshape(-1)]
+    y = np.empty(x2.shape, dtype=np.int8)
+    scale = np.empty(x2.shape[0], dtype=np.float32)
+    offset = np.empty(x2.shape[0], dtype=np.float32)
+    lo = 0
+    for e, hi in enumerate(gi):
+        hi = x2.shape[0] if e == len(gi) - 1 else min(max(hi, lo), x2.shape[0])
+        if hi > lo:
+            y[lo:hi], scale[lo:hi], offset[lo:hi] = dynamic_quant_asymmetric(x2[lo:hi], in_dtype, sm[e])
+        lo = max(lo, hi)
+    return y.reshape(x.shape), scale.reshape(x.shape[:-1]), offset.reshape(x.shape[:-1])
+
+
 def int8_gemm(a: np.ndarray, b: np.ndarray) -> np.ndarray:
     """a int8 [M,K] (row-major), b int8 [K,N] with arbitrary numpy strides -> int32 [M,N]."""
     a = _c(a, np.int8)

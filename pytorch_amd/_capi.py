@@ -14,7 +14,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
 
-EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant", "mi355_dynamic_quant_grouped", "mi355_dynamic_quant_int4",
+EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant", "mi355_dynamic_quant_grouped", "mi355_dynamic_quant_int4", "mi355_dynamic_quant_asymmetric_grouped",
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
@@ -55,6 +55,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_anti_quant.argtypes = [vp, i32, vp, i64, vp, i64, vp, i32, i64, i64, i64, i64, vp]
         L.mi355_unpack_int4.argtypes = [vp, vp, i64, i64, i64, i64, vp]
         L.mi355_dynamic_quant_asymmetric.argtypes = [vp, i32, vp, vp, vp, vp, i64, i64, i64, vp]
+        L.mi355_dynamic_quant_asymmetric_grouped.argtypes = [vp, i32, vp, vp, i64, vp, vp, vp, i64, i64, i64, vp]
         L.mi355_trans_quant_param.argtypes = [vp, i64, vp, i64, vp, i64, vp]
         L.mi355_quant_matmul_qparam.argtypes = [vp, vp, vp, i64, vp, i32, vp, i32, i64, i64, i64, i64, i64, i64, i64, vp, sz, vp]
         L.mi355_quantize.argtypes = [vp, i32, vp, i64, vp, i32, i64, vp, i32, i64, i64, i64, i32, vp]
@@ -366,14 +367,21 @@ def dynamic_quant_int4(x: torch.Tensor, smooth: torch.Tensor | None = None, grou
     return y, scale
 
 
-def dynamic_quant_asymmetric(x: torch.Tensor, smooth: torch.Tensor | None = None):
-    """x bf16/fp16 [rows, cols] (row pitch x.stride(0)) -> (int8 [rows, cols], scale float32 [rows], offset float32 [rows])."""
+def dynamic_quant_asymmetric(x: torch.Tensor, smooth: torch.Tensor | None = None, group_index: torch.Tensor | None = None):
+    """x bf16/fp16 [rows, cols] (row pitch x.stride(0)) -> (int8 [rows, cols], scale float32 [rows], offset float32 [rows]).
+    With group_index (int32 [E], running row totals per expert) smooth is [E, cols]."""
     _need_gpu(x, smooth)
     assert x.dim() == 2 and (x.numel() == 0 or x.stride(1) == 1)
     rows, cols = x.shape
     y = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
     scale = torch.zeros((rows,), dtype=torch.float32, device=x.device)
     offset = torch.zeros((rows,), dtype=torch.float32, device=x.device)
+    if group_index is not None:
+        _check(lib().mi355_dynamic_quant_asymmetric_grouped(_ptr(x), 1 if x.dtype == torch.float16 else 0, _ptr(smooth),
+                                                            _ptr(group_index), group_index.numel(), _ptr(y), _ptr(scale), _ptr(offset),
+                                                            rows, cols, x.stride(0) if rows > 1 else max(cols, 1), _stream()),
+               "mi355_dynamic_quant_asymmetric_grouped")
+        return y, scale, offset
     _check(lib().mi355_dynamic_quant_asymmetric(_ptr(x), 1 if x.dtype == torch.float16 else 0, _ptr(smooth), _ptr(y), _ptr(scale),
                                                 _ptr(offset), rows, cols, x.stride(0) if rows > 1 else max(cols, 1), _stream()),
            "mi355_dynamic_quant_asymmetric")

@@ -70,6 +70,18 @@ __device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2)
     return pack_bf16x2(s0 * bf16_lo(b2), s1 * bf16_hi(b2));
 }
 
+// Per-expert smooth scales (npu_dynamic_quant with group_index): `group_index` holds the running totals of the rows of
+// each expert, so row r belongs to the first expert e with r < group_index[e] (rows past the last total take the last
+// expert); returns the first element of that expert's scales.
+__device__ __forceinline__ const uint16_t *expert_scales(const uint16_t *smooth, const int32_t *group_index, int groups, int64_t row,
+                                                         int64_t cols)
+{
+    if (!group_index) return smooth;
+    int e = 0;
+    while (e < groups - 1 && row >= (int64_t)group_index[e]) e++;
+    return smooth + (int64_t)e * cols;
+}
+
 // Every workspace of this library starts with a zero area: kWorkspaceCounterCapacity bytes of arrival counters followed
 // by kWorkspaceZoneBytes for exchanges that recognise data by its being non-zero (weight_quant_decode.hip).  The area
 // is zero before the first launch and every launch leaves it zero; whatever else a launch keeps in the workspace

@@ -193,18 +193,6 @@ __global__ __launch_bounds__(BLOCK) void dq_rows_kernel(const uint16_t *__restri
     }
 }
 
-// Per-expert smooth scales (npu_dynamic_quant with group_index): `group_index` holds the running totals of the rows of
-// each expert, so row r belongs to the first expert e with r < group_index[e] (rows past the last total take the last
-// expert); returns the first element of that expert's scales.
-__device__ __forceinline__ const uint16_t *expert_scales(const uint16_t *smooth, const int32_t *group_index, int groups, int64_t row,
-                                                         int64_t cols)
-{
-    if (!group_index) return smooth;
-    int e = 0;
-    while (e < groups - 1 && row >= (int64_t)group_index[e]) e++;
-    return smooth + (int64_t)e * cols;
-}
-
 // Any shape, stride and alignment; optional smooth scales.  One block per row, two passes
 // over the row (the second one hits in cache), IEEE division per element.
 template <bool FP16>

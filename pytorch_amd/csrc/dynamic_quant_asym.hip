@@ -51,11 +51,14 @@ __device__ __forceinline__ uint32_t quant1_rcp(float x, float scale, float r, fl
 template <bool FP16, bool VEC, bool REG = false>
 __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ smooth,
                                                       int8_t *__restrict__ y, float *__restrict__ scale_out,
-                                                      float *__restrict__ offset_out, int64_t rows, int cols, int64_t row_stride)
+                                                      float *__restrict__ offset_out, int64_t rows, int cols, int64_t row_stride,
+                                                      const int32_t *__restrict__ group_index = nullptr, int groups = 0)
 {
     __shared__ float red[2][4];
     const int t = threadIdx.x;
+    const uint16_t *const smooth_all = smooth;
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        if (smooth_all) smooth = expert_scales(smooth_all, group_index, groups, row, cols);   // per-expert scales: this row's vector
         const uint16_t *xr = x + row * row_stride;
         int8_t *yr = y + row * (int64_t)cols;
         float mx = -INFINITY, mn = INFINITY;
@@ -154,8 +157,18 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
 extern "C" int mi355_dynamic_quant_asymmetric(const void *x, int in_dtype, const void *smooth, int8_t *y, float *scale,
                                               float *offset, int64_t rows, int64_t cols, int64_t x_row_stride, void *stream)
 {
+    return mi355_dynamic_quant_asymmetric_grouped(x, in_dtype, smooth, nullptr, 0, y, scale, offset, rows, cols, x_row_stride, stream);
+}
+
+extern "C" int mi355_dynamic_quant_asymmetric_grouped(const void *x, int in_dtype, const void *smooth, const int32_t *group_index,
+                                                      int64_t groups, int8_t *y, float *scale, float *offset, int64_t rows,
+                                                      int64_t cols, int64_t x_row_stride, void *stream)
+{
     using namespace mi355;
     if (rows < 0 || cols < 0) return MI355_ERR_BAD_ARGUMENT;
+    if (group_index && (!smooth || groups < 1 || groups > 0x7fffffff)) return MI355_ERR_BAD_ARGUMENT;
+    if (group_index && !aligned(group_index, 4)) return MI355_ERR_ALIGNMENT;
+    const int ng = group_index ? (int)groups : 0;
     if (in_dtype != MI355_DTYPE_BF16 && in_dtype != MI355_DTYPE_FP16) return MI355_ERR_BAD_ARGUMENT;
     if (rows == 0) return MI355_OK;
     if (!scale || !offset) return MI355_ERR_BAD_ARGUMENT;
@@ -168,7 +181,8 @@ extern "C" int mi355_dynamic_quant_asymmetric(const void *x, int in_dtype, const
     const unsigned blocks = (unsigned)(rows < 256 * 64 ? rows : 256 * 64);
     const bool f16 = in_dtype == MI355_DTYPE_FP16;
 #define MI355_DQA_LAUNCH(F, V, R) \
-    hipLaunchKernelGGL((dq_asym_kernel<F, V, R>), dim3(blocks), dim3(256), 0, s, xp, sp, y, scale, offset, rows, (int)cols, x_row_stride)
+    hipLaunchKernelGGL((dq_asym_kernel<F, V, R>), dim3(blocks), dim3(256), 0, s, xp, sp, y, scale, offset, rows, (int)cols, x_row_stride, \
+                       group_index, ng)
     const bool reg = vec && cols <= 8192;
     if (f16 && reg) MI355_DQA_LAUNCH(true, true, true);
     else if (f16 && vec) MI355_DQA_LAUNCH(true, true, false);

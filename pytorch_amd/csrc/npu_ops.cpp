@@ -59,17 +59,16 @@ void *stream_of(const Tensor &t)
 
 // ---------------------------------------------------------------- npu_dynamic_quant
 
-// `grouped_ok`: the operator takes per-expert smooth scales (smooth_scales [E, H] with group_index [E], the running
-// totals of the rows of each expert)
+// Per-expert smooth scales: smooth_scales [E, H] with group_index [E], the running totals of the rows of each expert.
+// `int4_ok`: the operator also packs int4 codes (dst_type torch.quint4x2).
 void dynamic_quant_check(const Tensor &input, const optional<Tensor> &smooth_scales, const optional<Tensor> &group_index,
-                         optional<at::ScalarType> dst_type, bool grouped_ok = false)
+                         optional<at::ScalarType> dst_type, bool int4_ok = false)
 {
     TORCH_CHECK(input.scalar_type() == at::kBFloat16 || input.scalar_type() == at::kHalf,
                 "npu_dynamic_quant: input must be bfloat16 or float16, got ", input.scalar_type());
     TORCH_CHECK(input.dim() >= 1, "npu_dynamic_quant: input must have at least one dimension");
-    TORCH_CHECK(grouped_ok || !opt(group_index), "npu_dynamic_quant: group_index (per-expert smooth scales) is not supported");
-    TORCH_CHECK(!dst_type.has_value() || *dst_type == at::kChar || (grouped_ok && *dst_type == at::kQUInt4x2),
-                "npu_dynamic_quant: dst_type must be torch.int8", grouped_ok ? " or torch.quint4x2" : "", ", got ", *dst_type);
+    TORCH_CHECK(!dst_type.has_value() || *dst_type == at::kChar || (int4_ok && *dst_type == at::kQUInt4x2),
+                "npu_dynamic_quant: dst_type must be torch.int8", int4_ok ? " or torch.quint4x2" : "", ", got ", *dst_type);
     if (dst_type.has_value() && *dst_type == at::kQUInt4x2)
         TORCH_CHECK(input.size(-1) % 8 == 0, "npu_dynamic_quant: dst_type=torch.quint4x2 packs eight values per int32 word: the last "
                     "dimension must be a multiple of 8, got ", input.size(-1));
@@ -174,7 +173,7 @@ std::tuple<Tensor, Tensor, Tensor> dynamic_quant_asym_hip(const Tensor &input, c
                                                           optional<at::ScalarType> dst_type)
 {
     dynamic_quant_check(input, smooth_scales, group_index, dst_type);
-    check_same_device("npu_dynamic_quant_asymmetric", {&input, opt(smooth_scales)});
+    check_same_device("npu_dynamic_quant_asymmetric", {&input, opt(smooth_scales), opt(group_index)});
     c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     auto [y, scale, offset] = dynamic_quant_asym_alloc(input);
     const int64_t cols = input.size(-1);
@@ -193,11 +192,14 @@ std::tuple<Tensor, Tensor, Tensor> dynamic_quant_asym_hip(const Tensor &input, c
     }
     Tensor smooth;
     if (const Tensor *s = opt(smooth_scales)) smooth = s->contiguous();
-    check_status(mi355_dynamic_quant_asymmetric(x.data_ptr(),
-                                                x.scalar_type() == at::kBFloat16 ? MI355_DTYPE_BF16 : MI355_DTYPE_FP16,
-                                                smooth.defined() ? smooth.data_ptr() : nullptr, y.data_ptr<int8_t>(),
-                                                scale.data_ptr<float>(), offset.data_ptr<float>(), rows, cols, row_stride,
-                                                stream_of(input)),
+    Tensor gi;
+    if (const Tensor *g = opt(group_index)) gi = g->to(at::kInt).contiguous();
+    check_status(mi355_dynamic_quant_asymmetric_grouped(x.data_ptr(),
+                                                        x.scalar_type() == at::kBFloat16 ? MI355_DTYPE_BF16 : MI355_DTYPE_FP16,
+                                                        smooth.defined() ? smooth.data_ptr() : nullptr,
+                                                        gi.defined() ? gi.data_ptr<int32_t>() : nullptr, gi.defined() ? gi.numel() : 0,
+                                                        y.data_ptr<int8_t>(), scale.data_ptr<float>(), offset.data_ptr<float>(), rows,
+                                                        cols, row_stride, stream_of(input)),
                  "npu_dynamic_quant_asymmetric");
     return {y, scale, offset};
 }

@@ -175,6 +175,19 @@ def test_dynamic_quant_int4_output(capi, golden, rows, cols, dt):
         assert np.array_equal(s[lo:hi].cpu().numpy(), sg) and np.array_equal(y[lo:hi].cpu().numpy(), yg)
 
 
+@pytest.mark.parametrize("rows,cols,totals", [(64, 4096, [10, 10, 37, 64]), (20, 8200, [5, 9, 12]), (9, 1000, [9])])
+def test_dynamic_quant_asymmetric_per_expert_smooth_scales(capi, golden, rows, cols, totals):
+    """group_index of npu_dynamic_quant_asymmetric: as for the symmetric operator, bit-exact against the oracle applied per
+    expert (register-resident, vector and scalar kernels)."""
+    g = torch.Generator().manual_seed(rows + cols)
+    x = (torch.randn(rows, cols, generator=g) * 3 + 0.5).to(torch.bfloat16)
+    sm = (torch.rand(len(totals), cols, generator=g) * 4 + 0.01).to(torch.bfloat16)
+    y, s, o = capi.dynamic_quant_asymmetric(x.cuda(), sm.cuda(), torch.tensor(totals, dtype=torch.int32).cuda())
+    yg, sg, og = golden.dynamic_quant_asymmetric_grouped(_bits(x), _bits(sm), totals)
+    assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(o.cpu().numpy(), og)
+    assert np.array_equal(y.cpu().numpy(), yg)
+
+
 # ------------------------------------------------------------------ quant_matmul
 
 QMM_SHAPES = [(1024, 4096, 1024), (256, 512, 352), (64, 4096, 512), (100, 256, 200), (1, 128, 16), (300, 1024, 1000),

@@ -96,6 +96,11 @@ def test_meta_dynamic_quant_asymmetric(pa):
     y, s, o = pa.npu_dynamic_quant_asymmetric(_m(4, 2048, 1024, dtype=torch.float16), smooth_scales=_m(1024, dtype=torch.float16))
     assert y.shape == (4, 2048, 1024) and y.dtype == torch.int8
     assert s.shape == (4, 2048) and s.dtype == torch.float32 and o.shape == (4, 2048) and o.dtype == torch.float32
+    y, s, o = pa.npu_dynamic_quant_asymmetric(_m(64, 1024, dtype=torch.float16), smooth_scales=_m(3, 1024, dtype=torch.float16),
+                                              group_index=_m(3, dtype=torch.int64))
+    assert y.shape == (64, 1024) and s.shape == (64,) and o.shape == (64,)
+    with pytest.raises(RuntimeError, match="dst_type must be torch.int8, got"):
+        pa.npu_dynamic_quant_asymmetric(_m(64, 1024, dtype=torch.float16), dst_type=torch.quint4x2)
 
 
 def test_meta_quant_matmul(pa):
