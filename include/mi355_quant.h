@@ -327,6 +327,15 @@ int mi355_swiglu_quant_smooth(const void *x_bf16, int activate_left, const void 
                               int64_t rows, int64_t half, int64_t x_row_stride, void *stream);
 
 /*
+ * The same with per-expert smooth scales (the `group_index` argument of torch_npu.npu_swiglu_quant; the operator is only
+ * named in the reference tree, the meaning is the vendor's published one): smooth_bf16 [groups, half], group_index
+ * [groups] int32 on the device, running totals of the rows of each expert as in mi355_dynamic_quant_grouped.
+ */
+int mi355_swiglu_quant_grouped(const void *x_bf16, int activate_left, const void *smooth_bf16, const int32_t *group_index,
+                               int64_t groups, int8_t *y, float *scale, int64_t rows, int64_t half, int64_t x_row_stride,
+                               void *stream);
+
+/*
  * npu_anti_quant: the standalone antiquantisation out = cast((float(x) + offset) * scale).
  * Replaces the aclnn AscendAntiQuant call behind torch_npu.npu_anti_quant (signature test/torch_npu_schema.json:2117-2119,
  * wrapper torch_npu/onnx/wrapper_onnx_ops.py:824-828; CPU golden test/custom_ops/test_npu_anti_quant.py:29-42, int4

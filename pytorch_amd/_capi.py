@@ -14,7 +14,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmi355_quant.so")
 
-EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant", "mi355_dynamic_quant_grouped", "mi355_dynamic_quant_int4", "mi355_dynamic_quant_asymmetric_grouped",
+EXPORTS = ("mi355_status_string", "mi355_quant_abi_version", "mi355_dynamic_quant", "mi355_dynamic_quant_grouped", "mi355_dynamic_quant_int4", "mi355_dynamic_quant_asymmetric_grouped", "mi355_swiglu_quant_grouped",
            "mi355_quant_matmul_workspace", "mi355_quant_matmul",
            "mi355_weight_quant_matmul_workspace", "mi355_weight_quant_matmul", "mi355_swiglu", "mi355_swiglu_quant",
            "mi355_anti_quant", "mi355_unpack_int4", "mi355_dynamic_quant_asymmetric", "mi355_quantize",
@@ -52,6 +52,7 @@ def lib() -> ctypes.CDLL:
         L.mi355_swiglu.argtypes = [vp, vp, i64, i64, i64, vp]
         L.mi355_swiglu_quant.argtypes = [vp, i32, vp, vp, i64, i64, i64, vp]
         L.mi355_swiglu_quant_smooth.argtypes = [vp, i32, vp, vp, vp, i64, i64, i64, vp]
+        L.mi355_swiglu_quant_grouped.argtypes = [vp, i32, vp, vp, i64, vp, vp, i64, i64, i64, vp]
         L.mi355_anti_quant.argtypes = [vp, i32, vp, i64, vp, i64, vp, i32, i64, i64, i64, i64, vp]
         L.mi355_unpack_int4.argtypes = [vp, vp, i64, i64, i64, i64, vp]
         L.mi355_dynamic_quant_asymmetric.argtypes = [vp, i32, vp, vp, vp, vp, i64, i64, i64, vp]
@@ -289,12 +290,16 @@ def swiglu(x):
     return out
 
 
-def swiglu_quant(x, activate_left: bool = True, smooth=None):
+def swiglu_quant(x, activate_left: bool = True, smooth=None, group_index=None):
     """x bf16 [rows, 2*half] -> (int8 [rows, half], float32 [rows]) = dynamic_quant(swiglu(x), smooth)."""
     _need_gpu(x, smooth)
     rows, two = x.shape
     y = torch.empty((rows, two // 2), dtype=torch.int8, device=x.device)
     scale = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    if group_index is not None:
+        _check(lib().mi355_swiglu_quant_grouped(_ptr(x), 1 if activate_left else 0, _ptr(smooth), _ptr(group_index), group_index.numel(),
+                                                _ptr(y), _ptr(scale), rows, two // 2, x.stride(0), _stream()), "mi355_swiglu_quant_grouped")
+        return y, scale
     if smooth is not None:
         _check(lib().mi355_swiglu_quant_smooth(_ptr(x), 1 if activate_left else 0, _ptr(smooth), _ptr(y), _ptr(scale), rows,
                                                two // 2, x.stride(0), _stream()), "mi355_swiglu_quant_smooth")

@@ -395,10 +395,12 @@ void launch_swiglu_rows(const uint16_t *x, int8_t *y, float *scale, int64_t rows
 __global__ __launch_bounds__(kBlock) void swiglu_dq_generic_kernel(const uint16_t *__restrict__ x, int8_t *__restrict__ y,
                                                                   float *__restrict__ scale_out, int64_t half,
                                                                   int64_t row_stride, int64_t act_off, int64_t mul_off,
-                                                                  const uint16_t *__restrict__ smooth = nullptr)
+                                                                  const uint16_t *__restrict__ smooth = nullptr,
+                                                                  const int32_t *__restrict__ group_index = nullptr, int groups = 0)
 {
     const int64_t row = blockIdx.x;
     const uint16_t *xr = x + row * row_stride;
+    if (smooth) smooth = expert_scales(smooth, group_index, groups, row, half);
     auto value = [&](int64_t j) {
         const float sl = silu_bf16(bf16_1(xr[act_off + j]));
         const float v = bf16_1(f32_to_bf16(sl * bf16_1(xr[mul_off + j])));
@@ -425,9 +427,12 @@ __global__ __launch_bounds__(kBlock) void swiglu_dq_generic_kernel(const uint16_
 namespace mi355 {
 namespace {
 int run_swiglu_quant(const void *x_bf16, int activate_left, const void *smooth, int8_t *y, float *scale, int64_t rows,
-                     int64_t half, int64_t x_row_stride, void *stream)
+                     int64_t half, int64_t x_row_stride, void *stream, const int32_t *group_index = nullptr, int64_t groups = 0)
 {
     if (rows < 0 || half < 0) return MI355_ERR_BAD_ARGUMENT;
+    if (group_index && (!smooth || groups < 1 || groups > 0x7fffffff)) return MI355_ERR_BAD_ARGUMENT;
+    if (group_index && !aligned(group_index, 4)) return MI355_ERR_ALIGNMENT;
+    const int ng = group_index ? (int)groups : 0;
     if (rows == 0) return MI355_OK;
     if (!scale) return MI355_ERR_BAD_ARGUMENT;
     if (half > 0 && (!x_bf16 || !y || x_row_stride < 2 * half)) return MI355_ERR_BAD_ARGUMENT;
@@ -445,22 +450,22 @@ int run_swiglu_quant(const void *x_bf16, int activate_left, const void *smooth, 
             const int c = (int)half, ao = (int)(act >> 3), mo = (int)(mul >> 3);
             if (rows <= kFewRows && nvec > 1024 && nvec <= 1024 * 4)      // measured: no gain up to 8192 elements
                 hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 4, 1024>), dim3((unsigned)rows), dim3(1024), 0, s, xp, sm,
-                                   y, scale, c, x_row_stride, ao, mo);
+                                   y, scale, c, x_row_stride, ao, mo, group_index, ng);
             else if (nvec <= kBlock * 4)
                 hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 4>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y,
-                                   scale, c, x_row_stride, ao, mo);
+                                   scale, c, x_row_stride, ao, mo, group_index, ng);
             else if (nvec <= kBlock * 8)
                 hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 8>), dim3((unsigned)rows), dim3(kBlock), 0, s, xp, sm, y,
-                                   scale, c, x_row_stride, ao, mo);
+                                   scale, c, x_row_stride, ao, mo, group_index, ng);
             else if (nvec <= 1024 * 4)
                 hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 4, 1024>), dim3((unsigned)rows), dim3(1024), 0, s, xp, sm,
-                                   y, scale, c, x_row_stride, ao, mo);
+                                   y, scale, c, x_row_stride, ao, mo, group_index, ng);
             else
                 hipLaunchKernelGGL((dq_smooth_rows_kernel<false, true, 8, 1024>), dim3((unsigned)rows), dim3(1024), 0, s, xp, sm,
-                                   y, scale, c, x_row_stride, ao, mo);
+                                   y, scale, c, x_row_stride, ao, mo, group_index, ng);
         } else {
             hipLaunchKernelGGL(swiglu_dq_generic_kernel, dim3((unsigned)rows), dim3(kBlock), 0, s, xp, y, scale, half,
-                               x_row_stride, act, mul, sm);
+                               x_row_stride, act, mul, sm, group_index, ng);
         }
         return check_launch();
     }
@@ -497,6 +502,14 @@ extern "C" int mi355_swiglu_quant_smooth(const void *x_bf16, int activate_left, 
 {
     if (!smooth_bf16 && rows > 0 && half > 0) return MI355_ERR_BAD_ARGUMENT;
     return mi355::run_swiglu_quant(x_bf16, activate_left, smooth_bf16, y, scale, rows, half, x_row_stride, stream);
+}
+
+extern "C" int mi355_swiglu_quant_grouped(const void *x_bf16, int activate_left, const void *smooth_bf16, const int32_t *group_index,
+                                          int64_t groups, int8_t *y, float *scale, int64_t rows, int64_t half,
+                                          int64_t x_row_stride, void *stream)
+{
+    if ((!smooth_bf16 || !group_index) && rows > 0 && half > 0) return MI355_ERR_BAD_ARGUMENT;
+    return mi355::run_swiglu_quant(x_bf16, activate_left, smooth_bf16, y, scale, rows, half, x_row_stride, stream, group_index, groups);
 }
 
 extern "C" int mi355_dynamic_quant(const void *x, int in_dtype, const void *smooth, int8_t *y, float *scale,

@@ -724,7 +724,8 @@ Tensor swiglu_hip(const Tensor &input, int64_t dim)
 
 // The operator is only named in the reference tree (docs/zh/release_notes.md:303); the argument list follows the
 // vendor's published Python signature.  Implemented: dynamic per-token quantisation (quant_mode = 1) of the SwiGLU
-// of the last dimension, optionally with one set of smooth scales; no static offsets, no expert groups.
+// of the last dimension, optionally with smooth scales - one set, or one per expert with group_index (the running totals
+// of the rows of each expert, or with group_list_type = 1 their counts); no static offsets.
 void swiglu_quant_check(const Tensor &x, const optional<Tensor> &smooth_scales, const optional<Tensor> &offsets,
                         const optional<Tensor> &group_index, int64_t quant_mode, int64_t group_list_type,
                         optional<at::ScalarType> dst_type)
@@ -734,14 +735,24 @@ void swiglu_quant_check(const Tensor &x, const optional<Tensor> &smooth_scales, 
     if (const Tensor *sm = opt(smooth_scales)) {
         TORCH_CHECK(sm->scalar_type() == at::kBFloat16, "npu_swiglu_quant: smooth_scales must be bfloat16 like x, got ",
                     sm->scalar_type());
-        TORCH_CHECK(sm->dim() == 1 && sm->size(0) == x.size(-1) / 2, "npu_swiglu_quant: smooth_scales must have shape [",
-                    x.size(-1) / 2, "] (one per output column; per-expert scales are not supported)");
+        if (const Tensor *g = opt(group_index)) {
+            TORCH_CHECK(sm->dim() == 2 && sm->size(0) == g->numel() && sm->size(1) == x.size(-1) / 2,
+                        "npu_swiglu_quant: with group_index, smooth_scales must have shape [", g->numel(), ", ", x.size(-1) / 2,
+                        "], got ", sm->sizes());
+        } else {
+            TORCH_CHECK(sm->dim() == 1 && sm->size(0) == x.size(-1) / 2, "npu_swiglu_quant: smooth_scales must have shape [",
+                        x.size(-1) / 2, "] (one per output column), got ", sm->sizes());
+        }
     }
     TORCH_CHECK(!opt(offsets), "npu_swiglu_quant: offsets (static quantisation) is not supported");
-    TORCH_CHECK(!opt(group_index), "npu_swiglu_quant: group_index is not supported");
+    if (const Tensor *g = opt(group_index)) {
+        TORCH_CHECK(opt(smooth_scales), "npu_swiglu_quant: group_index needs smooth_scales of shape [experts, ", x.size(-1) / 2, "]");
+        TORCH_CHECK((g->scalar_type() == at::kInt || g->scalar_type() == at::kLong) && g->dim() == 1 && g->numel() >= 1,
+                    "npu_swiglu_quant: group_index must be an int32 or int64 vector [experts]");
+    }
     TORCH_CHECK(quant_mode == 1, "npu_swiglu_quant: only quant_mode=1 (dynamic per-token quantisation) is supported, got ",
                 quant_mode);
-    TORCH_CHECK(group_list_type == 0, "npu_swiglu_quant: group_list_type is not supported");
+    TORCH_CHECK(group_list_type == 0 || group_list_type == 1, "npu_swiglu_quant: group_list_type must be 0 (running totals) or 1 (counts)");
     TORCH_CHECK(!dst_type.has_value() || *dst_type == at::kChar, "npu_swiglu_quant: only dst_type=torch.int8 is supported");
 }
 
@@ -770,7 +781,7 @@ std::tuple<Tensor, Tensor> swiglu_quant_hip(const Tensor &x, const optional<Tens
                                             optional<at::ScalarType> dst_type)
 {
     swiglu_quant_check(x, smooth_scales, offsets, group_index, quant_mode, group_list_type, dst_type);
-    check_same_device("npu_swiglu_quant", {&x, opt(smooth_scales)});
+    check_same_device("npu_swiglu_quant", {&x, opt(smooth_scales), opt(group_index)});
     c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
     auto [y, scale] = swiglu_quant_alloc(x);
     const int64_t half = x.size(-1) / 2;
@@ -785,6 +796,15 @@ std::tuple<Tensor, Tensor> swiglu_quant_hip(const Tensor &x, const optional<Tens
         row_stride = xin.stride(0);
     } else if (!xin.is_contiguous()) {
         xin = xin.contiguous();
+    }
+    if (const Tensor *g = opt(group_index)) {
+        Tensor sm = opt(smooth_scales)->contiguous();
+        Tensor gi = (group_list_type == 1 ? g->cumsum(0) : *g).to(at::kInt).contiguous();     // counts -> running totals
+        check_status(mi355_swiglu_quant_grouped(xin.data_ptr(), activate_left ? 1 : 0, sm.data_ptr(), gi.data_ptr<int32_t>(),
+                                                gi.numel(), y.data_ptr<int8_t>(), scale.data_ptr<float>(), rows, half, row_stride,
+                                                stream_of(x)),
+                     "npu_swiglu_quant");
+        return {y, scale};
     }
     if (const Tensor *smp = opt(smooth_scales)) {
         Tensor sm = smp->contiguous();

@@ -188,6 +188,18 @@ def test_dynamic_quant_asymmetric_per_expert_smooth_scales(capi, golden, rows, c
     assert np.array_equal(y.cpu().numpy(), yg)
 
 
+@pytest.mark.parametrize("rows,half,totals", [(48, 2048, [10, 10, 30, 48]), (20, 8200, [4, 20]), (9, 500, [2, 5, 9])])
+def test_swiglu_quant_per_expert_smooth_scales(capi, golden, rows, half, totals):
+    """group_index of npu_swiglu_quant: the SwiGLU of a row is multiplied by its expert's smooth scales before the row is
+    quantised; bit-exact against dynamic_quant_grouped(swiglu(x)) of the oracle (vector and scalar kernels)."""
+    g = torch.Generator().manual_seed(rows + half)
+    x = (torch.randn(rows, 2 * half, generator=g) * 2).to(torch.bfloat16)
+    sm = (torch.rand(len(totals), half, generator=g) * 4 + 0.01).to(torch.bfloat16)
+    y, s = capi.swiglu_quant(x.cuda(), True, sm.cuda(), torch.tensor(totals, dtype=torch.int32).cuda())
+    yg, sg = golden.dynamic_quant_grouped(golden.swiglu(_bits(x)), _bits(sm), totals)
+    assert np.array_equal(s.cpu().numpy(), sg) and np.array_equal(y.cpu().numpy(), yg)
+
+
 # ------------------------------------------------------------------ quant_matmul
 
 QMM_SHAPES = [(1024, 4096, 1024), (256, 512, 352), (64, 4096, 512), (100, 256, 200), (1, 128, 16), (300, 1024, 1000),

@@ -822,3 +822,17 @@ def test_npu_dynamic_quant_int4_operator(pa, golden):
     assert np.array_equal(y.cpu().numpy(), yg) and np.array_equal(s.cpu().numpy(), sg)
     codes = torch.from_numpy(golden.unpack_int4(yg)).float()
     assert float(((codes * torch.from_numpy(sg)[..., None]) - x.float()).abs().max()) <= 0.5 * float(sg.max()) * 1.001
+
+
+@pytest.mark.gpu
+def test_npu_swiglu_quant_group_index_operator(pa, golden):
+    """torch.ops.npu.npu_swiglu_quant with per-expert smooth scales, group_index as running totals (group_list_type 0) and
+    as counts (1)."""
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(40, 2048, generator=g) * 2).to(torch.bfloat16)
+    sm = (torch.rand(3, 1024, generator=g) + 0.5).to(torch.bfloat16)
+    yg, sg = golden.dynamic_quant_grouped(golden.swiglu(golden.bits_of(x)), golden.bits_of(sm), [8, 30, 40])
+    for gi, kind in ((torch.tensor([8, 30, 40]), 0), (torch.tensor([8, 22, 10]), 1)):
+        y, s = pa.npu_swiglu_quant(x.cuda(), smooth_scales=sm.cuda(), group_index=gi.cuda(), activate_left=True, quant_mode=1,
+                                   group_list_type=kind)
+        assert np.array_equal(y.cpu().numpy(), yg) and np.array_equal(s.cpu().numpy(), sg)

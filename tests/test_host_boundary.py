@@ -222,8 +222,15 @@ def test_meta_swiglu_quant(pa):
         pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16))                      # static quantisation is not built
     y, s = pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(4, dtype=torch.bfloat16), quant_mode=1)
     assert y.shape == (4, 4) and s.shape == (4,)
-    with pytest.raises(RuntimeError, match="smooth_scales must have shape"):       # per-expert scales are not built
+    with pytest.raises(RuntimeError, match="smooth_scales must have shape"):       # per-expert scales need group_index
         pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(2, 4, dtype=torch.bfloat16), quant_mode=1)
+    y, s = pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(2, 4, dtype=torch.bfloat16),
+                               group_index=_m(2, dtype=torch.int64), quant_mode=1, group_list_type=1)
+    assert y.shape == (4, 4) and s.shape == (4,)
+    with pytest.raises(RuntimeError, match="group_index needs smooth_scales"):
+        pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), group_index=_m(2, dtype=torch.int64), quant_mode=1)
+    with pytest.raises(RuntimeError, match="group_list_type"):
+        pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), quant_mode=1, group_list_type=2)
     with pytest.raises(RuntimeError, match="smooth_scales must be bfloat16"):
         pa.npu_swiglu_quant(_m(4, 8, dtype=torch.bfloat16), smooth_scales=_m(4, dtype=torch.float32), quant_mode=1)
 
