@@ -336,7 +336,8 @@ __device__ __forceinline__ void k_loop(i32x4v (&acc)[4][WTN], char *lds, const L
 
 
 // ---------------------------------------------------------------------------------------------------------------
-// Epilogue for the common case: per-token scale, one float32 scale per column, optional bf16 bias, bf16 / fp16 output
+// Epilogue for the common cases: per-token scales or none, one float32 scale per column or one for all, optional bf16 bias,
+// bf16 / fp16 output
 // with 16-byte aligned rows.  The three parameter vectors of the tile were requested into LDS (PARAM_BASE) before the
 // first K step, so nothing here waits for global memory.  Per block of 16 rows a wavefront converts its WTN accumulator
 // tiles, stages them in its own LDS rows and stores whole rows of the wavefront tile (16 bytes per lane) right away, so
@@ -356,13 +357,24 @@ constexpr int PARAM_PS = 0, PARAM_SCALE = 1024, PARAM_BIAS = 2048;
 
 // issued by one wavefront in front of its first stage requests (loads retire in order, so they have landed when
 // stage 0 has); rows / columns past the matrix read as zero
-__device__ __forceinline__ void request_params(char *lds, int param_base, const float *pertoken, const float *scale, const void *bias,
-                                                int m0, int n0, int rows, int cols, int lane)
+// (no per-token scales: the vector is filled with 1.0f, by which the epilogue's multiplication changes nothing; a single
+// scale for all columns is spread over the vector)
+__device__ __forceinline__ void request_params(char *lds, int param_base, const float *pertoken, const float *scale, bool one_scale,
+                                                const void *bias, int m0, int n0, int rows, int cols, int lane)
 {
-    const __amdgpu_buffer_rsrc_t r_ps = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(pertoken + m0), 0, rows * 4, 0x00020000);
-    const __amdgpu_buffer_rsrc_t r_sc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(scale + n0), 0, cols * 4, 0x00020000);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(r_ps, (lds_void *)(lds + param_base + PARAM_PS), 16, (uint32_t)lane * 16u, 0, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(r_sc, (lds_void *)(lds + param_base + PARAM_SCALE), 16, (uint32_t)lane * 16u, 0, 0, 0);
+    if (pertoken) {
+        const __amdgpu_buffer_rsrc_t r_ps = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(pertoken + m0), 0, rows * 4, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r_ps, (lds_void *)(lds + param_base + PARAM_PS), 16, (uint32_t)lane * 16u, 0, 0, 0);
+    } else {
+        *reinterpret_cast<f32x4 *>(lds + param_base + PARAM_PS + lane * 16) = f32x4{1.0f, 1.0f, 1.0f, 1.0f};
+    }
+    if (!one_scale) {
+        const __amdgpu_buffer_rsrc_t r_sc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(scale + n0), 0, cols * 4, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r_sc, (lds_void *)(lds + param_base + PARAM_SCALE), 16, (uint32_t)lane * 16u, 0, 0, 0);
+    } else {
+        const float s1 = scale[0];
+        *reinterpret_cast<f32x4 *>(lds + param_base + PARAM_SCALE + lane * 16) = f32x4{s1, s1, s1, s1};
+    }
     if (bias) {
         const __amdgpu_buffer_rsrc_t r_b =
             __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(static_cast<const uint16_t *>(bias) + n0), 0, cols * 2, 0x00020000);
