@@ -193,7 +193,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 
     // the wide loop's epilogue for the common case takes its parameters from LDS (quant_matmul_wide.h)
     const bool fast_epilogue = WIDE && !p.out_i32 && !p.out_i8 && !p.qparam && (p.scale_len == p.N || p.scale_len == 1) &&
-                               (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_BF16) && (p.ldc & 7) == 0 &&
+                               (p.ldc & 7) == 0 &&
                                aligned_dev(p.out, 16) && (!p.pertoken || aligned_dev(p.pertoken, 16)) &&
                                (p.scale_len == 1 || aligned_dev(p.scale, 16)) && (!p.bias || aligned_dev(p.bias, 16));
     // ... and so does the one for the re-quantised int8 output with per-channel parameter words
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         using G = wide::Geometry<WTN>;
         if (threadIdx.x < 16) reinterpret_cast<uint32_t *>(lds + G::FLAG_BASE)[threadIdx.x] = 0u;
         if (fast_epilogue && wave == 0)
-            wide::request_params(lds, G::PARAM_BASE, p.pertoken, p.scale, p.scale_len == 1, p.bias_kind == MI355_BIAS_BF16 ? p.bias : nullptr,
+            wide::request_params(lds, G::PARAM_BASE, p.pertoken, p.scale, p.scale_len == 1, p.bias, p.bias_kind == MI355_BIAS_BF16 ? 2 : 4,
                                  m0, n0, rows_a, rows_b, lane);
         if (fast_epilogue_i8 && wave == 0)
             wide::request_params_i8(lds, G::PARAM_BASE, p.qparam, p.bias_kind == MI355_BIAS_INT32 ? p.bias : nullptr, n0, rows_b, lane);
@@ -527,7 +527,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             e.N = p.N;
             e.m0 = m0;
             e.n0 = n0;
-            e.has_bias = p.bias_kind == MI355_BIAS_BF16;
+            e.has_bias = p.bias ? p.bias_kind : MI355_BIAS_NONE;
             e.out_f16 = p.out_f16;
             e.stream_out = p.stream_out;
             e.wm = wm;

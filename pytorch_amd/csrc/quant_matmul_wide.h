@@ -348,7 +348,7 @@ struct EpilogueArgs {
     int64_t ldc;
     int M, N;
     int m0, n0;                        // first row / column of the workgroup tile
-    int has_bias, out_f16;
+    int has_bias, out_f16;             // has_bias: the MI355_BIAS_* code of the 16-bit epilogue, 0 / 1 for the int8 one
     int stream_out;                    // store the rows with non-temporal stores (see the launcher's choice)
     int wm, wn;                        // position of the wavefront's 64 x 16 * WTN share in the workgroup tile
 };
@@ -360,7 +360,7 @@ constexpr int PARAM_PS = 0, PARAM_SCALE = 1024, PARAM_BIAS = 2048;
 // (no per-token scales: the vector is filled with 1.0f, by which the epilogue's multiplication changes nothing; a single
 // scale for all columns is spread over the vector)
 __device__ __forceinline__ void request_params(char *lds, int param_base, const float *pertoken, const float *scale, bool one_scale,
-                                                const void *bias, int m0, int n0, int rows, int cols, int lane)
+                                                const void *bias, int bias_size, int m0, int n0, int rows, int cols, int lane)
 {
     if (pertoken) {
         const __amdgpu_buffer_rsrc_t r_ps = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(pertoken + m0), 0, rows * 4, 0x00020000);
@@ -375,14 +375,15 @@ __device__ __forceinline__ void request_params(char *lds, int param_base, const 
         const float s1 = scale[0];
         *reinterpret_cast<f32x4 *>(lds + param_base + PARAM_SCALE + lane * 16) = f32x4{s1, s1, s1, s1};
     }
-    if (bias) {
-        const __amdgpu_buffer_rsrc_t r_b =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(static_cast<const uint16_t *>(bias) + n0), 0, cols * 2, 0x00020000);
+    if (bias) {                                               // bias_size bytes per column: bf16, or int32 / float32
+        const __amdgpu_buffer_rsrc_t r_b = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char *>(static_cast<const char *>(bias) + (size_t)n0 * bias_size), 0, cols * bias_size, 0x00020000);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(r_b, (lds_void *)(lds + param_base + PARAM_BIAS), 16, (uint32_t)lane * 16u, 0, 0, 0);
     }
 }
 
-template <int WTN, bool F16, bool BIAS, bool NT>
+// BIAS: 0 none, 1 bf16 (added last), 2 int32 (added to the accumulator, wrapping like it), 3 float32 (added last)
+template <int WTN, bool F16, int BIAS, bool NT>
 __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
 {
     using G = Geometry<WTN>;
@@ -399,9 +400,11 @@ __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, 
     for (int j = 0; j < WTN; j++) {
         const int c = wn * WTN * 16 + j * 16 + nquad;
         sc[j] = *reinterpret_cast<const f32x4 *>(par + PARAM_SCALE + c * 4);
-        if constexpr (BIAS) {
+        if constexpr (BIAS == 1) {
             const u32x2 b2 = *reinterpret_cast<const u32x2 *>(par + PARAM_BIAS + c * 2);
             bs[j] = f32x4{bf16_lo(b2.x), bf16_hi(b2.x), bf16_lo(b2.y), bf16_hi(b2.y)};
+        } else if constexpr (BIAS >= 2) {
+            bs[j] = *reinterpret_cast<const f32x4 *>(par + PARAM_BIAS + c * 4);       // int32: its bit patterns
         }
     }
     char *stg = lds + wave * (16 * ROWB);
@@ -413,10 +416,10 @@ __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, 
             float f[4];
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                float v = (float)acc[i][j][r];
+                float v = BIAS == 2 ? (float)(int32_t)((uint32_t)acc[i][j][r] + __float_as_uint(bs[j][r])) : (float)acc[i][j][r];
                 v = v * ps[i];
                 v = v * sc[j][r];
-                if constexpr (BIAS) v = v + bs[j][r];
+                if constexpr (BIAS == 1 || BIAS == 3) v = v + bs[j][r];
                 f[r] = v;
             }
             u32x2 pk;
@@ -447,20 +450,23 @@ __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, 
 template <int WTN>
 __device__ __forceinline__ void epilogue_fast(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
 {
-    // output type, bias presence and the kind of store are resolved once per wavefront
+    // output type, kind of bias and kind of store are resolved once per wavefront
     auto go = [&](auto f16, auto bias) {
         if (e.stream_out) epilogue_rows<WTN, decltype(f16)::value, decltype(bias)::value, true>(acc, lds, e, wave, lane);
         else epilogue_rows<WTN, decltype(f16)::value, decltype(bias)::value, false>(acc, lds, e, wave, lane);
     };
     using T = std::true_type;
     using F = std::false_type;
-    if (e.out_f16) {
-        if (e.has_bias) go(T{}, T{});
-        else go(T{}, F{});
-    } else {
-        if (e.has_bias) go(F{}, T{});
-        else go(F{}, F{});
-    }
+    auto by_bias = [&](auto f16) {
+        switch (e.has_bias) {                 // the MI355_BIAS_* code
+        case 1: go(f16, std::integral_constant<int, 1>{}); break;
+        case 2: go(f16, std::integral_constant<int, 2>{}); break;
+        case 3: go(f16, std::integral_constant<int, 3>{}); break;
+        default: go(f16, std::integral_constant<int, 0>{}); break;
+        }
+    };
+    if (e.out_f16) by_bias(T{});
+    else by_bias(F{});
 }
 
 // ---- the same for the re-quantised int8 output: clamp(rint(float(acc + int32 bias) * scale + offset)), scale and the
