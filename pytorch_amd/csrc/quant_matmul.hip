@@ -196,6 +196,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
                                (p.ldc & 7) == 0 &&
                                aligned_dev(p.out, 16) && (!p.pertoken || aligned_dev(p.pertoken, 16)) &&
                                (p.scale_len == 1 || aligned_dev(p.scale, 16)) && (!p.bias || aligned_dev(p.bias, 16));
+    // ... the same with the column scales taken from packed 64-bit parameter words (no per-token scales then)
+    const bool fast_epilogue_qp = WIDE && !p.out_i32 && !p.out_i8 && p.qparam && !p.pertoken && p.scale_len == p.N && (p.ldc & 7) == 0 &&
+                                  aligned_dev(p.out, 16) && aligned_dev(p.qparam, 16) && (!p.bias || aligned_dev(p.bias, 16));
     // ... and so does the one for the re-quantised int8 output with per-channel parameter words
     const bool fast_epilogue_i8 = WIDE && p.out_i8 && p.qparam && p.scale_len == p.N &&
                                   (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_INT32) && (p.ldc & 15) == 0 &&
@@ -208,6 +211,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         if (fast_epilogue && wave == 0)
             wide::request_params(lds, G::PARAM_BASE, p.pertoken, p.scale, p.scale_len == 1, p.bias, p.bias_kind == MI355_BIAS_BF16 ? 2 : 4,
                                  m0, n0, rows_a, rows_b, lane);
+        if (fast_epilogue_qp && wave == 0)
+            wide::request_params_i8(lds, G::PARAM_BASE, p.qparam, p.bias, n0, rows_b, lane, p.bias_kind == MI355_BIAS_BF16 ? 2 : 4);
         if (fast_epilogue_i8 && wave == 0)
             wide::request_params_i8(lds, G::PARAM_BASE, p.qparam, p.bias_kind == MI355_BIAS_INT32 ? p.bias : nullptr, n0, rows_b, lane);
         const int frow = lane & 15;
@@ -519,8 +524,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             wide::epilogue_fast_i8<WTN>(acc, lds, e, wave, lane);
             return;
         }
-        if (fast_epilogue) {
+        if (fast_epilogue || fast_epilogue_qp) {
             wide::EpilogueArgs e;
+            e.packed_scale = fast_epilogue_qp;
             e.out = p.out;
             e.ldc = p.ldc;
             e.M = p.M;

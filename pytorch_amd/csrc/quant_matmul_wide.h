@@ -351,6 +351,7 @@ struct EpilogueArgs {
     int has_bias, out_f16;             // has_bias: the MI355_BIAS_* code of the 16-bit epilogue, 0 / 1 for the int8 one
     int stream_out;                    // store the rows with non-temporal stores (see the launcher's choice)
     int wm, wn;                        // position of the wavefront's 64 x 16 * WTN share in the workgroup tile
+    int packed_scale;                  // 16-bit output: the column scales come from the packed 64-bit parameter words
 };
 
 constexpr int PARAM_PS = 0, PARAM_SCALE = 1024, PARAM_BIAS = 2048;
@@ -383,7 +384,9 @@ __device__ __forceinline__ void request_params(char *lds, int param_base, const 
 }
 
 // BIAS: 0 none, 1 bf16 (added last), 2 int32 (added to the accumulator, wrapping like it), 3 float32 (added last)
-template <int WTN, bool F16, int BIAS, bool NT>
+// QP: the column scales are the low words of the packed 64-bit parameters (request_params_i8's layout) and there are no
+// per-token scales
+template <int WTN, bool F16, int BIAS, bool NT, bool QP = false>
 __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
 {
     using G = Geometry<WTN>;
@@ -394,12 +397,18 @@ __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, 
     const char *par = lds + G::PARAM_BASE;
     float ps[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) ps[i] = *reinterpret_cast<const float *>(par + PARAM_PS + (wm * 64 + i * 16 + mrow) * 4);
+    for (int i = 0; i < 4; i++) ps[i] = QP ? 1.0f : *reinterpret_cast<const float *>(par + PARAM_PS + (wm * 64 + i * 16 + mrow) * 4);
     f32x4 sc[WTN], bs[WTN];
 #pragma unroll
     for (int j = 0; j < WTN; j++) {
         const int c = wn * WTN * 16 + j * 16 + nquad;
-        sc[j] = *reinterpret_cast<const f32x4 *>(par + PARAM_SCALE + c * 4);
+        if constexpr (QP) {
+            const u32x4 q01 = *reinterpret_cast<const u32x4 *>(par + c * 8);       // low, high words of columns c, c + 1
+            const u32x4 q23 = *reinterpret_cast<const u32x4 *>(par + c * 8 + 16);
+            sc[j] = f32x4{__uint_as_float(q01.x), __uint_as_float(q01.z), __uint_as_float(q23.x), __uint_as_float(q23.z)};
+        } else {
+            sc[j] = *reinterpret_cast<const f32x4 *>(par + PARAM_SCALE + c * 4);
+        }
         if constexpr (BIAS == 1) {
             const u32x2 b2 = *reinterpret_cast<const u32x2 *>(par + PARAM_BIAS + c * 2);
             bs[j] = f32x4{bf16_lo(b2.x), bf16_hi(b2.x), bf16_lo(b2.y), bf16_hi(b2.y)};
@@ -452,8 +461,15 @@ __device__ __forceinline__ void epilogue_fast(i32x4v (&acc)[4][WTN], char *lds, 
 {
     // output type, kind of bias and kind of store are resolved once per wavefront
     auto go = [&](auto f16, auto bias) {
-        if (e.stream_out) epilogue_rows<WTN, decltype(f16)::value, decltype(bias)::value, true>(acc, lds, e, wave, lane);
-        else epilogue_rows<WTN, decltype(f16)::value, decltype(bias)::value, false>(acc, lds, e, wave, lane);
+        constexpr bool H = decltype(f16)::value;
+        constexpr int B = decltype(bias)::value;
+        if (e.packed_scale) {
+            if (e.stream_out) epilogue_rows<WTN, H, B, true, true>(acc, lds, e, wave, lane);
+            else epilogue_rows<WTN, H, B, false, true>(acc, lds, e, wave, lane);
+        } else {
+            if (e.stream_out) epilogue_rows<WTN, H, B, true>(acc, lds, e, wave, lane);
+            else epilogue_rows<WTN, H, B, false>(acc, lds, e, wave, lane);
+        }
     };
     using T = std::true_type;
     using F = std::false_type;
@@ -475,15 +491,15 @@ __device__ __forceinline__ void epilogue_fast(i32x4v (&acc)[4][WTN], char *lds, 
 // stages its whole tile (a lane owns one 32-bit word of four columns per 16x16 tile) and stores 16 bytes per lane.
 constexpr int PARAM_QP = 0, PARAM_BIAS32 = 2048;
 
-__device__ __forceinline__ void request_params_i8(char *lds, int param_base, const uint64_t *qparam, const void *bias_i32, int n0,
-                                                   int cols, int lane)
+__device__ __forceinline__ void request_params_i8(char *lds, int param_base, const uint64_t *qparam, const void *bias, int n0,
+                                                   int cols, int lane, int bias_size = 4)
 {
     const __amdgpu_buffer_rsrc_t r_q = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint64_t *>(qparam + n0), 0, cols * 8, 0x00020000);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r_q, (lds_void *)(lds + param_base + PARAM_QP), 16, (uint32_t)lane * 16u, 0, 0, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r_q, (lds_void *)(lds + param_base + PARAM_QP + 1024), 16, (uint32_t)lane * 16u, 1024, 0, 0);
-    if (bias_i32) {
+    if (bias) {                                               // int32 for the int8 output; any kind for the 16-bit ones
         const __amdgpu_buffer_rsrc_t r_b = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<int32_t *>(static_cast<const int32_t *>(bias_i32) + n0), 0, cols * 4, 0x00020000);
+            const_cast<char *>(static_cast<const char *>(bias) + (size_t)n0 * bias_size), 0, cols * bias_size, 0x00020000);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(r_b, (lds_void *)(lds + param_base + PARAM_BIAS32), 16, (uint32_t)lane * 16u, 0, 0, 0);
     }
 }

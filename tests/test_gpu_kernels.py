@@ -419,7 +419,9 @@ def test_quant_matmul_wide_loop_tiles(capi, golden, tile, M, K, N):
                 capi.quant_matmul(x1, x2, None, None, bias_i32, out_dtype=torch.int32),
                 capi.quant_matmul_qparam(x1, x2, qp, bias_i32),
                 capi.quant_matmul_qparam(x1, x2, qp, None, out_dtype=torch.bfloat16),
-                capi.quant_matmul_qparam(x1, x2, qp, None)]
+                capi.quant_matmul_qparam(x1, x2, qp, None),
+                capi.quant_matmul_qparam(x1, x2, qp, bias_i32, out_dtype=torch.float16),
+                capi.quant_matmul(x1, x2, one, None, bias_f32)]
 
     capi.set_tuning("MI355_QMM_TILE", tile)
     try:
