@@ -119,6 +119,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     constexpr int A_BYTES = UNITS_A * 1024, B_BYTES = UNITS_BP * 1024;
     constexpr bool WIDE = LOOP == 1 || LOOP == 2;
     constexpr bool WHOLE = NS >= 4 || LOOP == 3;             // whole stages: activations get NS slots as well
+    // the epilogues that take their parameters from LDS (quant_matmul_wide.h: wavefronts of 64 rows): the wide loop's tiles
+    // and the whole-stage 128-row tiles, which keep the vectors behind their ring
+    constexpr bool LDSP = WIDE || (LOOP == 3 && WTM == 4);
     constexpr int NSA = WHOLE ? NS : 2;                      // activation slots; NS weight slots follow them in LDS
     constexpr uint32_t kOutOfRange = 0x80000000u;            // lane offset beyond every buffer: the load writes zeros
     static_assert(UNITS_A % NW == 0, "A units must divide evenly over the wavefronts");
@@ -192,29 +195,33 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         for (int j = 0; j < WTN; j++) acc[i][j] = i32x4v{0, 0, 0, 0};
 
     // the wide loop's epilogue for the common case takes its parameters from LDS (quant_matmul_wide.h)
-    const bool fast_epilogue = WIDE && !p.out_i32 && !p.out_i8 && !p.qparam && (p.scale_len == p.N || p.scale_len == 1) &&
+    const bool fast_epilogue = LDSP && !p.out_i32 && !p.out_i8 && !p.qparam && (p.scale_len == p.N || p.scale_len == 1) &&
                                (p.ldc & 7) == 0 &&
                                aligned_dev(p.out, 16) && (!p.pertoken || aligned_dev(p.pertoken, 16)) &&
                                (p.scale_len == 1 || aligned_dev(p.scale, 16)) && (!p.bias || aligned_dev(p.bias, 16));
     // ... the same with the column scales taken from packed 64-bit parameter words (no per-token scales then)
-    const bool fast_epilogue_qp = WIDE && !p.out_i32 && !p.out_i8 && p.qparam && !p.pertoken && p.scale_len == p.N && (p.ldc & 7) == 0 &&
+    const bool fast_epilogue_qp = LDSP && !p.out_i32 && !p.out_i8 && p.qparam && !p.pertoken && p.scale_len == p.N && (p.ldc & 7) == 0 &&
                                   aligned_dev(p.out, 16) && aligned_dev(p.qparam, 16) && (!p.bias || aligned_dev(p.bias, 16));
     // ... and so does the one for the re-quantised int8 output with per-channel parameter words
-    const bool fast_epilogue_i8 = WIDE && p.out_i8 && p.qparam && p.scale_len == p.N &&
+    const bool fast_epilogue_i8 = LDSP && p.out_i8 && p.qparam && p.scale_len == p.N &&
                                   (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_INT32) && (p.ldc & 15) == 0 &&
                                   aligned_dev(p.out, 16) && aligned_dev(p.qparam, 16) && (!p.bias || aligned_dev(p.bias, 16));
 
+    // requested by one wavefront in front of its first stage (loads retire in order: they have landed when stage 0 has)
+    constexpr int PARAM_BASE = WIDE ? wide::Geometry<WTN>::PARAM_BASE : NSA * A_BYTES + (NS > 0 ? NS : 1) * B_BYTES;
+    if constexpr (LDSP) {
+        if (fast_epilogue && wave == 0)
+            wide::request_params(lds, PARAM_BASE, p.pertoken, p.scale, p.scale_len == 1, p.bias, p.bias_kind == MI355_BIAS_BF16 ? 2 : 4,
+                                 m0, n0, rows_a, rows_b, lane);
+        if (fast_epilogue_qp && wave == 0)
+            wide::request_params_i8(lds, PARAM_BASE, p.qparam, p.bias, n0, rows_b, lane, p.bias_kind == MI355_BIAS_BF16 ? 2 : 4);
+        if (fast_epilogue_i8 && wave == 0)
+            wide::request_params_i8(lds, PARAM_BASE, p.qparam, p.bias_kind == MI355_BIAS_INT32 ? p.bias : nullptr, n0, rows_b, lane);
+    }
     if constexpr (WIDE) {
         static_assert(WGM == 4 && WGN == 2 && WTM == 4 && NS == 3, "wide loop: 4 x 2 wavefronts of 64 rows");
         using G = wide::Geometry<WTN>;
         if (threadIdx.x < 16) reinterpret_cast<uint32_t *>(lds + G::FLAG_BASE)[threadIdx.x] = 0u;
-        if (fast_epilogue && wave == 0)
-            wide::request_params(lds, G::PARAM_BASE, p.pertoken, p.scale, p.scale_len == 1, p.bias, p.bias_kind == MI355_BIAS_BF16 ? 2 : 4,
-                                 m0, n0, rows_a, rows_b, lane);
-        if (fast_epilogue_qp && wave == 0)
-            wide::request_params_i8(lds, G::PARAM_BASE, p.qparam, p.bias, n0, rows_b, lane, p.bias_kind == MI355_BIAS_BF16 ? 2 : 4);
-        if (fast_epilogue_i8 && wave == 0)
-            wide::request_params_i8(lds, G::PARAM_BASE, p.qparam, p.bias_kind == MI355_BIAS_INT32 ? p.bias : nullptr, n0, rows_b, lane);
         const int frow = lane & 15;
         const uint32_t sw0 = (uint32_t)(((lane >> 4) ^ ((frow >> 1) & 7)) * 16);
         wide::LoopState st;
@@ -507,9 +514,10 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         if (threadIdx.x == 0) __hip_atomic_store(p.counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
-    if constexpr (WIDE) {
+    if constexpr (LDSP) {
         if (fast_epilogue_i8) {
             wide::EpilogueArgs e;
+            e.param_base = PARAM_BASE;
             e.out = p.out;
             e.ldc = p.ldc;
             e.M = p.M;
@@ -526,6 +534,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         }
         if (fast_epilogue || fast_epilogue_qp) {
             wide::EpilogueArgs e;
+            e.param_base = PARAM_BASE;
             e.packed_scale = fast_epilogue_qp;
             e.out = p.out;
             e.ldc = p.ldc;
@@ -929,7 +938,7 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     constexpr int NS = DEEP < 0 ? 0 : DEEP ? DEEP : 2 * a_bytes + 2 * b_bytes <= 80 * 1024 && staging_bytes <= 80 * 1024 ? 2 : 3;
     // DEEP < 0: the streaming K loop (two activation chunks of 32 KiB and a 4 KiB turn-around tile per wavefront)
     constexpr size_t stage_bytes = DEEP < 0 ? (size_t)2 * 32768 + 8 * 4096 : (DEEP ? DEEP : 2) * a_bytes + NS * b_bytes;
-    constexpr size_t ring_bytes = LOOP == 1 || LOOP == 2 ? (size_t)wide::Geometry<WTN>::LDS_BYTES : stage_bytes;
+    constexpr size_t ring_bytes = LOOP == 1 || LOOP == 2 ? (size_t)wide::Geometry<WTN>::LDS_BYTES : stage_bytes + (LOOP == 3 ? 3072 : 0);
     constexpr size_t lds_bytes = ring_bytes > staging_bytes ? ring_bytes : staging_bytes;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
     p.tiles_m = (p.M + BM - 1) / BM;

@@ -352,6 +352,7 @@ struct EpilogueArgs {
     int stream_out;                    // store the rows with non-temporal stores (see the launcher's choice)
     int wm, wn;                        // position of the wavefront's 64 x 16 * WTN share in the workgroup tile
     int packed_scale;                  // 16-bit output: the column scales come from the packed 64-bit parameter words
+    int param_base;                    // LDS byte offset of the parameter vectors
 };
 
 constexpr int PARAM_PS = 0, PARAM_SCALE = 1024, PARAM_BIAS = 2048;
@@ -389,12 +390,11 @@ __device__ __forceinline__ void request_params(char *lds, int param_base, const 
 template <int WTN, bool F16, int BIAS, bool NT, bool QP = false>
 __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
 {
-    using G = Geometry<WTN>;
     constexpr int ROWB = WTN * 32 + 16;                       // padded pitch of a staged row: spreads rows over the banks
     constexpr int CHUNKS = WTN * 2;                           // 16-byte chunks per row of the wavefront tile
     const int wm = e.wm, wn = e.wn;
     const int mrow = lane & 15, nquad = (lane >> 4) * 4;
-    const char *par = lds + G::PARAM_BASE;
+    const char *par = lds + e.param_base;
     float ps[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) ps[i] = QP ? 1.0f : *reinterpret_cast<const float *>(par + PARAM_PS + (wm * 64 + i * 16 + mrow) * 4);
@@ -507,12 +507,11 @@ __device__ __forceinline__ void request_params_i8(char *lds, int param_base, con
 template <int WTN, bool BIAS, bool NT>
 __device__ __forceinline__ void epilogue_rows_i8(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
 {
-    using G = Geometry<WTN>;
     constexpr int ROWQ = WTN * 16 + 16;                       // padded pitch of a staged row of the wavefront tile
     constexpr int CHQ = WTN;                                  // 16-byte chunks per row
     const int wm = e.wm, wn = e.wn;
     const int mrow = lane & 15, nquad = (lane >> 4) * 4;
-    const char *par = lds + G::PARAM_BASE;
+    const char *par = lds + e.param_base;
     char *stq = lds + wave * (64 * ROWQ);
 #pragma unroll
     for (int j = 0; j < WTN; j++) {
