@@ -72,7 +72,7 @@ struct QmmArgs {
     int out_i32;
     const uint64_t *qparam;    // packed quantisation parameters [scale_len] (replace `scale`), or null
     int out_i8;                // re-quantised int8 output (needs qparam)
-    int stream_out;            // outputs with aligned rows: non-temporal row stores (chosen by the launcher)
+    int stream_out;            // 16-bit and int8 outputs with aligned rows: non-temporal row stores (chosen by the launcher)
     int tiles_m, tiles_n, tiles_per_xcd;
     int S;                     // workgroups that share the K range of a tile
     int32_t *partial;          // workspace [tile][chunk][wavefront][accumulator quad][lane] int32x4 (S > 1)
@@ -571,42 +571,6 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             }
         }
         const bool vec = (p.ldc & 3) == 0 && aligned_dev(p.out, 16);
-        if (vec) {
-            // Aligned rows: a block of 16 rows of the wavefront's tile goes through its own LDS region (the stage buffers are
-            // idle behind the last barrier) and leaves as 16-byte stores over whole tile rows, so that a store instruction
-            // covers runs of 64 * WTN bytes instead of 64.
-            constexpr int ROWI = WTN * 64 + 16;               // padded row pitch in bytes
-            constexpr int CHI = WTN * 4;                      // 16-byte chunks per row
-            char *sti = lds + wave * (16 * ROWI);
-            const int mw = m0 + wm * WTM * 16, nw = n0 + wn * WTN * 16;
-            auto rows = [&](auto nt_c) {
-                constexpr bool NT = decltype(nt_c)::value;
-#pragma unroll
-                for (int i = 0; i < WTM; i++) {
-#pragma unroll
-                    for (int j = 0; j < WTN; j++) *reinterpret_cast<i32x4v *>(sti + mrow * ROWI + (j * 16 + nquad) * 4) = acc[i][j];
-#pragma unroll
-                    for (int q0 = 0; q0 < 16 * CHI; q0 += 64) {
-                        const int q = q0 + lane;
-                        const int row = q / CHI, ch = q % CHI;
-                        const int m = mw + i * 16 + row, n = nw + ch * 4;
-                        if (m >= p.M || n >= p.N) continue;
-                        const i32x4v v = *reinterpret_cast<const i32x4v *>(sti + row * ROWI + ch * 16);
-                        int32_t *o = static_cast<int32_t *>(p.out) + (int64_t)m * p.ldc + n;
-                        if (n + 3 < p.N) {
-                            if constexpr (NT) __builtin_nontemporal_store(v, reinterpret_cast<i32x4v *>(o));
-                            else *reinterpret_cast<i32x4v *>(o) = v;
-                        } else {
-                            for (int r = 0; r < 4; r++)
-                                if (n + r < p.N) o[r] = v[r];
-                        }
-                    }
-                }
-            };
-            if (p.stream_out) rows(std::true_type{});
-            else rows(std::false_type{});
-            return;
-        }
 #pragma unroll
         for (int i = 0; i < WTM; i++) {
             const int m = m0 + (wm * WTM + i) * 16 + mrow;
@@ -615,8 +579,12 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
                 const int n = n0 + (wn * WTN + j) * 16 + nquad;
                 if (m >= p.M || n >= p.N) continue;
                 int32_t *o = static_cast<int32_t *>(p.out) + (int64_t)m * p.ldc + n;
-                for (int r = 0; r < 4; r++)
-                    if (n + r < p.N) o[r] = acc[i][j][r];
+                if (vec && n + 3 < p.N) {
+                    *reinterpret_cast<i32x4v *>(o) = acc[i][j];
+                } else {
+                    for (int r = 0; r < 4; r++)
+                        if (n + r < p.N) o[r] = acc[i][j][r];
+                }
             }
         }
         return;
@@ -1211,7 +1179,7 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     // ordinary stores.  MI355_QMM_STREAM_OUT: 1 never, 2 always.
     {
         const int so = knob(kKnobQmmStreamOut);
-        const uint64_t out_bytes = (uint64_t)M * (uint64_t)N * (out_i8 ? 1u : out_i32 ? 4u : 2u);
+        const uint64_t out_bytes = (uint64_t)M * (uint64_t)N * (out_i8 ? 1u : 2u);
         p.stream_out = so == 2 || (so != 1 && out_bytes <= kStreamOutMaxBytes);
     }
     const TileChoice c = pl.tile;
