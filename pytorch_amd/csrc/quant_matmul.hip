@@ -195,12 +195,15 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         for (int j = 0; j < WTN; j++) acc[i][j] = i32x4v{0, 0, 0, 0};
 
     // the wide loop's epilogue for the common case takes its parameters from LDS (quant_matmul_wide.h)
+    // (the widest wavefront tile keeps to the bias kinds of the common calls: every further variant of its epilogue costs the
+    // K loop registers it does not have - 2048x4096x28672 went from 203 to 219 us with all of them)
+    constexpr bool LEAN = WTN >= 7;
     const bool fast_epilogue = LDSP && !p.out_i32 && !p.out_i8 && !p.qparam && (p.scale_len == p.N || p.scale_len == 1) &&
-                               (p.ldc & 7) == 0 &&
+                               (!LEAN || p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_BF16) && (p.ldc & 7) == 0 &&
                                aligned_dev(p.out, 16) && (!p.pertoken || aligned_dev(p.pertoken, 16)) &&
                                (p.scale_len == 1 || aligned_dev(p.scale, 16)) && (!p.bias || aligned_dev(p.bias, 16));
     // ... the same with the column scales taken from packed 64-bit parameter words (no per-token scales then)
-    const bool fast_epilogue_qp = LDSP && !p.out_i32 && !p.out_i8 && p.qparam && !p.pertoken && p.scale_len == p.N && (p.ldc & 7) == 0 &&
+    const bool fast_epilogue_qp = LDSP && !LEAN && !p.out_i32 && !p.out_i8 && p.qparam && !p.pertoken && p.scale_len == p.N && (p.ldc & 7) == 0 &&
                                   aligned_dev(p.out, 16) && aligned_dev(p.qparam, 16) && (!p.bias || aligned_dev(p.bias, 16));
     // ... and so does the one for the re-quantised int8 output with per-channel parameter words
     const bool fast_epilogue_i8 = LDSP && p.out_i8 && p.qparam && p.scale_len == p.N &&

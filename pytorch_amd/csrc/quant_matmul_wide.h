@@ -463,7 +463,8 @@ __device__ __forceinline__ void epilogue_fast(i32x4v (&acc)[4][WTN], char *lds, 
     auto go = [&](auto f16, auto bias) {
         constexpr bool H = decltype(f16)::value;
         constexpr int B = decltype(bias)::value;
-        if (e.packed_scale) {
+        if constexpr (WTN >= 7 && B >= 2) return;           // not instantiated for the widest tile (the kernel never asks)
+        else if (WTN < 7 && e.packed_scale) {
             if (e.stream_out) epilogue_rows<WTN, H, B, true, true>(acc, lds, e, wave, lane);
             else epilogue_rows<WTN, H, B, false, true>(acc, lds, e, wave, lane);
         } else {
