@@ -412,11 +412,6 @@ QmmPlan quant_matmul_plan(const Tensor &x1, const Tensor &x2, const Tensor &scal
     }
     auto b1 = x1.sizes().slice(0, x1.dim() - 2), b2 = x2.sizes().slice(0, x2.dim() - 2);
     p.batch = at::infer_size(b1, b2);
-    if (opt(pertoken_scale)) {
-        int64_t nb = 1;
-        for (auto d : p.batch) nb *= d;
-        TORCH_CHECK(nb == 1 || x1.dim() == 2, "npu_quant_matmul: pertoken_scale with batched x1 is not supported");
-    }
     p.out_shape = p.batch;
     p.out_shape.push_back(p.M);
     p.out_shape.push_back(p.N);
@@ -498,6 +493,8 @@ Tensor quant_matmul_hip(const Tensor &x1, const Tensor &x2, const Tensor &scale,
     if (x2_single) {
         Tensor w2 = xb.dim() == 2 ? xb : xb.as_strided({p.K, p.N}, {xb.stride(-2), xb.stride(-1)});
         jobs.emplace_back(xa.reshape({-1, p.K}), w2);
+        // the [M] per-token scales apply to every matrix of the batch: one copy per matrix of the tall matmul
+        if (ps.defined() && p.M > 0 && jobs.back().first.size(0) != p.M) ps = ps.repeat({jobs.back().first.size(0) / p.M});
     } else {
         auto x1s = p.batch, x2s = p.batch;
         x1s.push_back(p.M), x1s.push_back(p.K), x2s.push_back(p.K), x2s.push_back(p.N);
@@ -552,7 +549,9 @@ WqPlan weight_quant_plan(const Tensor &x, const Tensor &weight, const Tensor &an
                 ": weight must be int8, or int32 holding 8 int4 values per word, got ", weight.scalar_type());
     TORCH_CHECK(x.dim() >= 2 && weight.dim() == 2, op, ": x must be [..., K] with at least 2 dimensions and weight 2-D");
     TORCH_CHECK(opt(quant_scale) || !opt(quant_offset), op, ": quant_offset needs quant_scale");
-    TORCH_CHECK(inner_precise == 0, op, ": inner_precise must be 0");
+    // inner_precise: 0 = high precision, 1 = the vendor's faster, less precise accumulation.  Every kernel here accumulates in
+    // float32, so both values give the high-precision result.
+    TORCH_CHECK(inner_precise == 0 || inner_precise == 1, op, ": inner_precise must be 0 or 1, got ", inner_precise);
     TORCH_CHECK(!weight_dtype.has_value(), op, ": weight_dtype is not supported");
     WqPlan p;
     p.bits = weight.scalar_type() == at::kInt ? 4 : 8;

@@ -73,6 +73,10 @@ def test_c4_w4a16_full_size(pa, golden, M):
     _, gold = golden.weight_quant_matmul(_bits(d["x"]), d["weight"].numpy(), _bits(d["antiquant_scale"]),
                                          _bits(d["antiquant_offset"]), group_size=128)
     print("C4", M, bf16_gate(out, torch.from_numpy(gold)))
+    # inner_precise=1 (the vendor's faster accumulation mode) is accepted and gives the high-precision result
+    fast = pa.npu_weight_quant_batchmatmul(d["x"].cuda(), d["weight"].cuda(), d["antiquant_scale"].cuda(),
+                                           d["antiquant_offset"].cuda(), None, None, None, 128, 1)
+    assert torch.equal(fast, out)
 
 
 def test_quant_matmul_batched_and_scale_variants(pa, golden):
@@ -86,6 +90,20 @@ def test_quant_matmul_batched_and_scale_variants(pa, golden):
         for b1 in range(3):
             want, _ = golden.quant_matmul(x1[b0, b1].numpy(), x2[b1].numpy(), s.numpy())
             assert np.array_equal(_bits(out[b0, b1]), want)
+    # per-token scales [M] with batches: they apply to every matrix of the batch (one weight, and a batch of weights)
+    ps = torch.rand(16, generator=g) + 0.5
+    bias16 = (torch.randn(48, generator=g) * 0.05).to(torch.bfloat16)
+    out = pa.npu_quant_matmul(x1.cuda(), x2[1].cuda(), s.cuda(), pertoken_scale=ps.cuda(), bias=bias16.cuda(),
+                              output_dtype=torch.bfloat16).cpu()
+    outb = pa.npu_quant_matmul(x1.cuda(), x2.cuda(), s.cuda(), pertoken_scale=ps.cuda(), bias=bias16.cuda(),
+                               output_dtype=torch.bfloat16).cpu()
+    assert out.shape == (2, 3, 16, 48) and outb.shape == (2, 3, 16, 48)
+    for b0 in range(2):
+        for b1 in range(3):
+            want, _ = golden.quant_matmul(x1[b0, b1].numpy(), x2[1].numpy(), s.numpy(), ps.numpy(), _bits(bias16))
+            assert np.array_equal(_bits(out[b0, b1]), want)
+            want, _ = golden.quant_matmul(x1[b0, b1].numpy(), x2[b1].numpy(), s.numpy(), ps.numpy(), _bits(bias16))
+            assert np.array_equal(_bits(outb[b0, b1]), want)
     # leading batch of x1 against one weight (shapes of test/test_fake_tensor.py:1886-1894), per-tensor bf16 scale
     x1 = torch.randint(-127, 128, (1, 1, 1024), generator=g, dtype=torch.int8)
     x2 = torch.randint(-127, 128, (1, 1024, 100), generator=g, dtype=torch.int8)

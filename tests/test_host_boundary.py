@@ -190,13 +190,15 @@ def test_meta_weight_quant_batchmatmul(pa):
         assert r.dtype == torch.int8 and r.shape == (1, 14336)
     r = pa.npu_weight_quant_batchmatmul(xs, w4, sg, og, _m(14336, dtype=torch.float32), _m(14336, dtype=torch.float32), None, 128)
     assert r.dtype == torch.int8
+    r = pa.npu_weight_quant_batchmatmul(xs, w4, sg, og, antiquant_group_size=128, inner_precise=1)
+    assert r.dtype == torch.bfloat16 and r.shape == (1, 14336)
     for kwargs, pat in [(dict(quant_offset=_m(14336, dtype=torch.float32)), "quant_offset needs quant_scale"),
                         (dict(quant_scale=_m(14336, dtype=torch.bfloat16)), "quant_scale must be float32"),
                         (dict(quant_scale=_m(100, dtype=torch.float32)), "quant_scale must have shape"),
                         (dict(quant_scale=_m(14336, dtype=torch.int64), quant_offset=_m(14336, dtype=torch.float32)),
                          "already holds the offset"),
                         (dict(bias=_m(14336, dtype=torch.float16)), "bias must have the dtype of x"),
-                        (dict(inner_precise=1), "inner_precise"),
+                        (dict(inner_precise=2), "inner_precise must be 0 or 1"),
                         (dict(weight_dtype=torch.int8), "weight_dtype")]:
         with pytest.raises(RuntimeError, match=pat):
             pa.npu_weight_quant_batchmatmul(xs, w4, sg, og, antiquant_group_size=128, **kwargs)
