@@ -354,10 +354,9 @@ __global__ __launch_bounds__(BLOCK) void dq_smooth_rows_kernel(const uint16_t *_
                 float v = f[i][k] * r;
                 v = __builtin_fmaf(__builtin_fmaf(-scale, v, f[i][k]), r, v);
                 v = __builtin_fmaf(__builtin_fmaf(-scale, v, f[i][k]), r, v);
-                v = __builtin_rintf(v);
-                v = v > 127.0f ? 127.0f : v;
-                v = v < -127.0f ? -127.0f : v;
-                q[k] = (uint32_t)(int)v;
+                // |v| <= 127 (1 + 2^-22) because |x| <= amax: adding 1.5 * 2^23 rounds to the integer (ties to even) and
+                // leaves it in the low byte; a NaN stays a quiet NaN, whose low byte is 0
+                q[k] = __float_as_uint(v + 12582912.0f);
             }
         } else {
 #pragma unroll
