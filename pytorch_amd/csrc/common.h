@@ -51,15 +51,18 @@ __device__ __forceinline__ float silu_f32(float a) { return a / (1.0f + expf(-a)
 // bf16(silu(a)) for an `a` that is itself a bf16 value, returned as a float.  Exponential and division through the
 // hardware's exp2 and reciprocal are a few units in the last place of binary32 off, which changes the bf16 result only
 // when the value lies next to a rounding boundary of bf16: those (lower 16 bits within 16 of 0x8000: one value in 2048),
-// arguments beyond +-8 (the rounding error of a * log2(e) grows with |a|, and far below zero the reciprocal leaves the
-// normal range) and NaN take the exact formula.  There are only 65536 arguments: tests compare all of them with the
-// exact formula and with the oracle.
+// arguments beyond +-80 (where the exponential or the reciprocal leaves the normal range) and NaN take the exact formula.
+// log2(e) is split into a head of 16 significant bits, whose product with the 8 significant bits of `a` is exact, and a
+// tail applied to the exponential as a factor 1 + a * tail * ln(2): the rounding of a * log2(e) would otherwise grow
+// with |a| (2^-18 of the result at a = -60) and send every argument below -8 - common among real gate activations - to
+// the exact formula.  There are only 65536 arguments: tests compare all of them with the exact formula and with the oracle.
 __device__ __forceinline__ float silu_bf16(float a)
 {
-    const float e = __builtin_amdgcn_exp2f(a * -1.44269504088896340736f);
+    const float e0 = __builtin_amdgcn_exp2f(a * -1.44268798828125f);                  // head: 0x3fb8aa00
+    const float e = __builtin_fmaf(e0, a * -4.888495152129525e-06f, e0);              // tail 7.0526077e-06 * ln(2)
     float s = a * __builtin_amdgcn_rcpf(1.0f + e);
     const uint32_t lo = __float_as_uint(s) & 0xffffu;
-    if (__builtin_expect((lo - 0x7ff0u) < 0x20u || !(fabsf(a) <= 8.0f), 0)) s = silu_f32(a);
+    if (__builtin_expect((lo - 0x7ff0u) < 0x20u || !(fabsf(a) <= 80.0f), 0)) s = silu_f32(a);
     return bf16_1(f32_to_bf16(s));
 }
 
