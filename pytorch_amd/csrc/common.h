@@ -44,6 +44,14 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
     return __builtin_bit_cast(uint32_t, v);
 }
 
+// low bytes of a, b, c, d -> one dword (a lowest)
+__device__ __forceinline__ uint32_t pack4(uint32_t a, uint32_t b, uint32_t c, uint32_t d)
+{
+    uint32_t ab = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);
+    uint32_t cd = __builtin_amdgcn_perm(d, c, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
+}
+
 // SwiGLU on two packed bf16 pairs the way eager bf16 tensor ops evaluate it: s = bf16(a / (1 + exp(-a))) in
 // float32, result = bf16(float(s) * float(b)).
 __device__ __forceinline__ float silu_f32(float a) { return a / (1.0f + expf(-a)); }

@@ -81,13 +81,6 @@ __device__ __forceinline__ uint32_t quant_exact(float x, float scale)
     return (uint32_t)(int)q;
 }
 
-__device__ __forceinline__ uint32_t pack4(uint32_t a, uint32_t b, uint32_t c, uint32_t d)
-{
-    // low bytes of a, b, c, d -> one dword (a lowest)
-    uint32_t ab = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);
-    uint32_t cd = __builtin_amdgcn_perm(d, c, 0x0c0c0400u);
-    return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
-}
 
 // TPR threads cooperate on one row (64 = one wavefront, no barrier; more = the whole block of BLOCK threads);
 // each thread holds ITERS vectors of 8 elements.

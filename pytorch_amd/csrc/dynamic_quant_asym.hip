@@ -46,6 +46,21 @@ __device__ __forceinline__ uint32_t quant1_rcp(float x, float scale, float r, fl
     return finish1(q, offset);
 }
 
+// The same for a row without a NaN: rounding by the addition of 1.5 * 2^23 (ties to even in the adder; the integer is then
+// the distance of the bit pattern from that constant's), clamped as an integer.  Sums beyond the range in which the
+// addition rounds to an integer leave a pattern that is far above or below the constant's on the same side, so the clamp
+// gives what clamping the rounded sum gives; a NaN would clamp to 127 instead of becoming 0, which is why rows with one
+// keep to quant1_rcp.
+__device__ __forceinline__ uint32_t quant1_rcp_nonan(float x, float scale, float r, float offset)
+{
+    float q = x * r;
+    q = __builtin_fmaf(__builtin_fmaf(-scale, q, x), r, q);
+    q = __builtin_fmaf(__builtin_fmaf(-scale, q, x), r, q);
+    const float t = (q + offset) + 12582912.0f;
+    const int k = (int)__float_as_uint(t) - 0x4b400000;
+    return (uint32_t)min(max(k, -128), 127);
+}
+
 // VEC: cols % 8 == 0, rows (and smooth) 16-byte aligned, y rows 8-byte aligned
 // REG (with VEC): cols <= 8192, the row stays in registers between the two passes (four 16-byte vectors per thread)
 template <bool FP16, bool VEC, bool REG = false>
@@ -62,6 +77,7 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
         const uint16_t *xr = x + row * row_stride;
         int8_t *yr = y + row * (int64_t)cols;
         float mx = -INFINITY, mn = INFINITY;
+        bool has_nan = false;                             // maximum and minimum skip a NaN: noted apart
         u32x4 kept[REG ? 4 : 1];
         if constexpr (REG) {
 #pragma unroll
@@ -83,6 +99,7 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
                     if (smooth) f = f * to_f32<FP16>((uint16_t)(s[i / 2] >> (16 * (i & 1))));
                     mx = fmaxf(mx, f);
                     mn = fminf(mn, f);
+                    has_nan = has_nan || f != f;
                 }
             }
         } else {
@@ -112,6 +129,7 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
         rcp = __builtin_fmaf(__builtin_fmaf(-scale, rcp, 1.0f), rcp, rcp);
         const bool fast = __builtin_amdgcn_readfirstlane(
                               (int)(scale >= 0x1p-60f && scale <= 0x1p60f && fmaxf(fabsf(mx), fabsf(mn)) <= 0x1p60f)) != 0;
+        const bool no_nan = __builtin_amdgcn_ballot_w64(has_nan) == 0;          // for this wavefront's elements
         if constexpr (VEC) {
             for (int v = t, it = 0; v < cols / 8; v += 256, it++) {
                 u32x4 a;
@@ -129,7 +147,10 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
                 if (flat) {
 #pragma unroll
                     for (int i = 0; i < 8; i++) q[i] = 0u;
-                } else if (fast) {                            // one branch: never both divisions
+                } else if (fast && no_nan) {                  // one branch: never both divisions
+#pragma unroll
+                    for (int i = 0; i < 8; i++) q[i] = quant1_rcp_nonan(f8[i], scale, rcp, offset);
+                } else if (fast) {
 #pragma unroll
                     for (int i = 0; i < 8; i++) q[i] = quant1_rcp(f8[i], scale, rcp, offset);
                 } else {
@@ -137,8 +158,8 @@ __global__ __launch_bounds__(256) void dq_asym_kernel(const uint16_t *__restrict
                     for (int i = 0; i < 8; i++) q[i] = quant1(f8[i], scale, offset);
                 }
                 u32x2 o;
-                o.x = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
-                o.y = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
+                o.x = pack4(q[0], q[1], q[2], q[3]);
+                o.y = pack4(q[4], q[5], q[6], q[7]);
                 __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(yr) + v);
             }
         } else {

@@ -1329,6 +1329,8 @@ def test_dynamic_quant_asymmetric_extreme_rows(capi, golden):
     x[3, :6] = torch.tensor([1e-30, -1e-30, 1e-38, 0.0, -0.0, 3e-20])   # tiny numerators, ordinary scale
     x[4] = 1000.0 + x[4] * 1e-3                                     # small spread around a large value
     x[5, 0] = 3e38
+    x[6, 10] = float("nan")                                         # a NaN is skipped by the extremes and becomes code 0;
+    x[7, ::67] = float("nan")                                       # its wavefront rounds the ordinary way, the others do not
     x = x.to(torch.bfloat16)
     with np.errstate(all="ignore"):
         wy, ws, wo = golden.dynamic_quant_asymmetric(_bits(x), "bf16", None)
@@ -1336,6 +1338,15 @@ def test_dynamic_quant_asymmetric_extreme_rows(capi, golden):
     assert np.array_equal(s.cpu().numpy().view(np.uint32), ws.view(np.uint32))
     assert np.array_equal(o.cpu().numpy().view(np.uint32), wo.view(np.uint32))
     assert np.array_equal(y.cpu().numpy(), wy)
+    assert y[6, 10] == 0 and not y[7, ::67].any() and y[6].any() and y[7].any()
+    # a wide row with one NaN: only the wavefront that holds it leaves the integer-clamp path
+    xw = (torch.randn(3, 4096, generator=g) * 3 + 1).to(torch.bfloat16)
+    xw[1, 1234] = float("nan")
+    wy, ws, wo = golden.dynamic_quant_asymmetric(_bits(xw), "bf16", None)
+    y, s, o = capi.dynamic_quant_asymmetric(xw.cuda(), None)
+    assert np.array_equal(y.cpu().numpy(), wy) and y[1, 1234] == 0
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+    assert np.array_equal(o.cpu().numpy().view(np.uint32), wo.view(np.uint32))
 
 
 # ------------------------------------------------------------------ error paths (host side, no kernel runs)
