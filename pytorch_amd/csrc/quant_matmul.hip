@@ -108,7 +108,8 @@ __device__ __forceinline__ int32_t requant1(int32_t a, int32_t bi, float sc, flo
 // LOOP 0: the generic K loop below; 3: the same with as many activation slots as weight slots (whole stages requested
 // NS steps ahead); 1, 2: the loop of quant_matmul_wide.h (4 x 2 wavefronts of 64 rows) with its
 // instruction order 0 (refills in a block) or 1 (refills spread over the step)
-template <int WGM, int WGN, int WTM, int WTN, int NS, int LOOP = 0>
+// EPI (the widest wavefront tile only, see LEAN below): which variants of the LDS-parameter epilogue this instantiation holds
+template <int WGM, int WGN, int WTM, int WTN, int NS, int LOOP = 0, int EPI = 0>
 __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 {
     constexpr int NW = WGM * WGN;
@@ -195,15 +196,19 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
         for (int j = 0; j < WTN; j++) acc[i][j] = i32x4v{0, 0, 0, 0};
 
     // the wide loop's epilogue for the common case takes its parameters from LDS (quant_matmul_wide.h)
-    // (the widest wavefront tile keeps to the bias kinds of the common calls: every further variant of its epilogue costs the
-    // K loop registers it does not have - 2048x4096x28672 went from 203 to 219 us with all of them)
+    // (the widest wavefront tile holds few variants of it at a time: every further one costs the K loop registers it does not
+    // have - 2048x4096x28672 went from 203 to 219 us with all of them in one kernel.  EPI 0: no bias or a bf16 one; 1: an
+    // int32 or float32 bias; 2: packed parameter words with no bias or an int32 one.)
     constexpr bool LEAN = WTN >= 7;
+    const bool lean_bias = EPI == 0 ? p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_BF16
+                                    : EPI == 1 && (p.bias_kind == MI355_BIAS_INT32 || p.bias_kind == MI355_BIAS_FP32);
+    const bool lean_qp = EPI == 2 && (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_INT32);
     const bool fast_epilogue = LDSP && !p.out_i32 && !p.out_i8 && !p.qparam && (p.scale_len == p.N || p.scale_len == 1) &&
-                               (!LEAN || p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_BF16) && (p.ldc & 7) == 0 &&
+                               (!LEAN || lean_bias) && (p.ldc & 7) == 0 &&
                                aligned_dev(p.out, 16) && (!p.pertoken || aligned_dev(p.pertoken, 16)) &&
                                (p.scale_len == 1 || aligned_dev(p.scale, 16)) && (!p.bias || aligned_dev(p.bias, 16));
     // ... the same with the column scales taken from packed 64-bit parameter words (no per-token scales then)
-    const bool fast_epilogue_qp = LDSP && !LEAN && !p.out_i32 && !p.out_i8 && p.qparam && !p.pertoken && p.scale_len == p.N && (p.ldc & 7) == 0 &&
+    const bool fast_epilogue_qp = LDSP && (!LEAN || lean_qp) && !p.out_i32 && !p.out_i8 && p.qparam && !p.pertoken && p.scale_len == p.N && (p.ldc & 7) == 0 &&
                                   aligned_dev(p.out, 16) && aligned_dev(p.qparam, 16) && (!p.bias || aligned_dev(p.bias, 16));
     // ... and so does the one for the re-quantised int8 output with per-channel parameter words
     const bool fast_epilogue_i8 = LDSP && p.out_i8 && p.qparam && p.scale_len == p.N &&
@@ -550,7 +555,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             e.stream_out = p.stream_out;
             e.wm = wm;
             e.wn = wn;
-            wide::epilogue_fast<WTN>(acc, lds, e, wave, lane);
+            wide::epilogue_fast<WTN, EPI>(acc, lds, e, wave, lane);
             MI355_TS(4)
             return;
         }
@@ -895,7 +900,7 @@ __global__ __launch_bounds__(256) void transpose_i8_wide_kernel(const int8_t *__
     }
 }
 
-template <int WGM, int WGN, int WTM, int WTN, int DEEP = 0, int LOOP = 0>
+template <int WGM, int WGN, int WTM, int WTN, int DEEP = 0, int LOOP = 0, int EPI = 0>
 int launch_qmm(QmmArgs p, hipStream_t s)
 {
     constexpr int BM = 16 * WTM * WGM, BN = 16 * WTN * WGN;
@@ -917,7 +922,7 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
     if (p.S > 1 && (uint64_t)p.S * BM * BN * 4 >= (1ull << 32)) return MI355_ERR_UNSUPPORTED;
-    auto kern = qmm_kernel<WGM, WGN, WTM, WTN, NS, LOOP>;
+    auto kern = qmm_kernel<WGM, WGN, WTM, WTN, NS, LOOP, EPI>;
     static int attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr_status != hipSuccess) return MI355_ERR_LAUNCH;
@@ -1198,7 +1203,14 @@ int run_quant_matmul(const int8_t *a, const int8_t *b, const float *pertoken_sca
     {
         const int lk = knob(kKnobQmmLoop);                 // 0: automatic; 1: the generic loop; 2, 3: the wide loop with refills in a block / spread; 4: see the planner
         if (lk != 1) {
-            if (c.bm == 256 && c.bn == 224) return lk == 2 ? launch_qmm<4, 2, 4, 7, 0, 1>(p, s) : launch_qmm<4, 2, 4, 7, 0, 2>(p, s);
+            if (c.bm == 256 && c.bn == 224) {
+                if (lk == 2) return launch_qmm<4, 2, 4, 7, 0, 1>(p, s);
+                // the instantiation whose LDS-parameter epilogue serves this call's kind of bias and scale
+                const bool to16 = !p.out_i32 && !p.out_i8;
+                if (to16 && !p.qparam && (p.bias_kind == MI355_BIAS_INT32 || p.bias_kind == MI355_BIAS_FP32)) return launch_qmm<4, 2, 4, 7, 0, 2, 1>(p, s);
+                if (to16 && p.qparam && !p.pertoken && (p.bias_kind == MI355_BIAS_NONE || p.bias_kind == MI355_BIAS_INT32)) return launch_qmm<4, 2, 4, 7, 0, 2, 2>(p, s);
+                return launch_qmm<4, 2, 4, 7, 0, 2>(p, s);
+            }
             if (c.bm == 256 && c.bn == 192) return lk == 2 ? launch_qmm<4, 2, 4, 6, 0, 1>(p, s) : launch_qmm<4, 2, 4, 6, 0, 2>(p, s);
         }
     }

@@ -456,18 +456,26 @@ __device__ __forceinline__ void epilogue_rows(i32x4v (&acc)[4][WTN], char *lds, 
     }
 }
 
-template <int WTN>
+// EPI: the variants a kernel of the widest tile holds (0: float32 scales with no bias or a bf16 one; 1: float32 scales with
+// an int32 or float32 bias; 2: packed parameter words with no bias or an int32 one); the narrower tiles hold them all.
+template <int WTN, int EPI = 0>
 __device__ __forceinline__ void epilogue_fast(i32x4v (&acc)[4][WTN], char *lds, const EpilogueArgs &e, int wave, int lane)
 {
     // output type, kind of bias and kind of store are resolved once per wavefront
     auto go = [&](auto f16, auto bias) {
         constexpr bool H = decltype(f16)::value;
         constexpr int B = decltype(bias)::value;
-        if constexpr (WTN >= 7 && B >= 2) return;           // not instantiated for the widest tile (the kernel never asks)
-        else if (WTN < 7 && e.packed_scale) {
-            if (e.stream_out) epilogue_rows<WTN, H, B, true, true>(acc, lds, e, wave, lane);
-            else epilogue_rows<WTN, H, B, false, true>(acc, lds, e, wave, lane);
-        } else {
+        constexpr bool LEAN = WTN >= 7;
+        constexpr bool PLAIN = !LEAN || (EPI == 0 && B < 2) || (EPI == 1 && B >= 2);   // variants with float32 scales
+        constexpr bool PACKED = !LEAN || (EPI == 2 && (B == 0 || B == 2));             // ... with packed parameter words
+        if constexpr (PACKED) {
+            if (LEAN || e.packed_scale) {
+                if (e.stream_out) epilogue_rows<WTN, H, B, true, true>(acc, lds, e, wave, lane);
+                else epilogue_rows<WTN, H, B, false, true>(acc, lds, e, wave, lane);
+                return;
+            }
+        }
+        if constexpr (PLAIN) {
             if (e.stream_out) epilogue_rows<WTN, H, B, true>(acc, lds, e, wave, lane);
             else epilogue_rows<WTN, H, B, false>(acc, lds, e, wave, lane);
         }
