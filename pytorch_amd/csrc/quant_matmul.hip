@@ -297,13 +297,17 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             wq[slot][0] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? voff_w[0] : kOutOfRange, kb, 2));
             wq[slot][1] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? voff_w[1] : kOutOfRange, kb, 2));
         };
-        // staging: the chunk is 64 rows x 512 bytes = 2048 pieces of 16 bytes, four per thread
+        // staging: the chunk is 64 rows x 512 bytes = 2048 pieces of 16 bytes, four per thread.  A wavefront's instruction
+        // takes 16 rows x 4 consecutive pieces (64 bytes of a row): in fragment order those are one contiguous KiB of LDS
+        // (piece g of row r at g * 256 + r * 16), so the store meets every bank once.  (With a row's 32 pieces on
+        // consecutive lanes the lanes of a store met in four banks.)
         i32x4v xst[4];
+        const int st_row = lane & 15, st_g = lane >> 4;
         auto stage_load = [&](int ch) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int pid = (int)threadIdx.x + 512 * j;
-                const int row = pid >> 5, q = pid & 31;
+                const int combo = wave * 4 + j;                              // (group of 16 rows, group of 4 pieces)
+                const int row = (combo % WTM) * 16 + st_row, q = (combo / WTM) * 4 + st_g;
                 const bool ok = ch * CH + (q >> 3) < KT;
                 xst[j] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(
                     rsrc_a, ok ? (uint32_t)(row * (int)p.lda + q * 16) : kOutOfRange, (uint32_t)(kt0 + ch * CH) * BK, 0));
@@ -313,10 +317,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             char *buf = lds + (ch & 1) * XBUF;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int pid = (int)threadIdx.x + 512 * j;
-                const int row = pid >> 5, q = pid & 31;
-                const int step = q >> 3, t = (q >> 2) & 1, gg = q & 3;
-                *reinterpret_cast<i32x4v *>(buf + ((((step * WTM + (row >> 4)) * 2 + t) * 64) + gg * 16 + (row & 15)) * 16) = xst[j];
+                const int combo = wave * 4 + j;
+                const int mt = combo % WTM, qg = combo / WTM;                // pieces 4 qg .. 4 qg + 3: step qg / 2, half qg % 2
+                *reinterpret_cast<i32x4v *>(buf + ((((qg >> 1) * WTM + mt) * 2 + (qg & 1)) * 64 + st_g * 16 + st_row) * 16) = xst[j];
             }
         };
         stage_load(0);                              // before the weights: loads retire in order, and these come from cache
