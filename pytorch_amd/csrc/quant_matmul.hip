@@ -297,41 +297,40 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             wq[slot][0] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? voff_w[0] : kOutOfRange, kb, 2));
             wq[slot][1] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? voff_w[1] : kOutOfRange, kb, 2));
         };
-        // staging: the chunk is 64 rows x 512 bytes = 2048 pieces of 16 bytes, four per thread.  A wavefront's instruction
-        // takes 16 rows x 4 consecutive pieces (64 bytes of a row): in fragment order those are one contiguous KiB of LDS
-        // (piece g of row r at g * 256 + r * 16), so the store meets every bank once.  (With a row's 32 pieces on
-        // consecutive lanes the lanes of a store met in four banks.)
-        i32x4v xst[4];
+        // staging: the chunk is 64 rows x 512 bytes = 2048 pieces of 16 bytes, four per thread, by direct-to-LDS loads.  A
+        // wavefront's instruction takes 16 rows x 4 consecutive pieces (64 bytes of a row): in fragment order those are one
+        // contiguous KiB of LDS (piece g of row r at g * 256 + r * 16), which is what a direct load writes (lane l at
+        // l * 16 behind the instruction's base).
         const int st_row = lane & 15, st_g = lane >> 4;
-        auto stage_load = [&](int ch) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int combo = wave * 4 + j;                              // (group of 16 rows, group of 4 pieces)
-                const int row = (combo % WTM) * 16 + st_row, q = (combo / WTM) * 4 + st_g;
-                const bool ok = ch * CH + (q >> 3) < KT;
-                xst[j] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(
-                    rsrc_a, ok ? (uint32_t)(row * (int)p.lda + q * 16) : kOutOfRange, (uint32_t)(kt0 + ch * CH) * BK, 0));
-            }
-        };
-        auto stage_store = [&](int ch) {
+        auto stage = [&](int ch) {
             char *buf = lds + (ch & 1) * XBUF;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int combo = wave * 4 + j;
+                const int combo = wave * 4 + j;                              // (group of 16 rows, group of 4 pieces)
                 const int mt = combo % WTM, qg = combo / WTM;                // pieces 4 qg .. 4 qg + 3: step qg / 2, half qg % 2
-                *reinterpret_cast<i32x4v *>(buf + ((((qg >> 1) * WTM + mt) * 2 + (qg & 1)) * 64 + st_g * 16 + st_row) * 16) = xst[j];
+                const int row = mt * 16 + st_row, q = qg * 4 + st_g;
+                const bool ok = ch * CH + (q >> 3) < KT;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void *)(buf + (((qg >> 1) * WTM + mt) * 2 + (qg & 1)) * 1024), 16,
+                                                         ok ? (uint32_t)(row * (int)p.lda + q * 16) : kOutOfRange,
+                                                         (uint32_t)(kt0 + ch * CH) * BK, 0, 0);
             }
         };
-        stage_load(0);                              // before the weights: loads retire in order, and these come from cache
+        // a chunk has landed: at most the `younger` loads issued behind its four are outstanding; and every wavefront is
+        // done with the other buffer
+        auto chunk_barrier = [&](auto younger) {
+            wait_vmcnt_lgkm0<decltype(younger)::value>();
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        };
+        stage(0);                                   // before the weights: loads retire in order, and these come from cache
 #pragma unroll
         for (int r = 0; r < R; r++) load_w(r, r);
-        stage_store(0);
-        __syncthreads();
+        chunk_barrier(std::integral_constant<int, 2 * R>{});
         *reinterpret_cast<i32x4v *>(tbuf + lane * 16) = wq[0][0];
         *reinterpret_cast<i32x4v *>(tbuf + 1024 + lane * 16) = wq[0][1];
         const int nchunks = (KT + CH - 1) / CH;
         for (int ch = 0; ch < nchunks; ch++) {
-            stage_load(ch + 1);                     // past the end: zeros, no memory traffic
+            stage(ch + 1);                          // into the other buffer; past the end: zeros, no memory traffic
             const char *xb = lds + (ch & 1) * XBUF + lane * 16;
 #pragma unroll
             for (int j = 0; j < CH; j++) {
@@ -357,9 +356,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 #pragma unroll
                 for (int mt = 0; mt < WTM; mt++) acc[mt][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, xa[1][mt], acc[mt][0], 0, 0, 0);
             }
-            stage_store(ch + 1);
-            __syncthreads();
+            chunk_barrier(std::integral_constant<int, 2 * CH>{});       // the chunk's weight loads were issued behind its activations
         }
+        wait_vmcnt<0>();                            // nothing is on its way into LDS when the epilogue takes it over
         __syncthreads();
     } else {
     // LDS read addressing: lane reads row (lane % 16) of a 16-row tile, 16-byte chunk (ks*4 + lane/16),
