@@ -270,18 +270,19 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
     } else if constexpr (NS == 0) {
         // ---- streaming K loop (at most 64 rows, few workgroups per CU: the weights are a pure HBM stream).  No workgroup
         // ring and no barrier per K step: a wavefront owns its 16 weight rows (= 16 output columns) for the whole K range
-        // of the workgroup, loads 128 bytes of each row per step straight into registers, four steps in flight - whole cache
-        // lines per instruction (lane l: 16 bytes of row l / 8, and of row 8 + l / 8) - and turns each step around through
-        // a private, XOR-swizzled 2 KiB LDS tile into operand order (a wavefront's LDS operations complete in order, so
-        // this needs no barrier).  Activations are staged through LDS in fragment order, four steps at a time, double
-        // buffered: the loads of the next chunk are issued at the top of a chunk and written to LDS at its end, one
-        // barrier per chunk.
+        // of the workgroup and loads 128 bytes of each row per step by direct-to-LDS loads into a private ring of five
+        // XOR-swizzled 2 KiB tiles, four steps in flight - whole cache lines per instruction (lane l: 16 bytes of row l / 8,
+        // and of row 8 + l / 8) -, from which it reads the step in operand order (its own loads and reads: no barrier, only
+        // the wait for the step's two loads).  Activations are staged in fragment order, four steps at a time, double
+        // buffered, by direct-to-LDS loads as well: the loads of the next chunk are issued at the top of a chunk, one
+        // barrier per chunk.  No register holds an operand before its fragment read.
         static_assert(WGM == 1 && WGN == 8 && WTM == 4 && WTN == 1, "streaming loop: eight wavefronts of 64 rows x 16 columns");
         constexpr int CH = 4;                                   // steps per chunk of activations
         constexpr int XBUF = CH * WTM * 2048;                   // bytes of one activation chunk: [step][m tile][half][lane] x 16
         constexpr int TBUF = 2048;
-        constexpr int R = 4;                                    // weight steps in registers per wavefront
-        char *const tbuf = lds + 2 * XBUF + wave * (2 * TBUF);
+        constexpr int R = 4;                                    // weight steps in flight per wavefront
+        constexpr int RING = R + 1;                             // ... and the one being read
+        char *const tbuf = lds + 2 * XBUF + wave * (RING * TBUF);
         const int c16 = lane & 15, g4 = lane >> 4;
         uint32_t voff_w[2];
 #pragma unroll
@@ -290,12 +291,14 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
             voff_w[h] = (uint32_t)((wn * 16 + rl) * (int)p.ldbt + (((lane & 7) ^ ((rl >> 1) & 7)) * 16));
         }
         const int t_rd = c16 * 128 + ((g4 ^ ((c16 >> 1) & 7)) * 16);   // chunk g of row c; chunk g + 4 is at slot ^ 4
-        i32x4v wq[R][2];
+        // a step's 16 rows x 128 bytes go straight into a slot of the wavefront's ring (lane l at l * 16, i.e. row l / 8 and
+        // row 8 + l / 8 in the swizzled piece order the reads expect)
         auto load_w = [&](int slot, int st) {
             const bool ok = st < KT;
             const uint32_t kb = (uint32_t)(kt0 + st) * BK;
-            wq[slot][0] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? voff_w[0] : kOutOfRange, kb, 2));
-            wq[slot][1] = __builtin_bit_cast(i32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? voff_w[1] : kOutOfRange, kb, 2));
+            char *dst = tbuf + slot * TBUF;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void *)dst, 16, ok ? voff_w[0] : kOutOfRange, kb, 0, 2);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void *)(dst + 1024), 16, ok ? voff_w[1] : kOutOfRange, kb, 0, 2);
         };
         // staging: the chunk is 64 rows x 512 bytes = 2048 pieces of 16 bytes, four per thread, by direct-to-LDS loads.  A
         // wavefront's instruction takes 16 rows x 4 consecutive pieces (64 bytes of a row): in fragment order those are one
@@ -326,30 +329,30 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
 #pragma unroll
         for (int r = 0; r < R; r++) load_w(r, r);
         chunk_barrier(std::integral_constant<int, 2 * R>{});
-        *reinterpret_cast<i32x4v *>(tbuf + lane * 16) = wq[0][0];
-        *reinterpret_cast<i32x4v *>(tbuf + 1024 + lane * 16) = wq[0][1];
         const int nchunks = (KT + CH - 1) / CH;
+        int slot0 = 0;                              // ring slot of the chunk's first step: (ch * CH) % RING
         for (int ch = 0; ch < nchunks; ch++) {
             stage(ch + 1);                          // into the other buffer; past the end: zeros, no memory traffic
             const char *xb = lds + (ch & 1) * XBUF + lane * 16;
 #pragma unroll
             for (int j = 0; j < CH; j++) {
                 const int st = ch * CH + j;
+                const int slot = slot0 + j >= RING ? slot0 + j - RING : slot0 + j;
                 i32x4v xa[2][WTM];
 #pragma unroll
                 for (int t = 0; t < 2; t++)
 #pragma unroll
                     for (int mt = 0; mt < WTM; mt++) xa[t][mt] = *reinterpret_cast<const i32x4v *>(xb + ((j * WTM + mt) * 2 + t) * 1024);
-                const char *tr = tbuf + (j & 1) * TBUF;
+                // this step's weights have landed: behind them are the loads of the R - 1 steps after it and the one chunk of
+                // activations requested within the last R steps (R = CH: always exactly one)
+                static_assert(R == CH, "the count below");
+                wait_vmcnt<2 * (R - 1) + 4>();
+                asm volatile("" ::: "memory");
+                const char *tr = tbuf + slot * TBUF;
                 const i32x4v w0 = *reinterpret_cast<const i32x4v *>(tr + t_rd);
                 const i32x4v w1 = *reinterpret_cast<const i32x4v *>(tr + (t_rd ^ 64));
-                {
-                    char *tw = tbuf + ((j + 1) & 1) * TBUF + lane * 16;      // the next step's registers take the other half
-                    *reinterpret_cast<i32x4v *>(tw) = wq[(j + 1) % R][0];
-                    *reinterpret_cast<i32x4v *>(tw + 1024) = wq[(j + 1) % R][1];
-                }
                 __builtin_amdgcn_sched_barrier(0);
-                load_w(j % R, st + R);                                       // this step's registers are free again
+                load_w(slot == 0 ? RING - 1 : slot - 1, st + R);             // the slot read one step ago
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int mt = 0; mt < WTM; mt++) acc[mt][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, xa[0][mt], acc[mt][0], 0, 0, 0);
@@ -357,6 +360,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, 1) void qmm_kernel(const QmmArgs p)
                 for (int mt = 0; mt < WTM; mt++) acc[mt][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, xa[1][mt], acc[mt][0], 0, 0, 0);
             }
             chunk_barrier(std::integral_constant<int, 2 * CH>{});       // the chunk's weight loads were issued behind its activations
+            slot0 = slot0 + CH >= RING ? slot0 + CH - RING : slot0 + CH;
         }
         wait_vmcnt<0>();                            // nothing is on its way into LDS when the epilogue takes it over
         __syncthreads();
@@ -914,8 +918,8 @@ int launch_qmm(QmmArgs p, hipStream_t s)
     constexpr size_t staging_bytes = (size_t)BM * WGN * ((BN / WGN) * 2 + 16);   // epilogue: padded bf16 tile rows
     // DEEP: that many whole stages, one workgroup per CU (for launches that put at most one of these small tiles on a CU)
     constexpr int NS = DEEP < 0 ? 0 : DEEP ? DEEP : 2 * a_bytes + 2 * b_bytes <= 80 * 1024 && staging_bytes <= 80 * 1024 ? 2 : 3;
-    // DEEP < 0: the streaming K loop (two activation chunks of 32 KiB and a 4 KiB turn-around tile per wavefront)
-    constexpr size_t stage_bytes = DEEP < 0 ? (size_t)2 * 32768 + 8 * 4096 : (DEEP ? DEEP : 2) * a_bytes + NS * b_bytes;
+    // DEEP < 0: the streaming K loop (two activation chunks of 32 KiB and a ring of five 2 KiB weight steps per wavefront)
+    constexpr size_t stage_bytes = DEEP < 0 ? (size_t)2 * 32768 + 8 * 5 * 2048 : (DEEP ? DEEP : 2) * a_bytes + NS * b_bytes;
     constexpr size_t ring_bytes = LOOP == 1 || LOOP == 2 ? (size_t)wide::Geometry<WTN>::LDS_BYTES : stage_bytes + (LOOP == 3 ? 3072 : 0);
     constexpr size_t lds_bytes = ring_bytes > staging_bytes ? ring_bytes : staging_bytes;
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
